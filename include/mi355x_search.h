@@ -1,0 +1,194 @@
+/* mi355x_search.h -- C ABI of the MI355X (gfx950) search & sampling library.
+ *
+ * One entry point per group of functions on onnxruntime-genai's per-step search-and-sampling path.
+ * Each declaration cites the reference interface it stands in for (paths relative to the reference
+ * tree).  All pointers marked "device" are HIP device pointers on the context's GPU; "host" pointers
+ * are ordinary host memory.  Every call is asynchronous on `stream` (a hipStream_t passed as void*)
+ * unless stated otherwise.  Return value: 0 on success, a negative MI355X_E_* code on failure, with a
+ * thread-local message available from mi355x_search_last_error().
+ *
+ * Tie rule everywhere: equal scores are ordered by ascending index (lowest index wins).
+ * -0.0 and +0.0 compare equal.  NaN scores order below every number, except in mi355x_argmax, which
+ * reproduces the reference's strict '>' scan (a NaN at index 0 is never beaten).
+ */
+#ifndef MI355X_SEARCH_H_
+#define MI355X_SEARCH_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355X_OK 0
+#define MI355X_E_INVALID (-1)     /* bad argument (null pointer, size out of range, ...) */
+#define MI355X_E_HIP (-2)         /* a HIP runtime call failed */
+#define MI355X_E_CAPACITY (-3)    /* rows/vocab exceed what the context was created for */
+#define MI355X_E_UNSUPPORTED (-4) /* valid request this build does not implement */
+
+#define MI355X_MAX_EOS 16
+
+/* Element type of a logits / KV tensor (values follow ONNXTensorElementDataType where one exists:
+ * FLOAT = 1, FLOAT16 = 10, the types DeviceInterface::ArgMax/TopKScores accept, src/smartptrs.h:249). */
+#define MI355X_F32 1
+#define MI355X_F16 10
+
+typedef struct mi355x_search_ctx mi355x_search_ctx;
+
+/* Logits processing fused into every selection entry point, applied per element in the reference's
+ * order (src/standard_decoding_strategy.cpp:24-32): grammar mask -> min-length -> repetition penalty.
+ *   mask     device [rows, (vocab-1)/32+1] uint32, bit set = token allowed, else the logit becomes
+ *            lowest() (src/constrained_logits_processor.cpp:246-258, layout :174-183); NULL = none.
+ *   history  device [rows, history_stride] int32 token ids, the first history_len of each row valid
+ *            (Sequences::GetSequence, src/sequences.h:18); every DISTINCT in-range id has its logit
+ *            s replaced by s<0 ? s*penalty : s/penalty (src/sampling_distribution.h:41-62).
+ *            NULL or penalty == 1.0f = none.
+ *   eos_ids  with apply_min_length != 0 each in-range id gets lowest()
+ *            (src/sampling_distribution.h:26-35; the caller evaluates current_length < min_length).
+ */
+typedef struct mi355x_logits_xform {
+  const uint32_t* mask;
+  const int32_t* history;
+  int32_t history_stride;
+  int32_t history_len;
+  float repetition_penalty;
+  int32_t apply_min_length;
+  int32_t n_eos;
+  int32_t eos_ids[MI355X_MAX_EOS];
+} mi355x_logits_xform;
+
+/* (k, p, temperature) of one row: BatchedSamplingParams, src/smartptrs.h:113-117.  Meaning as in
+ * ComputeSampledCategorical (src/sampling_distribution.h:233-297): k > 1 keeps the k best, then
+ * 0 < p < 1 cuts the nucleus inside them; k <= 1 takes the nucleus of the whole vocabulary
+ * (p <= 0 keeps the single best token, i.e. greedy). */
+typedef struct mi355x_sample_params {
+  int32_t k;
+  float p;
+  float temperature;
+} mi355x_sample_params;
+
+/* Creates a context on HIP device `device` with workspace for up to max_rows rows of up to max_vocab
+ * logits (allocates device memory; synchronous).  One context serves one stream at a time. */
+int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_ctx** out);
+void mi355x_search_destroy(mi355x_search_ctx* ctx);
+const char* mi355x_search_last_error(void);
+/* Device bytes held by the context's workspace. */
+size_t mi355x_search_workspace_bytes(const mi355x_search_ctx* ctx);
+
+/* In-place logits processing: stands in for DeviceInterface::LaunchAddLogitsMask
+ * (src/smartptrs.h:218), Search::ApplyMinLength and Search::ApplyRepetitionPenalty
+ * (src/search.h:122-123; CPU src/search.cpp:407-430).  logits: device [rows] rows of `vocab` floats,
+ * row r starting at logits + r*row_stride. */
+int mi355x_process_logits(mi355x_search_ctx* ctx, void* stream, float* logits, int64_t row_stride,
+                          int rows, int vocab, const mi355x_logits_xform* xf);
+
+/* Greedy argmax per row: GreedySearch_Cpu::SelectTop / ArgMax (src/search.cpp:178-192,
+ * src/search.h:9-29) and DeviceInterface::ArgMaxDevice (src/smartptrs.h:258).  dtype MI355X_F32 or
+ * MI355X_F16 (fp16 is widened exactly like FastFloat16ToFloat32, src/models/utils.cpp:103-109).
+ * xf may be NULL.  out_tokens: device [rows] int32. */
+int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype,
+                  int64_t row_stride, int rows, int vocab, const mi355x_logits_xform* xf,
+                  int32_t* out_tokens);
+
+/* Per-row k best (token id, raw fp32 score), best first: DeviceInterface::TopKScores
+ * (src/smartptrs.h:254).  out_tokens/out_scores: device [rows, k].  1 <= k <= 64. */
+int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype,
+                       int64_t row_stride, int rows, int vocab, int k, int32_t* out_tokens,
+                       float* out_scores);
+
+/* Top-k / top-p / top-k+top-p sampling of one token per row: GreedySearch_Cpu::SampleTopK,
+ * SampleTopP, SampleTopKTopP (src/search.cpp:203-254) = ComputeSampledCategorical +
+ * SampleCategoricalToken (src/sampling_distribution.h:218-297), and BatchedSampler::Sample
+ * (src/smartptrs.h:134-137).
+ *   params            used for every row when per_row_params is NULL.
+ *   per_row_params    HOST [rows], heterogeneous parameters (copied by the call).
+ *   uniforms          device [rows] doubles in [0,1): row r's categorical draw, the value
+ *                     std::discrete_distribution would take from generate_canonical<double,53>.
+ *                     A row whose kept set has one token ignores its uniform.
+ *   out_tokens        device [rows] int32.
+ *   kept_count/kept_ids/kept_probs  optional device outputs [rows], [rows,kept_capacity] x2: the
+ *                     kept distribution (ids best first, renormalised fp32 probabilities), truncated
+ *                     to kept_capacity entries per row; kept_count holds the untruncated size.
+ */
+int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int64_t row_stride,
+                  int rows, int vocab, const mi355x_logits_xform* xf, mi355x_sample_params params,
+                  const mi355x_sample_params* per_row_params, const double* uniforms,
+                  int32_t* out_tokens, int32_t* kept_count, int32_t* kept_ids, float* kept_probs,
+                  int kept_capacity);
+
+/* Softmax / log-softmax with temperature, in place, one row per `vocab` floats:
+ * Softmax and LogSoftMax (src/softmax.h:26-47).  Sums are accumulated in index order in fp32 exactly
+ * as the reference does, so results are bit-identical to it. */
+int mi355x_softmax(mi355x_search_ctx* ctx, void* stream, float* scores, int64_t row_stride, int rows,
+                   int vocab, float temperature, int log_softmax);
+
+/* Beam-search candidate selection: BeamSearch_Cpu::SelectTop up to the scorer call
+ * (src/search.cpp:101-164).  logits: device [batch*beams] rows (fp32 or fp16); beam_scores: device
+ * [batch*beams].  Per batch entry the 2*beams best of the beams*vocab values
+ * log_softmax(row)+beam_score, best first: out_scores/out_tokens/out_beam_indices device
+ * [batch, 2*beams] (beam index relative to the batch entry).  beams <= 16. */
+int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype,
+                       int64_t row_stride, int batch, int beams, int vocab, const float* beam_scores,
+                       float* out_scores, int32_t* out_tokens, int32_t* out_beam_indices);
+
+/* Device-resident BeamSearchScorer + Sequences (src/beam_search_scorer.{h,cpp}, src/sequences.{h,cpp},
+ * BeamSearch_Cpu::AppendNextTokensToSequences src/search.cpp:354-381). */
+typedef struct mi355x_beam_scorer mi355x_beam_scorer;
+int mi355x_beam_scorer_create(mi355x_search_ctx* ctx, int batch, int beams, int max_length,
+                              int pad_token_id, const int32_t* eos_ids, int n_eos,
+                              float length_penalty, int early_stopping, mi355x_beam_scorer** out);
+void mi355x_beam_scorer_destroy(mi355x_beam_scorer* s);
+/* Sets the prompt: tokens HOST [batch, prompt_len], replicated to every beam (BeamSearch_Cpu::AppendTokens,
+ * src/search.cpp:326-343). */
+int mi355x_beam_scorer_set_prompt(mi355x_beam_scorer* s, void* stream, const int32_t* tokens,
+                                  int prompt_len);
+/* One BeamSearchScorer::Process + AppendNextTokensToSequences on the candidates produced by
+ * mi355x_beam_select (device [batch, 2*beams]). */
+int mi355x_beam_scorer_step(mi355x_beam_scorer* s, void* stream, const float* cand_scores,
+                            const int32_t* cand_tokens, const int32_t* cand_beam_indices);
+/* Device views valid until the next step: next beam scores [batch*beams], tokens, indices
+ * (GetNextScores/GetNextTokens/GetNextIndices, src/beam_search_scorer.h:52-54). */
+const float* mi355x_beam_scorer_next_scores(const mi355x_beam_scorer* s);
+const int32_t* mi355x_beam_scorer_next_tokens(const mi355x_beam_scorer* s);
+const int32_t* mi355x_beam_scorer_next_indices(const mi355x_beam_scorer* s);
+/* Current sequences: device [batch*beams, max_length]; *length = tokens valid per row. */
+const int32_t* mi355x_beam_scorer_sequences(const mi355x_beam_scorer* s, int* length);
+/* Synchronises `stream` and reports IsDone() (all batch entries done or max_length reached). */
+int mi355x_beam_scorer_is_done(mi355x_beam_scorer* s, void* stream, int* done);
+/* BeamSearchScorer::Finalize + GetBeamHypotheses (src/beam_search_scorer.cpp:173-202): synchronous;
+ * copies hypothesis `index` (0 = best) of batch entry `batch` to HOST out (capacity tokens), returns
+ * its length in *length and its score in *score. */
+int mi355x_beam_scorer_hypothesis(mi355x_beam_scorer* s, void* stream, int batch, int index,
+                                  int32_t* out, int capacity, int* length, float* score);
+
+/* KV-cache beam reorder: DefaultKeyValueCache::PickPastState (src/models/kv_cache.cpp:710-740):
+ * for every tensor t and row j, past[t][j] = present[t][beam_indices[j]], blocks of block_bytes
+ * bytes (a multiple of 16).  present/past: HOST arrays of n_tensors device pointers (copied by the
+ * call); beam_indices: device [rows]. */
+int mi355x_kv_gather(mi355x_search_ctx* ctx, void* stream, const void* const* present,
+                     void* const* past, int n_tensors, const int32_t* beam_indices, int rows,
+                     size_t block_bytes);
+
+/* Speculative-decoding verification on dense distributions: ComputeAcceptProb, the accept loop of
+ * SpeculativeDecodingStrategy::RunRound (src/speculative_decoding_strategy.cpp:718-762) and
+ * SampleCorrectionToken / bonus sampling (src/speculative_sampling.h:32-57,140-146).
+ *   p_target, p_draft  device [batch, K+1, vocab] fp32 probabilities (row K of p_target = bonus row)
+ *   draft_tokens       device [batch, K]
+ *   accept_u           device [batch, K] floats in [0,1) (uniform_real_distribution<float> draws)
+ *   sample_u           device [batch] doubles in [0,1) (the round's single categorical draw)
+ *   accepted_len, final_token  device [batch] outputs.
+ */
+int mi355x_spec_verify(mi355x_search_ctx* ctx, void* stream, const float* p_target,
+                       const float* p_draft, const int32_t* draft_tokens, const float* accept_u,
+                       const double* sample_u, int batch, int K, int vocab, int32_t* accepted_len,
+                       int32_t* final_token);
+
+/* Diagnostics: number of rows, since the context was created, that the single-pass fast paths
+ * declined and the exact general path finished (synchronises `stream`). */
+int mi355x_search_fallback_rows(mi355x_search_ctx* ctx, void* stream, unsigned* rows);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_SEARCH_H_ */

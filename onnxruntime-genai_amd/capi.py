@@ -1,0 +1,185 @@
+"""ctypes binding of include/mi355x_search.h for Python callers (tests, bench).  Device memory is
+supplied by the caller as torch CUDA tensors; this module only passes pointers.  There is no CPU
+fallback: if the shared library is missing, loading fails."""
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+MI355X_F32 = 1
+MI355X_F16 = 10
+MAX_EOS = 16
+
+
+def library_path():
+    return os.path.join(_HERE, "libmi355x_search.so")
+
+
+class LogitsXformC(C.Structure):
+    _fields_ = [("mask", C.c_void_p), ("history", C.c_void_p), ("history_stride", C.c_int32),
+                ("history_len", C.c_int32), ("repetition_penalty", C.c_float), ("apply_min_length", C.c_int32),
+                ("n_eos", C.c_int32), ("eos_ids", C.c_int32 * MAX_EOS)]
+
+
+class SampleParams(C.Structure):
+    _fields_ = [("k", C.c_int32), ("p", C.c_float), ("temperature", C.c_float)]
+
+
+_lib = None
+
+
+def load_library():
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with __graft_entry__.build() (hipcc, gfx950); "
+                           "there is no CPU fallback")
+    L = C.CDLL(path)
+    vp, i32, i64, f32 = C.c_void_p, C.c_int, C.c_int64, C.c_float
+    L.mi355x_search_create.argtypes = [i32, i32, i32, C.POINTER(vp)]
+    L.mi355x_search_destroy.argtypes = [vp]
+    L.mi355x_search_destroy.restype = None
+    L.mi355x_search_last_error.restype = C.c_char_p
+    L.mi355x_search_workspace_bytes.argtypes = [vp]
+    L.mi355x_search_workspace_bytes.restype = C.c_size_t
+    L.mi355x_process_logits.argtypes = [vp, vp, vp, i64, i32, i32, C.POINTER(LogitsXformC)]
+    L.mi355x_argmax.argtypes = [vp, vp, vp, i32, i64, i32, i32, C.POINTER(LogitsXformC), vp]
+    L.mi355x_sample.argtypes = [vp, vp, vp, i64, i32, i32, C.POINTER(LogitsXformC), SampleParams,
+                                C.POINTER(SampleParams), vp, vp, vp, vp, vp, i32]
+    L.mi355x_search_fallback_rows.argtypes = [vp, vp, C.POINTER(C.c_uint)]
+    for name, args in {
+        "mi355x_topk_scores": [vp, vp, vp, i32, i64, i32, i32, i32, vp, vp],
+        "mi355x_softmax": [vp, vp, vp, i64, i32, i32, f32, i32],
+        "mi355x_beam_select": [vp, vp, vp, i32, i64, i32, i32, i32, vp, vp, vp, vp],
+        "mi355x_beam_scorer_create": [vp, i32, i32, i32, i32, C.POINTER(C.c_int32), i32, f32, i32, C.POINTER(vp)],
+        "mi355x_beam_scorer_set_prompt": [vp, vp, C.POINTER(C.c_int32), i32],
+        "mi355x_beam_scorer_step": [vp, vp, vp, vp, vp],
+        "mi355x_beam_scorer_is_done": [vp, vp, C.POINTER(C.c_int)],
+        "mi355x_beam_scorer_hypothesis": [vp, vp, i32, i32, C.POINTER(C.c_int32), i32, C.POINTER(C.c_int),
+                                          C.POINTER(C.c_float)],
+        "mi355x_kv_gather": [vp, vp, C.POINTER(vp), C.POINTER(vp), i32, vp, i32, C.c_size_t],
+        "mi355x_spec_verify": [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, vp],
+    }.items():
+        if hasattr(L, name):
+            getattr(L, name).argtypes = args
+    if hasattr(L, "mi355x_beam_scorer_destroy"):
+        L.mi355x_beam_scorer_destroy.argtypes = [vp]
+        L.mi355x_beam_scorer_destroy.restype = None
+        for n in ("next_scores", "next_tokens", "next_indices"):
+            f = getattr(L, "mi355x_beam_scorer_" + n)
+            f.argtypes = [vp]
+            f.restype = vp
+        L.mi355x_beam_scorer_sequences.argtypes = [vp, C.POINTER(C.c_int)]
+        L.mi355x_beam_scorer_sequences.restype = vp
+    _lib = L
+    return L
+
+
+class LogitsXform:
+    """Python-side description of the fused logits processing (mask / repetition penalty / min length).
+    Holds references to the tensors so they outlive the asynchronous call."""
+
+    def __init__(self, mask=None, history=None, history_len=None, repetition_penalty=1.0, eos_ids=(),
+                 apply_min_length=False):
+        self.mask, self.history = mask, history
+        c = self.c = LogitsXformC()
+        c.mask = mask.data_ptr() if mask is not None else None
+        if mask is not None:
+            assert mask.dtype == torch.int32 and mask.is_cuda and mask.is_contiguous()
+        if history is not None:
+            assert history.dtype == torch.int32 and history.is_cuda and history.is_contiguous() and history.dim() == 2
+            c.history = history.data_ptr()
+            c.history_stride = history.shape[1]
+            c.history_len = history.shape[1] if history_len is None else history_len
+        c.repetition_penalty = repetition_penalty
+        c.apply_min_length = int(apply_min_length)
+        c.n_eos = len(eos_ids)
+        for i, e in enumerate(eos_ids):
+            c.eos_ids[i] = e
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class SearchContext:
+    """Owns a mi355x_search_ctx.  All tensor arguments must be CUDA tensors on the context's device."""
+
+    def __init__(self, max_rows, max_vocab, device=0):
+        self.L = load_library()
+        torch.cuda.init()
+        h = C.c_void_p()
+        self._check(self.L.mi355x_search_create(device, max_rows, max_vocab, C.byref(h)))
+        self.h = h
+        self.device = torch.device("cuda", device)
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.L.mi355x_search_destroy(self.h)
+            self.h = None
+
+    __del__ = close
+
+    def _check(self, rc):
+        if rc != 0:
+            raise RuntimeError(f"mi355x_search error {rc}: {self.L.mi355x_search_last_error().decode()}")
+
+    def workspace_bytes(self):
+        return self.L.mi355x_search_workspace_bytes(self.h)
+
+    def fallback_rows(self):
+        n = C.c_uint()
+        self._check(self.L.mi355x_search_fallback_rows(self.h, _stream(), C.byref(n)))
+        return n.value
+
+    @staticmethod
+    def _rows(logits):
+        assert logits.is_cuda and logits.dim() == 2 and logits.stride(1) == 1
+        return logits.shape[0], logits.shape[1], logits.stride(0)
+
+    def process_logits(self, logits, xf):
+        rows, vocab, stride = self._rows(logits)
+        assert logits.dtype == torch.float32
+        self._check(self.L.mi355x_process_logits(self.h, _stream(), logits.data_ptr(), stride, rows, vocab,
+                                                 C.byref(xf.c)))
+        return logits
+
+    def argmax(self, logits, xf=None, out=None):
+        rows, vocab, stride = self._rows(logits)
+        dtype = {torch.float32: MI355X_F32, torch.float16: MI355X_F16}[logits.dtype]
+        if out is None:
+            out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        self._check(self.L.mi355x_argmax(self.h, _stream(), logits.data_ptr(), dtype, stride, rows, vocab,
+                                         C.byref(xf.c) if xf else None, out.data_ptr()))
+        return out
+
+    def sample(self, logits, uniforms, k=0, p=0.0, temperature=1.0, per_row=None, xf=None, out=None,
+               kept_capacity=0):
+        rows, vocab, stride = self._rows(logits)
+        assert logits.dtype == torch.float32 and uniforms.dtype == torch.float64 and uniforms.numel() >= rows
+        if out is None:
+            out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        pr = None
+        if per_row is not None:
+            pr = (SampleParams * rows)(*[SampleParams(int(a), float(b), float(c)) for a, b, c in per_row])
+        kc = ki = kp = None
+        if kept_capacity:
+            kc = torch.empty(rows, dtype=torch.int32, device=logits.device)
+            ki = torch.full((rows, kept_capacity), -1, dtype=torch.int32, device=logits.device)
+            kp = torch.zeros((rows, kept_capacity), dtype=torch.float32, device=logits.device)
+        self._check(self.L.mi355x_sample(self.h, _stream(), logits.data_ptr(), stride, rows, vocab,
+                                         C.byref(xf.c) if xf else None, SampleParams(int(k), float(p), float(temperature)),
+                                         pr, uniforms.data_ptr(), out.data_ptr(),
+                                         kc.data_ptr() if kept_capacity else None,
+                                         ki.data_ptr() if kept_capacity else None,
+                                         kp.data_ptr() if kept_capacity else None, kept_capacity))
+        if kept_capacity:
+            return out, kc, ki, kp
+        return out
+
+
+class BeamScorer:
+    pass

@@ -1,0 +1,283 @@
+// Device-side building blocks shared by the selection kernels: order-preserving keys, wave64
+// reductions / sorts, the element loader with fused logits processing.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "exact_math.h"
+#include "mi355x_search.h"
+
+namespace ms {
+
+constexpr int kBlock = 256;            // threads per streaming workgroup (4 wave64)
+constexpr int kElems = 32;             // logits held in registers per thread
+constexpr int kChunk = kBlock * kElems;  // logits per streaming workgroup
+constexpr int kSmallCap = 128;         // candidate slots per chunk on the k<=64 path
+constexpr float kLowest = -3.402823466e+38f;
+
+typedef unsigned long long u64;
+
+__device__ __forceinline__ int lane_id() {
+  return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+// Larger key <=> larger score.  +-0 share a key, NaN maps to 0 (below -inf, whose key is 0x007fffff).
+__device__ __forceinline__ uint32_t order_key(float f) {
+  const uint32_t b = __float_as_uint(f);
+  if (f != f) return 0u;
+  if ((b << 1) == 0u) return 0x80000000u;
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+__device__ __forceinline__ float key_to_float(uint32_t k) {
+  if (k == 0u) return __uint_as_float(0x7fc00000u);
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// (score key, index) packed so that a plain unsigned max / descending sort yields
+// "score descending, index ascending".  0 is the padding value (below every real element).
+__device__ __forceinline__ u64 make_key64(uint32_t okey, uint32_t idx) {
+  return (static_cast<u64>(okey) << 32) | static_cast<u64>(0xffffffffu - idx);
+}
+__device__ __forceinline__ uint32_t key64_index(u64 k) { return 0xffffffffu - static_cast<uint32_t>(k); }
+__device__ __forceinline__ uint32_t key64_okey(u64 k) { return static_cast<uint32_t>(k >> 32); }
+
+// ---- cross-lane helpers -------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ T shfl_xor_t(T v, int mask) {
+  return __shfl_xor(v, mask, 64);
+}
+template <>
+__device__ __forceinline__ u64 shfl_xor_t<u64>(u64 v, int mask) {
+  const uint32_t lo = __shfl_xor(static_cast<uint32_t>(v), mask, 64);
+  const uint32_t hi = __shfl_xor(static_cast<uint32_t>(v >> 32), mask, 64);
+  return (static_cast<u64>(hi) << 32) | lo;
+}
+template <typename T>
+__device__ __forceinline__ T shfl_t(T v, int lane) {
+  return __shfl(v, lane, 64);
+}
+template <>
+__device__ __forceinline__ u64 shfl_t<u64>(u64 v, int lane) {
+  const uint32_t lo = __shfl(static_cast<uint32_t>(v), lane, 64);
+  const uint32_t hi = __shfl(static_cast<uint32_t>(v >> 32), lane, 64);
+  return (static_cast<u64>(hi) << 32) | lo;
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_max(T v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    const T o = shfl_xor_t<T>(v, m);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_t<T>(v, m);
+  return v;
+}
+
+// Bitonic sort of one value per lane, descending by lane index (lane 0 ends with the maximum).
+template <typename T>
+__device__ __forceinline__ T wave_sort_desc(T x) {
+  const int lane = lane_id();
+#pragma unroll
+  for (int k = 2; k <= 64; k <<= 1) {
+#pragma unroll
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      const T y = shfl_xor_t<T>(x, j);
+      const bool desc_block = (lane & k) == 0;
+      const bool lower = (lane & j) == 0;
+      const T mx = x > y ? x : y;
+      const T mn = x > y ? y : x;
+      x = (lower == desc_block) ? mx : mn;
+    }
+  }
+  return x;
+}
+
+// Block-wide maximum; every thread gets the result.  `scratch` holds >= blockDim/64 entries.
+template <typename T>
+__device__ __forceinline__ T block_max(T v, T* scratch) {
+  v = wave_max(v);
+  const int lane = lane_id(), wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  T r = scratch[0];
+  for (int w = 1; w < nw; ++w) r = scratch[w] > r ? scratch[w] : r;
+  __syncthreads();
+  return r;
+}
+
+// A key tau such that at least k of the keys offered by the block's threads are >= tau
+// (1 <= k <= 64; threads without an element offer 0).  Each wave sorts its 64 keys, the best
+// 64/waves of every wave are pooled and sorted again; the k-th best of that pool is a valid bound
+// and equals the block's true k-th best unless one wave holds more than its share of the top k.
+// blockDim.x must be 256 (4 waves).  `pool` holds 64 entries.
+__device__ __forceinline__ uint32_t block_kth_bound(uint32_t key, int k, uint32_t* pool) {
+  const int lane = lane_id(), wave = threadIdx.x >> 6;
+  const uint32_t sorted = wave_sort_desc<uint32_t>(key);
+  if (lane < 16) pool[wave * 16 + lane] = sorted;
+  __syncthreads();
+  uint32_t v = pool[lane];
+  v = wave_sort_desc<uint32_t>(v);
+  const uint32_t tau = shfl_t<uint32_t>(v, k - 1);
+  __syncthreads();
+  return tau;
+}
+
+// Loads with agent-scope coherence, for data another workgroup of the same launch wrote.
+__device__ __forceinline__ u64 load_coherent(const u64* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t load_coherent(const uint32_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- fp16 widening ------------------------------------------------------------------------------
+// Same value as the reference's FastFloat16ToFloat32 (src/models/utils.cpp:103-109): IEEE for zeros,
+// subnormals and normals; an exponent field of 31 (Inf/NaN in IEEE) is decoded as an ordinary
+// exponent, giving +-65536*(1+m/1024).
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+  const uint32_t sign = (h & 0x8000u) << 16;
+  const uint32_t e = (h >> 10) & 0x1fu;
+  const uint32_t m = h & 0x3ffu;
+  if (e != 0u) return __uint_as_float(sign | ((e + 112u) << 23) | (m << 13));
+  // subnormal or zero: m * 2^-24, exact in fp32
+  const float mag = static_cast<float>(m) * 5.9604644775390625e-08f;
+  return __uint_as_float(sign | __float_as_uint(mag));
+}
+
+// ---- fused logits processing --------------------------------------------------------------------
+struct Xform {
+  const uint32_t* mask;
+  const int32_t* history;
+  int history_stride;
+  int history_len;
+  float penalty;
+  int n_eos;  // 0 unless min-length masking is active
+  int eos[MI355X_MAX_EOS];
+  __host__ __device__ bool active() const { return mask || use_penalty() || n_eos > 0; }
+  __host__ __device__ bool use_penalty() const { return history && history_len > 0 && penalty != 1.0f; }
+};
+
+// Marks, in an LDS bitmap covering vocabulary ids [base, base + kChunk), the ids present in the
+// row's history.  bits: kChunk/32 words.  Ends with a barrier.
+__device__ __forceinline__ void build_history_bitmap(const Xform& xf, int row, int base, uint32_t* bits) {
+  for (int i = threadIdx.x; i < kChunk / 32; i += blockDim.x) bits[i] = 0u;
+  __syncthreads();
+  const int32_t* h = xf.history + static_cast<size_t>(row) * xf.history_stride;
+  for (int i = threadIdx.x; i < xf.history_len; i += blockDim.x) {
+    const int rel = h[i] - base;
+    if (rel >= 0 && rel < kChunk) atomicOr(&bits[rel >> 5], 1u << (rel & 31));
+  }
+  __syncthreads();
+}
+
+// The reference's order: mask -> min-length -> repetition penalty.
+__device__ __forceinline__ float xform_value(float x, const Xform& xf, int idx, uint32_t mask_word,
+                                             bool has_mask, bool in_history) {
+  if (has_mask && !((mask_word >> (idx & 31)) & 1u)) x = kLowest;
+  for (int e = 0; e < xf.n_eos; ++e)
+    if (xf.eos[e] == idx) x = kLowest;
+  if (in_history) x = x < 0.0f ? x * xf.penalty : x / xf.penalty;
+  return x;
+}
+
+// Loads the kElems logits a thread owns in chunk `chunk` of a row, widened to fp32 and processed.
+// Thread t owns, for j = 0..NV-1, the VEC consecutive ids starting at
+// chunk*kChunk + (j*kBlock + t)*VEC; ids >= vocab yield 0 and must be ignored by the caller.
+template <typename InT>
+struct Loader;
+
+template <>
+struct Loader<float> {
+  static constexpr int VEC = 4;
+  static constexpr int NV = kElems / VEC;
+  __device__ static __forceinline__ int index_of(int chunk, int j, int c) {
+    return chunk * kChunk + (j * kBlock + static_cast<int>(threadIdx.x)) * VEC + c;
+  }
+  __device__ static __forceinline__ void load(const float* row, bool aligned, int vocab, int chunk,
+                                              float (&v)[kElems]) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i0 = index_of(chunk, j, 0);
+      if (aligned && i0 + VEC <= vocab) {
+        const float4 q = *reinterpret_cast<const float4*>(row + i0);
+        v[j * 4 + 0] = q.x;
+        v[j * 4 + 1] = q.y;
+        v[j * 4 + 2] = q.z;
+        v[j * 4 + 3] = q.w;
+      } else {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) v[j * 4 + c] = (i0 + c < vocab) ? row[i0 + c] : 0.0f;
+      }
+    }
+  }
+};
+
+template <>
+struct Loader<uint16_t> {  // IEEE binary16 bit patterns
+  static constexpr int VEC = 8;
+  static constexpr int NV = kElems / VEC;
+  __device__ static __forceinline__ int index_of(int chunk, int j, int c) {
+    return chunk * kChunk + (j * kBlock + static_cast<int>(threadIdx.x)) * VEC + c;
+  }
+  __device__ static __forceinline__ void load(const uint16_t* row, bool aligned, int vocab, int chunk,
+                                              float (&v)[kElems]) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i0 = index_of(chunk, j, 0);
+      if (aligned && i0 + VEC <= vocab) {
+        const uint4 q = *reinterpret_cast<const uint4*>(row + i0);
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          v[j * 8 + 2 * c] = half_bits_to_float(w[c] & 0xffffu);
+          v[j * 8 + 2 * c + 1] = half_bits_to_float(w[c] >> 16);
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) v[j * 8 + c] = (i0 + c < vocab) ? half_bits_to_float(row[i0 + c]) : 0.0f;
+      }
+    }
+  }
+};
+
+// Applies the logits processing to the registers loaded by Loader<InT>::load.
+template <typename InT>
+__device__ __forceinline__ void xform_chunk(const Xform& xf, int row, int vocab, int chunk,
+                                            const uint32_t* hist_bits, float (&v)[kElems]) {
+  using L = Loader<InT>;
+  const bool has_mask = xf.mask != nullptr;
+  const bool pen = xf.use_penalty();
+  const uint32_t* mrow = has_mask ? xf.mask + static_cast<size_t>(row) * ((vocab - 1) / 32 + 1) : nullptr;
+#pragma unroll
+  for (int j = 0; j < L::NV; ++j) {
+#pragma unroll
+    for (int c = 0; c < L::VEC; ++c) {
+      const int idx = L::index_of(chunk, j, c);
+      if (idx < vocab) {
+        const uint32_t mw = has_mask ? mrow[idx >> 5] : 0u;
+        const int rel = idx - chunk * kChunk;
+        const bool hit = pen && ((hist_bits[rel >> 5] >> (rel & 31)) & 1u);
+        v[j * L::VEC + c] = xform_value(v[j * L::VEC + c], xf, idx, mw, has_mask, hit);
+      }
+    }
+  }
+}
+
+// Single-element version for code that revisits a row outside the streaming layout.
+template <typename InT>
+__device__ __forceinline__ float load_one(const InT* row, int idx);
+template <>
+__device__ __forceinline__ float load_one<float>(const float* row, int idx) { return row[idx]; }
+template <>
+__device__ __forceinline__ float load_one<uint16_t>(const uint16_t* row, int idx) {
+  return half_bits_to_float(row[idx]);
+}
+
+}  // namespace ms

@@ -1,0 +1,58 @@
+// Argument blocks and launch entry points shared between the host API (api.cpp) and the kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include "device_utils.h"
+
+namespace ms {
+
+constexpr int kFinCap = 2048;        // merged candidates a finishing workgroup can hold (k <= 64 path)
+constexpr int kNucleusCap = 16384;   // sorted nucleus candidates held in LDS by the finish kernel
+constexpr int kFinishBlock = 1024;
+
+constexpr int kModeTopkSmall = 0;
+constexpr int kModeNucleus = 1;
+constexpr int kModeGeneral = 2;
+
+struct SampleArgs {
+  const float* logits;
+  int64_t row_stride;
+  int rows, vocab, chunks;
+  Xform xf;
+  mi355x_sample_params uniform;
+  const mi355x_sample_params* per_row;  // device, or null
+  const double* uniforms;
+  int32_t* out_tokens;
+  int32_t* kept_count;
+  int32_t* kept_ids;
+  float* kept_probs;
+  int kept_capacity;
+  // workspace
+  u64* cand_small;        // [rows][chunks][kSmallCap]
+  uint32_t* chunk_cnt;    // [rows][chunks]
+  uint32_t* chunk_max;    // [rows][chunks]
+  u64* chunk_next;        // [rows][chunks]
+  uint32_t* row_arrive;   // [rows], zero between launches
+  u64* big;               // [rows][big_stride]
+  size_t big_stride;
+  uint32_t* fallback_rows;  // cumulative count of rows finished by the general path
+};
+
+struct ArgmaxArgs {
+  const void* logits;
+  int64_t row_stride;
+  int rows, vocab, chunks;
+  Xform xf;
+  int32_t* out_tokens;
+  u64* row_best;         // [rows], zero between launches
+  uint32_t* row_arrive;  // [rows], zero between launches
+};
+
+}  // namespace ms
+
+extern "C" {
+hipError_t ms_sample_init();
+hipError_t ms_launch_sample(const ms::SampleArgs* a, bool any_nucleus, hipStream_t stream);
+hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipStream_t stream);
+hipError_t ms_launch_process_logits(float* logits, int64_t row_stride, int rows, int vocab,
+                                    const ms::Xform* xf, hipStream_t stream);
+}
