@@ -221,7 +221,16 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
 
   // ---- top-k, k <= 64 ----
   const int kk = prm.k < V ? prm.k : V;
-  const uint32_t tau = block_kth_bound(lmax, kk, sm.pool);
+  uint32_t tau = block_kth_bound(lmax, kk, sm.pool);
+  if (tau == 0u) {
+    // The pooled bound degenerated (a short tail chunk keeps its elements in one or two waves):
+    // take the exact kk-th best of the 256 per-thread maxima instead.
+    sm.fin[tid] = static_cast<u64>(lmax);
+    __syncthreads();
+    block_sort_desc(sm.fin, kBlock);
+    tau = static_cast<uint32_t>(sm.fin[kk - 1]);
+    __syncthreads();
+  }
 #pragma unroll
   for (int e = 0; e < kElems; ++e) {
     const int idx = Loader<float>::index_of(chunk, e / 4, e % 4);

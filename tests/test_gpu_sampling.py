@@ -132,7 +132,6 @@ def test_config2_topk_topp_batch64(ctx, orc):
         u = rng.random(rows)
         tok = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=50, p=0.9, temperature=0.7)
         assert np.array_equal(tok.cpu().numpy(), orc.sample_batch(x, 50, 0.9, 0.7, u))
-    assert ctx.fallback_rows() == 0 or True
 
 
 def test_sample_ties_and_degenerate_rows(ctx, orc):
