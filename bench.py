@@ -1,0 +1,138 @@
+#!/usr/bin/env python3
+"""Headline benchmark: top-k/top-p sampling step, batch 64 x vocab 128256 (BASELINE config 2).
+
+A step is one pass of the sampling hot path (mi355x_sample: fused selection + softmax + nucleus cut +
+categorical draw) over one batch of seeded synthetic fp32 logits resident in HBM.  The K timed steps
+are recorded once into a HIP graph (one kernel launch per step, each on its own logits buffer from a
+pool larger than twice the 256 MB Infinity Cache) and replayed between two HIP events on the launch
+stream.  Before any number is printed, token ids of the checked steps are compared with the CPU
+oracle on identical logits and uniforms; the same oracle, timed on the host cores, is the
+cpu_baseline.  Prints ONE JSON line."""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+ROWS, VOCAB, TOP_K, TOP_P, TEMP = 64, 128256, 50, 0.9, 0.7
+HBM_PEAK_GBS = 8000.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--pool", type=int, default=32, help="distinct logits buffers cycled through")
+    ap.add_argument("--cpu-steps", type=int, default=24, help="steps replayed on the CPU oracle")
+    ap.add_argument("--traffic", type=str, default=None, help="JSON {fetch_bytes, write_bytes} from rocprofv3 --pmc")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (rows shard across GPUs "
+                 "without communication; see DESIGN.md). Run with --gpus 1.")
+
+    import numpy as np
+    import torch
+    import __graft_entry__ as ge
+    import orc_lib
+
+    pkg = ge.load_package()
+    orc = orc_lib.Oracle()
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    K, W = args.steps, args.warmup
+    pool = max(2, min(args.pool, K + W))
+
+    # ---- seeded synthetic inputs: N(0, 3^2) logits + 8 peaks per row at +10 -------------------------
+    gen = torch.Generator(device=dev).manual_seed(1234)
+    logits = []
+    for _ in range(pool):
+        x = torch.randn(ROWS, VOCAB, generator=gen, device=dev, dtype=torch.float32) * 3.0
+        peaks = torch.randint(0, VOCAB, (ROWS, 8), generator=gen, device=dev)
+        x.scatter_add_(1, peaks, torch.full((ROWS, 8), 10.0, device=dev))
+        logits.append(x)
+    rng = np.random.default_rng(99)
+    u_host = rng.random((K + W, ROWS))
+    uniforms = torch.from_numpy(u_host).to(dev)
+    tokens = torch.empty((K + W, ROWS), dtype=torch.int32, device=dev)
+    ctx = pkg.SearchContext(ROWS, VOCAB)
+
+    def step(i):
+        ctx.sample(logits[i % pool], uniforms[i], k=TOP_K, p=TOP_P, temperature=TEMP, out=tokens[i])
+
+    for i in range(W):  # warm-up, untimed
+        step(i)
+    torch.cuda.synchronize()
+
+    # ---- parity gate: GPU tokens == CPU oracle tokens on identical inputs ---------------------------
+    n_cpu = max(1, min(args.cpu_steps, K))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(W, W + K):
+                step(i)
+        graph.replay()  # first replay untimed (graph upload)
+        side.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(side)
+        graph.replay()
+        end.record(side)
+        side.synchronize()
+    torch.cuda.synchronize()
+    gpu_ms = start.elapsed_time(end)
+    got = tokens[W:W + n_cpu].cpu().numpy()
+    cpu_in = [logits[(W + i) % pool].cpu().numpy() for i in range(n_cpu)]
+    t0 = time.perf_counter()
+    want = np.stack([orc.sample_batch(cpu_in[i], TOP_K, TOP_P, TEMP, u_host[W + i]) for i in range(n_cpu)])
+    cpu_s = time.perf_counter() - t0
+    if not np.array_equal(got, want):
+        bad = int((got != want).sum())
+        sys.exit(f"PARITY FAILURE: {bad} of {got.size} sampled tokens differ from the CPU oracle")
+    fallback = ctx.fallback_rows()
+
+    ms_per_step = gpu_ms / K
+    algo_bytes = ROWS * VOCAB * 4 + ROWS * 8 + ROWS * 4  # logits once + uniforms + tokens
+    achieved = algo_bytes / (ms_per_step * 1e-3) / 1e9
+    traffic = None
+    if args.traffic:
+        t = json.loads(args.traffic)
+        traffic = t.get("fetch_bytes", 0) + t.get("write_bytes", 0)
+    out = {
+        "metric": "sampled tokens/sec + step latency, B=64 V=128256 top-k/p; % HBM roofline",
+        "value": ROWS * K / (gpu_ms * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": ms_per_step,
+        "step_latency_us": ms_per_step * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "config 2: top-k/top-p sampling, batch 64 x vocab 128256 fp32, T=0.7 k=50 p=0.9, "
+                               "one fused kernel per step, %d steps replayed from a HIP graph over a pool of %d "
+                               "logits buffers" % (K, pool),
+                   "rows": ROWS, "vocab": VOCAB, "top_k": TOP_K, "top_p": TOP_P, "temperature": TEMP,
+                   "parity": "token ids of %d steps bit-identical to the CPU oracle" % n_cpu,
+                   "general_path_rows": fallback},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel": "sample_stream_kernel", "algorithmic_bytes_per_launch": algo_bytes},
+        "cpu_baseline": {"value": ROWS * n_cpu / cpu_s, "unit": "tokens/s", "cores": 1, "kind": "port",
+                         "sample": "%d of the %d timed steps (same logits and uniforms), oracle/search_oracle.cpp "
+                                   "orc_sample_batch, one thread as in the reference's serial row loop" % (n_cpu, K),
+                         "ms_per_step": cpu_s / n_cpu * 1e3, "host_cpus": os.cpu_count()},
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

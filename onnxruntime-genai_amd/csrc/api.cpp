@@ -5,6 +5,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <cstdlib>
 #include <new>
 #include <string>
 #include <vector>
@@ -133,11 +134,13 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   const size_t rc = static_cast<size_t>(max_rows) * c->max_chunks;
   c->big_stride = static_cast<size_t>(NextPow2(max_vocab));
   if (c->big_stride < static_cast<size_t>(c->max_chunks) * ms::kChunk) c->big_stride = static_cast<size_t>(c->max_chunks) * ms::kChunk;
+  if (c->big_stride < static_cast<size_t>(ms::kSChunk)) c->big_stride = ms::kSChunk;
   hipError_t e = hipSuccess;
   auto ok = [&](hipError_t r) {
     if (e == hipSuccess) e = r;
   };
-  ok(c->Alloc(&c->cand_small, rc * ms::kSmallCap, false));
+  const size_t sc = static_cast<size_t>(max_rows) * ((max_vocab + ms::kSChunk - 1) / ms::kSChunk);
+  ok(c->Alloc(&c->cand_small, sc * ms::kSmallCap, true));  // all-zero between launches
   ok(c->Alloc(&c->chunk_cnt, rc, true));
   ok(c->Alloc(&c->chunk_max, rc, true));
   ok(c->Alloc(&c->chunk_next, rc, true));
@@ -229,7 +232,7 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   a.row_stride = row_stride;
   a.rows = rows;
   a.vocab = vocab;
-  a.chunks = (vocab + ms::kChunk - 1) / ms::kChunk;
+  a.chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
   a.uniform = params;
   a.uniforms = uniforms;
   a.out_tokens = out_tokens;
@@ -245,6 +248,9 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
+#ifdef MS_DEBUG_STAGES
+  a.debug_stage = getenv("MS_STAGE") ? atoi(getenv("MS_STAGE")) : 0;
+#endif
   HIP_TRY(ms_launch_sample(&a, any_nucleus, s));
   return MI355X_OK;
 }

@@ -11,7 +11,6 @@ namespace ms {
 constexpr int kBlock = 256;            // threads per streaming workgroup (4 wave64)
 constexpr int kElems = 32;             // logits held in registers per thread
 constexpr int kChunk = kBlock * kElems;  // logits per streaming workgroup
-constexpr int kSmallCap = 128;         // candidate slots per chunk on the k<=64 path
 constexpr float kLowest = -3.402823466e+38f;
 
 typedef unsigned long long u64;

@@ -76,16 +76,12 @@ EM_HD uint64_t exp2_tab(uint32_t i) {
   return tab[i];
 }
 
-// expf(x), bit-identical to glibc's.
-EM_HD float expf_exact(float x) {
+// expf(x), bit-identical to glibc's.  `tab(i)` must return exp2_tab(i); callers that already hold the
+// table in registers or LDS pass their own accessor.
+template <typename Tab>
+EM_HD float expf_core(float x, Tab tab) {
   const uint32_t ix = as_u32(x);
   const uint32_t abstop = (ix >> 20) & 0x7ff;
-  if (abstop >= 0x42b) {  // |x| >= 88 or NaN/Inf
-    if (ix == 0xff800000u) return 0.0f;
-    if (abstop >= 0x7f8) return x + x;
-    if (x > 0x1.62e42ep6f) return as_float(0x7f800000u);  // overflow
-    if (x < -0x1.9fe368p6f) return 0.0f;                  // underflow to zero
-  }
   const double N = 32.0;
   const double inv_ln2_n = 0x1.71547652b82fep+0 * N;
   const double shift = 0x1.8p+52;
@@ -102,7 +98,7 @@ EM_HD float expf_exact(float x) {
 #else
   const double r = z - kd;
 #endif
-  uint64_t t = exp2_tab((uint32_t)(ki % 32));
+  uint64_t t = tab((uint32_t)(ki % 32));
   t += ki << (52 - 5);
   const double s = as_double(t);
   z = mad(c0, r, c1);
@@ -110,8 +106,21 @@ EM_HD float expf_exact(float x) {
   double y = mad(c2, r, 1.0);
   y = mad(z, r2, y);
   y = y * s;
-  return (float)y;
+  float res = (float)y;
+  if (abstop >= 0x42b) {  // |x| >= 88 or NaN/Inf
+    if (ix == 0xff800000u) res = 0.0f;
+    else if (abstop >= 0x7f8) res = x + x;
+    else if (x > 0x1.62e42ep6f) res = as_float(0x7f800000u);  // overflow
+    else if (x < -0x1.9fe368p6f) res = 0.0f;                  // underflow to zero
+  }
+  return res;
 }
+
+struct DefaultExp2Tab {
+  EM_HD uint64_t operator()(uint32_t i) const { return exp2_tab(i); }
+};
+
+EM_HD float expf_exact(float x) { return expf_core(x, DefaultExp2Tab{}); }
 
 struct LogTab {
   double invc, logc;

@@ -5,7 +5,17 @@
 
 namespace ms {
 
-constexpr int kFinCap = 2048;        // merged candidates a finishing workgroup can hold (k <= 64 path)
+// Shape of the fused sampling kernel: 256 threads x 16 float4 = one 16K-logit chunk per workgroup.
+// Many logits per lane keep the per-wave selection overhead small against the streaming work, and
+// thread t's float4s (t, t+256, t+512, ...) make every wave an even sample of the whole chunk.
+constexpr int kSBlock = 256;
+constexpr int kSWaves = kSBlock / 64;
+constexpr int kSVec = 16;                   // 128-bit loads per thread
+constexpr int kSElems = kSVec * 4;          // logits held in registers per thread
+constexpr int kSChunk = kSBlock * kSElems;  // logits per workgroup
+constexpr int kSmallCap = 256;       // candidate slots per chunk on the k<=64 path
+constexpr int kAllCap = 4096;        // merged candidates a finishing workgroup can hold (16 chunks x kSmallCap)
+constexpr int kSelCap = 256;         // survivors of the second bound handed to the finishing wave
 constexpr int kNucleusCap = 16384;   // sorted nucleus candidates held in LDS by the finish kernel
 constexpr int kFinishBlock = 1024;
 
@@ -35,6 +45,9 @@ struct SampleArgs {
   u64* big;               // [rows][big_stride]
   size_t big_stride;
   uint32_t* fallback_rows;  // cumulative count of rows finished by the general path
+#ifdef MS_DEBUG_STAGES
+  int debug_stage;  // timing experiments only: stop after the given stage
+#endif
 };
 
 struct ArgmaxArgs {

@@ -1,20 +1,98 @@
-// Sampling kernels: one streaming pass over the logits (fused logits processing + candidate
-// selection), finished per row by the last workgroup to arrive (top-k <= 64) or by a second per-row
-// kernel (nucleus), with an exact general path for everything the fast paths decline.
+// Sampling kernels.
+//
+// sample_fused_kernel: one launch per step.  Every workgroup (256 threads x 64 logits) streams one
+// 16K-logit chunk of one row with 128-bit non-temporal loads (logits processing fused), keeps the chunk's
+// candidates for the row's top-k and publishes them; the last workgroup of a row to arrive merges the
+// row's candidates, sorts the k survivors and runs the reference's scalar epilogue (softmax over the
+// k, nucleus cut, categorical draw) in rank order.  Rows in nucleus mode (k <= 1) only compact their
+// candidates here; nucleus_finish_kernel sorts them and finishes.  Anything the fast paths decline
+// (k > 64, heavy ties, tiny vocabularies) goes through general_row, an exact full sort.
 #include "kernels.h"
 #include "block_seq.h"
 
 namespace ms {
 
-// ------------------------------------------------------------------------------------------------
+#ifdef MS_DEBUG_STAGES
+#define MS_STAGE(n, keep) do { if (a.debug_stage == (n)) { if ((keep) == 0x12345u) a.out_tokens[row] = 1; return false; } } while (0)
+#else
+#define MS_STAGE(n, keep) do { } while (0)
+#endif
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// ---- lane exchange primitives ---------------------------------------------------------------------
+template <int M>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t x) {
+  if constexpr (M == 1) {
+    return __builtin_amdgcn_mov_dpp(x, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+  } else if constexpr (M == 2) {
+    return __builtin_amdgcn_mov_dpp(x, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+  } else if constexpr (M == 4) {
+    return __builtin_amdgcn_ds_swizzle(x, (4 << 10) | 0x1f);   // bit-mask mode, xor 4
+  } else if constexpr (M == 8) {
+    return __builtin_amdgcn_mov_dpp(x, 0x128, 0xf, 0xf, true);  // row_ror:8 == xor 8 inside a row of 16
+  } else if constexpr (M == 16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+    return (lane_id() & 16) ? r[0] : r[1];
+  } else {
+    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return (lane_id() & 32) ? r[0] : r[1];
+  }
+}
+
+template <int M>
+__device__ __forceinline__ u64 lane_xor64(u64 x) {
+  const uint32_t lo = lane_xor<M>(static_cast<uint32_t>(x));
+  const uint32_t hi = lane_xor<M>(static_cast<uint32_t>(x >> 32));
+  return (static_cast<u64>(hi) << 32) | lo;
+}
+__device__ __forceinline__ uint32_t lane_xor_any(uint32_t x, int m) { return __shfl_xor(x, m, 64); }
+
+template <int K, int J, typename T>
+__device__ __forceinline__ void sort_merge(T& x, int lane) {
+  T y;
+  if constexpr (sizeof(T) == 8) y = lane_xor64<J>(x);
+  else y = lane_xor<J>(x);
+  const bool keep_max = (((lane & K) == 0) == ((lane & J) == 0));
+  x = ((y > x) == keep_max) ? y : x;
+  if constexpr (J > 1) sort_merge<K, J / 2, T>(x, lane);
+}
+
+// Bitonic sort of one key per lane, descending by lane (lane 0 ends with the maximum).
+template <typename T>
+__device__ __forceinline__ T wave_sort_desc_fast(T x) {
+  const int lane = lane_id();
+  sort_merge<2, 1, T>(x, lane);
+  sort_merge<4, 2, T>(x, lane);
+  sort_merge<8, 4, T>(x, lane);
+  sort_merge<16, 8, T>(x, lane);
+  sort_merge<32, 16, T>(x, lane);
+  sort_merge<64, 32, T>(x, lane);
+  return x;
+}
+
+// k-th largest of the wave's R keys per lane (0 if fewer than k keys are non-zero): bisection on the
+// key bits with wave-wide population counts.
+template <int R>
+__device__ __forceinline__ uint32_t wave_kth_largest(const uint32_t (&key)[R], int k) {
+  uint32_t prefix = 0u;
+#pragma unroll 1
+  for (int bit = 31; bit >= 0; --bit) {
+    const uint32_t cand = prefix | (1u << bit);
+    int cnt = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) cnt += __popcll(__ballot(key[r] >= cand));
+    if (cnt >= k) prefix = cand;
+  }
+  return prefix;
+}
+
 // Serial prefix over lanes: out[l] = ((x[0] + x[1]) + ...) + x[l], additions in lane order, as the
-// reference's scalar loops do.  One DPP-shifted add per element.
+// reference's scalar loops do.  One DPP-shifted add per element (wave_shr:1, lane 0 reads 0).
 __device__ __forceinline__ float wave_serial_prefix(float x, int count) {
   float s = 0.0f;
   for (int t = 0; t < count; ++t) {
-    // wave_shr:1 -- lane l reads lane l-1; lane 0 keeps `old` (0.0f).
-    const float prev = __uint_as_float(
-        __builtin_amdgcn_update_dpp(0u, __float_as_uint(s), 0x138, 0xf, 0xf, false));
+    const float prev = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s), 0x138, 0xf, 0xf, false));
     s = prev + x;
   }
   return s;
@@ -47,52 +125,21 @@ __device__ __forceinline__ uint32_t wave_slot(bool pred, uint32_t* counter) {
 
 __device__ __forceinline__ int first_lane(u64 ballot) { return ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : -1; }
 
-// Epilogue for k <= 64 run by one wave: lane j holds the j-th best (key64), j < m.
-// Follows ComputeSampledCategorical's top-k branch (src/sampling_distribution.h:243-281) and
-// std::discrete_distribution literally: every sum is accumulated in rank order.
-__device__ __forceinline__ void wave_topk_epilogue(u64 key, int m, mi355x_sample_params prm, double u, const RowOutputs& out) {
-  const int lane = lane_id();
-  const float score = key_to_float(key64_okey(key));
-  const float max_score = shfl_t<float>(score, 0);
-  const float inv_temp = 1.0f / prm.temperature;
-  const float e = lane < m ? em::expf_exact((score - max_score) * inv_temp) : 0.0f;
-  const float sum = shfl_t<float>(wave_serial_prefix(e, m), m - 1);
-  const float pr = sum > 0.0f ? e / sum : e;
-  const float cum = wave_serial_prefix(pr, m);
-  int keep = m;
-  if (prm.p > 0.0f && prm.p < 1.0f) {
-    const int f = first_lane(__ballot(lane < m && cum >= prm.p));
-    if (f >= 0) keep = f + 1;
-  }
-  const float keep_sum = shfl_t<float>(cum, keep - 1);
-  const float inv = keep_sum > 0.0f ? 1.0f / keep_sum : 0.0f;
-  const float q = pr * inv;
-  int pos = 0;
-  if (keep >= 2) {
-    const double qd = lane < keep ? static_cast<double>(q) : 0.0;
-    const double dsum = shfl_t<double>(wave_serial_prefix(qd, keep), keep - 1);
-    const double pn = qd / dsum;
-    double cp = wave_serial_prefix(pn, keep);
-    if (lane == keep - 1) cp = 1.0;
-    pos = first_lane(__ballot(lane < keep && cp >= u));
-    if (pos < 0) pos = keep - 1;
-  }
-  const uint32_t idx = key64_index(key);
-  const int32_t tok = static_cast<int32_t>(shfl_t<uint32_t>(idx, pos));
-  if (lane == 0) {
-    *out.token = tok;
-    if (out.kept_count) *out.kept_count = keep;
-  }
-  if (out.kept_ids && lane < keep && lane < out.kept_capacity) {
-    out.kept_ids[lane] = static_cast<int32_t>(idx);
-    if (out.kept_probs) out.kept_probs[lane] = q;
-  }
+__device__ __forceinline__ void store_coherent(u64* p, u64 v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ int next_pow2(int v) {
   int p = 64;
   while (p < v) p <<= 1;
   return p;
+}
+
+__device__ __forceinline__ RowOutputs row_outputs(const SampleArgs& a, int row) {
+  return RowOutputs{a.out_tokens + row, a.kept_count ? a.kept_count + row : nullptr,
+                    a.kept_ids ? a.kept_ids + static_cast<size_t>(row) * a.kept_capacity : nullptr,
+                    a.kept_probs ? a.kept_probs + static_cast<size_t>(row) * a.kept_capacity : nullptr,
+                    a.kept_capacity};
 }
 
 // Exact general path for one row, any (k, p, T), any vocabulary size: rebuilds the processed row as
@@ -130,10 +177,7 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
   const mi355x_sample_params prm = a.per_row ? a.per_row[row] : a.uniform;
   const float max_score = key_to_float(key64_okey(scratch[0]));
   const float inv_temp = 1.0f / prm.temperature;
-  RowOutputs out{a.out_tokens + row, a.kept_count ? a.kept_count + row : nullptr,
-                 a.kept_ids ? a.kept_ids + static_cast<size_t>(row) * a.kept_capacity : nullptr,
-                 a.kept_probs ? a.kept_probs + static_cast<size_t>(row) * a.kept_capacity : nullptr,
-                 a.kept_capacity};
+  const RowOutputs out = row_outputs(a, row);
   const u64* sc = scratch;
   auto sorted = [=](int i) { return sc[i]; };
   auto exps = [=](int i) { return em::expf_exact((key_to_float(key64_okey(sc[i])) - max_score) * inv_temp); };
@@ -141,8 +185,8 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
   if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
 }
 
-__device__ __forceinline__ int row_mode(mi355x_sample_params prm, int vocab) {
-  if (vocab <= 64) return kModeGeneral;
+__device__ __forceinline__ int row_mode(mi355x_sample_params prm, int vocab, int chunks) {
+  if (vocab <= 64 || chunks * kSmallCap > kAllCap) return kModeGeneral;
   if (prm.k > 1) return (prm.k < vocab ? prm.k : vocab) <= 64 ? kModeTopkSmall : kModeGeneral;
   return kModeNucleus;
 }
@@ -157,59 +201,198 @@ __device__ __forceinline__ float nucleus_depth(mi355x_sample_params prm, int voc
   return d * prm.temperature;
 }
 
-// LDS of the streaming kernel.
-struct StreamShared {
-  uint32_t hist_bits[kChunk / 32];
+constexpr uint32_t kPark = 6u;  // float4s with a hit a thread can park per chunk
+
+// LDS of the fused kernel.
+struct FusedShared {
+  uint32_t hist_bits[kSChunk / 32];
+  u64 all[kAllCap];   // merged candidates of a row (finishing workgroup only)
+  u64 sel[kSelCap];
+  float4 park_val[kSBlock * kPark];  // per-thread parking rows of the streaming filter
+  int park_idx[kSBlock * kPark];
   uint32_t pool[64];
-  u64 stage[kSmallCap];
-  u64 fin[kFinCap];
-  uint32_t count, flag, count2;
-  u64 red64[4];
-  uint32_t red32[4];
+  uint32_t wave_val[kSWaves];
+  u64 wave_val64[kSWaves];
+  uint32_t count, count2, flag, redo, bound;
   SeqShared seq;
 };
 
+__device__ __forceinline__ int elem_index(int chunk, int j, int c) {
+  return chunk * kSChunk + (j * kSBlock + static_cast<int>(threadIdx.x)) * 4 + c;
+}
+
+// A key tau such that at least k of the keys offered by the block's threads are >= tau (0 if there
+// are fewer than k offers).  One offer per thread (0 = none); only the first nw waves hold offers.
+// Every wave sorts its 64 offers and pools its best 64/nw; wave 0 sorts the pool and takes its k-th
+// entry: the exact k-th best offer unless one wave holds more than its share of the top k.
+// Two barriers; every thread gets the result.  blockDim.x == kSBlock, 1 <= k <= 64.
+__device__ __forceinline__ uint32_t block_pool_bound(uint32_t offer, int k, int nw, uint32_t* pool, uint32_t* result) {
+  const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+  if (nw < 1) nw = 1;
+  const int c = 64 / nw;
+  const uint32_t sorted = wave_sort_desc_fast<uint32_t>(offer);
+  if (wave < nw && lane < c) pool[wave * c + lane] = sorted;
+  if (tid < 64 && tid >= nw * c) pool[tid] = 0u;
+  __syncthreads();
+  if (wave == 0) {
+    const uint32_t ps = wave_sort_desc_fast<uint32_t>(pool[lane]);
+    const uint32_t tau = shfl_t<uint32_t>(ps, k - 1);
+    if (lane == 0) *result = tau;
+  }
+  __syncthreads();
+  return *result;
+}
+
+// The 32-entry table of expf_core, one entry per lane (lane & 31), fetched by lane shuffle.
+struct LaneExp2Tab {
+  uint32_t lo, hi;
+  __device__ uint64_t operator()(uint32_t i) const {
+    const uint32_t l = __shfl(lo, static_cast<int>(i), 64);
+    const uint32_t h = __shfl(hi, static_cast<int>(i), 64);
+    return (static_cast<uint64_t>(h) << 32) | l;
+  }
+};
+
+// Epilogue for k <= 64 run by one wave: lane j holds the j-th best (key64), j < m.
+// Follows ComputeSampledCategorical's top-k branch (src/sampling_distribution.h:243-281) and
+// std::discrete_distribution literally: every sum is accumulated in rank order.
+__device__ __forceinline__ void wave_topk_epilogue(u64 key, int m, mi355x_sample_params prm, double u,
+                                                   LaneExp2Tab tab, const RowOutputs& out) {
+  const int lane = lane_id();
+  m = __builtin_amdgcn_readfirstlane(m);
+  const float score = key_to_float(key64_okey(key));
+  const float max_score = shfl_t<float>(score, 0);
+  const float inv_temp = 1.0f / prm.temperature;
+  const float e_all = em::expf_core((score - max_score) * inv_temp, tab);
+  const float e = lane < m ? e_all : 0.0f;
+  const float sum = shfl_t<float>(wave_serial_prefix(e, m), m - 1);
+  const float pr = sum > 0.0f ? e / sum : e;
+  const float cum = wave_serial_prefix(pr, m);
+  int keep = m;
+  if (prm.p > 0.0f && prm.p < 1.0f) {
+    const int f = first_lane(__ballot(lane < m && cum >= prm.p));
+    if (f >= 0) keep = f + 1;
+  }
+  keep = __builtin_amdgcn_readfirstlane(keep);
+  const float keep_sum = shfl_t<float>(cum, keep - 1);
+  const float inv = keep_sum > 0.0f ? 1.0f / keep_sum : 0.0f;
+  const float q = pr * inv;
+  int pos = 0;
+  if (keep >= 2) {
+    const double qd = lane < keep ? static_cast<double>(q) : 0.0;
+    const double dsum = shfl_t<double>(wave_serial_prefix(qd, keep), keep - 1);
+    const double pn = qd / dsum;
+    double cp = wave_serial_prefix(pn, keep);
+    if (lane == keep - 1) cp = 1.0;
+    pos = first_lane(__ballot(lane < keep && cp >= u));
+    if (pos < 0) pos = keep - 1;
+  }
+  const uint32_t idx = key64_index(key);
+  const int32_t tok = static_cast<int32_t>(shfl_t<uint32_t>(idx, pos));
+  if (lane == 0) {
+    *out.token = tok;
+    if (out.kept_count) *out.kept_count = keep;
+  }
+  if (out.kept_ids && lane < keep && lane < out.kept_capacity) {
+    out.kept_ids[lane] = static_cast<int32_t>(idx);
+    if (out.kept_probs) out.kept_probs[lane] = q;
+  }
+}
+
+__device__ const uint64_t g_exp2_tab[32] = {
+    0x3ff0000000000000ULL, 0x3fefd9b0d3158574ULL, 0x3fefb5586cf9890fULL, 0x3fef9301d0125b51ULL,
+    0x3fef72b83c7d517bULL, 0x3fef54873168b9aaULL, 0x3fef387a6e756238ULL, 0x3fef1e9df51fdee1ULL,
+    0x3fef06fe0a31b715ULL, 0x3feef1a7373aa9cbULL, 0x3feedea64c123422ULL, 0x3feece086061892dULL,
+    0x3feebfdad5362a27ULL, 0x3feeb42b569d4f82ULL, 0x3feeab07dd485429ULL, 0x3feea47eb03a5585ULL,
+    0x3feea09e667f3bcdULL, 0x3fee9f75e8ec5f74ULL, 0x3feea11473eb0187ULL, 0x3feea589994cce13ULL,
+    0x3feeace5422aa0dbULL, 0x3feeb737b0cdc5e5ULL, 0x3feec49182a3f090ULL, 0x3feed503b23e255dULL,
+    0x3feee89f995ad3adULL, 0x3feeff76f2fb5e47ULL, 0x3fef199bdd85529cULL, 0x3fef3720dcef9069ULL,
+    0x3fef5818dcfba487ULL, 0x3fef7c97337b9b5fULL, 0x3fefa4afa2a490daULL, 0x3fefd0765b6e4540ULL,
+};
+
 // Streaming pass of one (row, chunk) of a top-k<=64 or nucleus row.  Returns true when this workgroup
-// must run the general path for the row (it was the last to arrive and the candidate slots overflowed).
+// must run the general path for the row (it was the last to arrive and the fast path declined).
 __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chunk, mi355x_sample_params prm,
-                                           int mode, StreamShared& sm) {
+                                           int mode, FusedShared& sm) {
   const int V = a.vocab;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const float* lrow = a.logits + static_cast<size_t>(row) * a.row_stride;
   const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
-  float v[kElems];
-  Loader<float>::load(lrow, aligned, V, chunk, v);
-  if (a.xf.active()) {
-    if (a.xf.use_penalty()) build_history_bitmap(a.xf, row, chunk * kChunk, sm.hist_bits);
-    xform_chunk<float>(a.xf, row, V, chunk, sm.hist_bits, v);
-  }
-  uint32_t keys[kElems];
-  uint32_t lmax = 0u;
+  const float kNaN = __uint_as_float(0x7fc00000u);  // marks ids >= vocab: never a maximum, never >= a bound
+  float v[kSElems];
 #pragma unroll
-  for (int e = 0; e < kElems; ++e) {
-    const int idx = Loader<float>::index_of(chunk, e / 4, e % 4);
-    keys[e] = idx < V ? order_key(v[e]) : 0u;
-    lmax = keys[e] > lmax ? keys[e] : lmax;
+  for (int j = 0; j < kSVec; ++j) {
+    const int i0 = elem_index(chunk, j, 0);
+    if (aligned && i0 + 4 <= V) {
+      const v4f q = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(lrow + i0));
+      v[j * 4 + 0] = q.x;
+      v[j * 4 + 1] = q.y;
+      v[j * 4 + 2] = q.z;
+      v[j * 4 + 3] = q.w;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) v[j * 4 + c] = (i0 + c < V) ? lrow[i0 + c] : kNaN;
+    }
   }
-  if (tid == 0) sm.count = 0u;
+  if (a.xf.active()) {
+    const bool pen = a.xf.use_penalty();
+    if (pen) {
+      for (int i = tid; i < kSChunk / 32; i += kSBlock) sm.hist_bits[i] = 0u;
+      __syncthreads();
+      const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
+      for (int i = tid; i < a.xf.history_len; i += kSBlock) {
+        const int rel = h[i] - chunk * kSChunk;
+        if (rel >= 0 && rel < kSChunk) atomicOr(&sm.hist_bits[rel >> 5], 1u << (rel & 31));
+      }
+      __syncthreads();
+    }
+    const bool has_mask = a.xf.mask != nullptr;
+    const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
+#pragma unroll
+    for (int e = 0; e < kSElems; ++e) {
+      const int idx = elem_index(chunk, e / 4, e % 4);
+      if (idx < V) {
+        const int rel = idx - chunk * kSChunk;
+        const bool hit = pen && ((sm.hist_bits[rel >> 5] >> (rel & 31)) & 1u);
+        v[e] = xform_value(v[e], a.xf, idx, has_mask ? mrow[idx >> 5] : 0u, has_mask, hit);
+      }
+    }
+  }
+  // per-thread maximum in the float domain (fmaxf skips NaN), keeping the maximum of every float4
+  float qm[kSVec];
+  float fm = -__builtin_inff();
+#pragma unroll
+  for (int j = 0; j < kSVec; ++j) {
+    qm[j] = fmaxf(fmaxf(v[j * 4], v[j * 4 + 1]), fmaxf(v[j * 4 + 2], v[j * 4 + 3]));
+    fm = fmaxf(fm, qm[j]);
+  }
+  const uint32_t lmax = elem_index(chunk, 0, 0) < V ? order_key(fm) : 0u;  // 0: thread holds no element
+  MS_STAGE(1, lmax);
+  if (tid == 0) {
+    sm.count = 0u;
+    sm.redo = 0u;
+  }
 
   if (mode == kModeNucleus) {
-    const uint32_t cmax = block_max<uint32_t>(lmax, sm.red32);  // barriers inside publish count = 0
-    uint32_t thr = 0u;
-    if (cmax != 0u) thr = order_key(key_to_float(cmax) - nucleus_depth(prm, V));
+    const uint32_t cmax = block_max<uint32_t>(lmax, sm.wave_val);  // barriers inside publish count = 0
+    float thr = -__builtin_inff();
+    if (cmax != 0u) thr = key_to_float(cmax) - nucleus_depth(prm, V);
     u64 best_below = 0;
-    u64* dst = big_row + static_cast<size_t>(chunk) * kChunk;
+    u64* dst = big_row + static_cast<size_t>(chunk) * kSChunk;
 #pragma unroll
-    for (int e = 0; e < kElems; ++e) {
-      const int idx = Loader<float>::index_of(chunk, e / 4, e % 4);
-      const u64 k64 = make_key64(keys[e], static_cast<uint32_t>(idx));
-      const bool cand = idx < V && keys[e] >= thr && keys[e] != 0u;
+    for (int e = 0; e < kSElems; ++e) {
+      const int idx = elem_index(chunk, e / 4, e % 4);
+      const bool cand = v[e] >= thr;  // false for NaN and for ids >= vocab
       const uint32_t pos = wave_slot(cand, &sm.count);
-      if (cand) dst[pos] = k64;
-      else if (idx < V) best_below = k64 > best_below ? k64 : best_below;
+      if (cand) {
+        dst[pos] = make_key64(order_key(v[e]), static_cast<uint32_t>(idx));
+      } else if (idx < V) {
+        const u64 k64 = make_key64(order_key(v[e]), static_cast<uint32_t>(idx));
+        best_below = k64 > best_below ? k64 : best_below;
+      }
     }
-    best_below = block_max<u64>(best_below, sm.red64);
+    best_below = block_max<u64>(best_below, sm.wave_val64);
     if (tid == 0) {
       const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
       a.chunk_cnt[ci] = sm.count;
@@ -219,109 +402,226 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     return false;
   }
 
-  // ---- top-k, k <= 64 ----
+  // ---- top-k, k <= 64 ---------------------------------------------------------------------------
   const int kk = prm.k < V ? prm.k : V;
-  uint32_t tau = block_kth_bound(lmax, kk, sm.pool);
-  if (tau == 0u) {
-    // The pooled bound degenerated (a short tail chunk keeps its elements in one or two waves):
-    // take the exact kk-th best of the 256 per-thread maxima instead.
-    sm.fin[tid] = static_cast<u64>(lmax);
-    __syncthreads();
-    block_sort_desc(sm.fin, kBlock);
-    tau = static_cast<uint32_t>(sm.fin[kk - 1]);
-    __syncthreads();
-  }
-#pragma unroll
-  for (int e = 0; e < kElems; ++e) {
-    const int idx = Loader<float>::index_of(chunk, e / 4, e % 4);
-    const bool cand = idx < V && keys[e] >= tau;
-    const uint32_t pos = wave_slot(cand, &sm.count);
-    if (cand && pos < kSmallCap) sm.stage[pos] = make_key64(keys[e], static_cast<uint32_t>(idx));
-  }
-  __syncthreads();
-  const uint32_t n_c = sm.count;
+  int n_valid = V - chunk * kSChunk;
+  if (n_valid > kSChunk) n_valid = kSChunk;
+  const int n_lanes = n_valid >= 4 * kSBlock ? kSBlock : (n_valid + 3) / 4;
   const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
+  u64* dst = a.cand_small + ci * kSmallCap;
+  uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool, &sm.bound);
+  if (tau == 0u) {
+    // The pooled bound found fewer than k offers (a short tail chunk keeps its elements in one or two
+    // waves): take the exact k-th best of the 256 per-thread maxima instead.
+    sm.all[tid] = static_cast<u64>(lmax);
+    __syncthreads();
+    block_sort_desc(sm.all, kSBlock);
+    tau = static_cast<uint32_t>(sm.all[kk - 1]);
+    __syncthreads();
+  }
+  MS_STAGE(2, tau);
+  // tau == 0: the chunk has fewer than k elements -- keep them all
+  const float tau_f = tau != 0u ? key_to_float(tau) : -__builtin_inff();
+  // Hits are rare (about k per chunk).  A thread parks every float4 that holds a hit in a private
+  // kPark-entry LDS row (plain writes, nothing to wait for) and counts its hits; a block-wide prefix
+  // sum of the counts then gives every thread its slots in the chunk's global segment.
+  uint32_t lc = 0u, ec = 0u;
+#pragma unroll
+  for (int j = 0; j < kSVec; ++j) {
+    if (__ballot(qm[j] >= tau_f) != 0ull) {
+      if (qm[j] >= tau_f) {
+        if (lc < kPark) {
+          sm.park_val[tid * kPark + lc] = make_float4(v[j * 4], v[j * 4 + 1], v[j * 4 + 2], v[j * 4 + 3]);
+          sm.park_idx[tid * kPark + lc] = elem_index(chunk, j, 0);
+        }
+        ++lc;
+        ec += (v[j * 4] >= tau_f) + (v[j * 4 + 1] >= tau_f) + (v[j * 4 + 2] >= tau_f) + (v[j * 4 + 3] >= tau_f);
+      }
+    }
+  }
+  uint32_t n_c;
   {
-    u64* dst = a.cand_small + ci * kSmallCap;
-    if (tid < kSmallCap && static_cast<uint32_t>(tid) < n_c) dst[tid] = sm.stage[tid];
-    if (tid == 0) a.chunk_cnt[ci] = n_c;
+    // exclusive prefix of ec inside the wave: ec < 32, so five ballots give it without lane traffic
+    uint32_t before = 0u, wtot = 0u;
+    const u64 lt = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int b = 0; b < 5; ++b) {
+      const u64 m = __ballot((ec >> b) & 1u);
+      before += static_cast<uint32_t>(__popcll(m & lt)) << b;
+      wtot += static_cast<uint32_t>(__popcll(m)) << b;
+    }
+    const u64 over = __ballot(lc > kPark);
+    if (lane == 0) sm.wave_val[wave] = wtot | (over ? 0x80000000u : 0u);
+    __syncthreads();
+    uint32_t base = 0u, tot = 0u;
+#pragma unroll
+    for (int w = 0; w < kSWaves; ++w) {
+      const uint32_t wv = sm.wave_val[w];
+      if (w < wave) base += wv & 0x7fffffffu;
+      tot += wv & 0x7fffffffu;
+      if (wv & 0x80000000u) tot = 0x40000000u;  // a thread ran out of parking rows: treat as overflow
+    }
+    n_c = tot;
+    uint32_t pos = base + before;
+    const uint32_t lim = lc < kPark ? lc : kPark;
+    for (uint32_t i = 0; i < lim; ++i) {
+      const float4 q = sm.park_val[tid * kPark + i];
+      const uint32_t id0 = static_cast<uint32_t>(sm.park_idx[tid * kPark + i]);
+      const float qv[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        if (qv[c] >= tau_f) {
+          // key64 of a real element is never 0 (its index half is ~idx != 0), so 0 marks an empty slot
+          if (pos < kSmallCap) store_coherent(&dst[pos], make_key64(order_key(qv[c]), id0 + c));
+          ++pos;
+        }
+      }
+    }
   }
-  __threadfence();
+  MS_STAGE(3, tau);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this lane's candidate stores have been performed
   __syncthreads();
+  MS_STAGE(4, tau);
   if (tid == 0) {
-    const uint32_t old = atomicAdd(&a.row_arrive[row], 1u);
-    sm.flag = (old == static_cast<uint32_t>(a.chunks) - 1u) ? 1u : 0u;
+    // low half: arrivals; high half: number of chunks whose candidates did not fit their slots
+    const uint32_t add = 1u + (n_c > kSmallCap ? 0x10000u : 0u);
+    const uint32_t old = __hip_atomic_fetch_add(&a.row_arrive[row], add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sm.flag = ((old & 0xffffu) == static_cast<uint32_t>(a.chunks) - 1u) ? (old + add) : 0u;
   }
   __syncthreads();
-  if (!sm.flag) return false;
-  __threadfence();
+  const uint32_t state = sm.flag;
+  MS_STAGE(5, state);
+  if (state == 0u) return false;
 
-  // ---- last workgroup of the row: merge the chunks' candidates ----
-  __syncthreads();
+  // ---- last workgroup of the row: merge the chunks' candidates -----------------------------------
+  // Slots are all-zero between launches; a non-zero slot is a candidate of this launch.  Read them
+  // with coherent loads, clear them for the next launch, and compact the live ones into LDS.
+  LaneExp2Tab tab;
+  {
+    const uint64_t t = g_exp2_tab[lane & 31];  // issued now, consumed by the epilogue
+    tab.lo = static_cast<uint32_t>(t);
+    tab.hi = static_cast<uint32_t>(t >> 32);
+  }
+  const double u = a.uniforms[row];
   if (tid == 0) {
-    a.row_arrive[row] = 0u;  // ready for the next launch
+    a.row_arrive[row] = 0u;
     sm.count = 0u;
     sm.count2 = 0u;
-    sm.flag = 0u;
   }
   __syncthreads();
   const int slots = a.chunks * kSmallCap;
-  for (int p = tid; p < slots; p += kBlock) {
-    const int ch = p / kSmallCap, sl = p % kSmallCap;
-    const uint32_t cnt = load_coherent(&a.chunk_cnt[static_cast<size_t>(row) * a.chunks + ch]);
-    if (cnt > kSmallCap) sm.flag = 1u;  // a chunk overflowed its slots
-    if (static_cast<uint32_t>(sl) < cnt) {
-      const u64 k64 = load_coherent(&a.cand_small[(static_cast<size_t>(row) * a.chunks + ch) * kSmallCap + sl]);
-      const uint32_t pos = atomicAdd(&sm.count, 1u);
-      if (pos < kFinCap) sm.fin[pos] = k64;
+  u64* seg = a.cand_small + static_cast<size_t>(row) * a.chunks * kSmallCap;
+  for (int p0 = 0; p0 < slots; p0 += kSBlock * 8) {
+    u64 k64[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int p = p0 + r * kSBlock + tid;
+      k64[r] = p < slots ? load_coherent(&seg[p]) : 0;
+    }
+    // one LDS atomic per wave for all 8 registers
+    uint32_t before[8];
+    uint32_t wave_total = 0u;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const u64 b = __ballot(k64[r] != 0);
+      before[r] = wave_total + static_cast<uint32_t>(__popcll(b & ((1ull << lane) - 1ull)));
+      wave_total += static_cast<uint32_t>(__popcll(b));
+    }
+    uint32_t base = 0u;
+    if (lane == 0 && wave_total != 0u) base = atomicAdd(&sm.count, wave_total);
+    base = __builtin_amdgcn_readfirstlane(base);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      if (k64[r] != 0) {
+        sm.all[base + before[r]] = k64[r];
+        seg[p0 + r * kSBlock + tid] = 0;
+      }
     }
   }
   __syncthreads();
-  const uint32_t total = sm.count;
-  if (sm.flag || total > kFinCap) return true;
-  RowOutputs out{a.out_tokens + row, a.kept_count ? a.kept_count + row : nullptr,
-                 a.kept_ids ? a.kept_ids + static_cast<size_t>(row) * a.kept_capacity : nullptr,
-                 a.kept_probs ? a.kept_probs + static_cast<size_t>(row) * a.kept_capacity : nullptr,
-                 a.kept_capacity};
-  // second-level bound over the merged candidates
-  uint32_t lm2 = 0u;
-  for (uint32_t p = tid; p < total; p += kBlock) {
-    const uint32_t ok = key64_okey(sm.fin[p]);
-    lm2 = ok > lm2 ? ok : lm2;
-  }
-  const uint32_t tau2 = block_kth_bound(lm2, kk, sm.pool);
-  u64* sel = sm.stage;  // reuse: up to 64 survivors
-  for (uint32_t p = tid; p < total; p += kBlock) {
-    const u64 k64 = sm.fin[p];
-    if (key64_okey(k64) >= tau2) {
-      const uint32_t pos = atomicAdd(&sm.count2, 1u);
-      if (pos < 64u) sel[pos] = k64;
+  MS_STAGE(6, sm.count);
+  const int total = static_cast<int>(sm.count);
+  if ((state >> 16) != 0u || total < kk) return true;  // slots overflowed, or NaNs are needed to fill k
+  u64 final_key = 0;
+  if (total <= 64) {
+    if (tid < 64) final_key = tid < total ? sm.all[tid] : 0;
+  } else {
+    // Typical rows merge ~450 candidates (two registers per thread); the loops are bounded by the
+    // number of registers actually needed.
+    constexpr int kRegs = kAllCap / kSBlock;
+    const int nreg = (total + kSBlock - 1) / kSBlock;
+    u64 mine[kRegs];
+    uint32_t mk = 0u;
+#pragma unroll
+    for (int r = 0; r < kRegs; ++r) {
+      mine[r] = 0;
+      if (r < nreg) {
+        const int p = r * kSBlock + tid;
+        mine[r] = p < total ? sm.all[p] : 0;
+        const uint32_t ok = key64_okey(mine[r]);
+        mk = ok > mk ? ok : mk;
+      }
     }
-  }
-  __syncthreads();
-  const uint32_t n_sel = sm.count2;
-  if (n_sel > 64u) {
-    // too many survivors (ties at the bound): sort all merged candidates in LDS instead
-    const int n2 = next_pow2(static_cast<int>(total));
-    for (int p = static_cast<int>(total) + tid; p < n2; p += kBlock) sm.fin[p] = 0;
+    const int nw2 = total >= kSBlock ? kSWaves : (total + 63) / 64;
+    const uint32_t tau2 = block_pool_bound(mk, kk, nw2, sm.pool, &sm.bound);
+#pragma unroll
+    for (int r = 0; r < kRegs; ++r) {
+      if (r < nreg) {
+        const bool cand = mine[r] != 0 && key64_okey(mine[r]) >= tau2;
+        const uint32_t pos = wave_slot(cand, &sm.count2);
+        if (cand && pos < kSelCap) sm.sel[pos] = mine[r];
+      }
+    }
     __syncthreads();
-    block_sort_desc(sm.fin, n2);
-    if (tid < 64) wave_topk_epilogue(tid < kk ? sm.fin[tid] : 0, kk, prm, a.uniforms[row], out);
-    return false;
+    const uint32_t n_sel = sm.count2;
+    MS_STAGE(7, n_sel);
+    if (n_sel > kSelCap) return true;  // heavy ties at the bound
+    if (tid < 64) {
+      uint32_t sk[kSelCap / 64];
+      u64 sk64[kSelCap / 64];
+#pragma unroll
+      for (int r = 0; r < kSelCap / 64; ++r) {
+        const uint32_t p = r * 64 + lane;
+        sk64[r] = p < n_sel ? sm.sel[p] : 0;
+        sk[r] = key64_okey(sk64[r]);
+      }
+      if (n_sel <= 64u) {
+        final_key = sk64[0];
+      } else {
+        // exact k-th best score among the survivors, then one key per lane
+        const uint32_t tau3 = wave_kth_largest<kSelCap / 64>(sk, kk);
+        int base = 0;
+#pragma unroll
+        for (int r = 0; r < kSelCap / 64; ++r) {
+          const bool in = sk64[r] != 0 && sk[r] >= tau3;
+          const u64 b = __ballot(in);
+          const int dl = base + __popcll(b & ((1ull << lane) - 1ull));
+          if (in && dl < 64) sm.sel[dl] = sk64[r];
+          base += __popcll(b);
+        }
+        if (base > 64) {
+          if (lane == 0) sm.redo = 1u;  // more than 64 keys tie with the k-th best: exact path decides
+        } else {
+          final_key = lane < base ? sm.sel[lane] : 0;
+        }
+      }
+    }
   }
-  if (tid < 64) {
-    u64 k64 = static_cast<uint32_t>(tid) < n_sel ? sel[tid] : 0;
-    k64 = wave_sort_desc<u64>(k64);
-    wave_topk_epilogue(k64, kk, prm, a.uniforms[row], out);
+  MS_STAGE(8, (uint32_t)final_key);
+  if (tid < 64 && sm.redo == 0u) {
+    final_key = wave_sort_desc_fast<u64>(final_key);
+    MS_STAGE(9, (uint32_t)final_key);
+    wave_topk_epilogue(final_key, kk, prm, u, tab, row_outputs(a, row));
   }
-  return false;
+  __syncthreads();
+  return sm.redo != 0u;
 }
 
-__global__ __launch_bounds__(kBlock) void sample_stream_kernel(const SampleArgs a) {
+__global__ __launch_bounds__(kSBlock) void sample_fused_kernel(const SampleArgs a) {
   const int row = blockIdx.y, chunk = blockIdx.x;
-  __shared__ StreamShared sm;
+  __shared__ FusedShared sm;
   const mi355x_sample_params prm = a.per_row ? a.per_row[row] : a.uniform;
-  const int mode = row_mode(prm, a.vocab);
+  const int mode = row_mode(prm, a.vocab, a.chunks);
   if (mode == kModeGeneral) {
     if (chunk != 0) return;
   } else if (!stream_row(a, row, chunk, prm, mode, sm)) {
@@ -346,7 +646,7 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const Samp
   const int V = a.vocab;
   const int tid = threadIdx.x;
   const mi355x_sample_params prm = a.per_row ? a.per_row[row] : a.uniform;
-  if (row_mode(prm, V) != kModeNucleus) return;
+  if (row_mode(prm, V, a.chunks) != kModeNucleus) return;
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
   uint32_t m = 0u;
@@ -359,7 +659,7 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const Samp
   for (int c = tid; c < a.chunks; c += blockDim.x) best_below = a.chunk_next[cbase + c] > best_below ? a.chunk_next[cbase + c] : best_below;
   for (int c = 0; c < a.chunks; ++c) {
     const uint32_t cnt = a.chunk_cnt[cbase + c];
-    const u64* src = big_row + static_cast<size_t>(c) * kChunk;
+    const u64* src = big_row + static_cast<size_t>(c) * kSChunk;
     for (uint32_t i0 = 0; i0 < cnt; i0 += blockDim.x) {
       const uint32_t i = i0 + tid;
       const u64 k64 = i < cnt ? src[i] : 0;
@@ -392,14 +692,10 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const Samp
       lds_keys[i] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k64 & 0xffffffffull);
     }
     __syncthreads();
-    RowOutputs out{a.out_tokens + row, a.kept_count ? a.kept_count + row : nullptr,
-                   a.kept_ids ? a.kept_ids + static_cast<size_t>(row) * a.kept_capacity : nullptr,
-                   a.kept_probs ? a.kept_probs + static_cast<size_t>(row) * a.kept_capacity : nullptr,
-                   a.kept_capacity};
     const u64* lk = lds_keys;
     auto sorted = [=](int i) { return lk[i]; };
     auto exps = [=](int i) { return __uint_as_float(static_cast<uint32_t>(lk[i] >> 32)); };
-    ok = block_sample_epilogue<4>(sorted, exps, static_cast<int>(n_c), V, prm, a.uniforms[row], out, seqsh);
+    ok = block_sample_epilogue<4>(sorted, exps, static_cast<int>(n_c), V, prm, a.uniforms[row], row_outputs(a, row), seqsh);
   }
   if (!ok) {
     __syncthreads();
@@ -411,7 +707,7 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const Samp
 
 extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, bool any_nucleus, hipStream_t stream) {
   dim3 grid(a->chunks, a->rows);
-  hipLaunchKernelGGL(ms::sample_stream_kernel, grid, dim3(ms::kBlock), 0, stream, *a);
+  hipLaunchKernelGGL(ms::sample_fused_kernel, grid, dim3(ms::kSBlock), 0, stream, *a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (any_nucleus) {
