@@ -9,6 +9,7 @@
 // (k > 64, heavy ties, tiny vocabularies) goes through general_row, an exact full sort.
 #include "kernels.h"
 #include "block_seq.h"
+#include "wave_select.h"
 
 namespace ms {
 
@@ -19,73 +20,6 @@ namespace ms {
 #endif
 
 typedef float v4f __attribute__((ext_vector_type(4)));
-
-// ---- lane exchange primitives ---------------------------------------------------------------------
-template <int M>
-__device__ __forceinline__ uint32_t lane_xor(uint32_t x) {
-  if constexpr (M == 1) {
-    return __builtin_amdgcn_mov_dpp(x, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
-  } else if constexpr (M == 2) {
-    return __builtin_amdgcn_mov_dpp(x, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
-  } else if constexpr (M == 4) {
-    return __builtin_amdgcn_ds_swizzle(x, (4 << 10) | 0x1f);   // bit-mask mode, xor 4
-  } else if constexpr (M == 8) {
-    return __builtin_amdgcn_mov_dpp(x, 0x128, 0xf, 0xf, true);  // row_ror:8 == xor 8 inside a row of 16
-  } else if constexpr (M == 16) {
-    const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
-    return (lane_id() & 16) ? r[0] : r[1];
-  } else {
-    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
-    return (lane_id() & 32) ? r[0] : r[1];
-  }
-}
-
-template <int M>
-__device__ __forceinline__ u64 lane_xor64(u64 x) {
-  const uint32_t lo = lane_xor<M>(static_cast<uint32_t>(x));
-  const uint32_t hi = lane_xor<M>(static_cast<uint32_t>(x >> 32));
-  return (static_cast<u64>(hi) << 32) | lo;
-}
-__device__ __forceinline__ uint32_t lane_xor_any(uint32_t x, int m) { return __shfl_xor(x, m, 64); }
-
-template <int K, int J, typename T>
-__device__ __forceinline__ void sort_merge(T& x, int lane) {
-  T y;
-  if constexpr (sizeof(T) == 8) y = lane_xor64<J>(x);
-  else y = lane_xor<J>(x);
-  const bool keep_max = (((lane & K) == 0) == ((lane & J) == 0));
-  x = ((y > x) == keep_max) ? y : x;
-  if constexpr (J > 1) sort_merge<K, J / 2, T>(x, lane);
-}
-
-// Bitonic sort of one key per lane, descending by lane (lane 0 ends with the maximum).
-template <typename T>
-__device__ __forceinline__ T wave_sort_desc_fast(T x) {
-  const int lane = lane_id();
-  sort_merge<2, 1, T>(x, lane);
-  sort_merge<4, 2, T>(x, lane);
-  sort_merge<8, 4, T>(x, lane);
-  sort_merge<16, 8, T>(x, lane);
-  sort_merge<32, 16, T>(x, lane);
-  sort_merge<64, 32, T>(x, lane);
-  return x;
-}
-
-// k-th largest of the wave's R keys per lane (0 if fewer than k keys are non-zero): bisection on the
-// key bits with wave-wide population counts.
-template <int R>
-__device__ __forceinline__ uint32_t wave_kth_largest(const uint32_t (&key)[R], int k) {
-  uint32_t prefix = 0u;
-#pragma unroll 1
-  for (int bit = 31; bit >= 0; --bit) {
-    const uint32_t cand = prefix | (1u << bit);
-    int cnt = 0;
-#pragma unroll
-    for (int r = 0; r < R; ++r) cnt += __popcll(__ballot(key[r] >= cand));
-    if (cnt >= k) prefix = cand;
-  }
-  return prefix;
-}
 
 // Serial prefix over lanes: out[l] = ((x[0] + x[1]) + ...) + x[l], additions in lane order, as the
 // reference's scalar loops do.  One DPP-shifted add per element (wave_shr:1, lane 0 reads 0).
@@ -108,25 +42,6 @@ __device__ __forceinline__ double wave_serial_prefix(double x, int count) {
     s = prev + x;
   }
   return s;
-}
-
-// Slot allocation from a shared counter with one atomic per wave.  Must be reached by every lane of
-// the wave; lanes with pred == false get an unspecified value.
-__device__ __forceinline__ uint32_t wave_slot(bool pred, uint32_t* counter) {
-  const u64 b = __ballot(pred);
-  if (b == 0) return 0u;
-  const int lane = lane_id();
-  const int leader = __ffsll(static_cast<long long>(b)) - 1;
-  uint32_t base = 0u;
-  if (lane == leader) base = atomicAdd(counter, static_cast<uint32_t>(__popcll(b)));
-  base = __shfl(base, leader, 64);
-  return base + static_cast<uint32_t>(__popcll(b & ((1ull << lane) - 1ull)));
-}
-
-__device__ __forceinline__ int first_lane(u64 ballot) { return ballot ? __ffsll(static_cast<long long>(ballot)) - 1 : -1; }
-
-__device__ __forceinline__ void store_coherent(u64* p, u64 v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ int next_pow2(int v) {
@@ -219,28 +134,6 @@ struct FusedShared {
 
 __device__ __forceinline__ int elem_index(int chunk, int j, int c) {
   return chunk * kSChunk + (j * kSBlock + static_cast<int>(threadIdx.x)) * 4 + c;
-}
-
-// A key tau such that at least k of the keys offered by the block's threads are >= tau (0 if there
-// are fewer than k offers).  One offer per thread (0 = none); only the first nw waves hold offers.
-// Every wave sorts its 64 offers and pools its best 64/nw; wave 0 sorts the pool and takes its k-th
-// entry: the exact k-th best offer unless one wave holds more than its share of the top k.
-// Two barriers; every thread gets the result.  blockDim.x == kSBlock, 1 <= k <= 64.
-__device__ __forceinline__ uint32_t block_pool_bound(uint32_t offer, int k, int nw, uint32_t* pool, uint32_t* result) {
-  const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
-  if (nw < 1) nw = 1;
-  const int c = 64 / nw;
-  const uint32_t sorted = wave_sort_desc_fast<uint32_t>(offer);
-  if (wave < nw && lane < c) pool[wave * c + lane] = sorted;
-  if (tid < 64 && tid >= nw * c) pool[tid] = 0u;
-  __syncthreads();
-  if (wave == 0) {
-    const uint32_t ps = wave_sort_desc_fast<uint32_t>(pool[lane]);
-    const uint32_t tau = shfl_t<uint32_t>(ps, k - 1);
-    if (lane == 0) *result = tau;
-  }
-  __syncthreads();
-  return *result;
 }
 
 // The 32-entry table of expf_core, one entry per lane (lane & 31), fetched by lane shuffle.
