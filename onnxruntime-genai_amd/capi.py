@@ -181,5 +181,155 @@ class SearchContext:
         return out
 
 
+
+
+_hip_lib = None
+
+
+def _hip():
+    """The HIP runtime torch already loaded (device-to-device copies of library-owned buffers)."""
+    global _hip_lib
+    if _hip_lib is None:
+        _hip_lib = C.CDLL("libamdhip64.so")
+        _hip_lib.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        _hip_lib.hipMemcpy.restype = C.c_int
+    return _hip_lib
+
+
+def _dtype_code(t):
+    return {torch.float32: MI355X_F32, torch.float16: MI355X_F16}[t.dtype]
+
+
+def _topk_scores(self, logits, k):
+    rows, vocab, stride = self._rows(logits)
+    tok = torch.empty((rows, k), dtype=torch.int32, device=logits.device)
+    sc = torch.empty((rows, k), dtype=torch.float32, device=logits.device)
+    self._check(self.L.mi355x_topk_scores(self.h, _stream(), logits.data_ptr(), _dtype_code(logits), stride, rows,
+                                          vocab, k, tok.data_ptr(), sc.data_ptr()))
+    return tok, sc
+
+
+def _softmax(self, scores, temperature=1.0, log=False):
+    rows, vocab, stride = self._rows(scores)
+    assert scores.dtype == torch.float32
+    self._check(self.L.mi355x_softmax(self.h, _stream(), scores.data_ptr(), stride, rows, vocab, temperature, int(log)))
+    return scores
+
+
+def _beam_select(self, logits, batch, beams, beam_scores):
+    rows, vocab, stride = self._rows(logits)
+    assert rows == batch * beams and beam_scores.dtype == torch.float32 and beam_scores.numel() == rows
+    k = 2 * beams
+    sc = torch.empty((batch, k), dtype=torch.float32, device=logits.device)
+    tok = torch.empty((batch, k), dtype=torch.int32, device=logits.device)
+    idx = torch.empty((batch, k), dtype=torch.int32, device=logits.device)
+    self._check(self.L.mi355x_beam_select(self.h, _stream(), logits.data_ptr(), _dtype_code(logits), stride, batch,
+                                          beams, vocab, beam_scores.data_ptr(), sc.data_ptr(), tok.data_ptr(),
+                                          idx.data_ptr()))
+    return sc, tok, idx
+
+
+def _kv_gather(self, present, past, beam_indices):
+    """present/past: lists of equally shaped contiguous CUDA tensors [rows, ...]; past[t][j] = present[t][idx[j]]."""
+    n = len(present)
+    assert n == len(past) and beam_indices.dtype == torch.int32
+    block = present[0][0].numel() * present[0].element_size()
+    for a, b in zip(present, past):
+        assert a.is_contiguous() and b.is_contiguous() and a[0].numel() * a.element_size() == block
+    pp = (C.c_void_p * n)(*[t.data_ptr() for t in present])
+    qq = (C.c_void_p * n)(*[t.data_ptr() for t in past])
+    self._check(self.L.mi355x_kv_gather(self.h, _stream(), pp, qq, n, beam_indices.data_ptr(), beam_indices.numel(),
+                                        block))
+    return past
+
+
+def _spec_verify(self, p_target, p_draft, draft_tokens, accept_u, sample_u):
+    b, k1, v = p_target.shape
+    for t in (p_target, p_draft, draft_tokens, accept_u, sample_u):
+        assert t.is_cuda and t.is_contiguous()
+    assert p_target.dtype == torch.float32 and accept_u.dtype == torch.float32 and sample_u.dtype == torch.float64
+    acc = torch.empty(b, dtype=torch.int32, device=p_target.device)
+    tok = torch.empty(b, dtype=torch.int32, device=p_target.device)
+    self._check(self.L.mi355x_spec_verify(self.h, _stream(), p_target.data_ptr(), p_draft.data_ptr(),
+                                          draft_tokens.data_ptr(), accept_u.data_ptr(), sample_u.data_ptr(), b, k1 - 1,
+                                          v, acc.data_ptr(), tok.data_ptr()))
+    return acc, tok
+
+
+SearchContext.topk_scores = _topk_scores
+SearchContext.softmax = _softmax
+SearchContext.beam_select = _beam_select
+SearchContext.kv_gather = _kv_gather
+SearchContext.spec_verify = _spec_verify
+
+
 class BeamScorer:
-    pass
+    """Device-resident BeamSearchScorer + Sequences (mi355x_beam_scorer)."""
+
+    def __init__(self, ctx, batch, beams, max_length, pad, eos, length_penalty=1.0, early_stopping=True):
+        self.ctx, self.L = ctx, ctx.L
+        self.batch, self.beams, self.max_length = batch, beams, max_length
+        e = (C.c_int32 * max(1, len(eos)))(*eos)
+        h = C.c_void_p()
+        ctx._check(self.L.mi355x_beam_scorer_create(ctx.h, batch, beams, max_length, pad, e, len(eos),
+                                                    length_penalty, int(early_stopping), C.byref(h)))
+        self.h = h
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.L.mi355x_beam_scorer_destroy(self.h)
+            self.h = None
+
+    __del__ = close
+
+    def set_prompt(self, tokens):
+        import numpy as np
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        assert t.shape[0] == self.batch
+        self.ctx._check(self.L.mi355x_beam_scorer_set_prompt(self.h, _stream(), t.ctypes.data_as(C.POINTER(C.c_int32)),
+                                                             t.shape[1]))
+
+    def step(self, cand_scores, cand_tokens, cand_indices):
+        self.ctx._check(self.L.mi355x_beam_scorer_step(self.h, _stream(), cand_scores.data_ptr(),
+                                                       cand_tokens.data_ptr(), cand_indices.data_ptr()))
+
+    def _copy(self, ptr, dtype, count):
+        out = torch.empty(count, dtype=dtype, device=self.ctx.device)
+        torch.cuda.current_stream().synchronize()
+        rc = _hip().hipMemcpy(C.c_void_p(out.data_ptr()), C.c_void_p(ptr), C.c_size_t(count * out.element_size()), 3)
+        assert rc == 0, f"hipMemcpy failed: {rc}"
+        return out
+
+    @property
+    def next_scores(self):
+        return self._copy(self.L.mi355x_beam_scorer_next_scores(self.h), torch.float32, self.batch * self.beams)
+
+    @property
+    def next_tokens(self):
+        return self._copy(self.L.mi355x_beam_scorer_next_tokens(self.h), torch.int32, self.batch * self.beams)
+
+    @property
+    def next_indices(self):
+        return self._copy(self.L.mi355x_beam_scorer_next_indices(self.h), torch.int32, self.batch * self.beams)
+
+    def next_scores_ptr(self):
+        return self.L.mi355x_beam_scorer_next_scores(self.h)
+
+    def sequences(self):
+        n = C.c_int()
+        p = self.L.mi355x_beam_scorer_sequences(self.h, C.byref(n))
+        full = self._copy(p, torch.int32, self.batch * self.beams * self.max_length)
+        return full.view(self.batch * self.beams, self.max_length)[:, :n.value], n.value
+
+    def is_done(self):
+        d = C.c_int()
+        self.ctx._check(self.L.mi355x_beam_scorer_is_done(self.h, _stream(), C.byref(d)))
+        return bool(d.value)
+
+    def hypothesis(self, batch, index):
+        buf = (C.c_int32 * self.max_length)()
+        n = C.c_int()
+        sc = C.c_float()
+        self.ctx._check(self.L.mi355x_beam_scorer_hypothesis(self.h, _stream(), batch, index, buf, self.max_length,
+                                                             C.byref(n), C.byref(sc)))
+        return list(buf[:n.value]), sc.value

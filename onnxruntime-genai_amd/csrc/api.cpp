@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <cstdarg>
 #include <cstdio>
+#include <cmath>
 #include <cstring>
 #include <cstdlib>
 #include <new>
@@ -57,6 +58,10 @@ struct mi355x_search_ctx {
   mi355x_sample_params* params_dev{};
   void** ptr_table{};      // device copy of pointer tables (kv gather)
   size_t ptr_table_cap{};
+  float* beam_row_scores{};
+  int32_t* beam_row_tokens{};
+  float* widen{};          // fp32 copy of fp16 rows (top-k scores), grown on demand
+  size_t widen_elems{};
 
   template <typename T>
   hipError_t Alloc(T** p, size_t count, bool zero) {
@@ -149,6 +154,8 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->big, static_cast<size_t>(max_rows) * c->big_stride, false));
   ok(c->Alloc(&c->fallback_rows, 1, true));
   ok(c->Alloc(&c->params_dev, static_cast<size_t>(max_rows), false));
+  ok(c->Alloc(&c->beam_row_scores, static_cast<size_t>(max_rows) * ms::kBeamMaxCand, false));
+  ok(c->Alloc(&c->beam_row_tokens, static_cast<size_t>(max_rows) * ms::kBeamMaxCand, false));
   c->ptr_table_cap = 4096;
   ok(c->Alloc(&c->ptr_table, c->ptr_table_cap, false));
   if (e == hipSuccess) e = ms_sample_init();
@@ -164,6 +171,7 @@ void mi355x_search_destroy(mi355x_search_ctx* ctx) {
   if (!ctx) return;
   (void)hipSetDevice(ctx->device);
   for (void* p : ctx->allocs) (void)hipFree(p);
+  if (ctx->widen) (void)hipFree(ctx->widen);
   delete ctx;
 }
 
@@ -255,11 +263,287 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   return MI355X_OK;
 }
 
+int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype, int64_t row_stride,
+                       int rows, int vocab, int k, int32_t* out_tokens, float* out_scores) {
+  if (int r = CheckRows(ctx, rows, vocab)) return r;
+  if (!logits || !out_tokens || !out_scores) return Fail(MI355X_E_INVALID, "null logits or output");
+  if (dtype != MI355X_F32 && dtype != MI355X_F16) return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
+  if (k < 1 || k > 64 || k > vocab) return Fail(MI355X_E_INVALID, "k (%d) must be in [1, min(64, vocab)]", k);
+  if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float* src = static_cast<const float*>(logits);
+  if (dtype == MI355X_F16) {
+    // widened once into an fp32 scratch, as DeviceInterface::TopKScores does (src/cuda/interface.cpp:440-451)
+    const size_t need = static_cast<size_t>(rows) * vocab;
+    if (need > ctx->widen_elems) {
+      HIP_TRY(hipStreamSynchronize(s));
+      if (ctx->widen) (void)hipFree(ctx->widen);
+      ctx->widen = nullptr;
+      ctx->widen_elems = 0;
+      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&ctx->widen), need * sizeof(float)));
+      ctx->widen_elems = need;
+    }
+    HIP_TRY(ms_launch_widen_f16(logits, row_stride, ctx->widen, vocab, rows, vocab, s));
+    src = ctx->widen;
+    row_stride = vocab;
+  }
+  ms::SampleArgs a{};
+  if (int r = MakeXform(nullptr, &a.xf)) return r;
+  a.logits = src;
+  a.row_stride = row_stride;
+  a.rows = rows;
+  a.vocab = vocab;
+  a.chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
+  a.uniform = mi355x_sample_params{k, 0.0f, 1.0f};
+  a.out_tokens = out_tokens;
+  a.out_scores = out_scores;
+  a.emit_topk = 1;
+  a.cand_small = ctx->cand_small;
+  a.chunk_cnt = ctx->chunk_cnt;
+  a.chunk_max = ctx->chunk_max;
+  a.chunk_next = ctx->chunk_next;
+  a.row_arrive = ctx->row_arrive;
+  a.big = ctx->big;
+  a.big_stride = ctx->big_stride;
+  a.fallback_rows = ctx->fallback_rows;
+  HIP_TRY(ms_launch_sample(&a, false, s));
+  return MI355X_OK;
+}
+
+int mi355x_softmax(mi355x_search_ctx* ctx, void* stream, float* scores, int64_t row_stride, int rows, int vocab,
+                   float temperature, int log_softmax) {
+  if (!ctx) return Fail(MI355X_E_INVALID, "null context");
+  if (!scores || rows <= 0 || vocab <= 0) return Fail(MI355X_E_INVALID, "null scores or non-positive size");
+  if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
+  if (!(temperature > 0.0f)) return Fail(MI355X_E_INVALID, "temperature must be positive (got %g)", temperature);
+  HIP_TRY(ms_launch_softmax(scores, row_stride, rows, vocab, temperature, log_softmax, static_cast<hipStream_t>(stream)));
+  return MI355X_OK;
+}
+
+int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype, int64_t row_stride,
+                       int batch, int beams, int vocab, const float* beam_scores, float* out_scores,
+                       int32_t* out_tokens, int32_t* out_beam_indices) {
+  if (batch <= 0 || beams <= 0) return Fail(MI355X_E_INVALID, "batch and beams must be positive");
+  if (beams > ms::kBeamMaxCand / 2) return Fail(MI355X_E_UNSUPPORTED, "beams (%d) above the supported %d", beams, ms::kBeamMaxCand / 2);
+  if (int r = CheckRows(ctx, batch * beams, vocab)) return r;
+  if (!logits || !beam_scores || !out_scores || !out_tokens || !out_beam_indices)
+    return Fail(MI355X_E_INVALID, "null argument");
+  if (dtype != MI355X_F32 && dtype != MI355X_F16) return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
+  if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
+  if (static_cast<long long>(beams) * vocab < 2LL * beams)
+    return Fail(MI355X_E_INVALID, "beam search requires num_beams * vocab_size (%lld) >= 2 * num_beams (%d)",
+                static_cast<long long>(beams) * vocab, 2 * beams);
+  if (static_cast<unsigned long long>(beams) * static_cast<unsigned long long>(vocab) > 0xffffffffull)
+    return Fail(MI355X_E_UNSUPPORTED, "beams * vocab exceeds 2^32");
+  ms::BeamArgs a{};
+  a.logits = logits;
+  a.row_stride = row_stride;
+  a.batch = batch;
+  a.beams = beams;
+  a.vocab = vocab;
+  a.beam_scores = beam_scores;
+  a.row_scores = ctx->beam_row_scores;
+  a.row_tokens = ctx->beam_row_tokens;
+  a.out_scores = out_scores;
+  a.out_tokens = out_tokens;
+  a.out_beams = out_beam_indices;
+  HIP_TRY(ms_launch_beam_select(&a, dtype, static_cast<hipStream_t>(stream)));
+  return MI355X_OK;
+}
+
+int mi355x_kv_gather(mi355x_search_ctx* ctx, void* stream, const void* const* present, void* const* past,
+                     int n_tensors, const int32_t* beam_indices, int rows, size_t block_bytes) {
+  if (!ctx || !present || !past || !beam_indices) return Fail(MI355X_E_INVALID, "null argument");
+  if (n_tensors <= 0 || rows <= 0 || block_bytes == 0) return Fail(MI355X_E_INVALID, "non-positive size");
+  if (block_bytes % 16 != 0) return Fail(MI355X_E_INVALID, "block_bytes (%zu) must be a multiple of 16", block_bytes);
+  if (static_cast<size_t>(n_tensors) * 2 > ctx->ptr_table_cap || n_tensors > 65535 || rows > 65535)
+    return Fail(MI355X_E_CAPACITY, "too many tensors (%d) or rows (%d)", n_tensors, rows);
+  for (int t = 0; t < n_tensors; ++t) {
+    if (!present[t] || !past[t]) return Fail(MI355X_E_INVALID, "null tensor pointer at %d", t);
+    if ((reinterpret_cast<uintptr_t>(present[t]) | reinterpret_cast<uintptr_t>(past[t])) & 15u)
+      return Fail(MI355X_E_INVALID, "tensor %d is not 16-byte aligned", t);
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  HIP_TRY(hipMemcpyAsync(ctx->ptr_table, present, sizeof(void*) * n_tensors, hipMemcpyHostToDevice, s));
+  HIP_TRY(hipMemcpyAsync(ctx->ptr_table + n_tensors, past, sizeof(void*) * n_tensors, hipMemcpyHostToDevice, s));
+  HIP_TRY(ms_launch_kv_gather(ctx->ptr_table, ctx->ptr_table + n_tensors, n_tensors, beam_indices, rows, block_bytes, s));
+  return MI355X_OK;
+}
+
+int mi355x_spec_verify(mi355x_search_ctx* ctx, void* stream, const float* p_target, const float* p_draft,
+                       const int32_t* draft_tokens, const float* accept_u, const double* sample_u, int batch, int K,
+                       int vocab, int32_t* accepted_len, int32_t* final_token) {
+  if (!ctx || !p_target || !p_draft || !draft_tokens || !accept_u || !sample_u || !accepted_len || !final_token)
+    return Fail(MI355X_E_INVALID, "null argument");
+  if (batch <= 0 || K <= 0 || vocab < 2) return Fail(MI355X_E_INVALID, "batch, K must be positive and vocab >= 2");
+  HIP_TRY(ms_launch_spec_verify(p_target, p_draft, draft_tokens, accept_u, sample_u, batch, K, vocab, accepted_len,
+                                final_token, static_cast<hipStream_t>(stream)));
+  return MI355X_OK;
+}
+
 int mi355x_search_fallback_rows(mi355x_search_ctx* ctx, void* stream, unsigned* rows) {
   if (!ctx || !rows) return Fail(MI355X_E_INVALID, "null argument");
   HIP_TRY(hipMemcpyAsync(rows, ctx->fallback_rows, sizeof(unsigned), hipMemcpyDeviceToHost,
                          static_cast<hipStream_t>(stream)));
   HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return MI355X_OK;
+}
+
+// ---- device-resident beam scorer ---------------------------------------------------------------------
+struct mi355x_beam_scorer {
+  mi355x_search_ctx* ctx{};
+  ms::ScorerState st{};
+  std::vector<void*> allocs;
+  int32_t* seq[2]{};
+  int cur{};
+  int length{};
+  bool finalized{};
+  float* pow_dev{};
+};
+
+int mi355x_beam_scorer_create(mi355x_search_ctx* ctx, int batch, int beams, int max_length, int pad_token_id,
+                              const int32_t* eos_ids, int n_eos, float length_penalty, int early_stopping,
+                              mi355x_beam_scorer** out) {
+  if (!ctx || !out) return Fail(MI355X_E_INVALID, "null argument");
+  *out = nullptr;
+  if (batch <= 0 || beams <= 1 || max_length <= 0) return Fail(MI355X_E_INVALID, "batch, max_length must be positive and beams > 1");
+  if (beams > ms::kBeamMaxCand / 2) return Fail(MI355X_E_UNSUPPORTED, "beams (%d) above the supported %d", beams, ms::kBeamMaxCand / 2);
+  if (n_eos < 0 || n_eos > MI355X_MAX_EOS || (n_eos > 0 && !eos_ids)) return Fail(MI355X_E_INVALID, "bad eos list");
+  HIP_TRY(hipSetDevice(ctx->device));
+  auto* s = new (std::nothrow) mi355x_beam_scorer;
+  if (!s) return Fail(MI355X_E_INVALID, "out of host memory");
+  s->ctx = ctx;
+  const size_t bb = static_cast<size_t>(batch) * beams;
+  hipError_t e = hipSuccess;
+  auto alloc = [&](void** p, size_t bytes) {
+    if (e != hipSuccess) return;
+    e = hipMalloc(p, bytes ? bytes : 16);
+    if (e == hipSuccess) {
+      s->allocs.push_back(*p);
+      e = hipMemset(*p, 0, bytes ? bytes : 16);
+    }
+  };
+  ms::ScorerState& st = s->st;
+  st.batch = batch;
+  st.beams = beams;
+  st.max_length = max_length;
+  st.pad = pad_token_id;
+  st.early_stopping = early_stopping != 0;
+  st.n_eos = n_eos;
+  for (int i = 0; i < n_eos; ++i) st.eos[i] = eos_ids[i];
+  alloc(reinterpret_cast<void**>(&st.next_scores), bb * sizeof(float));
+  alloc(reinterpret_cast<void**>(&st.next_tokens), bb * sizeof(int32_t));
+  alloc(reinterpret_cast<void**>(&st.next_indices), bb * sizeof(int32_t));
+  alloc(reinterpret_cast<void**>(&st.hyp_score), bb * sizeof(float));
+  alloc(reinterpret_cast<void**>(&st.hyp_len), bb * sizeof(int));
+  alloc(reinterpret_cast<void**>(&st.hyp_slot), static_cast<size_t>(batch) * (beams + 1) * sizeof(int));
+  alloc(reinterpret_cast<void**>(&st.hyp_tokens), static_cast<size_t>(batch) * (beams + 1) * max_length * sizeof(int32_t));
+  alloc(reinterpret_cast<void**>(&st.hyp_used), batch * sizeof(int));
+  alloc(reinterpret_cast<void**>(&st.done), batch * sizeof(int));
+  alloc(reinterpret_cast<void**>(&st.not_done), sizeof(int));
+  alloc(reinterpret_cast<void**>(&s->pow_dev), (static_cast<size_t>(max_length) + 1) * sizeof(float));
+  alloc(reinterpret_cast<void**>(&s->seq[0]), bb * max_length * sizeof(int32_t));
+  alloc(reinterpret_cast<void**>(&s->seq[1]), bb * max_length * sizeof(int32_t));
+  if (e == hipSuccess) {
+    // initial beam scores 0, -1e9, -1e9, ... per batch entry (src/beam_search_scorer.cpp:76-81); rank -> row
+    // identity; pow(length, length_penalty) from the host libm, the function the reference calls.
+    std::vector<float> init(bb, 0.0f), powt(static_cast<size_t>(max_length) + 1);
+    for (int b = 0; b < batch; ++b)
+      for (int j = 1; j < beams; ++j) init[static_cast<size_t>(b) * beams + j] = -1e9;
+    std::vector<int> slots(static_cast<size_t>(batch) * (beams + 1));
+    for (size_t i = 0; i < slots.size(); ++i) slots[i] = static_cast<int>(i % (beams + 1));
+    for (int l = 0; l <= max_length; ++l) powt[l] = std::pow(static_cast<float>(l), length_penalty);
+    e = hipMemcpy(st.next_scores, init.data(), bb * sizeof(float), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(st.hyp_slot, slots.data(), slots.size() * sizeof(int), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(s->pow_dev, powt.data(), powt.size() * sizeof(float), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(st.not_done, &batch, sizeof(int), hipMemcpyHostToDevice);
+    st.pow_table = s->pow_dev;
+  }
+  if (e != hipSuccess) {
+    mi355x_beam_scorer_destroy(s);
+    return Fail(MI355X_E_HIP, "beam scorer allocation failed: %s", hipGetErrorString(e));
+  }
+  *out = s;
+  return MI355X_OK;
+}
+
+void mi355x_beam_scorer_destroy(mi355x_beam_scorer* s) {
+  if (!s) return;
+  for (void* p : s->allocs) (void)hipFree(p);
+  delete s;
+}
+
+int mi355x_beam_scorer_set_prompt(mi355x_beam_scorer* s, void* stream, const int32_t* tokens, int prompt_len) {
+  if (!s || !tokens) return Fail(MI355X_E_INVALID, "null argument");
+  if (prompt_len < 0 || prompt_len > s->st.max_length) return Fail(MI355X_E_INVALID, "User-defined tokens exceed max_length.");
+  const int bb = s->st.batch * s->st.beams;
+  std::vector<int32_t> host(static_cast<size_t>(bb) * s->st.max_length, 0);
+  for (int i = 0; i < bb; ++i)
+    std::memcpy(host.data() + static_cast<size_t>(i) * s->st.max_length,
+                tokens + static_cast<size_t>(i / s->st.beams) * prompt_len, sizeof(int32_t) * prompt_len);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  HIP_TRY(hipMemcpyAsync(s->seq[s->cur], host.data(), host.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
+  HIP_TRY(hipStreamSynchronize(st));  // `host` goes out of scope
+  s->length = prompt_len;
+  return MI355X_OK;
+}
+
+int mi355x_beam_scorer_step(mi355x_beam_scorer* s, void* stream, const float* cand_scores, const int32_t* cand_tokens,
+                            const int32_t* cand_beam_indices) {
+  if (!s || !cand_scores || !cand_tokens || !cand_beam_indices) return Fail(MI355X_E_INVALID, "null argument");
+  if (s->length >= s->st.max_length) return Fail(MI355X_E_INVALID, "sequence already at max_length (%d)", s->st.max_length);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  HIP_TRY(ms_launch_scorer_process(&s->st, s->seq[s->cur], s->length, cand_scores, cand_tokens, cand_beam_indices, st));
+  HIP_TRY(ms_launch_beam_append(s->seq[s->cur], s->seq[1 - s->cur], s->st.batch * s->st.beams, s->st.max_length,
+                                s->length, s->st.next_indices, s->st.next_tokens, st));
+  s->cur = 1 - s->cur;
+  s->length += 1;
+  return MI355X_OK;
+}
+
+const float* mi355x_beam_scorer_next_scores(const mi355x_beam_scorer* s) { return s ? s->st.next_scores : nullptr; }
+const int32_t* mi355x_beam_scorer_next_tokens(const mi355x_beam_scorer* s) { return s ? s->st.next_tokens : nullptr; }
+const int32_t* mi355x_beam_scorer_next_indices(const mi355x_beam_scorer* s) { return s ? s->st.next_indices : nullptr; }
+const int32_t* mi355x_beam_scorer_sequences(const mi355x_beam_scorer* s, int* length) {
+  if (!s) return nullptr;
+  if (length) *length = s->length;
+  return s->seq[s->cur];
+}
+
+int mi355x_beam_scorer_is_done(mi355x_beam_scorer* s, void* stream, int* done) {
+  if (!s || !done) return Fail(MI355X_E_INVALID, "null argument");
+  int nd = 0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  HIP_TRY(hipMemcpyAsync(&nd, s->st.not_done, sizeof(int), hipMemcpyDeviceToHost, st));
+  HIP_TRY(hipStreamSynchronize(st));
+  *done = (nd == 0) || (s->length == s->st.max_length);  // BeamSearch_Cpu::IsDone, src/search.cpp:345-352
+  return MI355X_OK;
+}
+
+int mi355x_beam_scorer_hypothesis(mi355x_beam_scorer* s, void* stream, int batch, int index, int32_t* out, int capacity,
+                                  int* length, float* score) {
+  if (!s || !out || !length) return Fail(MI355X_E_INVALID, "null argument");
+  if (batch < 0 || batch >= s->st.batch) return Fail(MI355X_E_INVALID, "batch index out of range");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (!s->finalized) {
+    HIP_TRY(ms_launch_scorer_finalize(&s->st, s->seq[s->cur], s->length, st));
+    s->finalized = true;
+  }
+  const int nb = s->st.beams;
+  int used = 0;
+  HIP_TRY(hipMemcpyAsync(&used, s->st.hyp_used + batch, sizeof(int), hipMemcpyDeviceToHost, st));
+  HIP_TRY(hipStreamSynchronize(st));
+  if (index < 0 || index >= used) return Fail(MI355X_E_INVALID, "GetHypothesis index out of bounds");
+  int len = 0, slot = 0;
+  float sc = 0.0f;
+  HIP_TRY(hipMemcpy(&len, s->st.hyp_len + batch * nb + index, sizeof(int), hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(&slot, s->st.hyp_slot + batch * (nb + 1) + index, sizeof(int), hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(&sc, s->st.hyp_score + batch * nb + index, sizeof(float), hipMemcpyDeviceToHost));
+  const int n = len < capacity ? len : capacity;
+  HIP_TRY(hipMemcpy(out, s->st.hyp_tokens + (static_cast<size_t>(batch) * (nb + 1) + slot) * s->st.max_length,
+                    sizeof(int32_t) * n, hipMemcpyDeviceToHost));
+  *length = len;
+  if (score) *score = sc;
   return MI355X_OK;
 }
 

@@ -1,0 +1,264 @@
+// Beam search: per-row log-softmax + candidate selection, per-batch merge to the 2*beams best, the
+// device-resident BeamSearchScorer and the beam-reordered sequence append.
+#include "kernels.h"
+#include "block_seq.h"
+#include "wave_select.h"
+
+namespace ms {
+
+constexpr int kBeamListCap = 1024;  // candidates a row may hold in LDS before the slow exact path
+
+// One 1024-thread block per batch-beam row.  BeamSearch_Cpu::SelectTop (src/search.cpp:101-123):
+// scores = ((x - max) * 1.0f - log(sum exp)) + beam_score, the sum accumulated in index order in
+// fp32 (reproduced exactly by the scan of seq_scan.h).  The value is monotone in x, so the row's
+// 2*beams best come from its largest logits: a pooled bound on per-thread maxima gives a cut whose
+// final score decides membership; everything at or above it is sorted by (score desc, token asc).
+template <typename InT>
+__global__ __launch_bounds__(1024) void beam_row_kernel(const BeamArgs a) {
+  __shared__ SeqShared sh;
+  __shared__ u64 list[kBeamListCap];
+  __shared__ uint32_t pool[64];
+  __shared__ uint32_t red[16];
+  __shared__ u64 red64[16];
+  __shared__ uint32_t bound, count;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int V = a.vocab, m = 2 * a.beams;
+  const InT* x = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
+  float fm = -__builtin_inff();
+  for (int i = tid; i < V; i += blockDim.x) fm = fmaxf(fm, load_one<InT>(x, i));
+  const uint32_t lkey = tid < V ? order_key(fm) : 0u;
+  const float max_score = key_to_float(block_max<uint32_t>(lkey, red));
+  const int n_lanes = V < 1024 ? V : 1024;
+  const uint32_t tau = block_pool_bound(lkey, m, (n_lanes + 63) / 64, pool, &bound);
+  auto e = [=](int i) { return em::expf_exact(load_one<InT>(x, i) - max_score); };
+  int dummy;
+  const float lse = em::logf_exact(block_seq_sum<8>(0.0f, V, e, NoStop{}, &dummy, sh));
+  const float bs = a.beam_scores[row];
+  auto final_score = [=](float v) { return ((v - max_score) - lse) + bs; };
+  // tau == 0: fewer than m offers (tiny vocabulary): every element is a candidate
+  const float cut = tau != 0u ? final_score(key_to_float(tau)) : -__builtin_inff();
+  if (tid == 0) count = 0u;
+  __syncthreads();
+  for (int i0 = 0; i0 < V; i0 += blockDim.x) {
+    const int i = i0 + tid;
+    float f = 0.0f;
+    bool cand = false;
+    if (i < V) {
+      f = final_score(load_one<InT>(x, i));
+      cand = (f >= cut) || (tau == 0u);
+    }
+    const uint32_t pos = wave_slot(cand, &count);
+    if (cand && pos < kBeamListCap) list[pos] = make_key64(order_key(f), static_cast<uint32_t>(i));
+  }
+  __syncthreads();
+  const uint32_t n = count;
+  float* out_s = a.row_scores + static_cast<size_t>(row) * kBeamMaxCand;
+  int32_t* out_t = a.row_tokens + static_cast<size_t>(row) * kBeamMaxCand;
+  if (n <= kBeamListCap) {
+    int n2 = 64;
+    while (n2 < static_cast<int>(n)) n2 <<= 1;
+    for (int p = static_cast<int>(n) + tid; p < n2; p += blockDim.x) list[p] = 0;
+    __syncthreads();
+    block_sort_desc(list, n2);
+    if (tid < m) {
+      const u64 k = tid < static_cast<int>(n) ? list[tid] : 0;
+      out_s[tid] = key_to_float(key64_okey(k));
+      out_t[tid] = k ? static_cast<int32_t>(key64_index(k)) : -1;
+    }
+    return;
+  }
+  // Heavy ties (e.g. a constant row): extract the m best one at a time, each the largest
+  // (score, lowest token) key strictly below the previous one.
+  u64 last = ~0ull;
+  for (int r = 0; r < m; ++r) {
+    u64 best = 0;
+    for (int i = tid; i < V; i += blockDim.x) {
+      const u64 k = make_key64(order_key(final_score(load_one<InT>(x, i))), static_cast<uint32_t>(i));
+      if (k < last && k > best) best = k;
+    }
+    best = block_max<u64>(best, red64);
+    if (tid == 0) {
+      out_s[r] = key_to_float(key64_okey(best));
+      out_t[r] = best ? static_cast<int32_t>(key64_index(best)) : -1;
+    }
+    last = best ? best : 0;
+  }
+}
+
+// One block per batch entry: the 2*beams best of the beams x 2*beams row candidates by
+// (score desc, beam*vocab+token asc), as the flat partial_sort of src/search.cpp:148-163 orders them.
+__global__ __launch_bounds__(256) void beam_merge_kernel(const BeamArgs a) {
+  __shared__ u64 keys[512];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const int m = 2 * a.beams, n = a.beams * m;
+  int n2 = 64;
+  while (n2 < n) n2 <<= 1;
+  for (int p = tid; p < n2; p += blockDim.x) {
+    u64 k = 0;
+    if (p < n) {
+      const int beam = p / m, j = p % m;
+      const size_t src = static_cast<size_t>(b * a.beams + beam) * kBeamMaxCand + j;
+      const int tok = a.row_tokens[src];
+      if (tok >= 0)
+        k = make_key64(order_key(a.row_scores[src]), static_cast<uint32_t>(beam) * static_cast<uint32_t>(a.vocab) +
+                                                         static_cast<uint32_t>(tok));
+    }
+    keys[p] = k;
+  }
+  __syncthreads();
+  block_sort_desc(keys, n2);
+  if (tid < m) {
+    const u64 k = keys[tid];
+    const uint32_t flat = key64_index(k);
+    a.out_scores[b * m + tid] = key_to_float(key64_okey(k));
+    a.out_tokens[b * m + tid] = static_cast<int32_t>(flat % static_cast<uint32_t>(a.vocab));
+    a.out_beams[b * m + tid] = static_cast<int32_t>(flat / static_cast<uint32_t>(a.vocab));
+  }
+}
+
+// ---- BeamSearchScorer::Process (src/beam_search_scorer.cpp:84-171), one wave per batch entry ----------
+// All lanes follow the same scalar control flow; the lanes only share the work of cloning sequences.
+__device__ __forceinline__ bool scorer_is_eos(const ScorerState& s, int tok) {
+  for (int i = 0; i < s.n_eos; ++i)
+    if (s.eos[i] == tok) return true;
+  return false;
+}
+
+// BeamHypotheses::Add (src/beam_search_scorer.cpp:19-39).  Hypotheses live in beams+1 token rows per
+// batch entry; `slot` maps rank -> row, so inserting shifts ranks, not tokens.
+__device__ __forceinline__ void scorer_add(const ScorerState& s, int batch, const int32_t* seq, int length,
+                                           float sum_logprobs) {
+  const int nb = s.beams, lane = lane_id();
+  float* hs = s.hyp_score + batch * nb;
+  int* hl = s.hyp_len + batch * nb;
+  int* slot = s.hyp_slot + batch * (nb + 1);
+  const float score = sum_logprobs / s.pow_table[length];
+  int index = s.hyp_used[batch];
+  int row;
+  if (index == nb) {
+    if (score <= hs[nb - 1]) return;
+    index = nb - 1;
+    row = slot[nb - 1];  // the evicted hypothesis' row is reused
+  } else {
+    row = slot[index];
+    if (lane == 0) s.hyp_used[batch] = index + 1;
+  }
+  int32_t* dst = s.hyp_tokens + (static_cast<size_t>(batch) * (nb + 1) + row) * s.max_length;
+  for (int i = lane; i < length; i += 64) dst[i] = seq[i];
+  __builtin_amdgcn_wave_barrier();
+  if (lane == 0) {
+    for (; index > 0 && score > hs[index - 1]; index--) {
+      hs[index] = hs[index - 1];
+      hl[index] = hl[index - 1];
+      slot[index] = slot[index - 1];
+    }
+    hs[index] = score;
+    hl[index] = length;
+    slot[index] = row;
+  }
+  __threadfence_block();
+  __builtin_amdgcn_wave_barrier();
+}
+
+__global__ __launch_bounds__(64) void beam_scorer_process_kernel(const ScorerState s, const int32_t* sequences,
+                                                                 int sequence_length, const float* cand_scores,
+                                                                 const int32_t* cand_tokens, const int32_t* cand_indices) {
+  const int batch = blockIdx.x, lane = lane_id();
+  const int nb = s.beams, top_k = 2 * nb;
+  if (s.done[batch]) {
+    if (lane < nb) {
+      s.next_scores[batch * nb + lane] = 0.0f;
+      s.next_tokens[batch * nb + lane] = s.pad;
+      s.next_indices[batch * nb + lane] = 0;
+    }
+    return;
+  }
+  int beam_idx = 0;
+  for (int j = 0; j < top_k; ++j) {
+    const int tok = cand_tokens[batch * top_k + j];
+    const float score = cand_scores[batch * top_k + j];
+    const int bbi = batch * nb + cand_indices[batch * top_k + j];
+    if (scorer_is_eos(s, tok)) {
+      if (j >= nb) continue;
+      scorer_add(s, batch, sequences + static_cast<size_t>(bbi) * s.max_length, sequence_length, score);
+    } else {
+      if (lane == 0) {
+        s.next_scores[batch * nb + beam_idx] = score;
+        s.next_tokens[batch * nb + beam_idx] = tok;
+        s.next_indices[batch * nb + beam_idx] = bbi;
+      }
+      ++beam_idx;
+    }
+    if (beam_idx == nb) break;
+  }
+  __builtin_amdgcn_wave_barrier();
+  if (lane != 0) return;
+  if (s.hyp_used[batch] < nb) return;
+  if (!s.early_stopping) {
+    // The reference's window starts at batch*beams rather than batch*2*beams (:161); kept as is.
+    float best = cand_scores[batch * nb];
+    for (int i = 1; i < top_k; ++i) best = fmaxf(best, cand_scores[batch * nb + i]);
+    const float current = best / s.pow_table[sequence_length];
+    if (s.hyp_score[batch * nb + nb - 1] < current) return;  // CanImprove
+  }
+  s.done[batch] = 1;
+  atomicSub(s.not_done, 1);
+}
+
+// BeamSearchScorer::Finalize (src/beam_search_scorer.cpp:173-196): open batch entries add their
+// current beams as hypotheses.
+__global__ __launch_bounds__(64) void beam_scorer_finalize_kernel(const ScorerState s, const int32_t* sequences,
+                                                                  int sequence_length) {
+  const int batch = blockIdx.x;
+  if (s.done[batch]) return;
+  for (int j = 0; j < s.beams; ++j) {
+    const int bbi = batch * s.beams + j;
+    scorer_add(s, batch, sequences + static_cast<size_t>(bbi) * s.max_length, sequence_length, s.next_scores[bbi]);
+  }
+}
+
+// BeamSearch_Cpu::AppendNextTokensToSequences (src/search.cpp:354-381).
+__global__ __launch_bounds__(256) void beam_append_kernel(const int32_t* seq, int32_t* seq_next, int max_length,
+                                                          int current_length, const int32_t* beam_indices,
+                                                          const int32_t* tokens) {
+  const int i = blockIdx.x;
+  const int32_t* src = seq + static_cast<size_t>(beam_indices[i]) * max_length;
+  int32_t* dst = seq_next + static_cast<size_t>(i) * max_length;
+  for (int t = threadIdx.x; t < current_length; t += blockDim.x) dst[t] = src[t];
+  if (threadIdx.x == 0) dst[current_length] = tokens[i];
+}
+
+}  // namespace ms
+
+extern "C" hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hipStream_t stream) {
+  const int rows = a->batch * a->beams;
+  if (dtype == MI355X_F16)
+    hipLaunchKernelGGL(ms::beam_row_kernel<uint16_t>, dim3(rows), dim3(1024), 0, stream, *a);
+  else
+    hipLaunchKernelGGL(ms::beam_row_kernel<float>, dim3(rows), dim3(1024), 0, stream, *a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(ms::beam_merge_kernel, dim3(a->batch), dim3(256), 0, stream, *a);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_scorer_process(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,
+                                               const float* cs, const int32_t* ct, const int32_t* ci, hipStream_t stream) {
+  hipLaunchKernelGGL(ms::beam_scorer_process_kernel, dim3(s->batch), dim3(64), 0, stream, *s, sequences, sequence_length,
+                     cs, ct, ci);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_scorer_finalize(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,
+                                                hipStream_t stream) {
+  hipLaunchKernelGGL(ms::beam_scorer_finalize_kernel, dim3(s->batch), dim3(64), 0, stream, *s, sequences, sequence_length);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_beam_append(const int32_t* seq, int32_t* seq_next, int rows, int max_length,
+                                            int current_length, const int32_t* beam_indices, const int32_t* tokens,
+                                            hipStream_t stream) {
+  hipLaunchKernelGGL(ms::beam_append_kernel, dim3(rows), dim3(256), 0, stream, seq, seq_next, max_length, current_length,
+                     beam_indices, tokens);
+  return hipGetLastError();
+}

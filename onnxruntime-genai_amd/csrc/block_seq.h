@@ -69,12 +69,16 @@ struct NoStop {
 template <int ITEMS, typename GetE, typename StopFn>
 __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop_index, SeqShared& sh) {
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
-  const int span = static_cast<int>(blockDim.x) * ITEMS;
   float s = s0;
   int i0 = 0, found = -1;
+  // Items per thread in the current window.  A window is redone from the element behind a binade
+  // change, and those cluster at the start of a sum, so windows start small and double while no
+  // change occurs.
+  int items = 1;
   while (i0 < n) {
     const SeqState st = seq_decompose(s);
-    const int base = i0 + tid * ITEMS;
+    const int span = static_cast<int>(blockDim.x) * items;
+    const int base = i0 + tid * items;
     const int window_end = (n - i0 < span) ? n : i0 + span;
     float ev[ITEMS];
     Step f[ITEMS];
@@ -82,7 +86,8 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
       const int idx = base + j;
-      ev[j] = idx < n ? get(idx) : 0.0f;
+      const bool on = j < items && idx < window_end;
+      ev[j] = on ? get(idx) : 0.0f;
       f[j] = seq_make_step(ev[j], st.se);
       agg = step_compose(agg, f[j]);
     }
@@ -105,7 +110,7 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
       const int idx = base + j;
-      if (idx < window_end) {
+      if (j < items && idx < window_end) {
         const uint32_t nn2 = step_apply(nn, f[j]);
         if (nn2 >= kMantLimit) {
           if (nn < kMantLimit) {  // the one addition that leaves the binade
@@ -137,7 +142,9 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
     if (gc == kIntMax) {
       s = seq_recompose(sh.n_last, st.se);
       i0 = window_end;
+      if (items < ITEMS) items *= 2;
     } else {
+      items = 1;
       const float e_cross = sh.e_cross;
       s = sh.s_before + e_cross;
       if (stop(s, e_cross, gc)) {

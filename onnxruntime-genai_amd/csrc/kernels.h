@@ -45,6 +45,8 @@ struct SampleArgs {
   u64* big;               // [rows][big_stride]
   size_t big_stride;
   uint32_t* fallback_rows;  // cumulative count of rows finished by the general path
+  int emit_topk;            // != 0: write the k best (id, raw score) per row instead of sampling
+  float* out_scores;        // [rows, k], emit_topk only (out_tokens is [rows, k] then)
 #ifdef MS_DEBUG_STAGES
   int debug_stage;  // timing experiments only: stop after the given stage
 #endif
@@ -60,6 +62,37 @@ struct ArgmaxArgs {
   uint32_t* row_arrive;  // [rows], zero between launches
 };
 
+constexpr int kBeamMaxCand = 32;  // 2 * beams, beams <= 16
+
+struct BeamArgs {
+  const void* logits;
+  int64_t row_stride;
+  int batch, beams, vocab;
+  const float* beam_scores;   // [batch*beams]
+  float* row_scores;          // workspace [batch*beams][kBeamMaxCand]
+  int32_t* row_tokens;        // workspace [batch*beams][kBeamMaxCand]
+  float* out_scores;          // [batch][2*beams]
+  int32_t* out_tokens;
+  int32_t* out_beams;
+};
+
+// Device-resident BeamSearchScorer state (all pointers device memory).
+struct ScorerState {
+  int batch, beams, max_length, pad, early_stopping, n_eos;
+  int eos[MI355X_MAX_EOS];
+  float* next_scores;     // [batch*beams]
+  int32_t* next_tokens;
+  int32_t* next_indices;
+  float* hyp_score;       // [batch][beams], best first
+  int* hyp_len;           // [batch][beams]
+  int* hyp_slot;          // [batch][beams+1]: rank -> token row
+  int32_t* hyp_tokens;    // [batch][beams+1][max_length]
+  int* hyp_used;          // [batch]
+  int* done;              // [batch]
+  int* not_done;          // [1]
+  const float* pow_table; // [max_length+1]: powf(length, length_penalty), computed by the host libm
+};
+
 }  // namespace ms
 
 extern "C" {
@@ -68,4 +101,21 @@ hipError_t ms_launch_sample(const ms::SampleArgs* a, bool any_nucleus, hipStream
 hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipStream_t stream);
 hipError_t ms_launch_process_logits(float* logits, int64_t row_stride, int rows, int vocab,
                                     const ms::Xform* xf, hipStream_t stream);
+hipError_t ms_launch_softmax(float* scores, int64_t row_stride, int rows, int vocab, float temperature,
+                             int log_softmax, hipStream_t stream);
+hipError_t ms_launch_kv_gather(const void* const* present_dev, void* const* past_dev, int n_tensors,
+                               const int32_t* beam_indices, int rows, size_t block_bytes, hipStream_t stream);
+hipError_t ms_launch_spec_verify(const float* p_target, const float* p_draft, const int32_t* draft_tokens,
+                                 const float* accept_u, const double* sample_u, int batch, int K, int vocab,
+                                 int32_t* accepted_len, int32_t* final_token, hipStream_t stream);
+hipError_t ms_launch_widen_f16(const void* in, int64_t in_stride, float* out, int64_t out_stride, int rows,
+                               int vocab, hipStream_t stream);
+hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hipStream_t stream);
+hipError_t ms_launch_scorer_process(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,
+                                    const float* cs, const int32_t* ct, const int32_t* ci, hipStream_t stream);
+hipError_t ms_launch_scorer_finalize(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,
+                                     hipStream_t stream);
+hipError_t ms_launch_beam_append(const int32_t* seq, int32_t* seq_next, int rows, int max_length,
+                                 int current_length, const int32_t* beam_indices, const int32_t* tokens,
+                                 hipStream_t stream);
 }

@@ -1,0 +1,165 @@
+// Softmax / log-softmax with the reference's sequential fp32 sum, the KV-cache beam gather, the
+// speculative-decoding verifier and the fp16 -> fp32 widening copy.
+#include "kernels.h"
+#include "block_seq.h"
+#include "wave_select.h"
+
+namespace ms {
+
+// ---- Softmax / LogSoftMax (src/softmax.h:26-47) ------------------------------------------------------
+// One 1024-thread block per row.  The sum of exponentials is accumulated in index order in fp32 --
+// reproduced exactly by the scan of seq_scan.h -- so every output bit equals the reference's.
+template <bool LOG>
+__global__ __launch_bounds__(1024) void softmax_kernel(float* scores, int64_t row_stride, int vocab, float temperature) {
+  __shared__ SeqShared sh;
+  __shared__ uint32_t red[16];
+  float* x = scores + static_cast<size_t>(blockIdx.x) * row_stride;
+  float m = -__builtin_inff();
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) m = fmaxf(m, x[i]);
+  const float max_score = key_to_float(block_max<uint32_t>(order_key(m), red));
+  const float inv_temp = 1.0f / temperature;
+  const float* xc = x;
+  auto e = [=](int i) { return em::expf_exact((xc[i] - max_score) * inv_temp); };
+  int dummy;
+  const float sum = block_seq_sum<8>(0.0f, vocab, e, NoStop{}, &dummy, sh);
+  if (LOG) {
+    const float lse = em::logf_exact(sum);
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+      const float s = (x[i] - max_score) * inv_temp;
+      x[i] = s - lse;
+    }
+  } else {
+    const float inv_sum = 1.0f / sum;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+      const float ex = em::expf_exact((x[i] - max_score) * inv_temp);
+      x[i] = sum > 0.0f ? ex * inv_sum : ex;
+    }
+  }
+}
+
+// ---- KV-cache beam gather (src/models/kv_cache.cpp:710-740) -----------------------------------------
+// past[t][j] = present[t][beam_indices[j]] for blocks of block_bytes bytes.  grid = (tiles, rows,
+// tensors); every block moves kGatherTile bytes with 128-bit non-temporal loads and stores.
+constexpr int kGatherTile = 16384;
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void kv_gather_kernel(const void* const* present, void* const* past,
+                                                        const int32_t* beam_indices, size_t block_bytes) {
+  const int row = blockIdx.y, t = blockIdx.z;
+  const size_t tile0 = static_cast<size_t>(blockIdx.x) * kGatherTile;
+  const char* src = static_cast<const char*>(present[t]) + static_cast<size_t>(beam_indices[row]) * block_bytes + tile0;
+  char* dst = static_cast<char*>(past[t]) + static_cast<size_t>(row) * block_bytes + tile0;
+  const size_t remain = block_bytes - tile0;
+  const int n16 = static_cast<int>((remain < static_cast<size_t>(kGatherTile) ? remain : kGatherTile) / 16);
+  v4u regs[kGatherTile / 16 / 256];
+#pragma unroll
+  for (int j = 0; j < kGatherTile / 16 / 256; ++j) {
+    const int i = j * 256 + threadIdx.x;
+    if (i < n16) regs[j] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(src) + i);
+  }
+#pragma unroll
+  for (int j = 0; j < kGatherTile / 16 / 256; ++j) {
+    const int i = j * 256 + threadIdx.x;
+    if (i < n16) __builtin_nontemporal_store(regs[j], reinterpret_cast<v4u*>(dst) + i);
+  }
+}
+
+// ---- speculative-decoding verification ---------------------------------------------------------------
+// One 1024-thread block per batch entry.  Accept loop of SpeculativeDecodingStrategy::RunRound
+// (src/speculative_decoding_strategy.cpp:718-762) on dense distributions, then the round's single
+// categorical draw: the residual max(p-q,0) at the first rejected position (SampleCorrectionToken,
+// src/speculative_sampling.h:39-57; the target row itself when the residual is all zero) or the
+// bonus row K on full acceptance.
+__global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target, const float* p_draft,
+                                                           const int32_t* draft_tokens, const float* accept_u,
+                                                           const double* sample_u, int K, int vocab,
+                                                           int32_t* accepted_len, int32_t* final_token) {
+  __shared__ SeqShared sh;
+  __shared__ int sh_n, sh_any;
+  const int b = blockIdx.x;
+  const size_t base = static_cast<size_t>(b) * (K + 1) * vocab;
+  if (threadIdx.x == 0) {
+    int n = 0;
+    for (; n < K; ++n) {
+      const int d = draft_tokens[b * K + n];
+      const float pt = p_target[base + static_cast<size_t>(n) * vocab + d];
+      const float pd = p_draft[base + static_cast<size_t>(n) * vocab + d];
+      const float acc = pd <= 0.0f ? 1.0f : fminf(1.0f, pt / pd);  // ComputeAcceptProb, :140-146
+      if (!(accept_u[b * K + n] < acc)) break;
+    }
+    sh_n = n;
+    sh_any = 0;
+  }
+  __syncthreads();
+  const int n = sh_n;
+  const float* pt = p_target + base + static_cast<size_t>(n) * vocab;
+  const float* pd = p_draft + base + static_cast<size_t>(n) * vocab;
+  bool use_residual = false;
+  if (n < K) {
+    int any = 0;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) any |= (pt[i] - pd[i] > 0.0f);
+    if (any) sh_any = 1;  // the reference's fp32 "sum > 0" holds iff some residual is positive
+    __syncthreads();
+    use_residual = sh_any != 0;
+  }
+  int pos;
+  if (use_residual) {
+    auto w = [=](int i) {
+      const float d = pt[i] - pd[i];
+      return d > 0.0f ? d : 0.0f;
+    };
+    pos = block_discrete_draw<4>(vocab, w, sample_u[b], sh);
+  } else {
+    auto w = [=](int i) { return pt[i]; };
+    pos = block_discrete_draw<4>(vocab, w, sample_u[b], sh);
+  }
+  if (threadIdx.x == 0) {
+    accepted_len[b] = n;
+    final_token[b] = pos;
+  }
+}
+
+// fp16 -> fp32 with the reference's FastFloat16ToFloat32 semantics (DeviceInterface::Cast).
+__global__ __launch_bounds__(256) void widen_f16_kernel(const uint16_t* in, int64_t in_stride, float* out,
+                                                        int64_t out_stride, int vocab) {
+  const uint16_t* src = in + static_cast<size_t>(blockIdx.y) * in_stride;
+  float* dst = out + static_cast<size_t>(blockIdx.y) * out_stride;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < vocab; i += gridDim.x * blockDim.x)
+    dst[i] = half_bits_to_float(src[i]);
+}
+
+}  // namespace ms
+
+extern "C" hipError_t ms_launch_softmax(float* scores, int64_t row_stride, int rows, int vocab, float temperature,
+                                        int log_softmax, hipStream_t stream) {
+  if (log_softmax)
+    hipLaunchKernelGGL(ms::softmax_kernel<true>, dim3(rows), dim3(1024), 0, stream, scores, row_stride, vocab, temperature);
+  else
+    hipLaunchKernelGGL(ms::softmax_kernel<false>, dim3(rows), dim3(1024), 0, stream, scores, row_stride, vocab, temperature);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_kv_gather(const void* const* present_dev, void* const* past_dev, int n_tensors,
+                                          const int32_t* beam_indices, int rows, size_t block_bytes, hipStream_t stream) {
+  const unsigned tiles = static_cast<unsigned>((block_bytes + ms::kGatherTile - 1) / ms::kGatherTile);
+  hipLaunchKernelGGL(ms::kv_gather_kernel, dim3(tiles, rows, n_tensors), dim3(256), 0, stream, present_dev, past_dev,
+                     beam_indices, block_bytes);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_spec_verify(const float* p_target, const float* p_draft, const int32_t* draft_tokens,
+                                            const float* accept_u, const double* sample_u, int batch, int K, int vocab,
+                                            int32_t* accepted_len, int32_t* final_token, hipStream_t stream) {
+  hipLaunchKernelGGL(ms::spec_verify_kernel, dim3(batch), dim3(1024), 0, stream, p_target, p_draft, draft_tokens,
+                     accept_u, sample_u, K, vocab, accepted_len, final_token);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_widen_f16(const void* in, int64_t in_stride, float* out, int64_t out_stride, int rows,
+                                          int vocab, hipStream_t stream) {
+  int gx = (vocab + 255) / 256;
+  if (gx > 512) gx = 512;
+  hipLaunchKernelGGL(ms::widen_f16_kernel, dim3(gx, rows), dim3(256), 0, stream, static_cast<const uint16_t*>(in),
+                     in_stride, out, out_stride, vocab);
+  return hipGetLastError();
+}

@@ -90,6 +90,15 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
   }
   block_sort_desc(scratch, n2);
   const mi355x_sample_params prm = a.per_row ? a.per_row[row] : a.uniform;
+  if (a.emit_topk) {
+    const int kk = prm.k < V ? prm.k : V;
+    for (int j = threadIdx.x; j < kk; j += blockDim.x) {
+      a.out_tokens[static_cast<size_t>(row) * prm.k + j] = static_cast<int32_t>(key64_index(scratch[j]));
+      a.out_scores[static_cast<size_t>(row) * prm.k + j] = key_to_float(key64_okey(scratch[j]));
+    }
+    if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
+    return;
+  }
   const float max_score = key_to_float(key64_okey(scratch[0]));
   const float inv_temp = 1.0f / prm.temperature;
   const RowOutputs out = row_outputs(a, row);
@@ -100,8 +109,9 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
   if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
 }
 
-__device__ __forceinline__ int row_mode(mi355x_sample_params prm, int vocab, int chunks) {
+__device__ __forceinline__ int row_mode(mi355x_sample_params prm, int vocab, int chunks, int emit_topk = 0) {
   if (vocab <= 64 || chunks * kSmallCap > kAllCap) return kModeGeneral;
+  if (emit_topk) return kModeTopkSmall;
   if (prm.k > 1) return (prm.k < vocab ? prm.k : vocab) <= 64 ? kModeTopkSmall : kModeGeneral;
   return kModeNucleus;
 }
@@ -395,7 +405,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     tab.lo = static_cast<uint32_t>(t);
     tab.hi = static_cast<uint32_t>(t >> 32);
   }
-  const double u = a.uniforms[row];
+  const double u = a.emit_topk ? 0.0 : a.uniforms[row];
   if (tid == 0) {
     a.row_arrive[row] = 0u;
     sm.count = 0u;
@@ -504,7 +514,14 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   if (tid < 64 && sm.redo == 0u) {
     final_key = wave_sort_desc_fast<u64>(final_key);
     MS_STAGE(9, (uint32_t)final_key);
-    wave_topk_epilogue(final_key, kk, prm, u, tab, row_outputs(a, row));
+    if (a.emit_topk) {
+      if (lane < kk) {
+        a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(key64_index(final_key));
+        a.out_scores[static_cast<size_t>(row) * prm.k + lane] = key_to_float(key64_okey(final_key));
+      }
+    } else {
+      wave_topk_epilogue(final_key, kk, prm, u, tab, row_outputs(a, row));
+    }
   }
   __syncthreads();
   return sm.redo != 0u;
@@ -514,7 +531,7 @@ __global__ __launch_bounds__(kSBlock) void sample_fused_kernel(const SampleArgs 
   const int row = blockIdx.y, chunk = blockIdx.x;
   __shared__ FusedShared sm;
   const mi355x_sample_params prm = a.per_row ? a.per_row[row] : a.uniform;
-  const int mode = row_mode(prm, a.vocab, a.chunks);
+  const int mode = row_mode(prm, a.vocab, a.chunks, a.emit_topk);
   if (mode == kModeGeneral) {
     if (chunk != 0) return;
   } else if (!stream_row(a, row, chunk, prm, mode, sm)) {

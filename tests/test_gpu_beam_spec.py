@@ -1,0 +1,209 @@
+"""GPU parity for the remaining entry points, through the C ABI, against the CPU oracle on the same
+seeded inputs: top-k scores, softmax / log-softmax (bit-exact: the sequential fp32 sum is emulated
+exactly), beam top-2B selection + BeamSearchScorer + sequence reorder, KV-cache gather (bit-exact)
+and speculative verification (bit-exact lengths and tokens)."""
+import numpy as np
+import pytest
+import torch
+
+import orc_lib
+from gpu_common import pkg, say
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = pkg().SearchContext(64, 201088)
+    yield c
+    c.close()
+
+
+def bits(a):
+    return np.asarray(a, np.float32).view(np.uint32)
+
+
+@pytest.mark.parametrize("rows,vocab,k,dtype", [(3, 32064, 8, np.float32), (9, 151936, 50, np.float16),
+                                                (2, 40, 5, np.float32), (2, 5000, 1, np.float32),
+                                                (17, 128256, 64, np.float32)])
+def test_topk_scores(ctx, orc, rows, vocab, k, dtype):
+    say("topk_scores", rows, vocab, k, dtype.__name__)
+    rng = np.random.default_rng(vocab + k)
+    x = (rng.standard_normal((rows, vocab)) * 2).astype(dtype)
+    tok, sc = ctx.topk_scores(torch.from_numpy(x).cuda(), k)
+    tok, sc = tok.cpu().numpy(), sc.cpu().numpy()
+    xf = orc.fp16_to_fp32(x) if dtype == np.float16 else x
+    for r in range(rows):
+        order = np.lexsort((np.arange(vocab), -xf[r].astype(np.float64)))[:k]  # score desc, index asc
+        assert np.array_equal(tok[r], order)
+        assert np.array_equal(sc[r], xf[r][order])
+
+
+@pytest.mark.parametrize("rows,vocab,t", [(4, 1000, 1.0), (3, 151936, 1.0), (2, 32064, 0.7), (2, 7, 2.0)])
+def test_softmax_bit_exact(ctx, orc, rows, vocab, t):
+    say("softmax", rows, vocab, t)
+    rng = np.random.default_rng(vocab)
+    x = (rng.standard_normal((rows, vocab)) * 2).astype(np.float32)
+    sm = ctx.softmax(torch.from_numpy(x.copy()).cuda(), t, log=False).cpu().numpy()
+    lsm = ctx.softmax(torch.from_numpy(x.copy()).cuda(), t, log=True).cpu().numpy()
+    for r in range(rows):
+        assert np.array_equal(bits(sm[r]), bits(orc.softmax(x[r], t)))  # tolerance allowed: 1e-5 rel; achieved: 0
+        assert np.array_equal(bits(lsm[r]), bits(orc.log_softmax(x[r], t)))
+
+
+def test_log_softmax_extreme_rows(ctx, orc):
+    """Sums that start subnormal, cross many binades, or hit exact ties in the running sum."""
+    say("softmax extreme")
+    rng = np.random.default_rng(1)
+    v = 20000
+    x = np.zeros((4, v), np.float32)
+    x[0] = np.linspace(-100, 0, v)  # first terms underflow / subnormal
+    x[1] = 0.0  # all ones: exact integer sums, ties to even past 2^24? (no) but every add exact
+    x[2] = np.where(rng.random(v) < 0.5, 0.0, -16.635532).astype(np.float32)  # ~2^-24 against 1.0
+    x[3] = rng.standard_normal(v) * 20
+    got = ctx.softmax(torch.from_numpy(x.copy()).cuda(), 1.0, log=True).cpu().numpy()
+    for r in range(4):
+        assert np.array_equal(bits(got[r]), bits(orc.log_softmax(x[r], 1.0))), r
+
+
+@pytest.mark.parametrize("batch,beams,vocab,dtype", [(2, 3, 1000, np.float32), (8, 4, 151936, np.float16),
+                                                     (1, 16, 5000, np.float32), (3, 2, 2, np.float32),
+                                                     (2, 4, 3000, np.float16)])
+def test_beam_select(ctx, orc, batch, beams, vocab, dtype):
+    say("beam_select", batch, beams, vocab, dtype.__name__)
+    rng = np.random.default_rng(vocab + beams)
+    x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(dtype)
+    bs = (rng.standard_normal(batch * beams) * 3).astype(np.float32)
+    bs[1::beams] = -1e9
+    sc, tok, idx = ctx.beam_select(torch.from_numpy(x).cuda(), batch, beams, torch.from_numpy(bs).cuda())
+    xf = orc.fp16_to_fp32(x) if dtype == np.float16 else x
+    osc, otok, oidx, _ = orc.beam_select_top(xf, batch, beams, bs)
+    assert np.array_equal(tok.cpu().numpy(), otok)
+    assert np.array_equal(idx.cpu().numpy(), oidx)
+    assert np.array_equal(bits(sc.cpu().numpy()), bits(osc))  # allowed 1e-5 relative; achieved bit-exact
+
+
+def test_beam_select_constant_rows(ctx, orc):
+    """All-equal logits: every candidate ties, selection must fall back to lowest flat index."""
+    say("beam_select ties")
+    batch, beams, vocab = 2, 3, 4000
+    x = np.zeros((batch * beams, vocab), np.float16)
+    x[4] = 1.0
+    bs = np.zeros(batch * beams, np.float32)
+    sc, tok, idx = ctx.beam_select(torch.from_numpy(x).cuda(), batch, beams, torch.from_numpy(bs).cuda())
+    osc, otok, oidx, _ = orc.beam_select_top(orc.fp16_to_fp32(x), batch, beams, bs)
+    assert np.array_equal(tok.cpu().numpy(), otok) and np.array_equal(idx.cpu().numpy(), oidx)
+
+
+def run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, length_penalty, early_stopping, seed,
+                    dtype=np.float16, eos_boost=0.0):
+    rng = np.random.default_rng(seed)
+    prompt = rng.integers(0, vocab, (batch, 3)).astype(np.int32)
+    dev = pkg().BeamScorer(ctx, batch, beams, max_length, 0, eos, length_penalty, early_stopping)
+    dev.set_prompt(prompt)
+    ref = orc_lib.BeamScorer(orc, batch, beams, max_length, 0, eos, length_penalty, early_stopping)
+    seq = np.zeros((batch * beams, max_length), np.int32)
+    seq[:, :3] = np.repeat(prompt, beams, axis=0)
+    length = 3
+    for step in range(steps):
+        say("beam search step", step)
+        x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(dtype)
+        for e in eos:
+            x[:, e] += eos_boost
+        xf = orc.fp16_to_fp32(x) if dtype == np.float16 else x
+        # device
+        dsc, dtok, didx = ctx.beam_select(torch.from_numpy(x).cuda(), batch, beams, dev.next_scores)
+        dev.step(dsc, dtok, didx)
+        # oracle
+        osc, otok, oidx, _ = orc.beam_select_top(xf, batch, beams, ref.next_scores)
+        ref.process(seq, length, osc, otok, oidx)
+        nxt = np.zeros_like(seq)
+        orc.lib.orc_beam_append(seq.reshape(-1), nxt.reshape(-1), batch * beams, max_length, length,
+                                ref.next_indices, ref.next_tokens)
+        seq, length = nxt, length + 1
+        assert np.array_equal(dtok.cpu().numpy(), otok) and np.array_equal(didx.cpu().numpy(), oidx)
+        assert np.array_equal(bits(dsc.cpu().numpy()), bits(osc))
+        assert np.array_equal(dev.next_tokens.cpu().numpy(), ref.next_tokens)
+        assert np.array_equal(dev.next_indices.cpu().numpy(), ref.next_indices)
+        assert np.array_equal(bits(dev.next_scores.cpu().numpy()), bits(ref.next_scores))
+        dseq, dlen = dev.sequences()
+        assert dlen == length and np.array_equal(dseq.cpu().numpy(), seq[:, :length])
+        assert dev.is_done() == (ref.is_done() or length == max_length)
+        if dev.is_done():
+            break
+    ref.finalize(seq, length)
+    for b in range(batch):
+        for i in range(ref.hyp_count(b)):
+            want_t, want_s = ref.hyp(b, i)
+            got_t, got_s = dev.hypothesis(b, i)
+            assert got_t == list(want_t) and np.float32(got_s) == np.float32(want_s), (b, i)
+    dev.close()
+
+
+def test_config3_beam_search_steps(ctx, orc):
+    """BASELINE config 3 shape (batch 8, beams 4, vocab 151936 fp16, length_penalty 1.0), 6 of the 64
+    steps: selection, scorer state, beam-reordered sequences and final hypotheses match the oracle."""
+    run_beam_search(ctx, orc, 8, 4, 151936, 6, [151935], 80, 1.0, True, 3)
+
+
+@pytest.mark.parametrize("early,lp", [(True, 1.0), (False, 1.0), (False, 0.6), (True, 2.0)])
+def test_beam_search_with_eos_hypotheses(ctx, orc, early, lp):
+    """Small vocabulary with a boosted EOS so hypotheses finish, batches become done and get padded."""
+    run_beam_search(ctx, orc, 3, 3, 50, 14, [7, 9], 20, lp, early, 11 + int(early), dtype=np.float32, eos_boost=2.5)
+
+
+def test_kv_gather_bit_exact(ctx, orc):
+    say("kv_gather")
+    rng = np.random.default_rng(5)
+    rows, shape = 8, (4, 96, 128)  # fp16 blocks of 96 KiB: exercises a partial last tile
+    present = [torch.from_numpy(rng.integers(0, 1 << 16, (rows,) + shape).astype(np.uint16).view(np.float16)).cuda()
+               for _ in range(6)]
+    past = [torch.zeros_like(p) for p in present]
+    idx = np.array([3, 3, 0, 7, 1, 1, 6, 2], np.int32)
+    ctx.kv_gather(present, past, torch.from_numpy(idx).cuda())
+    for p, q in zip(present, past):
+        want = orc.kv_gather(p.cpu().numpy().view(np.uint16), idx)
+        assert np.array_equal(q.cpu().numpy().view(np.uint16), want)
+
+
+def test_config3_kv_gather_full_block_size(ctx):
+    """Config-3 block (4 heads x 2048 x 128 fp16 = 2 MiB) on 2 of the 56 tensors, checked with torch."""
+    say("kv_gather 2MiB blocks")
+    g = torch.Generator(device="cuda").manual_seed(0)
+    present = [torch.randint(-30000, 30000, (32, 4, 2048, 128), generator=g, device="cuda", dtype=torch.int16)
+               .view(torch.float16) for _ in range(2)]
+    past = [torch.zeros_like(p) for p in present]
+    idx = torch.randint(0, 32, (32,), generator=g, device="cuda", dtype=torch.int32)
+    ctx.kv_gather(present, past, idx)
+    for p, q in zip(present, past):
+        assert torch.equal(q.view(torch.int16), p.view(torch.int16)[idx.long()])
+
+
+def softmax64(x):
+    z = x - x.max(-1, keepdims=True)
+    e = np.exp(z)
+    return (e / e.sum(-1, keepdims=True)).astype(np.float32)
+
+
+@pytest.mark.parametrize("batch,K,vocab", [(16, 8, 32064), (4, 3, 500), (5, 1, 2)])
+def test_spec_verify(ctx, orc, batch, K, vocab):
+    """BASELINE config 4 (first case): target/draft probabilities from N(0,2^2) logits, draft = target
+    logits + N(0,0.5^2); accept tests and residual / bonus resampling with shared uniforms."""
+    say("spec_verify", batch, K, vocab)
+    rng = np.random.default_rng(vocab + K)
+    lt = rng.standard_normal((batch, K + 1, vocab)) * 2
+    p = softmax64(lt)
+    q = softmax64(lt + rng.standard_normal((batch, K + 1, vocab)) * 0.5)
+    if batch > 2:
+        q[1] = p[1]  # identical distributions: always accepted -> bonus row
+        q[2, 0] = 0.0  # draft probability 0 -> accept probability 1
+    draft = np.stack([[rng.choice(vocab, p=q[b, i].astype(np.float64) / q[b, i].astype(np.float64).sum())
+                       if q[b, i].sum() > 0 else 0 for i in range(K)] for b in range(batch)]).astype(np.int32)
+    uf = rng.random((batch, K)).astype(np.float32)
+    ud = rng.random(batch)
+    acc, tok = ctx.spec_verify(torch.from_numpy(p).cuda(), torch.from_numpy(q).cuda(), torch.from_numpy(draft).cuda(),
+                               torch.from_numpy(uf).cuda(), torch.from_numpy(ud).cuda())
+    oacc, otok = orc.spec_verify_dense(p, q, draft, uf, ud)
+    assert np.array_equal(acc.cpu().numpy(), oacc)
+    assert np.array_equal(tok.cpu().numpy(), otok)
+    assert len(set(oacc.tolist())) > 1 or batch < 4
