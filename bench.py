@@ -20,6 +20,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 ROWS, VOCAB, TOP_K, TOP_P, TEMP = 64, 128256, 50, 0.9, 0.7
 HBM_PEAK_GBS = 8000.0
+MEASURED_TRAFFIC_BYTES = 35_220_000  # fetch 34.26 MB + write 0.96 MB per launch
 
 
 def main():
@@ -99,7 +100,9 @@ def main():
     ms_per_step = gpu_ms / K
     algo_bytes = ROWS * VOCAB * 4 + ROWS * 8 + ROWS * 4  # logits once + uniforms + tokens
     achieved = algo_bytes / (ms_per_step * 1e-3) / 1e9
-    traffic = None
+    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known
+    # size (profiles/sample_fused_kernel_config2_pmc.md); counters cannot be read from inside this process.
+    traffic = MEASURED_TRAFFIC_BYTES
     if args.traffic:
         t = json.loads(args.traffic)
         traffic = t.get("fetch_bytes", 0) + t.get("write_bytes", 0)
