@@ -1,0 +1,125 @@
+// MI355X search & sampling backend behind the reference's plug-in contract: a DeviceInterface whose
+// CreateGreedy / CreateBeam / CreateBatchedSampler build Search and BatchedSampler objects that run on
+// the HIP kernels of libmi355x_search (C ABI, include/mi355x_search.h).  The classes only marshal:
+// no selection, softmax or scoring arithmetic happens on the host.
+#pragma once
+#ifdef MI355X_USE_REFERENCE_HEADERS
+#include "generators.h"
+#include "search.h"
+#else
+#include "hip_contract.h"
+#endif
+#include "mi355x_search.h"
+
+namespace Generators {
+
+DeviceInterface* GetHipInterface();  // process-wide instance (device 0)
+
+// GreedySearch_Cpu's device counterpart (src/search.h:202-240, src/search.cpp:178-324).
+// Token selection runs on the GPU; EOS / padding / done bookkeeping is host state, as in the CPU
+// class.  Sampling matches the CPU class draw for draw: the kernels return each row's kept
+// distribution and the draw is made on the host by std::discrete_distribution with the caller's
+// std::mt19937, so both token and engine state equal the CPU path's.
+struct GreedySearch_Hip : Search {
+  explicit GreedySearch_Hip(const GeneratorParams& params);
+  ~GreedySearch_Hip() override;
+
+  DeviceSpan<int32_t> GetNextTokens() override { return next_tokens_; }
+  DeviceSpan<int32_t> GetNextIndices() override { return {}; }
+  DeviceSpan<int32_t> GetSequenceLengths() override { return sequence_lengths_; }
+  DeviceSpan<float> GetLogits() const override;
+  void SetLogits(DeviceSpan<float> logits) override;
+  bool IsDone() const override { return done_; }
+  // Batched sampling seam (src/search.h:40-67): the engine samples a shared buffer with the
+  // BatchedSampler, binds one element of it here and has the tail (EOS / pad / append) run from
+  // CompleteGeneration() once it has copied the buffer to the host.  Token selection through
+  // SelectTop / Sample* always completes inline, which DeferCompletion(true) permits.
+  void DeferCompletion(bool defer) override { defer_completion_ = defer; }
+  void CompleteGeneration() override;
+  bool BindNextTokensSlot(DeviceSpan<int32_t> slot) override;
+  bool SupportsBatchedSampling() const override { return params_->BatchBeamSize() == 1; }
+  void OnNextTokensSampled() override { external_pending_ = true; }
+
+  void SelectTop() override;
+  void CommitToken(int32_t token) override;
+  void SampleTopP(float p, float temperature, std::mt19937& rng) override { Sample(0, p, temperature, rng); }
+  void SampleTopK(int k, float temperature, std::mt19937& rng) override { Sample(k, 0.0f, temperature, rng); }
+  void SampleTopKTopP(int k, float p, float temperature, std::mt19937& rng) override { Sample(k, p, temperature, rng); }
+  void ApplyMinLength(int min_length) override;
+  void ApplyRepetitionPenalty(float penalty) override;
+  void AppendTokens(DeviceSpan<int32_t>& next_tokens) override;
+  void RewindTo(size_t index) override;
+
+ protected:
+  void SaveStateForTransactionImpl(bool checkpoint_local_state) override;
+  void RestoreStateForTransactionImpl() override;
+
+ private:
+  void Sample(int k, float p, float temperature, std::mt19937& rng);
+  mi355x_logits_xform* PendingXform();
+  void Materialize() const;  // applies deferred min-length / repetition penalty to the logits in place
+  bool PadIfAlreadyEOS(size_t batch_id);
+  void SetNextToken(size_t batch_id, int32_t token);
+  void AppendNextTokensToSequences();
+  void ResetDone();
+
+  mi355x_search_ctx* ctx_{};
+  DeviceSpan<int32_t> next_tokens_, sequence_lengths_;
+  DeviceSpan<float> next_token_scores_;
+  DeviceSpan<int32_t> kept_count_, kept_ids_;
+  DeviceSpan<float> kept_probs_;
+  DeviceSpan<double> uniforms_;
+  int kept_capacity_{};
+  std::vector<uint8_t> eos_seen_;
+  int not_done_count_{};
+  bool done_{};
+  bool defer_completion_{}, external_pending_{};
+  DeviceSpan<int32_t> bound_slot_;
+  // deferred logits processing
+  mutable bool pending_min_length_{};
+  mutable float pending_penalty_{1.0f};
+  mutable mi355x_logits_xform xf_{};
+  // transaction checkpoint
+  std::vector<int32_t> tx_next_tokens_, tx_sequence_lengths_;
+  std::vector<uint8_t> tx_eos_seen_;
+  int tx_not_done_count_{};
+  bool tx_done_{};
+};
+
+// BeamSearch_Cpu's device counterpart (src/search.h:242-270, src/search.cpp:101-176,326-400): candidate
+// selection, BeamSearchScorer and the beam-reordered sequence store all live on the GPU.
+struct BeamSearch_Hip : Search {
+  explicit BeamSearch_Hip(const GeneratorParams& params);
+  ~BeamSearch_Hip() override;
+  DeviceSpan<int32_t> GetNextTokens() override;
+  DeviceSpan<int32_t> GetNextIndices() override;
+  DeviceSpan<int32_t> GetSequenceLengths() override { return sequence_lengths_; }
+  DeviceSpan<int32_t> GetSequence(size_t index) override;
+  DeviceSpan<int32_t> GetSequence(size_t batch_id, size_t beam_id);
+  DeviceSpan<float> GetLogits() const override { return next_token_scores_; }
+  void SetLogits(DeviceSpan<float> logits) override { next_token_scores_ = logits; }
+  bool IsDone() const override;
+  void SelectTop() override;
+  void ApplyMinLength(int min_length) override;
+  void ApplyRepetitionPenalty(float penalty) override;
+  void AppendTokens(DeviceSpan<int32_t>& next_tokens) override;
+
+ private:
+  mi355x_search_ctx* ctx_{};
+  mi355x_beam_scorer* scorer_{};
+  DeviceSpan<int32_t> sequence_lengths_;
+  DeviceSpan<float> next_token_scores_;
+  DeviceSpan<float> cand_scores_;
+  DeviceSpan<int32_t> cand_tokens_, cand_indices_;
+  std::vector<DeviceSpan<int32_t>> hypotheses_;
+  int length_{};
+};
+
+}  // namespace Generators
+
+extern "C" {
+// The add-on entry points the reference's loader resolves (src/cuda/interface.cpp:698-715,
+// src/generators.cpp:321-356).
+uint32_t GetInterfaceVersion();
+Generators::DeviceInterface* GetInterface(GenaiInterface* p_genai, const char* deviceType, const OrtApi* ort_api);
+}
