@@ -128,7 +128,7 @@ def main():
                    "general_path_rows": fallback},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "sample_stream_kernel", "algorithmic_bytes_per_launch": algo_bytes},
+                     "kernel": "sample_fused_kernel", "algorithmic_bytes_per_launch": algo_bytes},
         "cpu_baseline": {"value": ROWS * n_cpu / cpu_s, "unit": "tokens/s", "cores": 1, "kind": "port",
                          "sample": "%d of the %d timed steps (same logits and uniforms), oracle/search_oracle.cpp "
                                    "orc_sample_batch, one thread as in the reference's serial row loop" % (n_cpu, K),
