@@ -17,6 +17,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
+sys.path.insert(0, os.path.join(ROOT, "onnxruntime-genai_amd"))
 
 ROWS, VOCAB, TOP_K, TOP_P, TEMP = 64, 128256, 50, 0.9, 0.7
 HBM_PEAK_GBS = 8000.0
@@ -31,6 +32,9 @@ def main():
     ap.add_argument("--pool", type=int, default=32, help="distinct logits buffers cycled through")
     ap.add_argument("--cpu-steps", type=int, default=24, help="steps replayed on the CPU oracle")
     ap.add_argument("--traffic", type=str, default=None, help="JSON {fetch_bytes, write_bytes} from rocprofv3 --pmc")
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
+                    help="c2 (default) is the headline configuration; the others time the remaining "
+                         "configurations with the same JSON shape")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (rows shard across GPUs "
@@ -45,6 +49,10 @@ def main():
     orc = orc_lib.Oracle()
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if args.workload != "c2":
+        import other_workloads
+        print(json.dumps(other_workloads.run(args, pkg, orc, orc_lib, dev)))
+        return
     K, W = args.steps, args.warmup
     pool = max(2, min(args.pool, K + W))
 

@@ -10,23 +10,19 @@ namespace ms {
 constexpr int kIntMax = 0x7fffffff;
 
 struct SeqShared {
-  Step wave_tot[16];
+  // block_seq_sum: double-buffered by pass parity so a pass needs two barriers only
+  Step wave_tot[2][16];
+  uint32_t ev_key[2][16];
+  float ev_a[2][16], ev_b[2][16];
+  uint32_t n_last[2];
+  // block_discrete_draw / block_min2
   int red_a[16];
   int red_b[16];
   double dred[16];
   double dscan[16];
-  float s_before, e_cross, result;
-  uint32_t n_last;
   int bcast_i;
   double bcast_d;
 };
-
-__device__ __forceinline__ Step shfl_up_step(Step x, int d) {
-  Step y;
-  y.d0 = __shfl_up(x.d0, d, 64);
-  y.d1 = __shfl_up(x.d1, d, 64);
-  return y;
-}
 
 __device__ __forceinline__ int wave_min_i(int v) {
 #pragma unroll
@@ -57,6 +53,36 @@ __device__ __forceinline__ void block_min2(int& a, int& b, SeqShared& sh) {
   b = rb;
 }
 
+// Value of the lane `d` below (row_shr inside a row of 16, then the row broadcasts), 0 where there
+// is no such lane: 0/0 is the identity Step, so the scan below needs no lane tests.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ Step step_from_below(Step x) {
+  Step y;
+  y.d0 = __builtin_amdgcn_update_dpp(0u, x.d0, CTRL, ROW_MASK, 0xf, false);
+  y.d1 = __builtin_amdgcn_update_dpp(0u, x.d1, CTRL, ROW_MASK, 0xf, false);
+  return y;
+}
+
+// Inclusive scan of Steps over the wave (lane order), data-parallel-primitive moves only.
+__device__ __forceinline__ Step wave_scan_steps(Step x) {
+  x = step_compose(step_from_below<0x111, 0xf>(x), x);  // row_shr:1
+  x = step_compose(step_from_below<0x112, 0xf>(x), x);  // row_shr:2
+  x = step_compose(step_from_below<0x114, 0xf>(x), x);  // row_shr:4
+  x = step_compose(step_from_below<0x118, 0xf>(x), x);  // row_shr:8
+  x = step_compose(step_from_below<0x142, 0xa>(x), x);  // row_bcast:15 into rows 1 and 3
+  x = step_compose(step_from_below<0x143, 0xc>(x), x);  // row_bcast:31 into rows 2 and 3
+  return x;
+}
+
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    const uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), m, 64));
+    v = o < v ? o : v;
+  }
+  return v;
+}
+
 struct NoStop {
   __device__ bool operator()(float, float, int) const { return false; }
 };
@@ -66,95 +92,107 @@ struct NoStop {
 // If stop(prefix_i, e(i), i) holds for some i -- prefix_i being the sum including e(i) -- the scan
 // ends at the first such i: *stop_index = i and the returned value is prefix_i.  Otherwise
 // *stop_index = -1 and the value is the full sum.  e(i) must be finite and >= 0.
+//
+// The addends of a window (blockDim * ITEMS elements) are evaluated once and kept in registers.  A
+// pass scans the part of the window not yet folded into the sum under the sum's current binade and
+// finds the first event: the addition that leaves the binade (done with a real float add, after
+// which the rest of the window is scanned again under the new binade) or the first index where the
+// predicate holds.  Passes cost two barriers; there is one per window plus one per binade change.
 template <int ITEMS, typename GetE, typename StopFn>
 __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop_index, SeqShared& sh) {
-  const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+  const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6, nw = static_cast<int>(blockDim.x) >> 6;
+  const int span = static_cast<int>(blockDim.x) * ITEMS;
+  constexpr uint32_t kNone = 0xffffffffu;
   float s = s0;
-  int i0 = 0, found = -1;
-  // Items per thread in the current window.  A window is redone from the element behind a binade
-  // change, and those cluster at the start of a sum, so windows start small and double while no
-  // change occurs.
-  int items = 1;
-  while (i0 < n) {
-    const SeqState st = seq_decompose(s);
-    const int span = static_cast<int>(blockDim.x) * items;
-    const int base = i0 + tid * items;
-    const int window_end = (n - i0 < span) ? n : i0 + span;
+  int found = -1;
+  int par = 0;
+  __syncthreads();  // a previous call's readers are done with the parity-0 buffers
+  for (int w0 = 0; w0 < n && found < 0; w0 += span) {
+    const int base = w0 + tid * ITEMS;
+    const int wend = (n - w0 < span) ? n : w0 + span;
     float ev[ITEMS];
-    Step f[ITEMS];
-    Step agg{0u, 0u};
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-      const int idx = base + j;
-      const bool on = j < items && idx < window_end;
-      ev[j] = on ? get(idx) : 0.0f;
-      f[j] = seq_make_step(ev[j], st.se);
-      agg = step_compose(agg, f[j]);
-    }
-    Step x = agg;
+    for (int j = 0; j < ITEMS; ++j) ev[j] = (base + j < wend) ? get(base + j) : 0.0f;
+    int start = w0;  // first index not yet folded into s
+    while (true) {
+      const SeqState st = seq_decompose(s);
+      Step f[ITEMS];
+      Step agg{0u, 0u};
 #pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const Step y = shfl_up_step(x, d);
-      if (lane >= d) x = step_compose(y, x);
-    }
-    if (lane == 63) sh.wave_tot[wave] = x;
-    __syncthreads();
-    Step ex = shfl_up_step(x, 1);
-    if (lane == 0) ex = Step{0u, 0u};
-    Step wp{0u, 0u};
-    for (int w = 0; w < wave; ++w) wp = step_compose(wp, sh.wave_tot[w]);
-    ex = step_compose(wp, ex);
-    uint32_t nn = step_apply(st.n, ex);
-    int lc = kIntMax, ls = kIntMax;
-    float lpf = 0.0f;
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-      const int idx = base + j;
-      if (j < items && idx < window_end) {
-        const uint32_t nn2 = step_apply(nn, f[j]);
-        if (nn2 >= kMantLimit) {
-          if (nn < kMantLimit) {  // the one addition that leaves the binade
-            sh.s_before = seq_recompose(nn, st.se);
-            sh.e_cross = ev[j];
-          }
-          lc = idx < lc ? idx : lc;
-        } else {
-          const float pf = seq_recompose(nn2, st.se);
-          if (ls == kIntMax && stop(pf, ev[j], idx)) {
-            ls = idx;
-            lpf = pf;
-          }
-          if (idx == window_end - 1) sh.n_last = nn2;
-        }
-        nn = nn2;
+      for (int j = 0; j < ITEMS; ++j) {
+        const int idx = base + j;
+        f[j] = (idx >= start && idx < wend) ? seq_make_step(ev[j], st.se) : Step{0u, 0u};
+        agg = step_compose(agg, f[j]);
       }
-    }
-    int gc = lc, gs = ls;
-    block_min2(gc, gs, sh);
-    if (gs < gc) {  // predicate satisfied before any binade change
-      if (ls == gs) sh.result = lpf;
+      const Step inc = wave_scan_steps(agg);
+      if (lane == 63) sh.wave_tot[par][wave] = inc;
       __syncthreads();
-      s = sh.result;
-      found = gs;
+      Step ex = step_from_below<0x138, 0xf>(inc);  // wave_shr:1, identity into lane 0
+      Step wp{0u, 0u};
+      for (int w = 0; w < wave; ++w) wp = step_compose(wp, sh.wave_tot[par][w]);
+      ex = step_compose(wp, ex);
+      uint32_t nn = step_apply(st.n, ex);
+      uint32_t key = kNone;
+      float pa = 0.0f, pb = 0.0f;
+#pragma unroll
+      for (int j = 0; j < ITEMS; ++j) {
+        const int idx = base + j;
+        if (idx >= start && idx < wend) {
+          const uint32_t nn2 = step_apply(nn, f[j]);
+          if (key == kNone) {
+            if (nn2 >= kMantLimit) {  // leaves the binade here (or an earlier thread's element did)
+              key = (static_cast<uint32_t>(idx) << 1) | 1u;
+              pa = seq_recompose(nn < kMantLimit ? nn : 0u, st.se);
+              pb = ev[j];
+            } else {
+              const float pf = seq_recompose(nn2, st.se);
+              if (stop(pf, ev[j], idx)) {
+                key = static_cast<uint32_t>(idx) << 1;
+                pa = pf;
+              }
+            }
+          }
+          nn = nn2;
+        }
+      }
+      if (wend - 1 >= base && wend - 1 < base + ITEMS) sh.n_last[par] = nn;
+      const uint32_t wkey = wave_min_u32(key);
+      if (key == wkey && (key != kNone || lane == 0)) {
+        sh.ev_key[par][wave] = key;
+        sh.ev_a[par][wave] = pa;
+        sh.ev_b[par][wave] = pb;
+      }
       __syncthreads();
-      break;
-    }
-    if (gc == kIntMax) {
-      s = seq_recompose(sh.n_last, st.se);
-      i0 = window_end;
-      if (items < ITEMS) items *= 2;
-    } else {
-      items = 1;
-      const float e_cross = sh.e_cross;
-      s = sh.s_before + e_cross;
-      if (stop(s, e_cross, gc)) {
-        found = gc;
-        __syncthreads();
+      uint32_t gk = kNone;
+      float ga = 0.0f, gb = 0.0f;
+      for (int w = 0; w < nw; ++w) {
+        const uint32_t k2 = sh.ev_key[par][w];
+        if (k2 < gk) {
+          gk = k2;
+          ga = sh.ev_a[par][w];
+          gb = sh.ev_b[par][w];
+        }
+      }
+      const uint32_t n_last = sh.n_last[par];
+      par ^= 1;
+      if (gk == kNone) {  // the rest of the window stayed inside the binade
+        s = seq_recompose(n_last, st.se);
         break;
       }
-      i0 = gc + 1;
+      const int at = static_cast<int>(gk >> 1);
+      if ((gk & 1u) == 0u) {  // predicate satisfied before any binade change
+        s = ga;
+        found = at;
+        break;
+      }
+      s = ga + gb;  // the one addition that leaves the binade
+      if (stop(s, gb, at)) {
+        found = at;
+        break;
+      }
+      start = at + 1;
+      if (start >= wend) break;
     }
-    __syncthreads();
   }
   *stop_index = found;
   return s;
