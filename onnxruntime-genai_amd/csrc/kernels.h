@@ -13,9 +13,9 @@ constexpr int kSWaves = kSBlock / 64;
 constexpr int kSVec = 16;                   // 128-bit loads per thread
 constexpr int kSElems = kSVec * 4;          // logits held in registers per thread
 constexpr int kSChunk = kSBlock * kSElems;  // logits per workgroup
-constexpr int kSmallCap = 256;       // candidate slots per chunk on the k<=64 path
-constexpr int kAllCap = 4096;        // merged candidates a finishing workgroup can hold (16 chunks x kSmallCap)
-constexpr int kSelCap = 256;         // survivors of the second bound handed to the finishing wave
+constexpr int kSmallCap = 64;        // sorted candidates a chunk publishes on the k<=64 path
+constexpr int kListCap = 128;        // candidates a chunk can hold before its sort
+constexpr int kAllCap = 1024;        // slots a finishing workgroup ranks (16 chunks x kSmallCap)
 constexpr int kNucleusCap = 16384;   // sorted nucleus candidates held in LDS by the finish kernel
 constexpr int kFinishBlock = 1024;
 
@@ -37,7 +37,7 @@ struct SampleArgs {
   float* kept_probs;
   int kept_capacity;
   // workspace
-  u64* cand_small;        // [rows][chunks][kSmallCap]
+  u64* cand_small;        // [rows][chunks][kSmallCap], every slot rewritten by every launch
   uint32_t* chunk_cnt;    // [rows][chunks]
   uint32_t* chunk_max;    // [rows][chunks]
   u64* chunk_next;        // [rows][chunks]

@@ -2,9 +2,10 @@
 //
 // sample_fused_kernel: one launch per step.  Every workgroup (256 threads x 64 logits) streams one
 // 16K-logit chunk of one row with 128-bit non-temporal loads (logits processing fused), keeps the chunk's
-// candidates for the row's top-k and publishes them; the last workgroup of a row to arrive merges the
-// row's candidates, sorts the k survivors and runs the reference's scalar epilogue (softmax over the
-// k, nucleus cut, categorical draw) in rank order.  Rows in nucleus mode (k <= 1) only compact their
+// best 64 candidates for the row's top-k and publishes them sorted; the last workgroup of a row to
+// arrive merges the chunks' sorted lists pairwise (bitonic merges in registers, three levels for
+// eight chunks) and runs the reference's scalar epilogue (softmax over the k, nucleus cut, categorical draw) in rank
+// order.  Rows in nucleus mode (k <= 1) only compact their
 // candidates here; nucleus_finish_kernel sorts them and finishes.  Anything the fast paths decline
 // (k > 64, heavy ties, tiny vocabularies) goes through general_row, an exact full sort.
 #include "kernels.h"
@@ -23,23 +24,30 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 // Serial prefix over lanes: out[l] = ((x[0] + x[1]) + ...) + x[l], additions in lane order, as the
 // reference's scalar loops do.  One DPP-shifted add per element (wave_shr:1, lane 0 reads 0).
+// Steps run in unrolled groups of 8: a step past `count` leaves lanes below `count` unchanged.
 __device__ __forceinline__ float wave_serial_prefix(float x, int count) {
   float s = 0.0f;
-  for (int t = 0; t < count; ++t) {
-    const float prev = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s), 0x138, 0xf, 0xf, false));
-    s = prev + x;
+  for (int t = 0; t < count; t += 8) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const float prev = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s), 0x138, 0xf, 0xf, false));
+      s = prev + x;
+    }
   }
   return s;
 }
 
 __device__ __forceinline__ double wave_serial_prefix(double x, int count) {
   double s = 0.0;
-  for (int t = 0; t < count; ++t) {
-    const u64 b = static_cast<u64>(__double_as_longlong(s));
-    const uint32_t lo = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b), 0x138, 0xf, 0xf, false);
-    const uint32_t hi = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b >> 32), 0x138, 0xf, 0xf, false);
-    const double prev = __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
-    s = prev + x;
+  for (int t = 0; t < count; t += 4) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const u64 b = static_cast<u64>(__double_as_longlong(s));
+      const uint32_t lo = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b), 0x138, 0xf, 0xf, false);
+      const uint32_t hi = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b >> 32), 0x138, 0xf, 0xf, false);
+      const double prev = __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
+      s = prev + x;
+    }
   }
   return s;
 }
@@ -131,14 +139,16 @@ constexpr uint32_t kPark = 6u;  // float4s with a hit a thread can park per chun
 // LDS of the fused kernel.
 struct FusedShared {
   uint32_t hist_bits[kSChunk / 32];
-  u64 all[kAllCap];   // merged candidates of a row (finishing workgroup only)
-  u64 sel[kSelCap];
+  u64 lists[kAllCap];   // the chunks' sorted candidate lists of a row (finishing workgroup only)
+  u64 list[kListCap];   // this chunk's candidates before the sort
+  u64 list_hi[64];      // second half of a long list, sorted ascending
+  u64 lists2[kAllCap / 2];  // second buffer of the merge tree
   float4 park_val[kSBlock * kPark];  // per-thread parking rows of the streaming filter
   int park_idx[kSBlock * kPark];
   uint32_t pool[64];
   uint32_t wave_val[kSWaves];
   u64 wave_val64[kSWaves];
-  uint32_t count, count2, flag, redo, bound;
+  uint32_t count, flag, bound;
   SeqShared seq;
 };
 
@@ -272,10 +282,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   }
   const uint32_t lmax = elem_index(chunk, 0, 0) < V ? order_key(fm) : 0u;  // 0: thread holds no element
   MS_STAGE(1, lmax);
-  if (tid == 0) {
-    sm.count = 0u;
-    sm.redo = 0u;
-  }
+  if (tid == 0) sm.count = 0u;
 
   if (mode == kModeNucleus) {
     const uint32_t cmax = block_max<uint32_t>(lmax, sm.wave_val);  // barriers inside publish count = 0
@@ -316,10 +323,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   if (tau == 0u) {
     // The pooled bound found fewer than k offers (a short tail chunk keeps its elements in one or two
     // waves): take the exact k-th best of the 256 per-thread maxima instead.
-    sm.all[tid] = static_cast<u64>(lmax);
+    sm.lists[tid] = static_cast<u64>(lmax);
     __syncthreads();
-    block_sort_desc(sm.all, kSBlock);
-    tau = static_cast<uint32_t>(sm.all[kk - 1]);
+    block_sort_desc(sm.lists, kSBlock);
+    tau = static_cast<uint32_t>(sm.lists[kk - 1]);
     __syncthreads();
   }
   MS_STAGE(2, tau);
@@ -374,31 +381,51 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         if (qv[c] >= tau_f) {
-          // key64 of a real element is never 0 (its index half is ~idx != 0), so 0 marks an empty slot
-          if (pos < kSmallCap) store_coherent(&dst[pos], make_key64(order_key(qv[c]), id0 + c));
+          if (pos < kListCap) sm.list[pos] = make_key64(order_key(qv[c]), id0 + c);
           ++pos;
         }
       }
     }
   }
-  MS_STAGE(3, tau);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this lane's candidate stores have been performed
   __syncthreads();
-  MS_STAGE(4, tau);
-  if (tid == 0) {
-    // low half: arrivals; high half: number of chunks whose candidates did not fit their slots
-    const uint32_t add = 1u + (n_c > kSmallCap ? 0x10000u : 0u);
-    const uint32_t old = __hip_atomic_fetch_add(&a.row_arrive[row], add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    sm.flag = ((old & 0xffffu) == static_cast<uint32_t>(a.chunks) - 1u) ? (old + add) : 0u;
+  MS_STAGE(3, tau);
+  // The chunk publishes its best 64 candidates sorted (best first, zero-padded): nothing ranked lower
+  // inside its own chunk can be among the row's k <= 64 best.  Waves 0 and 1 sort one half of the
+  // list each; wave 0 merges, stores, and -- once its stores have been performed -- signals arrival.
+  const bool overflow = n_c > static_cast<uint32_t>(kListCap);
+  const bool two_halves = n_c > 64u;
+  u64 mykey = 0;
+  if (wave < 2 && !overflow) {
+    const uint32_t p = static_cast<uint32_t>(wave) * 64u + static_cast<uint32_t>(lane);
+    mykey = p < n_c ? sm.list[p] : 0;
+    if (wave == 0 || two_halves) mykey = wave_sort_desc_fast<u64>(mykey);
+    if (wave == 1 && two_halves) sm.list_hi[63 - lane] = mykey;
+  }
+  if (two_halves && !overflow) __syncthreads();
+  if (wave == 0) {
+    if (!overflow) {
+      if (two_halves) {
+        const u64 other = sm.list_hi[lane];  // ascending against descending: a bitonic pair
+        mykey = other > mykey ? other : mykey;
+        sort_merge<64, 32, u64>(mykey, lane);
+      }
+      store_coherent(&dst[lane], mykey);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the wave's candidate stores have been performed
+    }
+    if (lane == 0) {
+      // low half: arrivals; high half: number of chunks whose candidates did not fit
+      const uint32_t add = 1u + (overflow ? 0x10000u : 0u);
+      const uint32_t old = __hip_atomic_fetch_add(&a.row_arrive[row], add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      sm.flag = ((old & 0xffffu) == static_cast<uint32_t>(a.chunks) - 1u) ? (old + add) : 0u;
+      sm.count = 0u;
+    }
   }
   __syncthreads();
   const uint32_t state = sm.flag;
   MS_STAGE(5, state);
   if (state == 0u) return false;
 
-  // ---- last workgroup of the row: merge the chunks' candidates -----------------------------------
-  // Slots are all-zero between launches; a non-zero slot is a candidate of this launch.  Read them
-  // with coherent loads, clear them for the next launch, and compact the live ones into LDS.
+  // ---- last workgroup of the row: rank the chunks' sorted lists against each other ----------------
   LaneExp2Tab tab;
   {
     const uint64_t t = g_exp2_tab[lane & 31];  // issued now, consumed by the epilogue
@@ -406,114 +433,63 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     tab.hi = static_cast<uint32_t>(t >> 32);
   }
   const double u = a.emit_topk ? 0.0 : a.uniforms[row];
-  if (tid == 0) {
-    a.row_arrive[row] = 0u;
-    sm.count = 0u;
-    sm.count2 = 0u;
-  }
-  __syncthreads();
-  const int slots = a.chunks * kSmallCap;
-  u64* seg = a.cand_small + static_cast<size_t>(row) * a.chunks * kSmallCap;
-  for (int p0 = 0; p0 < slots; p0 += kSBlock * 8) {
-    u64 k64[8];
+  if (tid == 0) a.row_arrive[row] = 0u;
+  if ((state >> 16) != 0u) return true;  // a chunk could not list its candidates
+  const int nslots = a.chunks * kSmallCap;
+  const u64* seg = a.cand_small + static_cast<size_t>(row) * a.chunks * kSmallCap;
+  constexpr int kRegs = kAllCap / kSBlock;
+  {
+    u64 mine[kRegs];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const int p = p0 + r * kSBlock + tid;
-      k64[r] = p < slots ? load_coherent(&seg[p]) : 0;
+    for (int r = 0; r < kRegs; ++r) {
+      const int p = r * kSBlock + tid;
+      mine[r] = p < nslots ? load_coherent(&seg[p]) : 0;
     }
-    // one LDS atomic per wave for all 8 registers
-    uint32_t before[8];
-    uint32_t wave_total = 0u;
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const u64 b = __ballot(k64[r] != 0);
-      before[r] = wave_total + static_cast<uint32_t>(__popcll(b & ((1ull << lane) - 1ull)));
-      wave_total += static_cast<uint32_t>(__popcll(b));
-    }
-    uint32_t base = 0u;
-    if (lane == 0 && wave_total != 0u) base = atomicAdd(&sm.count, wave_total);
-    base = __builtin_amdgcn_readfirstlane(base);
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      if (k64[r] != 0) {
-        sm.all[base + before[r]] = k64[r];
-        seg[p0 + r * kSBlock + tid] = 0;
-      }
+    for (int r = 0; r < kRegs; ++r) {
+      const int p = r * kSBlock + tid;
+      if (p < nslots) sm.lists[p] = mine[r];
     }
   }
   __syncthreads();
   MS_STAGE(6, sm.count);
-  const int total = static_cast<int>(sm.count);
-  if ((state >> 16) != 0u || total < kk) return true;  // slots overflowed, or NaNs are needed to fill k
+  // Merge tree over the sorted lists: a descending list against a reversed one is a bitonic pair
+  // whose lane-wise maximum holds the 64 best of both; six exchange stages sort it again.  Levels
+  // alternate between two LDS buffers; the last level leaves the row's 64 best in wave 0's lanes.
   u64 final_key = 0;
-  if (total <= 64) {
-    if (tid < 64) final_key = tid < total ? sm.all[tid] : 0;
-  } else {
-    // Typical rows merge ~450 candidates (two registers per thread); the loops are bounded by the
-    // number of registers actually needed.
-    constexpr int kRegs = kAllCap / kSBlock;
-    const int nreg = (total + kSBlock - 1) / kSBlock;
-    u64 mine[kRegs];
-    uint32_t mk = 0u;
-#pragma unroll
-    for (int r = 0; r < kRegs; ++r) {
-      mine[r] = 0;
-      if (r < nreg) {
-        const int p = r * kSBlock + tid;
-        mine[r] = p < total ? sm.all[p] : 0;
-        const uint32_t ok = key64_okey(mine[r]);
-        mk = ok > mk ? ok : mk;
-      }
-    }
-    const int nw2 = total >= kSBlock ? kSWaves : (total + 63) / 64;
-    const uint32_t tau2 = block_pool_bound(mk, kk, nw2, sm.pool, &sm.bound);
-#pragma unroll
-    for (int r = 0; r < kRegs; ++r) {
-      if (r < nreg) {
-        const bool cand = mine[r] != 0 && key64_okey(mine[r]) >= tau2;
-        const uint32_t pos = wave_slot(cand, &sm.count2);
-        if (cand && pos < kSelCap) sm.sel[pos] = mine[r];
-      }
-    }
-    __syncthreads();
-    const uint32_t n_sel = sm.count2;
-    MS_STAGE(7, n_sel);
-    if (n_sel > kSelCap) return true;  // heavy ties at the bound
-    if (tid < 64) {
-      uint32_t sk[kSelCap / 64];
-      u64 sk64[kSelCap / 64];
-#pragma unroll
-      for (int r = 0; r < kSelCap / 64; ++r) {
-        const uint32_t p = r * 64 + lane;
-        sk64[r] = p < n_sel ? sm.sel[p] : 0;
-        sk[r] = key64_okey(sk64[r]);
-      }
-      if (n_sel <= 64u) {
-        final_key = sk64[0];
-      } else {
-        // exact k-th best score among the survivors, then one key per lane
-        const uint32_t tau3 = wave_kth_largest<kSelCap / 64>(sk, kk);
-        int base = 0;
-#pragma unroll
-        for (int r = 0; r < kSelCap / 64; ++r) {
-          const bool in = sk64[r] != 0 && sk[r] >= tau3;
-          const u64 b = __ballot(in);
-          const int dl = base + __popcll(b & ((1ull << lane) - 1ull));
-          if (in && dl < 64) sm.sel[dl] = sk64[r];
-          base += __popcll(b);
+  {
+    u64* src = sm.lists;
+    u64* dstl = sm.lists2;
+    int n = a.chunks;
+    if (n == 1 && wave == 0) final_key = src[lane];
+    while (n > 1) {
+      const int pairs = (n + 1) >> 1;
+      for (int q = wave; q < pairs; q += kSWaves) {
+        u64 x = src[(2 * q) * kSmallCap + lane];
+        if (2 * q + 1 < n) {
+          const u64 y = src[(2 * q + 1) * kSmallCap + 63 - lane];
+          x = y > x ? y : x;
+          sort_merge<64, 32, u64>(x, lane);
         }
-        if (base > 64) {
-          if (lane == 0) sm.redo = 1u;  // more than 64 keys tie with the k-th best: exact path decides
-        } else {
-          final_key = lane < base ? sm.sel[lane] : 0;
-        }
+        if (pairs > 1) dstl[q * kSmallCap + lane] = x;
+        else final_key = x;
       }
+      if (pairs > 1) __syncthreads();
+      u64* t = src;
+      src = dstl;
+      dstl = t;
+      n = pairs;
     }
   }
-  MS_STAGE(8, (uint32_t)final_key);
-  if (tid < 64 && sm.redo == 0u) {
-    final_key = wave_sort_desc_fast<u64>(final_key);
-    MS_STAGE(9, (uint32_t)final_key);
+  if (tid < 64) {
+    const u64 kth = shfl_t<u64>(final_key, kk - 1);
+    if (lane == 0) sm.flag = kth != 0 ? 1u : 0u;
+  }
+  __syncthreads();
+  MS_STAGE(8, sm.count);
+  if (sm.flag == 0u) return true;  // NaNs are needed to fill k: the exact path decides
+  if (tid < 64) {
+    if (lane >= kk) final_key = 0;
     if (a.emit_topk) {
       if (lane < kk) {
         a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(key64_index(final_key));
@@ -523,8 +499,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
       wave_topk_epilogue(final_key, kk, prm, u, tab, row_outputs(a, row));
     }
   }
-  __syncthreads();
-  return sm.redo != 0u;
+  return false;
 }
 
 __global__ __launch_bounds__(kSBlock) void sample_fused_kernel(const SampleArgs a) {
