@@ -139,6 +139,7 @@ constexpr uint32_t kPark = 6u;  // float4s with a hit a thread can park per chun
 // LDS of the fused kernel.
 struct FusedShared {
   uint32_t hist_bits[kSChunk / 32];
+  uint32_t mask_bits[kSChunk / 32];
   u64 lists[kAllCap];   // the chunks' sorted candidate lists of a row (finishing workgroup only)
   u64 list[kListCap];   // this chunk's candidates before the sort
   u64 list_hi[64];      // second half of a long list, sorted ascending
@@ -249,10 +250,22 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     }
   }
   if (a.xf.active()) {
+    // The chunk's grammar-mask words and the bitmap of history ids are staged in LDS once; a thread
+    // then needs one nibble of each per float4.
     const bool pen = a.xf.use_penalty();
-    if (pen) {
+    const bool has_mask = a.xf.mask != nullptr;
+    if (pen)
       for (int i = tid; i < kSChunk / 32; i += kSBlock) sm.hist_bits[i] = 0u;
-      __syncthreads();
+    if (has_mask) {
+      const int words = (V - 1) / 32 + 1;
+      const uint32_t* mrow = a.xf.mask + static_cast<size_t>(row) * words;
+      for (int i = tid; i < kSChunk / 32; i += kSBlock) {
+        const int w = chunk * (kSChunk / 32) + i;
+        sm.mask_bits[i] = w < words ? mrow[w] : 0u;
+      }
+    }
+    __syncthreads();
+    if (pen) {
       const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
       for (int i = tid; i < a.xf.history_len; i += kSBlock) {
         const int rel = h[i] - chunk * kSChunk;
@@ -260,15 +273,24 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
       }
       __syncthreads();
     }
-    const bool has_mask = a.xf.mask != nullptr;
-    const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
+    const float penalty = a.xf.penalty;
 #pragma unroll
-    for (int e = 0; e < kSElems; ++e) {
-      const int idx = elem_index(chunk, e / 4, e % 4);
-      if (idx < V) {
-        const int rel = idx - chunk * kSChunk;
-        const bool hit = pen && ((sm.hist_bits[rel >> 5] >> (rel & 31)) & 1u);
-        v[e] = xform_value(v[e], a.xf, idx, has_mask ? mrow[idx >> 5] : 0u, has_mask, hit);
+    for (int j = 0; j < kSVec; ++j) {
+      const int rel0 = (j * kSBlock + tid) * 4;
+      const uint32_t mnib = has_mask ? (sm.mask_bits[rel0 >> 5] >> (rel0 & 31)) & 15u : 15u;
+      const uint32_t hnib = pen ? (sm.hist_bits[rel0 >> 5] >> (rel0 & 31)) & 15u : 0u;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int idx = chunk * kSChunk + rel0 + c;
+        float x = v[j * 4 + c];
+        if (idx < V) {
+          // the reference's order: mask -> min-length -> repetition penalty
+          if (!((mnib >> c) & 1u)) x = kLowest;
+          for (int e = 0; e < a.xf.n_eos; ++e)
+            if (a.xf.eos[e] == idx) x = kLowest;
+          if ((hnib >> c) & 1u) x = x < 0.0f ? x * penalty : x / penalty;
+        }
+        v[j * 4 + c] = x;
       }
     }
   }
@@ -285,27 +307,50 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   if (tid == 0) sm.count = 0u;
 
   if (mode == kModeNucleus) {
-    const uint32_t cmax = block_max<uint32_t>(lmax, sm.wave_val);  // barriers inside publish count = 0
+    // Everything within nucleus_depth of the chunk maximum goes to the row's key buffer.  Slots come
+    // from a prefix sum over per-thread counts (one barrier), not from per-element atomics.
+    const uint32_t cmax = block_max<uint32_t>(lmax, sm.wave_val);
     float thr = -__builtin_inff();
     if (cmax != 0u) thr = key_to_float(cmax) - nucleus_depth(prm, V);
-    u64 best_below = 0;
+    uint32_t cnt = 0u;
+    float fb = -__builtin_inff();  // best element below the threshold (first of equals) ...
+    int fi = -1;                   // ... and its id
+#pragma unroll
+    for (int e = 0; e < kSElems; ++e) {
+      const bool cand = v[e] >= thr;  // false for NaN and for ids >= vocab
+      cnt += cand ? 1u : 0u;
+      const float nb = v[e] < thr ? v[e] : -__builtin_inff();
+      if (nb > fb || (fi < 0 && v[e] < thr)) {
+        fb = nb;
+        fi = elem_index(chunk, e / 4, e % 4);
+      }
+    }
+    uint32_t inc = cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const uint32_t y = __shfl_up(inc, d, 64);
+      if (lane >= d) inc += y;
+    }
+    if (lane == 63) sm.wave_val[wave] = inc;
+    u64 best_below = fi >= 0 ? make_key64(order_key(fb), static_cast<uint32_t>(fi)) : 0;
+    best_below = block_max<u64>(best_below, sm.wave_val64);  // its barriers also publish wave_val
+    uint32_t pos = inc - cnt, total = 0u;
+#pragma unroll
+    for (int w = 0; w < kSWaves; ++w) {
+      if (w < wave) pos += sm.wave_val[w];
+      total += sm.wave_val[w];
+    }
     u64* dst = big_row + static_cast<size_t>(chunk) * kSChunk;
 #pragma unroll
     for (int e = 0; e < kSElems; ++e) {
-      const int idx = elem_index(chunk, e / 4, e % 4);
-      const bool cand = v[e] >= thr;  // false for NaN and for ids >= vocab
-      const uint32_t pos = wave_slot(cand, &sm.count);
-      if (cand) {
-        dst[pos] = make_key64(order_key(v[e]), static_cast<uint32_t>(idx));
-      } else if (idx < V) {
-        const u64 k64 = make_key64(order_key(v[e]), static_cast<uint32_t>(idx));
-        best_below = k64 > best_below ? k64 : best_below;
+      if (v[e] >= thr) {
+        dst[pos] = make_key64(order_key(v[e]), static_cast<uint32_t>(elem_index(chunk, e / 4, e % 4)));
+        ++pos;
       }
     }
-    best_below = block_max<u64>(best_below, sm.wave_val64);
     if (tid == 0) {
       const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
-      a.chunk_cnt[ci] = sm.count;
+      a.chunk_cnt[ci] = total;
       a.chunk_max[ci] = cmax;
       a.chunk_next[ci] = best_below;
     }
