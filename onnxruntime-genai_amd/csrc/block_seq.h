@@ -4,6 +4,7 @@
 #pragma once
 #include "device_utils.h"
 #include "seq_scan.h"
+#include "wave_select.h"
 
 namespace ms {
 
@@ -299,6 +300,84 @@ __device__ __forceinline__ void block_sort_desc(u64* a, int n) {
       __syncthreads();
     }
   }
+}
+
+// Compare-exchange of two keys held by one thread; `a` has the lower index.
+__device__ __forceinline__ void key_cmpx(u64& a, u64& b, bool desc) {
+  const bool sw = (a < b) == desc;
+  const u64 t = sw ? b : a;
+  b = sw ? a : b;
+  a = t;
+}
+
+template <int M, int R>
+__device__ __forceinline__ void wave_key_exchange(u64 (&x)[R], bool keep_max) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const u64 y = lane_xor64<M>(x[r]);
+    x[r] = ((y > x[r]) == keep_max) ? y : x[r];
+  }
+}
+
+// Bitonic sort, descending, of 1024*R keys in LDS by a block of 1024 threads, with the keys held in
+// registers: thread t owns the keys of indices t*R .. t*R+R-1.  Exchange distances below R stay
+// inside a thread, distances below 64*R cross lanes with data-parallel-primitive moves, and only the
+// ten stages with larger distances go through LDS.
+template <int R>
+__device__ void block_sort_desc_regs(u64* lds) {
+  constexpr int kT = 1024;
+  const int t = threadIdx.x;
+  u64 x[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) x[r] = lds[r * kT + t];  // any order of the unsorted input will do
+  __syncthreads();
+#pragma unroll
+  for (int k = 2; k <= R; k <<= 1) {
+#pragma unroll
+    for (int j = k >> 1; j >= 1; j >>= 1) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if ((r & j) == 0) key_cmpx(x[r], x[r | j], k < R ? (r & k) == 0 : (t & 1) == 0);
+    }
+  }
+  for (int kt = 2; kt <= kT; kt <<= 1) {
+    const bool desc = (t & kt) == 0;
+    for (int jt = kt >> 1; jt >= 1; jt >>= 1) {
+      const bool keep_max = ((t & jt) == 0) == desc;
+      if (jt >= 64) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) lds[r * kT + t] = x[r];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const u64 y = lds[r * kT + (t ^ jt)];
+          x[r] = ((y > x[r]) == keep_max) ? y : x[r];
+        }
+        __syncthreads();
+      } else if (jt == 32) {
+        wave_key_exchange<32, R>(x, keep_max);
+      } else if (jt == 16) {
+        wave_key_exchange<16, R>(x, keep_max);
+      } else if (jt == 8) {
+        wave_key_exchange<8, R>(x, keep_max);
+      } else if (jt == 4) {
+        wave_key_exchange<4, R>(x, keep_max);
+      } else if (jt == 2) {
+        wave_key_exchange<2, R>(x, keep_max);
+      } else {
+        wave_key_exchange<1, R>(x, keep_max);
+      }
+    }
+#pragma unroll
+    for (int j = R >> 1; j >= 1; j >>= 1) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if ((r & j) == 0) key_cmpx(x[r], x[r | j], desc);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) lds[t * R + r] = x[r];
+  __syncthreads();
 }
 
 struct RowOutputs {

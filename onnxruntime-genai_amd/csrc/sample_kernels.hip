@@ -563,11 +563,95 @@ __global__ __launch_bounds__(kSBlock) void sample_fused_kernel(const SampleArgs 
   general_row(a, row, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq);
 }
 
+// Sorts n keys (kFinishBlock < n <= kNucleusCap) in LDS, descending, by a block of kFinishBlock
+// threads: a counting pass over kSortBuckets buckets that are linear in the score (bucket 0 holds the
+// best scores) groups the keys, then every key finds its rank inside its bucket by comparing whole
+// keys.  The bucket of a score is a monotone function of it, so the result is the exact key order.
+// Returns false -- keys untouched in value, possibly permuted -- when a bucket holds more than
+// kBucketCap keys (heavy ties); the caller then uses the sorting network.
+constexpr int kSortBuckets = 4096;
+constexpr int kBucketCap = 64;
+constexpr size_t kFinishLds = kNucleusCap * sizeof(u64) + (kSortBuckets + 1) * sizeof(uint32_t);
+
+__device__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n, float fmax, float fthr, uint32_t* red) {
+  constexpr int R = kNucleusCap / kFinishBlock;
+  const int t = threadIdx.x;
+  u64 k[R];
+  uint32_t info[R];  // bucket << 8 | slot inside the bucket, later the final position
+#pragma unroll
+  for (int r = 0; r < R; ++r) k[r] = r * kFinishBlock + t < n ? keys[r * kFinishBlock + t] : 0;
+  for (int b = t; b <= kSortBuckets; b += kFinishBlock) start[b] = 0u;
+  __syncthreads();
+  const float span = fmax - fthr;
+  const float scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (r * kFinishBlock + t < n) {
+      const float x = key_to_float(key64_okey(k[r]));
+      float bf = (fmax - x) * scale;
+      bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);  // also NaN-safe
+      const uint32_t b = bf > 0.0f ? static_cast<uint32_t>(bf) : 0u;
+      const uint32_t slot = atomicAdd(&start[b], 1u);
+      info[r] = (b << 8) | (slot < 255u ? slot : 255u);
+    }
+  }
+  __syncthreads();
+  // exclusive scan of the bucket counts (4 consecutive buckets per thread) and the size check
+  constexpr int kPer = kSortBuckets / kFinishBlock;
+  uint32_t cnt[kPer], local = 0u, big = 0u;
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    cnt[i] = start[t * kPer + i];
+    local += cnt[i];
+    big |= cnt[i] > static_cast<uint32_t>(kBucketCap) ? 1u : 0u;
+  }
+  uint32_t inc = local;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t y = __shfl_up(inc, d, 64);
+    if ((t & 63) >= d) inc += y;
+  }
+  const uint32_t any_big = block_max<uint32_t>(big, red);
+  if ((t & 63) == 63) red[t >> 6] = inc;
+  __syncthreads();
+  if (any_big) return false;
+  uint32_t base = inc - local;
+  for (int w = 0; w < (t >> 6); ++w) base += red[w];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    start[t * kPer + i] = base;
+    base += cnt[i];
+  }
+  if (t == kFinishBlock - 1) start[kSortBuckets] = base;
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    if (r * kFinishBlock + t < n) keys[start[info[r] >> 8] + (info[r] & 255u)] = k[r];
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (r * kFinishBlock + t < n) {
+      const uint32_t b = info[r] >> 8;
+      const uint32_t lo = start[b], hi = start[b + 1];
+      uint32_t rank = 0u;
+      for (uint32_t j = lo; j < hi; ++j) rank += keys[j] > k[r] ? 1u : 0u;
+      info[r] = lo + rank;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    if (r * kFinishBlock + t < n) keys[info[r]] = k[r];
+  __syncthreads();
+  return true;
+}
+
 // Per-row finish of the nucleus path: gathers the candidates the streaming pass left in `big`,
 // sorts them in LDS and runs the exact epilogue.  One block of kFinishBlock threads per row;
-// dynamic LDS: kNucleusCap key64s.
+// dynamic LDS: kNucleusCap key64s + the bucket table of the sort.
 __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const SampleArgs a) {
   extern __shared__ u64 lds_keys[];
+  uint32_t* bucket_start = reinterpret_cast<uint32_t*>(lds_keys + kNucleusCap);  // kSortBuckets + 1 entries
   __shared__ SeqShared seqsh;
   __shared__ uint32_t sh_count;
   __shared__ uint32_t red32[16];
@@ -608,10 +692,25 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const Samp
   if (ok) {
     if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
     if (best_below != 0) n_c += 1;
-    const int n2 = next_pow2(static_cast<int>(n_c));
-    for (int p = static_cast<int>(n_c) + tid; p < n2; p += blockDim.x) lds_keys[p] = 0;
     __syncthreads();
-    block_sort_desc(lds_keys, n2);
+    bool sorted_done = false;
+    if (n_c > static_cast<uint32_t>(kFinishBlock) && rmax != 0u) {
+      sorted_done = bucket_sort_desc(lds_keys, bucket_start, static_cast<int>(n_c), key_to_float(rmax),
+                                     key_to_float(thr), red32);
+    }
+    if (!sorted_done) {
+      const int n2 = next_pow2(static_cast<int>(n_c));
+      for (int p = static_cast<int>(n_c) + tid; p < n2; p += blockDim.x) lds_keys[p] = 0;
+      __syncthreads();
+      switch (n2 / kFinishBlock) {
+        case 0:
+        case 1: block_sort_desc(lds_keys, n2); break;
+        case 2: block_sort_desc_regs<2>(lds_keys); break;
+        case 4: block_sort_desc_regs<4>(lds_keys); break;
+        case 8: block_sort_desc_regs<8>(lds_keys); break;
+        default: block_sort_desc_regs<16>(lds_keys); break;
+      }
+    }
     // cache exp((s - max)/T) in the score half of every entry
     const float max_score = key_to_float(key64_okey(lds_keys[0]));
     __syncthreads();
@@ -642,7 +741,7 @@ extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, bool any_nucleus
   if (e != hipSuccess) return e;
   if (any_nucleus) {
     hipLaunchKernelGGL(ms::nucleus_finish_kernel, dim3(a->rows), dim3(ms::kFinishBlock),
-                       ms::kNucleusCap * sizeof(ms::u64), stream, *a);
+                       ms::kFinishLds, stream, *a);
     e = hipGetLastError();
   }
   return e;
@@ -650,6 +749,5 @@ extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, bool any_nucleus
 
 extern "C" hipError_t ms_sample_init() {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(ms::nucleus_finish_kernel),
-                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                             ms::kNucleusCap * sizeof(ms::u64));
+                             hipFuncAttributeMaxDynamicSharedMemorySize, ms::kFinishLds);
 }

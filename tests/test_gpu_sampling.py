@@ -169,6 +169,33 @@ def test_sample_nucleus(ctx, orc, rows, vocab, p, t):
     sample_and_check(ctx, orc, x, u, 0, p, t, cap=128)
 
 
+@pytest.mark.parametrize("frac,quantum", [(0.004, 0.0), (0.012, 0.0), (0.03, 0.0), (0.012, 0.5), (0.03, 0.5),
+                                           (0.06, 0.25)])
+def test_nucleus_candidate_counts_and_ties(ctx, orc, frac, quantum):
+    """Masked nucleus rows whose candidate lists fall in every size class of the finish kernel's sort
+    (about 800 to 12000 keys); a quantum > 0 rounds the logits to a coarse grid so that hundreds of
+    candidates tie and the sort must fall back from score buckets to the sorting network."""
+    say("nucleus sizes", frac, quantum)
+    rng = np.random.default_rng(int(frac * 1000) + int(quantum * 8))
+    rows, vocab = 3, 201088
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    if quantum:
+        x = (np.round(x / quantum) * quantum).astype(np.float32)
+    mask = make_mask(rng, rows, vocab, frac)
+    u = rng.random(rows)
+    xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda())
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=0.95,
+                                 temperature=1.0, xf=xf, kept_capacity=16384)
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    proc = orc.apply_mask(x, mask)
+    for r in range(rows):
+        idx, probs = orc.sampled_categorical(proc[r], 0, 0.95, 1.0)
+        assert kc[r] == len(idx)
+        assert np.array_equal(ki[r, :len(idx)], idx)
+        assert np.array_equal(bits(kp[r, :len(idx)]), bits(probs))
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])]
+
+
 def test_config5_constrained_nucleus(ctx, orc):
     """BASELINE config 5 shape (8 of 256 rows per step, 2 steps): vocab 201088, 5 % grammar mask,
     T=1.0, top-p 0.95, repetition penalty 1.2 over 1024 ids."""
