@@ -59,6 +59,12 @@ struct mi355x_search_ctx {
   void** ptr_table{};      // device copy of pointer tables (kv gather)
   size_t ptr_table_cap{};
   float* beam_row_scores{};
+  int max_segs{};
+  uint32_t* seg_max{};
+  double* seg_sum{};
+  int4* seg_step{};
+  float* row_max{};
+  float* row_sum{};
   int32_t* beam_row_tokens{};
   float* widen{};          // fp32 copy of fp16 rows (top-k scores), grown on demand
   size_t widen_elems{};
@@ -156,6 +162,12 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->params_dev, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->beam_row_scores, static_cast<size_t>(max_rows) * ms::kBeamMaxCand, false));
   ok(c->Alloc(&c->beam_row_tokens, static_cast<size_t>(max_rows) * ms::kBeamMaxCand, false));
+  c->max_segs = (max_vocab + ms::kSegElems - 1) / ms::kSegElems;
+  ok(c->Alloc(&c->seg_max, static_cast<size_t>(max_rows) * c->max_segs, false));
+  ok(c->Alloc(&c->seg_sum, static_cast<size_t>(max_rows) * c->max_segs, false));
+  ok(c->Alloc(&c->seg_step, static_cast<size_t>(max_rows) * c->max_segs, false));
+  ok(c->Alloc(&c->row_max, static_cast<size_t>(max_rows), false));
+  ok(c->Alloc(&c->row_sum, static_cast<size_t>(max_rows), false));
   c->ptr_table_cap = 4096;
   ok(c->Alloc(&c->ptr_table, c->ptr_table_cap, false));
   if (e == hipSuccess) e = ms_sample_init();
@@ -310,13 +322,44 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   return MI355X_OK;
 }
 
+// Fills the argument block of the multi-workgroup sequential sum when the shape calls for it and the
+// context's workspace covers it (the exponentials go to the key buffer of the sampling paths, which
+// never run at the same time on one context).
+static bool FillSeqSum(mi355x_search_ctx* ctx, const void* x, int64_t row_stride, int rows, int vocab, float inv_temp,
+                       ms::SeqSumArgs* q) {
+  const int segs = (vocab + ms::kSegElems - 1) / ms::kSegElems;
+  if (vocab < ms::kSeqSumMinVocab || rows > ctx->max_rows || vocab > ctx->max_vocab || segs > ms::kMaxSegs) return false;
+  q->x = x;
+  q->row_stride = row_stride;
+  q->rows = rows;
+  q->vocab = vocab;
+  q->segs = segs;
+  q->inv_temp = inv_temp;
+  q->seg_max = ctx->seg_max;
+  q->seg_sum = ctx->seg_sum;
+  q->seg_step = ctx->seg_step;
+  q->e = reinterpret_cast<float*>(ctx->big);
+  q->e_stride = ctx->big_stride * 2;
+  q->out_max = ctx->row_max;
+  q->out_sum = ctx->row_sum;
+  return true;
+}
+
 int mi355x_softmax(mi355x_search_ctx* ctx, void* stream, float* scores, int64_t row_stride, int rows, int vocab,
                    float temperature, int log_softmax) {
   if (!ctx) return Fail(MI355X_E_INVALID, "null context");
   if (!scores || rows <= 0 || vocab <= 0) return Fail(MI355X_E_INVALID, "null scores or non-positive size");
   if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
   if (!(temperature > 0.0f)) return Fail(MI355X_E_INVALID, "temperature must be positive (got %g)", temperature);
-  HIP_TRY(ms_launch_softmax(scores, row_stride, rows, vocab, temperature, log_softmax, static_cast<hipStream_t>(stream)));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  ms::SeqSumArgs q{};
+  if (FillSeqSum(ctx, scores, row_stride, rows, vocab, 1.0f / temperature, &q)) {
+    // long rows: the exact sum is spread over the whole GPU, then an element-wise pass finishes
+    HIP_TRY(ms_launch_seqsum(&q, MI355X_F32, s));
+    HIP_TRY(ms_launch_softmax_apply(scores, row_stride, &q, log_softmax, s));
+  } else {
+    HIP_TRY(ms_launch_softmax(scores, row_stride, rows, vocab, temperature, log_softmax, s));
+  }
   return MI355X_OK;
 }
 
@@ -347,6 +390,12 @@ int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits,
   a.out_scores = out_scores;
   a.out_tokens = out_tokens;
   a.out_beams = out_beam_indices;
+  ms::SeqSumArgs q{};
+  if (FillSeqSum(ctx, logits, row_stride, batch * beams, vocab, 1.0f, &q)) {
+    HIP_TRY(ms_launch_seqsum(&q, dtype, static_cast<hipStream_t>(stream)));
+    a.row_max = q.out_max;
+    a.row_sum = q.out_sum;
+  }
   HIP_TRY(ms_launch_beam_select(&a, dtype, static_cast<hipStream_t>(stream)));
   return MI355X_OK;
 }

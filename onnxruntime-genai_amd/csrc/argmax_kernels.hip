@@ -47,6 +47,88 @@ __global__ __launch_bounds__(kBlock) void argmax_kernel(const ArgmaxArgs a) {
   }
 }
 
+// Small problems (a few rows of at most kRowKernelMaxVocab logits) are latency-bound: one 1024-thread
+// workgroup per row walks the whole row, so no cross-workgroup hand-over is needed.
+constexpr int kRowKernelMaxVocab = 65536;
+
+template <typename InT>
+__global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
+  constexpr int VEC = Loader<InT>::VEC;
+  constexpr int NB = 8;  // vectors a thread has in flight: all their loads are issued before any is used
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int V = a.vocab;
+  __shared__ uint32_t hist_bits[kRowKernelMaxVocab / 32];
+  __shared__ u64 red64[16];
+  const InT* lrow = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
+  const bool pen = a.xf.use_penalty();
+  const bool has_mask = a.xf.mask != nullptr;
+  const bool active = a.xf.active();
+  const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
+  u64 best = 0;
+  for (int base = 0; base < V; base += 1024 * VEC * NB) {
+    float v[NB][VEC];
+    uint32_t mw[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int i0 = base + (j * 1024 + tid) * VEC;
+      mw[j] = (has_mask && i0 < V) ? mrow[i0 >> 5] : 0u;  // VEC divides 32: one word covers the vector
+      if (aligned && i0 + VEC <= V) {
+        if constexpr (VEC == 4) {
+          const float4 q = *reinterpret_cast<const float4*>(lrow + i0);
+          v[j][0] = q.x, v[j][1] = q.y, v[j][2] = q.z, v[j][3] = q.w;
+        } else {
+          const uint4 q = *reinterpret_cast<const uint4*>(lrow + i0);
+          const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            v[j][2 * c] = half_bits_to_float(w[c] & 0xffffu);
+            v[j][2 * c + 1] = half_bits_to_float(w[c] >> 16);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) v[j][c] = (i0 + c < V) ? load_one<InT>(lrow, i0 + c) : 0.0f;
+      }
+    }
+    if (pen && base == 0) {  // built while the first batch of loads is in flight
+      const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
+      int hv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) hv[r] = (r * 1024 + tid < a.xf.history_len) ? h[r * 1024 + tid] : -1;
+      for (int i = tid; i < (V + 31) / 32; i += 1024) hist_bits[i] = 0u;
+      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (hv[r] >= 0 && hv[r] < V) atomicOr(&hist_bits[hv[r] >> 5], 1u << (hv[r] & 31));
+      for (int i = 4096 + tid; i < a.xf.history_len; i += 1024) {
+        const int t = h[i];
+        if (t >= 0 && t < V) atomicOr(&hist_bits[t >> 5], 1u << (t & 31));
+      }
+      __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int i0 = base + (j * 1024 + tid) * VEC;
+      const uint32_t hw = (pen && i0 < V) ? hist_bits[i0 >> 5] : 0u;
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) {
+        const int idx = i0 + c;
+        if (idx < V) {
+          float x = v[j][c];
+          if (active) x = xform_value(x, a.xf, idx, mw[j], has_mask, (hw >> (idx & 31)) & 1u);
+          u64 k = make_key64(order_key(x), static_cast<uint32_t>(idx));
+          if (idx == 0 && x != x) k = ~0ull;  // NaN at index 0 is sticky
+          if (k == 0) k = 1;
+          best = k > best ? k : best;
+        }
+      }
+    }
+  }
+  best = block_max<u64>(best, red64);
+  if (tid == 0) a.out_tokens[row] = static_cast<int32_t>(key64_index(best));
+}
+
 // mask -> min-length -> repetition penalty, written back in place
 // (LaunchAddLogitsMask / ApplyMinLength / ApplyRepetitionPenalty).
 __global__ __launch_bounds__(kBlock) void process_logits_kernel(float* logits, int64_t row_stride, int vocab, const Xform xf) {
@@ -74,6 +156,13 @@ __global__ __launch_bounds__(kBlock) void process_logits_kernel(float* logits, i
 }  // namespace ms
 
 extern "C" hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipStream_t stream) {
+  if (a->vocab <= ms::kRowKernelMaxVocab && a->rows * a->chunks < 256) {
+    if (dtype == MI355X_F16)
+      hipLaunchKernelGGL(ms::argmax_row_kernel<uint16_t>, dim3(a->rows), dim3(1024), 0, stream, *a);
+    else
+      hipLaunchKernelGGL(ms::argmax_row_kernel<float>, dim3(a->rows), dim3(1024), 0, stream, *a);
+    return hipGetLastError();
+  }
   dim3 grid(a->chunks, a->rows);
   if (dtype == MI355X_F16)
     hipLaunchKernelGGL(ms::argmax_kernel<uint16_t>, grid, dim3(ms::kBlock), 0, stream, *a);

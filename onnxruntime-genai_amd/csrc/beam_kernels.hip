@@ -16,6 +16,7 @@ constexpr int kBeamListCap = 1024;  // candidates a row may hold in LDS before t
 template <typename InT>
 __global__ __launch_bounds__(1024) void beam_row_kernel(const BeamArgs a) {
   __shared__ SeqShared sh;
+  __shared__ __align__(16) float stage[1024 * 8];
   __shared__ u64 list[kBeamListCap];
   __shared__ uint32_t pool[64];
   __shared__ uint32_t red[16];
@@ -25,14 +26,16 @@ __global__ __launch_bounds__(1024) void beam_row_kernel(const BeamArgs a) {
   const int V = a.vocab, m = 2 * a.beams;
   const InT* x = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
   float fm = -__builtin_inff();
+#pragma unroll 8
   for (int i = tid; i < V; i += blockDim.x) fm = fmaxf(fm, load_one<InT>(x, i));
   const uint32_t lkey = tid < V ? order_key(fm) : 0u;
-  const float max_score = key_to_float(block_max<uint32_t>(lkey, red));
+  const float own_max = key_to_float(block_max<uint32_t>(lkey, red));
+  const float max_score = a.row_max ? a.row_max[row] : own_max;
   const int n_lanes = V < 1024 ? V : 1024;
   const uint32_t tau = block_pool_bound(lkey, m, (n_lanes + 63) / 64, pool, &bound);
   auto e = [=](int i) { return em::expf_exact(load_one<InT>(x, i) - max_score); };
   int dummy;
-  const float lse = em::logf_exact(block_seq_sum<8>(0.0f, V, e, NoStop{}, &dummy, sh));
+  const float lse = em::logf_exact(a.row_sum ? a.row_sum[row] : block_seq_sum<8>(0.0f, V, e, NoStop{}, &dummy, sh, stage));
   const float bs = a.beam_scores[row];
   auto final_score = [=](float v) { return ((v - max_score) - lse) + bs; };
   // tau == 0: fewer than m offers (tiny vocabulary): every element is a candidate

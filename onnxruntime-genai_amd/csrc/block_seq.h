@@ -84,6 +84,38 @@ __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
   return v;
 }
 
+// Fetches the ITEMS consecutive addends thread t owns in the window [w0, wend): indices
+// w0 + t*ITEMS + j.  Asking get() for them directly makes every lane walk its own 4*ITEMS-byte strip of
+// global memory, which wastes most of every cache line fetched; with a staging buffer in LDS
+// (blockDim * ITEMS floats) the window is read with consecutive lanes on consecutive indices and
+// transposed through LDS instead.  Contains one barrier when staging; the caller's next barrier
+// separates these LDS reads from the next window's writes.
+template <int ITEMS, typename GetE>
+__device__ __forceinline__ void window_fetch(float (&ev)[ITEMS], int w0, int wend, GetE get, float* stage) {
+  const int tid = threadIdx.x, bd = static_cast<int>(blockDim.x);
+  if (stage == nullptr) {
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) ev[j] = (w0 + tid * ITEMS + j < wend) ? get(w0 + tid * ITEMS + j) : 0.0f;
+    return;
+  }
+  float tmp[ITEMS];
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) tmp[j] = (w0 + j * bd + tid < wend) ? get(w0 + j * bd + tid) : 0.0f;
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) stage[j * bd + tid] = tmp[j];
+  __syncthreads();
+  if constexpr (ITEMS % 4 == 0) {
+#pragma unroll
+    for (int j = 0; j < ITEMS; j += 4) {
+      const float4 q = *reinterpret_cast<const float4*>(stage + tid * ITEMS + j);
+      ev[j] = q.x, ev[j + 1] = q.y, ev[j + 2] = q.z, ev[j + 3] = q.w;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) ev[j] = stage[tid * ITEMS + j];
+  }
+}
+
 struct NoStop {
   __device__ bool operator()(float, float, int) const { return false; }
 };
@@ -100,7 +132,8 @@ struct NoStop {
 // which the rest of the window is scanned again under the new binade) or the first index where the
 // predicate holds.  Passes cost two barriers; there is one per window plus one per binade change.
 template <int ITEMS, typename GetE, typename StopFn>
-__device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop_index, SeqShared& sh) {
+__device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop_index, SeqShared& sh,
+                               float* stage = nullptr) {
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6, nw = static_cast<int>(blockDim.x) >> 6;
   const int span = static_cast<int>(blockDim.x) * ITEMS;
   constexpr uint32_t kNone = 0xffffffffu;
@@ -112,8 +145,7 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
     const int base = w0 + tid * ITEMS;
     const int wend = (n - w0 < span) ? n : w0 + span;
     float ev[ITEMS];
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) ev[j] = (base + j < wend) ? get(base + j) : 0.0f;
+    window_fetch<ITEMS>(ev, w0, wend, get, stage);
     int start = w0;  // first index not yet folded into s
     while (true) {
       const SeqState st = seq_decompose(s);
@@ -201,17 +233,19 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
 
 // Position std::discrete_distribution would return for weights w(0..n-1) and canonical draw u
 // (libstdc++ random.tcc: normalise by the double sum, partial sums in double, last forced to 1,
-// lower_bound).  The reference accumulates those doubles sequentially; here they are reduced and
-// scanned in parallel, which can move a cumulative value by at most a few n*2^-53.  If u lies that
-// close to any cumulative value the answer is recomputed sequentially, so the result always equals
-// the sequential one.
+// lower_bound).  The reference divides every weight by the sum and accumulates the quotients
+// sequentially; here the raw weights are reduced and scanned in parallel and compared with u * sum,
+// which differs from the reference's cumulative values by at most a few n*2^-53 (relative to the
+// sum).  If u lies that close to any cumulative value the answer is recomputed sequentially with the
+// reference's own operations, so the result always equals the sequential one.
 template <int ITEMS, typename GetW>
-__device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh) {
+__device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float* stage = nullptr) {
   if (n < 2) return 0;
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6, nw = blockDim.x >> 6;
   const int span = static_cast<int>(blockDim.x) * ITEMS;
   // total
   double part = 0.0;
+#pragma unroll 8
   for (int i = tid; i < n; i += blockDim.x) part += static_cast<double>(w(i));
   part = wave_sum<double>(part);
   if (lane == 0) sh.dred[wave] = part;
@@ -219,7 +253,8 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh) {
   double total = 0.0;
   for (int k = 0; k < nw; ++k) total += sh.dred[k];
   __syncthreads();
-  const double guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16;
+  const double guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16 * total;
+  const double target = u * total;
   double carry = 0.0;
   int first = kIntMax;
   int risky = 0;
@@ -227,11 +262,14 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh) {
     const int base = i0 + tid * ITEMS;
     double pv[ITEMS];
     double loc = 0.0;
+    {
+      float wv[ITEMS];
+      window_fetch<ITEMS>(wv, i0, (n - i0 < span) ? n : i0 + span, w, stage);
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-      const int idx = base + j;
-      pv[j] = idx < n ? static_cast<double>(w(idx)) / total : 0.0;
-      loc += pv[j];
+      for (int j = 0; j < ITEMS; ++j) {
+        pv[j] = static_cast<double>(wv[j]);
+        loc += pv[j];
+      }
     }
     double inc = loc;
 #pragma unroll
@@ -251,9 +289,8 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh) {
       const int idx = base + j;
       if (idx < n) {
         run += pv[j];
-        const double cp = (idx == n - 1) ? 1.0 : run;
-        if (idx != n - 1 && fabs(cp - u) <= guard) risky = 1;
-        if (cp >= u && idx < first) first = idx;
+        if (idx != n - 1 && fabs(run - target) <= guard) risky = 1;
+        if ((idx == n - 1 || run >= target) && idx < first) first = idx;  // the last value is forced to 1
       }
     }
     carry += block_total;

@@ -64,11 +64,32 @@ struct ArgmaxArgs {
 
 constexpr int kBeamMaxCand = 32;  // 2 * beams, beams <= 16
 
+// Multi-workgroup exact sequential sum (seqsum_kernels.hip).
+constexpr int kSegElems = 4096;   // elements per segment
+constexpr int kMaxSegs = 1024;    // segments per row the walk kernel can hold
+constexpr int kSeqSumMinVocab = 16384;  // shorter rows are summed by one workgroup in one launch
+
+struct SeqSumArgs {
+  const void* x;
+  int64_t row_stride;
+  int rows, vocab, segs;
+  float inv_temp;
+  uint32_t* seg_max;  // [rows][segs] order keys
+  double* seg_sum;    // [rows][segs]
+  int4* seg_step;     // [rows][segs]: d0, d1, binade (-1: scan the segment), unused
+  float* e;           // [rows][e_stride] exponentials
+  size_t e_stride;
+  float* out_max;     // [rows]
+  float* out_sum;     // [rows]
+};
+
 struct BeamArgs {
   const void* logits;
   int64_t row_stride;
   int batch, beams, vocab;
   const float* beam_scores;   // [batch*beams]
+  const float* row_max;       // [batch*beams] maximum and exact sum of exp(x - max) per row, or null:
+  const float* row_sum;       //   the row kernel then computes them itself
   float* row_scores;          // workspace [batch*beams][kBeamMaxCand]
   int32_t* row_tokens;        // workspace [batch*beams][kBeamMaxCand]
   float* out_scores;          // [batch][2*beams]
@@ -111,6 +132,9 @@ hipError_t ms_launch_spec_verify(const float* p_target, const float* p_draft, co
 hipError_t ms_launch_widen_f16(const void* in, int64_t in_stride, float* out, int64_t out_stride, int rows,
                                int vocab, hipStream_t stream);
 hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hipStream_t stream);
+hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, hipStream_t stream);
+hipError_t ms_launch_softmax_apply(float* scores, int64_t row_stride, const ms::SeqSumArgs* a, int log_softmax,
+                                   hipStream_t stream);
 hipError_t ms_launch_scorer_process(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,
                                     const float* cs, const int32_t* ct, const int32_t* ci, hipStream_t stream);
 hipError_t ms_launch_scorer_finalize(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,

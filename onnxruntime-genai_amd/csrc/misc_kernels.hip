@@ -13,23 +13,27 @@ template <bool LOG>
 __global__ __launch_bounds__(1024) void softmax_kernel(float* scores, int64_t row_stride, int vocab, float temperature) {
   __shared__ SeqShared sh;
   __shared__ uint32_t red[16];
+  __shared__ __align__(16) float stage[1024 * 8];
   float* x = scores + static_cast<size_t>(blockIdx.x) * row_stride;
   float m = -__builtin_inff();
+#pragma unroll 8
   for (int i = threadIdx.x; i < vocab; i += blockDim.x) m = fmaxf(m, x[i]);
   const float max_score = key_to_float(block_max<uint32_t>(order_key(m), red));
   const float inv_temp = 1.0f / temperature;
   const float* xc = x;
   auto e = [=](int i) { return em::expf_exact((xc[i] - max_score) * inv_temp); };
   int dummy;
-  const float sum = block_seq_sum<8>(0.0f, vocab, e, NoStop{}, &dummy, sh);
+  const float sum = block_seq_sum<8>(0.0f, vocab, e, NoStop{}, &dummy, sh, stage);
   if (LOG) {
     const float lse = em::logf_exact(sum);
+#pragma unroll 8
     for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
       const float s = (x[i] - max_score) * inv_temp;
       x[i] = s - lse;
     }
   } else {
     const float inv_sum = 1.0f / sum;
+#pragma unroll 8
     for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
       const float ex = em::expf_exact((x[i] - max_score) * inv_temp);
       x[i] = sum > 0.0f ? ex * inv_sum : ex;
@@ -75,20 +79,31 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
                                                            const double* sample_u, int K, int vocab,
                                                            int32_t* accepted_len, int32_t* final_token) {
   __shared__ SeqShared sh;
+  __shared__ __align__(16) float stage[1024 * 8];
   __shared__ int sh_n, sh_any;
   const int b = blockIdx.x;
   const size_t base = static_cast<size_t>(b) * (K + 1) * vocab;
-  if (threadIdx.x == 0) {
-    int n = 0;
-    for (; n < K; ++n) {
-      const int d = draft_tokens[b * K + n];
-      const float pt = p_target[base + static_cast<size_t>(n) * vocab + d];
-      const float pd = p_draft[base + static_cast<size_t>(n) * vocab + d];
-      const float acc = pd <= 0.0f ? 1.0f : fminf(1.0f, pt / pd);  // ComputeAcceptProb, :140-146
-      if (!(accept_u[b * K + n] < acc)) break;
+  if (threadIdx.x < 64) {
+    // every position's accept test at once (their loads overlap); the loop of the reference stops at
+    // the first failure, i.e. at the lowest failing lane
+    int rejected_at = K;
+    for (int n0 = 0; n0 < K && rejected_at == K; n0 += 64) {
+      const int n = n0 + static_cast<int>(threadIdx.x);
+      bool reject = false;
+      if (n < K) {
+        const int d = draft_tokens[b * K + n];
+        const float pt = p_target[base + static_cast<size_t>(n) * vocab + d];
+        const float pd = p_draft[base + static_cast<size_t>(n) * vocab + d];
+        const float acc = pd <= 0.0f ? 1.0f : fminf(1.0f, pt / pd);  // ComputeAcceptProb, :140-146
+        reject = !(accept_u[b * K + n] < acc);
+      }
+      const int f = first_lane(__ballot(reject));
+      if (f >= 0) rejected_at = n0 + f;
     }
-    sh_n = n;
-    sh_any = 0;
+    if (threadIdx.x == 0) {
+      sh_n = rejected_at;
+      sh_any = 0;
+    }
   }
   __syncthreads();
   const int n = sh_n;
@@ -97,6 +112,7 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
   bool use_residual = false;
   if (n < K) {
     int any = 0;
+#pragma unroll 8
     for (int i = threadIdx.x; i < vocab; i += blockDim.x) any |= (pt[i] - pd[i] > 0.0f);
     if (any) sh_any = 1;  // the reference's fp32 "sum > 0" holds iff some residual is positive
     __syncthreads();
@@ -108,10 +124,10 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
       const float d = pt[i] - pd[i];
       return d > 0.0f ? d : 0.0f;
     };
-    pos = block_discrete_draw<4>(vocab, w, sample_u[b], sh);
+    pos = block_discrete_draw<8>(vocab, w, sample_u[b], sh, stage);
   } else {
     auto w = [=](int i) { return pt[i]; };
-    pos = block_discrete_draw<4>(vocab, w, sample_u[b], sh);
+    pos = block_discrete_draw<8>(vocab, w, sample_u[b], sh, stage);
   }
   if (threadIdx.x == 0) {
     accepted_len[b] = n;

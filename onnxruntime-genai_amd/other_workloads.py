@@ -207,7 +207,7 @@ def c4(args, pkg, orc, dev):
     def step(i):
         outs[i % pool] = ctx.spec_verify(*devc[i % pool])
 
-    ms = _timed(step, K, W, graph=False)
+    ms = _timed(step, K, W)
     t0 = time.perf_counter()
     want = [orc.spec_verify_dense(*c) for c in cases]
     cpu_s = time.perf_counter() - t0
@@ -220,7 +220,7 @@ def c4(args, pkg, orc, dev):
     return _line(args, "speculative verification rounds/sec, B=16 K=8 V=32064", "rounds/s",
                  B * K / (ms * 1e-3), ms, K, W, "f32",
                  "config 4: accept loop + residual/bonus resampling on dense [16,9,32064] fp32 target/draft "
-                 "probabilities, %d steps launched back to back (latency-bound)" % K,
+                 "probabilities, %d steps replayed from a HIP graph (latency-bound)" % K,
                  {"mean_accepted_len": accepted / (pool * B),
                   "parity": "accepted lengths and tokens of %d distinct inputs identical to the CPU oracle" % pool}, algo,
                  _cpu(B * pool / cpu_s, "rounds/s", "%d inputs, orc_spec_verify_dense, one thread" % pool, cpu_s / pool * 1e3))

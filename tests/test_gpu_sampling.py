@@ -71,6 +71,30 @@ def test_config1_greedy_with_repetition_penalty(ctx, orc):
         assert got[0] == want
 
 
+@pytest.mark.parametrize("rows,vocab,dtype", [(2, 5000, np.float32), (3, 40000, np.float16), (40, 70001, np.float32),
+                                              (33, 128256, np.float16)])
+def test_argmax_with_fused_logits_processing(ctx, orc, rows, vocab, dtype):
+    """Greedy selection with grammar mask, min-length and repetition penalty fused, on the
+    single-workgroup-per-row kernel (small shapes) and the chunked kernel (large shapes)."""
+    say("argmax fused", rows, vocab, dtype.__name__)
+    rng = np.random.default_rng(rows + vocab)
+    x = (rng.standard_normal((rows, vocab)) * 2).astype(dtype)
+    x32 = orc.fp16_to_fp32(x) if dtype == np.float16 else x
+    mask = make_mask(rng, rows, vocab, 0.5)
+    hist = rng.integers(-2, vocab + 2, (rows, 300)).astype(np.int32)
+    top = np.argmax(x32, axis=1)
+    hist[:, 0] = top  # the raw maximum is penalised
+    eos = [int(np.argsort(x32[0])[-2]), vocab - 1]
+    xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                           repetition_penalty=1.7, eos_ids=eos, apply_min_length=True)
+    got = ctx.argmax(torch.from_numpy(x).cuda(), xf=xf).cpu().numpy()
+    proc = orc.apply_mask(x32, mask)
+    for r in range(rows):
+        row = orc.apply_min_length(proc[r], 0, 1, eos)
+        row = orc.apply_repetition_penalty(row, hist[r], 1.7)
+        assert got[r] == orc.argmax(row), r
+
+
 @pytest.mark.parametrize("vocab", [33, 1000, 8192, 40000])
 def test_process_logits_in_place(ctx, orc, vocab):
     say("process_logits", vocab)
