@@ -8,6 +8,48 @@ namespace ms {
 
 constexpr int kBeamListCap = 1024;  // candidates a row may hold in LDS before the slow exact path
 
+// Calls fn(index, value) for every element of a row, the block's threads taking 16-byte vectors in
+// turn (four vectors in flight per thread); every thread makes the same number of calls per vector
+// round, with index -1 past the end of the row, so fn may contain wave-wide operations.
+template <typename InT, typename Fn>
+__device__ __forceinline__ void row_for_each(const InT* x, int V, Fn fn) {
+  constexpr int VEC = 16 / sizeof(InT);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
+  const int step = static_cast<int>(blockDim.x) * VEC;
+  for (int base = 0; base < V; base += 4 * step) {
+    float v[4][VEC];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i0 = base + r * step + static_cast<int>(threadIdx.x) * VEC;
+      if (aligned && i0 + VEC <= V) {
+        const uint4 q = *reinterpret_cast<const uint4*>(x + i0);
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        if constexpr (VEC == 4) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[r][c] = __uint_as_float(w[c]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            v[r][2 * c] = half_bits_to_float(w[c] & 0xffffu);
+            v[r][2 * c + 1] = half_bits_to_float(w[c] >> 16);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) v[r][c] = (i0 + c < V) ? load_one<InT>(x, i0 + c) : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i0 = base + r * step + static_cast<int>(threadIdx.x) * VEC;
+      if (base + r * step < V) {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) fn(i0 + c < V ? i0 + c : -1, v[r][c]);
+      }
+    }
+  }
+}
+
 // One 1024-thread block per batch-beam row.  BeamSearch_Cpu::SelectTop (src/search.cpp:101-123):
 // scores = ((x - max) * 1.0f - log(sum exp)) + beam_score, the sum accumulated in index order in
 // fp32 (reproduced exactly by the scan of seq_scan.h).  The value is monotone in x, so the row's
@@ -26,33 +68,30 @@ __global__ __launch_bounds__(1024) void beam_row_kernel(const BeamArgs a) {
   const int V = a.vocab, m = 2 * a.beams;
   const InT* x = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
   float fm = -__builtin_inff();
-#pragma unroll 8
-  for (int i = tid; i < V; i += blockDim.x) fm = fmaxf(fm, load_one<InT>(x, i));
-  const uint32_t lkey = tid < V ? order_key(fm) : 0u;
+  row_for_each<InT>(x, V, [&](int i, float val) {
+    if (i >= 0) fm = fmaxf(fm, val);
+  });
+  constexpr int kVec = 16 / sizeof(InT);
+  const uint32_t lkey = tid * kVec < V ? order_key(fm) : 0u;
   const float own_max = key_to_float(block_max<uint32_t>(lkey, red));
   const float max_score = a.row_max ? a.row_max[row] : own_max;
-  const int n_lanes = V < 1024 ? V : 1024;
+  const int n_lanes = (V + kVec - 1) / kVec < 1024 ? (V + kVec - 1) / kVec : 1024;
   const uint32_t tau = block_pool_bound(lkey, m, (n_lanes + 63) / 64, pool, &bound);
   auto e = [=](int i) { return em::expf_exact(load_one<InT>(x, i) - max_score); };
   int dummy;
-  const float lse = em::logf_exact(a.row_sum ? a.row_sum[row] : block_seq_sum<8>(0.0f, V, e, NoStop{}, &dummy, sh, stage));
+  const float lse = em::logf_exact(a.row_sum ? a.row_sum[row] : block_seq_sum<8>(0.0f, V, e, NoStop{}, &dummy, sh, stage, 256));
   const float bs = a.beam_scores[row];
   auto final_score = [=](float v) { return ((v - max_score) - lse) + bs; };
   // tau == 0: fewer than m offers (tiny vocabulary): every element is a candidate
   const float cut = tau != 0u ? final_score(key_to_float(tau)) : -__builtin_inff();
   if (tid == 0) count = 0u;
   __syncthreads();
-  for (int i0 = 0; i0 < V; i0 += blockDim.x) {
-    const int i = i0 + tid;
-    float f = 0.0f;
-    bool cand = false;
-    if (i < V) {
-      f = final_score(load_one<InT>(x, i));
-      cand = (f >= cut) || (tau == 0u);
-    }
+  row_for_each<InT>(x, V, [&](int i, float val) {
+    const float f = final_score(val);
+    const bool cand = i >= 0 && ((f >= cut) || (tau == 0u));
     const uint32_t pos = wave_slot(cand, &count);
     if (cand && pos < kBeamListCap) list[pos] = make_key64(order_key(f), static_cast<uint32_t>(i));
-  }
+  });
   __syncthreads();
   const uint32_t n = count;
   float* out_s = a.row_scores + static_cast<size_t>(row) * kBeamMaxCand;

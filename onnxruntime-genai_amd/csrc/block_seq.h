@@ -2,6 +2,7 @@
 // "first index where a predicate on the running prefix holds" search), a double-precision CDF search,
 // an in-place bitonic sort, and the exact sampling epilogue shared by the nucleus and general paths.
 #pragma once
+#include <type_traits>
 #include "device_utils.h"
 #include "seq_scan.h"
 #include "wave_select.h"
@@ -16,6 +17,8 @@ struct SeqShared {
   uint32_t ev_key[2][16];
   float ev_a[2][16], ev_b[2][16];
   uint32_t n_last[2];
+  float head_sum;
+  int head_found;
   // block_discrete_draw / block_min2
   int red_a[16];
   int red_b[16];
@@ -116,6 +119,36 @@ __device__ __forceinline__ void window_fetch(float (&ev)[ITEMS], int w0, int wen
   }
 }
 
+// Serial prefix over lanes: out[l] = ((x[0] + x[1]) + ...) + x[l], additions in lane order, as the
+// reference's scalar loops do.  One DPP-shifted add per element (wave_shr:1, lane 0 reads 0).
+// Steps run in unrolled groups of 8: a step past `count` leaves lanes below `count` unchanged.
+__device__ __forceinline__ float wave_serial_prefix(float x, int count) {
+  float s = 0.0f;
+  for (int t = 0; t < count; t += 8) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const float prev = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s), 0x138, 0xf, 0xf, false));
+      s = prev + x;
+    }
+  }
+  return s;
+}
+
+__device__ __forceinline__ double wave_serial_prefix(double x, int count) {
+  double s = 0.0;
+  for (int t = 0; t < count; t += 4) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const u64 b = static_cast<u64>(__double_as_longlong(s));
+      const uint32_t lo = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b), 0x138, 0xf, 0xf, false);
+      const uint32_t hi = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b >> 32), 0x138, 0xf, 0xf, false);
+      const double prev = __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
+      s = prev + x;
+    }
+  }
+  return s;
+}
+
 struct NoStop {
   __device__ bool operator()(float, float, int) const { return false; }
 };
@@ -133,7 +166,7 @@ struct NoStop {
 // predicate holds.  Passes cost two barriers; there is one per window plus one per binade change.
 template <int ITEMS, typename GetE, typename StopFn>
 __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop_index, SeqShared& sh,
-                               float* stage = nullptr) {
+                               float* stage = nullptr, int head = 0) {
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6, nw = static_cast<int>(blockDim.x) >> 6;
   const int span = static_cast<int>(blockDim.x) * ITEMS;
   constexpr uint32_t kNone = 0xffffffffu;
@@ -141,7 +174,40 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
   int found = -1;
   int par = 0;
   __syncthreads();  // a previous call's readers are done with the parity-0 buffers
-  for (int w0 = 0; w0 < n && found < 0; w0 += span) {
+  // A sum that starts from nothing changes binade every few additions, and each change costs a pass
+  // of the scan below.  The first `head` elements are therefore added for real, 64 at a time, by a
+  // chain of lane-shifted float additions in wave 0 (about ten cycles per element).
+  int n_head = 0;
+  if (head > 0) {
+    n_head = head < n ? head : n;
+    if (wave == 0) {
+      float carry = s0;
+      int fnd = -1;
+      float x_next = lane < n_head ? get(lane) : 0.0f;
+      for (int r0 = 0; r0 < n_head && fnd < 0; r0 += 64) {
+        const float x = x_next;
+        const int idx = r0 + lane;
+        x_next = idx + 64 < n_head ? get(idx + 64) : 0.0f;  // in flight during this round's chain
+        const float sp = wave_serial_prefix(lane == 0 ? carry + x : x, 64);
+        const unsigned long long hit = __ballot(idx < n_head && stop(sp, x, idx));
+        if (hit != 0ull) {
+          const int l = __ffsll(static_cast<long long>(hit)) - 1;
+          fnd = r0 + l;
+          carry = __shfl(sp, l, 64);
+        } else {
+          carry = __shfl(sp, 63, 64);  // lanes past the end added zeros
+        }
+      }
+      if (lane == 0) {
+        sh.head_sum = carry;
+        sh.head_found = fnd;
+      }
+    }
+    __syncthreads();
+    s = sh.head_sum;
+    found = sh.head_found;
+  }
+  for (int w0 = n_head; w0 < n && found < 0; w0 += span) {
     const int base = w0 + tid * ITEMS;
     const int wend = (n - w0 < span) ? n : w0 + span;
     float ev[ITEMS];
@@ -167,25 +233,32 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
       uint32_t nn = step_apply(st.n, ex);
       uint32_t key = kNone;
       float pa = 0.0f, pb = 0.0f;
+      // Without a stop predicate only a binade change is of interest, and a thread whose last
+      // prefix is still inside the binade (prefixes never decrease) has none among its elements.
+      constexpr bool kPlain = std::is_same<StopFn, NoStop>::value;
+      if (kPlain && step_apply(nn, agg) < kMantLimit) {
+        nn = step_apply(nn, agg);
+      } else {
 #pragma unroll
-      for (int j = 0; j < ITEMS; ++j) {
-        const int idx = base + j;
-        if (idx >= start && idx < wend) {
-          const uint32_t nn2 = step_apply(nn, f[j]);
-          if (key == kNone) {
-            if (nn2 >= kMantLimit) {  // leaves the binade here (or an earlier thread's element did)
-              key = (static_cast<uint32_t>(idx) << 1) | 1u;
-              pa = seq_recompose(nn < kMantLimit ? nn : 0u, st.se);
-              pb = ev[j];
-            } else {
-              const float pf = seq_recompose(nn2, st.se);
-              if (stop(pf, ev[j], idx)) {
-                key = static_cast<uint32_t>(idx) << 1;
-                pa = pf;
+        for (int j = 0; j < ITEMS; ++j) {
+          const int idx = base + j;
+          if (idx >= start && idx < wend) {
+            const uint32_t nn2 = step_apply(nn, f[j]);
+            if (key == kNone) {
+              if (nn2 >= kMantLimit) {  // leaves the binade here (or an earlier thread's element did)
+                key = (static_cast<uint32_t>(idx) << 1) | 1u;
+                pa = seq_recompose(nn < kMantLimit ? nn : 0u, st.se);
+                pb = ev[j];
+              } else if (!kPlain) {
+                const float pf = seq_recompose(nn2, st.se);
+                if (stop(pf, ev[j], idx)) {
+                  key = static_cast<uint32_t>(idx) << 1;
+                  pa = pf;
+                }
               }
             }
+            nn = nn2;
           }
-          nn = nn2;
         }
       }
       if (wend - 1 >= base && wend - 1 < base + ITEMS) sh.n_last[par] = nn;
@@ -417,6 +490,8 @@ __device__ void block_sort_desc_regs(u64* lds) {
   __syncthreads();
 }
 
+constexpr int kEpiHead = 256;  // elements of every epilogue sum added by the serial head
+
 struct RowOutputs {
   int32_t* token;
   int32_t* kept_count;
@@ -442,7 +517,7 @@ __device__ bool block_sample_epilogue(Sorted sorted, Exps exps, int n_sorted, in
   if (prm.k > 1) {
     const int m = prm.k < vocab ? prm.k : vocab;
     if (m > n_sorted) return false;
-    sum = block_seq_sum<ITEMS>(0.0f, m, exps, NoStop{}, &idx_dummy, sh);
+    sum = block_seq_sum<ITEMS>(0.0f, m, exps, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead);
     divide_by_sum = sum > 0.0f;
     const float ssum = sum;
     const bool dv = divide_by_sum;
@@ -455,10 +530,10 @@ __device__ bool block_sample_epilogue(Sorted sorted, Exps exps, int n_sorted, in
     if (prm.p > 0.0f && prm.p < 1.0f) {
       const float p = prm.p;
       int si;
-      keep_sum = block_seq_sum<ITEMS>(0.0f, m, pr, [=](float pf, float, int) { return pf >= p; }, &si, sh);
+      keep_sum = block_seq_sum<ITEMS>(0.0f, m, pr, [=](float pf, float, int) { return pf >= p; }, &si, sh, nullptr, kEpiHead);
       if (si >= 0) keep = si + 1;
     } else {
-      keep_sum = block_seq_sum<ITEMS>(0.0f, m, pr, NoStop{}, &idx_dummy, sh);
+      keep_sum = block_seq_sum<ITEMS>(0.0f, m, pr, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead);
     }
     scale = keep_sum > 0.0f ? 1.0f / keep_sum : 0.0f;
   } else {
@@ -472,7 +547,7 @@ __device__ bool block_sample_epilogue(Sorted sorted, Exps exps, int n_sorted, in
           const float tail = static_cast<float>(V - i - 1) * e;
           return pf >= p * (pf + tail);
         },
-        &si, sh);
+        &si, sh, nullptr, kEpiHead);
     int cutoff;
     if (si >= 0) {
       cutoff = si + 1;
@@ -483,17 +558,18 @@ __device__ bool block_sample_epilogue(Sorted sorted, Exps exps, int n_sorted, in
     }
     if (vocab <= 64) {  // exact-partition override, src/sampling_distribution.h:186-203
       if (n_sorted < vocab) return false;
-      const float global = block_seq_sum<ITEMS>(0.0f, vocab, exps, NoStop{}, &idx_dummy, sh);
+      const float global = block_seq_sum<ITEMS>(0.0f, vocab, exps, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead);
       int sj;
       const float c = block_seq_sum<ITEMS>(0.0f, vocab, exps,
-                                           [=](float pf, float, int) { return pf >= p * global; }, &sj, sh);
+                                           [=](float pf, float, int) { return pf >= p * global; }, &sj, sh,
+                                           nullptr, kEpiHead);
       (void)c;
       if (sj >= 0) {
         cutoff = sj + 1;
         si = -1;
       }
     }
-    if (si < 0 || cutoff != si + 1) prefix = block_seq_sum<ITEMS>(0.0f, cutoff, exps, NoStop{}, &idx_dummy, sh);
+    if (si < 0 || cutoff != si + 1) prefix = block_seq_sum<ITEMS>(0.0f, cutoff, exps, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead);
     keep = cutoff;
     scale = prefix > 0.0f ? 1.0f / prefix : 0.0f;
   }

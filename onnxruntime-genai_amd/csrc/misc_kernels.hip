@@ -23,7 +23,7 @@ __global__ __launch_bounds__(1024) void softmax_kernel(float* scores, int64_t ro
   const float* xc = x;
   auto e = [=](int i) { return em::expf_exact((xc[i] - max_score) * inv_temp); };
   int dummy;
-  const float sum = block_seq_sum<8>(0.0f, vocab, e, NoStop{}, &dummy, sh, stage);
+  const float sum = block_seq_sum<8>(0.0f, vocab, e, NoStop{}, &dummy, sh, stage, 256);
   if (LOG) {
     const float lse = em::logf_exact(sum);
 #pragma unroll 8

@@ -22,36 +22,6 @@ namespace ms {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-// Serial prefix over lanes: out[l] = ((x[0] + x[1]) + ...) + x[l], additions in lane order, as the
-// reference's scalar loops do.  One DPP-shifted add per element (wave_shr:1, lane 0 reads 0).
-// Steps run in unrolled groups of 8: a step past `count` leaves lanes below `count` unchanged.
-__device__ __forceinline__ float wave_serial_prefix(float x, int count) {
-  float s = 0.0f;
-  for (int t = 0; t < count; t += 8) {
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const float prev = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s), 0x138, 0xf, 0xf, false));
-      s = prev + x;
-    }
-  }
-  return s;
-}
-
-__device__ __forceinline__ double wave_serial_prefix(double x, int count) {
-  double s = 0.0;
-  for (int t = 0; t < count; t += 4) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const u64 b = static_cast<u64>(__double_as_longlong(s));
-      const uint32_t lo = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b), 0x138, 0xf, 0xf, false);
-      const uint32_t hi = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b >> 32), 0x138, 0xf, 0xf, false);
-      const double prev = __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
-      s = prev + x;
-    }
-  }
-  return s;
-}
-
 __device__ __forceinline__ int next_pow2(int v) {
   int p = 64;
   while (p < v) p <<= 1;

@@ -64,33 +64,22 @@ EM_HD float seq_recompose(uint32_t n, int se) {
 }
 
 // The step function of adding e (finite, >= 0) to a running sum whose unit is 2^(se-150).
+// The two increments are read off real float additions: inside a binade consecutive floats have
+// consecutive bit patterns one unit apart, so adding e to the binade's first even value (mantissa
+// integer 2^23) and to its first odd one (2^23 + 1) and subtracting the bit patterns gives the
+// rounded increments for even and odd sums -- round-to-nearest-even included, done by the adder
+// itself.  If such a sum lands in a higher binade the increment is at least 2^23 - 1 units, which
+// takes every sum of that parity to 2^24 or beyond: it is reported as saturated ("left the binade")
+// and the caller performs that addition for real.
 EM_HD Step seq_make_step(float e, int se) {
-  const uint32_t b = em::as_u32(e) & 0x7fffffffu;
-  const uint32_t er = b >> 23;
-  const uint32_t m = er ? ((b & 0x7fffffu) | 0x800000u) : (b & 0x7fffffu);
-  const int ee = er ? static_cast<int>(er) : 1;
-  const int shift = se - ee;  // e = m * 2^(-shift) units
+  const uint32_t b0 = static_cast<uint32_t>(se) << 23;
+  const uint32_t b1 = b0 | 1u;
+  const uint32_t r0 = em::as_u32(em::as_float(b0) + e);
+  const uint32_t r1 = em::as_u32(em::as_float(b1) + e);
+  const uint32_t lim = b0 + 0x800000u;  // first bit pattern of the next binade
   Step f;
-  if (m == 0u) {
-    f.d0 = f.d1 = 0u;
-  } else if (shift <= 0) {
-    const uint32_t a = (-shift >= 6) ? kStepSat : (m << (-shift));  // m < 2^24, so m << 5 < 2^29
-    f.d0 = f.d1 = a > kStepSat ? kStepSat : a;
-  } else if (shift > 25) {
-    f.d0 = f.d1 = 0u;  // below half a unit
-  } else {
-    const uint32_t a = m >> shift;
-    const uint32_t rem = m & ((1u << shift) - 1u);
-    const uint32_t half = 1u << (shift - 1);
-    if (rem > half) {
-      f.d0 = f.d1 = a + 1u;
-    } else if (rem < half) {
-      f.d0 = f.d1 = a;
-    } else {  // tie: round to even
-      f.d0 = a + (a & 1u);
-      f.d1 = a + ((a & 1u) ^ 1u);
-    }
-  }
+  f.d0 = r0 < lim ? r0 - b0 : kStepSat;
+  f.d1 = r1 < lim ? r1 - b1 : kStepSat;
   return f;
 }
 

@@ -114,9 +114,13 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_kernel(const SeqSumArgs 
   if (tid == 0) a.seg_sum[static_cast<size_t>(row) * a.segs + seg] = (dred[0] + dred[1]) + (dred[2] + dred[3]);
 }
 
-// Largest relative distance between the float the reference holds after adding `count` non-negative
-// terms one by one and their exact sum (count * 2^-24 to first order), with a margin.
-__device__ __forceinline__ double seq_drift(int count) { return (static_cast<double>(count) + 8.0) * 6.3e-8; }
+// Expected relative distance between the float the reference holds after adding `count` non-negative
+// terms one by one and their exact sum: roundings mostly cancel, so it grows like sqrt(count) * 2^-24
+// (the worst case grows like count * 2^-24).  Only an estimate is needed: a segment classified on a
+// wrong estimate fails the walk's check and is scanned.
+__device__ __forceinline__ double seq_drift(int count) {
+  return (8.0 * sqrt(static_cast<double>(count)) + 8.0) * 6.0e-8;
+}
 
 __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs a) {
   __shared__ double dred[4];
@@ -158,12 +162,13 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs
   }
 }
 
-constexpr int kWalkBlock = 1024;
+constexpr int kWalkBlock = 256;
 
 __global__ __launch_bounds__(kWalkBlock) void seqsum_walk_kernel(const SeqSumArgs a) {
   __shared__ SeqShared sh;
   __shared__ uint32_t red[16];
   __shared__ int4 recs[kMaxSegs];
+  __shared__ __align__(16) float stage[kSegElems];
   const int row = blockIdx.x, tid = threadIdx.x;
   for (int s = tid; s < a.segs; s += kWalkBlock) recs[s] = a.seg_step[static_cast<size_t>(row) * a.segs + s];
   const float max_score = row_max_of_segments(a, row, red);  // its barriers also publish recs
@@ -185,7 +190,8 @@ __global__ __launch_bounds__(kWalkBlock) void seqsum_walk_kernel(const SeqSumArg
     const int n = a.vocab - first < kSegElems ? a.vocab - first : kSegElems;
     const float* e = erow + first;
     int dummy;
-    s = block_seq_sum<kSegElems / kWalkBlock>(s, n, [=](int i) { return e[i]; }, NoStop{}, &dummy, sh);
+    s = block_seq_sum<kSegElems / kWalkBlock>(s, n, [=](int i) { return e[i]; }, NoStop{}, &dummy, sh, stage,
+                                                 seg == 0 ? 1024 : 0);
   }
   if (tid == 0) {
     a.out_sum[row] = s;
