@@ -110,12 +110,18 @@ constexpr uint32_t kPark = 6u;  // float4s with a hit a thread can park per chun
 struct FusedShared {
   uint32_t hist_bits[kSChunk / 32];
   uint32_t mask_bits[kSChunk / 32];
-  u64 lists[kAllCap];   // the chunks' sorted candidate lists of a row (finishing workgroup only)
   u64 list[kListCap];   // this chunk's candidates before the sort
   u64 list_hi[64];      // second half of a long list, sorted ascending
-  u64 lists2[kAllCap / 2];  // second buffer of the merge tree
-  float4 park_val[kSBlock * kPark];  // per-thread parking rows of the streaming filter
-  int park_idx[kSBlock * kPark];
+  union {               // the parking rows are dead before the merge buffers come into use
+    struct {
+      v4f park_val[kSBlock * kPark];  // per-thread parking rows of the streaming filter
+      int park_idx[kSBlock * kPark];
+    };
+    struct {
+      u64 lists[kAllCap];       // the chunks' sorted candidate lists of a row (finishing workgroup only)
+      u64 lists2[kAllCap / 2];  // second buffer of the merge tree
+    };
+  };
   uint32_t pool[64];
   uint32_t wave_val[kSWaves];
   u64 wave_val64[kSWaves];
@@ -356,7 +362,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     if (__ballot(qm[j] >= tau_f) != 0ull) {
       if (qm[j] >= tau_f) {
         if (lc < kPark) {
-          sm.park_val[tid * kPark + lc] = make_float4(v[j * 4], v[j * 4 + 1], v[j * 4 + 2], v[j * 4 + 3]);
+          sm.park_val[tid * kPark + lc] = v4f{v[j * 4], v[j * 4 + 1], v[j * 4 + 2], v[j * 4 + 3]};
           sm.park_idx[tid * kPark + lc] = elem_index(chunk, j, 0);
         }
         ++lc;
@@ -390,7 +396,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     uint32_t pos = base + before;
     const uint32_t lim = lc < kPark ? lc : kPark;
     for (uint32_t i = 0; i < lim; ++i) {
-      const float4 q = sm.park_val[tid * kPark + i];
+      const v4f q = sm.park_val[tid * kPark + i];
       const uint32_t id0 = static_cast<uint32_t>(sm.park_idx[tid * kPark + i]);
       const float qv[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll

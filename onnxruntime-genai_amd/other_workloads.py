@@ -141,7 +141,7 @@ def c3(args, pkg, orc, orc_lib, dev):
         sc, tok, idx = ctx.beam_select(logits[i % pool], B, NB, scorer.next_scores)
         scorer.step(sc, tok, idx)
 
-    ms_sel = _timed(select_step, K, W, graph=False)
+    ms_sel = _timed(select_step, K, W, graph=False)  # the scorer step is not capturable
     beam_idx = scorer.next_indices.clone()
     # ---- phase 2: KV gather ------------------------------------------------------------------------
     shape = (BB, 4, 2048, 128)
