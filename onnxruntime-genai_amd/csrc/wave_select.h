@@ -13,7 +13,9 @@ __device__ __forceinline__ uint32_t lane_xor(uint32_t x) {
   } else if constexpr (M == 2) {
     return __builtin_amdgcn_mov_dpp(x, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
   } else if constexpr (M == 4) {
-    return __builtin_amdgcn_ds_swizzle(x, (4 << 10) | 0x1f);   // bit-mask mode, xor 4
+    // banks of four lanes: even banks read four lanes up (row_shl:4), odd banks four lanes down
+    const uint32_t t = __builtin_amdgcn_update_dpp(x, x, 0x104, 0xf, 0x5, false);
+    return __builtin_amdgcn_update_dpp(t, x, 0x114, 0xf, 0xa, false);
   } else if constexpr (M == 8) {
     return __builtin_amdgcn_mov_dpp(x, 0x128, 0xf, 0xf, true);  // row_ror:8 == xor 8 inside a row of 16
   } else if constexpr (M == 16) {
