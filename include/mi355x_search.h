@@ -32,7 +32,10 @@ extern "C" {
 /* Element type of a logits / KV tensor (values follow ONNXTensorElementDataType where one exists:
  * FLOAT = 1, FLOAT16 = 10, the types DeviceInterface::ArgMax/TopKScores accept, src/smartptrs.h:249). */
 #define MI355X_F32 1
+#define MI355X_I32 6
+#define MI355X_I64 7
 #define MI355X_F16 10
+#define MI355X_BF16 16
 
 typedef struct mi355x_search_ctx mi355x_search_ctx;
 
@@ -183,6 +186,23 @@ int mi355x_spec_verify(mi355x_search_ctx* ctx, void* stream, const float* p_targ
                        const float* p_draft, const int32_t* draft_tokens, const float* accept_u,
                        const double* sample_u, int batch, int K, int vocab, int32_t* accepted_len,
                        int32_t* final_token);
+
+/* Element-wise type conversion on the device: DeviceInterface::Cast (src/smartptrs.h:208-210; CPU
+ * src/cpu/interface.cpp:74-106).  Supported pairs, with the CPU path's arithmetic: F16->F32
+ * (FastFloat16ToFloat32), BF16->F32 (BFloat16ToFloat32), F32->F16 (FastFloat32ToFloat16), F32->BF16
+ * (upper 16 bits), I32->I64.  MI355X_E_INVALID when the two types are equal (the reference throws),
+ * MI355X_E_UNSUPPORTED for any other pair (the reference's optional-capability "false"). */
+int mi355x_cast(mi355x_search_ctx* ctx, void* stream, const void* in, int in_dtype, void* out,
+                int out_dtype, size_t count);
+
+/* Logits hand-off before the path: Logits::Get (src/models/logits.cpp:33-82) copies the logits of each
+ * row's last real token out of the model's [rows, seq_len, vocab] output and widens fp16/bf16 to fp32;
+ * here both happen in one pass.  raw: device, dtype MI355X_F32 / MI355X_F16 / MI355X_BF16;
+ * token_index: HOST [rows] positions inside seq_len (copied by the call), or NULL for seq_len - 1;
+ * out: device [rows] rows of vocab floats, row r at out + r*out_stride. */
+int mi355x_logits_handoff(mi355x_search_ctx* ctx, void* stream, const void* raw, int dtype, int rows,
+                          int seq_len, int vocab, const int32_t* token_index, float* out,
+                          int64_t out_stride);
 
 /* Diagnostics: number of rows, since the context was created, that the single-pass fast paths
  * declined and the exact general path finished (synchronises `stream`). */

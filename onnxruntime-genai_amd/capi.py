@@ -62,6 +62,8 @@ def load_library():
                                           C.POINTER(C.c_float)],
         "mi355x_kv_gather": [vp, vp, C.POINTER(vp), C.POINTER(vp), i32, vp, i32, C.c_size_t],
         "mi355x_spec_verify": [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, vp],
+        "mi355x_cast": [vp, vp, vp, i32, vp, i32, C.c_size_t],
+        "mi355x_logits_handoff": [vp, vp, vp, i32, i32, i32, i32, C.POINTER(C.c_int32), vp, i64],
     }.items():
         if hasattr(L, name):
             getattr(L, name).argtypes = args
@@ -256,6 +258,35 @@ def _spec_verify(self, p_target, p_draft, draft_tokens, accept_u, sample_u):
     return acc, tok
 
 
+_DTYPE_CODES = {torch.float32: 1, torch.int32: 6, torch.int64: 7, torch.float16: 10, torch.bfloat16: 16}
+
+
+def _cast(self, src, dtype):
+    """DeviceInterface::Cast: returns a new tensor of `dtype` with the reference CPU path's conversion."""
+    assert src.is_cuda and src.is_contiguous()
+    out = torch.empty(src.shape, dtype=dtype, device=src.device)
+    self._check(self.L.mi355x_cast(self.h, _stream(), src.data_ptr(), _DTYPE_CODES[src.dtype], out.data_ptr(),
+                                   _DTYPE_CODES[dtype], src.numel()))
+    return out
+
+
+def _logits_handoff(self, raw, token_index=None, out=None):
+    """Logits::Get: raw [rows, seq_len, vocab] (fp32 / fp16 / bf16) -> fp32 [rows, vocab] of each row's
+    token_index (a host sequence; the last token when None)."""
+    assert raw.is_cuda and raw.is_contiguous() and raw.dim() == 3
+    rows, seq_len, vocab = raw.shape
+    if out is None:
+        out = torch.empty((rows, vocab), dtype=torch.float32, device=raw.device)
+    ti = None
+    if token_index is not None:
+        ti = (C.c_int32 * rows)(*[int(t) for t in token_index])
+    self._check(self.L.mi355x_logits_handoff(self.h, _stream(), raw.data_ptr(), _DTYPE_CODES[raw.dtype], rows, seq_len,
+                                             vocab, ti, out.data_ptr(), out.stride(0)))
+    return out
+
+
+SearchContext.cast = _cast
+SearchContext.logits_handoff = _logits_handoff
 SearchContext.topk_scores = _topk_scores
 SearchContext.softmax = _softmax
 SearchContext.beam_select = _beam_select

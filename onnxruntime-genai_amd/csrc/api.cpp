@@ -65,6 +65,7 @@ struct mi355x_search_ctx {
   int4* seg_step{};
   float* row_max{};
   float* row_sum{};
+  int32_t* row_index{};  // device copy of per-row host indices (logits hand-off)
   int32_t* beam_row_tokens{};
   float* widen{};          // fp32 copy of fp16 rows (top-k scores), grown on demand
   size_t widen_elems{};
@@ -168,6 +169,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->seg_step, static_cast<size_t>(max_rows) * c->max_segs, false));
   ok(c->Alloc(&c->row_max, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->row_sum, static_cast<size_t>(max_rows), false));
+  ok(c->Alloc(&c->row_index, static_cast<size_t>(max_rows), false));
   c->ptr_table_cap = 4096;
   ok(c->Alloc(&c->ptr_table, c->ptr_table_cap, false));
   if (e == hipSuccess) e = ms_sample_init();
@@ -397,6 +399,44 @@ int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits,
     a.row_sum = q.out_sum;
   }
   HIP_TRY(ms_launch_beam_select(&a, dtype, static_cast<hipStream_t>(stream)));
+  return MI355X_OK;
+}
+
+int mi355x_cast(mi355x_search_ctx* ctx, void* stream, const void* in, int in_dtype, void* out, int out_dtype,
+                size_t count) {
+  if (!ctx || !in || !out) return Fail(MI355X_E_INVALID, "null argument");
+  if (in_dtype == out_dtype) return Fail(MI355X_E_INVALID, "Cast - input and output types are the same");
+  int kind = -1;
+  if (in_dtype == MI355X_F16 && out_dtype == MI355X_F32) kind = 0;
+  else if (in_dtype == MI355X_BF16 && out_dtype == MI355X_F32) kind = 1;
+  else if (in_dtype == MI355X_F32 && out_dtype == MI355X_F16) kind = 2;
+  else if (in_dtype == MI355X_F32 && out_dtype == MI355X_BF16) kind = 3;
+  else if (in_dtype == MI355X_I32 && out_dtype == MI355X_I64) kind = 4;
+  if (kind < 0) return Fail(MI355X_E_UNSUPPORTED, "cast from type %d to type %d is not implemented", in_dtype, out_dtype);
+  if (count == 0) return MI355X_OK;
+  HIP_TRY(ms_launch_cast(in, out, count, kind, static_cast<hipStream_t>(stream)));
+  return MI355X_OK;
+}
+
+int mi355x_logits_handoff(mi355x_search_ctx* ctx, void* stream, const void* raw, int dtype, int rows, int seq_len,
+                          int vocab, const int32_t* token_index, float* out, int64_t out_stride) {
+  if (!ctx || !raw || !out) return Fail(MI355X_E_INVALID, "null argument");
+  if (rows <= 0 || seq_len <= 0 || vocab <= 0) return Fail(MI355X_E_INVALID, "non-positive size");
+  if (out_stride < vocab) return Fail(MI355X_E_INVALID, "out_stride smaller than vocab");
+  if (rows > 65535) return Fail(MI355X_E_CAPACITY, "too many rows (%d)", rows);
+  const int kind = dtype == MI355X_F16 ? 0 : dtype == MI355X_BF16 ? 1 : dtype == MI355X_F32 ? 2 : -1;
+  if (kind < 0) return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int32_t* index_dev = nullptr;
+  if (token_index) {
+    if (rows > ctx->max_rows) return Fail(MI355X_E_CAPACITY, "rows (%d) exceed the context's %d", rows, ctx->max_rows);
+    for (int r = 0; r < rows; ++r)
+      if (token_index[r] < 0 || token_index[r] >= seq_len)
+        return Fail(MI355X_E_INVALID, "token_index[%d] = %d outside [0, %d)", r, token_index[r], seq_len);
+    HIP_TRY(hipMemcpyAsync(ctx->row_index, token_index, sizeof(int32_t) * rows, hipMemcpyHostToDevice, s));
+    index_dev = ctx->row_index;
+  }
+  HIP_TRY(ms_launch_logits_handoff(raw, kind, rows, seq_len, vocab, index_dev, out, out_stride, s));
   return MI355X_OK;
 }
 

@@ -150,6 +150,26 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
   return __uint_as_float(sign | __float_as_uint(mag));
 }
 
+// bfloat16 -> fp32 as BFloat16ToFloat32 does (src/models/utils.cpp:84-86 via :55-77): the bits moved to
+// the upper half, except that every NaN becomes the canonical quiet NaN.
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t h) {
+  if ((h & 0x7f80u) == 0x7f80u && (h & 0x7fu) != 0u) return __uint_as_float(0x7fc00000u);
+  return __uint_as_float(h << 16);
+}
+
+// fp32 -> fp16 with FastFloat32ToFloat16's arithmetic (src/models/utils.cpp:111-118): the rounding
+// bit is added before the fields are split, values beyond the fp16 range saturate to 0x7FFF.
+__device__ __forceinline__ uint32_t float_to_half_bits(float v) {
+  const uint32_t b = __float_as_uint(v) + 0x00001000u;
+  const uint32_t e = (b & 0x7F800000u) >> 23;
+  const uint32_t m = b & 0x007FFFFFu;
+  uint32_t r = (b & 0x80000000u) >> 16;
+  if (e > 112u) r |= (((e - 112u) << 10) & 0x7C00u) | (m >> 13);
+  if (e < 113u && e > 101u) r |= (((0x007FF000u + m) >> (125u - e)) + 1u) >> 1;
+  if (e > 143u) r |= 0x7FFFu;
+  return r & 0xffffu;
+}
+
 // ---- fused logits processing --------------------------------------------------------------------
 struct Xform {
   const uint32_t* mask;

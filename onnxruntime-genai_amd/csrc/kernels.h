@@ -131,6 +131,9 @@ hipError_t ms_launch_spec_verify(const float* p_target, const float* p_draft, co
                                  int32_t* accepted_len, int32_t* final_token, hipStream_t stream);
 hipError_t ms_launch_widen_f16(const void* in, int64_t in_stride, float* out, int64_t out_stride, int rows,
                                int vocab, hipStream_t stream);
+hipError_t ms_launch_cast(const void* in, void* out, size_t count, int kind, hipStream_t stream);
+hipError_t ms_launch_logits_handoff(const void* raw, int kind, int rows, int seq_len, int vocab,
+                                    const int32_t* token_index, float* out, int64_t out_stride, hipStream_t stream);
 hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hipStream_t stream);
 hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, hipStream_t stream);
 hipError_t ms_launch_softmax_apply(float* scores, int64_t row_stride, const ms::SeqSumArgs* a, int log_softmax,

@@ -144,7 +144,61 @@ __global__ __launch_bounds__(256) void widen_f16_kernel(const uint16_t* in, int6
     dst[i] = half_bits_to_float(src[i]);
 }
 
+// ---- DeviceInterface::Cast (src/cpu/interface.cpp:74-106) -----------------------------------------
+// kind: 0 fp16->fp32, 1 bf16->fp32, 2 fp32->fp16, 3 fp32->bf16 (upper 16 bits), 4 int32->int64.
+__global__ __launch_bounds__(256) void cast_kernel(const void* in, void* out, size_t count, int kind) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += stride) {
+    switch (kind) {
+      case 0: static_cast<float*>(out)[i] = half_bits_to_float(static_cast<const uint16_t*>(in)[i]); break;
+      case 1: static_cast<float*>(out)[i] = bf16_bits_to_float(static_cast<const uint16_t*>(in)[i]); break;
+      case 2: static_cast<uint16_t*>(out)[i] = static_cast<uint16_t>(float_to_half_bits(static_cast<const float*>(in)[i])); break;
+      case 3: static_cast<uint16_t*>(out)[i] = static_cast<uint16_t>(__float_as_uint(static_cast<const float*>(in)[i]) >> 16); break;
+      default: static_cast<int64_t*>(out)[i] = static_cast<const int32_t*>(in)[i]; break;
+    }
+  }
+}
+
+// ---- logits hand-off: last-token slice + widening in one pass (Logits::Get, src/models/logits.cpp:33-82)
+// raw is [rows, seq_len, vocab] of fp32 / fp16 / bf16; row r's source is token token_index[r] (the
+// last token when token_index is null).  out: [rows] rows of `vocab` floats at out_stride.
+template <int KIND>  // 0 fp16, 1 bf16, 2 fp32
+__global__ __launch_bounds__(256) void logits_handoff_kernel(const void* raw, int seq_len, int vocab,
+                                                             const int32_t* token_index, float* out, int64_t out_stride) {
+  const int row = blockIdx.y;
+  const int tok = token_index ? token_index[row] : seq_len - 1;
+  const size_t src0 = (static_cast<size_t>(row) * seq_len + tok) * vocab;
+  float* dst = out + static_cast<size_t>(row) * out_stride;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < vocab; i += gridDim.x * blockDim.x) {
+    if (KIND == 0) dst[i] = half_bits_to_float(static_cast<const uint16_t*>(raw)[src0 + i]);
+    else if (KIND == 1) dst[i] = bf16_bits_to_float(static_cast<const uint16_t*>(raw)[src0 + i]);
+    else dst[i] = static_cast<const float*>(raw)[src0 + i];
+  }
+}
+
 }  // namespace ms
+
+extern "C" hipError_t ms_launch_cast(const void* in, void* out, size_t count, int kind, hipStream_t stream) {
+  size_t blocks = (count + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(ms::cast_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, in, out, count, kind);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_logits_handoff(const void* raw, int kind, int rows, int seq_len, int vocab,
+                                               const int32_t* token_index, float* out, int64_t out_stride,
+                                               hipStream_t stream) {
+  int gx = (vocab + 255) / 256;
+  if (gx > 256) gx = 256;
+  const dim3 grid(gx, rows), block(256);
+  if (kind == 0)
+    hipLaunchKernelGGL(ms::logits_handoff_kernel<0>, grid, block, 0, stream, raw, seq_len, vocab, token_index, out, out_stride);
+  else if (kind == 1)
+    hipLaunchKernelGGL(ms::logits_handoff_kernel<1>, grid, block, 0, stream, raw, seq_len, vocab, token_index, out, out_stride);
+  else
+    hipLaunchKernelGGL(ms::logits_handoff_kernel<2>, grid, block, 0, stream, raw, seq_len, vocab, token_index, out, out_stride);
+  return hipGetLastError();
+}
 
 extern "C" hipError_t ms_launch_softmax(float* scores, int64_t row_stride, int rows, int vocab, float temperature,
                                         int log_softmax, hipStream_t stream) {

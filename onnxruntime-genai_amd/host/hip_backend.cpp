@@ -211,6 +211,18 @@ struct HipInterface final : DeviceInterface {
     return std::make_unique<HipBatchedSampler>(*this, max_batch_size, vocab_size);
   }
   void Synchronize() override { HIP_CHECK(hipStreamSynchronize(g_stream)); }
+  // src/smartptrs.h:208-210: true when the pair is converted on the device, false when the caller
+  // has to fall back; equal types throw, as in the CPU and CUDA interfaces.
+  bool Cast(void* input, void* output, ONNXTensorElementDataType input_type, ONNXTensorElementDataType output_type,
+            size_t element_count) override {
+    if (input_type == output_type) throw std::runtime_error("Cast - input and output types are the same");
+    std::lock_guard<std::mutex> lock(mutex_);
+    const int rc = mi355x_cast(Scratch(1, 64), g_stream, input, static_cast<int>(input_type), output,
+                               static_cast<int>(output_type), element_count);
+    if (rc == MI355X_E_UNSUPPORTED) return false;
+    AbiCheck(rc);
+    return true;
+  }
   void LaunchAddLogitsMask(float* batch_logits, int batch_beam_size, int vocab_size, const uint32_t* logits_mask) override {
     std::lock_guard<std::mutex> lock(mutex_);
     mi355x_logits_xform xf{};

@@ -31,6 +31,7 @@ enum ONNXTensorElementDataType : int {
   ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32 = 6,
   ONNX_TENSOR_ELEMENT_DATA_TYPE_INT64 = 7,
   ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16 = 10,
+  ONNX_TENSOR_ELEMENT_DATA_TYPE_BFLOAT16 = 16,
 };
 
 namespace Generators {

@@ -347,6 +347,53 @@ float orc_fp16_to_fp32(uint16_t x) {
   return out;
 }
 
+// src/models/utils.cpp:111-118 FastFloat32ToFloat16.
+uint16_t orc_fp32_to_fp16(float v) {
+  uint32_t bits;
+  std::memcpy(&bits, &v, 4);
+  const uint32_t b = bits + 0x00001000u;
+  const uint32_t e = (b & 0x7F800000u) >> 23;
+  const uint32_t m = b & 0x007FFFFFu;
+  return static_cast<uint16_t>((b & 0x80000000u) >> 16 | (e > 112) * ((((e - 112) << 10) & 0x7C00u) | m >> 13) |
+                               ((e < 113) & (e > 101)) * ((((0x007FF000u + m) >> (125 - e)) + 1) >> 1) |
+                               (e > 143) * 0x7FFFu);
+}
+
+// src/models/utils.cpp:84-86 BFloat16ToFloat32 = TFloatToFloat32<8, 7> (:55-77).
+float orc_bf16_to_fp32(uint16_t v) {
+  const uint32_t sign = v >> 15, exponent = (v >> 7) & 0xFFu, fraction = v & 0x7Fu;
+  if (exponent == 0) {
+    if (fraction == 0) return sign ? -0.0f : 0.0f;
+    return std::ldexp((sign ? -1.0f : 1.0f) * static_cast<float>(fraction) / 128.0f, 1 - 127);
+  }
+  if (exponent == 255) {
+    if (fraction == 0) return sign ? -std::numeric_limits<float>::infinity() : std::numeric_limits<float>::infinity();
+    return std::numeric_limits<float>::quiet_NaN();
+  }
+  return std::ldexp((sign ? -1.0f : 1.0f) * (1.0f + static_cast<float>(fraction) / 128.0f), static_cast<int>(exponent) - 127);
+}
+
+// src/models/utils.cpp:89-93 Float32ToBFloat16: the most significant 16 bits.
+uint16_t orc_fp32_to_bf16(float v) {
+  uint32_t bits;
+  std::memcpy(&bits, &v, 4);
+  return static_cast<uint16_t>(bits >> 16);
+}
+
+// DeviceInterface::Cast on the CPU (src/cpu/interface.cpp:74-106); kind as in the device kernel:
+// 0 fp16->fp32, 1 bf16->fp32, 2 fp32->fp16, 3 fp32->bf16, 4 int32->int64.
+void orc_cast(const void* in, void* out, size_t n, int kind) {
+  for (size_t i = 0; i < n; ++i) {
+    switch (kind) {
+      case 0: static_cast<float*>(out)[i] = orc_fp16_to_fp32(static_cast<const uint16_t*>(in)[i]); break;
+      case 1: static_cast<float*>(out)[i] = orc_bf16_to_fp32(static_cast<const uint16_t*>(in)[i]); break;
+      case 2: static_cast<uint16_t*>(out)[i] = orc_fp32_to_fp16(static_cast<const float*>(in)[i]); break;
+      case 3: static_cast<uint16_t*>(out)[i] = orc_fp32_to_bf16(static_cast<const float*>(in)[i]); break;
+      default: static_cast<int64_t*>(out)[i] = static_cast<const int32_t*>(in)[i]; break;
+    }
+  }
+}
+
 void orc_fp16_to_fp32_array(const uint16_t* in, float* out, size_t n) {
   for (size_t i = 0; i < n; ++i) out[i] = orc_fp16_to_fp32(in[i]);
 }

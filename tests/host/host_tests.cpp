@@ -278,6 +278,17 @@ void DeviceFastPaths() {
   }
   EXPECT(!Device()->TopKScores(half_logits.Span().data(), ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16, rows, vocab, 65,
                                top_tokens.data(), top_scores.data()));
+  // DeviceInterface::Cast: fp16 -> fp32 on the device equals the host-side widening used above
+  auto widened_dev = Device()->Allocate<float>(values.size());
+  EXPECT(Device()->Cast(half_logits.Span().data(), widened_dev.Span().data(), ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16,
+                        ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT, values.size()));
+  EXPECT(ToHost(widened_dev) == widened);
+  EXPECT(!Device()->Cast(widened_dev.Span().data(), half_logits.Span().data(), ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT,
+                         ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32, values.size()));
+  EXPECT(Throws<std::runtime_error>([&] {
+    Device()->Cast(widened_dev.Span().data(), widened_dev.Span().data(), ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT,
+                   ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT, 1);
+  }));
 }
 
 // test/sampling_tests.cpp:22-49: top_k = 1 sampling returns the argmax of every row

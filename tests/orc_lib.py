@@ -170,6 +170,16 @@ class Oracle:
         self.lib.orc_log_softmax_plain(s, s.size)
         return s
 
+    def cast(self, src, kind, out_dtype):
+        """kind: 0 fp16->fp32, 1 bf16->fp32, 2 fp32->fp16, 3 fp32->bf16, 4 int32->int64 (bit patterns in,
+        bit patterns out for the 16-bit types)."""
+        src = np.ascontiguousarray(src)
+        out = np.empty(src.shape, out_dtype)
+        self.lib.orc_cast.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        self.lib.orc_cast.restype = None
+        self.lib.orc_cast(src.ctypes.data, out.ctypes.data, src.size, kind)
+        return out
+
     def fp16_to_fp32(self, h):
         h = np.ascontiguousarray(h).view(np.uint16)
         out = np.empty(h.shape, np.float32)

@@ -207,3 +207,50 @@ def test_spec_verify(ctx, orc, batch, K, vocab):
     assert np.array_equal(acc.cpu().numpy(), oacc)
     assert np.array_equal(tok.cpu().numpy(), otok)
     assert len(set(oacc.tolist())) > 1 or batch < 4
+
+
+def test_cast_matches_cpu_path(ctx, orc):
+    """DeviceInterface::Cast, every supported pair, against the oracle's CPU conversions: all 65536
+    fp16 / bf16 patterns, random and special fp32 values, int32 extremes."""
+    say("cast")
+    h = torch.arange(65536, dtype=torch.int32).to(torch.int16).cuda()
+    got = ctx.cast(h.view(torch.float16), torch.float32).cpu().numpy()
+    assert np.array_equal(bits(got), bits(orc.cast(np.arange(65536, dtype=np.uint16), 0, np.float32)))
+    got = ctx.cast(h.view(torch.bfloat16), torch.float32).cpu().numpy()
+    assert np.array_equal(bits(got), bits(orc.cast(np.arange(65536, dtype=np.uint16), 1, np.float32)))
+    rng = np.random.default_rng(8)
+    x = np.concatenate([(rng.standard_normal(100000) * 10 ** rng.uniform(-9, 6, 100000)).astype(np.float32),
+                        np.array([0.0, -0.0, 65504.0, 65520.0, 1e9, -1e9, 1.0 + 2.0 ** -11, 6e-8, 3e-8, np.inf, -np.inf],
+                                 np.float32),
+                        rng.integers(0, 2 ** 32, 100000, dtype=np.uint64).astype(np.uint32).view(np.float32)])
+    got = ctx.cast(torch.from_numpy(x).cuda(), torch.float16).view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, orc.cast(x, 2, np.uint16))
+    got = ctx.cast(torch.from_numpy(x).cuda(), torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, orc.cast(x, 3, np.uint16))
+    i = np.array([0, -1, 5, 2 ** 31 - 1, -2 ** 31], np.int32)
+    assert np.array_equal(ctx.cast(torch.from_numpy(i).cuda(), torch.int64).cpu().numpy(), i.astype(np.int64))
+    with pytest.raises(RuntimeError, match="same"):
+        ctx.cast(torch.zeros(4, device="cuda"), torch.float32)
+    with pytest.raises(RuntimeError, match="not implemented"):
+        ctx.cast(torch.zeros(4, device="cuda", dtype=torch.int64), torch.int32)
+
+
+@pytest.mark.parametrize("dtype,kind", [(torch.float16, 0), (torch.bfloat16, 1), (torch.float32, None)])
+def test_logits_handoff_slices_and_widens(ctx, orc, dtype, kind):
+    """Logits::Get (src/models/logits.cpp:33-82): the logits of each row's last real token, widened to
+    fp32 with the CPU path's conversion, from a [rows, seq_len, vocab] model output."""
+    say("logits handoff", dtype)
+    rows, seq_len, vocab = 5, 7, 4099
+    g = torch.Generator(device="cuda").manual_seed(2)
+    raw = (torch.randn(rows, seq_len, vocab, generator=g, device="cuda") * 4).to(dtype)
+    tok = [6, 0, 3, 6, 2]
+    for index in (None, tok):
+        got = ctx.logits_handoff(raw, index).cpu().numpy()
+        picked = torch.stack([raw[r, seq_len - 1 if index is None else index[r]] for r in range(rows)])
+        if kind is None:
+            want = picked.cpu().numpy()
+        else:
+            want = orc.cast(picked.view(torch.int16).cpu().numpy().view(np.uint16), kind, np.float32)
+        assert np.array_equal(bits(got), bits(want))
+    with pytest.raises(RuntimeError, match="outside"):
+        ctx.logits_handoff(raw, [0, 0, 0, 0, 7])

@@ -290,3 +290,27 @@ def test_spec_verify_dense_statistics_match_target(orc):
     first = np.where(acc == 1, draft[:, 0], tok)  # the first committed token
     freq = np.bincount(first, minlength=v) / n
     assert np.abs(freq - p).max() < 0.015
+
+
+def test_cast_known_answers(orc):
+    """DeviceInterface::Cast on the CPU (src/cpu/interface.cpp:74-106).  fp32->fp16 is
+    FastFloat32ToFloat16: it equals IEEE round-to-nearest for values that are not exact ties (numpy
+    agrees there), rounds ties up, keeps -0, and saturates beyond the fp16 range to 0x7FFF.  bf16->fp32
+    moves the bits up and canonicalises NaN; fp32->bf16 truncates; int32->int64 sign-extends."""
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal(20000) * 50).astype(np.float32)
+    x = x[(np.abs(x) > 1e-3) & ((x.view(np.uint32) & 0x1FFF) != 0x1000)]  # no exact ties
+    got = orc.cast(x, 2, np.uint16)
+    ieee = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, ieee)
+    assert list(orc.cast(np.array([0.0, -0.0, 1.0, -2.0, 65504.0, 1e6, -1e6], np.float32), 2, np.uint16)) == \
+        [0x0000, 0x8000, 0x3C00, 0xC000, 0x7BFF, 0x7FFF, 0xFFFF]
+    tie = np.array([1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11], np.float32)  # halfway between fp16 neighbours
+    assert list(orc.cast(tie, 2, np.uint16)) == [0x3C01, 0x3C02]  # up, where IEEE would give 0x3C00, 0x3C02
+    b = np.array([0x3F80, 0xC000, 0x0001, 0x7F80, 0xFF80, 0x7FC1, 0xFFFF, 0x0000, 0x8000], np.uint16)
+    f = orc.cast(b, 1, np.float32).view(np.uint32)
+    assert list(f) == [0x3F800000, 0xC0000000, 0x00010000, 0x7F800000, 0xFF800000, 0x7FC00000, 0x7FC00000, 0, 0x80000000]
+    assert list(orc.cast(np.array([1.0, -1.5, 3.14159], np.float32), 3, np.uint16)) == [0x3F80, 0xBFC0, 0x4049]
+    assert list(orc.cast(np.array([-1, 2 ** 31 - 1, -2 ** 31], np.int32), 4, np.int64)) == [-1, 2 ** 31 - 1, -2 ** 31]
+    h = np.arange(65536, dtype=np.uint16)
+    assert np.array_equal(orc.cast(h, 0, np.float32), orc.fp16_to_fp32(h))
