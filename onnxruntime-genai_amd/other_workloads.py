@@ -10,6 +10,10 @@ import numpy as np
 import torch
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per step from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these same commands, scaled by a
+# known-size copy (profiles/beam_step_kernels_config3.md, profiles/nucleus_kernels_config5.md); counters
+# cannot be read from inside the process.  None where no counter run exists.
+MEASURED_TRAFFIC = {"c3": 6_222_000_000 + 82_000_000, "c5": 278_000_000}
 
 
 def _timed(fn_step, K, W, graph=True):
@@ -51,7 +55,8 @@ def _line(args, metric, unit, value, ms_total, K, W, dtype, workload, extra, alg
         "vs_baseline": None, "dtype": dtype, "data": "synthetic",
         "config": dict({"workload": workload}, **extra),
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_step": algo_bytes},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "algorithmic_bytes_per_step": algo_bytes},
         "cpu_baseline": cpu,
     }
 
