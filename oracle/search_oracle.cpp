@@ -23,6 +23,9 @@
 //   and a model, so they cannot be replayed: exact-value parity of the scorer against the reference
 //   binary is "parity unpinned".
 //   KV gather: pinned by numpy.take.
+//   Cast conversions (fp16/bf16 <-> fp32, int32 -> int64): pinned by known answers and, for
+//   fp32 -> fp16, by agreement with IEEE round-to-nearest on every value that is not an exact tie
+//   (the reference file, src/models/utils.cpp, does not build without ONNX Runtime headers).
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
