@@ -5,10 +5,11 @@
 
 namespace ms {
 
-// Shape of the fused sampling kernel: 256 threads x 16 float4 = one 16K-logit chunk per workgroup.
-// Many logits per lane keep the per-wave selection overhead small against the streaming work, and
-// thread t's float4s (t, t+256, t+512, ...) make every wave an even sample of the whole chunk.
-constexpr int kSBlock = 256;
+// Shape of the fused sampling kernel: 512 threads x 16 float4 = one 32K-logit chunk per workgroup.
+// Many logits per lane keep the per-wave selection overhead small against the streaming work, few
+// chunks per row keep the finishing merge shallow (a 128K vocabulary is four sorted lists, two merge
+// levels), and thread t's float4s (t, t+512, t+1024, ...) make every wave an even sample of the chunk.
+constexpr int kSBlock = 512;
 constexpr int kSWaves = kSBlock / 64;
 constexpr int kSVec = 16;                   // 128-bit loads per thread
 constexpr int kSElems = kSVec * 4;          // logits held in registers per thread

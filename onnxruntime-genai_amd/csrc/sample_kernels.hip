@@ -1,11 +1,11 @@
 // Sampling kernels.
 //
-// sample_fused_kernel: one launch per step.  Every workgroup (256 threads x 64 logits) streams one
-// 16K-logit chunk of one row with 128-bit non-temporal loads (logits processing fused), keeps the chunk's
+// sample_fused_kernel: one launch per step.  Every workgroup (512 threads x 64 logits) streams one
+// 32K-logit chunk of one row with 128-bit non-temporal loads (logits processing fused), keeps the chunk's
 // best 64 candidates for the row's top-k and publishes them sorted; the last workgroup of a row to
-// arrive merges the chunks' sorted lists pairwise (bitonic merges in registers, three levels for
-// eight chunks) and runs the reference's scalar epilogue (softmax over the k, nucleus cut, categorical draw) in rank
-// order.  Rows in nucleus mode (k <= 1) only compact their
+// arrive merges the chunks' sorted lists pairwise (bitonic merges in registers, two levels for four
+// chunks) and runs the reference's scalar epilogue (softmax over the k, nucleus cut, categorical
+// draw) in rank order.  Rows in nucleus mode (k <= 1) only compact their
 // candidates here; nucleus_finish_kernel sorts them and finishes.  Anything the fast paths decline
 // (k > 64, heavy ties, tiny vocabularies) goes through general_row, an exact full sort.
 #include "kernels.h"
