@@ -143,42 +143,97 @@ struct LaneExp2Tab {
   }
 };
 
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_from_below(double x) {
+  const u64 b = static_cast<u64>(__double_as_longlong(x));
+  const uint32_t lo = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b), CTRL, ROW_MASK, 0xf, false);
+  const uint32_t hi = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b >> 32), CTRL, ROW_MASK, 0xf, false);
+  return __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
+}
+
+// Inclusive prefix sums over the wave in tree order (lanes without a source add +0.0).
+__device__ __forceinline__ double wave_scan_add(double x) {
+  x += dpp_from_below<0x111, 0xf>(x);  // row_shr:1
+  x += dpp_from_below<0x112, 0xf>(x);  // row_shr:2
+  x += dpp_from_below<0x114, 0xf>(x);  // row_shr:4
+  x += dpp_from_below<0x118, 0xf>(x);  // row_shr:8
+  x += dpp_from_below<0x142, 0xa>(x);  // row_bcast:15 into rows 1 and 3
+  x += dpp_from_below<0x143, 0xc>(x);  // row_bcast:31 into rows 2 and 3
+  return x;
+}
+
+__device__ __forceinline__ float read_lane(float x, int l) {
+  return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(x), l));
+}
+__device__ __forceinline__ double read_lane(double x, int l) {
+  const u64 b = static_cast<u64>(__double_as_longlong(x));
+  const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(b), l);
+  const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(b >> 32), l);
+  return __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
+}
+
 // Epilogue for k <= 64 run by one wave: lane j holds the j-th best (key64), j < m.
 // Follows ComputeSampledCategorical's top-k branch (src/sampling_distribution.h:243-281) and
-// std::discrete_distribution literally: every sum is accumulated in rank order.
+// std::discrete_distribution literally: every fp32 sum is accumulated in rank order.  The fp64
+// cumulative distribution is first evaluated in tree order on the raw weights; only if the draw lies
+// within rounding distance of one of its values is it rebuilt with the reference's own sequence of
+// operations (division by the sum, sequential partial sums), so the chosen position is always the
+// sequential one.
 __device__ __forceinline__ void wave_topk_epilogue(u64 key, int m, mi355x_sample_params prm, double u,
                                                    LaneExp2Tab tab, const RowOutputs& out) {
   const int lane = lane_id();
   m = __builtin_amdgcn_readfirstlane(m);
   const float score = key_to_float(key64_okey(key));
-  const float max_score = shfl_t<float>(score, 0);
+  const float max_score = read_lane(score, 0);
   const float inv_temp = 1.0f / prm.temperature;
   const float e_all = em::expf_core((score - max_score) * inv_temp, tab);
   const float e = lane < m ? e_all : 0.0f;
-  const float sum = shfl_t<float>(wave_serial_prefix(e, m), m - 1);
+  const float sum = read_lane(wave_serial_prefix(e, m), m - 1);
   const float pr = sum > 0.0f ? e / sum : e;
-  const float cum = wave_serial_prefix(pr, m);
+  // cumulative probabilities, eight chain steps at a time; with a top-p cut the chain stops at the
+  // first group that contains the cut (lanes below the number of steps done hold final values)
+  const bool cut = prm.p > 0.0f && prm.p < 1.0f;
+  float cum = 0.0f;
   int keep = m;
-  if (prm.p > 0.0f && prm.p < 1.0f) {
-    const int f = first_lane(__ballot(lane < m && cum >= prm.p));
-    if (f >= 0) keep = f + 1;
+  for (int t = 0; t < m; t += 8) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const float prev = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(cum), 0x138, 0xf, 0xf, false));
+      cum = prev + pr;
+    }
+    if (cut) {
+      const int f = first_lane(__ballot(lane < t + 8 && lane < m && cum >= prm.p));
+      if (f >= 0) {
+        keep = f + 1;
+        break;
+      }
+    }
   }
   keep = __builtin_amdgcn_readfirstlane(keep);
-  const float keep_sum = shfl_t<float>(cum, keep - 1);
+  const float keep_sum = read_lane(cum, keep - 1);
   const float inv = keep_sum > 0.0f ? 1.0f / keep_sum : 0.0f;
   const float q = pr * inv;
   int pos = 0;
   if (keep >= 2) {
     const double qd = lane < keep ? static_cast<double>(q) : 0.0;
-    const double dsum = shfl_t<double>(wave_serial_prefix(qd, keep), keep - 1);
-    const double pn = qd / dsum;
-    double cp = wave_serial_prefix(pn, keep);
-    if (lane == keep - 1) cp = 1.0;
-    pos = first_lane(__ballot(lane < keep && cp >= u));
+    const double w = wave_scan_add(qd);
+    const double total = read_lane(w, keep - 1);
+    const double target = u * total;
+    const double guard = 16.0 * static_cast<double>(keep) * 1.1102230246251565e-16 * total;
+    const bool risky = __ballot(lane < keep - 1 && fabs(w - target) <= guard) != 0ull;
+    if (!risky) {
+      pos = first_lane(__ballot(lane < keep && (lane == keep - 1 || w >= target)));
+    } else {
+      const double dsum = read_lane(wave_serial_prefix(qd, keep), keep - 1);
+      const double pn = qd / dsum;
+      double cp = wave_serial_prefix(pn, keep);
+      if (lane == keep - 1) cp = 1.0;
+      pos = first_lane(__ballot(lane < keep && cp >= u));
+    }
     if (pos < 0) pos = keep - 1;
   }
   const uint32_t idx = key64_index(key);
-  const int32_t tok = static_cast<int32_t>(shfl_t<uint32_t>(idx, pos));
+  const int32_t tok = static_cast<int32_t>(__builtin_amdgcn_readlane(idx, pos));
   if (lane == 0) {
     *out.token = tok;
     if (out.kept_count) *out.kept_count = keep;

@@ -143,6 +143,32 @@ def test_sample_topk_topp_small_k(ctx, orc, rows, vocab, k, p, t):
     assert ctx.fallback_rows() == before  # all rows stayed on the single-pass path
 
 
+@pytest.mark.parametrize("vocab,k,p,t", [(128256, 50, 0.9, 0.7), (5000, 30, 0.0, 1.0), (201088, 0, 0.9, 1.0)])
+def test_draw_on_cdf_boundaries(ctx, orc, vocab, k, p, t):
+    """Uniform draws placed exactly on, just below and just above values of the cumulative distribution
+    std::discrete_distribution builds (double quotients summed in sequence): the kernels' tree-order
+    CDF cannot decide these and must fall back to the sequential construction."""
+    say("cdf boundaries", vocab, k, p, t)
+    rng = np.random.default_rng(vocab + k)
+    base = (rng.standard_normal(vocab) * 3).astype(np.float32)
+    idx, probs = orc.sampled_categorical(base, k, p, t)
+    assert len(idx) >= 3
+    total = 0.0
+    for q in probs:  # libstdc++: sum in double, in order
+        total += float(q)
+    cp, run = [], 0.0
+    for q in probs[:-1]:
+        run += float(q) / total
+        cp.append(run)
+    picks = [0, len(cp) // 2, len(cp) - 1]
+    us = []
+    for j in picks:
+        us += [cp[j], np.nextafter(cp[j], 0.0), np.nextafter(cp[j], 1.0)]
+    us = np.array([v for v in us if 0.0 <= v < 1.0], np.float64)
+    x = np.tile(base, (len(us), 1))
+    sample_and_check(ctx, orc, x, us, k, p, t, cap=64)
+
+
 def test_config2_topk_topp_batch64(ctx, orc):
     """BASELINE config 2 at full size: batch 64, vocab 128256, N(0,3^2) logits + 8 peaks/row at +10,
     T=0.7, k=50, p=0.9, shared uniforms; 4 of the 128 steps."""
