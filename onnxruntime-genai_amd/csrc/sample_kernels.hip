@@ -104,24 +104,16 @@ __device__ __forceinline__ float nucleus_depth(mi355x_sample_params prm, int voc
   return d * prm.temperature;
 }
 
-constexpr uint32_t kPark = 6u;  // float4s with a hit a thread can park per chunk
+constexpr int kWaveListCap = 128;  // hits one wave can list per chunk
 
 // LDS of the fused kernel.
 struct FusedShared {
   uint32_t hist_bits[kSChunk / 32];
   uint32_t mask_bits[kSChunk / 32];
-  u64 list[kListCap];   // this chunk's candidates before the sort
-  u64 list_hi[64];      // second half of a long list, sorted ascending
-  union {               // the parking rows are dead before the merge buffers come into use
-    struct {
-      v4f park_val[kSBlock * kPark];  // per-thread parking rows of the streaming filter
-      int park_idx[kSBlock * kPark];
-    };
-    struct {
-      u64 lists[kAllCap];       // the chunks' sorted candidate lists of a row (finishing workgroup only)
-      u64 lists2[kAllCap / 2];  // second buffer of the merge tree
-    };
-  };
+  u64 wave_list[kSWaves * kWaveListCap];  // each wave's hits of this chunk, before the sort
+  u64 list_hi[64];          // second half of a long list, sorted ascending
+  u64 lists[kAllCap];       // the chunks' sorted candidate lists of a row (finishing workgroup only)
+  u64 lists2[kAllCap / 2];  // second buffer of the merge tree
   uint32_t pool[64];
   uint32_t wave_val[kSWaves];
   u64 wave_val64[kSWaves];
@@ -408,72 +400,57 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   MS_STAGE(2, tau);
   // tau == 0: the chunk has fewer than k elements -- keep them all
   const float tau_f = tau != 0u ? key_to_float(tau) : -__builtin_inff();
-  // Hits are rare (about k per chunk).  A thread parks every float4 that holds a hit in a private
-  // kPark-entry LDS row (plain writes, nothing to wait for) and counts its hits; a block-wide prefix
-  // sum of the counts then gives every thread its slots in the chunk's global segment.
-  uint32_t lc = 0u, ec = 0u;
+  // Hits are rare (about k per chunk).  Every wave lists its own hits in a private LDS segment: the
+  // slot of a hit is the wave's running count (a scalar) plus the number of hitting lanes below, so
+  // no atomics, no second pass and no block-wide prefix are needed.
+  uint32_t woff = 0u;
 #pragma unroll
   for (int j = 0; j < kSVec; ++j) {
     if (__ballot(qm[j] >= tau_f) != 0ull) {
-      if (qm[j] >= tau_f) {
-        if (lc < kPark) {
-          sm.park_val[tid * kPark + lc] = v4f{v[j * 4], v[j * 4 + 1], v[j * 4 + 2], v[j * 4 + 3]};
-          sm.park_idx[tid * kPark + lc] = elem_index(chunk, j, 0);
-        }
-        ++lc;
-        ec += (v[j * 4] >= tau_f) + (v[j * 4 + 1] >= tau_f) + (v[j * 4 + 2] >= tau_f) + (v[j * 4 + 3] >= tau_f);
-      }
-    }
-  }
-  uint32_t n_c;
-  {
-    // exclusive prefix of ec inside the wave: ec < 32, so five ballots give it without lane traffic
-    uint32_t before = 0u, wtot = 0u;
-    const u64 lt = (1ull << lane) - 1ull;
-#pragma unroll
-    for (int b = 0; b < 5; ++b) {
-      const u64 m = __ballot((ec >> b) & 1u);
-      before += static_cast<uint32_t>(__popcll(m & lt)) << b;
-      wtot += static_cast<uint32_t>(__popcll(m)) << b;
-    }
-    const u64 over = __ballot(lc > kPark);
-    if (lane == 0) sm.wave_val[wave] = wtot | (over ? 0x80000000u : 0u);
-    __syncthreads();
-    uint32_t base = 0u, tot = 0u;
-#pragma unroll
-    for (int w = 0; w < kSWaves; ++w) {
-      const uint32_t wv = sm.wave_val[w];
-      if (w < wave) base += wv & 0x7fffffffu;
-      tot += wv & 0x7fffffffu;
-      if (wv & 0x80000000u) tot = 0x40000000u;  // a thread ran out of parking rows: treat as overflow
-    }
-    n_c = tot;
-    uint32_t pos = base + before;
-    const uint32_t lim = lc < kPark ? lc : kPark;
-    for (uint32_t i = 0; i < lim; ++i) {
-      const v4f q = sm.park_val[tid * kPark + i];
-      const uint32_t id0 = static_cast<uint32_t>(sm.park_idx[tid * kPark + i]);
-      const float qv[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        if (qv[c] >= tau_f) {
-          if (pos < kListCap) sm.list[pos] = make_key64(order_key(qv[c]), id0 + c);
-          ++pos;
+        const bool hit = v[j * 4 + c] >= tau_f;
+        const u64 b = __ballot(hit);
+        if (b == 0ull) continue;
+        if (hit) {
+          const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
+                                                                __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), 0u));
+          // key64 of a real element is never 0 (its index half is ~idx != 0), so 0 marks an empty slot
+          if (pos < kWaveListCap)
+            sm.wave_list[wave * kWaveListCap + pos] =
+                make_key64(order_key(v[j * 4 + c]), static_cast<uint32_t>(elem_index(chunk, j, c)));
         }
+        woff += static_cast<uint32_t>(__popcll(b));
       }
     }
   }
+  if (lane == 0) sm.wave_val[wave] = woff;
   __syncthreads();
   MS_STAGE(3, tau);
   // The chunk publishes its best 64 candidates sorted (best first, zero-padded): nothing ranked lower
   // inside its own chunk can be among the row's k <= 64 best.  Waves 0 and 1 sort one half of the
   // list each; wave 0 merges, stores, and -- once its stores have been performed -- signals arrival.
-  const bool overflow = n_c > static_cast<uint32_t>(kListCap);
+  uint32_t n_c = 0u;
+  bool overflow = false;
+#pragma unroll
+  for (int w = 0; w < kSWaves; ++w) {
+    n_c += sm.wave_val[w];
+    overflow = overflow || sm.wave_val[w] > static_cast<uint32_t>(kWaveListCap);
+  }
+  overflow = overflow || n_c > static_cast<uint32_t>(kListCap);
   const bool two_halves = n_c > 64u;
   u64 mykey = 0;
   if (wave < 2 && !overflow) {
-    const uint32_t p = static_cast<uint32_t>(wave) * 64u + static_cast<uint32_t>(lane);
-    mykey = p < n_c ? sm.list[p] : 0;
+    // entry p of the concatenated wave lists
+    uint32_t p = static_cast<uint32_t>(wave) * 64u + static_cast<uint32_t>(lane);
+    if (p < n_c) {
+      int w = 0;
+      while (p >= sm.wave_val[w]) {
+        p -= sm.wave_val[w];
+        ++w;
+      }
+      mykey = sm.wave_list[w * kWaveListCap + p];
+    }
     if (wave == 0 || two_halves) mykey = wave_sort_desc_fast<u64>(mykey);
     if (wave == 1 && two_halves) sm.list_hi[63 - lane] = mykey;
   }
