@@ -434,7 +434,7 @@ __device__ __forceinline__ void wave_key_exchange(u64 (&x)[R], bool keep_max) {
 // inside a thread, distances below 64*R cross lanes with data-parallel-primitive moves, and only the
 // ten stages with larger distances go through LDS.
 template <int R>
-__device__ void block_sort_desc_regs(u64* lds) {
+__device__ __noinline__ void block_sort_desc_regs(u64* lds) {
   constexpr int kT = 1024;
   const int t = threadIdx.x;
   u64 x[R];

@@ -581,7 +581,7 @@ constexpr int kSortBuckets = 4096;
 constexpr int kBucketCap = 64;
 constexpr size_t kFinishLds = kNucleusCap * sizeof(u64) + (kSortBuckets + 1) * sizeof(uint32_t);
 
-__device__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n, float fmax, float fthr, uint32_t* red) {
+__device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n, float fmax, float fthr, uint32_t* red) {
   constexpr int R = kNucleusCap / kFinishBlock;
   const int t = threadIdx.x;
   u64 k[R];
