@@ -539,22 +539,35 @@ __device__ bool block_sample_epilogue(Sorted sorted, Exps exps, int n_sorted, in
   } else {
     const float p = prm.p;
     const int limit = n_sorted < vocab ? n_sorted : vocab;
-    int si;
     const int V = vocab;
-    float prefix = block_seq_sum<ITEMS>(
-        0.0f, limit, exps,
-        [=](float pf, float e, int i) {
-          const float tail = static_cast<float>(V - i - 1) * e;
-          return pf >= p * (pf + tail);
-        },
-        &si, sh, nullptr, kEpiHead);
+    // The reference sorts in batches that end at 16, 64, 256, ... elements and recognises a stop
+    // only when it lies strictly inside a batch (src/sampling_distribution.h:166-181): a stop
+    // on the last element of a batch smaller than the row is missed and the search goes on in
+    // the next batch with the running sum it has.
+    int base = 0;
     int cutoff;
-    if (si >= 0) {
-      cutoff = si + 1;
-    } else if (limit == vocab) {
-      cutoff = vocab;
-    } else {
-      return false;
+    float prefix = 0.0f;
+    bool prefix_is_keep_sum = true;
+    for (;;) {
+      const int b = base;
+      int si;
+      prefix = block_seq_sum<ITEMS>(
+          prefix, limit - b, [=](int i) { return exps(i + b); },
+          [=](float pf, float e, int i) {
+            const float tail = static_cast<float>(V - (i + b) - 1) * e;
+            return pf >= p * (pf + tail);
+          },
+          &si, sh, nullptr, b == 0 ? kEpiHead : 0);
+      if (si < 0) {
+        if (limit != vocab) return false;
+        cutoff = vocab;
+        break;
+      }
+      cutoff = b + si + 1;
+      const bool batch_end = cutoff >= 16 && (cutoff & (cutoff - 1)) == 0 && ((__ffs(cutoff) - 1) & 1) == 0;
+      if (!batch_end || cutoff >= vocab) break;
+      if (cutoff >= limit) return false;
+      base = cutoff;
     }
     if (vocab <= 64) {  // exact-partition override, src/sampling_distribution.h:186-203
       if (n_sorted < vocab) return false;
@@ -566,10 +579,10 @@ __device__ bool block_sample_epilogue(Sorted sorted, Exps exps, int n_sorted, in
       (void)c;
       if (sj >= 0) {
         cutoff = sj + 1;
-        si = -1;
+        prefix_is_keep_sum = false;
       }
     }
-    if (si < 0 || cutoff != si + 1) prefix = block_seq_sum<ITEMS>(0.0f, cutoff, exps, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead);
+    if (!prefix_is_keep_sum) prefix = block_seq_sum<ITEMS>(0.0f, cutoff, exps, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead);
     keep = cutoff;
     scale = prefix > 0.0f ? 1.0f / prefix : 0.0f;
   }

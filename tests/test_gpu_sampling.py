@@ -1,6 +1,8 @@
 """GPU parity: argmax, logits processing and top-k / top-p sampling through the C ABI against the CPU
 oracle on the same seeded inputs.  Bit-exact token ids and indices; probabilities compared bitwise
 too (tolerance stated by the task: 1e-5 relative -- the kernels meet it with zero difference)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -219,6 +221,23 @@ def test_sample_nucleus(ctx, orc, rows, vocab, p, t):
     sample_and_check(ctx, orc, x, u, 0, p, t, cap=128)
 
 
+@pytest.mark.parametrize("vocab", [32, 128, 130, 512, 2048, 8192, 32768, 131072])
+def test_nucleus_stop_on_last_element_of_a_sort_batch(ctx, orc, vocab):
+    """Constant rows with p = 0.5 meet the tail-bound stop at element vocab/2; where that is the end of one of
+    the reference's sort batches (16, 64, 256, ...) the stop is only noticed one element later
+    (src/sampling_distribution.h:166-181), so vocab/2 + 1 tokens are kept."""
+    say("nucleus batch end", vocab)
+    rng = np.random.default_rng(vocab)
+    x = np.full((3, vocab), -0.5, np.float32)
+    x[1, :] = 0.0
+    x[2, vocab // 2:] = -0.5000001  # a second, slightly lower level
+    u = rng.random(3)
+    sample_and_check(ctx, orc, x, u, 0, 0.5, 1.0, cap=256)
+    idx, _ = orc.sampled_categorical(x[0], 0, 0.5, 1.0)
+    quirk = vocab > 64 and vocab // 2 in (16, 64, 256, 1024, 4096, 16384, 65536)
+    assert len(idx) == vocab // 2 + (1 if quirk else 0)
+
+
 @pytest.mark.parametrize("frac,quantum", [(0.004, 0.0), (0.012, 0.0), (0.03, 0.0), (0.012, 0.5), (0.03, 0.5),
                                            (0.06, 0.25)])
 def test_nucleus_candidate_counts_and_ties(ctx, orc, frac, quantum):
@@ -284,6 +303,61 @@ def test_sample_heterogeneous_rows(ctx, orc):
     for r, (k, p, t) in enumerate(params):
         assert tok[r] == orc.sample_row(x[r], k, p, t, u[r]), r
     assert tok[0] == orc.argmax(x[0])
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("MI355X_RANDOM_CASES", "300"))))
+def test_sample_randomised_shapes_and_parameters(ctx, orc, seed):
+    """Differential test over random shapes (vocabularies around the 32768-logit chunk edges included),
+    per-row (k, p, T) mixes, logit scales, coarse grids (ties), grammar masks, repetition penalties and
+    min-length masking: tokens of every row and the kept sets of uniform-parameter cases must equal
+    the oracle's."""
+    rng = np.random.default_rng(1000 + seed)
+    edges = [1, 2, 63, 64, 65, 255, 4097, 32767, 32768, 32769, 65536, 65537, 98304, 131071, 131073, 196608, 201088]
+    vocab = int(rng.choice(edges)) if seed % 2 else int(rng.integers(2, 140000))
+    rows = int(rng.integers(1, 7))
+    scale = float(rng.choice([0.05, 1.0, 3.0, 30.0]))
+    x = (rng.standard_normal((rows, vocab)) * scale).astype(np.float32)
+    if seed % 3 == 0:
+        x = (np.round(x * 2) / 2).astype(np.float32)  # heavy ties
+    if seed % 5 == 0:
+        x[0, :] = 1.25  # a constant row
+    say("sample random", seed, rows, vocab, scale)
+    xf, proc = None, x
+    if seed % 4 in (1, 2):
+        mask = make_mask(rng, rows, vocab, float(rng.choice([0.02, 0.5, 0.98])))
+        hist = rng.integers(0, vocab, (rows, int(rng.integers(1, 200)))).astype(np.int32)
+        pen = float(rng.choice([1.0, 1.3, 0.8]))
+        eos = [int(rng.integers(0, vocab))]
+        xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                               repetition_penalty=pen, eos_ids=eos, apply_min_length=bool(seed % 8 == 1))
+        proc = orc.apply_mask(x, mask)
+        proc = np.stack([orc.apply_repetition_penalty(orc.apply_min_length(proc[r], 0, 1 if seed % 8 == 1 else 0, eos),
+                                                       hist[r], pen) for r in range(rows)])
+    u = rng.random(rows)
+
+    def params():
+        k = int(rng.choice([0, 1, 2, 5, 40, 50, 64, 65, 200, vocab, vocab + 7]))
+        p = float(rng.choice([0.0, 0.1, 0.5, 0.9, 0.999, 1.0]))
+        return k, p, float(rng.uniform(0.3, 2.0))
+
+    if seed % 2:  # heterogeneous rows
+        per_row = [params() for _ in range(rows)]
+        tok = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), per_row=per_row, xf=xf).cpu().numpy()
+        for r, (k, p, t) in enumerate(per_row):
+            assert tok[r] == orc.sample_row(proc[r], k, p, t, u[r]), (r, k, p, t)
+    else:
+        k, p, t = params()
+        cap = 256
+        tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=k, p=p, temperature=t,
+                                     xf=xf, kept_capacity=cap)
+        tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+        for r in range(rows):
+            idx, probs = orc.sampled_categorical(proc[r], k, p, t)
+            n = min(len(idx), cap)
+            assert kc[r] == len(idx), (r, k, p, t)
+            assert np.array_equal(ki[r, :n], idx[:n]), (r, k, p, t)
+            assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), (r, k, p, t)
+            assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (r, k, p, t)
 
 
 def test_argument_errors(ctx):

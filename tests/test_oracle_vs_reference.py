@@ -39,6 +39,22 @@ def test_sampled_categorical_nucleus_bit_exact(orc, ref):
             assert np.array_equal(i1, i2) and np.array_equal(bits(p1), bits(p2))
 
 
+def test_nucleus_stop_on_last_element_of_a_sort_batch(orc, ref):
+    """A constant row of V logits with p = 0.5 satisfies the tail-bound stop first at element V/2.  When
+    V/2 is the end of a sort batch (16, 64, 256, ... elements) the reference does not notice the stop until
+    the next batch, so V/2 + 1 elements are kept; otherwise V/2.  Rows of at most 64 logits take the
+    exact-partition override and keep V/2.  Only lengths and probabilities are compared: the order of
+    tied ids under std::partial_sort is unspecified."""
+    for v, want in ((32, 16), (128, 65), (512, 257), (2048, 1025), (8192, 4097), (32768, 16385), (131072, 65537),
+                    (130, 65), (1000, 500), (2046, 1023)):
+        x = np.full(v, 0.75, np.float32)
+        i1, p1 = orc.sampled_categorical(x, 0, 0.5, 1.0)
+        i2, p2 = ref.sampled_categorical(x, 0, 0.5, 1.0)
+        assert len(i1) == len(i2) == want, (v, len(i1), len(i2))
+        assert np.array_equal(bits(p1), bits(p2))
+        assert np.array_equal(i1, np.arange(want))  # the oracle's tie rule: lowest index first
+
+
 def test_config_shaped_rows_bit_exact(orc, ref):
     rng = np.random.default_rng(12)
     # C2-like: V=128256, 8 peaks at +10, T=0.7, k=50, p=0.9
