@@ -326,6 +326,9 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float
   double total = 0.0;
   for (int k = 0; k < nw; ++k) total += sh.dred[k];
   __syncthreads();
+  // A NaN weight (a row of -inf logits gives exp(-inf - -inf)) makes every quotient w/sum NaN; the
+  // binary search of std::discrete_distribution over NaNs and the forced final 1.0 ends on 0.
+  if (total != total) return 0;
   const double guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16 * total;
   const double target = u * total;
   double carry = 0.0;

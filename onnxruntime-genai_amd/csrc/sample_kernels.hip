@@ -223,6 +223,7 @@ __device__ __forceinline__ void wave_topk_epilogue(u64 key, int m, mi355x_sample
       pos = first_lane(__ballot(lane < keep && cp >= u));
     }
     if (pos < 0) pos = keep - 1;
+    if (total != total) pos = 0;  // NaN weights: std::lower_bound over NaN quotients ends on 0
   }
   const uint32_t idx = key64_index(key);
   const int32_t tok = static_cast<int32_t>(__builtin_amdgcn_readlane(idx, pos));

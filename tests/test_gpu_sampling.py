@@ -201,6 +201,24 @@ def test_sample_ties_and_degenerate_rows(ctx, orc):
     sample_and_check(ctx, orc, x, u, 10, 0.0, 1.0)
 
 
+@pytest.mark.parametrize("vocab", [2, 70, 5000, 40000])
+def test_sample_rows_without_finite_logits(ctx, orc, vocab):
+    """A row of -inf logits (everything masked, then a penalty above 1 applied to lowest()) has NaN
+    weights; the reference's draw then lands on position 0 of its kept list whatever the uniform is."""
+    say("sample all -inf", vocab)
+    x = np.full((2, vocab), -np.inf, np.float32)
+    x[1, vocab // 2] = 0.0
+    u = np.array([0.73, 0.41])
+    for k, p in ((0, 0.9), (1, 0.0), (5, 0.5), (50, 0.0), (200, 0.9)):
+        tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=k, p=p, temperature=0.8,
+                                     kept_capacity=64)
+        for r in range(2):
+            idx, probs = orc.sampled_categorical(x[r], k, p, 0.8)
+            assert kc[r].item() == len(idx), (k, p, r)
+            assert tok[r].item() == idx[orc.discrete_draw(probs, u[r])], (k, p, r)
+        assert tok[0].item() == 0 and tok[1].item() == vocab // 2
+
+
 def test_sample_large_k_general_path(ctx, orc):
     say("sample k=200")
     rng = np.random.default_rng(4)
