@@ -167,7 +167,8 @@ int mi355x_beam_scorer_hypothesis(mi355x_beam_scorer* s, void* stream, int batch
 
 /* KV-cache beam reorder: DefaultKeyValueCache::PickPastState (src/models/kv_cache.cpp:710-740):
  * for every tensor t and row j, past[t][j] = present[t][beam_indices[j]], blocks of block_bytes
- * bytes (a multiple of 16).  present/past: HOST arrays of n_tensors device pointers (copied by the
+ * bytes (any size; blocks and tensors aligned to 16 bytes move with 128-bit accesses, others with the
+ * widest access they are aligned to).  present/past: HOST arrays of n_tensors device pointers (copied by the
  * call); beam_indices: device [rows]. */
 int mi355x_kv_gather(mi355x_search_ctx* ctx, void* stream, const void* const* present,
                      void* const* past, int n_tensors, const int32_t* beam_indices, int rows,

@@ -444,18 +444,20 @@ int mi355x_kv_gather(mi355x_search_ctx* ctx, void* stream, const void* const* pr
                      int n_tensors, const int32_t* beam_indices, int rows, size_t block_bytes) {
   if (!ctx || !present || !past || !beam_indices) return Fail(MI355X_E_INVALID, "null argument");
   if (n_tensors <= 0 || rows <= 0 || block_bytes == 0) return Fail(MI355X_E_INVALID, "non-positive size");
-  if (block_bytes % 16 != 0) return Fail(MI355X_E_INVALID, "block_bytes (%zu) must be a multiple of 16", block_bytes);
   if (static_cast<size_t>(n_tensors) * 2 > ctx->ptr_table_cap || n_tensors > 65535 || rows > 65535)
     return Fail(MI355X_E_CAPACITY, "too many tensors (%d) or rows (%d)", n_tensors, rows);
+  // Widest power-of-two access (at most 16 bytes) that every block of every tensor is aligned to.
+  uintptr_t align = static_cast<uintptr_t>(block_bytes);
   for (int t = 0; t < n_tensors; ++t) {
     if (!present[t] || !past[t]) return Fail(MI355X_E_INVALID, "null tensor pointer at %d", t);
-    if ((reinterpret_cast<uintptr_t>(present[t]) | reinterpret_cast<uintptr_t>(past[t])) & 15u)
-      return Fail(MI355X_E_INVALID, "tensor %d is not 16-byte aligned", t);
+    align |= reinterpret_cast<uintptr_t>(present[t]) | reinterpret_cast<uintptr_t>(past[t]);
   }
+  int width = 16;
+  while (align & static_cast<uintptr_t>(width - 1)) width >>= 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
   HIP_TRY(hipMemcpyAsync(ctx->ptr_table, present, sizeof(void*) * n_tensors, hipMemcpyHostToDevice, s));
   HIP_TRY(hipMemcpyAsync(ctx->ptr_table + n_tensors, past, sizeof(void*) * n_tensors, hipMemcpyHostToDevice, s));
-  HIP_TRY(ms_launch_kv_gather(ctx->ptr_table, ctx->ptr_table + n_tensors, n_tensors, beam_indices, rows, block_bytes, s));
+  HIP_TRY(ms_launch_kv_gather(ctx->ptr_table, ctx->ptr_table + n_tensors, n_tensors, beam_indices, rows, block_bytes, width, s));
   return MI355X_OK;
 }
 

@@ -126,7 +126,8 @@ hipError_t ms_launch_process_logits(float* logits, int64_t row_stride, int rows,
 hipError_t ms_launch_softmax(float* scores, int64_t row_stride, int rows, int vocab, float temperature,
                              int log_softmax, hipStream_t stream);
 hipError_t ms_launch_kv_gather(const void* const* present_dev, void* const* past_dev, int n_tensors,
-                               const int32_t* beam_indices, int rows, size_t block_bytes, hipStream_t stream);
+                               const int32_t* beam_indices, int rows, size_t block_bytes, int width,
+                               hipStream_t stream);
 hipError_t ms_launch_spec_verify(const float* p_target, const float* p_draft, const int32_t* draft_tokens,
                                  const float* accept_u, const double* sample_u, int batch, int K, int vocab,
                                  int32_t* accepted_len, int32_t* final_token, hipStream_t stream);

@@ -68,6 +68,21 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(const void* const* prese
   }
 }
 
+// The same gather for blocks or tensors that are not 16-byte aligned (odd head sizes, sliced views): T is
+// the widest unsigned type that divides the block size and every tensor address.  grid = (tiles, rows,
+// tensors); a workgroup strides over its row's block.
+template <typename T>
+__global__ __launch_bounds__(256) void kv_gather_narrow_kernel(const void* const* present, void* const* past,
+                                                               const int32_t* beam_indices, size_t block_bytes) {
+  const int row = blockIdx.y, t = blockIdx.z;
+  const T* src = reinterpret_cast<const T*>(static_cast<const char*>(present[t]) +
+                                            static_cast<size_t>(beam_indices[row]) * block_bytes);
+  T* dst = reinterpret_cast<T*>(static_cast<char*>(past[t]) + static_cast<size_t>(row) * block_bytes);
+  const size_t n = block_bytes / sizeof(T);
+  for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += static_cast<size_t>(gridDim.x) * 256)
+    dst[i] = src[i];
+}
+
 // ---- speculative-decoding verification ---------------------------------------------------------------
 // One 1024-thread block per batch entry.  Accept loop of SpeculativeDecodingStrategy::RunRound
 // (src/speculative_decoding_strategy.cpp:718-762) on dense distributions, then the round's single
@@ -210,10 +225,38 @@ extern "C" hipError_t ms_launch_softmax(float* scores, int64_t row_stride, int r
 }
 
 extern "C" hipError_t ms_launch_kv_gather(const void* const* present_dev, void* const* past_dev, int n_tensors,
-                                          const int32_t* beam_indices, int rows, size_t block_bytes, hipStream_t stream) {
-  const unsigned tiles = static_cast<unsigned>((block_bytes + ms::kGatherTile - 1) / ms::kGatherTile);
-  hipLaunchKernelGGL(ms::kv_gather_kernel, dim3(tiles, rows, n_tensors), dim3(256), 0, stream, present_dev, past_dev,
-                     beam_indices, block_bytes);
+                                          const int32_t* beam_indices, int rows, size_t block_bytes, int width,
+                                          hipStream_t stream) {
+  if (width == 16) {
+    const unsigned tiles = static_cast<unsigned>((block_bytes + ms::kGatherTile - 1) / ms::kGatherTile);
+    hipLaunchKernelGGL(ms::kv_gather_kernel, dim3(tiles, rows, n_tensors), dim3(256), 0, stream, present_dev, past_dev,
+                       beam_indices, block_bytes);
+    return hipGetLastError();
+  }
+  const size_t per_wg = static_cast<size_t>(256) * 8 * width;  // eight elements per thread
+  size_t tiles = (block_bytes + per_wg - 1) / per_wg;
+  if (tiles > 4096) tiles = 4096;
+  const dim3 grid(static_cast<unsigned>(tiles), rows, n_tensors);
+  switch (width) {
+    case 8:
+      hipLaunchKernelGGL(ms::kv_gather_narrow_kernel<uint64_t>, grid, dim3(256), 0, stream, present_dev, past_dev,
+                         beam_indices, block_bytes);
+      break;
+    case 4:
+      hipLaunchKernelGGL(ms::kv_gather_narrow_kernel<uint32_t>, grid, dim3(256), 0, stream, present_dev, past_dev,
+                         beam_indices, block_bytes);
+      break;
+    case 2:
+      hipLaunchKernelGGL(ms::kv_gather_narrow_kernel<uint16_t>, grid, dim3(256), 0, stream, present_dev, past_dev,
+                         beam_indices, block_bytes);
+      break;
+    case 1:
+      hipLaunchKernelGGL(ms::kv_gather_narrow_kernel<uint8_t>, grid, dim3(256), 0, stream, present_dev, past_dev,
+                         beam_indices, block_bytes);
+      break;
+    default:
+      return hipErrorInvalidValue;
+  }
   return hipGetLastError();
 }
 

@@ -71,8 +71,9 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
   if (a.emit_topk) {
     const int kk = prm.k < V ? prm.k : V;
     for (int j = threadIdx.x; j < kk; j += blockDim.x) {
-      a.out_tokens[static_cast<size_t>(row) * prm.k + j] = static_cast<int32_t>(key64_index(scratch[j]));
-      a.out_scores[static_cast<size_t>(row) * prm.k + j] = key_to_float(key64_okey(scratch[j]));
+      const uint32_t id = key64_index(scratch[j]);
+      a.out_tokens[static_cast<size_t>(row) * prm.k + j] = static_cast<int32_t>(id);
+      a.out_scores[static_cast<size_t>(row) * prm.k + j] = lrow[id];  // the value itself: keys do not tell -0 from +0
     }
     if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
     return;
@@ -546,8 +547,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     if (lane >= kk) final_key = 0;
     if (a.emit_topk) {
       if (lane < kk) {
-        a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(key64_index(final_key));
-        a.out_scores[static_cast<size_t>(row) * prm.k + lane] = key_to_float(key64_okey(final_key));
+        const uint32_t id = key64_index(final_key);
+        a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(id);
+        a.out_scores[static_cast<size_t>(row) * prm.k + lane] =
+            a.logits[static_cast<size_t>(row) * a.row_stride + id];  // keys do not tell -0 from +0
       }
     } else {
       wave_topk_epilogue(final_key, kk, prm, u, tab, row_outputs(a, row));
