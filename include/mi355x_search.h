@@ -40,15 +40,27 @@ extern "C" {
 typedef struct mi355x_search_ctx mi355x_search_ctx;
 
 /* Logits processing fused into every selection entry point, applied per element in the reference's
- * order (src/standard_decoding_strategy.cpp:24-32): grammar mask -> min-length -> repetition penalty.
+ * order (src/standard_decoding_strategy.cpp:24-32; LogitsPenaltyProcessor::Apply,
+ * src/sampling_distribution.h:100-110): grammar mask -> min-length -> repetition penalty ->
+ * no-repeat-n-gram ban.
  *   mask     device [rows, (vocab-1)/32+1] uint32, bit set = token allowed, else the logit becomes
  *            lowest() (src/constrained_logits_processor.cpp:246-258, layout :174-183); NULL = none.
  *   history  device [rows, history_stride] int32 token ids, the first history_len of each row valid
  *            (Sequences::GetSequence, src/sequences.h:18); every DISTINCT in-range id has its logit
  *            s replaced by s<0 ? s*penalty : s/penalty (src/sampling_distribution.h:41-62).
- *            NULL or penalty == 1.0f = none.
+ *            NULL or penalty == 1.0f = none.  history_stride 0 lets all rows share one buffer.
  *   eos_ids  with apply_min_length != 0 each in-range id gets lowest()
  *            (src/sampling_distribution.h:26-35; the caller evaluates current_length < min_length).
+ *   history_lens  optional device [rows] int32: row r uses the first history_lens[r] ids of its
+ *            history row instead of history_len, and -- when min_length > 0 -- gets the EOS masking
+ *            only if history_lens[r] < min_length.  This is the (current_length, prefix) pair of
+ *            ComputeTargetTokenSelection (src/speculative_sampling.h:59-79), where the verify rows
+ *            of one sequence see prefixes that grow by one proposal token per row
+ *            (src/speculative_decoding_strategy.cpp:645-656).
+ *   no_repeat_ngram_size  n > 0: every id that followed an earlier occurrence of the row's last n-1
+ *            history ids gets lowest(), after the penalty (ApplyNoRepeatNgramToLogits,
+ *            src/sampling_distribution.h:64-79; Search_Cpu::ApplyNoRepeatNgram,
+ *            src/search.cpp:432-469).  Needs history.
  */
 typedef struct mi355x_logits_xform {
   const uint32_t* mask;
@@ -59,6 +71,9 @@ typedef struct mi355x_logits_xform {
   int32_t apply_min_length;
   int32_t n_eos;
   int32_t eos_ids[MI355X_MAX_EOS];
+  const int32_t* history_lens;
+  int32_t min_length;
+  int32_t no_repeat_ngram_size;
 } mi355x_logits_xform;
 
 /* (k, p, temperature) of one row: BatchedSamplingParams, src/smartptrs.h:113-117.  Meaning as in

@@ -19,7 +19,8 @@ def library_path():
 class LogitsXformC(C.Structure):
     _fields_ = [("mask", C.c_void_p), ("history", C.c_void_p), ("history_stride", C.c_int32),
                 ("history_len", C.c_int32), ("repetition_penalty", C.c_float), ("apply_min_length", C.c_int32),
-                ("n_eos", C.c_int32), ("eos_ids", C.c_int32 * MAX_EOS)]
+                ("n_eos", C.c_int32), ("eos_ids", C.c_int32 * MAX_EOS), ("history_lens", C.c_void_p),
+                ("min_length", C.c_int32), ("no_repeat_ngram_size", C.c_int32)]
 
 
 class SampleParams(C.Structure):
@@ -81,12 +82,15 @@ def load_library():
 
 
 class LogitsXform:
-    """Python-side description of the fused logits processing (mask / repetition penalty / min length).
-    Holds references to the tensors so they outlive the asynchronous call."""
+    """Python-side description of the fused logits processing (mask / min length / repetition penalty /
+    no-repeat n-grams).  Holds references to the tensors so they outlive the asynchronous call.
+    shared_history=True lets every row read the one history row given (stride 0), with history_lens
+    telling how much of it each row sees: the verify rows of speculative decoding."""
 
     def __init__(self, mask=None, history=None, history_len=None, repetition_penalty=1.0, eos_ids=(),
-                 apply_min_length=False):
-        self.mask, self.history = mask, history
+                 apply_min_length=False, history_lens=None, min_length=0, no_repeat_ngram_size=0,
+                 shared_history=False):
+        self.mask, self.history, self.history_lens = mask, history, history_lens
         c = self.c = LogitsXformC()
         c.mask = mask.data_ptr() if mask is not None else None
         if mask is not None:
@@ -94,10 +98,15 @@ class LogitsXform:
         if history is not None:
             assert history.dtype == torch.int32 and history.is_cuda and history.is_contiguous() and history.dim() == 2
             c.history = history.data_ptr()
-            c.history_stride = history.shape[1]
+            c.history_stride = 0 if shared_history else history.shape[1]
             c.history_len = history.shape[1] if history_len is None else history_len
+        if history_lens is not None:
+            assert history_lens.dtype == torch.int32 and history_lens.is_cuda and history_lens.is_contiguous()
+            c.history_lens = history_lens.data_ptr()
         c.repetition_penalty = repetition_penalty
         c.apply_min_length = int(apply_min_length)
+        c.min_length = min_length
+        c.no_repeat_ngram_size = no_repeat_ngram_size
         c.n_eos = len(eos_ids)
         for i, e in enumerate(eos_ids):
             c.eos_ids[i] = e

@@ -55,6 +55,7 @@ struct mi355x_search_ctx {
   ms::u64* big{};
   size_t big_stride{};
   uint32_t* fallback_rows{};
+  uint32_t* ban{};  // [max_rows, mask words]: ids banned by the no-repeat-n-gram rule
   mi355x_sample_params* params_dev{};
   void** ptr_table{};      // device copy of pointer tables (kv gather)
   size_t ptr_table_cap{};
@@ -98,7 +99,11 @@ int CheckRows(const mi355x_search_ctx* ctx, int rows, int vocab) {
   return MI355X_OK;
 }
 
-int MakeXform(const mi355x_logits_xform* in, ms::Xform* out) {
+// Validates the caller's logits-processing request and turns it into the kernels' form.  With a
+// no-repeat-n-gram size it also launches the kernel that writes the rows' banned-id bitmaps into
+// the context's workspace.
+int MakeXform(mi355x_search_ctx* ctx, const mi355x_logits_xform* in, int rows, int vocab, hipStream_t stream,
+              ms::Xform* out) {
   std::memset(out, 0, sizeof(*out));
   out->penalty = 1.0f;
   if (!in) return MI355X_OK;
@@ -106,15 +111,25 @@ int MakeXform(const mi355x_logits_xform* in, ms::Xform* out) {
   out->history = in->history;
   out->history_stride = in->history_stride;
   out->history_len = in->history_len;
+  out->history_lens = in->history ? in->history_lens : nullptr;
+  out->min_length = in->min_length;
   out->penalty = in->repetition_penalty;
-  if (in->history && in->history_len > in->history_stride)
+  if (in->history && !in->history_lens && in->history_stride != 0 && in->history_len > in->history_stride)
     return Fail(MI355X_E_INVALID, "history_len (%d) exceeds history_stride (%d)", in->history_len, in->history_stride);
-  if (in->history_len < 0) return Fail(MI355X_E_INVALID, "negative history_len");
-  if (in->apply_min_length) {
+  if (in->history_len < 0 || in->history_stride < 0) return Fail(MI355X_E_INVALID, "negative history_len or history_stride");
+  if (in->history_lens && !in->history) return Fail(MI355X_E_INVALID, "history_lens given without history");
+  if (in->apply_min_length || (in->history_lens && in->min_length > 0)) {
     if (in->n_eos < 0 || in->n_eos > MI355X_MAX_EOS)
       return Fail(MI355X_E_INVALID, "n_eos (%d) out of range [0, %d]", in->n_eos, MI355X_MAX_EOS);
     out->n_eos = in->n_eos;
     for (int i = 0; i < in->n_eos; ++i) out->eos[i] = in->eos_ids[i];
+  }
+  if (in->no_repeat_ngram_size > 0) {
+    if (!in->history) return Fail(MI355X_E_INVALID, "no_repeat_ngram_size needs a history");
+    if (out->history_lens || out->history_len >= in->no_repeat_ngram_size) {
+      HIP_TRY(ms_launch_ngram_ban(out, rows, vocab, in->no_repeat_ngram_size, ctx->ban, stream));
+      out->ban = ctx->ban;
+    }
   }
   return MI355X_OK;
 }
@@ -160,6 +175,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->row_best, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->big, static_cast<size_t>(max_rows) * c->big_stride, false));
   ok(c->Alloc(&c->fallback_rows, 1, true));
+  ok(c->Alloc(&c->ban, static_cast<size_t>(max_rows) * ((max_vocab - 1) / 32 + 1), false));
   ok(c->Alloc(&c->params_dev, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->beam_row_scores, static_cast<size_t>(max_rows) * ms::kBeamMaxCand, false));
   ok(c->Alloc(&c->beam_row_tokens, static_cast<size_t>(max_rows) * ms::kBeamMaxCand, false));
@@ -197,7 +213,7 @@ int mi355x_process_logits(mi355x_search_ctx* ctx, void* stream, float* logits, i
   if (!logits) return Fail(MI355X_E_INVALID, "null logits");
   if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride (%lld) smaller than vocab (%d)", (long long)row_stride, vocab);
   ms::Xform x;
-  if (int r = MakeXform(xf, &x)) return r;
+  if (int r = MakeXform(ctx, xf, rows, vocab, static_cast<hipStream_t>(stream), &x)) return r;
   if (!x.active()) return MI355X_OK;
   HIP_TRY(ms_launch_process_logits(logits, row_stride, rows, vocab, &x, static_cast<hipStream_t>(stream)));
   return MI355X_OK;
@@ -210,7 +226,7 @@ int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int 
   if (dtype != MI355X_F32 && dtype != MI355X_F16) return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
   if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
   ms::ArgmaxArgs a{};
-  if (int r = MakeXform(xf, &a.xf)) return r;
+  if (int r = MakeXform(ctx, xf, rows, vocab, static_cast<hipStream_t>(stream), &a.xf)) return r;
   a.logits = logits;
   a.row_stride = row_stride;
   a.rows = rows;
@@ -234,7 +250,7 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   if (kept_probs && !kept_ids) return Fail(MI355X_E_INVALID, "kept_probs requires kept_ids");
   hipStream_t s = static_cast<hipStream_t>(stream);
   ms::SampleArgs a{};
-  if (int r = MakeXform(xf, &a.xf)) return r;
+  if (int r = MakeXform(ctx, xf, rows, vocab, s, &a.xf)) return r;
   bool any_nucleus = false;
   auto check = [&](const mi355x_sample_params& p) -> int {
     if (!(p.temperature > 0.0f)) return Fail(MI355X_E_INVALID, "temperature must be positive (got %g)", p.temperature);
@@ -302,7 +318,7 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
     row_stride = vocab;
   }
   ms::SampleArgs a{};
-  if (int r = MakeXform(nullptr, &a.xf)) return r;
+  if (int r = MakeXform(ctx, nullptr, rows, vocab, s, &a.xf)) return r;
   a.logits = src;
   a.row_stride = row_stride;
   a.rows = rows;

@@ -65,6 +65,9 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
   const bool has_mask = a.xf.mask != nullptr;
   const bool active = a.xf.active();
   const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
+  const int n_eos = active ? a.xf.eos_count(row) : 0;
+  const uint32_t* ban_row = a.xf.ban_row(row, V);
+  const int hlen = pen ? a.xf.hist_len(row) : 0;
   u64 best = 0;
   for (int base = 0; base < V; base += 1024 * VEC * NB) {
     float v[NB][VEC];
@@ -95,13 +98,13 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
       const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
       int hv[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) hv[r] = (r * 1024 + tid < a.xf.history_len) ? h[r * 1024 + tid] : -1;
+      for (int r = 0; r < 4; ++r) hv[r] = (r * 1024 + tid < hlen) ? h[r * 1024 + tid] : -1;
       for (int i = tid; i < (V + 31) / 32; i += 1024) hist_bits[i] = 0u;
       __syncthreads();
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         if (hv[r] >= 0 && hv[r] < V) atomicOr(&hist_bits[hv[r] >> 5], 1u << (hv[r] & 31));
-      for (int i = 4096 + tid; i < a.xf.history_len; i += 1024) {
+      for (int i = 4096 + tid; i < hlen; i += 1024) {
         const int t = h[i];
         if (t >= 0 && t < V) atomicOr(&hist_bits[t >> 5], 1u << (t & 31));
       }
@@ -116,7 +119,7 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
         const int idx = i0 + c;
         if (idx < V) {
           float x = v[j][c];
-          if (active) x = xform_value(x, a.xf, idx, mw[j], has_mask, (hw >> (idx & 31)) & 1u);
+          if (active) x = xform_value(x, a.xf, idx, mw[j], has_mask, (hw >> (idx & 31)) & 1u, n_eos, ban_row);
           u64 k = make_key64(order_key(x), static_cast<uint32_t>(idx));
           if (idx == 0 && x != x) k = ~0ull;  // NaN at index 0 is sticky
           if (k == 0) k = 1;

@@ -179,8 +179,22 @@ struct Xform {
   float penalty;
   int n_eos;  // 0 unless min-length masking is active
   int eos[MI355X_MAX_EOS];
+  const int32_t* history_lens;  // per-row number of valid history ids, or null (history_len for every row)
+  int min_length;               // with history_lens: only rows shorter than this get the EOS masking
+  const uint32_t* ban;          // per-row bitmap (mask layout) of ids the no-repeat-n-gram rule bans, or null
   __host__ __device__ bool active() const { return mask || use_penalty() || n_eos > 0; }
-  __host__ __device__ bool use_penalty() const { return history && history_len > 0 && penalty != 1.0f; }
+  // true when elements must be tested against the row's history: a penalty to apply or banned ids to
+  // look up (a banned id always occurs in the history; a penalty of 1.0f leaves a value unchanged)
+  __host__ __device__ bool use_penalty() const {
+    return history && (history_lens || history_len > 0) && (penalty != 1.0f || ban);
+  }
+  __device__ int hist_len(int row) const { return history_lens ? history_lens[row] : history_len; }
+  __device__ int eos_count(int row) const {
+    return (history_lens && min_length > 0 && history_lens[row] >= min_length) ? 0 : n_eos;
+  }
+  __device__ const uint32_t* ban_row(int row, int vocab) const {
+    return ban ? ban + static_cast<size_t>(row) * ((vocab - 1) / 32 + 1) : nullptr;
+  }
 };
 
 // Marks, in an LDS bitmap covering vocabulary ids [base, base + kChunk), the ids present in the
@@ -189,20 +203,26 @@ __device__ __forceinline__ void build_history_bitmap(const Xform& xf, int row, i
   for (int i = threadIdx.x; i < kChunk / 32; i += blockDim.x) bits[i] = 0u;
   __syncthreads();
   const int32_t* h = xf.history + static_cast<size_t>(row) * xf.history_stride;
-  for (int i = threadIdx.x; i < xf.history_len; i += blockDim.x) {
+  const int hlen = xf.hist_len(row);
+  for (int i = threadIdx.x; i < hlen; i += blockDim.x) {
     const int rel = h[i] - base;
     if (rel >= 0 && rel < kChunk) atomicOr(&bits[rel >> 5], 1u << (rel & 31));
   }
   __syncthreads();
 }
 
-// The reference's order: mask -> min-length -> repetition penalty.
+// The reference's order: mask -> min-length -> repetition penalty -> no-repeat-n-gram ban
+// (src/standard_decoding_strategy.cpp:24-32, src/sampling_distribution.h:100-110).  n_eos and
+// ban_row are the row's values (Xform::eos_count, Xform::ban_row).
 __device__ __forceinline__ float xform_value(float x, const Xform& xf, int idx, uint32_t mask_word,
-                                             bool has_mask, bool in_history) {
+                                             bool has_mask, bool in_history, int n_eos, const uint32_t* ban_row) {
   if (has_mask && !((mask_word >> (idx & 31)) & 1u)) x = kLowest;
-  for (int e = 0; e < xf.n_eos; ++e)
+  for (int e = 0; e < n_eos; ++e)
     if (xf.eos[e] == idx) x = kLowest;
-  if (in_history) x = x < 0.0f ? x * xf.penalty : x / xf.penalty;
+  if (in_history) {
+    x = x < 0.0f ? x * xf.penalty : x / xf.penalty;
+    if (ban_row && ((ban_row[idx >> 5] >> (idx & 31)) & 1u)) x = kLowest;
+  }
   return x;
 }
 
@@ -274,6 +294,8 @@ __device__ __forceinline__ void xform_chunk(const Xform& xf, int row, int vocab,
   const bool has_mask = xf.mask != nullptr;
   const bool pen = xf.use_penalty();
   const uint32_t* mrow = has_mask ? xf.mask + static_cast<size_t>(row) * ((vocab - 1) / 32 + 1) : nullptr;
+  const int n_eos = xf.eos_count(row);
+  const uint32_t* ban_row = xf.ban_row(row, vocab);
 #pragma unroll
   for (int j = 0; j < L::NV; ++j) {
 #pragma unroll
@@ -283,7 +305,7 @@ __device__ __forceinline__ void xform_chunk(const Xform& xf, int row, int vocab,
         const uint32_t mw = has_mask ? mrow[idx >> 5] : 0u;
         const int rel = idx - chunk * kChunk;
         const bool hit = pen && ((hist_bits[rel >> 5] >> (rel & 31)) & 1u);
-        v[j * L::VEC + c] = xform_value(v[j * L::VEC + c], xf, idx, mw, has_mask, hit);
+        v[j * L::VEC + c] = xform_value(v[j * L::VEC + c], xf, idx, mw, has_mask, hit, n_eos, ban_row);
       }
     }
   }

@@ -125,6 +125,8 @@ hipError_t ms_launch_process_logits(float* logits, int64_t row_stride, int rows,
                                     const ms::Xform* xf, hipStream_t stream);
 hipError_t ms_launch_softmax(float* scores, int64_t row_stride, int rows, int vocab, float temperature,
                              int log_softmax, hipStream_t stream);
+// Writes, for every row, the bitmap of ids the no-repeat-n-gram rule bans (mask layout) into `ban`.
+hipError_t ms_launch_ngram_ban(const ms::Xform* xf, int rows, int vocab, int ngram, uint32_t* ban, hipStream_t stream);
 hipError_t ms_launch_kv_gather(const void* const* present_dev, void* const* past_dev, int n_tensors,
                                const int32_t* beam_indices, int rows, size_t block_bytes, int width,
                                hipStream_t stream);

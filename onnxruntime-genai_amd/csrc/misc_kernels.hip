@@ -41,6 +41,37 @@ __global__ __launch_bounds__(1024) void softmax_kernel(float* scores, int64_t ro
   }
 }
 
+// ---- no-repeat-n-gram bans (src/sampling_distribution.h:64-79, src/search.cpp:432-469) -------------------
+// One workgroup per row.  Every earlier occurrence of the row's last ngram-1 history ids marks the id
+// that followed it.  The row's bitmap is assembled in LDS, one window of kBanWindow ids at a time,
+// and written out whole, so rows without any ban get an all-zero bitmap.
+constexpr int kBanWindow = 1 << 18;
+
+__global__ __launch_bounds__(256) void ngram_ban_kernel(const Xform xf, int vocab, int ngram, uint32_t* ban) {
+  __shared__ uint32_t bits[kBanWindow / 32];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int words = (vocab - 1) / 32 + 1;
+  uint32_t* brow = ban + static_cast<size_t>(row) * words;
+  const int32_t* h = xf.history + static_cast<size_t>(row) * xf.history_stride;
+  const int n = xf.hist_len(row);
+  const int pl = ngram - 1;
+  for (int base = 0; base < vocab; base += kBanWindow) {
+    for (int i = tid; i < kBanWindow / 32; i += 256) bits[i] = 0u;
+    __syncthreads();
+    for (int start = tid; start + ngram <= n; start += 256) {
+      bool match = true;
+      for (int j = 0; j < pl && match; ++j) match = h[start + j] == h[n - pl + j];
+      if (match) {
+        const int tok = h[start + pl];
+        if (tok >= base && tok < vocab && tok - base < kBanWindow) atomicOr(&bits[(tok - base) >> 5], 1u << ((tok - base) & 31));
+      }
+    }
+    __syncthreads();
+    for (int i = tid; i < kBanWindow / 32 && base / 32 + i < words; i += 256) brow[base / 32 + i] = bits[i];
+    __syncthreads();
+  }
+}
+
 // ---- KV-cache beam gather (src/models/kv_cache.cpp:710-740) -----------------------------------------
 // past[t][j] = present[t][beam_indices[j]] for blocks of block_bytes bytes.  grid = (tiles, rows,
 // tensors); every block moves kGatherTile bytes with 128-bit non-temporal loads and stores.
@@ -221,6 +252,12 @@ extern "C" hipError_t ms_launch_softmax(float* scores, int64_t row_stride, int r
     hipLaunchKernelGGL(ms::softmax_kernel<true>, dim3(rows), dim3(1024), 0, stream, scores, row_stride, vocab, temperature);
   else
     hipLaunchKernelGGL(ms::softmax_kernel<false>, dim3(rows), dim3(1024), 0, stream, scores, row_stride, vocab, temperature);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_ngram_ban(const ms::Xform* xf, int rows, int vocab, int ngram, uint32_t* ban,
+                                          hipStream_t stream) {
+  hipLaunchKernelGGL(ms::ngram_ban_kernel, dim3(rows), dim3(256), 0, stream, *xf, vocab, ngram, ban);
   return hipGetLastError();
 }
 

@@ -44,10 +44,12 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
   const int n2 = next_pow2(V);
   const bool has_mask = a.xf.mask != nullptr;
   const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
+  const int n_eos = a.xf.eos_count(row);
+  const uint32_t* ban_row = a.xf.ban_row(row, V);
   for (int i = threadIdx.x; i < n2; i += blockDim.x) {
     u64 k = 0;
     if (i < V) {
-      const float x = xform_value(lrow[i], a.xf, i, has_mask ? mrow[i >> 5] : 0u, has_mask, false);
+      const float x = xform_value(lrow[i], a.xf, i, has_mask ? mrow[i >> 5] : 0u, has_mask, false, n_eos, ban_row);
       k = make_key64(order_key(x), static_cast<uint32_t>(i));
     }
     scratch[i] = k;
@@ -55,13 +57,14 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
   __syncthreads();
   if (a.xf.use_penalty()) {
     const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
-    for (int j = threadIdx.x; j < a.xf.history_len; j += blockDim.x) {
+    const int hlen = a.xf.hist_len(row);
+    for (int j = threadIdx.x; j < hlen; j += blockDim.x) {
       const int tok = h[j];
       if (tok < 0 || tok >= V) continue;
       bool dup = false;
       for (int jj = 0; jj < j && !dup; ++jj) dup = (h[jj] == tok);
       if (dup) continue;
-      const float x = xform_value(lrow[tok], a.xf, tok, has_mask ? mrow[tok >> 5] : 0u, has_mask, true);
+      const float x = xform_value(lrow[tok], a.xf, tok, has_mask ? mrow[tok >> 5] : 0u, has_mask, true, n_eos, ban_row);
       scratch[tok] = make_key64(order_key(x), static_cast<uint32_t>(tok));
     }
     __syncthreads();
@@ -292,13 +295,16 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     __syncthreads();
     if (pen) {
       const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
-      for (int i = tid; i < a.xf.history_len; i += kSBlock) {
+      const int hlen = a.xf.hist_len(row);
+      for (int i = tid; i < hlen; i += kSBlock) {
         const int rel = h[i] - chunk * kSChunk;
         if (rel >= 0 && rel < kSChunk) atomicOr(&sm.hist_bits[rel >> 5], 1u << (rel & 31));
       }
       __syncthreads();
     }
     const float penalty = a.xf.penalty;
+    const int n_eos = a.xf.eos_count(row);
+    const uint32_t* ban_row = a.xf.ban_row(row, V);
 #pragma unroll
     for (int j = 0; j < kSVec; ++j) {
       const int rel0 = (j * kSBlock + tid) * 4;
@@ -311,9 +317,12 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
         if (idx < V) {
           // the reference's order: mask -> min-length -> repetition penalty
           if (!((mnib >> c) & 1u)) x = kLowest;
-          for (int e = 0; e < a.xf.n_eos; ++e)
+          for (int e = 0; e < n_eos; ++e)
             if (a.xf.eos[e] == idx) x = kLowest;
-          if ((hnib >> c) & 1u) x = x < 0.0f ? x * penalty : x / penalty;
+          if ((hnib >> c) & 1u) {
+            x = x < 0.0f ? x * penalty : x / penalty;
+            if (ban_row && ((ban_row[idx >> 5] >> (idx & 31)) & 1u)) x = kLowest;  // no-repeat-n-gram ban
+          }
         }
         v[j * 4 + c] = x;
       }

@@ -336,8 +336,7 @@ void GreedySearch_Hip::ResetDone() {
 
 void GreedySearch_Hip::SetLogits(DeviceSpan<float> logits) {
   next_token_scores_ = logits;
-  pending_min_length_ = false;
-  pending_penalty_ = 1.0f;
+  ClearPending();
 }
 
 DeviceSpan<float> GreedySearch_Hip::GetLogits() const {
@@ -345,25 +344,45 @@ DeviceSpan<float> GreedySearch_Hip::GetLogits() const {
   return next_token_scores_;
 }
 
+// The three processors are deferred and fused into the next selection in the order the kernels apply
+// them (min-length, repetition penalty, n-gram ban: the order RunStandardDecodingStep calls them in,
+// src/standard_decoding_strategy.cpp:29-32).  A call that arrives out of that order first applies
+// what is pending.
 void GreedySearch_Hip::ApplyMinLength(int min_length) {
   if (sequences_.GetSequenceLength() >= min_length) return;
-  pending_min_length_ = true;  // fused into the next selection (or applied by GetLogits)
+  if (pending_penalty_ != 1.0f || pending_ngram_ > 0) Materialize();
+  pending_min_length_ = true;
 }
 
 void GreedySearch_Hip::ApplyRepetitionPenalty(float penalty) {
   if (penalty == 1.0f) return;
-  if (pending_penalty_ != 1.0f) Materialize();  // two penalties in one step: apply the first now
+  if (pending_penalty_ != 1.0f || pending_ngram_ > 0) Materialize();
   pending_penalty_ = penalty;
 }
 
+// Search_Cpu::ApplyNoRepeatNgram (src/search.cpp:432-469) on the device (the reference's CUDA search
+// rejects the option, src/search.h:125-130).
+void GreedySearch_Hip::ApplyNoRepeatNgram(int ngram_size) {
+  if (ngram_size <= 0 || sequences_.GetSequenceLength() < ngram_size) return;
+  if (pending_ngram_ > 0) Materialize();
+  pending_ngram_ = ngram_size;
+}
+
+void GreedySearch_Hip::ClearPending() const {
+  pending_min_length_ = false;
+  pending_penalty_ = 1.0f;
+  pending_ngram_ = 0;
+}
+
 mi355x_logits_xform* GreedySearch_Hip::PendingXform() {
-  if (!pending_min_length_ && pending_penalty_ == 1.0f) return nullptr;
+  if (!pending_min_length_ && pending_penalty_ == 1.0f && pending_ngram_ == 0) return nullptr;
   xf_ = mi355x_logits_xform{};
   xf_.repetition_penalty = pending_penalty_;
-  if (pending_penalty_ != 1.0f && sequences_.GetSequenceLength() > 0) {
+  if ((pending_penalty_ != 1.0f || pending_ngram_ > 0) && sequences_.GetSequenceLength() > 0) {
     xf_.history = sequences_.GetSequences().Span().data();
     xf_.history_stride = sequences_.max_length_;
     xf_.history_len = sequences_.GetSequenceLength();
+    xf_.no_repeat_ngram_size = pending_ngram_;
   }
   if (pending_min_length_) {
     xf_.apply_min_length = 1;
@@ -379,8 +398,7 @@ void GreedySearch_Hip::Materialize() const {
     AbiCheck(mi355x_process_logits(ctx_, g_stream, self->next_token_scores_.Span().data(), vocab,
                                    params_->search.batch_size, vocab, xf));
   }
-  pending_min_length_ = false;
-  pending_penalty_ = 1.0f;
+  ClearPending();
 }
 
 bool GreedySearch_Hip::PadIfAlreadyEOS(size_t batch_id) {
@@ -412,8 +430,7 @@ void GreedySearch_Hip::SelectTop() {
   const int batch = params_->search.batch_size, vocab = params_->config.model.vocab_size;
   AbiCheck(mi355x_argmax(ctx_, g_stream, next_token_scores_.Span().data(), MI355X_F32, vocab, batch, vocab,
                          PendingXform(), next_tokens_.Span().data()));
-  pending_min_length_ = false;
-  pending_penalty_ = 1.0f;
+  ClearPending();
   const std::vector<int32_t> picked = [&] {
     auto h = next_tokens_.CopyDeviceToCpu();
     return std::vector<int32_t>(h.begin(), h.end());
@@ -466,8 +483,7 @@ void GreedySearch_Hip::Sample(int k, float p, float temperature, std::mt19937& r
                          mi355x_sample_params{k, p, temperature}, nullptr, uniforms_.Span().data(),
                          next_tokens_.Span().data(), kept_count_.Span().data(), kept_ids_.Span().data(),
                          kept_probs_.Span().data(), kept_capacity_));
-  pending_min_length_ = false;
-  pending_penalty_ = 1.0f;
+  ClearPending();
   const std::vector<int32_t> counts = [&] {
     auto h = kept_count_.CopyDeviceToCpu();
     return std::vector<int32_t>(h.begin(), h.end());
@@ -598,6 +614,19 @@ void BeamSearch_Hip::ApplyRepetitionPenalty(float penalty) {
   xf.history_stride = params_->search.max_length;
   xf.history_len = len;
   xf.repetition_penalty = penalty;
+  const int vocab = params_->config.model.vocab_size;
+  AbiCheck(mi355x_process_logits(ctx_, g_stream, next_token_scores_.Span().data(), vocab, params_->BatchBeamSize(), vocab, &xf));
+}
+
+void BeamSearch_Hip::ApplyNoRepeatNgram(int ngram_size) {
+  if (ngram_size <= 0 || length_ < ngram_size) return;
+  mi355x_logits_xform xf{};
+  int len = 0;
+  xf.history = mi355x_beam_scorer_sequences(scorer_, &len);
+  xf.history_stride = params_->search.max_length;
+  xf.history_len = len;
+  xf.repetition_penalty = 1.0f;
+  xf.no_repeat_ngram_size = ngram_size;
   const int vocab = params_->config.model.vocab_size;
   AbiCheck(mi355x_process_logits(ctx_, g_stream, next_token_scores_.Span().data(), vocab, params_->BatchBeamSize(), vocab, &xf));
 }

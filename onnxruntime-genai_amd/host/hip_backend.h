@@ -47,6 +47,7 @@ struct GreedySearch_Hip : Search {
   void SampleTopKTopP(int k, float p, float temperature, std::mt19937& rng) override { Sample(k, p, temperature, rng); }
   void ApplyMinLength(int min_length) override;
   void ApplyRepetitionPenalty(float penalty) override;
+  void ApplyNoRepeatNgram(int ngram_size) override;
   void AppendTokens(DeviceSpan<int32_t>& next_tokens) override;
   void RewindTo(size_t index) override;
 
@@ -57,7 +58,8 @@ struct GreedySearch_Hip : Search {
  private:
   void Sample(int k, float p, float temperature, std::mt19937& rng);
   mi355x_logits_xform* PendingXform();
-  void Materialize() const;  // applies deferred min-length / repetition penalty to the logits in place
+  void Materialize() const;  // applies the deferred logits processing to the logits in place
+  void ClearPending() const;
   bool PadIfAlreadyEOS(size_t batch_id);
   void SetNextToken(size_t batch_id, int32_t token);
   void AppendNextTokensToSequences();
@@ -78,6 +80,7 @@ struct GreedySearch_Hip : Search {
   // deferred logits processing
   mutable bool pending_min_length_{};
   mutable float pending_penalty_{1.0f};
+  mutable int pending_ngram_{};
   mutable mi355x_logits_xform xf_{};
   // transaction checkpoint
   std::vector<int32_t> tx_next_tokens_, tx_sequence_lengths_;
@@ -102,6 +105,7 @@ struct BeamSearch_Hip : Search {
   void SelectTop() override;
   void ApplyMinLength(int min_length) override;
   void ApplyRepetitionPenalty(float penalty) override;
+  void ApplyNoRepeatNgram(int ngram_size) override;
   void AppendTokens(DeviceSpan<int32_t>& next_tokens) override;
 
  private:

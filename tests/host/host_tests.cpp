@@ -22,6 +22,7 @@ extern "C" {
 int32_t orc_argmax(const float* v, int n);
 void orc_apply_min_length(float* logits, int vocab, int current_length, int min_length, const int32_t* eos, int n_eos);
 void orc_apply_repetition_penalty(float* logits, int vocab, const int32_t* prefix, int n, float penalty);
+void orc_apply_no_repeat_ngram(float* logits, int vocab, const int32_t* prefix, int n, int ngram);
 int orc_sampled_categorical(const float* scores, int vocab, int top_k, float top_p, float temperature, int32_t* scratch,
                             int32_t* indices, float* out_probs);
 void orc_beam_select_top(float* scores, int batch, int beams, int vocab, const float* beam_scores, float* out_scores,
@@ -116,12 +117,13 @@ struct GreedyModel {
       if (--not_done == 0) done = true;
     }
   }
-  void Process(std::vector<float>& logits, int min_length, float penalty) {
+  void Process(std::vector<float>& logits, int min_length, float penalty, int ngram = 0) {
     for (int b = 0; b < batch; ++b) {
       float* row = logits.data() + static_cast<size_t>(b) * vocab;
+      const int32_t* seq = sequences.data() + static_cast<size_t>(b) * config.search.max_length;
       orc_apply_min_length(row, vocab, length, min_length, eos.data(), static_cast<int>(eos.size()));
-      if (penalty != 1.0f)
-        orc_apply_repetition_penalty(row, vocab, sequences.data() + static_cast<size_t>(b) * config.search.max_length, length, penalty);
+      if (penalty != 1.0f) orc_apply_repetition_penalty(row, vocab, seq, length, penalty);
+      orc_apply_no_repeat_ngram(row, vocab, seq, length, ngram);
     }
   }
   void SelectTop(const std::vector<float>& logits) {
@@ -533,7 +535,7 @@ void BatchedSamplerLargeVocabulary() {
 }
 
 // A whole generation against the host model of GreedySearch_Cpu: prompt, min-length, repetition
-// penalty, the four selection methods in rotation, EOS padding, rewind, max_length.  Tokens, done
+// penalty, no-repeat n-grams, the four selection methods in rotation, EOS padding, rewind, max_length.  Tokens, done
 // flag, sequences and the std::mt19937 state must agree after every step.
 void GreedyGenerationMatchesCpuSearch() {
   constexpr int batch = 6, vocab = 2003, max_length = 24, min_length = 6;
@@ -542,6 +544,7 @@ void GreedyGenerationMatchesCpuSearch() {
   std::mt19937 gen(99), rng(4321), model_rng(4321);
   std::vector<int32_t> prompt(batch * 3);
   for (auto& t : prompt) t = static_cast<int32_t>(gen() % vocab);
+  for (int b = 0; b < batch; b += 2) prompt[b * 3 + 2] = prompt[b * 3];  // "x y x": the bigram rule bans y next
   auto prompt_dev = ToDevice(prompt);
   f.search->AppendTokens(prompt_dev);
   model.AppendPrompt(prompt);
@@ -549,13 +552,16 @@ void GreedyGenerationMatchesCpuSearch() {
     auto logits = RandomLogits(gen, static_cast<size_t>(batch) * vocab, 3.0f);
     for (int b = 0; b < batch; ++b) {
       logits[static_cast<size_t>(b) * vocab + prompt[b * 3]] += 6.0f;       // make the penalty matter
+      logits[static_cast<size_t>(b) * vocab + prompt[b * 3 + 1]] += 30.0f;  // the banned id would win
       if ((step + b) % 5 == 4) logits[static_cast<size_t>(b) * vocab + 17] = 40.0f;  // drive rows to EOS
     }
     const float penalty = step % 2 ? 1.3f : 1.0f;
+    const int ngram = step % 3 == 2 ? 0 : 2;
     f.SetLogits(logits);
     f.search->ApplyMinLength(min_length);
     f.search->ApplyRepetitionPenalty(penalty);
-    model.Process(logits, min_length, penalty);
+    f.search->ApplyNoRepeatNgram(ngram);
+    model.Process(logits, min_length, penalty, ngram);
     if (step == 3) {  // GetLogits must show the processed values
       const auto seen = ToHost(f.search->GetLogits());
       EXPECT(seen == logits);
@@ -592,7 +598,6 @@ void GreedyGenerationMatchesCpuSearch() {
   one.search->CommitToken(3);
   EXPECT(one.search->IsDone());
   EXPECT_EQ(one.search->GetSequenceLength(), 1);
-  EXPECT(Throws<std::runtime_error>([&] { one.search->ApplyNoRepeatNgram(2); }));
 }
 
 // Beam search against orc_beam_select_top + the oracle's BeamSearchScorer, step by step and on the
@@ -631,14 +636,18 @@ void BeamSearchMatchesCpuSearch() {
     auto logits = RandomLogits(gen, static_cast<size_t>(bb) * vocab, 2.0f);
     for (int i = 0; i < bb; ++i)
       if (gen() % 3 == 0) logits[static_cast<size_t>(i) * vocab + eos] = 7.5f;  // EOS candidates turn up
+    for (int i = 0; i < bb; ++i)  // a token of the row's own history would win if it were not banned
+      logits[static_cast<size_t>(i) * vocab + seq[static_cast<size_t>(i) * max_length + length - 1]] += 9.0f;
     auto dev = ToDevice(logits);
     search->SetLogits(dev);
     search->ApplyMinLength(4);
     search->ApplyRepetitionPenalty(1.1f);
+    search->ApplyNoRepeatNgram(1);
     for (int i = 0; i < bb; ++i) {
       float* row = logits.data() + static_cast<size_t>(i) * vocab;
       orc_apply_min_length(row, vocab, length, 4, &eos, 1);
       orc_apply_repetition_penalty(row, vocab, seq.data() + static_cast<size_t>(i) * max_length, length, 1.1f);
+      orc_apply_no_repeat_ngram(row, vocab, seq.data() + static_cast<size_t>(i) * max_length, length, 1);
     }
     search->SelectTop();
     orc_beam_select_top(logits.data(), batch, beams, vocab, orc_beam_scorer_next_scores(scorer), cs.data(), ct.data(), ci.data());

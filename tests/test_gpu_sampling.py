@@ -386,3 +386,83 @@ def test_argument_errors(ctx):
     big = torch.zeros((257, 10), device="cuda")
     with pytest.raises(RuntimeError, match="capacity"):
         ctx.argmax(big)
+
+
+@pytest.mark.parametrize("vocab,ngram,hist_len", [(1000, 2, 60), (40000, 3, 300), (70001, 1, 17), (300, 4, 2), (5000, 2, 1500)])
+def test_no_repeat_ngram_ban(ctx, orc, vocab, ngram, hist_len):
+    """ApplyNoRepeatNgramToLogits after mask, min-length and penalty (LogitsPenaltyProcessor::Apply order):
+    in-place processing, greedy argmax and sampling all see the banned ids as lowest()."""
+    say("no-repeat ngram", vocab, ngram, hist_len)
+    rng = np.random.default_rng(vocab + ngram)
+    rows = 4
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    hist = rng.integers(0, 6, (rows, hist_len)).astype(np.int32)  # six distinct ids: every n-gram repeats
+    hist[1, :] = rng.integers(0, vocab, hist_len)  # a row whose n-grams hardly ever repeat
+    x[:, :6] += 8.0  # the banned ids would otherwise win
+    mask = make_mask(rng, rows, vocab, 0.9)
+    eos = [3, vocab - 1]
+    for pen in (1.0, 1.3):
+        xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                               repetition_penalty=pen, eos_ids=eos, apply_min_length=True, no_repeat_ngram_size=ngram)
+        want = orc.apply_mask(x, mask)
+        for r in range(rows):
+            w = orc.apply_min_length(want[r], 0, 1, eos)
+            w = orc.apply_repetition_penalty(w, hist[r], pen)
+            want[r] = orc.apply_no_repeat_ngram(w, hist[r], ngram)
+        got = ctx.process_logits(torch.from_numpy(x.copy()).cuda(), xf).cpu().numpy()
+        assert np.array_equal(bits(got), bits(want))
+        if hist_len >= ngram:
+            assert (want[0] != orc.apply_repetition_penalty(orc.apply_min_length(orc.apply_mask(x, mask)[0], 0, 1, eos),
+                                                             hist[0], pen)).any()  # something was banned
+        tok = ctx.argmax(torch.from_numpy(x).cuda(), xf=xf).cpu().numpy()
+        assert np.array_equal(tok, orc.argmax_batch(want))
+        u = rng.random(rows)
+        for k, p in ((40, 0.9), (0, 0.8)):
+            tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=k, p=p, temperature=0.9,
+                                         xf=xf, kept_capacity=64)
+            for r in range(rows):
+                idx, probs = orc.sampled_categorical(want[r], k, p, 0.9)
+                n = min(len(idx), 64)
+                assert kc[r].item() == len(idx)
+                assert np.array_equal(ki[r, :n].cpu().numpy(), idx[:n])
+                assert np.array_equal(bits(kp[r, :n].cpu().numpy()), bits(probs[:n]))
+                assert tok[r].item() == idx[orc.discrete_draw(probs, u[r])]
+
+
+@pytest.mark.parametrize("vocab,K,seed_len,greedy", [(32064, 8, 40, False), (32064, 8, 40, True), (5000, 3, 2, False),
+                                                     (140000, 5, 700, False)])
+def test_target_selection_of_verify_rows(ctx, orc, vocab, K, seed_len, greedy):
+    """ComputeTargetTokenSelection for the K+1 verify rows of one sequence (src/speculative_sampling.h:59-79,
+    src/speculative_decoding_strategy.cpp:632-656): row i is processed with current_length = seed + i and
+    the prefix seed tokens + the first i proposal tokens -- one shared history buffer, per-row lengths --
+    then reduced to the greedy token or the kept (ids, probabilities)."""
+    say("target selection", vocab, K, seed_len, greedy)
+    rng = np.random.default_rng(vocab + K + seed_len)
+    rows = K + 1
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    seq = rng.integers(0, 8, seed_len + K).astype(np.int32)  # few distinct ids: n-grams repeat
+    x[:, :8] += 6.0
+    eos = [5, 7]
+    min_len = seed_len + 3  # the first rows are still too short for EOS
+    lens = (seed_len + np.arange(rows)).astype(np.int32)
+    xf = pkg().LogitsXform(history=torch.from_numpy(seq[None, :]).cuda(), shared_history=True,
+                           history_lens=torch.from_numpy(lens).cuda(), repetition_penalty=1.2, eos_ids=eos,
+                           min_length=min_len, no_repeat_ngram_size=2)
+    k, p, t = 50, 0.9, 0.8
+    u = rng.random(rows)
+    if greedy:
+        tok = ctx.argmax(torch.from_numpy(x).cuda(), xf=xf).cpu().numpy()
+    else:
+        tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=k, p=p, temperature=t,
+                                     xf=xf, kept_capacity=64)
+        tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    for i in range(rows):
+        g, idx, probs = orc.target_selection(x[i], int(lens[i]), seq[:lens[i]], greedy, k, p, t, rep_pen=1.2,
+                                             min_len=min_len, ngram=2, eos=eos)
+        if greedy:
+            assert tok[i] == g, i
+        else:
+            assert kc[i] == len(idx), i
+            assert np.array_equal(ki[i, :len(idx)], idx), i
+            assert np.array_equal(bits(kp[i, :len(idx)]), bits(probs)), i
+            assert tok[i] == idx[orc.discrete_draw(probs, u[i])], i
