@@ -203,6 +203,37 @@ int mi355x_spec_verify(mi355x_search_ctx* ctx, void* stream, const float* p_targ
                        const double* sample_u, int batch, int K, int vocab, int32_t* accepted_len,
                        int32_t* final_token);
 
+/* Speculative-decoding verification on SPARSE selections, the form the reference's strategies use:
+ * the kept sets mi355x_sample returns (kept_count / kept_ids / kept_probs) for the K+1 verify rows of
+ * each sequence are the TargetTokenSelection rows of SpeculativeDecodingStrategy::RunRound.
+ *   target_count [batch, K+1], target_ids / target_probs [batch, K+1, target_capacity]  device; row i
+ *                judges proposal token i, row K supplies the bonus token.
+ *   draft_count [batch, K], draft_ids / draft_probs [batch, K, draft_capacity]  device; the proposal's
+ *                own distributions (mode 0 only, else NULL).
+ *   proposal     device [batch, K] proposed token ids.
+ *   mode 0       stochastic accept loop (src/speculative_decoding_strategy.cpp:718-762) with
+ *                GetSparseTokenProbability, ComputeAcceptProb, SampleCorrectionToken and
+ *                SampleSparseToken (src/speculative_sampling.h:22-57,140-146).  accept_u: device
+ *                [batch, K] uniform_real_distribution<float> draws in the order the loop takes them;
+ *                sample_u: device [batch, K+1] doubles, entry e = the generate_canonical<double,53>
+ *                value the engine would yield after e accept draws (the loop's single categorical draw
+ *                follows one accept draw per evaluated position).
+ *   mode 1       VerifyDeterministicProposal (src/speculative_sampling.h:96-127): sample_u [batch, K+1]
+ *                holds the categorical draws in the order rows with at least two entries consume them;
+ *                accept_u unused.
+ *   mode 2       greedy targets: entry 0 of every target row is its greedy token; no draws.
+ *   accepted_len, final_token, engine_draws  device [batch] outputs; engine_draws = 32-bit engine outputs
+ *                the reference would have consumed (a categorical draw over fewer than two entries takes
+ *                none), so the caller can advance its std::mt19937 by that many.
+ * A sequence with a row whose count exceeds its capacity reports accepted_len = final_token = -1.
+ * 1 <= K <= 64. */
+int mi355x_spec_verify_sparse(mi355x_search_ctx* ctx, void* stream, const int32_t* target_count,
+                              const int32_t* target_ids, const float* target_probs, int target_capacity,
+                              const int32_t* draft_count, const int32_t* draft_ids,
+                              const float* draft_probs, int draft_capacity, const int32_t* proposal,
+                              const float* accept_u, const double* sample_u, int batch, int K, int mode,
+                              int32_t* accepted_len, int32_t* final_token, int32_t* engine_draws);
+
 /* Element-wise type conversion on the device: DeviceInterface::Cast (src/smartptrs.h:208-210; CPU
  * src/cpu/interface.cpp:74-106).  Supported pairs, with the CPU path's arithmetic: F16->F32
  * (FastFloat16ToFloat32), BF16->F32 (BFloat16ToFloat32), F32->F16 (FastFloat32ToFloat16), F32->BF16

@@ -63,6 +63,7 @@ def load_library():
                                           C.POINTER(C.c_float)],
         "mi355x_kv_gather": [vp, vp, C.POINTER(vp), C.POINTER(vp), i32, vp, i32, C.c_size_t],
         "mi355x_spec_verify": [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, vp],
+        "mi355x_spec_verify_sparse": [vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, vp, vp, vp],
         "mi355x_cast": [vp, vp, vp, i32, vp, i32, C.c_size_t],
         "mi355x_logits_handoff": [vp, vp, vp, i32, i32, i32, i32, C.POINTER(C.c_int32), vp, i64],
     }.items():
@@ -267,6 +268,26 @@ def _spec_verify(self, p_target, p_draft, draft_tokens, accept_u, sample_u):
     return acc, tok
 
 
+def _spec_verify_sparse(self, target, draft, proposal, accept_u, sample_u, mode=0):
+    """target = (count [b, K+1], ids [b, K+1, cap], probs [b, K+1, cap]) as mi355x_sample returns them;
+    draft likewise with K rows (None unless mode 0).  Returns (accepted_len, final_token, engine_draws)."""
+    tc, ti, tp = target
+    b, k = proposal.shape
+    assert tuple(tc.shape) == (b, k + 1) and tuple(ti.shape[:2]) == (b, k + 1)
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    for t in (tc, ti, tp, proposal, accept_u, sample_u) + (tuple(draft) if draft is not None else ()):
+        assert t is None or (t.is_cuda and t.is_contiguous())
+    dc, di, dp = draft if draft is not None else (None, None, None)
+    acc = torch.empty(b, dtype=torch.int32, device=proposal.device)
+    tok = torch.empty(b, dtype=torch.int32, device=proposal.device)
+    used = torch.empty(b, dtype=torch.int32, device=proposal.device)
+    self._check(self.L.mi355x_spec_verify_sparse(self.h, _stream(), ptr(tc), ptr(ti), ptr(tp), ti.shape[2], ptr(dc), ptr(di),
+                                                 ptr(dp), di.shape[2] if di is not None else 0, ptr(proposal),
+                                                 ptr(accept_u), ptr(sample_u), b, k, mode, acc.data_ptr(), tok.data_ptr(),
+                                                 used.data_ptr()))
+    return acc, tok, used
+
+
 _DTYPE_CODES = {torch.float32: 1, torch.int32: 6, torch.int64: 7, torch.float16: 10, torch.bfloat16: 16}
 
 
@@ -299,6 +320,7 @@ SearchContext.logits_handoff = _logits_handoff
 SearchContext.topk_scores = _topk_scores
 SearchContext.softmax = _softmax
 SearchContext.beam_select = _beam_select
+SearchContext.spec_verify_sparse = _spec_verify_sparse
 SearchContext.kv_gather = _kv_gather
 SearchContext.spec_verify = _spec_verify
 

@@ -418,6 +418,46 @@ int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits,
   return MI355X_OK;
 }
 
+int mi355x_spec_verify_sparse(mi355x_search_ctx* ctx, void* stream, const int32_t* target_count,
+                              const int32_t* target_ids, const float* target_probs, int target_capacity,
+                              const int32_t* draft_count, const int32_t* draft_ids, const float* draft_probs,
+                              int draft_capacity, const int32_t* proposal, const float* accept_u,
+                              const double* sample_u, int batch, int K, int mode, int32_t* accepted_len,
+                              int32_t* final_token, int32_t* engine_draws) {
+  if (!ctx || !target_count || !target_ids || !proposal || !accepted_len || !final_token || !engine_draws)
+    return Fail(MI355X_E_INVALID, "null argument");
+  if (mode < 0 || mode > 2) return Fail(MI355X_E_INVALID, "mode (%d) must be 0, 1 or 2", mode);
+  if (batch <= 0 || K < 1 || K > 64) return Fail(MI355X_E_INVALID, "batch (%d) must be positive and K (%d) in [1, 64]", batch, K);
+  if (target_capacity <= 0) return Fail(MI355X_E_INVALID, "target_capacity must be positive");
+  if (mode != 2 && (!target_probs || !sample_u)) return Fail(MI355X_E_INVALID, "null target_probs or sample_u");
+  if (mode == 0 && (!draft_count || !draft_ids || !draft_probs || !accept_u || draft_capacity <= 0))
+    return Fail(MI355X_E_INVALID, "mode 0 needs the draft distributions and accept_u");
+  if (batch > ctx->max_rows) return Fail(MI355X_E_CAPACITY, "batch=%d exceeds the context's capacity (%d)", batch, ctx->max_rows);
+  if (static_cast<size_t>(target_capacity) > 2 * ctx->big_stride)
+    return Fail(MI355X_E_CAPACITY, "target_capacity=%d exceeds the context's workspace (%zu)", target_capacity, 2 * ctx->big_stride);
+  ms::SpecSparseArgs a{};
+  a.t_count = target_count;
+  a.t_ids = target_ids;
+  a.t_probs = target_probs;
+  a.t_cap = target_capacity;
+  a.d_count = draft_count;
+  a.d_ids = draft_ids;
+  a.d_probs = draft_probs;
+  a.d_cap = draft_capacity;
+  a.proposal = proposal;
+  a.accept_u = accept_u;
+  a.sample_u = sample_u;
+  a.K = K;
+  a.mode = mode;
+  a.residual = reinterpret_cast<float*>(ctx->big);
+  a.residual_stride = 2 * ctx->big_stride;
+  a.accepted_len = accepted_len;
+  a.final_token = final_token;
+  a.engine_draws = engine_draws;
+  HIP_TRY(ms_launch_spec_verify_sparse(&a, batch, static_cast<hipStream_t>(stream)));
+  return MI355X_OK;
+}
+
 int mi355x_cast(mi355x_search_ctx* ctx, void* stream, const void* in, int in_dtype, void* out, int out_dtype,
                 size_t count) {
   if (!ctx || !in || !out) return Fail(MI355X_E_INVALID, "null argument");

@@ -84,6 +84,27 @@ struct SeqSumArgs {
   float* out_sum;     // [rows]
 };
 
+struct SpecSparseArgs {
+  const int32_t* t_count;  // [batch, K+1]
+  const int32_t* t_ids;    // [batch, K+1, t_cap]
+  const float* t_probs;
+  int t_cap;
+  const int32_t* d_count;  // [batch, K]
+  const int32_t* d_ids;    // [batch, K, d_cap]
+  const float* d_probs;
+  int d_cap;
+  const int32_t* proposal;  // [batch, K]
+  const float* accept_u;    // [batch, K]
+  const double* sample_u;   // [batch, K+1]
+  int K;
+  int mode;
+  float* residual;  // workspace [batch, residual_stride]
+  size_t residual_stride;
+  int32_t* accepted_len;
+  int32_t* final_token;
+  int32_t* engine_draws;
+};
+
 struct BeamArgs {
   const void* logits;
   int64_t row_stride;
@@ -133,6 +154,7 @@ hipError_t ms_launch_kv_gather(const void* const* present_dev, void* const* past
 hipError_t ms_launch_spec_verify(const float* p_target, const float* p_draft, const int32_t* draft_tokens,
                                  const float* accept_u, const double* sample_u, int batch, int K, int vocab,
                                  int32_t* accepted_len, int32_t* final_token, hipStream_t stream);
+hipError_t ms_launch_spec_verify_sparse(const ms::SpecSparseArgs* a, int batch, hipStream_t stream);
 hipError_t ms_launch_widen_f16(const void* in, int64_t in_stride, float* out, int64_t out_stride, int rows,
                                int vocab, hipStream_t stream);
 hipError_t ms_launch_cast(const void* in, void* out, size_t count, int kind, hipStream_t stream);

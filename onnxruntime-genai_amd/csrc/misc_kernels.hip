@@ -181,6 +181,152 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
   }
 }
 
+// ---- speculative verification on sparse selections ----------------------------------------------------
+// One 256-thread block per sequence.  Target rows 0..K (row i judges proposal token i, row K is the
+// bonus row) and draft rows 0..K-1 are kept sets: count, ids, probabilities, padded to a capacity.
+//   mode 0  the accept loop of SpeculativeDecodingStrategy::RunRound
+//           (src/speculative_decoding_strategy.cpp:718-762): GetSparseTokenProbability,
+//           ComputeAcceptProb, then SampleCorrectionToken at the first reject (residual over the target
+//           row's ids; the target row itself when the residual sums to zero) or SampleSparseToken on
+//           the bonus row (src/speculative_sampling.h:22-57,140-146).  sample_u[e] is the categorical
+//           draw available after e accept draws.
+//   mode 1  VerifyDeterministicProposal (src/speculative_sampling.h:96-127): sample every target row in
+//           turn until the sample differs from the proposal; sample_u holds the draws in the order rows
+//           with at least two entries consume them.
+//   mode 2  greedy targets: entry 0 of every target row is the row's greedy token.
+// A row whose count exceeds its capacity was truncated by the producer: the sequence reports -1.
+constexpr int kSpecMaxK = 64;
+
+__device__ __forceinline__ float wave_sparse_prob(const int32_t* ids, const float* probs, int n, int32_t token) {
+  const int lane = lane_id();
+  for (int j0 = 0; j0 < n; j0 += 64) {
+    const int j = j0 + lane;
+    const int f = first_lane(__ballot(j < n && ids[j] == token));
+    if (f >= 0) return probs[j0 + f];
+  }
+  return 0.0f;
+}
+
+__global__ __launch_bounds__(256) void spec_verify_sparse_kernel(const SpecSparseArgs a) {
+  __shared__ SeqShared sh;
+  __shared__ float s_pt[kSpecMaxK], s_pd[kSpecMaxK];
+  __shared__ int s_n, s_bad;
+  const int b = blockIdx.x, tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+  const int K = a.K;
+  const int32_t* tc = a.t_count + static_cast<size_t>(b) * (K + 1);
+  const int32_t* prop = a.proposal + static_cast<size_t>(b) * K;
+  auto t_ids = [&](int r) { return a.t_ids + (static_cast<size_t>(b) * (K + 1) + r) * a.t_cap; };
+  auto t_probs = [&](int r) { return a.t_probs + (static_cast<size_t>(b) * (K + 1) + r) * a.t_cap; };
+  if (tid == 0) s_bad = 0;
+  __syncthreads();
+  for (int r = tid; r <= K; r += 256) {
+    bool bad = tc[r] > a.t_cap || tc[r] < (a.mode == 2 ? 0 : 1);
+    if (a.mode == 0 && r < K) bad = bad || a.d_count[static_cast<size_t>(b) * K + r] > a.d_cap;
+    if (bad) s_bad = 1;
+  }
+  __syncthreads();
+  if (s_bad) {
+    if (tid == 0) {
+      a.accepted_len[b] = -1;
+      a.final_token[b] = -1;
+      a.engine_draws[b] = 0;
+    }
+    return;
+  }
+  if (a.mode == 2) {
+    if (tid == 0) {
+      int n = 0;
+      while (n < K && t_ids(n)[0] == prop[n]) ++n;
+      a.accepted_len[b] = n;
+      a.final_token[b] = t_ids(n)[0];
+      a.engine_draws[b] = 0;
+    }
+    return;
+  }
+  if (a.mode == 1) {
+    int used = 0, accepted = 0;
+    int32_t tok = -1;
+    for (int i = 0; i <= K; ++i) {
+      const int n = tc[i];
+      const float* pr = t_probs(i);
+      const int pos = block_discrete_draw<4>(n, [=](int j) { return pr[j]; },
+                                             n >= 2 ? a.sample_u[static_cast<size_t>(b) * (K + 1) + used] : 0.0, sh);
+      if (n >= 2) ++used;
+      tok = t_ids(i)[pos];
+      if (i == K || tok != prop[i]) break;
+      ++accepted;
+    }
+    if (tid == 0) {
+      a.accepted_len[b] = accepted;
+      a.final_token[b] = tok;
+      a.engine_draws[b] = 2 * used;
+    }
+    return;
+  }
+  // mode 0: every position's two look-ups at once, a wave per position
+  const int32_t* dc = a.d_count + static_cast<size_t>(b) * K;
+  for (int i = wave; i < K; i += 4) {
+    const float pt = wave_sparse_prob(t_ids(i), t_probs(i), tc[i], prop[i]);
+    const float pd = wave_sparse_prob(a.d_ids + (static_cast<size_t>(b) * K + i) * a.d_cap,
+                                      a.d_probs + (static_cast<size_t>(b) * K + i) * a.d_cap, dc[i], prop[i]);
+    if (lane == 0) {
+      s_pt[i] = pt;
+      s_pd[i] = pd;
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int n = 0;
+    for (; n < K; ++n) {
+      const float acc = s_pd[n] <= 0.0f ? 1.0f : fminf(1.0f, s_pt[n] / s_pd[n]);  // ComputeAcceptProb
+      if (!(a.accept_u[static_cast<size_t>(b) * K + n] < acc)) break;
+    }
+    s_n = n;
+  }
+  __syncthreads();
+  const int n = s_n;
+  const int evaluated = n < K ? n + 1 : K;
+  const int nt = tc[n];
+  const int32_t* ids = t_ids(n);
+  const float* pr = t_probs(n);
+  bool use_residual = false;
+  float* res = a.residual + static_cast<size_t>(b) * a.residual_stride;
+  if (n < K) {
+    const int32_t* di = a.d_ids + (static_cast<size_t>(b) * K + n) * a.d_cap;
+    const float* dp = a.d_probs + (static_cast<size_t>(b) * K + n) * a.d_cap;
+    const int nd = dc[n];
+    int any = 0;
+    for (int j = tid; j < nt; j += 256) {
+      const int32_t id = ids[j];
+      float q = 0.0f;
+      for (int m = 0; m < nd; ++m)
+        if (di[m] == id) {
+          q = dp[m];
+          break;
+        }
+      const float d = pr[j] - q;
+      const float r = d > 0.0f ? d : 0.0f;
+      res[j] = r;
+      any |= r > 0.0f;
+    }
+    // the reference's sequential fp32 sum of non-negative terms is positive iff one of them is
+    use_residual = __syncthreads_or(any) != 0;
+  }
+  const double u = a.sample_u[static_cast<size_t>(b) * (K + 1) + evaluated];
+  int pos;
+  if (use_residual) {
+    const float* rr = res;
+    pos = block_discrete_draw<4>(nt, [=](int j) { return rr[j]; }, u, sh);
+  } else {
+    pos = block_discrete_draw<4>(nt, [=](int j) { return pr[j]; }, u, sh);
+  }
+  if (tid == 0) {
+    a.accepted_len[b] = n;
+    a.final_token[b] = ids[pos];
+    a.engine_draws[b] = evaluated + (nt >= 2 ? 2 : 0);
+  }
+}
+
 // fp16 -> fp32 with the reference's FastFloat16ToFloat32 semantics (DeviceInterface::Cast).
 __global__ __launch_bounds__(256) void widen_f16_kernel(const uint16_t* in, int64_t in_stride, float* out,
                                                         int64_t out_stride, int vocab) {
@@ -302,6 +448,11 @@ extern "C" hipError_t ms_launch_spec_verify(const float* p_target, const float* 
                                             int32_t* accepted_len, int32_t* final_token, hipStream_t stream) {
   hipLaunchKernelGGL(ms::spec_verify_kernel, dim3(batch), dim3(1024), 0, stream, p_target, p_draft, draft_tokens,
                      accept_u, sample_u, K, vocab, accepted_len, final_token);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_spec_verify_sparse(const ms::SpecSparseArgs* a, int batch, hipStream_t stream) {
+  hipLaunchKernelGGL(ms::spec_verify_sparse_kernel, dim3(batch), dim3(256), 0, stream, *a);
   return hipGetLastError();
 }
 

@@ -144,4 +144,56 @@ int ref_verify_deterministic(const int32_t* proposal, int n_prop, const int32_t*
   return result.accepted_count;
 }
 
+// The accept loop of SpeculativeDecodingStrategy::RunRound (src/speculative_decoding_strategy.cpp:718-762;
+// the strategy itself needs models and ONNX Runtime, so the loop is driven here) with the reference's own
+// ComputeAcceptProb, GetSparseTokenProbability, SampleCorrectionToken and SampleSparseToken and a real
+// std::mt19937{seed}.  accept_u_out (capacity K) and sample_u_out (capacity K+1: the canonical double
+// the engine would yield after e accept draws) report the uniforms in the oracle's explicit-draw form;
+// *engine_draws = engine outputs consumed by the round.
+void ref_spec_round_sparse(const int32_t* proposal, int K, const int32_t* t_off, const int32_t* t_idx,
+                           const float* t_probs, const int32_t* d_off, const int32_t* d_idx,
+                           const float* d_probs, uint32_t seed, float* accept_u_out, double* sample_u_out,
+                           int32_t* accepted_len, int32_t* final_token, int32_t* engine_draws) {
+  auto row = [](const int32_t* off, const int32_t* idx, const float* probs, int r) {
+    TargetTokenSelection sel;
+    sel.indices.assign(idx + off[r], idx + off[r + 1]);
+    sel.probs.assign(probs + off[r], probs + off[r + 1]);
+    return sel;
+  };
+  {
+    std::mt19937 probe{seed};
+    std::uniform_real_distribution<float> uni(0.f, 1.f);
+    for (int e = 0; e <= K; ++e) {
+      std::mt19937 at = probe;
+      sample_u_out[e] = CanonicalDouble(at);
+      if (e < K) accept_u_out[e] = uni(probe);
+    }
+  }
+  std::mt19937 rng{seed};
+  std::uniform_real_distribution<float> uni(0.f, 1.f);
+  int n_direct = 0;
+  int32_t tok = -1;
+  for (int i = 0; i < K; i++) {
+    const TargetTokenSelection target = row(t_off, t_idx, t_probs, i);
+    const TargetTokenSelection draft = row(d_off, d_idx, d_probs, i);
+    const float p_t = GetTargetTokenProbability(target, proposal[i]);
+    const float p_d = GetTargetTokenProbability(draft, proposal[i]);
+    if (uni(rng) < ComputeAcceptProb(p_t, p_d)) {
+      n_direct++;
+    } else {
+      tok = SampleCorrectionToken(target.indices, target.probs, draft.indices, draft.probs, rng);
+      break;
+    }
+  }
+  if (n_direct == K) {
+    const TargetTokenSelection bonus = row(t_off, t_idx, t_probs, K);
+    tok = SampleSparseToken(bonus.indices, bonus.probs, rng);
+  }
+  int used = 0;
+  for (std::mt19937 walk{seed}; !(walk == rng); walk.discard(1)) ++used;
+  *accepted_len = n_direct;
+  *final_token = tok;
+  *engine_draws = used;
+}
+
 }  // extern "C"

@@ -671,6 +671,44 @@ void orc_spec_verify_dense(const float* p_target, const float* p_draft, const in
   }
 }
 
+// ---- a16/a17 on sparse selections, the production form of the accept loop
+// (src/speculative_decoding_strategy.cpp:718-762): target row i (t_off[i]..t_off[i+1]) judges proposal
+// token i, target row K supplies the bonus token; draft row i is the proposal's own distribution at
+// position i.  accept_u[i] is the i-th uniform_real_distribution<float> draw; sample_u[e] is the
+// categorical draw the engine would yield after e accept draws have been taken (the loop takes one per
+// evaluated position, so the round's single categorical draw uses sample_u[evaluated]).  *engine_draws
+// = 32-bit engine outputs the reference would have consumed: one per evaluated position plus two for
+// the categorical draw unless its distribution has fewer than two entries.
+void orc_spec_verify_sparse(const int32_t* proposal, int K, const int32_t* t_off, const int32_t* t_idx,
+                            const float* t_probs, const int32_t* d_off, const int32_t* d_idx,
+                            const float* d_probs, const float* accept_u, const double* sample_u,
+                            int32_t* accepted_len, int32_t* final_token, int32_t* engine_draws) {
+  int n_direct = 0, n_evaluated = 0, final_n = 0;
+  int32_t tok = -1;
+  for (int i = 0; i < K; ++i) {
+    n_evaluated++;
+    const int nt = t_off[i + 1] - t_off[i], nd = d_off[i + 1] - d_off[i];
+    const float p_t = orc_sparse_prob(t_idx + t_off[i], t_probs + t_off[i], nt, proposal[i]);
+    const float p_d = orc_sparse_prob(d_idx + d_off[i], d_probs + d_off[i], nd, proposal[i]);
+    if (accept_u[i] < orc_accept_prob(p_t, p_d)) {
+      n_direct++;
+      continue;
+    }
+    tok = orc_sample_correction(t_idx + t_off[i], t_probs + t_off[i], nt, d_idx + d_off[i], d_probs + d_off[i], nd,
+                                sample_u[n_evaluated]);
+    final_n = nt;
+    break;
+  }
+  if (n_direct == K) {
+    const int nt = t_off[K + 1] - t_off[K];
+    tok = t_idx[t_off[K] + DiscreteDraw(t_probs + t_off[K], nt, sample_u[n_evaluated])];
+    final_n = nt;
+  }
+  *accepted_len = n_direct;
+  *final_token = tok;
+  *engine_draws = n_evaluated + (final_n >= 2 ? 2 : 0);
+}
+
 // ---- a18: src/speculative_sampling.h:59-79 ComputeTargetTokenSelection with
 // LogitsPenaltyProcessor::Apply (src/sampling_distribution.h:100-110): copy, min-length,
 // repetition, n-gram, then argmax (greedy) or the kept distribution.  Returns kept count (0 if greedy).

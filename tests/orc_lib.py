@@ -27,6 +27,16 @@ def _i32(a):
     return np.ascontiguousarray(np.asarray(a, dtype=np.int32))
 
 
+def _csr(rows):
+    """(ids, probs) rows -> offsets, concatenated ids, concatenated probs."""
+    off = np.zeros(len(rows) + 1, np.int32)
+    for i, (ix, _) in enumerate(rows):
+        off[i + 1] = off[i] + len(ix)
+    idx = np.concatenate([np.asarray(r[0], np.int32) for r in rows] + [np.zeros(1, np.int32)])
+    probs = np.concatenate([np.asarray(r[1], np.float32) for r in rows] + [np.zeros(1, np.float32)])
+    return off, np.ascontiguousarray(idx, np.int32), np.ascontiguousarray(probs, np.float32)
+
+
 def _f32(a):
     return np.ascontiguousarray(np.asarray(a, dtype=np.float32))
 
@@ -85,6 +95,8 @@ class Oracle:
         L.orc_target_selection.argtypes = [f32p, C.c_int, C.c_int, i32p, C.c_int, C.c_int, C.c_int, C.c_float,
                                            C.c_float, C.c_float, C.c_int, C.c_int, i32p, C.c_int,
                                            C.POINTER(C.c_int32), i32p, f32p]
+        L.orc_spec_verify_sparse.argtypes = [i32p, C.c_int, i32p, i32p, f32p, i32p, i32p, f32p, f32p, f64p,
+                                             C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
         L.orc_verify_deterministic.restype = C.c_int
         L.orc_verify_deterministic.argtypes = [i32p, C.c_int, i32p, i32p, f32p, f64p, C.POINTER(C.c_int32),
                                                C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]
@@ -231,6 +243,20 @@ class Oracle:
                                        v, acc, tok)
         return acc, tok
 
+    def spec_verify_sparse(self, proposal, target_rows, draft_rows, accept_u, sample_u):
+        """One sequence's round: K+1 target rows and K draft rows of (ids, probs), K accept uniforms and the
+        K+1 candidate categorical draws.  Returns (accepted, final token, engine draws consumed)."""
+        proposal = _i32(proposal)
+        k = proposal.size
+        assert len(target_rows) == k + 1 and len(draft_rows) == k
+        toff, tidx, tprob = _csr(target_rows)
+        doff, didx, dprob = _csr(draft_rows)
+        acc, tok, used = C.c_int32(), C.c_int32(), C.c_int32()
+        self.lib.orc_spec_verify_sparse(proposal, k, toff, tidx, tprob, doff, didx, dprob, _f32(accept_u),
+                                        np.ascontiguousarray(sample_u, np.float64), C.byref(acc), C.byref(tok),
+                                        C.byref(used))
+        return acc.value, tok.value, used.value
+
     def target_selection(self, logits, cur_len, prefix, greedy, k, p, t, rep_pen=1.0, min_len=0, ngram=0, eos=()):
         logits = _f32(logits)
         prefix = _i32(prefix)
@@ -346,6 +372,8 @@ class Reference:
         L.ref_target_selection.argtypes = [f32p, C.c_int, C.c_int, i32p, C.c_int, C.c_int, C.c_int, C.c_float,
                                            C.c_float, C.c_float, C.c_int, C.c_int, i32p, C.c_int,
                                            C.POINTER(C.c_int32), i32p, f32p]
+        L.ref_spec_round_sparse.argtypes = [i32p, C.c_int, i32p, i32p, f32p, i32p, i32p, f32p, C.c_uint32, f32p, f64p,
+                                            C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
         L.ref_verify_deterministic.restype = C.c_int
         L.ref_verify_deterministic.argtypes = [i32p, C.c_int, i32p, i32p, f32p, C.c_uint32, C.POINTER(C.c_int32),
                                                C.POINTER(C.c_int), C.POINTER(C.c_int), f64p, C.POINTER(C.c_int)]
@@ -420,6 +448,20 @@ class Reference:
         n = self.lib.ref_target_selection(logits, v, cur_len, prefix, prefix.size, int(greedy), k, p, t, rep_pen,
                                           min_len, ngram, eos, eos.size, C.byref(g), idx, probs)
         return g.value, idx[:n].copy(), probs[:n].copy()
+
+    def spec_round_sparse(self, proposal, target_rows, draft_rows, seed):
+        """The reference's accept loop with std::mt19937{seed}: returns (accepted, final token, engine draws
+        consumed, accept uniforms [K], candidate categorical draws [K+1])."""
+        proposal = _i32(proposal)
+        k = proposal.size
+        toff, tidx, tprob = _csr(target_rows)
+        doff, didx, dprob = _csr(draft_rows)
+        au = np.zeros(max(k, 1), np.float32)
+        su = np.zeros(k + 1, np.float64)
+        acc, tok, used = C.c_int32(), C.c_int32(), C.c_int32()
+        self.lib.ref_spec_round_sparse(proposal, k, toff, tidx, tprob, doff, didx, dprob, seed, au, su, C.byref(acc),
+                                       C.byref(tok), C.byref(used))
+        return acc.value, tok.value, used.value, au[:k].copy(), su
 
     def verify_deterministic(self, proposal, selections, seed):
         proposal = _i32(proposal)

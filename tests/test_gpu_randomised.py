@@ -203,3 +203,111 @@ def test_kv_gather_randomised(ctx, orc, seed):
     ctx.kv_gather(present, past, torch.from_numpy(idx).cuda())
     for p, q in zip(present, past):
         assert torch.equal(q.view(torch.int8).cpu(), p.view(torch.int8).cpu()[torch.from_numpy(idx).long()])
+
+
+def pack_rows(rows_per_seq, cap):
+    """[(ids, probs), ...] per sequence -> count [b, n], ids [b, n, cap], probs [b, n, cap] (padded)."""
+    b, n = len(rows_per_seq), len(rows_per_seq[0])
+    cnt = np.zeros((b, n), np.int32)
+    ids = np.full((b, n, cap), -7, np.int32)
+    pr = np.zeros((b, n, cap), np.float32)
+    for s, rows in enumerate(rows_per_seq):
+        for r, (ix, p) in enumerate(rows):
+            cnt[s, r] = len(ix)
+            ids[s, r, :len(ix)] = ix
+            pr[s, r, :len(ix)] = p
+    return tuple(torch.from_numpy(t).cuda() for t in (cnt, ids, pr))
+
+
+def random_round(rng, orc, vocab, K, big):
+    def rows(n):
+        out = []
+        for _ in range(n):
+            x = (rng.standard_normal(vocab) * 2).astype(np.float32)
+            k = int(rng.choice([0, 1, 2, 5, 50])) if big else int(rng.choice([1, 2, 5, 50]))
+            p = float(rng.choice([0.0, 0.6, 0.95])) if k else float(rng.choice([0.5, 0.9]))
+            out.append(orc.sampled_categorical(x, k, p, float(rng.choice([0.7, 1.0]))))
+        return out
+    target, draft = rows(K + 1), rows(K)
+    for i in range(K):
+        if rng.random() < 0.6:
+            draft[i] = (target[i][0].copy(), target[i][1].copy())
+            if len(draft[i][0]) > 2 and rng.random() < 0.5:
+                draft[i] = (draft[i][0][::-1].copy(), draft[i][1].copy())
+    proposal = np.array([d[0][rng.integers(0, len(d[0]))] for d in draft], np.int32)
+    for i in range(K):
+        if rng.random() < 0.1:
+            proposal[i] = rng.integers(0, vocab)
+    return proposal, target, draft
+
+
+@pytest.mark.parametrize("seed", range(max(CASES // 4, 1)))
+def test_spec_verify_sparse_randomised(ctx, orc, seed):
+    """The three modes of mi355x_spec_verify_sparse on kept sets (top-k sized, and nucleus sized for every
+    fourth seed) against orc_spec_verify_sparse / orc_verify_deterministic: accepted length, final token
+    and the number of engine outputs the reference would have consumed."""
+    rng = np.random.default_rng(9000 + seed)
+    batch = int(rng.integers(1, 7))
+    K = int(rng.integers(1, 9))
+    big = seed % 4 == 0
+    vocab = int(rng.choice([3, 60, 500, 5000])) if not big else 3000
+    say("spec_verify_sparse random", seed, batch, K, vocab, big)
+    rounds = [random_round(rng, orc, vocab, K, big) for _ in range(batch)]
+    cap_t = max(len(r[0]) for _, t, _ in rounds for r in t)
+    cap_d = max(len(r[0]) for _, _, d in rounds for r in d)
+    target = pack_rows([t for _, t, _ in rounds], cap_t + int(rng.integers(0, 3)))
+    draft = pack_rows([d for _, _, d in rounds], cap_d)
+    proposal = torch.from_numpy(np.stack([p for p, _, _ in rounds])).cuda()
+    au = rng.random((batch, K)).astype(np.float32)
+    su = rng.random((batch, K + 1))
+    acc, tok, used = ctx.spec_verify_sparse(target, draft, proposal, torch.from_numpy(au).cuda(),
+                                            torch.from_numpy(su).cuda(), mode=0)
+    for s, (prop, t, d) in enumerate(rounds):
+        assert (acc[s].item(), tok[s].item(), used[s].item()) == orc.spec_verify_sparse(prop, t, d, au[s], su[s]), s
+    # deterministic proposals: make them likely to match by proposing the oracle's own samples now and then
+    acc, tok, used = ctx.spec_verify_sparse(target, None, proposal, None, torch.from_numpy(su).cuda(), mode=1)
+    for s, (prop, t, _) in enumerate(rounds):
+        want = orc.verify_deterministic(prop, t, su[s])
+        assert (acc[s].item(), tok[s].item(), used[s].item()) == (want["accepted"], want["final_token"],
+                                                                   2 * want["draws_used"]), s
+    # greedy targets
+    acc, tok, used = ctx.spec_verify_sparse(target, None, proposal, None, None, mode=2)
+    for s, (prop, t, _) in enumerate(rounds):
+        n = 0
+        while n < K and t[n][0][0] == prop[n]:
+            n += 1
+        assert (acc[s].item(), tok[s].item(), used[s].item()) == (n, int(t[n][0][0]), 0), s
+
+
+def test_spec_verify_sparse_end_to_end_with_sampler_outputs(ctx, orc):
+    """The verify rows' kept sets come straight from mi355x_sample (device buffers, no host round trip) and
+    the proposal is built so that the first positions are accepted; a truncated kept set is reported as -1."""
+    say("spec_verify_sparse end to end")
+    rng = np.random.default_rng(77)
+    batch, K, vocab, cap = 3, 4, 32064, 64
+    x = (rng.standard_normal((batch * (K + 1), vocab)) * 3).astype(np.float32)
+    u = rng.random(batch * (K + 1))
+    _, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=50, p=0.9, temperature=0.8,
+                               kept_capacity=cap)
+    target = (kc.view(batch, K + 1), ki.view(batch, K + 1, cap), kp.view(batch, K + 1, cap))
+    rows = [[orc.sampled_categorical(x[s * (K + 1) + r], 50, 0.9, 0.8) for r in range(K + 1)] for s in range(batch)]
+    draft_rows = [[(t[0][:8].copy(), np.full(min(8, len(t[0])), 1.0 / min(8, len(t[0])), np.float32)) for t in seq[:K]]
+                  for seq in rows]
+    proposal = np.array([[seq[i][0][0] for i in range(K)] for seq in rows], np.int32)  # the targets' best tokens
+    proposal[1, 2] = 5  # an id the draft holds and the target row does not: certain reject
+    draft_rows[1][2][0][0] = 5
+    draft = pack_rows(draft_rows, 8)
+    au = rng.random((batch, K)).astype(np.float32)
+    su = rng.random((batch, K + 1))
+    acc, tok, used = ctx.spec_verify_sparse(target, draft, torch.from_numpy(proposal).cuda(),
+                                            torch.from_numpy(au).cuda(), torch.from_numpy(su).cuda(), mode=0)
+    for s in range(batch):
+        assert (acc[s].item(), tok[s].item(), used[s].item()) == orc.spec_verify_sparse(proposal[s], rows[s], draft_rows[s],
+                                                                                        au[s], su[s]), s
+    assert acc[1].item() <= 2
+    kc2 = kc.clone()
+    kc2[K + 2] = cap + 1  # sequence 1, row 1 claims more entries than the buffers hold
+    acc, tok, used = ctx.spec_verify_sparse((kc2.view(batch, K + 1), target[1], target[2]), draft,
+                                            torch.from_numpy(proposal).cuda(), torch.from_numpy(au).cuda(),
+                                            torch.from_numpy(su).cuda(), mode=0)
+    assert acc[1].item() == -1 and tok[1].item() == -1 and acc[0].item() >= 0

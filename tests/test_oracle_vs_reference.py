@@ -172,3 +172,47 @@ def test_verify_deterministic_matches_reference(orc, ref):
         for key in ("accepted", "evaluated", "final_token", "used_bonus"):
             assert o[key] == r[key], (seed, key)
         assert o["draws_used"] == len(r["draws"])
+
+
+def random_sparse_round(rng, vocab, K, orc):
+    """K+1 target rows and K draft rows as kept sets of random logits, plus proposal tokens drawn from the
+    draft rows (sometimes replaced by ids the target does not hold)."""
+    def rows(n, scale):
+        out = []
+        for _ in range(n):
+            x = (rng.standard_normal(vocab) * scale).astype(np.float32)
+            k = int(rng.choice([1, 2, 5, 50]))
+            p = float(rng.choice([0.0, 0.6, 0.95]))
+            out.append(orc.sampled_categorical(x, k, p, float(rng.choice([0.7, 1.0]))))
+        return out
+    target = rows(K + 1, 2.0)
+    draft = rows(K, 2.0)
+    for i in range(K):  # correlate drafts with targets so that accepts and rejects both occur
+        if rng.random() < 0.6:
+            draft[i] = (target[i][0].copy(), target[i][1].copy())
+            if len(draft[i][0]) > 2 and rng.random() < 0.5:
+                draft[i] = (draft[i][0][::-1].copy(), draft[i][1].copy())  # same ids, different probabilities
+    proposal = np.array([d[0][rng.integers(0, len(d[0]))] for d in draft], np.int32)
+    for i in range(K):
+        if rng.random() < 0.1:
+            proposal[i] = rng.integers(0, vocab)
+    return proposal, target, draft
+
+
+def test_sparse_accept_loop_matches_reference_with_real_engine(orc, ref):
+    """orc_spec_verify_sparse (explicit uniforms) against the reference's ComputeAcceptProb /
+    SampleCorrectionToken / SampleSparseToken driven by std::mt19937: accepted length, final token and the
+    number of engine outputs consumed (one per evaluated position, two for a categorical draw over at least
+    two entries)."""
+    rng = np.random.default_rng(21)
+    outcomes = set()
+    for case in range(300):
+        K = int(rng.integers(1, 9))
+        vocab = int(rng.choice([3, 60, 500]))
+        proposal, target, draft = random_sparse_round(rng, vocab, K, orc)
+        seed = int(rng.integers(0, 2 ** 31))
+        acc2, tok2, used2, au, su = ref.spec_round_sparse(proposal, target, draft, seed)
+        acc1, tok1, used1 = orc.spec_verify_sparse(proposal, target, draft, au, su)
+        assert (acc1, tok1, used1) == (acc2, tok2, used2), case
+        outcomes.add((acc1 == K, used1 - min(acc1 + 1, K)))
+    assert outcomes == {(True, 0), (True, 2), (False, 0), (False, 2)}  # bonus / correction, with and without a draw
