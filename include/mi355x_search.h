@@ -234,6 +234,20 @@ int mi355x_spec_verify_sparse(mi355x_search_ctx* ctx, void* stream, const int32_
                               const float* accept_u, const double* sample_u, int batch, int K, int mode,
                               int32_t* accepted_len, int32_t* final_token, int32_t* engine_draws);
 
+/* Tail of a greedy / sampling step on the device: Launch_CheckForEOSAndPad followed by
+ * Launch_AppendNextTokensToSequences (src/cuda/search_cuda.cu:33-48,80-117), i.e. PadIfAlreadyEOS,
+ * SetNextToken and AppendNextTokensToSequences of the CPU search (src/search.cpp:194-201,256-296):
+ * a row that has already produced EOS gets pad_token_id; a row whose token is an EOS id is marked; the
+ * (possibly padded) tokens are written to column current_length of the sequences; *done becomes 1 once
+ * every row is marked (it is never cleared here).  As in the CUDA search the append is unconditional
+ * while current_length < max_length: the caller advances its length only if the step did not finish.
+ *   next_tokens  device [batch] in/out      eos_seen  device [batch] int32 flags in/out
+ *   eos_ids      HOST [n_eos], n_eos <= MI355X_MAX_EOS
+ *   sequences    device [batch, max_length]  done  device int32 */
+int mi355x_greedy_tail(mi355x_search_ctx* ctx, void* stream, int32_t* next_tokens, int32_t* eos_seen,
+                       int batch, const int32_t* eos_ids, int n_eos, int32_t pad_token_id,
+                       int32_t* sequences, int max_length, int current_length, int32_t* done);
+
 /* Element-wise type conversion on the device: DeviceInterface::Cast (src/smartptrs.h:208-210; CPU
  * src/cpu/interface.cpp:74-106).  Supported pairs, with the CPU path's arithmetic: F16->F32
  * (FastFloat16ToFloat32), BF16->F32 (BFloat16ToFloat32), F32->F16 (FastFloat32ToFloat16), F32->BF16

@@ -64,6 +64,7 @@ def load_library():
         "mi355x_kv_gather": [vp, vp, C.POINTER(vp), C.POINTER(vp), i32, vp, i32, C.c_size_t],
         "mi355x_spec_verify": [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, vp],
         "mi355x_spec_verify_sparse": [vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, vp, vp, vp],
+        "mi355x_greedy_tail": [vp, vp, vp, vp, i32, C.POINTER(C.c_int32), i32, i32, vp, i32, i32, vp],
         "mi355x_cast": [vp, vp, vp, i32, vp, i32, C.c_size_t],
         "mi355x_logits_handoff": [vp, vp, vp, i32, i32, i32, i32, C.POINTER(C.c_int32), vp, i64],
     }.items():
@@ -288,6 +289,16 @@ def _spec_verify_sparse(self, target, draft, proposal, accept_u, sample_u, mode=
     return acc, tok, used
 
 
+def _greedy_tail(self, next_tokens, eos_seen, eos_ids, pad, sequences, current_length, done):
+    """EOS padding / marking, append at column current_length, all-rows-finished flag; all in place."""
+    for t in (next_tokens, eos_seen, sequences, done):
+        assert t.is_cuda and t.is_contiguous() and t.dtype == torch.int32
+    eos = (C.c_int32 * max(len(eos_ids), 1))(*eos_ids)
+    self._check(self.L.mi355x_greedy_tail(self.h, _stream(), next_tokens.data_ptr(), eos_seen.data_ptr(),
+                                          next_tokens.numel(), eos, len(eos_ids), pad, sequences.data_ptr(),
+                                          sequences.shape[1], current_length, done.data_ptr()))
+
+
 _DTYPE_CODES = {torch.float32: 1, torch.int32: 6, torch.int64: 7, torch.float16: 10, torch.bfloat16: 16}
 
 
@@ -321,6 +332,7 @@ SearchContext.topk_scores = _topk_scores
 SearchContext.softmax = _softmax
 SearchContext.beam_select = _beam_select
 SearchContext.spec_verify_sparse = _spec_verify_sparse
+SearchContext.greedy_tail = _greedy_tail
 SearchContext.kv_gather = _kv_gather
 SearchContext.spec_verify = _spec_verify
 

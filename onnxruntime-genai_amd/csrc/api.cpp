@@ -458,6 +458,20 @@ int mi355x_spec_verify_sparse(mi355x_search_ctx* ctx, void* stream, const int32_
   return MI355X_OK;
 }
 
+int mi355x_greedy_tail(mi355x_search_ctx* ctx, void* stream, int32_t* next_tokens, int32_t* eos_seen, int batch,
+                       const int32_t* eos_ids, int n_eos, int32_t pad_token_id, int32_t* sequences, int max_length,
+                       int current_length, int32_t* done) {
+  if (!ctx || !next_tokens || !eos_seen || !sequences || !done) return Fail(MI355X_E_INVALID, "null argument");
+  if (batch <= 0 || max_length <= 0 || current_length < 0)
+    return Fail(MI355X_E_INVALID, "batch (%d) and max_length (%d) must be positive, current_length (%d) not negative",
+                batch, max_length, current_length);
+  if (n_eos < 0 || n_eos > MI355X_MAX_EOS || (n_eos > 0 && !eos_ids))
+    return Fail(MI355X_E_INVALID, "n_eos (%d) out of range [0, %d] or null eos_ids", n_eos, MI355X_MAX_EOS);
+  HIP_TRY(ms_launch_greedy_tail(next_tokens, eos_seen, batch, eos_ids, n_eos, pad_token_id, sequences, max_length,
+                                current_length, done, static_cast<hipStream_t>(stream)));
+  return MI355X_OK;
+}
+
 int mi355x_cast(mi355x_search_ctx* ctx, void* stream, const void* in, int in_dtype, void* out, int out_dtype,
                 size_t count) {
   if (!ctx || !in || !out) return Fail(MI355X_E_INVALID, "null argument");

@@ -154,6 +154,9 @@ hipError_t ms_launch_kv_gather(const void* const* present_dev, void* const* past
 hipError_t ms_launch_spec_verify(const float* p_target, const float* p_draft, const int32_t* draft_tokens,
                                  const float* accept_u, const double* sample_u, int batch, int K, int vocab,
                                  int32_t* accepted_len, int32_t* final_token, hipStream_t stream);
+hipError_t ms_launch_greedy_tail(int32_t* next_tokens, int32_t* eos_seen, int batch, const int32_t* eos_ids, int n_eos,
+                                 int32_t pad, int32_t* sequences, int max_length, int current_length, int32_t* done,
+                                 hipStream_t stream);
 hipError_t ms_launch_spec_verify_sparse(const ms::SpecSparseArgs* a, int batch, hipStream_t stream);
 hipError_t ms_launch_widen_f16(const void* in, int64_t in_stride, float* out, int64_t out_stride, int rows,
                                int vocab, hipStream_t stream);

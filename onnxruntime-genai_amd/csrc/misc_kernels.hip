@@ -181,6 +181,34 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
   }
 }
 
+// ---- EOS bookkeeping and sequence append after token selection --------------------------------------
+// CheckForEOSAndPad + AppendNextTokensToSequences (src/cuda/search_cuda.cu:33-48,80-117) in one launch of
+// one workgroup.
+struct TailEos {
+  int n;
+  int32_t ids[MI355X_MAX_EOS];
+};
+
+__global__ __launch_bounds__(256) void greedy_tail_kernel(int32_t* next_tokens, int32_t* eos_seen, int batch, TailEos eos,
+                                                          int32_t pad, int32_t* sequences, int max_length,
+                                                          int current_length, int32_t* done) {
+  int live = 0;
+  for (int b = threadIdx.x; b < batch; b += 256) {
+    int32_t tok = next_tokens[b];
+    int seen = eos_seen[b];
+    if (seen) {
+      tok = pad;
+      next_tokens[b] = tok;
+    } else {
+      for (int e = 0; e < eos.n; ++e) seen |= (tok == eos.ids[e]);
+      if (seen) eos_seen[b] = 1;
+    }
+    live |= !seen;
+    if (current_length < max_length) sequences[static_cast<size_t>(b) * max_length + current_length] = tok;
+  }
+  if (__syncthreads_or(live) == 0 && threadIdx.x == 0) *done = 1;
+}
+
 // ---- speculative verification on sparse selections ----------------------------------------------------
 // One 256-thread block per sequence.  Target rows 0..K (row i judges proposal token i, row K is the
 // bonus row) and draft rows 0..K-1 are kept sets: count, ids, probabilities, padded to a capacity.
@@ -448,6 +476,17 @@ extern "C" hipError_t ms_launch_spec_verify(const float* p_target, const float* 
                                             int32_t* accepted_len, int32_t* final_token, hipStream_t stream) {
   hipLaunchKernelGGL(ms::spec_verify_kernel, dim3(batch), dim3(1024), 0, stream, p_target, p_draft, draft_tokens,
                      accept_u, sample_u, K, vocab, accepted_len, final_token);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_greedy_tail(int32_t* next_tokens, int32_t* eos_seen, int batch, const int32_t* eos_ids,
+                                            int n_eos, int32_t pad, int32_t* sequences, int max_length,
+                                            int current_length, int32_t* done, hipStream_t stream) {
+  ms::TailEos eos{};
+  eos.n = n_eos;
+  for (int i = 0; i < n_eos; ++i) eos.ids[i] = eos_ids[i];
+  hipLaunchKernelGGL(ms::greedy_tail_kernel, dim3(1), dim3(256), 0, stream, next_tokens, eos_seen, batch, eos, pad,
+                     sequences, max_length, current_length, done);
   return hipGetLastError();
 }
 

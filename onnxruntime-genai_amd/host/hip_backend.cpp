@@ -294,8 +294,6 @@ struct HipInterface final : DeviceInterface {
   DeviceSpan<float> small_scores_;
 };
 
-bool Contains(const std::vector<int>& v, int32_t t) { return std::find(v.begin(), v.end(), t) != v.end(); }
-
 void FillEos(const Config::Model& model, mi355x_logits_xform& xf) {
   if (model.eos_token_id.size() > MI355X_MAX_EOS) throw std::runtime_error("more EOS ids than the HIP backend supports");
   xf.n_eos = static_cast<int32_t>(model.eos_token_id.size());
@@ -322,16 +320,19 @@ GreedySearch_Hip::GreedySearch_Hip(const GeneratorParams& params) : Search{param
   uniforms_ = dev.Allocate<double>(batch);
   uniforms_.Zero();
   kept_count_ = dev.Allocate<int32_t>(batch);
-  eos_seen_.assign(batch, 0);
-  not_done_count_ = batch;
+  state_ = dev.Allocate<int32_t>(batch + 1);
+  state_.Zero();
+  tx_state_ = dev.Allocate<int32_t>(batch + 1);
+  if (params.config.model.eos_token_id.size() > MI355X_MAX_EOS)
+    throw std::runtime_error("more EOS ids than the HIP backend supports");
+  eos_ids_.assign(params.config.model.eos_token_id.begin(), params.config.model.eos_token_id.end());
 }
 
 GreedySearch_Hip::~GreedySearch_Hip() { mi355x_search_destroy(ctx_); }
 
 void GreedySearch_Hip::ResetDone() {
   done_ = false;
-  not_done_count_ = params_->search.batch_size;
-  std::fill(eos_seen_.begin(), eos_seen_.end(), 0);
+  state_.Zero();
 }
 
 void GreedySearch_Hip::SetLogits(DeviceSpan<float> logits) {
@@ -401,27 +402,29 @@ void GreedySearch_Hip::Materialize() const {
   ClearPending();
 }
 
-bool GreedySearch_Hip::PadIfAlreadyEOS(size_t batch_id) {
-  if (!eos_seen_[batch_id]) return false;
-  next_tokens_.CpuSpan()[batch_id] = params_->config.model.pad_token_id;
-  return true;
-}
-
-void GreedySearch_Hip::SetNextToken(size_t batch_id, int32_t token) {
-  next_tokens_.CpuSpan()[batch_id] = token;
-  if (Contains(params_->config.model.eos_token_id, token)) {
-    eos_seen_[batch_id] = 1;
-    if (--not_done_count_ == 0) done_ = true;
-  }
-}
-
-void GreedySearch_Hip::AppendNextTokensToSequences() {
+// The tail of a step runs on the device like the CUDA search's LaunchNextTokensTail
+// (src/cuda/search_cuda.cpp:268-288): finished rows are padded, EOS rows marked, the tokens appended
+// and the all-rows-finished flag raised by one kernel over the device-resident state (per-row EOS
+// flags followed by the flag).
+void GreedySearch_Hip::LaunchTail(int32_t* tokens) {
   const int batch = params_->BatchBeamSize();
-  const int cur = sequences_.GetSequenceLength();
-  // one token per row into column `cur` of the [batch, max_length] store
-  HIP_CHECK(hipMemcpy2DAsync(sequences_.GetSequences().Span().data() + cur, sizeof(int32_t) * sequences_.max_length_,
-                             next_tokens_.Span().data(), sizeof(int32_t), sizeof(int32_t), batch,
-                             hipMemcpyDeviceToDevice, g_stream));
+  AbiCheck(mi355x_greedy_tail(ctx_, g_stream, tokens, state_.Span().data(), batch, eos_ids_.data(),
+                              static_cast<int>(eos_ids_.size()), params_->config.model.pad_token_id,
+                              sequences_.GetSequences().Span().data(), sequences_.max_length_,
+                              sequences_.GetSequenceLength(), state_.Span().data() + batch));
+}
+
+// CompleteGeneration of the CUDA search (src/cuda/search_cuda.cpp:290-308): one synchronisation brings
+// back the (padded) tokens and the flag; the length advances only if the step did not finish.
+void GreedySearch_Hip::FinishStep() {
+  const int batch = params_->BatchBeamSize();
+  int32_t all_finished = 0;
+  HIP_CHECK(hipMemcpyAsync(next_tokens_.CpuSpan().data(), next_tokens_.Span().data(), sizeof(int32_t) * batch,
+                           hipMemcpyDeviceToHost, g_stream));
+  HIP_CHECK(hipMemcpyAsync(&all_finished, state_.Span().data() + batch, sizeof(int32_t), hipMemcpyDeviceToHost, g_stream));
+  HIP_CHECK(hipStreamSynchronize(g_stream));
+  if (all_finished) done_ = true;
+  if (done_) return;
   sequences_.AfterAppendNextTokens(next_tokens_, batch);
   if (sequences_.GetSequenceLength() == params_->search.max_length) done_ = true;
 }
@@ -431,22 +434,15 @@ void GreedySearch_Hip::SelectTop() {
   AbiCheck(mi355x_argmax(ctx_, g_stream, next_token_scores_.Span().data(), MI355X_F32, vocab, batch, vocab,
                          PendingXform(), next_tokens_.Span().data()));
   ClearPending();
-  const std::vector<int32_t> picked = [&] {
-    auto h = next_tokens_.CopyDeviceToCpu();
-    return std::vector<int32_t>(h.begin(), h.end());
-  }();
-  for (size_t b = 0; b < static_cast<size_t>(batch); ++b) {
-    if (PadIfAlreadyEOS(b)) continue;
-    SetNextToken(b, picked[b]);
-  }
-  next_tokens_.CopyCpuToDevice();  // the device copy always shows EOS padding, also on the last step
-  if (!done_) AppendNextTokensToSequences();
+  LaunchTail(next_tokens_.Span().data());
+  FinishStep();
 }
 
 void GreedySearch_Hip::CommitToken(int32_t token) {
-  SetNextToken(0, token);
-  next_tokens_.CopyCpuToDevice();  // the device copy always shows EOS padding, also on the last step
-  if (!done_) AppendNextTokensToSequences();
+  next_tokens_.CpuSpan()[0] = token;
+  next_tokens_.CopyCpuToDevice();
+  LaunchTail(next_tokens_.Span().data());
+  FinishStep();
 }
 
 bool GreedySearch_Hip::BindNextTokensSlot(DeviceSpan<int32_t> slot) {
@@ -455,20 +451,21 @@ bool GreedySearch_Hip::BindNextTokensSlot(DeviceSpan<int32_t> slot) {
   return true;
 }
 
+// The batched sampler has written this search's token into the bound element of the shared buffer:
+// the tail runs on it in place (so the caller's single copy of the buffer to the host already shows
+// the padding) and the result is mirrored into next_tokens_.
+void GreedySearch_Hip::OnNextTokensSampled() {
+  if (bound_slot_.size() != 1) throw std::runtime_error("OnNextTokensSampled without a bound next-token slot");
+  LaunchTail(bound_slot_.Span().data());
+  HIP_CHECK(hipMemcpyAsync(next_tokens_.Span().data(), bound_slot_.Span().data(), sizeof(int32_t),
+                           hipMemcpyDeviceToDevice, g_stream));
+  external_pending_ = true;
+}
+
 void GreedySearch_Hip::CompleteGeneration() {
   if (!external_pending_) return;
   external_pending_ = false;
-  // the caller has copied the shared buffer to the host after OnNextTokensSampled()
-  auto slot = bound_slot_.CpuSpan();
-  if (PadIfAlreadyEOS(0)) {
-    slot[0] = params_->config.model.pad_token_id;
-    HIP_CHECK(hipMemcpyAsync(bound_slot_.Span().data(), next_tokens_.CpuSpan().data(), sizeof(int32_t),
-                             hipMemcpyHostToDevice, g_stream));
-  } else {
-    SetNextToken(0, slot[0]);
-  }
-  next_tokens_.CopyCpuToDevice();  // the device copy always shows EOS padding, also on the last step
-  if (!done_) AppendNextTokensToSequences();
+  FinishStep();
 }
 
 void GreedySearch_Hip::Sample(int k, float p, float temperature, std::mt19937& rng) {
@@ -488,10 +485,14 @@ void GreedySearch_Hip::Sample(int k, float p, float temperature, std::mt19937& r
     auto h = kept_count_.CopyDeviceToCpu();
     return std::vector<int32_t>(h.begin(), h.end());
   }();
+  const std::vector<int32_t> finished = [&] {
+    auto h = state_.CopyDeviceToCpu();
+    return std::vector<int32_t>(h.begin(), h.begin() + batch);
+  }();
   std::vector<int32_t> ids;
   std::vector<float> probs;
   for (size_t b = 0; b < static_cast<size_t>(batch); ++b) {
-    if (PadIfAlreadyEOS(b)) continue;  // a finished row consumes no draw, as in the CPU loop
+    if (finished[b]) continue;  // a finished row consumes no draw, as in the CPU loop; the tail pads it
     const int n = counts[b];
     ids.resize(n);
     probs.resize(n);
@@ -500,10 +501,11 @@ void GreedySearch_Hip::Sample(int k, float p, float temperature, std::mt19937& r
     HIP_CHECK(hipStreamSynchronize(g_stream));
     // SampleCategoricalToken (src/sampling_distribution.h:218-227): same distribution object, same engine
     std::discrete_distribution<int> distribution(probs.begin(), probs.end());
-    SetNextToken(b, ids[static_cast<size_t>(distribution(rng))]);
+    next_tokens_.CpuSpan()[b] = ids[static_cast<size_t>(distribution(rng))];
   }
-  next_tokens_.CopyCpuToDevice();  // the device copy always shows EOS padding, also on the last step
-  if (!done_) AppendNextTokensToSequences();
+  next_tokens_.CopyCpuToDevice();
+  LaunchTail(next_tokens_.Span().data());
+  FinishStep();
 }
 
 void GreedySearch_Hip::AppendTokens(DeviceSpan<int32_t>& next_tokens) {
@@ -542,8 +544,8 @@ void GreedySearch_Hip::SaveStateForTransactionImpl(bool) {
   tx_next_tokens_.assign(host.begin(), host.end());
   auto lengths = sequence_lengths_.CopyDeviceToCpu();
   tx_sequence_lengths_.assign(lengths.begin(), lengths.end());
-  tx_eos_seen_ = eos_seen_;
-  tx_not_done_count_ = not_done_count_;
+  HIP_CHECK(hipMemcpyAsync(tx_state_.Span().data(), state_.Span().data(), sizeof(int32_t) * state_.size(),
+                           hipMemcpyDeviceToDevice, g_stream));
   tx_done_ = done_;
 }
 
@@ -553,8 +555,8 @@ void GreedySearch_Hip::RestoreStateForTransactionImpl() {
   std::copy(tx_sequence_lengths_.begin(), tx_sequence_lengths_.end(), sequence_lengths_.CpuSpan().begin());
   sequence_lengths_.CopyCpuToDevice();
   external_pending_ = false;
-  eos_seen_ = tx_eos_seen_;
-  not_done_count_ = tx_not_done_count_;
+  HIP_CHECK(hipMemcpyAsync(state_.Span().data(), tx_state_.Span().data(), sizeof(int32_t) * state_.size(),
+                           hipMemcpyDeviceToDevice, g_stream));
   done_ = tx_done_;
 }
 

@@ -31,14 +31,15 @@ struct GreedySearch_Hip : Search {
   void SetLogits(DeviceSpan<float> logits) override;
   bool IsDone() const override { return done_; }
   // Batched sampling seam (src/search.h:40-67): the engine samples a shared buffer with the
-  // BatchedSampler, binds one element of it here and has the tail (EOS / pad / append) run from
-  // CompleteGeneration() once it has copied the buffer to the host.  Token selection through
-  // SelectTop / Sample* always completes inline, which DeferCompletion(true) permits.
+  // BatchedSampler, binds one element of it here, and OnNextTokensSampled() launches the device tail
+  // (EOS / pad / append) on that element; CompleteGeneration() synchronises and advances the length.
+  // Token selection through SelectTop / Sample* always completes inline, which DeferCompletion(true)
+  // permits.
   void DeferCompletion(bool defer) override { defer_completion_ = defer; }
   void CompleteGeneration() override;
   bool BindNextTokensSlot(DeviceSpan<int32_t> slot) override;
   bool SupportsBatchedSampling() const override { return params_->BatchBeamSize() == 1; }
-  void OnNextTokensSampled() override { external_pending_ = true; }
+  void OnNextTokensSampled() override;
 
   void SelectTop() override;
   void CommitToken(int32_t token) override;
@@ -60,9 +61,8 @@ struct GreedySearch_Hip : Search {
   mi355x_logits_xform* PendingXform();
   void Materialize() const;  // applies the deferred logits processing to the logits in place
   void ClearPending() const;
-  bool PadIfAlreadyEOS(size_t batch_id);
-  void SetNextToken(size_t batch_id, int32_t token);
-  void AppendNextTokensToSequences();
+  void LaunchTail(int32_t* tokens);
+  void FinishStep();
   void ResetDone();
 
   mi355x_search_ctx* ctx_{};
@@ -72,8 +72,8 @@ struct GreedySearch_Hip : Search {
   DeviceSpan<float> kept_probs_;
   DeviceSpan<double> uniforms_;
   int kept_capacity_{};
-  std::vector<uint8_t> eos_seen_;
-  int not_done_count_{};
+  DeviceSpan<int32_t> state_, tx_state_;  // per-row EOS flags followed by the all-rows-finished flag
+  std::vector<int32_t> eos_ids_;
   bool done_{};
   bool defer_completion_{}, external_pending_{};
   DeviceSpan<int32_t> bound_slot_;
@@ -84,8 +84,6 @@ struct GreedySearch_Hip : Search {
   mutable mi355x_logits_xform xf_{};
   // transaction checkpoint
   std::vector<int32_t> tx_next_tokens_, tx_sequence_lengths_;
-  std::vector<uint8_t> tx_eos_seen_;
-  int tx_not_done_count_{};
   bool tx_done_{};
 };
 

@@ -466,3 +466,36 @@ def test_target_selection_of_verify_rows(ctx, orc, vocab, K, seed_len, greedy):
             assert np.array_equal(ki[i, :len(idx)], idx), i
             assert np.array_equal(bits(kp[i, :len(idx)]), bits(probs)), i
             assert tok[i] == idx[orc.discrete_draw(probs, u[i])], i
+
+
+@pytest.mark.parametrize("batch", [1, 7, 300])
+def test_greedy_tail_eos_pad_append(ctx, batch):
+    """CheckForEOSAndPad + AppendNextTokensToSequences against the CPU search's PadIfAlreadyEOS / SetNextToken /
+    AppendNextTokensToSequences loop (src/search.cpp:194-201,256-296) over a whole generation."""
+    say("greedy tail", batch)
+    rng = np.random.default_rng(batch)
+    max_length, eos, pad = 12, [3, 9], 1
+    seq = np.zeros((batch, max_length), np.int32)
+    seen = np.zeros(batch, bool)
+    d_seq = torch.zeros((batch, max_length), dtype=torch.int32, device="cuda")
+    d_seen = torch.zeros(batch, dtype=torch.int32, device="cuda")
+    d_done = torch.zeros(1, dtype=torch.int32, device="cuda")
+    length, done = 0, False
+    while not done and length < max_length:
+        tokens = rng.integers(0, 12 if length > 3 else 40, batch).astype(np.int32)
+        d_tok = torch.from_numpy(tokens).cuda()
+        ctx.greedy_tail(d_tok, d_seen, eos, pad, d_seq, length, d_done)
+        want = np.where(seen, pad, tokens)
+        seen |= np.isin(want, eos) & ~seen
+        done = bool(seen.all())
+        assert np.array_equal(d_tok.cpu().numpy(), want)
+        assert np.array_equal(d_seen.cpu().numpy().astype(bool), seen)
+        assert bool(d_done.item()) == done
+        if not done:  # the CPU search appends only while some row is alive; the device writes the column anyway
+            seq[:, length] = want
+            length += 1
+            assert np.array_equal(d_seq.cpu().numpy()[:, :length], seq[:, :length])
+    assert done or length == max_length
+    before = d_seq.clone()
+    ctx.greedy_tail(torch.zeros(batch, dtype=torch.int32, device="cuda"), d_seen, eos, pad, d_seq, max_length, d_done)
+    assert torch.equal(before, d_seq)  # nothing is written beyond max_length
