@@ -108,6 +108,11 @@ __device__ __forceinline__ float nucleus_depth(mi355x_sample_params prm, int voc
   return d * prm.temperature;
 }
 
+// Values of a published candidate slot that are not keys (a key's low half is ~id, far above these).
+constexpr u64 kSlotEmpty = 1, kSlotOverflow = 2;
+// Polls (about a microsecond each) after which a finishing workgroup stops waiting for a list and lets
+// the exact path compute the row.
+constexpr int kSpinLimit = 1 << 21;
 constexpr int kWaveListCap = 128;  // hits one wave can list per chunk
 
 // LDS of the fused kernel.
@@ -116,8 +121,8 @@ struct FusedShared {
   uint32_t mask_bits[kSChunk / 32];
   u64 wave_list[kSWaves * kWaveListCap];  // each wave's hits of this chunk, before the sort
   u64 list_hi[64];          // second half of a long list, sorted ascending
-  u64 lists[kAllCap];       // the chunks' sorted candidate lists of a row (finishing workgroup only)
-  u64 lists2[kAllCap / 2];  // second buffer of the merge tree
+  u64 own[64];              // the finishing workgroup's own list
+  u64 lists[kAllCap / 4];   // first-level results of the finishing workgroup's merge (rows of > 4 chunks)
   uint32_t pool[64];
   uint32_t wave_val[kSWaves];
   u64 wave_val64[kSWaves];
@@ -160,6 +165,11 @@ __device__ __forceinline__ double wave_scan_add(double x) {
 
 __device__ __forceinline__ float read_lane(float x, int l) {
   return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(x), l));
+}
+__device__ __forceinline__ u64 read_lane(u64 x, int l) {
+  const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(x), l);
+  const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(x >> 32), l);
+  return (static_cast<u64>(hi) << 32) | lo;
 }
 __device__ __forceinline__ double read_lane(double x, int l) {
   const u64 b = static_cast<u64>(__double_as_longlong(x));
@@ -262,6 +272,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   const float* lrow = a.logits + static_cast<size_t>(row) * a.row_stride;
   const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
   const float kNaN = __uint_as_float(0x7fc00000u);  // marks ids >= vocab: never a maximum, never >= a bound
+  const uint32_t poison = *a.fallback_rows;  // needed after the streaming pass only
   float v[kSElems];
 #pragma unroll
   for (int j = 0; j < kSVec; ++j) {
@@ -392,6 +403,9 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   }
 
   // ---- top-k, k <= 64 ---------------------------------------------------------------------------
+  // A finishing workgroup that once gave up waiting may have left published lists behind; from then on
+  // (bit 31 of the fallback counter) every row takes the exact path, which reads no such state.
+  if (poison >> 31) return chunk == a.chunks - 1;
   const int kk = prm.k < V ? prm.k : V;
   int n_valid = V - chunk * kSChunk;
   if (n_valid > kSChunk) n_valid = kSChunk;
@@ -438,9 +452,15 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   if (lane == 0) sm.wave_val[wave] = woff;
   __syncthreads();
   MS_STAGE(3, tau);
-  // The chunk publishes its best 64 candidates sorted (best first, zero-padded): nothing ranked lower
-  // inside its own chunk can be among the row's k <= 64 best.  Waves 0 and 1 sort one half of the
-  // list each; wave 0 merges, stores, and -- once its stores have been performed -- signals arrival.
+  // The chunk's best 64 candidates, sorted (best first): nothing ranked lower inside its own chunk can
+  // be among the row's k <= 64 best.  Waves 0 and 1 sort one half of the list each, wave 0 merges.
+  // The workgroup of the row's LAST chunk finishes the row; every other workgroup publishes its list
+  // and is done.  A published slot is never 0: kSlotEmpty pads a short list, kSlotOverflow replaces a
+  // list that did not fit.  The finishing workgroup polls the slots until all of them are non-zero and
+  // clears them again for the next launch; no counter, no wait for the stores and no second round
+  // trip lie between a chunk's sort and the row's merge.  Workgroups are dispatched in index order
+  // and a publishing workgroup never waits, so the lists a finishing workgroup polls for belong to
+  // workgroups that are running or done.
   uint32_t n_c = 0u;
   bool overflow = false;
 #pragma unroll
@@ -450,6 +470,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   }
   overflow = overflow || n_c > static_cast<uint32_t>(kListCap);
   const bool two_halves = n_c > 64u;
+  const bool finisher = chunk == a.chunks - 1;
   u64 mykey = 0;
   if (wave < 2 && !overflow) {
     // entry p of the concatenated wave lists
@@ -467,29 +488,19 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   }
   if (two_halves && !overflow) __syncthreads();
   if (wave == 0) {
-    if (!overflow) {
-      if (two_halves) {
-        const u64 other = sm.list_hi[lane];  // ascending against descending: a bitonic pair
-        mykey = other > mykey ? other : mykey;
-        sort_merge<64, 32, u64>(mykey, lane);
-      }
-      store_coherent(&dst[lane], mykey);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the wave's candidate stores have been performed
+    if (!overflow && two_halves) {
+      const u64 other = sm.list_hi[lane];  // ascending against descending: a bitonic pair
+      mykey = other > mykey ? other : mykey;
+      sort_merge<64, 32, u64>(mykey, lane);
     }
-    if (lane == 0) {
-      // low half: arrivals; high half: number of chunks whose candidates did not fit
-      const uint32_t add = 1u + (overflow ? 0x10000u : 0u);
-      const uint32_t old = __hip_atomic_fetch_add(&a.row_arrive[row], add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      sm.flag = ((old & 0xffffu) == static_cast<uint32_t>(a.chunks) - 1u) ? (old + add) : 0u;
-      sm.count = 0u;
-    }
+    const u64 slot = overflow ? kSlotOverflow : (mykey != 0 ? mykey : kSlotEmpty);
+    if (finisher) sm.own[lane] = slot;
+    else store_coherent(&dst[lane], slot);
   }
-  __syncthreads();
-  const uint32_t state = sm.flag;
-  MS_STAGE(5, state);
-  if (state == 0u) return false;
+  MS_STAGE(5, n_c);
+  if (!finisher) return false;
 
-  // ---- last workgroup of the row: rank the chunks' sorted lists against each other ----------------
+  // ---- the row's finishing workgroup ---------------------------------------------------------------
   LaneExp2Tab tab;
   {
     const uint64_t t = g_exp2_tab[lane & 31];  // issued now, consumed by the epilogue
@@ -497,75 +508,81 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     tab.hi = static_cast<uint32_t>(t >> 32);
   }
   const double u = a.emit_topk ? 0.0 : a.uniforms[row];
-  if (tid == 0) a.row_arrive[row] = 0u;
-  if ((state >> 16) != 0u) return true;  // a chunk could not list its candidates
-  const int nslots = a.chunks * kSmallCap;
-  const u64* seg = a.cand_small + static_cast<size_t>(row) * a.chunks * kSmallCap;
-  constexpr int kRegs = kAllCap / kSBlock;
-  {
-    u64 mine[kRegs];
-#pragma unroll
-    for (int r = 0; r < kRegs; ++r) {
-      const int p = r * kSBlock + tid;
-      mine[r] = p < nslots ? load_coherent(&seg[p]) : 0;
-    }
-#pragma unroll
-    for (int r = 0; r < kRegs; ++r) {
-      const int p = r * kSBlock + tid;
-      if (p < nslots) sm.lists[p] = mine[r];
-    }
-  }
-  __syncthreads();
-  MS_STAGE(6, sm.count);
-  // Merge tree over the sorted lists: a descending list against a reversed one is a bitonic pair
-  // whose lane-wise maximum holds the 64 best of both; six exchange stages sort it again.  Levels
-  // alternate between two LDS buffers; the last level leaves the row's 64 best in wave 0's lanes.
+  __syncthreads();  // sm.own
+  u64* seg = a.cand_small + static_cast<size_t>(row) * a.chunks * kSmallCap;
+  // Wave w merges the sorted lists of chunks 4w .. 4w+3 in registers, straight from global memory;
+  // rows of more than four chunks need a second level through LDS.  Wave 0 ends with the row's 64
+  // best, checks that there are k of them, and runs the epilogue while the other waves wait at the
+  // barrier that tells the workgroup whether the exact path is needed after all.
+  const int chunks = a.chunks;
+  const int groups = (chunks + 3) >> 2;
   u64 final_key = 0;
-  {
-    u64* src = sm.lists;
-    u64* dstl = sm.lists2;
-    int n = a.chunks;
-    if (n == 1 && wave == 0) final_key = src[lane];
-    while (n > 1) {
-      const int pairs = (n + 1) >> 1;
-      for (int q = wave; q < pairs; q += kSWaves) {
-        u64 x = src[(2 * q) * kSmallCap + lane];
-        if (2 * q + 1 < n) {
-          const u64 y = src[(2 * q + 1) * kSmallCap + 63 - lane];
-          x = y > x ? y : x;
-          sort_merge<64, 32, u64>(x, lane);
-        }
-        if (pairs > 1) dstl[q * kSmallCap + lane] = x;
-        else final_key = x;
+  bool bad = false;  // a list is missing (overflow, or the wait below gave up)
+  if (wave < groups) {
+    const int c0 = wave * 4;
+    // lane's four slots, in the orientation wave_merge4 wants them
+    const int cc[4] = {c0, c0 + 1, c0 + 2, c0 + 3};
+    const int ii[4] = {lane, 63 - lane, 63 - lane, lane};
+    u64 got[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (cc[q] >= chunks) got[q] = kSlotEmpty;
+      else if (cc[q] == chunks - 1) got[q] = sm.own[ii[q]];
+      else got[q] = 0;
+    }
+    int spins = 0;
+    while (true) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (got[q] == 0) got[q] = load_coherent(&seg[cc[q] * kSmallCap + ii[q]]);
+      if (__ballot(got[0] == 0 || got[1] == 0 || got[2] == 0 || got[3] == 0) == 0ull) break;
+      if (++spins == kSpinLimit) {
+        if (lane == 0) atomicOr(a.fallback_rows, 0x80000000u);
+        break;
       }
-      if (pairs > 1) __syncthreads();
-      u64* t = src;
-      src = dstl;
-      dstl = t;
-      n = pairs;
+      __builtin_amdgcn_s_sleep(2);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (cc[q] < chunks - 1 && got[q] != 0) store_coherent(&seg[cc[q] * kSmallCap + ii[q]], 0);  // for the next launch
+      bad = bad || got[q] == 0 || got[q] == kSlotOverflow;
+      if (got[q] <= kSlotOverflow) got[q] = 0;
+    }
+    bad = __ballot(bad) != 0ull;
+    const u64* g4 = got;
+    final_key = wave_merge4([&](int c, int) -> u64 { return g4[c]; }, lane);
+    if (groups > 1) sm.lists[wave * kSmallCap + lane] = final_key;
+    if (bad && lane == 0) sm.count = 1u;  // zeroed by thread 0 before the barriers of the bound
+  }
+  if (groups > 1) {
+    __syncthreads();
+    if (wave == 0) {
+      const u64* l = sm.lists;
+      final_key = wave_merge4([&](int c, int i) -> u64 { return c < groups ? l[c * kSmallCap + i] : 0; }, lane);
+      bad = sm.count != 0u;
     }
   }
-  if (tid < 64) {
-    const u64 kth = shfl_t<u64>(final_key, kk - 1);
-    if (lane == 0) sm.flag = kth != 0 ? 1u : 0u;
+  MS_STAGE(8, sm.count);
+  if (wave == 0) {
+    const u64 kth = read_lane(final_key, kk - 1);
+    const bool enough = !bad && kth != 0;  // otherwise NaNs are needed to fill k: the exact path decides
+    if (lane == 0) sm.flag = enough ? 1u : 0u;
+    if (enough) {
+      if (lane >= kk) final_key = 0;
+      if (a.emit_topk) {
+        if (lane < kk) {
+          const uint32_t id = key64_index(final_key);
+          a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(id);
+          a.out_scores[static_cast<size_t>(row) * prm.k + lane] =
+              a.logits[static_cast<size_t>(row) * a.row_stride + id];  // keys do not tell -0 from +0
+        }
+      } else {
+        wave_topk_epilogue(final_key, kk, prm, u, tab, row_outputs(a, row));
+      }
+    }
   }
   __syncthreads();
-  MS_STAGE(8, sm.count);
-  if (sm.flag == 0u) return true;  // NaNs are needed to fill k: the exact path decides
-  if (tid < 64) {
-    if (lane >= kk) final_key = 0;
-    if (a.emit_topk) {
-      if (lane < kk) {
-        const uint32_t id = key64_index(final_key);
-        a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(id);
-        a.out_scores[static_cast<size_t>(row) * prm.k + lane] =
-            a.logits[static_cast<size_t>(row) * a.row_stride + id];  // keys do not tell -0 from +0
-      }
-    } else {
-      wave_topk_epilogue(final_key, kk, prm, u, tab, row_outputs(a, row));
-    }
-  }
-  return false;
+  return sm.flag == 0u;
 }
 
 __global__ __launch_bounds__(kSBlock) void sample_fused_kernel(const SampleArgs a) {

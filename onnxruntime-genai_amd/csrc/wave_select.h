@@ -45,6 +45,34 @@ __device__ __forceinline__ void sort_merge(T& x, int lane) {
   if constexpr (J > 1) sort_merge<K, J / 2, T>(x, lane);
 }
 
+// Bitonic merge of a bitonic sequence held one key per lane: the result is sorted by lane, descending,
+// or ascending if ASC.
+template <int J, bool ASC, typename T>
+__device__ __forceinline__ void bitonic_merge(T& x, int lane) {
+  T y;
+  if constexpr (sizeof(T) == 8) y = lane_xor64<J>(x);
+  else y = lane_xor<J>(x);
+  const bool keep_max = ((lane & J) == 0) != ASC;
+  x = ((y > x) == keep_max) ? y : x;
+  if constexpr (J > 1) bitonic_merge<J / 2, ASC, T>(x, lane);
+}
+
+// The 64 largest of four lists of 64 keys, each sorted descending (list(c, i) = i-th best of list c, 0 for
+// a missing list), one result per lane, sorted descending.  A descending list against an ascending
+// one is a bitonic pair whose lane-wise maximum holds the 64 best of both; the two first-level
+// merges are independent and the second one is produced ascending so that no lane reversal is needed.
+template <typename List>
+__device__ __forceinline__ u64 wave_merge4(List list, int lane) {
+  const u64 a0 = list(0, lane), a1 = list(1, 63 - lane), b0 = list(2, 63 - lane), b1 = list(3, lane);
+  u64 a = a1 > a0 ? a1 : a0;
+  u64 b = b1 > b0 ? b1 : b0;
+  bitonic_merge<32, false, u64>(a, lane);
+  bitonic_merge<32, true, u64>(b, lane);
+  u64 g = b > a ? b : a;
+  bitonic_merge<32, false, u64>(g, lane);
+  return g;
+}
+
 // Bitonic sort of one key per lane, descending by lane (lane 0 ends with the maximum).
 template <typename T>
 __device__ __forceinline__ T wave_sort_desc_fast(T x) {
