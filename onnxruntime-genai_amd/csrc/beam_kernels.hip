@@ -63,7 +63,7 @@ __global__ __launch_bounds__(1024) void beam_row_kernel(const BeamArgs a) {
   __shared__ uint32_t pool[64];
   __shared__ uint32_t red[16];
   __shared__ u64 red64[16];
-  __shared__ uint32_t bound, count;
+  __shared__ uint32_t count;
   const int row = blockIdx.x, tid = threadIdx.x;
   const int V = a.vocab, m = 2 * a.beams;
   const InT* x = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(1024) void beam_row_kernel(const BeamArgs a) {
   const float own_max = key_to_float(block_max<uint32_t>(lkey, red));
   const float max_score = a.row_max ? a.row_max[row] : own_max;
   const int n_lanes = (V + kVec - 1) / kVec < 1024 ? (V + kVec - 1) / kVec : 1024;
-  const uint32_t tau = block_pool_bound(lkey, m, (n_lanes + 63) / 64, pool, &bound);
+  const uint32_t tau = block_pool_bound(lkey, m, (n_lanes + 63) / 64, pool);
   auto e = [=](int i) { return em::expf_exact(load_one<InT>(x, i) - max_score); };
   int dummy;
   const float lse = em::logf_exact(a.row_sum ? a.row_sum[row] : block_seq_sum<8>(0.0f, V, e, NoStop{}, &dummy, sh, stage, 256));

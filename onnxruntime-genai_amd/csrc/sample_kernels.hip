@@ -126,7 +126,7 @@ struct FusedShared {
   uint32_t pool[64];
   uint32_t wave_val[kSWaves];
   u64 wave_val64[kSWaves];
-  uint32_t count, flag, bound;
+  uint32_t count, flag;
   SeqShared seq;
 };
 
@@ -412,7 +412,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   const int n_lanes = n_valid >= 4 * kSBlock ? kSBlock : (n_valid + 3) / 4;
   const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
   u64* dst = a.cand_small + ci * kSmallCap;
-  uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool, &sm.bound);
+  uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool);
   if (tau == 0u) {
     // The pooled bound found fewer than k offers (a short tail chunk keeps its elements in one or two
     // waves): take the exact k-th best of the 256 per-thread maxima instead.
@@ -441,9 +441,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
           const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
                                                                 __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), 0u));
           // key64 of a real element is never 0 (its index half is ~idx != 0), so 0 marks an empty slot
+          // listed with the raw float bits; the few entries that survive get their order keys later
           if (pos < kWaveListCap)
             sm.wave_list[wave * kWaveListCap + pos] =
-                make_key64(order_key(v[j * 4 + c]), static_cast<uint32_t>(elem_index(chunk, j, c)));
+                make_key64(__float_as_uint(v[j * 4 + c]), static_cast<uint32_t>(elem_index(chunk, j, c)));
         }
         woff += static_cast<uint32_t>(__popcll(b));
       }
@@ -462,26 +463,34 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   // and a publishing workgroup never waits, so the lists a finishing workgroup polls for belong to
   // workgroups that are running or done.
   uint32_t n_c = 0u;
+  uint32_t cnt[kSWaves];
   bool overflow = false;
 #pragma unroll
   for (int w = 0; w < kSWaves; ++w) {
-    n_c += sm.wave_val[w];
-    overflow = overflow || sm.wave_val[w] > static_cast<uint32_t>(kWaveListCap);
+    cnt[w] = sm.wave_val[w];
+    n_c += cnt[w];
+    overflow = overflow || cnt[w] > static_cast<uint32_t>(kWaveListCap);
   }
   overflow = overflow || n_c > static_cast<uint32_t>(kListCap);
   const bool two_halves = n_c > 64u;
   const bool finisher = chunk == a.chunks - 1;
   u64 mykey = 0;
   if (wave < 2 && !overflow) {
-    // entry p of the concatenated wave lists
-    uint32_t p = static_cast<uint32_t>(wave) * 64u + static_cast<uint32_t>(lane);
+    // entry p of the concatenated wave lists: list w covers [start_w, start_w + count_w)
+    const uint32_t p = static_cast<uint32_t>(wave) * 64u + static_cast<uint32_t>(lane);
     if (p < n_c) {
-      int w = 0;
-      while (p >= sm.wave_val[w]) {
-        p -= sm.wave_val[w];
-        ++w;
+      uint32_t start = 0u, w = 0u, off = 0u;
+#pragma unroll
+      for (int i = 0; i < kSWaves - 1; ++i) {
+        start += cnt[i];
+        if (p >= start) {
+          w = static_cast<uint32_t>(i) + 1u;
+          off = start;
+        }
       }
-      mykey = sm.wave_list[w * kWaveListCap + p];
+      const u64 raw = sm.wave_list[w * kWaveListCap + (p - off)];
+      mykey = (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw >> 32)))) << 32) |
+              (raw & 0xffffffffull);
     }
     if (wave == 0 || two_halves) mykey = wave_sort_desc_fast<u64>(mykey);
     if (wave == 1 && two_halves) sm.list_hi[63 - lane] = mykey;

@@ -123,24 +123,29 @@ __device__ __forceinline__ void store_coherent(u64* p, u64 v) {
 
 // A key tau such that at least k of the keys offered by the block's threads are >= tau (0 if there
 // are fewer than k offers).  One offer per thread (0 = none); only the first nw waves hold offers.
-// Every wave sorts its 64 offers and pools its best 64/nw; wave 0 sorts the pool and takes its k-th
-// entry: the exact k-th best offer unless one wave holds more than its share of the top k.
-// Two barriers; every thread gets the result.  Any block of up to 16 waves, 1 <= k <= 64.
-__device__ __forceinline__ uint32_t block_pool_bound(uint32_t offer, int k, int nw, uint32_t* pool, uint32_t* result) {
+// Every wave sorts its 64 offers and pools its best 64/nw; the pool's k-th entry is the exact k-th
+// best offer unless one wave holds more than its share of the top k.  Waves write their shares in
+// alternating directions, so the pool arrives as sorted runs that only the last merge levels of the
+// sorting network have to join, and every wave sorts the pool for itself: one barrier, no broadcast.
+// Any block of up to 16 waves, 1 <= k <= 64.
+__device__ __forceinline__ uint32_t block_pool_bound(uint32_t offer, int k, int nw, uint32_t* pool) {
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
   if (nw < 1) nw = 1;
   const int c = 64 / nw;
   const uint32_t sorted = wave_sort_desc_fast<uint32_t>(offer);
-  if (wave < nw && lane < c) pool[wave * c + lane] = sorted;
+  const bool runs = (nw == 8);  // shares of 8: the sorting network's state before its 16-merge level
+  if (wave < nw && lane < c) pool[wave * c + ((runs && (wave & 1)) ? c - 1 - lane : lane)] = sorted;
   if (tid < 64 && tid >= nw * c) pool[tid] = 0u;
   __syncthreads();
-  if (wave == 0) {
-    const uint32_t ps = wave_sort_desc_fast<uint32_t>(pool[lane]);
-    const uint32_t tau = shfl_t<uint32_t>(ps, k - 1);
-    if (lane == 0) *result = tau;
+  uint32_t ps = pool[lane];
+  if (runs) {
+    sort_merge<16, 8, uint32_t>(ps, lane);
+    sort_merge<32, 16, uint32_t>(ps, lane);
+    sort_merge<64, 32, uint32_t>(ps, lane);
+  } else {
+    ps = wave_sort_desc_fast<uint32_t>(ps);
   }
-  __syncthreads();
-  return *result;
+  return static_cast<uint32_t>(__builtin_amdgcn_readlane(ps, k - 1));
 }
 
 }  // namespace ms
