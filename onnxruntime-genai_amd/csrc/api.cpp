@@ -286,9 +286,6 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
-#ifdef MS_DEBUG_STAGES
-  a.debug_stage = getenv("MS_STAGE") ? atoi(getenv("MS_STAGE")) : 0;
-#endif
   HIP_TRY(ms_launch_sample(&a, any_nucleus, s));
   return MI355X_OK;
 }

@@ -48,9 +48,6 @@ struct SampleArgs {
   uint32_t* fallback_rows;  // cumulative count of rows finished by the general path
   int emit_topk;            // != 0: write the k best (id, raw score) per row instead of sampling
   float* out_scores;        // [rows, k], emit_topk only (out_tokens is [rows, k] then)
-#ifdef MS_DEBUG_STAGES
-  int debug_stage;  // timing experiments only: stop after the given stage
-#endif
 };
 
 struct ArgmaxArgs {

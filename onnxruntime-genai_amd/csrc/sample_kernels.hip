@@ -14,12 +14,6 @@
 
 namespace ms {
 
-#ifdef MS_DEBUG_STAGES
-#define MS_STAGE(n, keep) do { if (a.debug_stage == (n)) { if ((keep) == 0x12345u) a.out_tokens[row] = 1; return false; } } while (0)
-#else
-#define MS_STAGE(n, keep) do { } while (0)
-#endif
-
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ int next_pow2(int v) {
@@ -348,7 +342,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     fm = fmaxf(fm, qm[j]);
   }
   const uint32_t lmax = elem_index(chunk, 0, 0) < V ? order_key(fm) : 0u;  // 0: thread holds no element
-  MS_STAGE(1, lmax);
   if (tid == 0) sm.count = 0u;
 
   if (mode == kModeNucleus) {
@@ -422,7 +415,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     tau = static_cast<uint32_t>(sm.lists[kk - 1]);
     __syncthreads();
   }
-  MS_STAGE(2, tau);
   // tau == 0: the chunk has fewer than k elements -- keep them all
   const float tau_f = tau != 0u ? key_to_float(tau) : -__builtin_inff();
   // Hits are rare (about k per chunk).  Every wave lists its own hits in a private LDS segment: the
@@ -452,7 +444,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   }
   if (lane == 0) sm.wave_val[wave] = woff;
   __syncthreads();
-  MS_STAGE(3, tau);
   // The chunk's best 64 candidates, sorted (best first): nothing ranked lower inside its own chunk can
   // be among the row's k <= 64 best.  Waves 0 and 1 sort one half of the list each, wave 0 merges.
   // The workgroup of the row's LAST chunk finishes the row; every other workgroup publishes its list
@@ -506,7 +497,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     if (finisher) sm.own[lane] = slot;
     else store_coherent(&dst[lane], slot);
   }
-  MS_STAGE(5, n_c);
   if (!finisher) return false;
 
   // ---- the row's finishing workgroup ---------------------------------------------------------------
@@ -571,7 +561,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
       bad = sm.count != 0u;
     }
   }
-  MS_STAGE(8, sm.count);
   if (wave == 0) {
     const u64 kth = read_lane(final_key, kk - 1);
     const bool enough = !bad && kth != 0;  // otherwise NaNs are needed to fill k: the exact path decides
