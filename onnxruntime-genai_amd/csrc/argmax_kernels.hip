@@ -56,18 +56,31 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
   constexpr int VEC = Loader<InT>::VEC;
   constexpr int NB = 8;  // vectors a thread has in flight: all their loads are issued before any is used
   const int row = blockIdx.x, tid = threadIdx.x;
-  const int V = a.vocab;
+  // everything this latency-bound kernel reads from its arguments, fetched together
+  const int V = arg_now(a.vocab);
+  const int64_t row_stride = arg_now(a.row_stride);
+  const InT* const logits = static_cast<const InT*>(arg_now(a.logits));
+  int32_t* const out_tokens = arg_now(a.out_tokens);
+  const uint32_t* const mask = arg_now(a.xf.mask);
+  const int32_t* const history = arg_now(a.xf.history);
+  const int32_t* const history_lens = arg_now(a.xf.history_lens);
+  const uint32_t* const ban = arg_now(a.xf.ban);
+  const int history_stride = arg_now(a.xf.history_stride);
+  const int history_len = arg_now(a.xf.history_len);
+  const int min_length = arg_now(a.xf.min_length);
+  const int n_eos_all = arg_now(a.xf.n_eos);
+  const float penalty = arg_now(a.xf.penalty);
   __shared__ uint32_t hist_bits[kRowKernelMaxVocab / 32];
   __shared__ u64 red64[16];
-  const InT* lrow = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
+  const InT* lrow = logits + static_cast<size_t>(row) * row_stride;
   const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
-  const bool pen = a.xf.use_penalty();
-  const bool has_mask = a.xf.mask != nullptr;
-  const bool active = a.xf.active();
-  const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
-  const int n_eos = active ? a.xf.eos_count(row) : 0;
-  const uint32_t* ban_row = a.xf.ban_row(row, V);
-  const int hlen = pen ? a.xf.hist_len(row) : 0;
+  const bool pen = history && (history_lens || history_len > 0) && (penalty != 1.0f || ban);  // Xform::use_penalty
+  const bool has_mask = mask != nullptr;
+  const bool active = has_mask || pen || n_eos_all > 0;
+  const uint32_t* mrow = has_mask ? mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
+  const int hlen = pen ? (history_lens ? history_lens[row] : history_len) : 0;
+  const int n_eos = (history_lens && min_length > 0 && history_lens[row] >= min_length) ? 0 : n_eos_all;
+  const uint32_t* ban_row = ban ? ban + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
   u64 best = 0;
   for (int base = 0; base < V; base += 1024 * VEC * NB) {
     float v[NB][VEC];
@@ -95,7 +108,7 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
       }
     }
     if (pen && base == 0) {  // built while the first batch of loads is in flight
-      const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
+      const int32_t* h = history + static_cast<size_t>(row) * history_stride;
       int hv[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) hv[r] = (r * 1024 + tid < hlen) ? h[r * 1024 + tid] : -1;
@@ -119,7 +132,7 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
         const int idx = i0 + c;
         if (idx < V) {
           float x = v[j][c];
-          if (active) x = xform_value(x, a.xf, idx, mw[j], has_mask, (hw >> (idx & 31)) & 1u, n_eos, ban_row);
+          if (active) x = xform_value(x, penalty, a.xf.eos, idx, mw[j], has_mask, (hw >> (idx & 31)) & 1u, n_eos, ban_row);
           u64 k = make_key64(order_key(x), static_cast<uint32_t>(idx));
           if (idx == 0 && x != x) k = ~0ull;  // NaN at index 0 is sticky
           if (k == 0) k = 1;
@@ -129,7 +142,7 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
     }
   }
   best = block_max<u64>(best, red64);
-  if (tid == 0) a.out_tokens[row] = static_cast<int32_t>(key64_index(best));
+  if (tid == 0) out_tokens[row] = static_cast<int32_t>(key64_index(best));
 }
 
 // mask -> min-length -> repetition penalty, written back in place

@@ -197,6 +197,16 @@ struct Xform {
   }
 };
 
+// Kernel arguments live in memory and are read with scalar loads of a few hundred cycles each.  Left to
+// the compiler, each is fetched where it is first needed, one wait after the other, which shows in
+// latency-bound kernels.  arg_now() makes the value exist at the point of the call, so that a group of
+// calls puts all those loads in flight together.
+template <typename T>
+__device__ __forceinline__ T arg_now(T x) {
+  asm volatile("" : "+s"(x));
+  return x;
+}
+
 // Marks, in an LDS bitmap covering vocabulary ids [base, base + kChunk), the ids present in the
 // row's history.  bits: kChunk/32 words.  Ends with a barrier.
 __device__ __forceinline__ void build_history_bitmap(const Xform& xf, int row, int base, uint32_t* bits) {
@@ -214,13 +224,13 @@ __device__ __forceinline__ void build_history_bitmap(const Xform& xf, int row, i
 // The reference's order: mask -> min-length -> repetition penalty -> no-repeat-n-gram ban
 // (src/standard_decoding_strategy.cpp:24-32, src/sampling_distribution.h:100-110).  n_eos and
 // ban_row are the row's values (Xform::eos_count, Xform::ban_row).
-__device__ __forceinline__ float xform_value(float x, const Xform& xf, int idx, uint32_t mask_word,
+__device__ __forceinline__ float xform_value(float x, float penalty, const int* eos, int idx, uint32_t mask_word,
                                              bool has_mask, bool in_history, int n_eos, const uint32_t* ban_row) {
   if (has_mask && !((mask_word >> (idx & 31)) & 1u)) x = kLowest;
   for (int e = 0; e < n_eos; ++e)
-    if (xf.eos[e] == idx) x = kLowest;
+    if (eos[e] == idx) x = kLowest;
   if (in_history) {
-    x = x < 0.0f ? x * xf.penalty : x / xf.penalty;
+    x = x < 0.0f ? x * penalty : x / penalty;
     if (ban_row && ((ban_row[idx >> 5] >> (idx & 31)) & 1u)) x = kLowest;
   }
   return x;
@@ -305,7 +315,7 @@ __device__ __forceinline__ void xform_chunk(const Xform& xf, int row, int vocab,
         const uint32_t mw = has_mask ? mrow[idx >> 5] : 0u;
         const int rel = idx - chunk * kChunk;
         const bool hit = pen && ((hist_bits[rel >> 5] >> (rel & 31)) & 1u);
-        v[j * L::VEC + c] = xform_value(v[j * L::VEC + c], xf, idx, mw, has_mask, hit, n_eos, ban_row);
+        v[j * L::VEC + c] = xform_value(v[j * L::VEC + c], xf.penalty, xf.eos, idx, mw, has_mask, hit, n_eos, ban_row);
       }
     }
   }

@@ -43,7 +43,7 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
   for (int i = threadIdx.x; i < n2; i += blockDim.x) {
     u64 k = 0;
     if (i < V) {
-      const float x = xform_value(lrow[i], a.xf, i, has_mask ? mrow[i >> 5] : 0u, has_mask, false, n_eos, ban_row);
+      const float x = xform_value(lrow[i], a.xf.penalty, a.xf.eos, i, has_mask ? mrow[i >> 5] : 0u, has_mask, false, n_eos, ban_row);
       k = make_key64(order_key(x), static_cast<uint32_t>(i));
     }
     scratch[i] = k;
@@ -58,7 +58,7 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
       bool dup = false;
       for (int jj = 0; jj < j && !dup; ++jj) dup = (h[jj] == tok);
       if (dup) continue;
-      const float x = xform_value(lrow[tok], a.xf, tok, has_mask ? mrow[tok >> 5] : 0u, has_mask, true, n_eos, ban_row);
+      const float x = xform_value(lrow[tok], a.xf.penalty, a.xf.eos, tok, has_mask ? mrow[tok >> 5] : 0u, has_mask, true, n_eos, ban_row);
       scratch[tok] = make_key64(order_key(x), static_cast<uint32_t>(tok));
     }
     __syncthreads();
@@ -282,6 +282,17 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
       for (int c = 0; c < 4; ++c) v[j * 4 + c] = (i0 + c < V) ? lrow[i0 + c] : kNaN;
     }
   }
+  // The arguments the phases after the streaming pass need are fetched now, while the logits are in
+  // flight, instead of one by one where they are first used.
+  const int n_chunks = arg_now(a.chunks);
+  u64* const cand_small = arg_now(a.cand_small);
+  const double* const uniforms = arg_now(a.uniforms);
+  const int emit_topk = arg_now(a.emit_topk);
+  const RowOutputs outputs = {arg_now(a.out_tokens) + row,
+                              arg_now(a.kept_count),
+                              arg_now(a.kept_ids),
+                              arg_now(a.kept_probs),
+                              arg_now(a.kept_capacity)};
   if (a.xf.active()) {
     // The chunk's grammar-mask words and the bitmap of history ids are staged in LDS once; a thread
     // then needs one nibble of each per float4.
@@ -398,13 +409,13 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   // ---- top-k, k <= 64 ---------------------------------------------------------------------------
   // A finishing workgroup that once gave up waiting may have left published lists behind; from then on
   // (bit 31 of the fallback counter) every row takes the exact path, which reads no such state.
-  if (poison >> 31) return chunk == a.chunks - 1;
+  if (poison >> 31) return chunk == n_chunks - 1;
   const int kk = prm.k < V ? prm.k : V;
   int n_valid = V - chunk * kSChunk;
   if (n_valid > kSChunk) n_valid = kSChunk;
   const int n_lanes = n_valid >= 4 * kSBlock ? kSBlock : (n_valid + 3) / 4;
-  const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
-  u64* dst = a.cand_small + ci * kSmallCap;
+  const size_t ci = static_cast<size_t>(row) * n_chunks + chunk;
+  u64* dst = cand_small + ci * kSmallCap;
   uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool);
   if (tau == 0u) {
     // The pooled bound found fewer than k offers (a short tail chunk keeps its elements in one or two
@@ -464,7 +475,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   }
   overflow = overflow || n_c > static_cast<uint32_t>(kListCap);
   const bool two_halves = n_c > 64u;
-  const bool finisher = chunk == a.chunks - 1;
+  const bool finisher = chunk == n_chunks - 1;
   u64 mykey = 0;
   if (wave < 2 && !overflow) {
     // entry p of the concatenated wave lists: list w covers [start_w, start_w + count_w)
@@ -506,14 +517,14 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     tab.lo = static_cast<uint32_t>(t);
     tab.hi = static_cast<uint32_t>(t >> 32);
   }
-  const double u = a.emit_topk ? 0.0 : a.uniforms[row];
+  const double u = emit_topk ? 0.0 : uniforms[row];
   __syncthreads();  // sm.own
-  u64* seg = a.cand_small + static_cast<size_t>(row) * a.chunks * kSmallCap;
+  u64* seg = cand_small + static_cast<size_t>(row) * n_chunks * kSmallCap;
   // Wave w merges the sorted lists of chunks 4w .. 4w+3 in registers, straight from global memory;
   // rows of more than four chunks need a second level through LDS.  Wave 0 ends with the row's 64
   // best, checks that there are k of them, and runs the epilogue while the other waves wait at the
   // barrier that tells the workgroup whether the exact path is needed after all.
-  const int chunks = a.chunks;
+  const int chunks = n_chunks;
   const int groups = (chunks + 3) >> 2;
   u64 final_key = 0;
   bool bad = false;  // a list is missing (overflow, or the wait below gave up)
@@ -567,7 +578,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     if (lane == 0) sm.flag = enough ? 1u : 0u;
     if (enough) {
       if (lane >= kk) final_key = 0;
-      if (a.emit_topk) {
+      if (emit_topk) {
         if (lane < kk) {
           const uint32_t id = key64_index(final_key);
           a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(id);
@@ -575,7 +586,13 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
               a.logits[static_cast<size_t>(row) * a.row_stride + id];  // keys do not tell -0 from +0
         }
       } else {
-        wave_topk_epilogue(final_key, kk, prm, u, tab, row_outputs(a, row));
+        {
+          RowOutputs out = outputs;  // pointers to this row's slots
+          out.kept_count = out.kept_count ? out.kept_count + row : nullptr;
+          out.kept_ids = out.kept_ids ? out.kept_ids + static_cast<size_t>(row) * out.kept_capacity : nullptr;
+          out.kept_probs = out.kept_probs ? out.kept_probs + static_cast<size_t>(row) * out.kept_capacity : nullptr;
+          wave_topk_epilogue(final_key, kk, prm, u, tab, out);
+        }
       }
     }
   }
