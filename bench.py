@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Headline benchmark: top-k/top-p sampling step, batch 64 x vocab 128256 (BASELINE config 2).
+"""Headline benchmark: top-k/top-p sampling step, batch 64 x vocab 128256 (Benchmark configuration 2).
 
 A step is one pass of the sampling hot path (mi355x_sample: fused selection + softmax + nucleus cut +
 categorical draw) over one batch of seeded synthetic fp32 logits resident in HBM.  The K timed steps
@@ -38,7 +38,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (rows shard across GPUs "
-                 "without communication; see DESIGN.md). Run with --gpus 1.")
+                 "without communication). Run with --gpus 1.")
 
     import numpy as np
     import torch

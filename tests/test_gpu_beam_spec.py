@@ -141,7 +141,7 @@ def run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, lengt
 
 
 def test_config3_beam_search_steps(ctx, orc):
-    """BASELINE config 3 shape (batch 8, beams 4, vocab 151936 fp16, length_penalty 1.0), 6 of the 64
+    """Benchmark configuration 3 shape (batch 8, beams 4, vocab 151936 fp16, length_penalty 1.0), 6 of the 64
     steps: selection, scorer state, beam-reordered sequences and final hypotheses match the oracle."""
     run_beam_search(ctx, orc, 8, 4, 151936, 6, [151935], 80, 1.0, True, 3)
 
@@ -187,7 +187,7 @@ def softmax64(x):
 
 @pytest.mark.parametrize("batch,K,vocab", [(16, 8, 32064), (4, 3, 500), (5, 1, 2)])
 def test_spec_verify(ctx, orc, batch, K, vocab):
-    """BASELINE config 4 (first case): target/draft probabilities from N(0,2^2) logits, draft = target
+    """Benchmark configuration 4 (first case): target/draft probabilities from N(0,2^2) logits, draft = target
     logits + N(0,0.5^2); accept tests and residual / bonus resampling with shared uniforms."""
     say("spec_verify", batch, K, vocab)
     rng = np.random.default_rng(vocab + K)

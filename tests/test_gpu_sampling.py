@@ -58,7 +58,7 @@ def test_argmax_fp16(ctx, orc):
 
 
 def test_config1_greedy_with_repetition_penalty(ctx, orc):
-    """BASELINE config 1: batch 1, vocab 32064, N(0,2^2) logits with a +8 spike, repetition penalty
+    """Benchmark configuration 1: batch 1, vocab 32064, N(0,2^2) logits with a +8 spike, repetition penalty
     1.1 over 512 history ids, greedy argmax per step (16 of the 256 steps here)."""
     rng = np.random.default_rng(1)
     vocab = 32064
@@ -172,7 +172,7 @@ def test_draw_on_cdf_boundaries(ctx, orc, vocab, k, p, t):
 
 
 def test_config2_topk_topp_batch64(ctx, orc):
-    """BASELINE config 2 at full size: batch 64, vocab 128256, N(0,3^2) logits + 8 peaks/row at +10,
+    """Benchmark configuration 2 at full size: batch 64, vocab 128256, N(0,3^2) logits + 8 peaks/row at +10,
     T=0.7, k=50, p=0.9, shared uniforms; 4 of the 128 steps."""
     rng = np.random.default_rng(2)
     rows, vocab = 64, 128256
@@ -284,7 +284,7 @@ def test_nucleus_candidate_counts_and_ties(ctx, orc, frac, quantum):
 
 
 def test_config5_constrained_nucleus(ctx, orc):
-    """BASELINE config 5 shape (8 of 256 rows per step, 2 steps): vocab 201088, 5 % grammar mask,
+    """Benchmark configuration 5 shape (8 of 256 rows per step, 2 steps): vocab 201088, 5 % grammar mask,
     T=1.0, top-p 0.95, repetition penalty 1.2 over 1024 ids."""
     rng = np.random.default_rng(5)
     rows, vocab = 8, 201088
