@@ -419,11 +419,13 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool);
   if (tau == 0u) {
     // The pooled bound found fewer than k offers (a short tail chunk keeps its elements in one or two
-    // waves): take the exact k-th best of the 256 per-thread maxima instead.
-    sm.lists[tid] = static_cast<u64>(lmax);
+    // waves): take the exact k-th best of the 512 per-thread maxima instead.
+    static_assert(kSWaves * kWaveListCap >= kSBlock, "the hit lists double as the sort buffer of this path");
+    u64* scratch = sm.wave_list;  // free until the hits are listed
+    scratch[tid] = static_cast<u64>(lmax);
     __syncthreads();
-    block_sort_desc(sm.lists, kSBlock);
-    tau = static_cast<uint32_t>(sm.lists[kk - 1]);
+    block_sort_desc(scratch, kSBlock);
+    tau = static_cast<uint32_t>(scratch[kk - 1]);
     __syncthreads();
   }
   // tau == 0: the chunk has fewer than k elements -- keep them all
