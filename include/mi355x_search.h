@@ -225,7 +225,7 @@ int mi355x_spec_verify(mi355x_search_ctx* ctx, void* stream, const float* p_targ
  *   accepted_len, final_token, engine_draws  device [batch] outputs; engine_draws = 32-bit engine outputs
  *                the reference would have consumed (a categorical draw over fewer than two entries takes
  *                none), so the caller can advance its std::mt19937 by that many.
- * A sequence with a row whose count exceeds its capacity reports accepted_len = final_token = -1.
+ * A sequence with a row whose count exceeds its capacity or is below 1 reports accepted_len = final_token = -1.
  * 1 <= K <= 64. */
 int mi355x_spec_verify_sparse(mi355x_search_ctx* ctx, void* stream, const int32_t* target_count,
                               const int32_t* target_ids, const float* target_probs, int target_capacity,

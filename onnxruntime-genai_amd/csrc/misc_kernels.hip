@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256) void greedy_tail_kernel(int32_t* next_tokens, 
 //           turn until the sample differs from the proposal; sample_u holds the draws in the order rows
 //           with at least two entries consume them.
 //   mode 2  greedy targets: entry 0 of every target row is the row's greedy token.
-// A row whose count exceeds its capacity was truncated by the producer: the sequence reports -1.
+// A row whose count exceeds its capacity (truncated by the producer) or is below 1: the sequence reports -1.
 constexpr int kSpecMaxK = 64;
 
 __device__ __forceinline__ float wave_sparse_prob(const int32_t* ids, const float* probs, int n, int32_t token) {
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(256) void spec_verify_sparse_kernel(const SpecSpars
   if (tid == 0) s_bad = 0;
   __syncthreads();
   for (int r = tid; r <= K; r += 256) {
-    bool bad = tc[r] > a.t_cap || tc[r] < (a.mode == 2 ? 0 : 1);
+    bool bad = tc[r] > a.t_cap || tc[r] < 1;
     if (a.mode == 0 && r < K) bad = bad || a.d_count[static_cast<size_t>(b) * K + r] > a.d_cap;
     if (bad) s_bad = 1;
   }
