@@ -24,6 +24,44 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = 33_510_000  # fetch 33.31 MB + write 0.20 MB per launch
 
 
+def time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, tokens, pool, W, K):
+    """Times the K steps issued round-robin over n_streams streams / contexts in one HIP graph and checks
+    that the tokens equal those of the sequential run already in `tokens`.  Returns milliseconds."""
+    seq_tokens = tokens[W:W + K].clone()
+    tokens[W:W + K].zero_()
+    ctxs = [ctx] + [pkg.SearchContext(ROWS, VOCAB) for _ in range(n_streams - 1)]
+    streams = [side] + [torch.cuda.Stream() for _ in range(n_streams - 1)]
+    for s, c in zip(streams[1:], ctxs[1:]):
+        with torch.cuda.stream(s):
+            c.sample(logits[0], uniforms[0], k=TOP_K, p=TOP_P, temperature=TEMP, out=tokens[0])
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        graph3 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph3, stream=side):
+            for s in streams[1:]:
+                s.wait_stream(side)
+            for i in range(W, W + K):
+                with torch.cuda.stream(streams[i % n_streams]):
+                    ctxs[i % n_streams].sample(logits[i % pool], uniforms[i], k=TOP_K, p=TOP_P, temperature=TEMP,
+                                               out=tokens[i])
+            for s in streams[1:]:
+                side.wait_stream(s)
+        graph3.replay()
+        side.synchronize()
+        start3, end3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start3.record(side)
+        graph3.replay()
+        end3.record(side)
+        side.synchronize()
+    torch.cuda.synchronize()
+    if not torch.equal(tokens[W:W + K], seq_tokens):
+        sys.exit("PARITY FAILURE: tokens differ between the sequential run and the run with several batches in flight")
+    overlapped_ms = start3.elapsed_time(end3)
+    for c in ctxs[1:]:
+        c.close()
+    return overlapped_ms
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -35,6 +73,10 @@ def main():
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
                     help="c2 (default) is the headline configuration; the others time the remaining "
                          "configurations with the same JSON shape")
+    ap.add_argument("--batches-in-flight", type=int, default=3,
+                    help="c2 only: after the timed sequential run, also time the same steps spread over this many "
+                         "streams and contexts (informational field of the JSON line; 0 skips it, which keeps a "
+                         "profiler's per-kernel statistics to the sequential launches)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (rows shard across GPUs "
@@ -110,39 +152,10 @@ def main():
     # `value` measures.  An engine that serves several independent batches can keep one sampling step
     # per batch in flight; the steps then overlap each other's latency-bound tails.  Three contexts on
     # three streams inside one HIP graph, same inputs, tokens required to be identical.
-    n_streams = 3
-    seq_tokens = tokens[W:W + K].clone()
-    tokens[W:W + K].zero_()
-    ctxs = [ctx] + [pkg.SearchContext(ROWS, VOCAB) for _ in range(n_streams - 1)]
-    streams = [side] + [torch.cuda.Stream() for _ in range(n_streams - 1)]
-    for s, c in zip(streams[1:], ctxs[1:]):
-        with torch.cuda.stream(s):
-            c.sample(logits[0], uniforms[0], k=TOP_K, p=TOP_P, temperature=TEMP, out=tokens[0])
-    torch.cuda.synchronize()
-    with torch.cuda.stream(side):
-        graph3 = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph3, stream=side):
-            for s in streams[1:]:
-                s.wait_stream(side)
-            for i in range(W, W + K):
-                with torch.cuda.stream(streams[i % n_streams]):
-                    ctxs[i % n_streams].sample(logits[i % pool], uniforms[i], k=TOP_K, p=TOP_P, temperature=TEMP,
-                                               out=tokens[i])
-            for s in streams[1:]:
-                side.wait_stream(s)
-        graph3.replay()
-        side.synchronize()
-        start3, end3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start3.record(side)
-        graph3.replay()
-        end3.record(side)
-        side.synchronize()
-    torch.cuda.synchronize()
-    if not torch.equal(tokens[W:W + K], seq_tokens):
-        sys.exit("PARITY FAILURE: tokens differ between the sequential run and the run with three batches in flight")
-    overlapped_ms = start3.elapsed_time(end3)
-    for c in ctxs[1:]:
-        c.close()
+    n_streams = args.batches_in_flight
+    overlapped_ms = None
+    if n_streams >= 2:
+        overlapped_ms = time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, tokens, pool, W, K)
 
     ms_per_step = gpu_ms / K
     algo_bytes = ROWS * VOCAB * 4 + ROWS * 8 + ROWS * 4  # logits once + uniforms + tokens
@@ -173,9 +186,9 @@ def main():
                    "rows": ROWS, "vocab": VOCAB, "top_k": TOP_K, "top_p": TOP_P, "temperature": TEMP,
                    "parity": "token ids of %d steps bit-identical to the CPU oracle" % n_cpu,
                    "general_path_rows": fallback,
-                   "independent_batches_in_flight": {
-                       "note": "informational, not `value`: the same steps issued round-robin on 3 streams / 3 "
-                               "contexts in one HIP graph (tokens identical)",
+                   "independent_batches_in_flight": None if overlapped_ms is None else {
+                       "note": "informational, not `value`: the same steps issued round-robin on %d streams / "
+                               "contexts in one HIP graph (tokens identical)" % n_streams,
                        "streams": n_streams, "us_per_step": overlapped_ms / K * 1e3,
                        "tokens_per_s": ROWS * K / (overlapped_ms * 1e-3),
                        "roofline_frac": algo_bytes / (overlapped_ms / K * 1e-3) / 1e9 / HBM_PEAK_GBS}},
