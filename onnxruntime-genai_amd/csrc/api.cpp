@@ -252,6 +252,8 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   ms::SampleArgs a{};
   if (int r = MakeXform(ctx, xf, rows, vocab, s, &a.xf)) return r;
   bool any_nucleus = false;
+  ms::InlineParams table;
+  bool use_table = false;
   auto check = [&](const mi355x_sample_params& p) -> int {
     if (!(p.temperature > 0.0f)) return Fail(MI355X_E_INVALID, "temperature must be positive (got %g)", p.temperature);
     if (p.k <= 1 && vocab > 64) any_nucleus = true;
@@ -260,9 +262,14 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   if (per_row_params) {
     for (int r = 0; r < rows; ++r)
       if (int rc = check(per_row_params[r])) return rc;
-    HIP_TRY(hipMemcpyAsync(ctx->params_dev, per_row_params, sizeof(mi355x_sample_params) * rows,
-                           hipMemcpyHostToDevice, s));
-    a.per_row = ctx->params_dev;
+    if (rows <= ms::kInlineParamRows) {
+      for (int r = 0; r < rows; ++r) table.row[r] = per_row_params[r];
+      use_table = true;
+    } else {
+      HIP_TRY(hipMemcpyAsync(ctx->params_dev, per_row_params, sizeof(mi355x_sample_params) * rows,
+                             hipMemcpyHostToDevice, s));
+      a.per_row = ctx->params_dev;
+    }
   } else {
     if (int rc = check(params)) return rc;
   }
@@ -286,7 +293,7 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
-  HIP_TRY(ms_launch_sample(&a, any_nucleus, s));
+  HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_nucleus, s));
   return MI355X_OK;
 }
 
@@ -333,7 +340,7 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
-  HIP_TRY(ms_launch_sample(&a, false, s));
+  HIP_TRY(ms_launch_sample(&a, nullptr, false, s));
   return MI355X_OK;
 }
 

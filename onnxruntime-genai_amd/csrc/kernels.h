@@ -24,6 +24,14 @@ constexpr int kModeTopkSmall = 0;
 constexpr int kModeNucleus = 1;
 constexpr int kModeGeneral = 2;
 
+// Heterogeneous (k, p, T) of a batch of at most kInlineParamRows rows travel inside the kernel
+// arguments, as a second argument of kernel variants of their own, so that no copy to the device
+// precedes the launch and the kernels of the uniform case keep their small argument block.
+constexpr int kInlineParamRows = 64;
+struct InlineParams {
+  mi355x_sample_params row[kInlineParamRows];
+};
+
 struct SampleArgs {
   const float* logits;
   int64_t row_stride;
@@ -137,7 +145,8 @@ struct ScorerState {
 
 extern "C" {
 hipError_t ms_sample_init();
-hipError_t ms_launch_sample(const ms::SampleArgs* a, bool any_nucleus, hipStream_t stream);
+// `table`, when not null, holds the parameters of rows 0 .. a->rows-1 (a->rows <= kInlineParamRows).
+hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_nucleus, hipStream_t stream);
 hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipStream_t stream);
 hipError_t ms_launch_process_logits(float* logits, int64_t row_stride, int rows, int vocab,
                                     const ms::Xform* xf, hipStream_t stream);

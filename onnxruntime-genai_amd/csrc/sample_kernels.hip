@@ -16,6 +16,27 @@ namespace ms {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// (k, p, T) of a row.  INLINE kernels carry a table as their second argument and read it through the
+// kernel-argument segment itself (constant address space, scalar loads): indexing the by-value
+// argument object with a run-time row would make the compiler copy the whole object to private memory.
+static_assert(sizeof(SampleArgs) % alignof(InlineParams) == 0, "the table follows the first argument without padding");
+template <bool INLINE>
+__device__ __forceinline__ mi355x_sample_params row_params(const SampleArgs& a, int row) {
+  if constexpr (INLINE) {
+    typedef __attribute__((address_space(4))) const char* KernargPtr;
+    const KernargPtr base = (KernargPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    typedef __attribute__((address_space(4))) const mi355x_sample_params* TablePtr;
+    const TablePtr table = (TablePtr)(base + sizeof(SampleArgs));
+    mi355x_sample_params q;
+    q.k = table[row].k;
+    q.p = table[row].p;
+    q.temperature = table[row].temperature;
+    return q;
+  } else {
+    return a.per_row ? a.per_row[row] : a.uniform;
+  }
+}
+
 __device__ __forceinline__ int next_pow2(int v) {
   int p = 64;
   while (p < v) p <<= 1;
@@ -32,7 +53,7 @@ __device__ __forceinline__ RowOutputs row_outputs(const SampleArgs& a, int row) 
 // Exact general path for one row, any (k, p, T), any vocabulary size: rebuilds the processed row as
 // key64s in global scratch, sorts all of it, then runs the reference algorithm on the sorted row.
 // Run by one whole block.  scratch holds next_pow2(vocab) entries.
-__device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* scratch, SeqShared& sh) {
+__device__ __forceinline__ void general_row(const SampleArgs& a, int row, const mi355x_sample_params prm, u64* scratch, SeqShared& sh) {
   const int V = a.vocab;
   const float* lrow = a.logits + static_cast<size_t>(row) * a.row_stride;
   const int n2 = next_pow2(V);
@@ -64,7 +85,6 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, u64* s
     __syncthreads();
   }
   block_sort_desc(scratch, n2);
-  const mi355x_sample_params prm = a.per_row ? a.per_row[row] : a.uniform;
   if (a.emit_topk) {
     const int kk = prm.k < V ? prm.k : V;
     for (int j = threadIdx.x; j < kk; j += blockDim.x) {
@@ -602,10 +622,11 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   return sm.flag == 0u;
 }
 
-__global__ __launch_bounds__(kSBlock) void sample_fused_kernel(const SampleArgs a) {
+template <bool INLINE>
+__device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
   const int row = blockIdx.y, chunk = blockIdx.x;
   __shared__ FusedShared sm;
-  const mi355x_sample_params prm = a.per_row ? a.per_row[row] : a.uniform;
+  const mi355x_sample_params prm = row_params<INLINE>(a, row);
   const int mode = row_mode(prm, a.vocab, a.chunks, a.emit_topk);
   if (mode == kModeGeneral) {
     if (chunk != 0) return;
@@ -615,7 +636,12 @@ __global__ __launch_bounds__(kSBlock) void sample_fused_kernel(const SampleArgs 
   // Rows the fast paths decline end here, in the exact general path (a single inlined call site keeps
   // the argument block in scalar registers instead of a scratch copy).
   __syncthreads();
-  general_row(a, row, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq);
+  general_row(a, row, prm, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq);
+}
+
+__global__ __launch_bounds__(kSBlock) void sample_fused_kernel(const SampleArgs a) { sample_fused_body<false>(a); }
+__global__ __launch_bounds__(kSBlock) void sample_fused_rows_kernel(const SampleArgs a, const InlineParams) {
+  sample_fused_body<true>(a);
 }
 
 // Sorts n keys (kFinishBlock < n <= kNucleusCap) in LDS, descending, by a block of kFinishBlock
@@ -704,7 +730,8 @@ __device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n,
 // Per-row finish of the nucleus path: gathers the candidates the streaming pass left in `big`,
 // sorts them in LDS and runs the exact epilogue.  One block of kFinishBlock threads per row;
 // dynamic LDS: kNucleusCap key64s + the bucket table of the sort.
-__global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const SampleArgs a) {
+template <bool INLINE>
+__device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   extern __shared__ u64 lds_keys[];
   uint32_t* bucket_start = reinterpret_cast<uint32_t*>(lds_keys + kNucleusCap);  // kSortBuckets + 1 entries
   __shared__ SeqShared seqsh;
@@ -714,7 +741,7 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const Samp
   const int row = blockIdx.x;
   const int V = a.vocab;
   const int tid = threadIdx.x;
-  const mi355x_sample_params prm = a.per_row ? a.per_row[row] : a.uniform;
+  const mi355x_sample_params prm = row_params<INLINE>(a, row);
   if (row_mode(prm, V, a.chunks) != kModeNucleus) return;
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
@@ -783,26 +810,43 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const Samp
   }
   if (!ok) {
     __syncthreads();
-    general_row(a, row, big_row, seqsh);
+    general_row(a, row, prm, big_row, seqsh);
   }
+}
+
+__global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const SampleArgs a) { nucleus_finish_body<false>(a); }
+__global__ __launch_bounds__(kFinishBlock) void nucleus_finish_rows_kernel(const SampleArgs a, const InlineParams) {
+  nucleus_finish_body<true>(a);
 }
 
 }  // namespace ms
 
-extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, bool any_nucleus, hipStream_t stream) {
+extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_nucleus,
+                                       hipStream_t stream) {
   dim3 grid(a->chunks, a->rows);
-  hipLaunchKernelGGL(ms::sample_fused_kernel, grid, dim3(ms::kSBlock), 0, stream, *a);
+  if (table) {
+    hipLaunchKernelGGL(ms::sample_fused_rows_kernel, grid, dim3(ms::kSBlock), 0, stream, *a, *table);
+  } else {
+    hipLaunchKernelGGL(ms::sample_fused_kernel, grid, dim3(ms::kSBlock), 0, stream, *a);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   if (any_nucleus) {
-    hipLaunchKernelGGL(ms::nucleus_finish_kernel, dim3(a->rows), dim3(ms::kFinishBlock),
-                       ms::kFinishLds, stream, *a);
+    if (table) {
+      hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, dim3(a->rows), dim3(ms::kFinishBlock), ms::kFinishLds, stream,
+                         *a, *table);
+    } else {
+      hipLaunchKernelGGL(ms::nucleus_finish_kernel, dim3(a->rows), dim3(ms::kFinishBlock), ms::kFinishLds, stream, *a);
+    }
     e = hipGetLastError();
   }
   return e;
 }
 
 extern "C" hipError_t ms_sample_init() {
-  return hipFuncSetAttribute(reinterpret_cast<const void*>(ms::nucleus_finish_kernel),
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ms::nucleus_finish_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, ms::kFinishLds);
+  if (e != hipSuccess) return e;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(ms::nucleus_finish_rows_kernel),
                              hipFuncAttributeMaxDynamicSharedMemorySize, ms::kFinishLds);
 }

@@ -309,14 +309,17 @@ def test_config5_constrained_nucleus(ctx, orc):
             assert tok[r] == idx[orc.discrete_draw(probs, u[r])]
 
 
-def test_sample_heterogeneous_rows(ctx, orc):
-    """BatchedSampler semantics: per-row (k, p, T), greedy = (1, 0, 1)."""
-    say("sample heterogeneous")
+@pytest.mark.parametrize("rows,vocab", [(6, 30000), (64, 40000), (70, 9000)])
+def test_sample_heterogeneous_rows(ctx, orc, rows, vocab):
+    """BatchedSampler semantics: per-row (k, p, T), greedy = (1, 0, 1).  Up to 64 rows the parameters
+    travel inside the kernel arguments, above that through a table on the device: both sides of that edge."""
+    say("sample heterogeneous", rows, vocab)
     rng = np.random.default_rng(6)
-    rows, vocab = 6, 30000
     x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
     u = rng.random(rows)
-    params = [(1, 0.0, 1.0), (50, 0.9, 0.7), (0, 0.9, 1.0), (8, 1.0, 1.5), (-1, 0.5, 0.8), (100, 0.0, 1.0)]
+    kinds = [(1, 0.0, 1.0), (50, 0.9, 0.7), (0, 0.9, 1.0), (8, 1.0, 1.5), (-1, 0.5, 0.8), (100, 0.0, 1.0)]
+    params = [kinds[(r * 5 + r // 6) % 6] for r in range(rows)]
+    params[0] = kinds[0]
     tok = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), per_row=params).cpu().numpy()
     for r, (k, p, t) in enumerate(params):
         assert tok[r] == orc.sample_row(x[r], k, p, t, u[r]), r
