@@ -120,7 +120,9 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
  * SampleCategoricalToken (src/sampling_distribution.h:218-297), and BatchedSampler::Sample
  * (src/smartptrs.h:134-137).
  *   params            used for every row when per_row_params is NULL.
- *   per_row_params    HOST [rows], heterogeneous parameters (copied by the call).
+ *   per_row_params    HOST [rows], heterogeneous parameters (copied by the call: up to 64 rows travel
+ *                     inside the kernel arguments, larger batches through one asynchronous copy to a
+ *                     table in the context).
  *   uniforms          device [rows] doubles in [0,1): row r's categorical draw, the value
  *                     std::discrete_distribution would take from generate_canonical<double,53>.
  *                     A row whose kept set has one token ignores its uniform.
