@@ -251,12 +251,15 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   hipStream_t s = static_cast<hipStream_t>(stream);
   ms::SampleArgs a{};
   if (int r = MakeXform(ctx, xf, rows, vocab, s, &a.xf)) return r;
-  bool any_nucleus = false;
+  bool any_nucleus = false, any_other = false;
+  const int chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
   ms::InlineParams table;
   bool use_table = false;
   auto check = [&](const mi355x_sample_params& p) -> int {
     if (!(p.temperature > 0.0f)) return Fail(MI355X_E_INVALID, "temperature must be positive (got %g)", p.temperature);
+    // the kernels' own rule (row_mode) decides; these flags only have to cover it
     if (p.k <= 1 && vocab > 64) any_nucleus = true;
+    if (!(p.k <= 1 && vocab > 64 && chunks * ms::kSmallCap <= ms::kAllCap)) any_other = true;
     return MI355X_OK;
   };
   if (per_row_params) {
@@ -277,7 +280,7 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   a.row_stride = row_stride;
   a.rows = rows;
   a.vocab = vocab;
-  a.chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
+  a.chunks = chunks;
   a.uniform = params;
   a.uniforms = uniforms;
   a.out_tokens = out_tokens;
@@ -293,7 +296,7 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
-  HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_nucleus, s));
+  HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_other, any_nucleus, s));
   return MI355X_OK;
 }
 
@@ -340,7 +343,7 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
-  HIP_TRY(ms_launch_sample(&a, nullptr, false, s));
+  HIP_TRY(ms_launch_sample(&a, nullptr, true, false, s));
   return MI355X_OK;
 }
 

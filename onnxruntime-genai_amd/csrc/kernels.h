@@ -146,7 +146,9 @@ struct ScorerState {
 extern "C" {
 hipError_t ms_sample_init();
 // `table`, when not null, holds the parameters of rows 0 .. a->rows-1 (a->rows <= kInlineParamRows).
-hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_nucleus, hipStream_t stream);
+// any_nucleus: some row may be in nucleus mode; any_other: some row may be in another mode.
+hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_other, bool any_nucleus,
+                            hipStream_t stream);
 hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipStream_t stream);
 hipError_t ms_launch_process_logits(float* logits, int64_t row_stride, int rows, int vocab,
                                     const ms::Xform* xf, hipStream_t stream);

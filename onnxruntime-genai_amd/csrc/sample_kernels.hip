@@ -28,9 +28,9 @@ __device__ __forceinline__ mi355x_sample_params row_params(const SampleArgs& a, 
     typedef __attribute__((address_space(4))) const mi355x_sample_params* TablePtr;
     const TablePtr table = (TablePtr)(base + sizeof(SampleArgs));
     mi355x_sample_params q;
-    q.k = table[row].k;
-    q.p = table[row].p;
-    q.temperature = table[row].temperature;
+    q.k = __builtin_amdgcn_readfirstlane(table[row].k);
+    q.p = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(table[row].p)));
+    q.temperature = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(table[row].temperature)));
     return q;
   } else {
     return a.per_row ? a.per_row[row] : a.uniform;
@@ -128,6 +128,8 @@ constexpr u64 kSlotEmpty = 1, kSlotOverflow = 2;
 // the exact path compute the row.
 constexpr int kSpinLimit = 1 << 21;
 constexpr int kWaveListCap = 128;  // hits one wave can list per chunk
+constexpr int kExtraCap = 2048;    // distinct history ids one chunk can hold; beyond, the row takes the exact path
+constexpr uint32_t kChunkCntOverflow = 0xffffffffu;  // chunk_cnt of a nucleus chunk that gave up
 
 // LDS of the fused kernel.
 struct FusedShared {
@@ -141,6 +143,9 @@ struct FusedShared {
   uint32_t wave_val[kSWaves];
   u64 wave_val64[kSWaves];
   uint32_t count, flag;
+  uint32_t n_extra;
+  float extra_val[kExtraCap];     // processed logits of the history ids of this chunk ...
+  uint32_t extra_idx[kExtraCap];  // ... and their ids
   SeqShared seq;
 };
 
@@ -276,10 +281,62 @@ __device__ const uint64_t g_exp2_tab[32] = {
     0x3fef5818dcfba487ULL, 0x3fef7c97337b9b5fULL, 0x3fefa4afa2a490daULL, 0x3fefd0765b6e4540ULL,
 };
 
+// Workgroup barrier that orders LDS accesses only: unlike __syncthreads() it does not wait for the
+// global loads still in flight.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// block_max with barriers that do not wait for global memory.
+template <typename T>
+__device__ __forceinline__ T block_max_lds(T v, T* scratch) {
+  v = wave_max(v);
+  const int lane = lane_id(), wave = threadIdx.x >> 6;
+  if (lane == 0) scratch[wave] = v;
+  lds_barrier();
+  T r = scratch[0];
+#pragma unroll
+  for (int w = 1; w < kSWaves; ++w) r = scratch[w] > r ? scratch[w] : r;
+  lds_barrier();
+  return r;
+}
+
+// Applies the two LDS bitmaps of a chunk to the registers of a thread: an id whose bit in `allowed` is
+// clear becomes kLowest, an id whose bit in `history` is set becomes NaN (its processed value lives in
+// the extras list).  Branch-free: the bit, spread over a word, selects between the two bit patterns.
+template <bool ALLOWED, bool HISTORY>
+__device__ __forceinline__ void mask_registers(float (&v)[kSElems], const uint32_t* allowed, const uint32_t* history,
+                                               int tid) {
+#pragma unroll
+  for (int j = 0; j < kSVec; ++j) {
+    const int rel0 = (j * kSBlock + tid) * 4;
+    const uint32_t anib = ALLOWED ? allowed[rel0 >> 5] >> (rel0 & 31) : 0u;
+    const uint32_t hnib = HISTORY ? history[rel0 >> 5] >> (rel0 & 31) : 0u;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      uint32_t x = __float_as_uint(v[j * 4 + c]);
+      if (ALLOWED) {
+        uint32_t keep = static_cast<uint32_t>(static_cast<int32_t>(anib << (31 - c)) >> 31);
+        asm volatile("" : "+v"(keep));  // stays a bitwise select (one instruction) instead of compare + select
+        x = (x & keep) | (0xff7fffffu & ~keep);  // bits of kLowest
+      }
+      if (HISTORY) {
+        const uint32_t drop = static_cast<uint32_t>(static_cast<int32_t>(hnib << (31 - c)) >> 31);
+        x |= drop;  // all ones is a NaN
+      }
+      v[j * 4 + c] = __uint_as_float(x);
+    }
+    if ((j & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most eight bitmap words in registers at a time
+  }
+}
+
 // Streaming pass of one (row, chunk) of a top-k<=64 or nucleus row.  Returns true when this workgroup
 // must run the general path for the row (it was the last to arrive and the fast path declined).
+template <bool NUCLEUS, bool XFORM>
 __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chunk, mi355x_sample_params prm,
-                                           int mode, FusedShared& sm) {
+                                           FusedShared& sm) {
   const int V = a.vocab;
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
@@ -313,56 +370,82 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
                               arg_now(a.kept_ids),
                               arg_now(a.kept_probs),
                               arg_now(a.kept_capacity)};
-  if (a.xf.active()) {
-    // The chunk's grammar-mask words and the bitmap of history ids are staged in LDS once; a thread
-    // then needs one nibble of each per float4.
-    const bool pen = a.xf.use_penalty();
-    const bool has_mask = a.xf.mask != nullptr;
-    if (pen)
-      for (int i = tid; i < kSChunk / 32; i += kSBlock) sm.hist_bits[i] = 0u;
+  // ---- logits processing ----------------------------------------------------------------------
+  // Grammar mask and min-length masking reach the registers as one LDS bitmap of allowed ids (a clear
+  // bit -> kLowest; ids past the vocabulary count as allowed and keep their NaN).  The ids of the row's
+  // history are few and their processing (a correctly rounded division, the n-gram ban) is long, so
+  // they leave the register arrays altogether: a second bitmap turns them into NaN there, and the
+  // threads that marked them compute their processed values into a short list in LDS, `extras`, which
+  // every later phase visits next to the registers.
+  // The bitmap words and the first history ids of this thread are requested before anything waits.
+  static_assert(kSChunk / 32 == 2 * kSBlock, "two bitmap words per thread");
+  const bool active = XFORM && a.xf.active();  // kernels without logits processing carry none of its code
+  const bool pen = active && a.xf.use_penalty();
+  const bool has_mask = active && a.xf.mask != nullptr;
+  const int words = (V - 1) / 32 + 1;
+  const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * words : nullptr;
+  const int32_t* hist = pen ? a.xf.history + static_cast<size_t>(row) * a.xf.history_stride : nullptr;
+  const bool hist_ahead = pen && a.xf.history_lens == nullptr;  // the length is known without a load
+  int hist_pre[2] = {-1, -1};
+  uint32_t mask_pre[2] = {~0u, ~0u};
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    if (hist_ahead && tid + q * kSBlock < a.xf.history_len) hist_pre[q] = hist[tid + q * kSBlock];
     if (has_mask) {
-      const int words = (V - 1) / 32 + 1;
-      const uint32_t* mrow = a.xf.mask + static_cast<size_t>(row) * words;
-      for (int i = tid; i < kSChunk / 32; i += kSBlock) {
-        const int w = chunk * (kSChunk / 32) + i;
-        sm.mask_bits[i] = w < words ? mrow[w] : 0u;
-      }
+      const int w = chunk * (kSChunk / 32) + tid + q * kSBlock;
+      mask_pre[q] = w < words ? mrow[w] : 0u;
     }
-    __syncthreads();
-    if (pen) {
-      const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
-      const int hlen = a.xf.hist_len(row);
-      for (int i = tid; i < hlen; i += kSBlock) {
-        const int rel = h[i] - chunk * kSChunk;
-        if (rel >= 0 && rel < kSChunk) atomicOr(&sm.hist_bits[rel >> 5], 1u << (rel & 31));
-      }
-      __syncthreads();
-    }
-    const float penalty = a.xf.penalty;
+  }
+  uint32_t n_extra = 0u;
+  bool extra_overflow = false;
+  if (XFORM && active) {
     const int n_eos = a.xf.eos_count(row);
-    const uint32_t* ban_row = a.xf.ban_row(row, V);
+    if (tid == 0) sm.n_extra = 0u;
 #pragma unroll
-    for (int j = 0; j < kSVec; ++j) {
-      const int rel0 = (j * kSBlock + tid) * 4;
-      const uint32_t mnib = has_mask ? (sm.mask_bits[rel0 >> 5] >> (rel0 & 31)) & 15u : 15u;
-      const uint32_t hnib = pen ? (sm.hist_bits[rel0 >> 5] >> (rel0 & 31)) & 15u : 0u;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const int idx = chunk * kSChunk + rel0 + c;
-        float x = v[j * 4 + c];
-        if (idx < V) {
-          // the reference's order: mask -> min-length -> repetition penalty
-          if (!((mnib >> c) & 1u)) x = kLowest;
-          for (int e = 0; e < n_eos; ++e)
-            if (a.xf.eos[e] == idx) x = kLowest;
-          if ((hnib >> c) & 1u) {
-            x = x < 0.0f ? x * penalty : x / penalty;
-            if (ban_row && ((ban_row[idx >> 5] >> (idx & 31)) & 1u)) x = kLowest;  // no-repeat-n-gram ban
+    for (int q = 0; q < 2; ++q) {
+      const int i = tid + q * kSBlock;
+      const int w = chunk * (kSChunk / 32) + i;
+      uint32_t word = mask_pre[q];
+      for (int e = 0; e < n_eos; ++e)
+        if ((a.xf.eos[e] >> 5) == w) word &= ~(1u << (a.xf.eos[e] & 31));
+      const int n_real = V - w * 32;  // ids of this word inside the vocabulary
+      if (n_real < 32) word |= n_real <= 0 ? ~0u : (~0u << n_real);
+      sm.mask_bits[i] = word;
+      sm.hist_bits[i] = 0u;
+    }
+    lds_barrier();
+    if (pen) {
+      const int hlen = a.xf.hist_len(row);
+      const float penalty = a.xf.penalty;
+      const uint32_t* ban_row = a.xf.ban_row(row, V);
+      // the thread that is first to mark an id computes its processed value
+      auto visit = [&](int id) {
+        const int rel = id - chunk * kSChunk;
+        if (rel >= 0 && rel < kSChunk && id < V) {
+          const uint32_t bit = 1u << (rel & 31);
+          if (!(atomicOr(&sm.hist_bits[rel >> 5], bit) & bit)) {
+            const uint32_t slot = atomicAdd(&sm.n_extra, 1u);
+            if (slot < static_cast<uint32_t>(kExtraCap)) {
+              const uint32_t mw = has_mask ? mrow[id >> 5] : 0u;
+              sm.extra_val[slot] = xform_value(lrow[id], penalty, a.xf.eos, id, mw, has_mask, true, n_eos, ban_row);
+              sm.extra_idx[slot] = static_cast<uint32_t>(id);
+            }
           }
         }
-        v[j * 4 + c] = x;
+      };
+      int first = tid;
+      if (hist_ahead) {
+        if (tid < hlen) visit(hist_pre[0]);
+        if (tid + kSBlock < hlen) visit(hist_pre[1]);
+        first = tid + 2 * kSBlock;
       }
+      for (int i = first; i < hlen; i += kSBlock) visit(hist[i]);
+      lds_barrier();
+      n_extra = sm.n_extra;
+      extra_overflow = n_extra > static_cast<uint32_t>(kExtraCap);  // the row takes the exact path
+      if (extra_overflow) n_extra = 0u;
     }
+    mask_registers<true, true>(v, sm.mask_bits, sm.hist_bits, tid);
   }
   // per-thread maximum in the float domain (fmaxf skips NaN), keeping the maximum of every float4
   float qm[kSVec];
@@ -372,54 +455,102 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     qm[j] = fmaxf(fmaxf(v[j * 4], v[j * 4 + 1]), fmaxf(v[j * 4 + 2], v[j * 4 + 3]));
     fm = fmaxf(fm, qm[j]);
   }
-  const uint32_t lmax = elem_index(chunk, 0, 0) < V ? order_key(fm) : 0u;  // 0: thread holds no element
+  for (uint32_t i = tid; i < n_extra; i += kSBlock) fm = fmaxf(fm, sm.extra_val[i]);
+  // 0: the thread holds no element
+  const uint32_t lmax = (elem_index(chunk, 0, 0) < V || static_cast<uint32_t>(tid) < n_extra) ? order_key(fm) : 0u;
   if (tid == 0) sm.count = 0u;
 
-  if (mode == kModeNucleus) {
-    // Everything within nucleus_depth of the chunk maximum goes to the row's key buffer.  Slots come
-    // from a prefix sum over per-thread counts (one barrier), not from per-element atomics.
+  if constexpr (NUCLEUS) {
+    // Everything within nucleus_depth of the chunk maximum goes to the row's key buffer, in no
+    // particular order (the finish kernel sorts).  A wave counts its candidates, reserves a range of
+    // the chunk's list with one LDS atomic and fills it; the slot of a candidate is the wave's running
+    // count plus the number of candidate lanes below.
     const uint32_t cmax = block_max<uint32_t>(lmax, sm.wave_val);
     float thr = -__builtin_inff();
     if (cmax != 0u) thr = key_to_float(cmax) - nucleus_depth(prm, V);
-    uint32_t cnt = 0u;
-    float fb = -__builtin_inff();  // best element below the threshold (first of equals) ...
-    int fi = -1;                   // ... and its id
+    // First pass: the wave's number of candidates.
+    uint32_t wcnt = 0u;
+#pragma unroll
+    for (int e = 0; e < kSElems; ++e) wcnt += static_cast<uint32_t>(__popcll(__ballot(v[e] >= thr)));  // false for NaN
+    for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
+      const uint32_t i = i0 + tid;
+      wcnt += static_cast<uint32_t>(__popcll(__ballot(i < n_extra && sm.extra_val[i] >= thr)));
+    }
+    uint32_t woff = 0u;
+    if (lane == 0) woff = atomicAdd(&sm.count, wcnt);
+    woff = __builtin_amdgcn_readfirstlane(woff);
+    // Second pass: the stores.  The list holds (raw float bits, ~id): the finish kernel turns the bits
+    // into order keys.  The compares are made afresh against a copy of the threshold the compiler
+    // cannot identify with the first one, so that the 64 lane masks of the first pass need not stay
+    // alive.  Nothing below waits for the stores.
+    char* const dst = reinterpret_cast<char*>(big_row + static_cast<size_t>(chunk) * kSChunk);
+    float thr2 = thr;
+    asm volatile("" : "+v"(thr2));
+    const uint32_t nid0 = ~static_cast<uint32_t>(elem_index(chunk, 0, 0));  // ~(id0 + d) = ~id0 - d
 #pragma unroll
     for (int e = 0; e < kSElems; ++e) {
-      const bool cand = v[e] >= thr;  // false for NaN and for ids >= vocab
-      cnt += cand ? 1u : 0u;
-      const float nb = v[e] < thr ? v[e] : -__builtin_inff();
-      if (nb > fb || (fi < 0 && v[e] < thr)) {
-        fb = nb;
-        fi = elem_index(chunk, e / 4, e % 4);
+      const bool cand = v[e] >= thr2;
+      const u64 b = __ballot(cand);
+      if (cand) {
+        const uint32_t pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
+                                                       __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), woff));
+        const uint32_t nid = nid0 - static_cast<uint32_t>((e / 4) * kSBlock * 4 + (e % 4));
+        *reinterpret_cast<u64*>(dst + pos * 8u) = make_key64(__float_as_uint(v[e]), ~nid);
       }
+      woff += static_cast<uint32_t>(__popcll(b));
+      __builtin_amdgcn_sched_barrier(0);  // keeps the keys of later elements from being built early
     }
-    uint32_t inc = cnt;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const uint32_t y = __shfl_up(inc, d, 64);
-      if (lane >= d) inc += y;
+    u64 extra_below = 0;  // the best of this thread's extras below the threshold, as a whole key
+    for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
+      const uint32_t i = i0 + tid;
+      const float ev = i < n_extra ? sm.extra_val[i] : kNaN;
+      const uint32_t ei = i < n_extra ? sm.extra_idx[i] : 0u;
+      const bool cand = ev >= thr2;
+      const u64 b = __ballot(cand);
+      if (cand) {
+        const uint32_t pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
+                                                       __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), woff));
+        *reinterpret_cast<u64*>(dst + pos * 8u) = make_key64(__float_as_uint(ev), ei);
+      }
+      woff += static_cast<uint32_t>(__popcll(b));
+      const u64 key = make_key64(order_key(ev), ei);
+      if (ev < thr2 && key > extra_below) extra_below = key;
     }
-    if (lane == 63) sm.wave_val[wave] = inc;
-    u64 best_below = fi >= 0 ? make_key64(order_key(fb), static_cast<uint32_t>(fi)) : 0;
-    best_below = block_max<u64>(best_below, sm.wave_val64);  // its barriers also publish wave_val
-    uint32_t pos = inc - cnt, total = 0u;
-#pragma unroll
-    for (int w = 0; w < kSWaves; ++w) {
-      if (w < wave) pos += sm.wave_val[w];
-      total += sm.wave_val[w];
-    }
-    u64* dst = big_row + static_cast<size_t>(chunk) * kSChunk;
+    // The best element below the threshold, first of equals: the block agrees on the best score, then
+    // the few threads that hold it look up its lowest id.
+    float thr3 = thr;
+    asm volatile("" : "+v"(thr3));
+    float fb = -__builtin_inff();
 #pragma unroll
     for (int e = 0; e < kSElems; ++e) {
-      if (v[e] >= thr) {
-        dst[pos] = make_key64(order_key(v[e]), static_cast<uint32_t>(elem_index(chunk, e / 4, e % 4)));
-        ++pos;
-      }
+      if (v[e] < thr3 && v[e] > fb) fb = v[e];  // compares are false for NaN
+      __builtin_amdgcn_sched_barrier(0);        // each lane mask is used at once
     }
+    uint32_t fbk = 0u;  // 0: the thread has no element below the threshold
+    if (fb > -__builtin_inff()) {
+      fbk = order_key(fb);
+    } else if (thr3 > -__builtin_inff()) {  // an element equal to -inf is one, too
+      bool any = false;
+#pragma unroll
+      for (int e = 0; e < kSElems; ++e) any = any || v[e] == -__builtin_inff();
+      if (any) fbk = order_key(-__builtin_inff());
+    }
+    const uint32_t ebk = key64_okey(extra_below);
+    const uint32_t bbk = block_max_lds<uint32_t>(fbk > ebk ? fbk : ebk, sm.wave_val);
+    u64 best_below = ebk == bbk ? extra_below : 0;
+    if (bbk != 0u && fbk == bbk) {
+      const float bbf = key_to_float(bbk);
+      int fe = 0;
+#pragma unroll
+      for (int e = kSElems - 1; e >= 0; --e)
+        if (v[e] == bbf) fe = e;
+      const u64 key = make_key64(bbk, static_cast<uint32_t>(elem_index(chunk, fe >> 2, fe & 3)));
+      best_below = key > best_below ? key : best_below;
+    }
+    best_below = block_max_lds<u64>(best_below, sm.wave_val64);  // its barriers also order the atomics on sm.count
     if (tid == 0) {
       const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
-      a.chunk_cnt[ci] = total;
+      a.chunk_cnt[ci] = extra_overflow ? kChunkCntOverflow : sm.count;
       a.chunk_max[ci] = cmax;
       a.chunk_next[ci] = best_below;
     }
@@ -433,7 +564,8 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   const int kk = prm.k < V ? prm.k : V;
   int n_valid = V - chunk * kSChunk;
   if (n_valid > kSChunk) n_valid = kSChunk;
-  const int n_lanes = n_valid >= 4 * kSBlock ? kSBlock : (n_valid + 3) / 4;
+  int n_lanes = n_valid >= 4 * kSBlock ? kSBlock : (n_valid + 3) / 4;  // threads that hold elements
+  if (static_cast<uint32_t>(n_lanes) < n_extra) n_lanes = n_extra < static_cast<uint32_t>(kSBlock) ? static_cast<int>(n_extra) : kSBlock;
   const size_t ci = static_cast<size_t>(row) * n_chunks + chunk;
   u64* dst = cand_small + ci * kSmallCap;
   uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool);
@@ -475,6 +607,18 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
       }
     }
   }
+  for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
+    const uint32_t i = i0 + tid;
+    const float ev = i < n_extra ? sm.extra_val[i] : kNaN;
+    const bool hit = ev >= tau_f;
+    const u64 b = __ballot(hit);
+    if (hit) {
+      const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
+                                                            __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), 0u));
+      if (pos < kWaveListCap) sm.wave_list[wave * kWaveListCap + pos] = make_key64(__float_as_uint(ev), sm.extra_idx[i]);
+    }
+    woff += static_cast<uint32_t>(__popcll(b));
+  }
   if (lane == 0) sm.wave_val[wave] = woff;
   __syncthreads();
   // The chunk's best 64 candidates, sorted (best first): nothing ranked lower inside its own chunk can
@@ -488,7 +632,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   // workgroups that are running or done.
   uint32_t n_c = 0u;
   uint32_t cnt[kSWaves];
-  bool overflow = false;
+  bool overflow = extra_overflow;
 #pragma unroll
   for (int w = 0; w < kSWaves; ++w) {
     cnt[w] = sm.wave_val[w];
@@ -622,27 +766,45 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   return sm.flag == 0u;
 }
 
-template <bool INLINE>
+// Rows in nucleus mode and all other rows are streamed by kernels of their own (a launch may need
+// both): each kernel holds the code of its mode only, and a change to one path leaves the machine
+// code of the other as it was.
+template <bool INLINE, bool NUCLEUS, bool XFORM>
 __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
   const int row = blockIdx.y, chunk = blockIdx.x;
   __shared__ FusedShared sm;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
   const int mode = row_mode(prm, a.vocab, a.chunks, a.emit_topk);
-  if (mode == kModeGeneral) {
-    if (chunk != 0) return;
-  } else if (!stream_row(a, row, chunk, prm, mode, sm)) {
-    return;
+  if constexpr (NUCLEUS) {
+    if (mode == kModeNucleus) stream_row<true, XFORM>(a, row, chunk, prm, sm);
+  } else {
+    if (mode == kModeNucleus) return;
+    if (mode == kModeGeneral) {
+      if (chunk != 0) return;
+    } else if (!stream_row<false, XFORM>(a, row, chunk, prm, sm)) {
+      return;
+    }
+    // Rows the fast paths decline end here, in the exact general path (a single inlined call site keeps
+    // the argument block in scalar registers instead of a scratch copy).
+    __syncthreads();
+    general_row(a, row, prm, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq);
   }
-  // Rows the fast paths decline end here, in the exact general path (a single inlined call site keeps
-  // the argument block in scalar registers instead of a scratch copy).
-  __syncthreads();
-  general_row(a, row, prm, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq);
 }
 
-__global__ __launch_bounds__(kSBlock) void sample_fused_kernel(const SampleArgs a) { sample_fused_body<false>(a); }
-__global__ __launch_bounds__(kSBlock) void sample_fused_rows_kernel(const SampleArgs a, const InlineParams) {
-  sample_fused_body<true>(a);
-}
+// Kernel variants: per-row parameter table in the arguments or not (_rows), nucleus rows or all other
+// rows, with or without the code of the logits processing (_xf).
+#define MS_STREAM_KERNEL(NAME, NUCLEUS, XFORM)                                                                      \
+  __global__ __launch_bounds__(kSBlock) void NAME##_kernel(const SampleArgs a) {                                    \
+    sample_fused_body<false, NUCLEUS, XFORM>(a);                                                                    \
+  }                                                                                                                 \
+  __global__ __launch_bounds__(kSBlock) void NAME##_rows_kernel(const SampleArgs a, const InlineParams) {           \
+    sample_fused_body<true, NUCLEUS, XFORM>(a);                                                                     \
+  }
+MS_STREAM_KERNEL(sample_fused, false, false)
+MS_STREAM_KERNEL(sample_fused_xf, false, true)
+MS_STREAM_KERNEL(nucleus_stream, true, false)
+MS_STREAM_KERNEL(nucleus_stream_xf, true, true)
+#undef MS_STREAM_KERNEL
 
 // Sorts n keys (kFinishBlock < n <= kNucleusCap) in LDS, descending, by a block of kFinishBlock
 // threads: a counting pass over kSortBuckets buckets that are linear in the score (bucket 0 holds the
@@ -746,19 +908,27 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
   uint32_t m = 0u;
-  for (int c = tid; c < a.chunks; c += blockDim.x) m = a.chunk_max[cbase + c] > m ? a.chunk_max[cbase + c] : m;
+  for (int c = tid; c < a.chunks; c += blockDim.x) {
+    m = a.chunk_max[cbase + c] > m ? a.chunk_max[cbase + c] : m;
+    if (a.chunk_cnt[cbase + c] == kChunkCntOverflow) m = 0xffffffffu;  // above every key: the exact path
+  }
   if (tid == 0) sh_count = 0u;
   const uint32_t rmax = block_max<uint32_t>(m, red32);
+  const bool gave_up = rmax == 0xffffffffu;
   uint32_t thr = 0u;
   if (rmax != 0u) thr = order_key(key_to_float(rmax) - nucleus_depth(prm, V));
   u64 best_below = 0;
   for (int c = tid; c < a.chunks; c += blockDim.x) best_below = a.chunk_next[cbase + c] > best_below ? a.chunk_next[cbase + c] : best_below;
   for (int c = 0; c < a.chunks; ++c) {
-    const uint32_t cnt = a.chunk_cnt[cbase + c];
+    const uint32_t cnt = gave_up ? 0u : a.chunk_cnt[cbase + c];
     const u64* src = big_row + static_cast<size_t>(c) * kSChunk;
     for (uint32_t i0 = 0; i0 < cnt; i0 += blockDim.x) {
       const uint32_t i = i0 + tid;
-      const u64 k64 = i < cnt ? src[i] : 0;
+      u64 k64 = 0;
+      if (i < cnt) {  // the list holds raw float bits in the score half
+        const u64 raw = src[i];
+        k64 = (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw >> 32)))) << 32) | (raw & 0xffffffffull);
+      }
       const bool cand = i < cnt && key64_okey(k64) >= thr;
       const uint32_t pos = wave_slot(cand, &sh_count);
       if (cand) {
@@ -770,7 +940,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   }
   best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
   uint32_t n_c = sh_count;
-  bool ok = n_c < kNucleusCap;  // room for the next-best element too
+  bool ok = !gave_up && n_c < kNucleusCap;  // room for the next-best element too
   if (ok) {
     if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
     if (best_below != 0) n_c += 1;
@@ -821,21 +991,31 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_rows_kernel(const
 
 }  // namespace ms
 
-extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_nucleus,
-                                       hipStream_t stream) {
-  dim3 grid(a->chunks, a->rows);
-  if (table) {
-    hipLaunchKernelGGL(ms::sample_fused_rows_kernel, grid, dim3(ms::kSBlock), 0, stream, *a, *table);
-  } else {
-    hipLaunchKernelGGL(ms::sample_fused_kernel, grid, dim3(ms::kSBlock), 0, stream, *a);
+extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_other,
+                                       bool any_nucleus, hipStream_t stream) {
+  const dim3 grid(a->chunks, a->rows), block(ms::kSBlock);
+  const bool xf = a->xf.active();
+  hipError_t e = hipSuccess;
+  if (any_other) {
+    if (table) {
+      if (xf) hipLaunchKernelGGL(ms::sample_fused_xf_rows_kernel, grid, block, 0, stream, *a, *table);
+      else hipLaunchKernelGGL(ms::sample_fused_rows_kernel, grid, block, 0, stream, *a, *table);
+    } else {
+      if (xf) hipLaunchKernelGGL(ms::sample_fused_xf_kernel, grid, block, 0, stream, *a);
+      else hipLaunchKernelGGL(ms::sample_fused_kernel, grid, block, 0, stream, *a);
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
   }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
   if (any_nucleus) {
     if (table) {
+      if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_rows_kernel, grid, block, 0, stream, *a, *table);
+      else hipLaunchKernelGGL(ms::nucleus_stream_rows_kernel, grid, block, 0, stream, *a, *table);
       hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, dim3(a->rows), dim3(ms::kFinishBlock), ms::kFinishLds, stream,
                          *a, *table);
     } else {
+      if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_kernel, grid, block, 0, stream, *a);
+      else hipLaunchKernelGGL(ms::nucleus_stream_kernel, grid, block, 0, stream, *a);
       hipLaunchKernelGGL(ms::nucleus_finish_kernel, dim3(a->rows), dim3(ms::kFinishBlock), ms::kFinishLds, stream, *a);
     }
     e = hipGetLastError();
