@@ -9,11 +9,10 @@ namespace ms {
 // Many logits per lane keep the per-wave selection overhead small against the streaming work, few
 // chunks per row keep the finishing merge shallow (a 128K vocabulary is four sorted lists, two merge
 // levels), and thread t's float4s (t, t+512, t+1024, ...) make every wave an even sample of the chunk.
-constexpr int kSBlock = 512;
-constexpr int kSWaves = kSBlock / 64;
-constexpr int kSVec = 16;                   // 128-bit loads per thread
-constexpr int kSElems = kSVec * 4;          // logits held in registers per thread
-constexpr int kSChunk = kSBlock * kSElems;  // logits per workgroup
+constexpr int kSChunk = 32768;        // logits per workgroup of the streaming kernels
+constexpr int kTopkBlock = 512;       // threads of a workgroup that streams a top-k row (16 128-bit loads each) ...
+constexpr int kNucleusBlock = 1024;   // ... and a nucleus row (8 each: lighter threads, twice the waves in flight)
+constexpr int kSMaxWaves = 16;
 constexpr int kSmallCap = 64;        // sorted candidates a chunk publishes on the k<=64 path
 constexpr int kListCap = 128;        // candidates a chunk can hold before its sort
 constexpr int kAllCap = 1024;        // slots a finishing workgroup ranks (16 chunks x kSmallCap)

@@ -135,13 +135,13 @@ constexpr uint32_t kChunkCntOverflow = 0xffffffffu;  // chunk_cnt of a nucleus c
 struct FusedShared {
   uint32_t hist_bits[kSChunk / 32];
   uint32_t mask_bits[kSChunk / 32];
-  u64 wave_list[kSWaves * kWaveListCap];  // each wave's hits of this chunk, before the sort
+  u64 wave_list[kSMaxWaves * kWaveListCap];  // each wave's hits of this chunk, before the sort
   u64 list_hi[64];          // second half of a long list, sorted ascending
   u64 own[64];              // the finishing workgroup's own list
   u64 lists[kAllCap / 4];   // first-level results of the finishing workgroup's merge (rows of > 4 chunks)
   uint32_t pool[64];
-  uint32_t wave_val[kSWaves];
-  u64 wave_val64[kSWaves];
+  uint32_t wave_val[kSMaxWaves];
+  u64 wave_val64[kSMaxWaves];
   uint32_t count, flag;
   uint32_t n_extra;
   float extra_val[kExtraCap];     // processed logits of the history ids of this chunk ...
@@ -149,8 +149,9 @@ struct FusedShared {
   SeqShared seq;
 };
 
+template <int BLOCK>
 __device__ __forceinline__ int elem_index(int chunk, int j, int c) {
-  return chunk * kSChunk + (j * kSBlock + static_cast<int>(threadIdx.x)) * 4 + c;
+  return chunk * kSChunk + (j * BLOCK + static_cast<int>(threadIdx.x)) * 4 + c;
 }
 
 // The 32-entry table of expf_core, one entry per lane (lane & 31), fetched by lane shuffle.
@@ -290,7 +291,7 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 // block_max with barriers that do not wait for global memory.
-template <typename T>
+template <int kSWaves, typename T>
 __device__ __forceinline__ T block_max_lds(T v, T* scratch) {
   v = wave_max(v);
   const int lane = lane_id(), wave = threadIdx.x >> 6;
@@ -306,9 +307,10 @@ __device__ __forceinline__ T block_max_lds(T v, T* scratch) {
 // Applies the two LDS bitmaps of a chunk to the registers of a thread: an id whose bit in `allowed` is
 // clear becomes kLowest, an id whose bit in `history` is set becomes NaN (its processed value lives in
 // the extras list).  Branch-free: the bit, spread over a word, selects between the two bit patterns.
-template <bool ALLOWED, bool HISTORY>
-__device__ __forceinline__ void mask_registers(float (&v)[kSElems], const uint32_t* allowed, const uint32_t* history,
-                                               int tid) {
+template <int kSBlock, bool ALLOWED, bool HISTORY>
+__device__ __forceinline__ void mask_registers(float (&v)[kSChunk / kSBlock], const uint32_t* allowed,
+                                               const uint32_t* history, int tid) {
+  constexpr int kSVec = kSChunk / (kSBlock * 4);
 #pragma unroll
   for (int j = 0; j < kSVec; ++j) {
     const int rel0 = (j * kSBlock + tid) * 4;
@@ -337,6 +339,10 @@ __device__ __forceinline__ void mask_registers(float (&v)[kSElems], const uint32
 template <bool NUCLEUS, bool XFORM>
 __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chunk, mi355x_sample_params prm,
                                            FusedShared& sm) {
+  constexpr int kSBlock = NUCLEUS ? kNucleusBlock : kTopkBlock;  // threads of this workgroup
+  constexpr int kSWaves = kSBlock / 64;
+  constexpr int kSVec = kSChunk / (kSBlock * 4);  // 128-bit loads per thread
+  constexpr int kSElems = kSVec * 4;              // logits held in registers per thread
   const int V = a.vocab;
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
@@ -347,7 +353,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   float v[kSElems];
 #pragma unroll
   for (int j = 0; j < kSVec; ++j) {
-    const int i0 = elem_index(chunk, j, 0);
+    const int i0 = elem_index<kSBlock>(chunk, j, 0);
     if (aligned && i0 + 4 <= V) {
       const v4f q = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(lrow + i0));
       v[j * 4 + 0] = q.x;
@@ -378,7 +384,8 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   // threads that marked them compute their processed values into a short list in LDS, `extras`, which
   // every later phase visits next to the registers.
   // The bitmap words and the first history ids of this thread are requested before anything waits.
-  static_assert(kSChunk / 32 == 2 * kSBlock, "two bitmap words per thread");
+  constexpr int kWordsPerThread = kSChunk / 32 / kSBlock;  // bitmap words a thread stages
+  static_assert(kWordsPerThread >= 1 && kSChunk / 32 == kWordsPerThread * kSBlock, "whole bitmap words per thread");
   const bool active = XFORM && a.xf.active();  // kernels without logits processing carry none of its code
   const bool pen = active && a.xf.use_penalty();
   const bool has_mask = active && a.xf.mask != nullptr;
@@ -387,10 +394,13 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   const int32_t* hist = pen ? a.xf.history + static_cast<size_t>(row) * a.xf.history_stride : nullptr;
   const bool hist_ahead = pen && a.xf.history_lens == nullptr;  // the length is known without a load
   int hist_pre[2] = {-1, -1};
-  uint32_t mask_pre[2] = {~0u, ~0u};
+  uint32_t mask_pre[kWordsPerThread];
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
+  for (int q = 0; q < 2; ++q)
     if (hist_ahead && tid + q * kSBlock < a.xf.history_len) hist_pre[q] = hist[tid + q * kSBlock];
+#pragma unroll
+  for (int q = 0; q < kWordsPerThread; ++q) {
+    mask_pre[q] = ~0u;
     if (has_mask) {
       const int w = chunk * (kSChunk / 32) + tid + q * kSBlock;
       mask_pre[q] = w < words ? mrow[w] : 0u;
@@ -402,7 +412,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     const int n_eos = a.xf.eos_count(row);
     if (tid == 0) sm.n_extra = 0u;
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+    for (int q = 0; q < kWordsPerThread; ++q) {
       const int i = tid + q * kSBlock;
       const int w = chunk * (kSChunk / 32) + i;
       uint32_t word = mask_pre[q];
@@ -445,7 +455,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
       extra_overflow = n_extra > static_cast<uint32_t>(kExtraCap);  // the row takes the exact path
       if (extra_overflow) n_extra = 0u;
     }
-    mask_registers<true, true>(v, sm.mask_bits, sm.hist_bits, tid);
+    mask_registers<kSBlock, true, true>(v, sm.mask_bits, sm.hist_bits, tid);
   }
   // per-thread maximum in the float domain (fmaxf skips NaN), keeping the maximum of every float4
   float qm[kSVec];
@@ -457,7 +467,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   }
   for (uint32_t i = tid; i < n_extra; i += kSBlock) fm = fmaxf(fm, sm.extra_val[i]);
   // 0: the thread holds no element
-  const uint32_t lmax = (elem_index(chunk, 0, 0) < V || static_cast<uint32_t>(tid) < n_extra) ? order_key(fm) : 0u;
+  const uint32_t lmax = (elem_index<kSBlock>(chunk, 0, 0) < V || static_cast<uint32_t>(tid) < n_extra) ? order_key(fm) : 0u;
   if (tid == 0) sm.count = 0u;
 
   if constexpr (NUCLEUS) {
@@ -486,7 +496,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     char* const dst = reinterpret_cast<char*>(big_row + static_cast<size_t>(chunk) * kSChunk);
     float thr2 = thr;
     asm volatile("" : "+v"(thr2));
-    const uint32_t nid0 = ~static_cast<uint32_t>(elem_index(chunk, 0, 0));  // ~(id0 + d) = ~id0 - d
+    const uint32_t nid0 = ~static_cast<uint32_t>(elem_index<kSBlock>(chunk, 0, 0));  // ~(id0 + d) = ~id0 - d
 #pragma unroll
     for (int e = 0; e < kSElems; ++e) {
       const bool cand = v[e] >= thr2;
@@ -536,7 +546,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
       if (any) fbk = order_key(-__builtin_inff());
     }
     const uint32_t ebk = key64_okey(extra_below);
-    const uint32_t bbk = block_max_lds<uint32_t>(fbk > ebk ? fbk : ebk, sm.wave_val);
+    const uint32_t bbk = block_max_lds<kSWaves, uint32_t>(fbk > ebk ? fbk : ebk, sm.wave_val);
     u64 best_below = ebk == bbk ? extra_below : 0;
     if (bbk != 0u && fbk == bbk) {
       const float bbf = key_to_float(bbk);
@@ -544,10 +554,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
 #pragma unroll
       for (int e = kSElems - 1; e >= 0; --e)
         if (v[e] == bbf) fe = e;
-      const u64 key = make_key64(bbk, static_cast<uint32_t>(elem_index(chunk, fe >> 2, fe & 3)));
+      const u64 key = make_key64(bbk, static_cast<uint32_t>(elem_index<kSBlock>(chunk, fe >> 2, fe & 3)));
       best_below = key > best_below ? key : best_below;
     }
-    best_below = block_max_lds<u64>(best_below, sm.wave_val64);  // its barriers also order the atomics on sm.count
+    best_below = block_max_lds<kSWaves, u64>(best_below, sm.wave_val64);  // its barriers also order the atomics on sm.count
     if (tid == 0) {
       const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
       a.chunk_cnt[ci] = extra_overflow ? kChunkCntOverflow : sm.count;
@@ -601,7 +611,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
           // listed with the raw float bits; the few entries that survive get their order keys later
           if (pos < kWaveListCap)
             sm.wave_list[wave * kWaveListCap + pos] =
-                make_key64(__float_as_uint(v[j * 4 + c]), static_cast<uint32_t>(elem_index(chunk, j, c)));
+                make_key64(__float_as_uint(v[j * 4 + c]), static_cast<uint32_t>(elem_index<kSBlock>(chunk, j, c)));
         }
         woff += static_cast<uint32_t>(__popcll(b));
       }
@@ -794,10 +804,11 @@ __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
 // Kernel variants: per-row parameter table in the arguments or not (_rows), nucleus rows or all other
 // rows, with or without the code of the logits processing (_xf).
 #define MS_STREAM_KERNEL(NAME, NUCLEUS, XFORM)                                                                      \
-  __global__ __launch_bounds__(kSBlock) void NAME##_kernel(const SampleArgs a) {                                    \
+  __global__ __launch_bounds__(NUCLEUS ? kNucleusBlock : kTopkBlock) void NAME##_kernel(const SampleArgs a) {      \
     sample_fused_body<false, NUCLEUS, XFORM>(a);                                                                    \
   }                                                                                                                 \
-  __global__ __launch_bounds__(kSBlock) void NAME##_rows_kernel(const SampleArgs a, const InlineParams) {           \
+  __global__ __launch_bounds__(NUCLEUS ? kNucleusBlock : kTopkBlock) void NAME##_rows_kernel(const SampleArgs a,   \
+                                                                                            const InlineParams) { \
     sample_fused_body<true, NUCLEUS, XFORM>(a);                                                                     \
   }
 MS_STREAM_KERNEL(sample_fused, false, false)
@@ -907,35 +918,70 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   if (row_mode(prm, V, a.chunks) != kModeNucleus) return;
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
+  // Thread c reads everything chunk c left behind; the barriers of the first reduction publish the counts.
+  __shared__ uint32_t sh_cnt[kAllCap / kSmallCap];       // candidates per chunk
+  __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // their prefix sums
   uint32_t m = 0u;
-  for (int c = tid; c < a.chunks; c += blockDim.x) {
-    m = a.chunk_max[cbase + c] > m ? a.chunk_max[cbase + c] : m;
-    if (a.chunk_cnt[cbase + c] == kChunkCntOverflow) m = 0xffffffffu;  // above every key: the exact path
+  u64 best_below = 0;
+  if (tid < a.chunks) {
+    const uint32_t cnt = a.chunk_cnt[cbase + tid];
+    m = cnt == kChunkCntOverflow ? 0xffffffffu : a.chunk_max[cbase + tid];  // above every key: the exact path
+    best_below = a.chunk_next[cbase + tid];
+    sh_cnt[tid] = cnt;
   }
   if (tid == 0) sh_count = 0u;
   const uint32_t rmax = block_max<uint32_t>(m, red32);
   const bool gave_up = rmax == 0xffffffffu;
   uint32_t thr = 0u;
   if (rmax != 0u) thr = order_key(key_to_float(rmax) - nucleus_depth(prm, V));
-  u64 best_below = 0;
-  for (int c = tid; c < a.chunks; c += blockDim.x) best_below = a.chunk_next[cbase + c] > best_below ? a.chunk_next[cbase + c] : best_below;
-  for (int c = 0; c < a.chunks; ++c) {
-    const uint32_t cnt = gave_up ? 0u : a.chunk_cnt[cbase + c];
-    const u64* src = big_row + static_cast<size_t>(c) * kSChunk;
-    for (uint32_t i0 = 0; i0 < cnt; i0 += blockDim.x) {
-      const uint32_t i = i0 + tid;
-      u64 k64 = 0;
-      if (i < cnt) {  // the list holds raw float bits in the score half
-        const u64 raw = src[i];
-        k64 = (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw >> 32)))) << 32) | (raw & 0xffffffffull);
+  if (tid == 0) {
+    uint32_t run = 0u;
+    for (int c = 0; c < a.chunks; ++c) {
+      sh_first[c] = run;
+      run += gave_up ? 0u : sh_cnt[c];
+    }
+    sh_first[a.chunks] = run;
+  }
+  __syncthreads();
+  // The chunks' lists are read as one flat sequence, kGather entries per thread in flight at a time;
+  // a wave reserves LDS slots for the candidates of such a batch with one atomic.
+  constexpr int kGather = 8;
+  const uint32_t total = sh_first[a.chunks];
+  const int lane = lane_id();
+  for (uint32_t f0 = 0; f0 < total; f0 += kGather * blockDim.x) {
+    u64 raw[kGather];
+#pragma unroll
+    for (int u = 0; u < kGather; ++u) {
+      const uint32_t f = f0 + u * blockDim.x + tid;
+      raw[u] = 0;
+      if (f < total) {
+        int c = 0;
+        for (int cc = 1; cc < a.chunks; ++cc) c += f >= sh_first[cc] ? 1 : 0;
+        raw[u] = big_row[static_cast<size_t>(c) * kSChunk + (f - sh_first[c])];
       }
-      const bool cand = i < cnt && key64_okey(k64) >= thr;
-      const uint32_t pos = wave_slot(cand, &sh_count);
-      if (cand) {
-        if (pos < kNucleusCap) lds_keys[pos] = k64;
-      } else {
-        best_below = k64 > best_below ? k64 : best_below;
-      }
+    }
+    u64 k64[kGather], hits[kGather];
+    uint32_t wcnt = 0u;
+#pragma unroll
+    for (int u = 0; u < kGather; ++u) {  // the lists hold raw float bits in the score half
+      const bool valid = f0 + u * blockDim.x + tid < total;
+      k64[u] = valid ? (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)))) << 32) |
+                           (raw[u] & 0xffffffffull)
+                     : 0;
+      const bool cand = valid && key64_okey(k64[u]) >= thr;
+      hits[u] = __ballot(cand);
+      wcnt += static_cast<uint32_t>(__popcll(hits[u]));
+      if (!cand) best_below = k64[u] > best_below ? k64[u] : best_below;
+    }
+    uint32_t base = 0u;
+    if (lane == 0 && wcnt != 0u) base = atomicAdd(&sh_count, wcnt);
+    base = __builtin_amdgcn_readfirstlane(base);
+#pragma unroll
+    for (int u = 0; u < kGather; ++u) {
+      const uint32_t pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(hits[u] >> 32),
+                                                     __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(hits[u]), base));
+      if (((hits[u] >> lane) & 1ull) && pos < kNucleusCap) lds_keys[pos] = k64[u];
+      base += static_cast<uint32_t>(__popcll(hits[u]));
     }
   }
   best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
@@ -993,7 +1039,7 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_rows_kernel(const
 
 extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_other,
                                        bool any_nucleus, hipStream_t stream) {
-  const dim3 grid(a->chunks, a->rows), block(ms::kSBlock);
+  const dim3 grid(a->chunks, a->rows), block(ms::kTopkBlock), nblock(ms::kNucleusBlock);
   const bool xf = a->xf.active();
   hipError_t e = hipSuccess;
   if (any_other) {
@@ -1009,13 +1055,13 @@ extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::Inline
   }
   if (any_nucleus) {
     if (table) {
-      if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_rows_kernel, grid, block, 0, stream, *a, *table);
-      else hipLaunchKernelGGL(ms::nucleus_stream_rows_kernel, grid, block, 0, stream, *a, *table);
+      if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_rows_kernel, grid, nblock, 0, stream, *a, *table);
+      else hipLaunchKernelGGL(ms::nucleus_stream_rows_kernel, grid, nblock, 0, stream, *a, *table);
       hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, dim3(a->rows), dim3(ms::kFinishBlock), ms::kFinishLds, stream,
                          *a, *table);
     } else {
-      if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_kernel, grid, block, 0, stream, *a);
-      else hipLaunchKernelGGL(ms::nucleus_stream_kernel, grid, block, 0, stream, *a);
+      if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_kernel, grid, nblock, 0, stream, *a);
+      else hipLaunchKernelGGL(ms::nucleus_stream_kernel, grid, nblock, 0, stream, *a);
       hipLaunchKernelGGL(ms::nucleus_finish_kernel, dim3(a->rows), dim3(ms::kFinishBlock), ms::kFinishLds, stream, *a);
     }
     e = hipGetLastError();
