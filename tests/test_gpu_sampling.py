@@ -309,6 +309,74 @@ def test_config5_constrained_nucleus(ctx, orc):
             assert tok[r] == idx[orc.discrete_draw(probs, u[r])]
 
 
+@pytest.mark.parametrize("vocab,hist_len,span,k,p", [
+    (40000, 2200, 40000, 50, 0.9),    # a history longer than two ids per thread, spread over two chunks
+    (40000, 2200, 40000, 0, 0.9),
+    (70001, 8000, 2500, 40, 1.0),     # more distinct history ids in one chunk than its list holds: exact path
+    (70001, 8000, 2500, 0, 0.95),
+    (33000, 300, 232, 8, 0.0),        # the short last chunk holds history ids
+    (33000, 300, 232, 0, 0.8),
+])
+def test_sample_long_and_dense_histories(ctx, orc, vocab, hist_len, span, k, p):
+    """History ids are processed apart from the other logits (a list per 32768-id chunk): long histories,
+    duplicates, ids outside the vocabulary, lists that overflow, ids in a short last chunk."""
+    say("sample histories", vocab, hist_len, span, k, p)
+    rng = np.random.default_rng(hist_len + span + k)
+    rows = 3
+    scale = 2.0 if k else 6.0           # nucleus rows stay peaked, so that their candidates fit the fast path
+    x = (rng.standard_normal((rows, vocab)) * scale).astype(np.float32)
+    hist = (vocab - span + rng.integers(0, span, (rows, hist_len))).astype(np.int32)
+    hist[:, :40] = hist[:, 40:80]       # duplicates
+    hist[0, 5] = vocab + 3              # beyond the vocabulary: ignored
+    hist[1, 7] = -2                     # negative: ignored
+    x[:, hist[2, 100:110]] = 4.6 * scale  # penalised ids among the best of their rows
+    mask = make_mask(rng, rows, vocab, 0.7)
+    u = rng.random(rows)
+    before = ctx.fallback_rows()
+    for pen in (1.3, 0.75):
+        xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                               repetition_penalty=pen)
+        tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=k, p=p, temperature=0.9,
+                                     xf=xf, kept_capacity=4096)
+        tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+        proc = orc.apply_mask(x, mask)
+        for r in range(rows):
+            valid = hist[r][(hist[r] >= 0) & (hist[r] < vocab)]
+            row = orc.apply_repetition_penalty(proc[r], valid, pen)
+            idx, probs = orc.sampled_categorical(row, k, p, 0.9)
+            assert kc[r] == len(idx), (r, pen)
+            n = min(len(idx), 4096)
+            assert np.array_equal(ki[r, :n], idx[:n]), (r, pen)
+            assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), (r, pen)
+            assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (r, pen)
+    took_exact = ctx.fallback_rows() - before
+    assert (took_exact > 0) == (span == 2500), took_exact  # only the overflowing lists go to the exact path
+
+
+@pytest.mark.parametrize("vocab", [5000, 70001])
+def test_nucleus_with_minus_infinity_below_the_threshold(ctx, orc, vocab):
+    """Rows whose elements outside the candidate range are all -inf: the element after the nucleus, which a
+    stop on a sort-batch end keeps, is then a -inf one (probability 0) with the lowest id."""
+    say("nucleus -inf tail", vocab)
+    rng = np.random.default_rng(vocab)
+    rows = 4
+    x = np.full((rows, vocab), -np.inf, np.float32)
+    for r, n in enumerate([16, 64, 15, 256]):   # 16, 64, 256: the nucleus ends on a batch end when p is near 1
+        ids = rng.choice(vocab, n, replace=False)
+        x[r, ids] = rng.standard_normal(n).astype(np.float32)
+    u = rng.random(rows)
+    for p in (0.9999999, 0.5):
+        tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=p, temperature=1.0,
+                                     kept_capacity=1024)
+        tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+        for r in range(rows):
+            idx, probs = orc.sampled_categorical(x[r], 0, p, 1.0)
+            assert kc[r] == len(idx), (r, p, kc[r], len(idx))
+            assert np.array_equal(ki[r, :len(idx)], idx), (r, p)
+            assert np.array_equal(bits(kp[r, :len(idx)]), bits(probs)), (r, p)
+            assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (r, p)
+
+
 @pytest.mark.parametrize("rows,vocab", [(6, 30000), (64, 40000), (70, 9000)])
 def test_sample_heterogeneous_rows(ctx, orc, rows, vocab):
     """BatchedSampler semantics: per-row (k, p, T), greedy = (1, 0, 1).  Up to 64 rows the parameters
