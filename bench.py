@@ -6,8 +6,10 @@ categorical draw) over one batch of seeded synthetic fp32 logits resident in HBM
 are recorded once into a HIP graph (one kernel launch per step, each on its own logits buffer from a
 pool larger than twice the 256 MB Infinity Cache) and replayed between two HIP events on the launch
 stream.  Before any number is printed, token ids of the checked steps are compared with the CPU
-oracle on identical logits and uniforms; the same oracle, timed on the host cores, is the
-cpu_baseline.  Prints ONE JSON line."""
+oracle on identical logits and uniforms and, where the reference's own headers were compiled into
+oracle/_ref, with the reference's ComputeSampledCategorical + SampleCategoricalToken driven by
+std::mt19937 engines of the same seeds; that reference build (else the oracle), timed on one host
+core, is the cpu_baseline.  Prints ONE JSON line."""
 import argparse
 import json
 import os
@@ -108,6 +110,18 @@ def main():
         logits.append(x)
     rng = np.random.default_rng(99)
     u_host = rng.random((K + W, ROWS))
+    # Where the reference's own headers were compiled (oracle/_ref), the draws of the checked steps are
+    # the ones its std::mt19937 engines produce from known seeds, so that the reference's tokens can be
+    # compared with the GPU's one to one.
+    ref = orc_lib.Reference.load()
+    n_cpu = max(1, min(args.cpu_steps, K))
+    seeds = None
+    if ref is not None:
+        seeds = np.arange(n_cpu * ROWS, dtype=np.uint32).reshape(n_cpu, ROWS) * np.uint32(2654435761) + np.uint32(12345)
+        two = (np.array([0, 1], np.int32), np.array([0.5, 0.5], np.float32))
+        for i in range(n_cpu):
+            for r in range(ROWS):
+                u_host[W + i, r] = ref.sample_categorical(two[0], two[1], int(seeds[i, r]))[1]
     uniforms = torch.from_numpy(u_host).to(dev)
     tokens = torch.empty((K + W, ROWS), dtype=torch.int32, device=dev)
     ctx = pkg.SearchContext(ROWS, VOCAB)
@@ -120,7 +134,6 @@ def main():
     torch.cuda.synchronize()
 
     # ---- parity gate: GPU tokens == CPU oracle tokens on identical inputs ---------------------------
-    n_cpu = max(1, min(args.cpu_steps, K))
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -146,6 +159,30 @@ def main():
         bad = int((got != want).sum())
         sys.exit(f"PARITY FAILURE: {bad} of {got.size} sampled tokens differ from the CPU oracle")
     fallback = ctx.fallback_rows()
+    # ---- CPU baseline: the reference's own functions where they were built, else the oracle ---------
+    baseline = {"value": ROWS * n_cpu / cpu_s, "unit": "tokens/s", "cores": 1, "kind": "port",
+                "sample": "%d of the %d timed steps (same logits and uniforms), oracle/search_oracle.cpp "
+                          "orc_sample_batch, one thread as in the reference's serial row loop" % (n_cpu, K),
+                "ms_per_step": cpu_s / n_cpu * 1e3, "host_cpus": os.cpu_count()}
+    parity = "token ids of %d steps bit-identical to the CPU oracle" % n_cpu
+    if ref is not None:
+        t0 = time.perf_counter()
+        ref_tok = np.empty((n_cpu, ROWS), np.int32)
+        for i in range(n_cpu):
+            for r in range(ROWS):
+                idx, probs = ref.sampled_categorical(cpu_in[i][r], TOP_K, TOP_P, TEMP)
+                ref_tok[i, r] = ref.sample_categorical(idx, probs, int(seeds[i, r]))[0]
+        ref_s = time.perf_counter() - t0
+        if not np.array_equal(got, ref_tok):
+            bad = int((got != ref_tok).sum())
+            sys.exit(f"PARITY FAILURE: {bad} of {got.size} sampled tokens differ from the reference's own functions")
+        baseline = {"value": ROWS * n_cpu / ref_s, "unit": "tokens/s", "cores": 1, "kind": "reference",
+                    "sample": "%d of the %d timed steps (same logits; draws from std::mt19937 engines with the same "
+                              "seeds): the reference's ComputeSampledCategorical + SampleCategoricalToken compiled "
+                              "from its own headers (oracle/_ref), one thread as in its serial row loop" % (n_cpu, K),
+                    "ms_per_step": ref_s / n_cpu * 1e3, "host_cpus": os.cpu_count(),
+                    "oracle_port_ms_per_step": cpu_s / n_cpu * 1e3}
+        parity += " and to the reference's own functions"
 
     # ---- informational: the same K steps with three independent batches in flight ------------------
     # A generation loop is sequential (a step's tokens feed the next step's logits), which is what
@@ -184,7 +221,7 @@ def main():
                                "one fused kernel per step, %d steps replayed from a HIP graph over a pool of %d "
                                "logits buffers" % (K, pool),
                    "rows": ROWS, "vocab": VOCAB, "top_k": TOP_K, "top_p": TOP_P, "temperature": TEMP,
-                   "parity": "token ids of %d steps bit-identical to the CPU oracle" % n_cpu,
+                   "parity": parity,
                    "general_path_rows": fallback,
                    "independent_batches_in_flight": None if overlapped_ms is None else {
                        "note": "informational, not `value`: the same steps issued round-robin on %d streams / "
@@ -195,10 +232,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": "sample_fused_kernel", "algorithmic_bytes_per_launch": algo_bytes},
-        "cpu_baseline": {"value": ROWS * n_cpu / cpu_s, "unit": "tokens/s", "cores": 1, "kind": "port",
-                         "sample": "%d of the %d timed steps (same logits and uniforms), oracle/search_oracle.cpp "
-                                   "orc_sample_batch, one thread as in the reference's serial row loop" % (n_cpu, K),
-                         "ms_per_step": cpu_s / n_cpu * 1e3, "host_cpus": os.cpu_count()},
+        "cpu_baseline": baseline,
     }
     print(json.dumps(out))
 
