@@ -292,7 +292,6 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   a.chunk_cnt = ctx->chunk_cnt;
   a.chunk_max = ctx->chunk_max;
   a.chunk_next = ctx->chunk_next;
-  a.row_arrive = ctx->row_arrive;
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
@@ -339,7 +338,6 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   a.chunk_cnt = ctx->chunk_cnt;
   a.chunk_max = ctx->chunk_max;
   a.chunk_next = ctx->chunk_next;
-  a.row_arrive = ctx->row_arrive;
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;

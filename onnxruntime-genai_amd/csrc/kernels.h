@@ -45,11 +45,10 @@ struct SampleArgs {
   float* kept_probs;
   int kept_capacity;
   // workspace
-  u64* cand_small;        // [rows][chunks][kSmallCap], every slot rewritten by every launch
+  u64* cand_small;        // [rows][chunks][kSmallCap]; zero between launches (published, then cleared by the finisher)
   uint32_t* chunk_cnt;    // [rows][chunks]
   uint32_t* chunk_max;    // [rows][chunks]
   u64* chunk_next;        // [rows][chunks]
-  uint32_t* row_arrive;   // [rows], zero between launches
   u64* big;               // [rows][big_stride]
   size_t big_stride;
   uint32_t* fallback_rows;  // cumulative count of rows finished by the general path

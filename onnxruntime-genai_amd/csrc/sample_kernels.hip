@@ -1,13 +1,16 @@
 // Sampling kernels.
 //
-// sample_fused_kernel: one launch per step.  Every workgroup (512 threads x 64 logits) streams one
-// 32K-logit chunk of one row with 128-bit non-temporal loads (logits processing fused), keeps the chunk's
-// best 64 candidates for the row's top-k and publishes them sorted; the last workgroup of a row to
-// arrive merges the chunks' sorted lists pairwise (bitonic merges in registers, two levels for four
-// chunks) and runs the reference's scalar epilogue (softmax over the k, nucleus cut, categorical
-// draw) in rank order.  Rows in nucleus mode (k <= 1) only compact their
-// candidates here; nucleus_finish_kernel sorts them and finishes.  Anything the fast paths decline
-// (k > 64, heavy ties, tiny vocabularies) goes through general_row, an exact full sort.
+// sample_fused_kernel (top-k rows, k <= 64; one launch per step): every workgroup (512 threads x 64
+// logits) streams one 32K-logit chunk of one row with 128-bit non-temporal loads, logits processing
+// fused, keeps the chunk's best 64 candidates and publishes them sorted; the workgroup of a row's last
+// chunk polls for the other chunks' lists, merges them four at a time (bitonic merges in registers)
+// and runs the reference's scalar epilogue (softmax over the k, nucleus cut, categorical draw) in rank
+// order.  nucleus_stream_kernel (rows with k <= 1; 1024 threads x 32 logits per workgroup) compacts
+// every chunk's candidates into the row's key buffer; nucleus_finish_kernel sorts them and finishes.
+// Anything the fast paths decline (k > 64, heavy ties, tiny vocabularies, more history ids in a chunk
+// than its list holds) goes through general_row, an exact full sort.  Each streaming kernel exists
+// with and without the code of the logits processing (_xf) and with the per-row parameters in a
+// device table or inside the kernel arguments (_rows).
 #include "kernels.h"
 #include "block_seq.h"
 #include "wave_select.h"
