@@ -921,9 +921,22 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   if (row_mode(prm, V, a.chunks) != kModeNucleus) return;
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
+  // The head of every chunk's list (kAhead entries per thread) is requested before the counts are
+  // known -- whatever lies past a list's end is discarded later -- so that these loads overlap the
+  // round trip for the counts.  Rows of more than kAheadChunks chunks read everything afterwards.
+  constexpr int kGather = 8, kAheadChunks = 8, kAhead = 1;
+  static_assert((kAheadChunks * kAhead) % kGather == 0, "the head is consumed in whole batches");
+  const bool ahead = a.chunks <= kAheadChunks;
+  const uint32_t head = ahead ? kAhead * kFinishBlock : 0u;  // entries of a list read ahead
+  u64 pre[kAheadChunks * kAhead];
+#pragma unroll
+  for (int c = 0; c < kAheadChunks; ++c)
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u)
+      pre[c * kAhead + u] = (ahead && c < a.chunks) ? big_row[static_cast<size_t>(c) * kSChunk + u * kFinishBlock + tid] : 0;
   // Thread c reads everything chunk c left behind; the barriers of the first reduction publish the counts.
   __shared__ uint32_t sh_cnt[kAllCap / kSmallCap];       // candidates per chunk
-  __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // their prefix sums
+  __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // prefix sums of the entries past the heads
   uint32_t m = 0u;
   u64 best_below = 0;
   if (tid < a.chunks) {
@@ -941,37 +954,24 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     uint32_t run = 0u;
     for (int c = 0; c < a.chunks; ++c) {
       sh_first[c] = run;
-      run += gave_up ? 0u : sh_cnt[c];
+      run += (gave_up || sh_cnt[c] <= head) ? 0u : sh_cnt[c] - head;
     }
     sh_first[a.chunks] = run;
   }
   __syncthreads();
-  // The chunks' lists are read as one flat sequence, kGather entries per thread in flight at a time;
-  // a wave reserves LDS slots for the candidates of such a batch with one atomic.
-  constexpr int kGather = 8;
-  const uint32_t total = sh_first[a.chunks];
+  // A batch of kGather entries per thread: float bits become order keys, candidates (at or above the
+  // row's threshold) go to LDS at slots a wave reserves with one atomic per batch, the best of the
+  // others is kept.
   const int lane = lane_id();
-  for (uint32_t f0 = 0; f0 < total; f0 += kGather * blockDim.x) {
-    u64 raw[kGather];
-#pragma unroll
-    for (int u = 0; u < kGather; ++u) {
-      const uint32_t f = f0 + u * blockDim.x + tid;
-      raw[u] = 0;
-      if (f < total) {
-        int c = 0;
-        for (int cc = 1; cc < a.chunks; ++cc) c += f >= sh_first[cc] ? 1 : 0;
-        raw[u] = big_row[static_cast<size_t>(c) * kSChunk + (f - sh_first[c])];
-      }
-    }
+  auto consume = [&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
     u64 k64[kGather], hits[kGather];
     uint32_t wcnt = 0u;
 #pragma unroll
-    for (int u = 0; u < kGather; ++u) {  // the lists hold raw float bits in the score half
-      const bool valid = f0 + u * blockDim.x + tid < total;
-      k64[u] = valid ? (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)))) << 32) |
-                           (raw[u] & 0xffffffffull)
-                     : 0;
-      const bool cand = valid && key64_okey(k64[u]) >= thr;
+    for (int u = 0; u < kGather; ++u) {
+      k64[u] = valid[u] ? (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)))) << 32) |
+                              (raw[u] & 0xffffffffull)
+                        : 0;
+      const bool cand = valid[u] && key64_okey(k64[u]) >= thr;
       hits[u] = __ballot(cand);
       wcnt += static_cast<uint32_t>(__popcll(hits[u]));
       if (!cand) best_below = k64[u] > best_below ? k64[u] : best_below;
@@ -986,6 +986,40 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       if (((hits[u] >> lane) & 1ull) && pos < kNucleusCap) lds_keys[pos] = k64[u];
       base += static_cast<uint32_t>(__popcll(hits[u]));
     }
+  };
+  if (ahead && !gave_up) {
+#pragma unroll
+    for (int b = 0; b < kAheadChunks * kAhead / kGather; ++b) {
+      if (b * kGather / kAhead < a.chunks) {
+        u64 raw[kGather];
+        bool valid[kGather];
+#pragma unroll
+        for (int u = 0; u < kGather; ++u) {
+          const int q = b * kGather + u, c = q / kAhead;
+          raw[u] = pre[q];
+          valid[u] = c < a.chunks && static_cast<uint32_t>((q % kAhead) * kFinishBlock + tid) < sh_cnt[c < a.chunks ? c : 0];
+        }
+        consume(raw, valid);
+      }
+    }
+  }
+  // what the heads did not cover, as one flat sequence
+  const uint32_t total = sh_first[a.chunks];
+  for (uint32_t f0 = 0; f0 < total; f0 += kGather * blockDim.x) {
+    u64 raw[kGather];
+    bool valid[kGather];
+#pragma unroll
+    for (int u = 0; u < kGather; ++u) {
+      const uint32_t f = f0 + u * blockDim.x + tid;
+      raw[u] = 0;
+      valid[u] = f < total;
+      if (valid[u]) {
+        int c = 0;
+        for (int cc = 1; cc < a.chunks; ++cc) c += f >= sh_first[cc] ? 1 : 0;
+        raw[u] = big_row[static_cast<size_t>(c) * kSChunk + head + (f - sh_first[c])];
+      }
+    }
+    consume(raw, valid);
   }
   best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
   uint32_t n_c = sh_count;
