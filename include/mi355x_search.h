@@ -271,6 +271,16 @@ int mi355x_logits_handoff(mi355x_search_ctx* ctx, void* stream, const void* raw,
  * declined and the exact general path finished (synchronises `stream`). */
 int mi355x_search_fallback_rows(mi355x_search_ctx* ctx, void* stream, unsigned* rows);
 
+/* Failure handling of the top-k path (no counterpart in the reference).  The workgroup that finishes
+ * a row waits for the candidate lists of the row's other workgroups by polling, at most `polls`
+ * times (default 2^21, a few seconds); a wait that gives up hands its row to the exact path and
+ * makes every later call on the context use the exact path for top-k rows, so that results stay
+ * correct and no kernel ever waits without bound.  mi355x_search_wait_gave_up reports whether that
+ * has happened (synchronises `stream`).  mi355x_search_set_poll_limit exists for tests of this
+ * recovery: 0 lets every wait that is not satisfied at once give up. */
+int mi355x_search_wait_gave_up(mi355x_search_ctx* ctx, void* stream, int* gave_up);
+int mi355x_search_set_poll_limit(mi355x_search_ctx* ctx, int polls);
+
 #ifdef __cplusplus
 }
 #endif

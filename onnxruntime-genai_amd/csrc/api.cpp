@@ -55,6 +55,7 @@ struct mi355x_search_ctx {
   ms::u64* big{};
   size_t big_stride{};
   uint32_t* fallback_rows{};
+  int poll_limit{ms::kDefaultPollLimit};
   uint32_t* ban{};  // [max_rows, mask words]: ids banned by the no-repeat-n-gram rule
   mi355x_sample_params* params_dev{};
   void** ptr_table{};      // device copy of pointer tables (kv gather)
@@ -295,6 +296,7 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
+  a.poll_limit = ctx->poll_limit;
   HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_other, any_nucleus, s));
   return MI355X_OK;
 }
@@ -341,6 +343,7 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   a.big = ctx->big;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
+  a.poll_limit = ctx->poll_limit;
   HIP_TRY(ms_launch_sample(&a, nullptr, true, false, s));
   return MI355X_OK;
 }
@@ -552,6 +555,24 @@ int mi355x_search_fallback_rows(mi355x_search_ctx* ctx, void* stream, unsigned* 
   HIP_TRY(hipMemcpyAsync(rows, ctx->fallback_rows, sizeof(unsigned), hipMemcpyDeviceToHost,
                          static_cast<hipStream_t>(stream)));
   HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  *rows &= 0x7fffffffu;  // bit 31 is the flag mi355x_search_wait_gave_up reports
+  return MI355X_OK;
+}
+
+int mi355x_search_wait_gave_up(mi355x_search_ctx* ctx, void* stream, int* gave_up) {
+  if (!ctx || !gave_up) return Fail(MI355X_E_INVALID, "null argument");
+  unsigned word = 0;
+  HIP_TRY(hipMemcpyAsync(&word, ctx->fallback_rows, sizeof(unsigned), hipMemcpyDeviceToHost,
+                         static_cast<hipStream_t>(stream)));
+  HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  *gave_up = static_cast<int>(word >> 31);
+  return MI355X_OK;
+}
+
+int mi355x_search_set_poll_limit(mi355x_search_ctx* ctx, int polls) {
+  if (!ctx) return Fail(MI355X_E_INVALID, "null context");
+  if (polls < 0) return Fail(MI355X_E_INVALID, "negative poll limit");
+  ctx->poll_limit = polls;
   return MI355X_OK;
 }
 

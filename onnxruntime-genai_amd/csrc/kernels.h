@@ -13,6 +13,9 @@ constexpr int kSChunk = 32768;        // logits per workgroup of the streaming k
 constexpr int kTopkBlock = 512;       // threads of a workgroup that streams a top-k row (16 128-bit loads each) ...
 constexpr int kNucleusBlock = 1024;   // ... and a nucleus row (8 each: lighter threads, twice the waves in flight)
 constexpr int kSMaxWaves = 16;
+// Polls (about a microsecond each) after which a finishing workgroup stops waiting for another
+// workgroup's list and lets the exact path compute the row: a few seconds by default.
+constexpr int kDefaultPollLimit = 1 << 21;
 constexpr int kSmallCap = 64;        // sorted candidates a chunk publishes on the k<=64 path
 constexpr int kListCap = 128;        // candidates a chunk can hold before its sort
 constexpr int kAllCap = 1024;        // slots a finishing workgroup ranks (16 chunks x kSmallCap)
@@ -51,7 +54,8 @@ struct SampleArgs {
   u64* chunk_next;        // [rows][chunks]
   u64* big;               // [rows][big_stride]
   size_t big_stride;
-  uint32_t* fallback_rows;  // cumulative count of rows finished by the general path
+  uint32_t* fallback_rows;  // cumulative count of rows finished by the general path; bit 31: a wait gave up
+  int poll_limit;           // polls a finishing workgroup waits for another workgroup's list
   int emit_topk;            // != 0: write the k best (id, raw score) per row instead of sampling
   float* out_scores;        // [rows, k], emit_topk only (out_tokens is [rows, k] then)
 };

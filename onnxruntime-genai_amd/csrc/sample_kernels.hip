@@ -127,9 +127,6 @@ __device__ __forceinline__ float nucleus_depth(mi355x_sample_params prm, int voc
 
 // Values of a published candidate slot that are not keys (a key's low half is ~id, far above these).
 constexpr u64 kSlotEmpty = 1, kSlotOverflow = 2;
-// Polls (about a microsecond each) after which a finishing workgroup stops waiting for a list and lets
-// the exact path compute the row.
-constexpr int kSpinLimit = 1 << 21;
 constexpr int kWaveListCap = 128;  // hits one wave can list per chunk
 constexpr int kExtraCap = 2048;    // distinct history ids one chunk can hold; beyond, the row takes the exact path
 constexpr uint32_t kChunkCntOverflow = 0xffffffffu;  // chunk_cnt of a nucleus chunk that gave up
@@ -374,6 +371,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   u64* const cand_small = arg_now(a.cand_small);
   const double* const uniforms = arg_now(a.uniforms);
   const int emit_topk = arg_now(a.emit_topk);
+  const int poll_limit = arg_now(a.poll_limit);
   const RowOutputs outputs = {arg_now(a.out_tokens) + row,
                               arg_now(a.kept_count),
                               arg_now(a.kept_ids),
@@ -725,7 +723,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
       for (int q = 0; q < 4; ++q)
         if (got[q] == 0) got[q] = load_coherent(&seg[cc[q] * kSmallCap + ii[q]]);
       if (__ballot(got[0] == 0 || got[1] == 0 || got[2] == 0 || got[3] == 0) == 0ull) break;
-      if (++spins == kSpinLimit) {
+      if (spins++ >= poll_limit) {
         if (lane == 0) atomicOr(a.fallback_rows, 0x80000000u);
         break;
       }

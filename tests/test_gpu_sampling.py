@@ -449,6 +449,38 @@ def test_sample_randomised_shapes_and_parameters(ctx, orc, seed):
             assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (r, k, p, t)
 
 
+def test_wait_that_gives_up_hands_rows_to_the_exact_path(orc):
+    """Failure handling of the top-k hand-over between workgroups, forced from the host: with a poll limit
+    of 0 a finishing workgroup gives up on every list that has not arrived yet.  Its row must come out of
+    the exact path unchanged, the context must report the event, and every later call must still be right
+    (all its top-k rows then take the exact path)."""
+    say("poll limit 0")
+    rng = np.random.default_rng(77)
+    rows, vocab = 128, 201088  # seven workgroups per row, far more workgroups than the GPU runs at once
+    c = pkg().SearchContext(rows, vocab)
+    try:
+        x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+        u = rng.random(rows)
+        want = np.array([orc.sample_row(x[r], 50, 0.9, 0.7, u[r]) for r in range(rows)], np.int32)
+        xd, ud = torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda()
+        assert np.array_equal(c.sample(xd, ud, k=50, p=0.9, temperature=0.7).cpu().numpy(), want)
+        assert not c.wait_gave_up() and c.fallback_rows() == 0
+        c.set_poll_limit(0)
+        assert np.array_equal(c.sample(xd, ud, k=50, p=0.9, temperature=0.7).cpu().numpy(), want)
+        assert c.wait_gave_up()
+        assert 0 < c.fallback_rows() <= rows
+        c.set_poll_limit(1 << 21)
+        before = c.fallback_rows()
+        assert np.array_equal(c.sample(xd, ud, k=50, p=0.9, temperature=0.7).cpu().numpy(), want)
+        assert c.fallback_rows() - before == rows  # the fast path stays off for this context
+        tk, ts = c.topk_scores(xd[:4], 8)
+        for r in range(4):
+            order = np.lexsort((np.arange(vocab), -x[r].astype(np.float64)))[:8]
+            assert np.array_equal(tk[r].cpu().numpy(), order.astype(np.int32))
+    finally:
+        c.close()
+
+
 def test_argument_errors(ctx):
     x = torch.zeros((2, 100), device="cuda")
     u = torch.zeros(2, dtype=torch.float64, device="cuda")
