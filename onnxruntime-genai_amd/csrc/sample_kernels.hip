@@ -580,58 +580,83 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   const size_t ci = static_cast<size_t>(row) * n_chunks + chunk;
   u64* dst = cand_small + ci * kSmallCap;
   uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool);
-  if (tau == 0u) {
-    // The pooled bound found fewer than k offers (a short tail chunk keeps its elements in one or two
-    // waves): take the exact k-th best of the 512 per-thread maxima instead.
-    static_assert(kSWaves * kWaveListCap >= kSBlock, "the hit lists double as the sort buffer of this path");
+  // The pooled bound is exact unless one wave holds more than its share of the best k; with k close to
+  // 64 it can sit low enough for the hits to overflow their lists, and in a short tail chunk it may
+  // find fewer than k offers (0).  Either way the exact k-th best of the per-thread maxima takes its
+  // place: about k + k*k/1024 elements reach that one.
+  static_assert(kSWaves * kWaveListCap >= kSBlock, "the hit lists double as the sort buffer of the exact bound");
+  uint32_t n_c = 0u, cnt[kSWaves];
+  bool overflow = false;
+  // exact k-th best of the per-thread maxima
+  auto exact_bound = [&]() {
     u64* scratch = sm.wave_list;  // free until the hits are listed
     scratch[tid] = static_cast<u64>(lmax);
     __syncthreads();
     block_sort_desc(scratch, kSBlock);
-    tau = static_cast<uint32_t>(scratch[kk - 1]);
+    const uint32_t t = static_cast<uint32_t>(scratch[kk - 1]);
     __syncthreads();
-  }
-  // tau == 0: the chunk has fewer than k elements -- keep them all
-  const float tau_f = tau != 0u ? key_to_float(tau) : -__builtin_inff();
+    return t;
+  };
   // Hits are rare (about k per chunk).  Every wave lists its own hits in a private LDS segment: the
   // slot of a hit is the wave's running count (a scalar) plus the number of hitting lanes below, so
-  // no atomics, no second pass and no block-wide prefix are needed.
-  uint32_t woff = 0u;
+  // no atomics, no second pass and no block-wide prefix are needed.  Ends with the per-wave counts.
+  auto list_hits = [&](uint32_t bound) {
+    // bound == 0: the chunk has fewer than k elements -- keep them all
+    const float tau_f = bound != 0u ? key_to_float(bound) : -__builtin_inff();
+    uint32_t woff = 0u;
 #pragma unroll
-  for (int j = 0; j < kSVec; ++j) {
-    if (__ballot(qm[j] >= tau_f) != 0ull) {
+    for (int j = 0; j < kSVec; ++j) {
+      if (__ballot(qm[j] >= tau_f) != 0ull) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const bool hit = v[j * 4 + c] >= tau_f;
-        const u64 b = __ballot(hit);
-        if (b == 0ull) continue;
-        if (hit) {
-          const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
-                                                                __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), 0u));
-          // key64 of a real element is never 0 (its index half is ~idx != 0), so 0 marks an empty slot
-          // listed with the raw float bits; the few entries that survive get their order keys later
-          if (pos < kWaveListCap)
-            sm.wave_list[wave * kWaveListCap + pos] =
-                make_key64(__float_as_uint(v[j * 4 + c]), static_cast<uint32_t>(elem_index<kSBlock>(chunk, j, c)));
+        for (int c = 0; c < 4; ++c) {
+          const bool hit = v[j * 4 + c] >= tau_f;
+          const u64 b = __ballot(hit);
+          if (b == 0ull) continue;
+          if (hit) {
+            const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
+                                                                  __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), 0u));
+            // key64 of a real element is never 0 (its index half is ~idx != 0), so 0 marks an empty slot
+            // listed with the raw float bits; the few entries that survive get their order keys later
+            if (pos < kWaveListCap)
+              sm.wave_list[wave * kWaveListCap + pos] =
+                  make_key64(__float_as_uint(v[j * 4 + c]), static_cast<uint32_t>(elem_index<kSBlock>(chunk, j, c)));
+          }
+          woff += static_cast<uint32_t>(__popcll(b));
         }
-        woff += static_cast<uint32_t>(__popcll(b));
       }
     }
-  }
-  for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
-    const uint32_t i = i0 + tid;
-    const float ev = i < n_extra ? sm.extra_val[i] : kNaN;
-    const bool hit = ev >= tau_f;
-    const u64 b = __ballot(hit);
-    if (hit) {
-      const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
-                                                            __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), 0u));
-      if (pos < kWaveListCap) sm.wave_list[wave * kWaveListCap + pos] = make_key64(__float_as_uint(ev), sm.extra_idx[i]);
+    for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
+      const uint32_t i = i0 + tid;
+      const float ev = i < n_extra ? sm.extra_val[i] : kNaN;
+      const bool hit = ev >= tau_f;
+      const u64 b = __ballot(hit);
+      if (hit) {
+        const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
+                                                              __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), 0u));
+        if (pos < kWaveListCap) sm.wave_list[wave * kWaveListCap + pos] = make_key64(__float_as_uint(ev), sm.extra_idx[i]);
+      }
+      woff += static_cast<uint32_t>(__popcll(b));
     }
-    woff += static_cast<uint32_t>(__popcll(b));
+    if (lane == 0) sm.wave_val[wave] = woff;
+    __syncthreads();
+    n_c = 0u;
+    overflow = false;
+#pragma unroll
+    for (int w = 0; w < kSWaves; ++w) {
+      cnt[w] = sm.wave_val[w];
+      n_c += cnt[w];
+      overflow = overflow || cnt[w] > static_cast<uint32_t>(kWaveListCap);
+    }
+    overflow = overflow || n_c > static_cast<uint32_t>(kListCap);
+  };
+  const bool pooled = tau != 0u;
+  if (__builtin_expect(!pooled, 0)) tau = exact_bound();
+  list_hits(tau);
+  if (__builtin_expect(overflow && pooled, 0)) {  // rare: a second, separate copy of the listing code, with the exact bound
+    tau = exact_bound();
+    list_hits(tau);
   }
-  if (lane == 0) sm.wave_val[wave] = woff;
-  __syncthreads();
+  overflow = overflow || extra_overflow;
   // The chunk's best 64 candidates, sorted (best first): nothing ranked lower inside its own chunk can
   // be among the row's k <= 64 best.  Waves 0 and 1 sort one half of the list each, wave 0 merges.
   // The workgroup of the row's LAST chunk finishes the row; every other workgroup publishes its list
@@ -641,16 +666,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   // trip lie between a chunk's sort and the row's merge.  Workgroups are dispatched in index order
   // and a publishing workgroup never waits, so the lists a finishing workgroup polls for belong to
   // workgroups that are running or done.
-  uint32_t n_c = 0u;
-  uint32_t cnt[kSWaves];
-  bool overflow = extra_overflow;
-#pragma unroll
-  for (int w = 0; w < kSWaves; ++w) {
-    cnt[w] = sm.wave_val[w];
-    n_c += cnt[w];
-    overflow = overflow || cnt[w] > static_cast<uint32_t>(kWaveListCap);
-  }
-  overflow = overflow || n_c > static_cast<uint32_t>(kListCap);
   const bool two_halves = n_c > 64u;
   const bool finisher = chunk == n_chunks - 1;
   u64 mykey = 0;

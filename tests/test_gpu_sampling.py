@@ -449,6 +449,36 @@ def test_sample_randomised_shapes_and_parameters(ctx, orc, seed):
             assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (r, k, p, t)
 
 
+@pytest.mark.parametrize("k", [50, 57, 64])
+def test_topk_with_clustered_best_tokens_stays_on_the_fast_path(ctx, orc, k):
+    """The per-chunk bound pools the best eight per-thread maxima of every wave; rows whose best tokens
+    sit next to each other (one wave holds most of them) or whose k is close to 64 let many more than k
+    elements past it.  The kernel then takes the exact bound and lists again: results equal the oracle's
+    and no row needs the full-sort path."""
+    say("clustered top-k", k)
+    rng = np.random.default_rng(900 + k)
+    rows, vocab = 12, 128256
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    for r in range(rows // 2):
+        start = int(rng.integers(0, vocab - 1024)) // 256 * 256
+        if r % 2:   # 24 neighbouring ids hold the row's best tokens (six threads with four of them each)
+            x[r, start:start + 24] = 14.0 + rng.standard_normal(24).astype(np.float32)
+        else:       # 60 of the best tokens at every fourth id of one 256-id strip: one each in 60 threads of one wave
+            x[r, start:start + 240:4] = 14.0 + rng.standard_normal(60).astype(np.float32)
+    u = rng.random(rows)
+    before = ctx.fallback_rows()
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=k, p=0.95, temperature=0.8,
+                                 kept_capacity=64)
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    for r in range(rows):
+        idx, probs = orc.sampled_categorical(x[r], k, 0.95, 0.8)
+        assert kc[r] == len(idx), r
+        assert np.array_equal(ki[r, :len(idx)], idx), r
+        assert np.array_equal(bits(kp[r, :len(idx)]), bits(probs)), r
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+    assert ctx.fallback_rows() == before
+
+
 def test_wait_that_gives_up_hands_rows_to_the_exact_path(orc):
     """Failure handling of the top-k hand-over between workgroups, forced from the host: with a poll limit
     of 0 a finishing workgroup gives up on every list that has not arrived yet.  Its row must come out of
