@@ -252,15 +252,19 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   hipStream_t s = static_cast<hipStream_t>(stream);
   ms::SampleArgs a{};
   if (int r = MakeXform(ctx, xf, rows, vocab, s, &a.xf)) return r;
-  bool any_nucleus = false, any_other = false;
+  bool any_nucleus = false, any_other = false, any_large_k = false;
   const int chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
   ms::InlineParams table;
   bool use_table = false;
   auto check = [&](const mi355x_sample_params& p) -> int {
     if (!(p.temperature > 0.0f)) return Fail(MI355X_E_INVALID, "temperature must be positive (got %g)", p.temperature);
     // the kernels' own rule (row_mode) decides; these flags only have to cover it
-    if (p.k <= 1 && vocab > 64) any_nucleus = true;
-    if (!(p.k <= 1 && vocab > 64 && chunks * ms::kSmallCap <= ms::kAllCap)) any_other = true;
+    const int kk = p.k < vocab ? p.k : vocab;
+    const bool fits = vocab > 64 && chunks * ms::kSmallCap <= ms::kAllCap;
+    const bool nucleus = p.k <= 1, large_k = p.k > 1 && kk > 64 && kk <= ms::kLargeKMax;
+    if (nucleus && vocab > 64) any_nucleus = true;
+    if (large_k && vocab > 64) any_large_k = true;
+    if (!((nucleus || large_k) && fits)) any_other = true;
     return MI355X_OK;
   };
   if (per_row_params) {
@@ -297,7 +301,7 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
   a.poll_limit = ctx->poll_limit;
-  HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_other, any_nucleus, s));
+  HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_other, any_nucleus, any_large_k, s));
   return MI355X_OK;
 }
 
@@ -344,7 +348,7 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
   a.poll_limit = ctx->poll_limit;
-  HIP_TRY(ms_launch_sample(&a, nullptr, true, false, s));
+  HIP_TRY(ms_launch_sample(&a, nullptr, true, false, false, s));
   return MI355X_OK;
 }
 

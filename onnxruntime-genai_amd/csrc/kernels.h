@@ -25,6 +25,10 @@ constexpr int kFinishBlock = 1024;
 constexpr int kModeTopkSmall = 0;
 constexpr int kModeNucleus = 1;
 constexpr int kModeGeneral = 2;
+constexpr int kModeTopkLarge = 3;  // 64 < k <= kLargeKMax: streamed and finished by the nucleus kernels
+// The per-chunk bound of such rows is the k-th best of the 1024 per-thread maxima of a nucleus workgroup; up to half
+// the threads it stays tight (about 1.4 k elements reach it), towards all of them it lets a third of the chunk through.
+constexpr int kLargeKMax = 512;
 
 // Heterogeneous (k, p, T) of a batch of at most kInlineParamRows rows travel inside the kernel
 // arguments, as a second argument of kernel variants of their own, so that no copy to the device
@@ -148,9 +152,10 @@ struct ScorerState {
 extern "C" {
 hipError_t ms_sample_init();
 // `table`, when not null, holds the parameters of rows 0 .. a->rows-1 (a->rows <= kInlineParamRows).
-// any_nucleus: some row may be in nucleus mode; any_other: some row may be in another mode.
+// any_nucleus / any_large_k / any_other: some row may be in nucleus mode / a top-k row with
+// 64 < k <= kLargeKMax / in another mode (each mode has kernels of its own).
 hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_other, bool any_nucleus,
-                            hipStream_t stream);
+                            bool any_large_k, hipStream_t stream);
 hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipStream_t stream);
 hipError_t ms_launch_process_logits(float* logits, int64_t row_stride, int rows, int vocab,
                                     const ms::Xform* xf, hipStream_t stream);

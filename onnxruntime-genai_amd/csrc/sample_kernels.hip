@@ -36,7 +36,18 @@ __device__ __forceinline__ mi355x_sample_params row_params(const SampleArgs& a, 
     q.temperature = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(table[row].temperature)));
     return q;
   } else {
-    return a.per_row ? a.per_row[row] : a.uniform;
+    // The device table is read-only during the launch: read through the constant address space, its
+    // entries come by scalar loads like the uniform parameters from the kernel arguments, the row's mode
+    // is a scalar, and nothing here waits for a vector load before the logits are requested.
+    mi355x_sample_params q = a.uniform;
+    if (a.per_row) {
+      typedef __attribute__((address_space(4))) const mi355x_sample_params* TablePtr;
+      const TablePtr table = (TablePtr)a.per_row;
+      q.k = table[row].k;
+      q.p = table[row].p;
+      q.temperature = table[row].temperature;
+    }
+    return q;
   }
 }
 
@@ -111,7 +122,10 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const 
 __device__ __forceinline__ int row_mode(mi355x_sample_params prm, int vocab, int chunks, int emit_topk = 0) {
   if (vocab <= 64 || chunks * kSmallCap > kAllCap) return kModeGeneral;
   if (emit_topk) return kModeTopkSmall;
-  if (prm.k > 1) return (prm.k < vocab ? prm.k : vocab) <= 64 ? kModeTopkSmall : kModeGeneral;
+  if (prm.k > 1) {
+    const int kk = prm.k < vocab ? prm.k : vocab;
+    return kk <= 64 ? kModeTopkSmall : (kk <= kLargeKMax ? kModeTopkLarge : kModeGeneral);
+  }
   return kModeNucleus;
 }
 
@@ -336,7 +350,7 @@ __device__ __forceinline__ void mask_registers(float (&v)[kSChunk / kSBlock], co
 
 // Streaming pass of one (row, chunk) of a top-k<=64 or nucleus row.  Returns true when this workgroup
 // must run the general path for the row (it was the last to arrive and the fast path declined).
-template <bool NUCLEUS, bool XFORM>
+template <bool NUCLEUS, bool XFORM, bool LARGEK = false>
 __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chunk, mi355x_sample_params prm,
                                            FusedShared& sm) {
   constexpr int kSBlock = NUCLEUS ? kNucleusBlock : kTopkBlock;  // threads of this workgroup
@@ -476,9 +490,24 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     // particular order (the finish kernel sorts).  A wave counts its candidates, reserves a range of
     // the chunk's list with one LDS atomic and fills it; the slot of a candidate is the wave's running
     // count plus the number of candidate lanes below.
+    // Rows with 64 < k <= kLargeKMax come here too: their candidates are the elements that reach the
+    // exact k-th best per-thread maximum of the chunk (at least k elements do; with fewer than k
+    // threads holding elements, all), which contain the chunk's k best.
+    static_assert(kLargeKMax <= kSBlock && kSMaxWaves * kWaveListCap >= kSBlock, "one offer per thread, sorted in the hit lists' LDS");
+    constexpr bool large_k = LARGEK;
     const uint32_t cmax = block_max<uint32_t>(lmax, sm.wave_val);
     float thr = -__builtin_inff();
-    if (cmax != 0u) thr = key_to_float(cmax) - nucleus_depth(prm, V);
+    if (large_k) {
+      u64* scratch = sm.wave_list;
+      scratch[tid] = static_cast<u64>(lmax);
+      __syncthreads();
+      block_sort_desc(scratch, kSBlock);
+      const uint32_t kth = static_cast<uint32_t>(scratch[(prm.k < V ? prm.k : V) - 1]);
+      if (kth != 0u) thr = key_to_float(kth);
+      __syncthreads();
+    } else if (cmax != 0u) {
+      thr = key_to_float(cmax) - nucleus_depth(prm, V);
+    }
     // First pass: the wave's number of candidates.
     uint32_t wcnt = 0u;
 #pragma unroll
@@ -795,16 +824,16 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
 // Rows in nucleus mode and all other rows are streamed by kernels of their own (a launch may need
 // both): each kernel holds the code of its mode only, and a change to one path leaves the machine
 // code of the other as it was.
-template <bool INLINE, bool NUCLEUS, bool XFORM>
+template <bool INLINE, bool NUCLEUS, bool XFORM, bool LARGEK = false>
 __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
   const int row = blockIdx.y, chunk = blockIdx.x;
   __shared__ FusedShared sm;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
   const int mode = row_mode(prm, a.vocab, a.chunks, a.emit_topk);
   if constexpr (NUCLEUS) {
-    if (mode == kModeNucleus) stream_row<true, XFORM>(a, row, chunk, prm, sm);
+    if (mode == (LARGEK ? kModeTopkLarge : kModeNucleus)) stream_row<true, XFORM, LARGEK>(a, row, chunk, prm, sm);
   } else {
-    if (mode == kModeNucleus) return;
+    if (mode == kModeNucleus || mode == kModeTopkLarge) return;
     if (mode == kModeGeneral) {
       if (chunk != 0) return;
     } else if (!stream_row<false, XFORM>(a, row, chunk, prm, sm)) {
@@ -817,20 +846,22 @@ __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
   }
 }
 
-// Kernel variants: per-row parameter table in the arguments or not (_rows), nucleus rows or all other
-// rows, with or without the code of the logits processing (_xf).
-#define MS_STREAM_KERNEL(NAME, NUCLEUS, XFORM)                                                                      \
+// Kernel variants: per-row parameter table in the arguments or not (_rows); nucleus rows, top-k rows with
+// 64 < k <= kLargeKMax (largek) or all other rows; with or without the code of the logits processing (_xf).
+#define MS_STREAM_KERNEL(NAME, NUCLEUS, XFORM, LARGEK)                                                              \
   __global__ __launch_bounds__(NUCLEUS ? kNucleusBlock : kTopkBlock) void NAME##_kernel(const SampleArgs a) {      \
-    sample_fused_body<false, NUCLEUS, XFORM>(a);                                                                    \
+    sample_fused_body<false, NUCLEUS, XFORM, LARGEK>(a);                                                            \
   }                                                                                                                 \
   __global__ __launch_bounds__(NUCLEUS ? kNucleusBlock : kTopkBlock) void NAME##_rows_kernel(const SampleArgs a,   \
                                                                                             const InlineParams) { \
-    sample_fused_body<true, NUCLEUS, XFORM>(a);                                                                     \
+    sample_fused_body<true, NUCLEUS, XFORM, LARGEK>(a);                                                             \
   }
-MS_STREAM_KERNEL(sample_fused, false, false)
-MS_STREAM_KERNEL(sample_fused_xf, false, true)
-MS_STREAM_KERNEL(nucleus_stream, true, false)
-MS_STREAM_KERNEL(nucleus_stream_xf, true, true)
+MS_STREAM_KERNEL(sample_fused, false, false, false)
+MS_STREAM_KERNEL(sample_fused_xf, false, true, false)
+MS_STREAM_KERNEL(nucleus_stream, true, false, false)
+MS_STREAM_KERNEL(nucleus_stream_xf, true, true, false)
+MS_STREAM_KERNEL(largek_stream, true, false, true)
+MS_STREAM_KERNEL(largek_stream_xf, true, true, true)
 #undef MS_STREAM_KERNEL
 
 // Sorts n keys (kFinishBlock < n <= kNucleusCap) in LDS, descending, by a block of kFinishBlock
@@ -919,7 +950,7 @@ __device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n,
 // Per-row finish of the nucleus path: gathers the candidates the streaming pass left in `big`,
 // sorts them in LDS and runs the exact epilogue.  One block of kFinishBlock threads per row;
 // dynamic LDS: kNucleusCap key64s + the bucket table of the sort.
-template <bool INLINE>
+template <bool INLINE, bool LARGEK>
 __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   extern __shared__ u64 lds_keys[];
   uint32_t* bucket_start = reinterpret_cast<uint32_t*>(lds_keys + kNucleusCap);  // kSortBuckets + 1 entries
@@ -931,7 +962,8 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   const int V = a.vocab;
   const int tid = threadIdx.x;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
-  if (row_mode(prm, V, a.chunks) != kModeNucleus) return;
+  if (row_mode(prm, V, a.chunks) != (LARGEK ? kModeTopkLarge : kModeNucleus)) return;
+  constexpr bool large_k = LARGEK;  // then every listed element is a candidate and no element after them is needed
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
   // The head of every chunk's list (kAhead entries per thread) is requested before the counts are
@@ -955,14 +987,14 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   if (tid < a.chunks) {
     const uint32_t cnt = a.chunk_cnt[cbase + tid];
     m = cnt == kChunkCntOverflow ? 0xffffffffu : a.chunk_max[cbase + tid];  // above every key: the exact path
-    best_below = a.chunk_next[cbase + tid];
+    best_below = large_k ? 0 : a.chunk_next[cbase + tid];
     sh_cnt[tid] = cnt;
   }
   if (tid == 0) sh_count = 0u;
   const uint32_t rmax = block_max<uint32_t>(m, red32);
   const bool gave_up = rmax == 0xffffffffu;
   uint32_t thr = 0u;
-  if (rmax != 0u) thr = order_key(key_to_float(rmax) - nucleus_depth(prm, V));
+  if (rmax != 0u && !large_k) thr = order_key(key_to_float(rmax) - nucleus_depth(prm, V));
   if (tid == 0) {
     uint32_t run = 0u;
     for (int c = 0; c < a.chunks; ++c) {
@@ -976,6 +1008,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // row's threshold) go to LDS at slots a wave reserves with one atomic per batch, the best of the
   // others is kept.
   const int lane = lane_id();
+  uint32_t lowest = 0xffffffffu;  // lowest candidate key this thread has seen
   auto consume = [&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
     u64 k64[kGather], hits[kGather];
     uint32_t wcnt = 0u;
@@ -988,6 +1021,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       hits[u] = __ballot(cand);
       wcnt += static_cast<uint32_t>(__popcll(hits[u]));
       if (!cand) best_below = k64[u] > best_below ? k64[u] : best_below;
+      if (cand && key64_okey(k64[u]) < lowest) lowest = key64_okey(k64[u]);
     }
     uint32_t base = 0u;
     if (lane == 0 && wcnt != 0u) base = atomicAdd(&sh_count, wcnt);
@@ -1037,6 +1071,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
   uint32_t n_c = sh_count;
   bool ok = !gave_up && n_c < kNucleusCap;  // room for the next-best element too
+  if (large_k) thr = ~block_max<uint32_t>(~lowest, red32);  // the lowest candidate score: the sort scales its buckets by it
   if (ok) {
     if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
     if (best_below != 0) n_c += 1;
@@ -1080,16 +1115,21 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   }
 }
 
-__global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const SampleArgs a) { nucleus_finish_body<false>(a); }
+__global__ __launch_bounds__(kFinishBlock) void nucleus_finish_kernel(const SampleArgs a) { nucleus_finish_body<false, false>(a); }
 __global__ __launch_bounds__(kFinishBlock) void nucleus_finish_rows_kernel(const SampleArgs a, const InlineParams) {
-  nucleus_finish_body<true>(a);
+  nucleus_finish_body<true, false>(a);
+}
+__global__ __launch_bounds__(kFinishBlock) void largek_finish_kernel(const SampleArgs a) { nucleus_finish_body<false, true>(a); }
+__global__ __launch_bounds__(kFinishBlock) void largek_finish_rows_kernel(const SampleArgs a, const InlineParams) {
+  nucleus_finish_body<true, true>(a);
 }
 
 }  // namespace ms
 
 extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_other,
-                                       bool any_nucleus, hipStream_t stream) {
+                                       bool any_nucleus, bool any_large_k, hipStream_t stream) {
   const dim3 grid(a->chunks, a->rows), block(ms::kTopkBlock), nblock(ms::kNucleusBlock);
+  const dim3 fgrid(a->rows), fblock(ms::kFinishBlock);
   const bool xf = a->xf.active();
   hipError_t e = hipSuccess;
   if (any_other) {
@@ -1107,12 +1147,24 @@ extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::Inline
     if (table) {
       if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_rows_kernel, grid, nblock, 0, stream, *a, *table);
       else hipLaunchKernelGGL(ms::nucleus_stream_rows_kernel, grid, nblock, 0, stream, *a, *table);
-      hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, dim3(a->rows), dim3(ms::kFinishBlock), ms::kFinishLds, stream,
-                         *a, *table);
+      hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
     } else {
       if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_kernel, grid, nblock, 0, stream, *a);
       else hipLaunchKernelGGL(ms::nucleus_stream_kernel, grid, nblock, 0, stream, *a);
-      hipLaunchKernelGGL(ms::nucleus_finish_kernel, dim3(a->rows), dim3(ms::kFinishBlock), ms::kFinishLds, stream, *a);
+      hipLaunchKernelGGL(ms::nucleus_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  if (any_large_k) {
+    if (table) {
+      if (xf) hipLaunchKernelGGL(ms::largek_stream_xf_rows_kernel, grid, nblock, 0, stream, *a, *table);
+      else hipLaunchKernelGGL(ms::largek_stream_rows_kernel, grid, nblock, 0, stream, *a, *table);
+      hipLaunchKernelGGL(ms::largek_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
+    } else {
+      if (xf) hipLaunchKernelGGL(ms::largek_stream_xf_kernel, grid, nblock, 0, stream, *a);
+      else hipLaunchKernelGGL(ms::largek_stream_kernel, grid, nblock, 0, stream, *a);
+      hipLaunchKernelGGL(ms::largek_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
     }
     e = hipGetLastError();
   }
@@ -1120,9 +1172,13 @@ extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::Inline
 }
 
 extern "C" hipError_t ms_sample_init() {
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ms::nucleus_finish_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, ms::kFinishLds);
-  if (e != hipSuccess) return e;
-  return hipFuncSetAttribute(reinterpret_cast<const void*>(ms::nucleus_finish_rows_kernel),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, ms::kFinishLds);
+  const void* finish[] = {reinterpret_cast<const void*>(ms::nucleus_finish_kernel),
+                          reinterpret_cast<const void*>(ms::nucleus_finish_rows_kernel),
+                          reinterpret_cast<const void*>(ms::largek_finish_kernel),
+                          reinterpret_cast<const void*>(ms::largek_finish_rows_kernel)};
+  for (const void* f : finish) {
+    const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, ms::kFinishLds);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }

@@ -228,6 +228,40 @@ def test_sample_large_k_general_path(ctx, orc):
     sample_and_check(ctx, orc, x, u, 6000, 0.0, 1.0, cap=64)  # k > vocab clamps
 
 
+@pytest.mark.parametrize("vocab,k,p,t,quantum", [
+    (128256, 65, 0.9, 0.7, 0.0), (128256, 100, 1.0, 1.0, 0.0), (128256, 512, 0.95, 1.3, 0.0), (201088, 300, 0.0, 0.8, 0.0),
+    (128256, 513, 0.95, 1.3, 0.0),  # beyond the limit of this route: the full-sort path
+    (33000, 100, 0.9, 1.0, 0.0),    # the short last chunk holds fewer than k threads' worth of elements
+    (40000, 500, 0.99, 1.0, 0.25),  # ties across the cut
+    (700, 500, 0.9, 1.0, 0.0),      # k close to the vocabulary
+])
+def test_sample_large_k_through_the_candidate_lists(ctx, orc, vocab, k, p, t, quantum):
+    """Top-k rows with 64 < k <= 512 are streamed like nucleus rows (candidates = elements at or above
+    the k-th best per-thread maximum of their chunk) and finished by the sorting kernel, not by the
+    full-sort path; kept sets, probabilities and tokens equal the oracle's."""
+    say("sample large k", vocab, k, p, t, quantum)
+    rng = np.random.default_rng(vocab + k)
+    rows = 5
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    if quantum:
+        x = (np.round(x / quantum) * quantum).astype(np.float32)
+    x[1, :] = np.float32(0.5)            # a constant row: heavy ties, the exact path is allowed here
+    x[2, rng.integers(0, vocab, 50)] = -np.inf
+    u = rng.random(rows)
+    before = ctx.fallback_rows()
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=k, p=p, temperature=t,
+                                 kept_capacity=1024)
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    for r in range(rows):
+        idx, probs = orc.sampled_categorical(x[r], k, p, t)
+        assert kc[r] == len(idx), r
+        assert np.array_equal(ki[r, :len(idx)], idx), r
+        assert np.array_equal(bits(kp[r, :len(idx)]), bits(probs)), r
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+    if k <= 512:
+        assert ctx.fallback_rows() - before <= 1  # at most the constant row
+
+
 @pytest.mark.parametrize("rows,vocab,p,t", [(3, 5000, 0.9, 1.0), (2, 128256, 0.95, 0.7), (2, 40, 0.6, 1.0),
                                             (2, 64, 0.9, 1.0), (2, 65, 0.9, 1.0), (3, 3000, 0.0, 1.0),
                                             (2, 3000, 0.3, 2.0)])
