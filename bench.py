@@ -23,7 +23,7 @@ sys.path.insert(0, os.path.join(ROOT, "onnxruntime-genai_amd"))
 
 ROWS, VOCAB, TOP_K, TOP_P, TEMP = 64, 128256, 50, 0.9, 0.7
 HBM_PEAK_GBS = 8000.0
-MEASURED_TRAFFIC_BYTES = 33_450_000  # fetch 33.25 MB + write 0.20 MB per launch
+MEASURED_TRAFFIC_BYTES = 33_460_000  # fetch 33.26 MB + write 0.20 MB per launch
 
 
 def time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, tokens, pool, W, K):

@@ -13,7 +13,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per step from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these same commands, scaled by a
 # known-size copy (profiles/beam_step_kernels_config3.md, profiles/nucleus_kernels_config5.md); counters
 # cannot be read from inside the process.  None where no counter run exists.
-MEASURED_TRAFFIC = {"c3": 6_222_000_000 + 82_000_000, "c5": 287_000_000}
+MEASURED_TRAFFIC = {"c3": 6_222_000_000 + 82_000_000, "c5": 289_000_000}
 
 
 def _timed(fn_step, K, W, graph=True):
