@@ -509,7 +509,7 @@ struct RowOutputs {
 // exp((score_i - score_0) * inv_temp) as a float (callers may cache it).  Returns false -- without
 // writing outputs -- when the nucleus does not end inside the n_sorted available elements.
 template <int ITEMS, typename Sorted, typename Exps>
-__device__ bool block_sample_epilogue(Sorted sorted, Exps exps, int n_sorted, int vocab,
+__device__ __forceinline__ bool block_sample_epilogue(Sorted sorted, Exps exps, int n_sorted, int vocab,
                                       mi355x_sample_params prm, double u, const RowOutputs& out,
                                       SeqShared& sh) {
   int keep;

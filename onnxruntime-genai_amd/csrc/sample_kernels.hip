@@ -966,22 +966,11 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   constexpr bool large_k = LARGEK;  // then every listed element is a candidate and no element after them is needed
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
-  // The head of every chunk's list (kAhead entries per thread) is requested before the counts are
-  // known -- whatever lies past a list's end is discarded later -- so that these loads overlap the
-  // round trip for the counts.  Rows of more than kAheadChunks chunks read everything afterwards.
-  constexpr int kGather = 8, kAheadChunks = 8, kAhead = 1;
-  static_assert((kAheadChunks * kAhead) % kGather == 0, "the head is consumed in whole batches");
-  const bool ahead = a.chunks <= kAheadChunks;
-  const uint32_t head = ahead ? kAhead * kFinishBlock : 0u;  // entries of a list read ahead
-  u64 pre[kAheadChunks * kAhead];
-#pragma unroll
-  for (int c = 0; c < kAheadChunks; ++c)
-#pragma unroll
-    for (int u = 0; u < kAhead; ++u)
-      pre[c * kAhead + u] = (ahead && c < a.chunks) ? big_row[static_cast<size_t>(c) * kSChunk + u * kFinishBlock + tid] : 0;
+  constexpr int kGather = 8;  // entries of the chunks' lists a thread has in flight
   // Thread c reads everything chunk c left behind; the barriers of the first reduction publish the counts.
   __shared__ uint32_t sh_cnt[kAllCap / kSmallCap];       // candidates per chunk
-  __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // prefix sums of the entries past the heads
+  __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // their prefix sums
+  __shared__ int sh_trim;
   uint32_t m = 0u;
   u64 best_below = 0;
   if (tid < a.chunks) {
@@ -999,15 +988,103 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     uint32_t run = 0u;
     for (int c = 0; c < a.chunks; ++c) {
       sh_first[c] = run;
-      run += (gave_up || sh_cnt[c] <= head) ? 0u : sh_cnt[c] - head;
+      run += gave_up ? 0u : sh_cnt[c];
     }
     sh_first[a.chunks] = run;
   }
   __syncthreads();
+  const int lane = lane_id();
+  // Calls fn(entries, valid) for batches of kGather entries per thread of the flat sequence made of the
+  // chunks' lists (sh_first[c] = entries of the chunks before c).
+  auto flat_batches = [&](auto fn) {
+    const uint32_t total = sh_first[a.chunks];
+    for (uint32_t f0 = 0; f0 < total; f0 += kGather * blockDim.x) {
+      u64 raw[kGather];
+      bool valid[kGather];
+#pragma unroll
+      for (int u = 0; u < kGather; ++u) {
+        const uint32_t f = f0 + u * blockDim.x + tid;
+        raw[u] = 0;
+        valid[u] = f < total;
+        if (valid[u]) {
+          int c = 0;
+          for (int cc = 1; cc < a.chunks; ++cc) c += f >= sh_first[cc] ? 1 : 0;
+          raw[u] = big_row[static_cast<size_t>(c) * kSChunk + (f - sh_first[c])];
+        }
+      }
+      fn(raw, valid);
+    }
+  };
+  // More candidates listed than the sort holds (a flat distribution): the threshold is raised to the
+  // lowest score that still leaves room, found from a histogram of the candidates over the sort's
+  // score-linear buckets.  The nucleus test of the epilogue only looks at the elements it is given, in
+  // rank order, and reports when they do not contain the nucleus; only then does the row need the
+  // exact path.
+  bool trim_failed = false;
+  if (!large_k && sh_first[a.chunks] >= static_cast<uint32_t>(kNucleusCap)) {
+    const float fmax = key_to_float(rmax), fthr = key_to_float(thr);
+    const float span = fmax - fthr;
+    const float scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
+    auto bucket_of = [=](float x) {
+      float bf = (fmax - x) * scale;
+      bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);
+      return bf > 0.0f ? static_cast<int>(bf) : 0;
+    };
+    for (int b = tid; b < kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;
+    __syncthreads();
+    const uint32_t thr0 = thr;
+    flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
+#pragma unroll
+      for (int u = 0; u < kGather; ++u) {
+        const float x = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
+        if (valid[u] && order_key(x) >= thr0) atomicAdd(&bucket_start[bucket_of(x)], 1u);
+      }
+    });
+    __syncthreads();
+    // last bucket up to which the candidates fit (one slot stays free for the element after them)
+    if (tid < 64) {
+      constexpr int kPer = kSortBuckets / 64;
+      const uint32_t limit = static_cast<uint32_t>(kNucleusCap - 2);
+      uint32_t own = 0u;
+      for (int i = 0; i < kPer; ++i) own += bucket_start[tid * kPer + i];
+      uint32_t inc = own;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t y = __shfl_up(inc, d, 64);
+        if (lane >= d) inc += y;
+      }
+      const int crossing = first_lane(__ballot(inc > limit));  // -1: everything fits
+      if (crossing < 0) {
+        if (tid == 0) sh_trim = kSortBuckets - 1;
+      } else if (tid == crossing) {
+        uint32_t run = inc - own;
+        int last = tid * kPer - 1;
+        for (int i = 0; i < kPer; ++i) {
+          run += bucket_start[tid * kPer + i];
+          if (run > limit) break;
+          last = tid * kPer + i;
+        }
+        sh_trim = last;
+      }
+    }
+    __syncthreads();
+    const int last_bucket = sh_trim;
+    if (last_bucket < 0) {
+      trim_failed = true;  // the best bucket alone does not fit (heavy ties)
+    } else if (last_bucket < kSortBuckets - 1) {
+      // the lowest score whose bucket is still kept: the bucket is a non-increasing function of the score
+      uint32_t lo = thr, hi = rmax;
+      while (lo < hi) {
+        const uint32_t mid = lo + ((hi - lo) >> 1);
+        if (bucket_of(key_to_float(mid)) <= last_bucket) hi = mid;
+        else lo = mid + 1u;
+      }
+      thr = hi;
+    }
+  }
   // A batch of kGather entries per thread: float bits become order keys, candidates (at or above the
   // row's threshold) go to LDS at slots a wave reserves with one atomic per batch, the best of the
   // others is kept.
-  const int lane = lane_id();
   uint32_t lowest = 0xffffffffu;  // lowest candidate key this thread has seen
   auto consume = [&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
     u64 k64[kGather], hits[kGather];
@@ -1034,43 +1111,10 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       base += static_cast<uint32_t>(__popcll(hits[u]));
     }
   };
-  if (ahead && !gave_up) {
-#pragma unroll
-    for (int b = 0; b < kAheadChunks * kAhead / kGather; ++b) {
-      if (b * kGather / kAhead < a.chunks) {
-        u64 raw[kGather];
-        bool valid[kGather];
-#pragma unroll
-        for (int u = 0; u < kGather; ++u) {
-          const int q = b * kGather + u, c = q / kAhead;
-          raw[u] = pre[q];
-          valid[u] = c < a.chunks && static_cast<uint32_t>((q % kAhead) * kFinishBlock + tid) < sh_cnt[c < a.chunks ? c : 0];
-        }
-        consume(raw, valid);
-      }
-    }
-  }
-  // what the heads did not cover, as one flat sequence
-  const uint32_t total = sh_first[a.chunks];
-  for (uint32_t f0 = 0; f0 < total; f0 += kGather * blockDim.x) {
-    u64 raw[kGather];
-    bool valid[kGather];
-#pragma unroll
-    for (int u = 0; u < kGather; ++u) {
-      const uint32_t f = f0 + u * blockDim.x + tid;
-      raw[u] = 0;
-      valid[u] = f < total;
-      if (valid[u]) {
-        int c = 0;
-        for (int cc = 1; cc < a.chunks; ++cc) c += f >= sh_first[cc] ? 1 : 0;
-        raw[u] = big_row[static_cast<size_t>(c) * kSChunk + head + (f - sh_first[c])];
-      }
-    }
-    consume(raw, valid);
-  }
+  flat_batches(consume);
   best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
   uint32_t n_c = sh_count;
-  bool ok = !gave_up && n_c < kNucleusCap;  // room for the next-best element too
+  bool ok = !gave_up && !trim_failed && n_c < kNucleusCap;  // room for the next-best element too
   if (large_k) thr = ~block_max<uint32_t>(~lowest, red32);  // the lowest candidate score: the sort scales its buckets by it
   if (ok) {
     if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;

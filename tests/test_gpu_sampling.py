@@ -273,6 +273,33 @@ def test_sample_nucleus(ctx, orc, rows, vocab, p, t):
     sample_and_check(ctx, orc, x, u, 0, p, t, cap=128)
 
 
+@pytest.mark.parametrize("vocab,sigma,p,fast", [(128256, 4.0, 0.95, True), (201088, 5.0, 0.9, True), (128256, 2.0, 0.95, False),
+                                                (40000, 4.0, 0.999, False)])
+def test_nucleus_with_more_candidates_than_the_sort_holds(ctx, orc, vocab, sigma, p, fast):
+    """Unmasked rows: nearly the whole vocabulary lies within the candidate depth of the maximum.  The finish
+    kernel then keeps the best ~16000 by raising its threshold; when they contain the nucleus (peaked rows)
+    the row stays on the fast path, otherwise the exact path takes it.  Results equal the oracle's either way."""
+    say("nucleus trim", vocab, sigma, p)
+    rng = np.random.default_rng(int(vocab + sigma * 10))
+    rows = 4
+    x = (rng.standard_normal((rows, vocab)) * sigma).astype(np.float32)
+    x[3] = (np.round(x[3] * 2) / 2).astype(np.float32)  # ties at the raised threshold
+    u = rng.random(rows)
+    before = ctx.fallback_rows()
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=p, temperature=1.0,
+                                 kept_capacity=4096)
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    for r in range(rows):
+        idx, probs = orc.sampled_categorical(x[r], 0, p, 1.0)
+        assert kc[r] == len(idx), (r, kc[r], len(idx))
+        n = min(len(idx), 4096)
+        assert np.array_equal(ki[r, :n], idx[:n]), r
+        assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), r
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+    took_exact = ctx.fallback_rows() - before
+    assert took_exact == 0 if fast else took_exact > 0, took_exact
+
+
 @pytest.mark.parametrize("vocab", [32, 128, 130, 512, 2048, 8192, 32768, 131072])
 def test_nucleus_stop_on_last_element_of_a_sort_batch(ctx, orc, vocab):
     """Constant rows with p = 0.5 meet the tail-bound stop at element vocab/2; where that is the end of one of
