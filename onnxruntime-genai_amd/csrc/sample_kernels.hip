@@ -966,11 +966,24 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   constexpr bool large_k = LARGEK;  // then every listed element is a candidate and no element after them is needed
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
-  constexpr int kGather = 8;  // entries of the chunks' lists a thread has in flight
+  // The head of every chunk's list (kAhead entries per thread) is requested before the counts are
+  // known -- whatever lies past a list's end is discarded later -- so that these loads overlap the
+  // round trip for the counts.  Rows of more than kAheadChunks chunks, and rows whose lists hold more
+  // than the sort has room for, read everything afterwards.
+  constexpr int kGather = 8, kAheadChunks = 8, kAhead = 2;  // kGather: entries a thread has in flight
+  static_assert((kAheadChunks * kAhead) % kGather == 0, "the head is consumed in whole batches");
+  u64 pre[kAheadChunks * kAhead];
+#pragma unroll
+  for (int c = 0; c < kAheadChunks; ++c)
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u)
+      pre[c * kAhead + u] =
+          (a.chunks <= kAheadChunks && c < a.chunks) ? big_row[static_cast<size_t>(c) * kSChunk + u * kFinishBlock + tid] : 0;
   // Thread c reads everything chunk c left behind; the barriers of the first reduction publish the counts.
   __shared__ uint32_t sh_cnt[kAllCap / kSmallCap];       // candidates per chunk
   __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // their prefix sums
   __shared__ int sh_trim;
+  __shared__ uint32_t sh_head, sh_all;
   uint32_t m = 0u;
   u64 best_below = 0;
   if (tid < a.chunks) {
@@ -985,17 +998,24 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   uint32_t thr = 0u;
   if (rmax != 0u && !large_k) thr = order_key(key_to_float(rmax) - nucleus_depth(prm, V));
   if (tid == 0) {
+    uint32_t all = 0u;
+    for (int c = 0; c < a.chunks; ++c) all += gave_up ? 0u : sh_cnt[c];
+    const uint32_t head =
+        (a.chunks <= kAheadChunks && all < static_cast<uint32_t>(kNucleusCap)) ? kAhead * kFinishBlock : 0u;
     uint32_t run = 0u;
     for (int c = 0; c < a.chunks; ++c) {
       sh_first[c] = run;
-      run += gave_up ? 0u : sh_cnt[c];
+      run += (gave_up || sh_cnt[c] <= head) ? 0u : sh_cnt[c] - head;
     }
     sh_first[a.chunks] = run;
+    sh_head = head;
+    sh_all = all;
   }
   __syncthreads();
   const int lane = lane_id();
   // Calls fn(entries, valid) for batches of kGather entries per thread of the flat sequence made of the
-  // chunks' lists (sh_first[c] = entries of the chunks before c).
+  // chunks' lists past their heads (sh_first[c] = such entries of the chunks before c).
+  const uint32_t head = sh_head;
   auto flat_batches = [&](auto fn) {
     const uint32_t total = sh_first[a.chunks];
     for (uint32_t f0 = 0; f0 < total; f0 += kGather * blockDim.x) {
@@ -1009,7 +1029,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
         if (valid[u]) {
           int c = 0;
           for (int cc = 1; cc < a.chunks; ++cc) c += f >= sh_first[cc] ? 1 : 0;
-          raw[u] = big_row[static_cast<size_t>(c) * kSChunk + (f - sh_first[c])];
+          raw[u] = big_row[static_cast<size_t>(c) * kSChunk + head + (f - sh_first[c])];
         }
       }
       fn(raw, valid);
@@ -1021,7 +1041,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // rank order, and reports when they do not contain the nucleus; only then does the row need the
   // exact path.
   bool trim_failed = false;
-  if (!large_k && sh_first[a.chunks] >= static_cast<uint32_t>(kNucleusCap)) {
+  if (!large_k && sh_all >= static_cast<uint32_t>(kNucleusCap)) {  // head == 0 here
     const float fmax = key_to_float(rmax), fthr = key_to_float(thr);
     const float span = fmax - fthr;
     const float scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
@@ -1111,6 +1131,22 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       base += static_cast<uint32_t>(__popcll(hits[u]));
     }
   };
+  if (head != 0u) {
+#pragma unroll
+    for (int b = 0; b < kAheadChunks * kAhead / kGather; ++b) {
+      if (b * kGather / kAhead < a.chunks) {
+        u64 raw[kGather];
+        bool valid[kGather];
+#pragma unroll
+        for (int u = 0; u < kGather; ++u) {
+          const int q = b * kGather + u, c = q / kAhead;
+          raw[u] = pre[q];
+          valid[u] = c < a.chunks && static_cast<uint32_t>((q % kAhead) * kFinishBlock + tid) < sh_cnt[c < a.chunks ? c : 0];
+        }
+        consume(raw, valid);
+      }
+    }
+  }
   flat_batches(consume);
   best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
   uint32_t n_c = sh_count;
