@@ -226,6 +226,32 @@ int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int 
   if (!logits || !out_tokens) return Fail(MI355X_E_INVALID, "null logits or output");
   if (dtype != MI355X_F32 && dtype != MI355X_F16) return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
   if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
+  // fp32 rows of more than a few workgroups' worth go through the fused selection kernel (k = 1, ids only)
+  const int fused_chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
+  if (dtype == MI355X_F32 && vocab > 64 && fused_chunks * ms::kSmallCap <= ms::kAllCap &&
+      rows * fused_chunks >= ms::kArgmaxFusedMinBlocks) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    ms::SampleArgs f{};
+    if (int r = MakeXform(ctx, xf, rows, vocab, s, &f.xf)) return r;
+    f.logits = static_cast<const float*>(logits);
+    f.row_stride = row_stride;
+    f.rows = rows;
+    f.vocab = vocab;
+    f.chunks = fused_chunks;
+    f.uniform = mi355x_sample_params{1, 0.0f, 1.0f};
+    f.out_tokens = out_tokens;
+    f.emit_topk = ms::kEmitArgmax;
+    f.cand_small = ctx->cand_small;
+    f.chunk_cnt = ctx->chunk_cnt;
+    f.chunk_max = ctx->chunk_max;
+    f.chunk_next = ctx->chunk_next;
+    f.big = ctx->big;
+    f.big_stride = ctx->big_stride;
+    f.fallback_rows = ctx->fallback_rows;
+    f.poll_limit = ctx->poll_limit;
+    HIP_TRY(ms_launch_sample(&f, nullptr, true, false, false, s));
+    return MI355X_OK;
+  }
   ms::ArgmaxArgs a{};
   if (int r = MakeXform(ctx, xf, rows, vocab, static_cast<hipStream_t>(stream), &a.xf)) return r;
   a.logits = logits;

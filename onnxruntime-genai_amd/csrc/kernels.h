@@ -22,6 +22,8 @@ constexpr int kAllCap = 1024;        // slots a finishing workgroup ranks (16 ch
 constexpr int kNucleusCap = 16384;   // sorted nucleus candidates held in LDS by the finish kernel
 constexpr int kFinishBlock = 1024;
 
+constexpr int kEmitArgmax = 2;
+constexpr int kArgmaxFusedMinBlocks = 1;  // rows x 32768-id chunks from which mi355x_argmax uses the fused kernel
 constexpr int kModeTopkSmall = 0;
 constexpr int kModeNucleus = 1;
 constexpr int kModeGeneral = 2;
@@ -60,8 +62,9 @@ struct SampleArgs {
   size_t big_stride;
   uint32_t* fallback_rows;  // cumulative count of rows finished by the general path; bit 31: a wait gave up
   int poll_limit;           // polls a finishing workgroup waits for another workgroup's list
-  int emit_topk;            // != 0: write the k best (id, raw score) per row instead of sampling
-  float* out_scores;        // [rows, k], emit_topk only (out_tokens is [rows, k] then)
+  int emit_topk;            // 1: write the k best (id, raw score) per row instead of sampling; 2 (kEmitArgmax): the
+                            // best id only, k = 1, with ArgMax's rule that a NaN at id 0 wins (src/search.h:9-29)
+  float* out_scores;        // [rows, k], emit_topk == 1 only (out_tokens is [rows, k] then)
 };
 
 struct ArgmaxArgs {

@@ -80,6 +80,7 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const 
     if (i < V) {
       const float x = xform_value(lrow[i], a.xf.penalty, a.xf.eos, i, has_mask ? mrow[i >> 5] : 0u, has_mask, false, n_eos, ban_row);
       k = make_key64(order_key(x), static_cast<uint32_t>(i));
+      if (i == 0 && x != x && a.emit_topk == kEmitArgmax) k = ~0ull;  // ArgMax starts from id 0 and nothing compares above a NaN
     }
     scratch[i] = k;
   }
@@ -94,7 +95,7 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const 
       for (int jj = 0; jj < j && !dup; ++jj) dup = (h[jj] == tok);
       if (dup) continue;
       const float x = xform_value(lrow[tok], a.xf.penalty, a.xf.eos, tok, has_mask ? mrow[tok >> 5] : 0u, has_mask, true, n_eos, ban_row);
-      scratch[tok] = make_key64(order_key(x), static_cast<uint32_t>(tok));
+      scratch[tok] = (tok == 0 && x != x && a.emit_topk == kEmitArgmax) ? ~0ull : make_key64(order_key(x), static_cast<uint32_t>(tok));
     }
     __syncthreads();
   }
@@ -104,7 +105,7 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const 
     for (int j = threadIdx.x; j < kk; j += blockDim.x) {
       const uint32_t id = key64_index(scratch[j]);
       a.out_tokens[static_cast<size_t>(row) * prm.k + j] = static_cast<int32_t>(id);
-      a.out_scores[static_cast<size_t>(row) * prm.k + j] = lrow[id];  // the value itself: keys do not tell -0 from +0
+      if (a.out_scores) a.out_scores[static_cast<size_t>(row) * prm.k + j] = lrow[id];  // the value itself: keys do not tell -0 from +0
     }
     if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
     return;
@@ -157,6 +158,7 @@ struct FusedShared {
   uint32_t wave_val[kSMaxWaves];
   u64 wave_val64[kSMaxWaves];
   uint32_t count, flag;
+  uint32_t nan0;  // the processed logit of id 0 is a NaN (set in chunk 0; used by the argmax output)
   uint32_t n_extra;
   float extra_val[kExtraCap];     // processed logits of the history ids of this chunk ...
   uint32_t extra_idx[kExtraCap];  // ... and their ids
@@ -425,7 +427,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   bool extra_overflow = false;
   if (XFORM && active) {
     const int n_eos = a.xf.eos_count(row);
-    if (tid == 0) sm.n_extra = 0u;
+    if (tid == 0) {
+      sm.n_extra = 0u;
+      sm.nan0 = 0u;
+    }
 #pragma unroll
     for (int q = 0; q < kWordsPerThread; ++q) {
       const int i = tid + q * kSBlock;
@@ -452,8 +457,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
             const uint32_t slot = atomicAdd(&sm.n_extra, 1u);
             if (slot < static_cast<uint32_t>(kExtraCap)) {
               const uint32_t mw = has_mask ? mrow[id >> 5] : 0u;
-              sm.extra_val[slot] = xform_value(lrow[id], penalty, a.xf.eos, id, mw, has_mask, true, n_eos, ban_row);
+              const float val = xform_value(lrow[id], penalty, a.xf.eos, id, mw, has_mask, true, n_eos, ban_row);
+              sm.extra_val[slot] = val;
               sm.extra_idx[slot] = static_cast<uint32_t>(id);
+              if (id == 0 && val != val) sm.nan0 = 1u;
             }
           }
         }
@@ -483,7 +490,16 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   for (uint32_t i = tid; i < n_extra; i += kSBlock) fm = fmaxf(fm, sm.extra_val[i]);
   // 0: the thread holds no element
   const uint32_t lmax = (elem_index<kSBlock>(chunk, 0, 0) < V || static_cast<uint32_t>(tid) < n_extra) ? order_key(fm) : 0u;
-  if (tid == 0) sm.count = 0u;
+  if (tid == 0) {
+    sm.count = 0u;
+    if constexpr (!NUCLEUS) {
+      // id 0's processed value is v[0] unless id 0 is in the history (then its owner has set the flag)
+      const bool in_history = XFORM && pen && (sm.hist_bits[0] & 1u) != 0u;
+      const bool is_nan = chunk == 0 && !in_history && v[0] != v[0];
+      if (!(XFORM && active)) sm.nan0 = is_nan ? 1u : 0u;
+      else if (is_nan) sm.nan0 = 1u;
+    }
+  }
 
   if constexpr (NUCLEUS) {
     // Everything within nucleus_depth of the chunk maximum goes to the row's key buffer, in no
@@ -725,6 +741,8 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
       mykey = other > mykey ? other : mykey;
       sort_merge<64, 32, u64>(mykey, lane);
     }
+    // ArgMax starts from id 0 and nothing compares above a NaN (src/search.h:9-29): such a row's answer is 0
+    if (emit_topk == kEmitArgmax && chunk == 0 && lane == 0 && sm.nan0 != 0u) mykey = ~0ull;
     const u64 slot = overflow ? kSlotOverflow : (mykey != 0 ? mykey : kSlotEmpty);
     if (finisher) sm.own[lane] = slot;
     else store_coherent(&dst[lane], slot);
@@ -803,8 +821,9 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
         if (lane < kk) {
           const uint32_t id = key64_index(final_key);
           a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(id);
-          a.out_scores[static_cast<size_t>(row) * prm.k + lane] =
-              a.logits[static_cast<size_t>(row) * a.row_stride + id];  // keys do not tell -0 from +0
+          if (emit_topk == 1)
+            a.out_scores[static_cast<size_t>(row) * prm.k + lane] =
+                a.logits[static_cast<size_t>(row) * a.row_stride + id];  // keys do not tell -0 from +0
         }
       } else {
         {
