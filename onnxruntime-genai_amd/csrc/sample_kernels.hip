@@ -67,7 +67,13 @@ __device__ __forceinline__ RowOutputs row_outputs(const SampleArgs& a, int row) 
 // Exact general path for one row, any (k, p, T), any vocabulary size: rebuilds the processed row as
 // key64s in global scratch, sorts all of it, then runs the reference algorithm on the sorted row.
 // Run by one whole block.  scratch holds next_pow2(vocab) entries.
-__device__ __forceinline__ void general_row(const SampleArgs& a, int row, const mi355x_sample_params prm, u64* scratch, SeqShared& sh) {
+struct SortInGlobalMemory {
+  __device__ void operator()(u64* keys, int n2, int) const { block_sort_desc(keys, n2); }
+};
+
+template <typename SortFn = SortInGlobalMemory>
+__device__ __forceinline__ void general_row(const SampleArgs& a, int row, const mi355x_sample_params prm, u64* scratch, SeqShared& sh,
+                                            SortFn sort_desc = SortFn{}) {
   const int V = a.vocab;
   const float* lrow = a.logits + static_cast<size_t>(row) * a.row_stride;
   const int n2 = next_pow2(V);
@@ -99,7 +105,7 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const 
     }
     __syncthreads();
   }
-  block_sort_desc(scratch, n2);
+  sort_desc(scratch, n2, V);  // descending; entries from V on are 0
   if (a.emit_topk) {
     const int kk = prm.k < V ? prm.k : V;
     for (int j = threadIdx.x; j < kk; j += blockDim.x) {
@@ -966,6 +972,72 @@ __device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n,
   return true;
 }
 
+// Sorts n2 keys (a power of two, at least two tiles) in global memory, descending, by a block of
+// kFinishBlock threads with a tile of kNucleusCap keys in LDS: every tile is sorted in LDS (alternating
+// directions), then the remaining levels of the bitonic network run their long-distance steps in
+// global memory and the 14 short-distance steps of each level tile by tile in LDS.  The first n_real
+// keys are real, the rest 0.  About six times faster than the same network entirely in global memory.
+__device__ __noinline__ void tiled_sort_desc(u64* g, int n2, int n_real, u64* lds, uint32_t* bucket_start, uint32_t* red32) {
+  constexpr int T = kNucleusCap;
+  const int tid = threadIdx.x;
+  const int tiles = n2 / T;
+  for (int t = 0; t < tiles; ++t) {
+    u64* src = g + static_cast<size_t>(t) * T;
+    int n_t = n_real - t * T;
+    n_t = n_t < 0 ? 0 : (n_t > T ? T : n_t);
+    uint32_t kmax = 0u, kmin_c = 0u;  // largest score key, complement of the smallest
+    for (int i = tid; i < T; i += kFinishBlock) {
+      const u64 k = src[i];
+      lds[i] = k;
+      if (i < n_t) {
+        kmax = key64_okey(k) > kmax ? key64_okey(k) : kmax;
+        kmin_c = ~key64_okey(k) > kmin_c ? ~key64_okey(k) : kmin_c;
+      }
+    }
+    kmax = block_max<uint32_t>(kmax, red32);
+    kmin_c = block_max<uint32_t>(kmin_c, red32);  // the barriers also publish the tile
+    bool done = false;
+    if (n_t > kFinishBlock && kmax != 0u && ~kmin_c != 0u)
+      done = bucket_sort_desc(lds, bucket_start, n_t, key_to_float(kmax), key_to_float(~kmin_c), red32);
+    if (!done) block_sort_desc_regs<T / kFinishBlock>(lds);  // the whole tile, zeros last
+    for (int i = tid; i < T; i += kFinishBlock) src[(t & 1) ? T - 1 - i : i] = lds[i];
+    __syncthreads();
+  }
+  for (int k = 2 * T; k <= n2; k <<= 1) {
+    for (int j = k >> 1; j >= T; j >>= 1) {
+      for (int p = tid; p < n2 / 2; p += kFinishBlock) {
+        const int i = ((p & ~(j - 1)) << 1) | (p & (j - 1));  // bit j clear
+        const u64 x = g[i], y = g[i | j];
+        const bool desc = (i & k) == 0;
+        if ((x < y) == desc) {
+          g[i] = y;
+          g[i | j] = x;
+        }
+      }
+      __syncthreads();
+    }
+    for (int t = 0; t < tiles; ++t) {
+      u64* src = g + static_cast<size_t>(t) * T;
+      for (int i = tid; i < T; i += kFinishBlock) lds[i] = src[i];
+      __syncthreads();
+      const bool desc = ((t * T) & k) == 0;  // one direction per tile: k >= 2 T
+      for (int j = T >> 1; j >= 1; j >>= 1) {
+        for (int p = tid; p < T / 2; p += kFinishBlock) {
+          const int i = ((p & ~(j - 1)) << 1) | (p & (j - 1));
+          const u64 x = lds[i], y = lds[i | j];
+          if ((x < y) == desc) {
+            lds[i] = y;
+            lds[i | j] = x;
+          }
+        }
+        __syncthreads();
+      }
+      for (int i = tid; i < T; i += kFinishBlock) src[i] = lds[i];
+      __syncthreads();
+    }
+  }
+}
+
 // Per-row finish of the nucleus path: gathers the candidates the streaming pass left in `big`,
 // sorts them in LDS and runs the exact epilogue.  One block of kFinishBlock threads per row;
 // dynamic LDS: kNucleusCap key64s + the bucket table of the sort.
@@ -1210,7 +1282,11 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   }
   if (!ok) {
     __syncthreads();
-    general_row(a, row, prm, big_row, seqsh);
+    u64* const tile = lds_keys;
+    general_row(a, row, prm, big_row, seqsh, [=](u64* keys, int n2, int n_real) {
+      if (n2 >= 2 * kNucleusCap) tiled_sort_desc(keys, n2, n_real, tile, bucket_start, red32);
+      else block_sort_desc(keys, n2);
+    });
   }
 }
 
