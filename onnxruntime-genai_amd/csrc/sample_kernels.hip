@@ -763,7 +763,8 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
     tab.hi = static_cast<uint32_t>(t >> 32);
   }
   const double u = emit_topk ? 0.0 : uniforms[row];
-  __syncthreads();  // sm.own
+  // sm.own is written by wave 0; with at most four chunks wave 0 alone reads it (a wave's LDS accesses execute in order)
+  if (n_chunks > 4) __syncthreads();
   u64* seg = cand_small + static_cast<size_t>(row) * n_chunks * kSmallCap;
   // Wave w merges the sorted lists of chunks 4w .. 4w+3 in registers, straight from global memory;
   // rows of more than four chunks need a second level through LDS.  Wave 0 ends with the row's 64
