@@ -115,6 +115,103 @@ __global__ __launch_bounds__(256) void kv_gather_narrow_kernel(const void* const
 }
 
 // ---- speculative-decoding verification ---------------------------------------------------------------
+// block_discrete_draw for at most WINDOWS windows of blockDim * ITEMS weights, read once: the weights stay in
+// registers between the pass that sums them and the pass that scans them.  Reports weights that sum to
+// exactly 0 through all_zero instead of drawing from them.  Same arithmetic and the same sequential
+// replay near a boundary as block_discrete_draw.
+template <int ITEMS, int WINDOWS, typename GetW>
+__device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u, SeqShared& sh, float* stage, bool* all_zero) {
+  const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6, nw = blockDim.x >> 6;
+  const int span = static_cast<int>(blockDim.x) * ITEMS;
+  *all_zero = false;
+  float wv[WINDOWS][ITEMS];
+  double part = 0.0;
+#pragma unroll
+  for (int c = 0; c < WINDOWS; ++c) {
+    const int i0 = c * span;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) wv[c][j] = 0.0f;
+    if (i0 < n) {
+      window_fetch<ITEMS>(wv[c], i0, (n - i0 < span) ? n : i0 + span, w, stage);
+      __syncthreads();  // the staging buffer is rewritten by the next window
+#pragma unroll
+      for (int j = 0; j < ITEMS; ++j) part += static_cast<double>(wv[c][j]);
+    }
+  }
+  part = wave_sum<double>(part);
+  if (lane == 0) sh.dred[wave] = part;
+  __syncthreads();
+  double total = 0.0;
+  for (int k = 0; k < nw; ++k) total += sh.dred[k];
+  __syncthreads();
+  if (total != total) return 0;  // NaN weights: see block_discrete_draw
+  if (total == 0.0) {
+    *all_zero = true;
+    return 0;
+  }
+  if (n < 2) return 0;
+  const double guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16 * total;
+  const double target = u * total;
+  double carry = 0.0;
+  int first = kIntMax;
+  int risky = 0;
+#pragma unroll
+  for (int c = 0; c < WINDOWS; ++c) {
+    const int i0 = c * span;
+    if (i0 < n) {
+      const int base = i0 + tid * ITEMS;
+      double loc = 0.0;
+#pragma unroll
+      for (int j = 0; j < ITEMS; ++j) loc += static_cast<double>(wv[c][j]);
+      double inc = loc;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const double y = __shfl_up(inc, d, 64);
+        if (lane >= d) inc += y;
+      }
+      if (lane == 63) sh.dscan[wave] = inc;
+      __syncthreads();
+      double wp = carry;
+      for (int k = 0; k < wave; ++k) wp += sh.dscan[k];
+      double block_total = 0.0;
+      for (int k = 0; k < nw; ++k) block_total += sh.dscan[k];
+      double run = wp + (inc - loc);
+#pragma unroll
+      for (int j = 0; j < ITEMS; ++j) {
+        const int idx = base + j;
+        if (idx < n) {
+          run += static_cast<double>(wv[c][j]);
+          if (idx != n - 1 && fabs(run - target) <= guard) risky = 1;
+          if ((idx == n - 1 || run >= target) && idx < first) first = idx;  // the last value is forced to 1
+        }
+      }
+      carry += block_total;
+      __syncthreads();
+    }
+  }
+  int a = first, b = risky ? 0 : 1;
+  block_min2(a, b, sh);
+  if (b != 0) return a;
+  if (tid == 0) {  // sequential replay with the reference's own operations
+    double sum = 0.0;
+    for (int i = 0; i < n; ++i) sum += static_cast<double>(w(i));
+    double cp = 0.0;
+    int pos = n - 1;
+    for (int i = 0; i < n - 1; ++i) {
+      cp += static_cast<double>(w(i)) / sum;
+      if (cp >= u) {
+        pos = i;
+        break;
+      }
+    }
+    sh.bcast_i = pos;
+  }
+  __syncthreads();
+  const int pos = sh.bcast_i;
+  __syncthreads();
+  return pos;
+}
+
 // One 1024-thread block per batch entry.  Accept loop of SpeculativeDecodingStrategy::RunRound
 // (src/speculative_decoding_strategy.cpp:718-762) on dense distributions, then the round's single
 // categorical draw: the residual max(p-q,0) at the first rejected position (SampleCorrectionToken,
@@ -126,7 +223,7 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
                                                            int32_t* accepted_len, int32_t* final_token) {
   __shared__ SeqShared sh;
   __shared__ __align__(16) float stage[1024 * 8];
-  __shared__ int sh_n, sh_any;
+  __shared__ int sh_n;
   const int b = blockIdx.x;
   const size_t base = static_cast<size_t>(b) * (K + 1) * vocab;
   if (threadIdx.x < 64) {
@@ -146,34 +243,41 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
       const int f = first_lane(__ballot(reject));
       if (f >= 0) rejected_at = n0 + f;
     }
-    if (threadIdx.x == 0) {
-      sh_n = rejected_at;
-      sh_any = 0;
-    }
+    if (threadIdx.x == 0) sh_n = rejected_at;
   }
   __syncthreads();
   const int n = sh_n;
   const float* pt = p_target + base + static_cast<size_t>(n) * vocab;
   const float* pd = p_draft + base + static_cast<size_t>(n) * vocab;
-  bool use_residual = false;
-  if (n < K) {
-    int any = 0;
-#pragma unroll 8
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) any |= (pt[i] - pd[i] > 0.0f);
-    if (any) sh_any = 1;  // the reference's fp32 "sum > 0" holds iff some residual is positive
-    __syncthreads();
-    use_residual = sh_any != 0;
-  }
-  int pos;
-  if (use_residual) {
+  // The residual max(p - q, 0) at the first rejected position is drawn from unless it is all zero
+  // (the reference's fp32 "sum > 0" holds iff some residual is positive, and so does the double sum
+  // the draw starts with): then, and on full acceptance, the target row itself is.  Vocabularies of up
+  // to four windows are read once per draw.
+  constexpr int kItems = 8, kWindows = 4;
+  const bool once = vocab <= kWindows * kItems * 1024;
+  int pos = 0;
+  bool from_target = n >= K;
+  if (!from_target) {
     auto w = [=](int i) {
       const float d = pt[i] - pd[i];
       return d > 0.0f ? d : 0.0f;
     };
-    pos = block_discrete_draw<8>(vocab, w, sample_u[b], sh, stage);
-  } else {
+    if (once) {
+      pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &from_target);
+    } else {
+      int any = 0;
+#pragma unroll 8
+      for (int i = threadIdx.x; i < vocab; i += blockDim.x) any |= (pt[i] - pd[i] > 0.0f);
+      from_target = __syncthreads_or(any) == 0;
+      if (!from_target) pos = block_discrete_draw<kItems>(vocab, w, sample_u[b], sh, stage);
+    }
+    __syncthreads();
+  }
+  if (from_target) {
     auto w = [=](int i) { return pt[i]; };
-    pos = block_discrete_draw<8>(vocab, w, sample_u[b], sh, stage);
+    bool unused;
+    pos = once ? block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &unused)
+               : block_discrete_draw<kItems>(vocab, w, sample_u[b], sh, stage);
   }
   if (threadIdx.x == 0) {
     accepted_len[b] = n;
