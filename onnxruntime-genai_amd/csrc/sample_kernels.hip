@@ -978,7 +978,7 @@ __device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n,
 // directions), then the remaining levels of the bitonic network run their long-distance steps in
 // global memory and the 14 short-distance steps of each level tile by tile in LDS.  The first n_real
 // keys are real, the rest 0.  About six times faster than the same network entirely in global memory.
-__device__ __noinline__ void tiled_sort_desc(u64* g, int n2, int n_real, u64* lds, uint32_t* bucket_start, uint32_t* red32) {
+__device__ __forceinline__ void tiled_sort_desc(u64* g, int n2, int n_real, u64* lds, uint32_t* bucket_start, uint32_t* red32) {
   constexpr int T = kNucleusCap;
   const int tid = threadIdx.x;
   const int tiles = n2 / T;
@@ -987,6 +987,7 @@ __device__ __noinline__ void tiled_sort_desc(u64* g, int n2, int n_real, u64* ld
     int n_t = n_real - t * T;
     n_t = n_t < 0 ? 0 : (n_t > T ? T : n_t);
     uint32_t kmax = 0u, kmin_c = 0u;  // largest score key, complement of the smallest
+#pragma unroll 4
     for (int i = tid; i < T; i += kFinishBlock) {
       const u64 k = src[i];
       lds[i] = k;
@@ -1001,11 +1002,13 @@ __device__ __noinline__ void tiled_sort_desc(u64* g, int n2, int n_real, u64* ld
     if (n_t > kFinishBlock && kmax != 0u && ~kmin_c != 0u)
       done = bucket_sort_desc(lds, bucket_start, n_t, key_to_float(kmax), key_to_float(~kmin_c), red32);
     if (!done) block_sort_desc_regs<T / kFinishBlock>(lds);  // the whole tile, zeros last
+#pragma unroll 4
     for (int i = tid; i < T; i += kFinishBlock) src[(t & 1) ? T - 1 - i : i] = lds[i];
     __syncthreads();
   }
   for (int k = 2 * T; k <= n2; k <<= 1) {
     for (int j = k >> 1; j >= T; j >>= 1) {
+#pragma unroll 2
       for (int p = tid; p < n2 / 2; p += kFinishBlock) {
         const int i = ((p & ~(j - 1)) << 1) | (p & (j - 1));  // bit j clear
         const u64 x = g[i], y = g[i | j];
@@ -1019,10 +1022,12 @@ __device__ __noinline__ void tiled_sort_desc(u64* g, int n2, int n_real, u64* ld
     }
     for (int t = 0; t < tiles; ++t) {
       u64* src = g + static_cast<size_t>(t) * T;
+#pragma unroll 4
       for (int i = tid; i < T; i += kFinishBlock) lds[i] = src[i];
       __syncthreads();
       const bool desc = ((t * T) & k) == 0;  // one direction per tile: k >= 2 T
       for (int j = T >> 1; j >= 1; j >>= 1) {
+#pragma unroll 2
         for (int p = tid; p < T / 2; p += kFinishBlock) {
           const int i = ((p & ~(j - 1)) << 1) | (p & (j - 1));
           const u64 x = lds[i], y = lds[i | j];
@@ -1033,6 +1038,7 @@ __device__ __noinline__ void tiled_sort_desc(u64* g, int n2, int n_real, u64* ld
         }
         __syncthreads();
       }
+#pragma unroll 4
       for (int i = tid; i < T; i += kFinishBlock) src[i] = lds[i];
       __syncthreads();
     }
