@@ -976,32 +976,19 @@ __device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n,
 // Sorts n2 keys (a power of two, at least two tiles) in global memory, descending, by a block of
 // kFinishBlock threads with a tile of kNucleusCap keys in LDS: every tile is sorted in LDS (alternating
 // directions), then the remaining levels of the bitonic network run their long-distance steps in
-// global memory and the 14 short-distance steps of each level tile by tile in LDS.  The first n_real
-// keys are real, the rest 0.  About six times faster than the same network entirely in global memory.
-__device__ __forceinline__ void tiled_sort_desc(u64* g, int n2, int n_real, u64* lds, uint32_t* bucket_start, uint32_t* red32) {
+// global memory and the 14 short-distance steps of each level tile by tile in LDS.  About twice as
+// fast as the same network entirely in global memory.
+__device__ __forceinline__ void tiled_sort_desc(u64* g, int n2, u64* lds) {
   constexpr int T = kNucleusCap;
   const int tid = threadIdx.x;
   const int tiles = n2 / T;
   for (int t = 0; t < tiles; ++t) {
     u64* src = g + static_cast<size_t>(t) * T;
-    int n_t = n_real - t * T;
-    n_t = n_t < 0 ? 0 : (n_t > T ? T : n_t);
-    uint32_t kmax = 0u, kmin_c = 0u;  // largest score key, complement of the smallest
-#pragma unroll 4
-    for (int i = tid; i < T; i += kFinishBlock) {
-      const u64 k = src[i];
-      lds[i] = k;
-      if (i < n_t) {
-        kmax = key64_okey(k) > kmax ? key64_okey(k) : kmax;
-        kmin_c = ~key64_okey(k) > kmin_c ? ~key64_okey(k) : kmin_c;
-      }
-    }
-    kmax = block_max<uint32_t>(kmax, red32);
-    kmin_c = block_max<uint32_t>(kmin_c, red32);  // the barriers also publish the tile
-    bool done = false;
-    if (n_t > kFinishBlock && kmax != 0u && ~kmin_c != 0u)
-      done = bucket_sort_desc(lds, bucket_start, n_t, key_to_float(kmax), key_to_float(~kmin_c), red32);
-    if (!done) block_sort_desc_regs<T / kFinishBlock>(lds);  // the whole tile, zeros last
+    for (int i = tid; i < T; i += kFinishBlock) lds[i] = src[i];
+    __syncthreads();
+    // the whole tile, zeros last; the plain network, inline: a call to one of the faster out-of-line sorts inside
+    // this loop makes the kernel spill, and a kernel that uses scratch memory at all starts 2.5 us later
+    block_sort_desc(lds, T);
 #pragma unroll 4
     for (int i = tid; i < T; i += kFinishBlock) src[(t & 1) ? T - 1 - i : i] = lds[i];
     __syncthreads();
@@ -1291,7 +1278,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     __syncthreads();
     u64* const tile = lds_keys;
     general_row(a, row, prm, big_row, seqsh, [=](u64* keys, int n2, int n_real) {
-      if (n2 >= 2 * kNucleusCap) tiled_sort_desc(keys, n2, n_real, tile, bucket_start, red32);
+      if (n2 >= 2 * kNucleusCap) tiled_sort_desc(keys, n2, tile);
       else block_sort_desc(keys, n2);
     });
   }
