@@ -18,10 +18,13 @@
 //   accept/correction math: pinned by the reference's own known-answer tests and, where it builds,
 //   by oracle/_ref (the unmodified reference headers compiled from /root/reference).
 //   beam top-2B selection: pinned by brute force (full stable sort) on small inputs.
-//   BeamSearchScorer / BeamHypotheses / sequence append: pinned by hand-worked cases and invariants
-//   of the HuggingFace algorithm it follows; the reference's golden beam sequences need ONNX Runtime
-//   and a model, so they cannot be replayed: exact-value parity of the scorer against the reference
-//   binary is "parity unpinned".
+//   argmax, BeamSearch_Cpu::SelectTop, BeamSearchScorer::Process (candidates that are not EOS), Finalize,
+//   GetBeamHypotheses and the beam sequence append: pinned by the reference's own golden generations
+//   (ModelTests.GreedySearchGptFp32 / BeamSearchGptFp32, test/model_tests.cpp:57-130), replayed from
+//   the logits of the tiny GPT-2 those tests load (tests/golden/gpt2_search_vectors.npz).
+//   BeamSearchScorer's EOS branch (BeamHypotheses::Add / CanImprove, done batches, padding): no EOS
+//   is produced in those golden runs; it is pinned only by hand-worked cases and invariants of the
+//   HuggingFace algorithm it follows, so the exact values of that branch are "parity unpinned".
 //   KV gather: pinned by numpy.take.
 //   Cast conversions (fp16/bf16 <-> fp32, int32 -> int64): pinned by known answers and, for
 //   fp32 -> fp16, by agreement with IEEE round-to-nearest on every value that is not an exact tie
