@@ -61,6 +61,7 @@ struct mi355x_search_ctx {
   void** ptr_table{};      // device copy of pointer tables (kv gather)
   size_t ptr_table_cap{};
   float* beam_row_scores{};
+  ms::u64* seg_cand{};  // [max_rows][max_segs][kBeamMaxCand] beam-search candidates per segment
   int max_segs{};
   uint32_t* seg_max{};
   double* seg_sum{};
@@ -183,6 +184,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   c->max_segs = (max_vocab + ms::kSegElems - 1) / ms::kSegElems;
   ok(c->Alloc(&c->seg_max, static_cast<size_t>(max_rows) * c->max_segs, false));
   ok(c->Alloc(&c->seg_sum, static_cast<size_t>(max_rows) * c->max_segs, false));
+  ok(c->Alloc(&c->seg_cand, static_cast<size_t>(max_rows) * c->max_segs * ms::kBeamMaxCand, false));
   ok(c->Alloc(&c->seg_step, static_cast<size_t>(max_rows) * c->max_segs, false));
   ok(c->Alloc(&c->row_max, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->row_sum, static_cast<size_t>(max_rows), false));
@@ -411,7 +413,7 @@ int mi355x_softmax(mi355x_search_ctx* ctx, void* stream, float* scores, int64_t 
   ms::SeqSumArgs q{};
   if (FillSeqSum(ctx, scores, row_stride, rows, vocab, 1.0f / temperature, &q)) {
     // long rows: the exact sum is spread over the whole GPU, then an element-wise pass finishes
-    HIP_TRY(ms_launch_seqsum(&q, MI355X_F32, s));
+    HIP_TRY(ms_launch_seqsum(&q, MI355X_F32, 0, s));
     HIP_TRY(ms_launch_softmax_apply(scores, row_stride, &q, log_softmax, s));
   } else {
     HIP_TRY(ms_launch_softmax(scores, row_stride, rows, vocab, temperature, log_softmax, s));
@@ -448,9 +450,20 @@ int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits,
   a.out_beams = out_beam_indices;
   ms::SeqSumArgs q{};
   if (FillSeqSum(ctx, logits, row_stride, batch * beams, vocab, 1.0f, &q)) {
-    HIP_TRY(ms_launch_seqsum(&q, dtype, static_cast<hipStream_t>(stream)));
     a.row_max = q.out_max;
     a.row_sum = q.out_sum;
+    if (static_cast<long long>(beams) * q.segs * 2 * beams <= ms::kBeamFinCap) {
+      // long rows: the segments list their best logits while the maxima are taken, the exact sums follow,
+      // and one workgroup per batch entry scores the listed candidates
+      a.seg_cand = ctx->seg_cand;
+      a.seg_max = q.seg_max;
+      a.segs = q.segs;
+      HIP_TRY(ms_launch_beam_segments(&a, dtype, static_cast<hipStream_t>(stream)));
+      HIP_TRY(ms_launch_seqsum(&q, dtype, 1, static_cast<hipStream_t>(stream)));
+      HIP_TRY(ms_launch_beam_finish(&a, dtype, static_cast<hipStream_t>(stream)));
+      return MI355X_OK;
+    }
+    HIP_TRY(ms_launch_seqsum(&q, dtype, 0, static_cast<hipStream_t>(stream)));
   }
   HIP_TRY(ms_launch_beam_select(&a, dtype, static_cast<hipStream_t>(stream)));
   return MI355X_OK;

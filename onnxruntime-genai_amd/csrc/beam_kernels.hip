@@ -3,6 +3,7 @@
 #include "kernels.h"
 #include "block_seq.h"
 #include "wave_select.h"
+#include "seg_io.h"
 
 namespace ms {
 
@@ -270,6 +271,179 @@ __global__ __launch_bounds__(256) void beam_append_kernel(const int32_t* seq, in
   if (threadIdx.x == 0) dst[current_length] = tokens[i];
 }
 
+
+// ---- long rows: candidates per segment, scored once the exact sum is known --------------------------------
+//
+// The final score ((x - max) - log(sum)) + beam_score is a non-decreasing function of the logit x, so the
+// 2*beams best final scores of a batch entry belong to elements that are among the 2*beams largest logits of
+// their own segment.  beam_seg_kernel lists those per segment (and writes the segment maxima the exact sum
+// needs, which saves that kernel's own pass); beam_fin_kernel scores the listed elements and keeps the best by
+// (final score desc, beam * vocab + token asc), the order of the flat partial_sort of src/search.cpp:148-163.
+// Rounding can give different logits the same final score, and then the lowest index wins, which the logit
+// order does not know.  A segment whose list is full (it may hold more elements of the same final score as its
+// last entry) and whose last entry reaches the final score of the entry's 2*beams-th best makes the finishing
+// workgroup rescan the rows themselves; so do non-finite maxima and entries with fewer than 2*beams numbers.
+
+constexpr int kSegCandCap = 512;        // candidates a segment may list before it reports an overflow
+constexpr u64 kSegOverflow = ~0ull;     // first entry of a segment that listed more than kSegCandCap
+
+template <typename InT>
+__global__ __launch_bounds__(kSegBlock) void beam_seg_kernel(const BeamArgs a) {
+  __shared__ u64 list[kSegCandCap];
+  __shared__ uint32_t pool[64];
+  __shared__ uint32_t red[4];
+  __shared__ uint32_t count;
+  const int seg = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
+  const int V = a.vocab, m = 2 * a.beams;
+  const InT* x = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
+  float v[kSegPer];
+  seg_load<InT>(x, aligned, V, seg, -__builtin_inff(), v);
+  float fm = -__builtin_inff();
+#pragma unroll
+  for (int e = 0; e < kSegPer; ++e) fm = fmaxf(fm, v[e]);
+  const uint32_t mkey = order_key(fm);
+  const uint32_t smax = block_max<uint32_t>(mkey, red);
+  if (tid == 0) a.seg_max[static_cast<size_t>(row) * a.segs + seg] = smax;
+  const uint32_t offer = seg_index<InT>(seg, 0) < V ? mkey : 0u;  // threads past the end of the row offer nothing
+  const uint32_t tau = block_pool_bound(offer, m, kSegBlock / 64, pool);
+  if (tid == 0) count = 0u;
+  __syncthreads();
+#pragma unroll
+  for (int e = 0; e < kSegPer; ++e) {
+    const int idx = seg_index<InT>(seg, e);
+    const uint32_t k = order_key(v[e]);
+    const bool cand = idx < V && (tau == 0u || k >= tau);  // tau == 0: fewer than m offers, list everything
+    const uint32_t pos = wave_slot(cand, &count);
+    if (cand && pos < kSegCandCap) list[pos] = make_key64(k, static_cast<uint32_t>(idx));
+  }
+  __syncthreads();
+  const int n = static_cast<int>(count);
+  u64* out = a.seg_cand + (static_cast<size_t>(row) * a.segs + seg) * m;
+  if (n > kSegCandCap) {
+    if (tid < m) out[tid] = tid == 0 ? kSegOverflow : 0ull;
+    return;
+  }
+  if (n <= 64) {  // the usual case: one wave sorts the list in registers
+    if (tid < 64) {
+      const u64 k = wave_sort_desc_fast<u64>(tid < n ? list[tid] : 0ull);
+      if (tid < m) out[tid] = k;
+    }
+    return;
+  }
+  int n2 = 128;
+  while (n2 < n) n2 <<= 1;
+  for (int p = n + tid; p < n2; p += kSegBlock) list[p] = 0ull;
+  __syncthreads();
+  block_sort_desc(list, n2);
+  if (tid < m) out[tid] = list[tid];
+}
+
+template <typename InT>
+__global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a) {
+  constexpr int R = kBeamFinCap / 256;
+  __shared__ u64 red64[4];
+  __shared__ uint32_t red[4];
+  __shared__ u64 best_list[kBeamMaxCand];
+  __shared__ float s_max[kBeamMaxCand / 2], s_lse[kBeamMaxCand / 2], s_bs[kBeamMaxCand / 2];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const int V = a.vocab, m = 2 * a.beams, per_row = a.segs * m, n = a.beams * per_row;
+  bool odd = false;  // a row whose maximum is not a finite number: its scores need not follow the logit order
+  if (tid < a.beams) {
+    const int row = b * a.beams + tid;
+    s_max[tid] = a.row_max[row];
+    s_lse[tid] = em::logf_exact(a.row_sum[row]);
+    s_bs[tid] = a.beam_scores[row];
+    odd = !(fabsf(s_max[tid]) < __builtin_inff());
+  }
+  __syncthreads();
+  u64 key[R];
+  uint32_t full_reach = odd ? 0xffffffffu : 0u;  // best final score among the last entries of full lists
+  // entry p = tid + 256 r of the batch entry's lists: beam p / per_row, position j = p % m inside its list
+  int beam = tid / per_row, j = tid % m;
+  int q = tid - beam * per_row;
+  const int dj = 256 % m;
+  const u64* cand = a.seg_cand + static_cast<size_t>(b * a.beams) * per_row;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    key[r] = 0ull;
+    if (tid + r * 256 < n) {
+      const u64 c = cand[tid + r * 256];
+      if (c == kSegOverflow) {
+        full_reach = 0xffffffffu;
+      } else if (c != 0ull) {
+        const float f = ((key_to_float(key64_okey(c)) - s_max[beam]) - s_lse[beam]) + s_bs[beam];
+        const uint32_t fk = order_key(f);
+        key[r] = make_key64(fk, static_cast<uint32_t>(beam) * static_cast<uint32_t>(V) + key64_index(c));
+        if (j == m - 1 && fk > full_reach) full_reach = fk;
+      }
+    }
+    q += 256;
+    while (q >= per_row) q -= per_row, ++beam;
+    j += dj;
+    if (j >= m) j -= m;
+  }
+  u64 last = ~0ull;
+  for (int j = 0; j < m; ++j) {
+    u64 best = 0ull;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (key[r] < last && key[r] > best) best = key[r];
+    best = block_max<u64>(best, red64);
+    if (tid == 0) best_list[j] = best;
+    last = best;  // 0 once nothing is left: later rounds find nothing either
+  }
+  const uint32_t cut = key64_okey(last);
+  const uint32_t reach = block_max<uint32_t>(full_reach, red);
+  if (cut == 0u || reach >= cut) {
+    // rescan the rows: the m best one at a time, each the largest key strictly below the previous one
+    last = ~0ull;
+    for (int j = 0; j < m; ++j) {
+      u64 best = 0ull;
+      for (int beam = 0; beam < a.beams; ++beam) {
+        const InT* x = static_cast<const InT*>(a.logits) + static_cast<size_t>(b * a.beams + beam) * a.row_stride;
+        const float mx = s_max[beam], lse = s_lse[beam], bs = s_bs[beam];
+        for (int i = tid; i < V; i += 256) {
+          const float f = ((load_one<InT>(x, i) - mx) - lse) + bs;
+          const u64 k = make_key64(order_key(f), static_cast<uint32_t>(beam) * static_cast<uint32_t>(V) + static_cast<uint32_t>(i));
+          if (k < last && k > best) best = k;
+        }
+      }
+      best = block_max<u64>(best, red64);
+      if (tid == 0) best_list[j] = best;
+      last = best;
+    }
+  }
+  __syncthreads();
+  if (tid < m) {
+    const u64 k = best_list[tid];
+    const uint32_t flat = key64_index(k);
+    a.out_scores[b * m + tid] = key_to_float(key64_okey(k));
+    a.out_tokens[b * m + tid] = static_cast<int32_t>(flat % static_cast<uint32_t>(V));
+    a.out_beams[b * m + tid] = static_cast<int32_t>(flat / static_cast<uint32_t>(V));
+  }
+}
+
+}  // namespace ms
+
+extern "C" hipError_t ms_launch_beam_segments(const ms::BeamArgs* a, int dtype, hipStream_t stream) {
+  const dim3 grid(a->segs, a->batch * a->beams), block(ms::kSegBlock);
+  if (dtype == MI355X_F16)
+    hipLaunchKernelGGL(ms::beam_seg_kernel<uint16_t>, grid, block, 0, stream, *a);
+  else
+    hipLaunchKernelGGL(ms::beam_seg_kernel<float>, grid, block, 0, stream, *a);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_beam_finish(const ms::BeamArgs* a, int dtype, hipStream_t stream) {
+  if (dtype == MI355X_F16)
+    hipLaunchKernelGGL(ms::beam_fin_kernel<uint16_t>, dim3(a->batch), dim3(256), 0, stream, *a);
+  else
+    hipLaunchKernelGGL(ms::beam_fin_kernel<float>, dim3(a->batch), dim3(256), 0, stream, *a);
+  return hipGetLastError();
+}
+
+namespace ms {
 }  // namespace ms
 
 extern "C" hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hipStream_t stream) {

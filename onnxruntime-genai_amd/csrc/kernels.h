@@ -131,7 +131,12 @@ struct BeamArgs {
   float* out_scores;          // [batch][2*beams]
   int32_t* out_tokens;
   int32_t* out_beams;
+  // segmented path (long rows): every kSegElems-element segment of a row lists its 2*beams largest logits
+  u64* seg_cand;              // workspace [batch*beams][segs][2*beams] keys (raw logit, token), best first
+  uint32_t* seg_max;          // [batch*beams][segs] order keys of the segment maxima (read by the exact sum)
+  int segs;
 };
+constexpr int kBeamFinCap = 4096;  // beams * segs * 2*beams keys one finishing workgroup holds
 
 // Device-resident BeamSearchScorer state (all pointers device memory).
 struct ScorerState {
@@ -182,7 +187,9 @@ hipError_t ms_launch_cast(const void* in, void* out, size_t count, int kind, hip
 hipError_t ms_launch_logits_handoff(const void* raw, int kind, int rows, int seq_len, int vocab,
                                     const int32_t* token_index, float* out, int64_t out_stride, hipStream_t stream);
 hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hipStream_t stream);
-hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, hipStream_t stream);
+hipError_t ms_launch_beam_segments(const ms::BeamArgs* a, int dtype, hipStream_t stream);
+hipError_t ms_launch_beam_finish(const ms::BeamArgs* a, int dtype, hipStream_t stream);
+hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, int have_seg_max, hipStream_t stream);
 hipError_t ms_launch_softmax_apply(float* scores, int64_t row_stride, const ms::SeqSumArgs* a, int log_softmax,
                                    hipStream_t stream);
 hipError_t ms_launch_scorer_process(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,

@@ -18,50 +18,9 @@
 // costs a scan.
 #include "kernels.h"
 #include "block_seq.h"
+#include "seg_io.h"
 
 namespace ms {
-
-typedef float v4f __attribute__((ext_vector_type(4)));
-typedef uint32_t v4u __attribute__((ext_vector_type(4)));
-
-constexpr int kSegBlock = 256;
-constexpr int kSegPer = kSegElems / kSegBlock;  // 16 elements per thread
-
-// Loads the 16 elements of thread t in segment `seg`: for j, the VEC consecutive ids starting at
-// seg*kSegElems + (j*256 + t)*VEC (VEC = 4 for fp32, 8 for fp16).  Ids >= vocab yield `fill`.
-template <typename InT>
-__device__ __forceinline__ void seg_load(const InT* row, bool aligned, int vocab, int seg, float fill,
-                                         float (&v)[kSegPer]) {
-  constexpr int VEC = sizeof(InT) == 4 ? 4 : 8;
-  constexpr int NV = kSegPer / VEC;
-#pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    const int i0 = seg * kSegElems + (j * kSegBlock + static_cast<int>(threadIdx.x)) * VEC;
-    if (aligned && i0 + VEC <= vocab) {
-      if constexpr (VEC == 4) {
-        const v4f q = *reinterpret_cast<const v4f*>(row + i0);
-        v[j * 4] = q.x, v[j * 4 + 1] = q.y, v[j * 4 + 2] = q.z, v[j * 4 + 3] = q.w;
-      } else {
-        const v4u q = *reinterpret_cast<const v4u*>(row + i0);
-        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          v[j * 8 + 2 * c] = half_bits_to_float(w[c] & 0xffffu);
-          v[j * 8 + 2 * c + 1] = half_bits_to_float(w[c] >> 16);
-        }
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < VEC; ++c) v[j * VEC + c] = (i0 + c < vocab) ? load_one<InT>(row, i0 + c) : fill;
-    }
-  }
-}
-
-template <typename InT>
-__device__ __forceinline__ int seg_index(int seg, int e) {
-  constexpr int VEC = sizeof(InT) == 4 ? 4 : 8;
-  return seg * kSegElems + ((e / VEC) * kSegBlock + static_cast<int>(threadIdx.x)) * VEC + e % VEC;
-}
 
 template <typename InT>
 __global__ __launch_bounds__(kSegBlock) void seqsum_max_kernel(const SeqSumArgs a) {
@@ -226,13 +185,14 @@ __global__ __launch_bounds__(kSegBlock) void softmax_apply_kernel(float* scores,
 
 }  // namespace ms
 
-extern "C" hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, hipStream_t stream) {
+// have_seg_max != 0: the segment maxima in a->seg_max were already written by the caller's own kernel.
+extern "C" hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, int have_seg_max, hipStream_t stream) {
   const dim3 grid(a->segs, a->rows), block(ms::kSegBlock);
   if (dtype == MI355X_F16) {
-    hipLaunchKernelGGL(ms::seqsum_max_kernel<uint16_t>, grid, block, 0, stream, *a);
+    if (!have_seg_max) hipLaunchKernelGGL(ms::seqsum_max_kernel<uint16_t>, grid, block, 0, stream, *a);
     hipLaunchKernelGGL(ms::seqsum_exp_kernel<uint16_t>, grid, block, 0, stream, *a);
   } else {
-    hipLaunchKernelGGL(ms::seqsum_max_kernel<float>, grid, block, 0, stream, *a);
+    if (!have_seg_max) hipLaunchKernelGGL(ms::seqsum_max_kernel<float>, grid, block, 0, stream, *a);
     hipLaunchKernelGGL(ms::seqsum_exp_kernel<float>, grid, block, 0, stream, *a);
   }
   hipLaunchKernelGGL(ms::seqsum_step_kernel, grid, block, 0, stream, *a);

@@ -95,6 +95,79 @@ def test_beam_select_constant_rows(ctx, orc):
     assert np.array_equal(tok.cpu().numpy(), otok) and np.array_equal(idx.cpu().numpy(), oidx)
 
 
+def _check_beam_select(ctx, orc, x, batch, beams, bs):
+    dev_x = torch.from_numpy(x).cuda()
+    sc, tok, idx = ctx.beam_select(dev_x, batch, beams, torch.from_numpy(bs).cuda())
+    xf = orc.fp16_to_fp32(x) if x.dtype == np.float16 else x
+    osc, otok, oidx, _ = orc.beam_select_top(xf, batch, beams, bs)
+    assert np.array_equal(tok.cpu().numpy(), otok)
+    assert np.array_equal(idx.cpu().numpy(), oidx)
+    assert np.array_equal(bits(sc.cpu().numpy()), bits(osc))
+
+
+@pytest.mark.parametrize("case", ["random_fp32", "beams16", "constant", "one_segment", "equal_finals_spread",
+                                  "equal_finals_dense", "minus_inf", "ragged_fp16", "strided_fp32"])
+def test_beam_select_long_rows_through_segment_lists(ctx, orc, case):
+    """Rows of at least 16384 logits: every 4096-element segment lists its 2*beams largest logits and one
+    workgroup per batch entry scores them.  The cases force the lists' limits: all candidates of an entry inside
+    one segment, different logits that round to one final score (lowest flat index must win, with and without the
+    lists being full), constant rows (list overflow), -inf fill, rows that end inside a vector, strided rows."""
+    say("beam_select long rows", case)
+    rng = np.random.default_rng(len(case))
+    if case == "random_fp32":
+        batch, beams, vocab = 3, 4, 50001
+        x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float32)
+    elif case == "beams16":
+        batch, beams, vocab = 2, 16, 20000
+        x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float16)
+    elif case == "constant":
+        batch, beams, vocab = 2, 3, 20000
+        x = np.zeros((batch * beams, vocab), np.float16)
+        x[4] = 1.0
+    elif case == "one_segment":
+        batch, beams, vocab = 2, 4, 40000
+        x = rng.standard_normal((batch * beams, vocab)).astype(np.float32)
+        for r in range(batch * beams):
+            x[r, 3 * 4096 + rng.choice(4096, 12, replace=False)] += 10
+    elif case in ("equal_finals_spread", "equal_finals_dense"):
+        # logits within a few ulp of 1e-3 above a negative bulk: (x - max) - log(sum) rounds them all to one score
+        batch, beams, vocab = 2, 2, 30000
+        x = (-np.abs(rng.standard_normal((batch * beams, vocab))) - 1).astype(np.float32)
+        top = np.float32(1e-3)
+        ladder = [top]
+        for _ in range(5):
+            ladder.append(np.nextafter(ladder[-1], np.float32(1), dtype=np.float32))
+        for r in range(batch * beams):
+            if case == "equal_finals_spread":
+                pos = np.concatenate([s * 4096 + rng.choice(4096, 2, replace=False) for s in range(7)])
+            else:
+                pos = 2 * 4096 + rng.choice(4096, 40, replace=False)
+            x[r, pos] = rng.choice(ladder, pos.size)
+    elif case == "minus_inf":
+        batch, beams, vocab = 2, 2, 17000
+        x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float32)
+        x[:, rng.choice(vocab, 9000, replace=False)] = -np.inf
+        x[1, :] = -np.inf
+        x[1, 16999] = 0.5  # one number in the row
+    elif case == "ragged_fp16":
+        batch, beams, vocab = 2, 3, 16384 + 4099
+        x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float16)  # odd row length: unaligned rows
+    else:
+        batch, beams, vocab = 2, 2, 24001
+        full = (rng.standard_normal((batch * beams, vocab + 7)) * 2).astype(np.float32)
+        bs = (rng.standard_normal(batch * beams) * 3).astype(np.float32)
+        dev = torch.from_numpy(full).cuda()[:, :vocab]
+        sc, tok, idx = ctx.beam_select(dev, batch, beams, torch.from_numpy(bs).cuda())
+        osc, otok, oidx, _ = orc.beam_select_top(np.ascontiguousarray(full[:, :vocab]), batch, beams, bs)
+        assert np.array_equal(tok.cpu().numpy(), otok) and np.array_equal(idx.cpu().numpy(), oidx)
+        assert np.array_equal(bits(sc.cpu().numpy()), bits(osc))
+        return
+    bs = (rng.standard_normal(batch * beams) * 3).astype(np.float32)
+    if case in ("constant", "equal_finals_spread", "equal_finals_dense"):
+        bs[:] = 0.25  # equal running scores: ties run across the beams of an entry
+    _check_beam_select(ctx, orc, x, batch, beams, bs)
+
+
 def run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, length_penalty, early_stopping, seed,
                     dtype=np.float16, eos_boost=0.0):
     rng = np.random.default_rng(seed)
