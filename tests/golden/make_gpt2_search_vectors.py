@@ -13,9 +13,9 @@ vocabulary 1000).  The reference's C++ cannot run here (it needs ONNX Runtime), 
   * drives the oracle's search functions with those logits, and
   * REFUSES to write anything unless the resulting sequences equal the reference's expected outputs.
 What is stored: prompts, expected outputs, search options, and for every step along the golden trajectory the logits
-and (beam search) the token rows they were computed for -- inputs and expected outputs only.  tests/test_gpt2_golden.py replays them through the oracle (CPU) and through the
-HIP kernels (GPU); each replay also checks that the sequences it feeds back are the ones the logits were computed
-for.
+and (beam search) the token rows they were computed for -- inputs and expected outputs only.
+tests/test_gpt2_golden.py replays them through the oracle (CPU) and through the HIP kernels (GPU); each replay also
+checks that the sequences it feeds back are the ones the logits were computed for.
 
 Run where /root/reference exists:  python tests/golden/make_gpt2_search_vectors.py"""
 import os
@@ -30,7 +30,6 @@ import orc_lib  # noqa: E402
 
 MODEL = "/root/reference/test/models/hf-internal-testing/tiny-random-gpt2-fp32/past.onnx"
 PAD = EOS = 98  # genai_config.json beside the model
-VOCAB = 1000
 
 # test/model_tests.cpp:58-63
 GREEDY_PROMPT = np.array([[0, 0, 0, 52], [0, 0, 195, 731]], np.int32)
