@@ -64,6 +64,34 @@ def time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, t
     return overlapped_ms
 
 
+def step_latencies(torch, np, step, tokens, side, W, K):
+    """Distribution of the step latency, outside the timed region: every one of the K steps launched eagerly
+    between its own pair of HIP events on the launch stream (GPU time of one step), and the host-clock time
+    from the call of a single step to its token ids being on the host (launch + kernel + copy back)."""
+    n = min(K, 128)
+    with torch.cuda.stream(side):
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for j, (e0, e1) in enumerate(pairs):
+            e0.record(side)
+            step(W + j)
+            e1.record(side)
+        side.synchronize()
+        per_step = np.array([e0.elapsed_time(e1) for e0, e1 in pairs]) * 1e3
+        host = []
+        for j in range(min(n, 64)):
+            t0 = time.perf_counter()
+            step(W + j)
+            tokens[W + j].cpu()
+            host.append((time.perf_counter() - t0) * 1e6)
+    torch.cuda.synchronize()
+    return {"note": "informational: single eager launches, each between its own HIP events; host clock from the "
+                    "call to the token ids on the host",
+            "gpu_us_mean": float(per_step.mean()), "gpu_us_p50": float(np.percentile(per_step, 50)),
+            "gpu_us_p95": float(np.percentile(per_step, 95)),
+            "launch_to_result_us_p50": float(np.percentile(host, 50)),
+            "launch_to_result_us_p95": float(np.percentile(host, 95))}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -159,6 +187,7 @@ def main():
         bad = int((got != want).sum())
         sys.exit(f"PARITY FAILURE: {bad} of {got.size} sampled tokens differ from the CPU oracle")
     fallback = ctx.fallback_rows()
+    latency = step_latencies(torch, np, step, tokens, side, W, K)
     # ---- CPU baseline: the reference's own functions where they were built, else the oracle ---------
     baseline = {"value": ROWS * n_cpu / cpu_s, "unit": "tokens/s", "cores": 1, "kind": "port",
                 "sample": "%d of the %d timed steps (same logits and uniforms), oracle/search_oracle.cpp "
@@ -223,6 +252,7 @@ def main():
                    "rows": ROWS, "vocab": VOCAB, "top_k": TOP_K, "top_p": TOP_P, "temperature": TEMP,
                    "parity": parity,
                    "general_path_rows": fallback,
+                   "single_step_latency": latency,
                    "independent_batches_in_flight": None if overlapped_ms is None else {
                        "note": "informational, not `value`: the same steps issued round-robin on %d streams / "
                                "contexts in one HIP graph (tokens identical)" % n_streams,
