@@ -64,6 +64,23 @@ def time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, t
     return overlapped_ms
 
 
+def hbm_copy_probe(torch, dev):
+    """GB/s (read + write) of a plain device-to-device copy of 1 GiB, ten times between two events: what this
+    GPU's HBM sustains for the simplest streaming kernel, reported next to the nominal 8 TB/s."""
+    n = 1 << 28
+    src = torch.ones(n, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    return 2 * n * 4 * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+
 def step_latencies(torch, np, step, tokens, side, W, K):
     """Distribution of the step latency, outside the timed region: every one of the K steps launched eagerly
     between its own pair of HIP events on the launch stream (GPU time of one step), and the host-clock time
@@ -223,6 +240,7 @@ def main():
     if n_streams >= 2:
         overlapped_ms = time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, tokens, pool, W, K)
 
+    copy_gbps = hbm_copy_probe(torch, dev)
     ms_per_step = gpu_ms / K
     algo_bytes = ROWS * VOCAB * 4 + ROWS * 8 + ROWS * 4  # logits once + uniforms + tokens
     achieved = algo_bytes / (ms_per_step * 1e-3) / 1e9
@@ -261,7 +279,8 @@ def main():
                        "roofline_frac": algo_bytes / (overlapped_ms / K * 1e-3) / 1e9 / HBM_PEAK_GBS}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "sample_fused_kernel", "algorithmic_bytes_per_launch": algo_bytes},
+                     "kernel": "sample_fused_kernel", "algorithmic_bytes_per_launch": algo_bytes,
+                     "measured_copy_GBps": copy_gbps},
         "cpu_baseline": baseline,
     }
     print(json.dumps(out))
