@@ -134,7 +134,7 @@ def main():
     import __graft_entry__ as ge
     import orc_lib
 
-    pkg = ge.load_package()
+    pkg = ge.ensure_built()
     orc = orc_lib.Oracle()
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)

@@ -12,7 +12,7 @@ LOWEST = np.finfo(np.float32).min
 
 def pkg():
     import __graft_entry__ as ge
-    return ge.load_package()
+    return ge.ensure_built()
 
 
 def say(*a):

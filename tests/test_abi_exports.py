@@ -2,8 +2,18 @@
 import ctypes
 import os
 import re
+import sys
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+import pytest  # noqa: E402
+
+import __graft_entry__ as ge  # noqa: E402
+
+
+@pytest.fixture(scope="module", autouse=True)
+def built():
+    ge.ensure_built()  # compiles only where no library has been built yet
 
 
 def test_every_declared_symbol_is_exported():
