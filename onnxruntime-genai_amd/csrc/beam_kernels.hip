@@ -348,6 +348,12 @@ __global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a) {
   __shared__ float s_max[kBeamMaxCand / 2], s_lse[kBeamMaxCand / 2], s_bs[kBeamMaxCand / 2];
   const int b = blockIdx.x, tid = threadIdx.x;
   const int V = a.vocab, m = 2 * a.beams, per_row = a.segs * m, n = a.beams * per_row;
+  // the listed candidates are requested before anything waits (they do not depend on the rows' sums)
+  const u64* cand = a.seg_cand + static_cast<size_t>(b * a.beams) * per_row;
+  const int nr = (n + 255) >> 8;  // key slots per thread in use
+  u64 raw[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) raw[r] = (r < nr && tid + r * 256 < n) ? cand[tid + r * 256] : 0ull;
   bool odd = false;  // a row whose maximum is not a finite number: its scores need not follow the logit order
   if (tid < a.beams) {
     const int row = b * a.beams + tid;
@@ -363,12 +369,11 @@ __global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a) {
   int beam = tid / per_row, j = tid % m;
   int q = tid - beam * per_row;
   const int dj = 256 % m;
-  const u64* cand = a.seg_cand + static_cast<size_t>(b * a.beams) * per_row;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     key[r] = 0ull;
-    if (tid + r * 256 < n) {
-      const u64 c = cand[tid + r * 256];
+    if (r < nr && tid + r * 256 < n) {
+      const u64 c = raw[r];
       if (c == kSegOverflow) {
         full_reach = 0xffffffffu;
       } else if (c != 0ull) {
@@ -388,7 +393,7 @@ __global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a) {
     u64 best = 0ull;
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (key[r] < last && key[r] > best) best = key[r];
+      if (r < nr && key[r] < last && key[r] > best) best = key[r];
     best = block_max<u64>(best, red64);
     if (tid == 0) best_list[j] = best;
     last = best;  // 0 once nothing is left: later rounds find nothing either
