@@ -22,9 +22,11 @@
 //   GetBeamHypotheses and the beam sequence append: pinned by the reference's own golden generations
 //   (ModelTests.GreedySearchGptFp32 / BeamSearchGptFp32, test/model_tests.cpp:57-130), replayed from
 //   the logits of the tiny GPT-2 those tests load (tests/golden/gpt2_search_vectors.npz).
-//   BeamSearchScorer's EOS branch (BeamHypotheses::Add / CanImprove, done batches, padding): no EOS
-//   is produced in those golden runs; it is pinned only by hand-worked cases and invariants of the
-//   HuggingFace algorithm it follows, so the exact values of that branch are "parity unpinned".
+//   BeamSearchScorer's EOS branch (BeamHypotheses::Add / CanImprove, done batches, padding, the
+//   done window's offset): no EOS is produced in those golden runs; pinned by hand-worked cases
+//   with literal expected values derived from the reference source (tests/beam_scorer_cases.py,
+//   tests/test_beam_scorer_handworked.py), each of sixteen one-line mistakes patched into this file
+//   failing at least one of them.
 //   KV gather: pinned by numpy.take.
 //   Cast conversions (fp16/bf16 <-> fp32, int32 -> int64): pinned by known answers and, for
 //   fp32 -> fp16, by agreement with IEEE round-to-nearest on every value that is not an exact tie

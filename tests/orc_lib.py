@@ -42,8 +42,9 @@ def _f32(a):
 
 
 class Oracle:
-    def __init__(self):
-        L = self.lib = C.CDLL(_ensure_built())
+    def __init__(self, path=None):
+        """`path`: a differently built copy of the oracle library (the mutation tests load patched ones)."""
+        L = self.lib = C.CDLL(path or _ensure_built())
         L.orc_argmax.restype = C.c_int32
         L.orc_argmax.argtypes = [f32p, C.c_int]
         L.orc_apply_min_length.argtypes = [f32p, C.c_int, C.c_int, C.c_int, i32p, C.c_int]

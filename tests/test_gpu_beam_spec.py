@@ -225,6 +225,45 @@ def test_beam_search_with_eos_hypotheses(ctx, orc, early, lp):
     run_beam_search(ctx, orc, 3, 3, 50, 14, [7, 9], 20, lp, early, 11 + int(early), dtype=np.float32, eos_boost=2.5)
 
 
+@pytest.mark.parametrize("name", sorted(__import__("beam_scorer_cases").CASES))
+def test_device_scorer_matches_handworked_case(ctx, name):
+    """mi355x_beam_scorer_* against literal expectations worked out by hand from the reference source
+    (tests/beam_scorer_cases.py): EOS hypotheses, eviction, ties, CanImprove with its window offset, early
+    stopping, padding of done entries, Finalize.  No oracle involved."""
+    from beam_scorer_cases import CASES
+    from test_beam_scorer_handworked import check_hyps
+    case = CASES[name]
+    say("hand-worked scorer case", name)
+    batch, beams, ml = case["batch"], case["beams"], case["max_length"]
+    dev = pkg().BeamScorer(ctx, batch, beams, ml, case["pad"], case["eos"], case["length_penalty"],
+                           case["early_stopping"])
+    dev.set_prompt(np.asarray(case["prompt"], np.int32))
+    init = np.tile(np.array([0.0] + [-1e9] * (beams - 1), np.float32), batch)
+    assert np.array_equal(dev.next_scores.cpu().numpy(), init)
+    length = len(case["prompt"][0])
+    for si, step in enumerate(case["steps"]):
+        cs = torch.tensor([[c[0] for c in row] for row in step["cands"]], dtype=torch.float32).cuda()
+        ct = torch.tensor([[c[1] for c in row] for row in step["cands"]], dtype=torch.int32).cuda()
+        ci = torch.tensor([[c[2] for c in row] for row in step["cands"]], dtype=torch.int32).cuda()
+        dev.step(cs, ct, ci)
+        length += 1
+        got_s, got_t, got_i = (dev.next_scores.cpu().numpy(), dev.next_tokens.cpu().numpy(),
+                               dev.next_indices.cpu().numpy())
+        for r, (ws, wt, wi) in enumerate(step["next"]):
+            assert got_s[r] == np.float32(ws) and got_t[r] == wt and got_i[r] == wi, (si, r, got_s, got_t, got_i)
+        dseq, dlen = dev.sequences()
+        assert dlen == length and dseq.cpu().numpy().tolist() == step["sequences"], si
+        assert dev.is_done() == (step["all_done"] or length == ml), si
+    for b in range(batch):
+        got = []
+        for i in range(len(case["final"][b])):
+            got.append(dev.hypothesis(b, i))
+        check_hyps(("final", b), got, case["final"][b])
+        with pytest.raises(RuntimeError, match="out of bounds"):
+            dev.hypothesis(b, len(case["final"][b]))
+    dev.close()
+
+
 def test_kv_gather_bit_exact(ctx, orc):
     say("kv_gather")
     rng = np.random.default_rng(5)
