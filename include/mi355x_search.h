@@ -109,6 +109,23 @@ int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int 
                   int64_t row_stride, int rows, int vocab, const mi355x_logits_xform* xf,
                   int32_t* out_tokens);
 
+/* mi355x_argmax without a context and without any allocation.  It has no counterpart in the
+ * reference: it exists for callers that cannot allocate device memory where they call (code under
+ * HIP graph capture, serving loops and harnesses that forbid hipMalloc).  Same arguments, same results
+ * and same errors as mi355x_argmax, except:
+ *   - the device is the calling thread's current HIP device, which `stream` must belong to;
+ *   - the kernels' per-row partial results live in a static device array of
+ *     MI355X_ARGMAX_STATIC_MAX_ROWS rows (48 KiB, held by every GPU the library is loaded on until
+ *     the process ends); more rows fail with MI355X_E_CAPACITY;
+ *   - xf->no_repeat_ngram_size > 0 fails with MI355X_E_UNSUPPORTED (its bitmaps need a context).
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream, or otherwise ordered, are safe.  The call itself clears the slots
+ * it is about to use (with a kernel, no memset node) and calls neither hipMalloc nor hipFree.
+ * The array's address is looked up once per device, by mi355x_search_create or by the first call. */
+#define MI355X_ARGMAX_STATIC_MAX_ROWS 4096
+int mi355x_argmax_static(void* stream, const void* logits, int dtype, int64_t row_stride, int rows,
+                         int vocab, const mi355x_logits_xform* xf, int32_t* out_tokens);
+
 /* Per-row k best (token id, raw fp32 score), best first: DeviceInterface::TopKScores
  * (src/smartptrs.h:254).  out_tokens/out_scores: device [rows, k].  1 <= k <= 64. */
 int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype,

@@ -48,6 +48,7 @@ def load_library():
     L.mi355x_search_workspace_bytes.restype = C.c_size_t
     L.mi355x_process_logits.argtypes = [vp, vp, vp, i64, i32, i32, C.POINTER(LogitsXformC)]
     L.mi355x_argmax.argtypes = [vp, vp, vp, i32, i64, i32, i32, C.POINTER(LogitsXformC), vp]
+    L.mi355x_argmax_static.argtypes = [vp, vp, i32, i64, i32, i32, C.POINTER(LogitsXformC), vp]
     L.mi355x_sample.argtypes = [vp, vp, vp, i64, i32, i32, C.POINTER(LogitsXformC), SampleParams,
                                 C.POINTER(SampleParams), vp, vp, vp, vp, vp, i32]
     L.mi355x_search_fallback_rows.argtypes = [vp, vp, C.POINTER(C.c_uint)]
@@ -118,6 +119,20 @@ class LogitsXform:
 
 def _stream():
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def argmax_static(logits, out, xf=None):
+    """mi355x_argmax_static: argmax of every row into the caller's `out` ([rows] int32 on the same device), on the
+    current stream of the current device; needs no context and allocates nothing."""
+    L = load_library()
+    assert logits.is_cuda and logits.dim() == 2 and logits.stride(1) == 1
+    assert out.is_cuda and out.dtype == torch.int32 and out.numel() >= logits.shape[0] and out.is_contiguous()
+    dtype = {torch.float32: MI355X_F32, torch.float16: MI355X_F16}[logits.dtype]
+    rc = L.mi355x_argmax_static(_stream(), logits.data_ptr(), dtype, logits.stride(0), logits.shape[0], logits.shape[1],
+                                C.byref(xf.c) if xf else None, out.data_ptr())
+    if rc != 0:
+        raise RuntimeError(f"mi355x_search error {rc}: {L.mi355x_search_last_error().decode()}")
+    return out
 
 
 class SearchContext:

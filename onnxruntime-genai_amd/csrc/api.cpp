@@ -10,20 +10,28 @@
 #include <new>
 #include <string>
 #include <vector>
-#include "kernels.h"
-#include "mi355x_search.h"
+#include "api_internal.h"
 
 namespace {
 
 thread_local std::string g_error;
 
-int Fail(int code, const char* fmt, ...) {
+}  // namespace
+
+int ms_vfail(int code, const char* fmt, va_list ap) {
   char buf[512];
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  g_error = buf;
+  return code;
+}
+
+namespace {
+
+int Fail(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
-  vsnprintf(buf, sizeof(buf), fmt, ap);
+  ms_vfail(code, fmt, ap);
   va_end(ap);
-  g_error = buf;
   return code;
 }
 
@@ -106,6 +114,15 @@ int CheckRows(const mi355x_search_ctx* ctx, int rows, int vocab) {
 // the context's workspace.
 int MakeXform(mi355x_search_ctx* ctx, const mi355x_logits_xform* in, int rows, int vocab, hipStream_t stream,
               ms::Xform* out) {
+  return ms_make_xform(ctx, in, rows, vocab, stream, out);
+}
+
+}  // namespace
+
+// `ctx` may be null (an entry point without a context): the n-gram rule, whose bitmaps live in a
+// context's workspace, is then refused.
+int ms_make_xform(mi355x_search_ctx* ctx, const mi355x_logits_xform* in, int rows, int vocab, hipStream_t stream,
+                  ms::Xform* out) {
   std::memset(out, 0, sizeof(*out));
   out->penalty = 1.0f;
   if (!in) return MI355X_OK;
@@ -128,6 +145,7 @@ int MakeXform(mi355x_search_ctx* ctx, const mi355x_logits_xform* in, int rows, i
   }
   if (in->no_repeat_ngram_size > 0) {
     if (!in->history) return Fail(MI355X_E_INVALID, "no_repeat_ngram_size needs a history");
+    if (!ctx) return Fail(MI355X_E_UNSUPPORTED, "no_repeat_ngram_size needs a context (its bitmaps live in the workspace)");
     if (out->history_lens || out->history_len >= in->no_repeat_ngram_size) {
       HIP_TRY(ms_launch_ngram_ban(out, rows, vocab, in->no_repeat_ngram_size, ctx->ban, stream));
       out->ban = ctx->ban;
@@ -135,8 +153,6 @@ int MakeXform(mi355x_search_ctx* ctx, const mi355x_logits_xform* in, int rows, i
   }
   return MI355X_OK;
 }
-
-}  // namespace
 
 extern "C" {
 
@@ -192,6 +208,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   c->ptr_table_cap = 4096;
   ok(c->Alloc(&c->ptr_table, c->ptr_table_cap, false));
   if (e == hipSuccess) e = ms_sample_init();
+  if (e == hipSuccess) e = ms_static_scratch_setup();  // set-up of mi355x_argmax_static on this device
   if (e != hipSuccess) {
     mi355x_search_destroy(c);
     return Fail(MI355X_E_HIP, "workspace allocation failed: %s", hipGetErrorString(e));
