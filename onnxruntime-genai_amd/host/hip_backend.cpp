@@ -68,11 +68,13 @@ struct HipMemory final : DeviceBuffer {
   bool owned_;
 };
 
+}  // namespace
+
 // Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3"): counter-based, so a
 // request's stream depends only on (seed, draws so far), never on its position in a batch.
-double PhiloxUniform(uint64_t seed, uint64_t counter) {
-  uint32_t c[4] = {static_cast<uint32_t>(counter), static_cast<uint32_t>(counter >> 32), 0u, 0u};
-  uint32_t k[2] = {static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)};
+void Philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]) {
+  uint32_t c[4] = {counter[0], counter[1], counter[2], counter[3]};
+  uint32_t k[2] = {key[0], key[1]};
   for (int r = 0; r < 10; ++r) {
     const uint64_t p0 = 0xD2511F53ull * c[0], p1 = 0xCD9E8D57ull * c[2];
     const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c[1] ^ k[0];
@@ -83,9 +85,21 @@ double PhiloxUniform(uint64_t seed, uint64_t counter) {
     k[0] += 0x9E3779B9u;
     k[1] += 0xBB67AE85u;
   }
-  const uint64_t bits53 = ((static_cast<uint64_t>(c[0]) << 32) | c[1]) >> 11;
+  for (int i = 0; i < 4; ++i) out[i] = c[i];
+}
+
+// Draw number `counter` of the stream `seed`: counter words (lo, hi, 0, 0), key words (lo, hi) of the seed;
+// the first two output words give the 53 bits of a double in [0, 1).
+double PhiloxUniform(uint64_t seed, uint64_t counter) {
+  const uint32_t c[4] = {static_cast<uint32_t>(counter), static_cast<uint32_t>(counter >> 32), 0u, 0u};
+  const uint32_t k[2] = {static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32)};
+  uint32_t o[4];
+  Philox4x32_10(c, k, o);
+  const uint64_t bits53 = ((static_cast<uint64_t>(o[0]) << 32) | o[1]) >> 11;
   return static_cast<double>(bits53) * 0x1.0p-53;
 }
+
+namespace {
 
 struct HipBatchedSampler;
 struct HipSamplerState final : BatchedSamplerState {

@@ -15,6 +15,11 @@ namespace Generators {
 
 DeviceInterface* GetHipInterface();  // process-wide instance (device 0)
 
+// The random stream of a HipBatchedSampler request: Philox4x32 with 10 rounds, and the double in [0, 1) that
+// draw number `counter` of the stream with seed `seed` feeds to the sampling kernel.
+void Philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+double PhiloxUniform(uint64_t seed, uint64_t counter);
+
 // GreedySearch_Cpu's device counterpart (src/search.h:202-240, src/search.cpp:178-324).
 // Token selection runs on the GPU; EOS / padding / done bookkeeping is host state, as in the CPU
 // class.  Sampling matches the CPU class draw for draw: the kernels return each row's kept

@@ -15,6 +15,7 @@
 #include <functional>
 #include <limits>
 #include <numeric>
+#include <random>
 
 using namespace Generators;
 
@@ -534,6 +535,117 @@ void BatchedSamplerLargeVocabulary() {
   EXPECT_EQ(ToHost(sampler->Sample(rows, params, states, vocab_size)), (std::vector<int32_t>{1, 2, 3}));
 }
 
+// Known-answer vectors of Philox4x32-10 from Random123's kat_vectors (counter words, key words -> output
+// words): all zero, all ones, and the digits of pi.  PhiloxUniform must be the first two output words of
+// counter (draw, 0, 0, 0) under key (seed lo, seed hi), top 53 bits, scaled to [0, 1).
+void PhiloxKnownAnswers() {
+  struct Kat {
+    uint32_t c[4], k[2], want[4];
+  };
+  const Kat kats[] = {
+      {{0u, 0u, 0u, 0u}, {0u, 0u}, {0x6627e8d5u, 0xe169c58du, 0xbc57ac4cu, 0x9b00dbd8u}},
+      {{0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu}, {0xffffffffu, 0xffffffffu},
+       {0x408f276du, 0x41c83b0eu, 0xa20bc7c6u, 0x6d5451fdu}},
+      {{0x243f6a88u, 0x85a308d3u, 0x13198a2eu, 0x03707344u}, {0xa4093822u, 0x299f31d0u},
+       {0xd16cfe09u, 0x94fdccebu, 0x5001e420u, 0x24126ea1u}},
+  };
+  for (const Kat& t : kats) {
+    uint32_t out[4];
+    Philox4x32_10(t.c, t.k, out);
+    for (int i = 0; i < 4; ++i) EXPECT_EQ(out[i], t.want[i]);
+  }
+  // seed 0, draw 0 is the all-zero vector: 0x6627e8d5e169c58d >> 11 = 0xCC4FD1ABC2D38, times 2^-53
+  EXPECT_EQ(PhiloxUniform(0, 0), static_cast<double>(0x6627e8d5e169c58dull >> 11) * 0x1.0p-53);
+  EXPECT(PhiloxUniform(0, 0) > 0.399 && PhiloxUniform(0, 0) < 0.4);  // 0x6627... / 2^64 = 0.39904...
+  // the seed is the key, the draw number the counter: neither aliases the other
+  EXPECT(PhiloxUniform(1, 0) != PhiloxUniform(0, 1));
+  uint32_t out[4];
+  const uint32_t c1[4] = {7u, 1u, 0u, 0u}, k1[2] = {5u, 9u};
+  Philox4x32_10(c1, k1, out);
+  EXPECT_EQ(PhiloxUniform((9ull << 32) | 5u, (1ull << 32) | 7u),
+            static_cast<double>(((static_cast<uint64_t>(out[0]) << 32) | out[1]) >> 11) * 0x1.0p-53);
+}
+
+// The distribution of the batched sampler's own draws, after RunSamplingTest (test/sampling_tests.cpp:262-365):
+// identical logits in every row with the scores num_top .. 1 on shuffled token ids, a fresh seeded state per
+// row and iteration, 5 rows x 1000 iterations; every token's frequency within 0.015 of its probability and
+// tokens outside the kept set never drawn.
+void BatchedSamplerDistribution(int k, float p, int vocab_size, float temperature) {
+  constexpr int batch_size = 5, num_iter = 1000;
+  const int num_top = k > 0 ? k : vocab_size;
+  std::vector<float> single(vocab_size, 0.0f);
+  std::vector<int32_t> top_indices(vocab_size);
+  std::iota(top_indices.begin(), top_indices.end(), 0);
+  std::mt19937 shuffle_engine(12345);
+  std::shuffle(top_indices.begin(), top_indices.end(), shuffle_engine);
+  for (int j = 0; j < num_top; ++j) single[top_indices[j]] = static_cast<float>(num_top - j);
+  // expected: softmax(score / T) over the kept prefix (the top-p cut keeps the first j with cumulative >= p)
+  std::vector<double> expected(num_top);
+  double z = 0.0;
+  for (int j = 0; j < num_top; ++j) z += (expected[j] = std::exp((num_top - j) / static_cast<double>(temperature)));
+  for (double& e : expected) e /= z;
+  if (p < 1.0f) {
+    double cum = 0.0, kept = 0.0;
+    int keep = num_top;
+    for (int j = 0; j < num_top; ++j)
+      if ((cum += expected[j]) >= p) {
+        keep = j + 1;
+        break;
+      }
+    for (int j = 0; j < num_top; ++j) kept += j < keep ? expected[j] : 0.0;
+    for (int j = 0; j < num_top; ++j) expected[j] = j < keep ? expected[j] / kept : 0.0;
+  }
+  auto sampler = Device()->CreateBatchedSampler(batch_size, vocab_size);
+  std::vector<float> all;
+  for (int b = 0; b < batch_size; ++b) all.insert(all.end(), single.begin(), single.end());
+  auto scores = ToDevice(all);
+  std::vector<DeviceSpan<float>> rows;
+  for (int b = 0; b < batch_size; ++b) rows.push_back(scores.subspan(static_cast<size_t>(b) * vocab_size, vocab_size));
+  const std::vector<BatchedSamplingParams> params(batch_size, BatchedSamplingParams{k, p, temperature});
+  std::vector<int> counts(vocab_size, 0);
+  std::mt19937 engine(12345);
+  std::uniform_int_distribution<int> dist;
+  for (int i = 0; i < num_iter; ++i) {
+    std::vector<std::unique_ptr<BatchedSamplerState>> owned;
+    std::vector<BatchedSamplerState*> states;
+    for (int b = 0; b < batch_size; ++b) {
+      owned.push_back(sampler->CreateState(dist(engine)));
+      states.push_back(owned.back().get());
+    }
+    for (int32_t t : ToHost(sampler->Sample(rows, params, states, vocab_size))) {
+      EXPECT(t >= 0 && t < vocab_size);
+      if (t >= 0 && t < vocab_size) counts[t]++;
+    }
+  }
+  const double total = batch_size * num_iter;
+  int in_top = 0;
+  for (int j = 0; j < num_top; ++j) {
+    const double actual = counts[top_indices[j]] / total;
+    in_top += counts[top_indices[j]];
+    if (expected[j] > 0) EXPECT(std::fabs(actual - expected[j]) < 0.015);
+    else EXPECT_EQ(counts[top_indices[j]], 0);
+  }
+  EXPECT_EQ(in_top, batch_size * num_iter);
+}
+void BatchedSamplerDistributionTopK() { BatchedSamplerDistribution(5, 1.0f, 13, 0.8f); }         // RandomizedSamplingTopK
+void BatchedSamplerDistributionTopPAndK() { BatchedSamplerDistribution(7, 0.75f, 21, 1.0f); }    // RandomizedSamplingTopPAndK
+void BatchedSamplerDistributionTopPOnly() { BatchedSamplerDistribution(0, 0.95f, 21, 1.0f); }    // RandomizedSamplingTopPOnly
+// one stream, consecutive draws (the counter path): 5000 draws of one request at a 100-id vocabulary
+void BatchedSamplerStreamIsUniform() {
+  constexpr int vocab_size = 100, draws = 5000;
+  auto sampler = Device()->CreateBatchedSampler(1, vocab_size);
+  auto state = sampler->CreateState(2024);
+  std::array<BatchedSamplerState*, 1> states{state.get()};
+  std::array<DeviceSpan<float>, 1> rows{ToDevice(std::vector<float>(vocab_size, 0.5f))};
+  const std::array<BatchedSamplingParams, 1> params{BatchedSamplingParams{-1, 1.0f, 1.0f}};  // whole vocabulary, flat
+  std::vector<int> counts(vocab_size, 0);
+  for (int i = 0; i < draws; ++i) counts[ToHost(sampler->Sample(rows, params, states, vocab_size))[0]]++;
+  // chi-square over 100 equally likely ids: 99 degrees of freedom, mean 99, sd 14.1; 170 is five sd away
+  double chi2 = 0.0;
+  for (int c : counts) chi2 += (c - 50.0) * (c - 50.0) / 50.0;
+  EXPECT(chi2 < 170.0 && chi2 > 40.0);
+}
+
 // A whole generation against the host model of GreedySearch_Cpu: prompt, min-length, repetition
 // penalty, no-repeat n-grams, the four selection methods in rotation, EOS padding, rewind, max_length.  Tokens, done
 // flag, sequences and the std::mt19937 state must agree after every step.
@@ -695,6 +807,11 @@ int main(int argc, char** argv) {
       {"BatchedSamplerPreservesRngAcrossBatchReorder", BatchedSamplerPreservesRngAcrossBatchReorder},
       {"BatchedSamplerKeepsRngRowsAlignedForContiguousBatch", BatchedSamplerKeepsRngRowsAlignedForContiguousBatch},
       {"BatchedSamplerLargeVocabulary", BatchedSamplerLargeVocabulary},
+      {"PhiloxKnownAnswers", PhiloxKnownAnswers},
+      {"BatchedSamplerDistributionTopK", BatchedSamplerDistributionTopK},
+      {"BatchedSamplerDistributionTopPAndK", BatchedSamplerDistributionTopPAndK},
+      {"BatchedSamplerDistributionTopPOnly", BatchedSamplerDistributionTopPOnly},
+      {"BatchedSamplerStreamIsUniform", BatchedSamplerStreamIsUniform},
       {"GreedyGenerationMatchesCpuSearch", GreedyGenerationMatchesCpuSearch},
       {"BeamSearchMatchesCpuSearch", BeamSearchMatchesCpuSearch},
   };
