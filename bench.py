@@ -19,11 +19,48 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
-sys.path.insert(0, os.path.join(ROOT, "onnxruntime-genai_amd"))
 
 ROWS, VOCAB, TOP_K, TOP_P, TEMP = 64, 128256, 50, 0.9, 0.7
 HBM_PEAK_GBS = 8000.0
-MEASURED_TRAFFIC_BYTES = 33_460_000  # fetch 33.26 MB + write 0.20 MB per launch
+# HBM bytes per launch of the dominant kernel (fetch 33.26 MB + write 0.20 MB), a constant taken from the
+# rocprofv3 --pmc summary named below: counters cannot be read from inside this process.
+MEASURED_TRAFFIC_BYTES = 33_460_000
+TRAFFIC_SOURCE = "offline profile constant: profiles/sample_fused_kernel_config2_pmc.md"
+
+
+def time_fp16_steps(torch, np, orc, ctx, side, logits, uniforms, u_host, W, K, pool, n_cpu):
+    """The same K steps on fp16 copies of the logits, read directly by the sampling kernel (no widening pass):
+    graph replay between two events as for the fp32 run; the tokens of the first n_cpu steps must equal the CPU
+    oracle's on the rows widened as the reference's CPU path widens them.  Returns milliseconds for the K steps."""
+    half = [x.half() for x in logits]
+    tok16 = torch.empty((K + W, ROWS), dtype=torch.int32, device=uniforms.device)
+
+    def step16(i):
+        ctx.sample(half[i % pool], uniforms[i], k=TOP_K, p=TOP_P, temperature=TEMP, out=tok16[i])
+
+    with torch.cuda.stream(side):
+        for i in range(W):
+            step16(i)
+        side.synchronize()
+        g16 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g16, stream=side):
+            for i in range(W, W + K):
+                step16(i)
+        g16.replay()
+        side.synchronize()
+        s16, e16 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s16.record(side)
+        g16.replay()
+        e16.record(side)
+        side.synchronize()
+    torch.cuda.synchronize()
+    n = min(n_cpu, 4)
+    for i in range(n):
+        wide = orc.fp16_to_fp32(half[(W + i) % pool].cpu().numpy())
+        want = orc.sample_batch(wide, TOP_K, TOP_P, TEMP, u_host[W + i])
+        if not np.array_equal(tok16[W + i].cpu().numpy(), want):
+            sys.exit("PARITY FAILURE: tokens sampled from fp16 logits differ from the CPU oracle on the widened rows")
+    return s16.elapsed_time(e16), n
 
 
 def time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, tokens, pool, W, K):
@@ -139,8 +176,8 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     if args.workload != "c2":
-        import other_workloads
-        print(json.dumps(other_workloads.run(args, pkg, orc, orc_lib, dev)))
+        import bench_workloads
+        print(json.dumps(bench_workloads.run(args, pkg, orc, orc_lib, dev)))
         return
     K, W = args.steps, args.warmup
     pool = max(2, min(args.pool, K + W))
@@ -240,6 +277,7 @@ def main():
     if n_streams >= 2:
         overlapped_ms = time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, tokens, pool, W, K)
 
+    fp16_ms, fp16_checked = time_fp16_steps(torch, np, orc, ctx, side, logits, uniforms, u_host, W, K, pool, n_cpu)
     copy_gbps = hbm_copy_probe(torch, dev)
     ms_per_step = gpu_ms / K
     algo_bytes = ROWS * VOCAB * 4 + ROWS * 8 + ROWS * 4  # logits once + uniforms + tokens
@@ -271,6 +309,11 @@ def main():
                    "parity": parity,
                    "general_path_rows": fallback,
                    "single_step_latency": latency,
+                   "fp16_logits": {
+                       "note": "informational, not `value`: the same steps with fp16 logits read directly by the "
+                               "kernel (tokens of %d steps identical to the CPU oracle on the widened rows)" % fp16_checked,
+                       "us_per_step": fp16_ms / K * 1e3, "tokens_per_s": ROWS * K / (fp16_ms * 1e-3),
+                       "roofline_frac": (ROWS * VOCAB * 2) / (fp16_ms / K * 1e-3) / 1e9 / HBM_PEAK_GBS},
                    "independent_batches_in_flight": None if overlapped_ms is None else {
                        "note": "informational, not `value`: the same steps issued round-robin on %d streams / "
                                "contexts in one HIP graph (tokens identical)" % n_streams,
@@ -279,6 +322,7 @@ def main():
                        "roofline_frac": algo_bytes / (overlapped_ms / K * 1e-3) / 1e9 / HBM_PEAK_GBS}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_source": "rocprofv3 --pmc passed with --traffic" if args.traffic else TRAFFIC_SOURCE,
                      "kernel": "sample_fused_kernel", "algorithmic_bytes_per_launch": algo_bytes,
                      "measured_copy_GBps": copy_gbps},
         "cpu_baseline": baseline,

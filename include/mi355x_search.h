@@ -102,8 +102,9 @@ int mi355x_process_logits(mi355x_search_ctx* ctx, void* stream, float* logits, i
                           int rows, int vocab, const mi355x_logits_xform* xf);
 
 /* Greedy argmax per row: GreedySearch_Cpu::SelectTop / ArgMax (src/search.cpp:178-192,
- * src/search.h:9-29) and DeviceInterface::ArgMaxDevice (src/smartptrs.h:258).  dtype MI355X_F32 or
- * MI355X_F16 (fp16 is widened exactly like FastFloat16ToFloat32, src/models/utils.cpp:103-109).
+ * src/search.h:9-29) and DeviceInterface::ArgMaxDevice (src/smartptrs.h:258).  dtype MI355X_F32,
+ * MI355X_F16 (widened exactly like FastFloat16ToFloat32, src/models/utils.cpp:103-109) or MI355X_BF16
+ * (BFloat16ToFloat32, :84-86; rows of 65 to 524288 logits only).
  * xf may be NULL.  out_tokens: device [rows] int32. */
 int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype,
                   int64_t row_stride, int rows, int vocab, const mi355x_logits_xform* xf,
@@ -127,7 +128,8 @@ int mi355x_argmax_static(void* stream, const void* logits, int dtype, int64_t ro
                          int vocab, const mi355x_logits_xform* xf, int32_t* out_tokens);
 
 /* Per-row k best (token id, raw fp32 score), best first: DeviceInterface::TopKScores
- * (src/smartptrs.h:254).  out_tokens/out_scores: device [rows, k].  1 <= k <= 64. */
+ * (src/smartptrs.h:254).  dtype MI355X_F32, MI355X_F16 or MI355X_BF16 (the scores of sixteen-bit rows are
+ * the widened values).  out_tokens/out_scores: device [rows, k].  1 <= k <= 64. */
 int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype,
                        int64_t row_stride, int rows, int vocab, int k, int32_t* out_tokens,
                        float* out_scores);
@@ -153,6 +155,17 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
                   const mi355x_sample_params* per_row_params, const double* uniforms,
                   int32_t* out_tokens, int32_t* kept_count, int32_t* kept_ids, float* kept_probs,
                   int kept_capacity);
+
+/* mi355x_sample on rows of any supported element type: dtype MI355X_F32, MI355X_F16 or MI355X_BF16, row_stride
+ * in elements.  Sixteen-bit logits are read as they are and widened in registers exactly as the reference
+ * widens them before the search sees them (Logits::Get casts the model's fp16/bf16 output to fp32,
+ * src/models/logits.cpp:72-76, with FastFloat16ToFloat32 / BFloat16ToFloat32, src/models/utils.cpp:84-109):
+ * the results equal mi355x_sample on the widened copy, without the pass that writes and re-reads it. */
+int mi355x_sample_typed(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype,
+                        int64_t row_stride, int rows, int vocab, const mi355x_logits_xform* xf,
+                        mi355x_sample_params params, const mi355x_sample_params* per_row_params,
+                        const double* uniforms, int32_t* out_tokens, int32_t* kept_count,
+                        int32_t* kept_ids, float* kept_probs, int kept_capacity);
 
 /* Softmax / log-softmax with temperature, in place, one row per `vocab` floats:
  * Softmax and LogSoftMax (src/softmax.h:26-47).  Sums are accumulated in index order in fp32 exactly

@@ -51,6 +51,8 @@ def load_library():
     L.mi355x_argmax_static.argtypes = [vp, vp, i32, i64, i32, i32, C.POINTER(LogitsXformC), vp]
     L.mi355x_sample.argtypes = [vp, vp, vp, i64, i32, i32, C.POINTER(LogitsXformC), SampleParams,
                                 C.POINTER(SampleParams), vp, vp, vp, vp, vp, i32]
+    L.mi355x_sample_typed.argtypes = [vp, vp, vp, i32, i64, i32, i32, C.POINTER(LogitsXformC), SampleParams,
+                                      C.POINTER(SampleParams), vp, vp, vp, vp, vp, i32]
     L.mi355x_search_fallback_rows.argtypes = [vp, vp, C.POINTER(C.c_uint)]
     L.mi355x_search_wait_gave_up.argtypes = [vp, vp, C.POINTER(C.c_int)]
     L.mi355x_search_set_poll_limit.argtypes = [vp, C.c_int]
@@ -115,6 +117,9 @@ class LogitsXform:
         c.n_eos = len(eos_ids)
         for i, e in enumerate(eos_ids):
             c.eos_ids[i] = e
+
+
+_DTYPE_CODES = {torch.float32: 1, torch.int32: 6, torch.int64: 7, torch.float16: 10, torch.bfloat16: 16}
 
 
 def _stream():
@@ -187,7 +192,7 @@ class SearchContext:
 
     def argmax(self, logits, xf=None, out=None):
         rows, vocab, stride = self._rows(logits)
-        dtype = {torch.float32: MI355X_F32, torch.float16: MI355X_F16}[logits.dtype]
+        dtype = _DTYPE_CODES[logits.dtype]
         if out is None:
             out = torch.empty(rows, dtype=torch.int32, device=logits.device)
         self._check(self.L.mi355x_argmax(self.h, _stream(), logits.data_ptr(), dtype, stride, rows, vocab,
@@ -197,7 +202,7 @@ class SearchContext:
     def sample(self, logits, uniforms, k=0, p=0.0, temperature=1.0, per_row=None, xf=None, out=None,
                kept_capacity=0):
         rows, vocab, stride = self._rows(logits)
-        assert logits.dtype == torch.float32 and uniforms.dtype == torch.float64 and uniforms.numel() >= rows
+        assert uniforms.dtype == torch.float64 and uniforms.numel() >= rows
         if out is None:
             out = torch.empty(rows, dtype=torch.int32, device=logits.device)
         pr = None
@@ -208,12 +213,13 @@ class SearchContext:
             kc = torch.empty(rows, dtype=torch.int32, device=logits.device)
             ki = torch.full((rows, kept_capacity), -1, dtype=torch.int32, device=logits.device)
             kp = torch.zeros((rows, kept_capacity), dtype=torch.float32, device=logits.device)
-        self._check(self.L.mi355x_sample(self.h, _stream(), logits.data_ptr(), stride, rows, vocab,
-                                         C.byref(xf.c) if xf else None, SampleParams(int(k), float(p), float(temperature)),
-                                         pr, uniforms.data_ptr(), out.data_ptr(),
-                                         kc.data_ptr() if kept_capacity else None,
-                                         ki.data_ptr() if kept_capacity else None,
-                                         kp.data_ptr() if kept_capacity else None, kept_capacity))
+        args = (stride, rows, vocab, C.byref(xf.c) if xf else None, SampleParams(int(k), float(p), float(temperature)),
+                pr, uniforms.data_ptr(), out.data_ptr(), kc.data_ptr() if kept_capacity else None,
+                ki.data_ptr() if kept_capacity else None, kp.data_ptr() if kept_capacity else None, kept_capacity)
+        if logits.dtype == torch.float32:
+            self._check(self.L.mi355x_sample(self.h, _stream(), logits.data_ptr(), *args))
+        else:  # fp16 / bf16 rows are read as they are
+            self._check(self.L.mi355x_sample_typed(self.h, _stream(), logits.data_ptr(), _DTYPE_CODES[logits.dtype], *args))
         if kept_capacity:
             return out, kc, ki, kp
         return out
@@ -235,7 +241,7 @@ def _hip():
 
 
 def _dtype_code(t):
-    return {torch.float32: MI355X_F32, torch.float16: MI355X_F16}[t.dtype]
+    return _DTYPE_CODES[t.dtype]
 
 
 def _topk_scores(self, logits, k):
@@ -324,7 +330,6 @@ def _greedy_tail(self, next_tokens, eos_seen, eos_ids, pad, sequences, current_l
                                           sequences.shape[1], current_length, done.data_ptr()))
 
 
-_DTYPE_CODES = {torch.float32: 1, torch.int32: 6, torch.int64: 7, torch.float16: 10, torch.bfloat16: 16}
 
 
 def _cast(self, src, dtype):

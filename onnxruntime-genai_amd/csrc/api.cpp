@@ -78,8 +78,6 @@ struct mi355x_search_ctx {
   float* row_sum{};
   int32_t* row_index{};  // device copy of per-row host indices (logits hand-off)
   int32_t* beam_row_tokens{};
-  float* widen{};          // fp32 copy of fp16 rows (top-k scores), grown on demand
-  size_t widen_elems{};
 
   template <typename T>
   hipError_t Alloc(T** p, size_t count, bool zero) {
@@ -221,7 +219,6 @@ void mi355x_search_destroy(mi355x_search_ctx* ctx) {
   if (!ctx) return;
   (void)hipSetDevice(ctx->device);
   for (void* p : ctx->allocs) (void)hipFree(p);
-  if (ctx->widen) (void)hipFree(ctx->widen);
   delete ctx;
 }
 
@@ -243,16 +240,20 @@ int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int 
                   int rows, int vocab, const mi355x_logits_xform* xf, int32_t* out_tokens) {
   if (int r = CheckRows(ctx, rows, vocab)) return r;
   if (!logits || !out_tokens) return Fail(MI355X_E_INVALID, "null logits or output");
-  if (dtype != MI355X_F32 && dtype != MI355X_F16) return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
+  if (dtype != MI355X_F32 && dtype != MI355X_F16 && dtype != MI355X_BF16)
+    return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
   if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
-  // fp32 rows of more than a few workgroups' worth go through the fused selection kernel (k = 1, ids only)
+  // rows of more than 64 logits go through the fused selection kernel (k = 1, ids only), whatever their type
   const int fused_chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
-  if (dtype == MI355X_F32 && vocab > 64 && fused_chunks * ms::kSmallCap <= ms::kAllCap &&
-      rows * fused_chunks >= ms::kArgmaxFusedMinBlocks) {
+  const bool fused = vocab > 64 && fused_chunks * ms::kSmallCap <= ms::kAllCap && rows * fused_chunks >= ms::kArgmaxFusedMinBlocks;
+  if (dtype == MI355X_BF16 && !fused)
+    return Fail(MI355X_E_UNSUPPORTED, "bf16 rows need 64 < vocab <= %d", ms::kAllCap / ms::kSmallCap * ms::kSChunk);
+  if (fused) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     ms::SampleArgs f{};
     if (int r = MakeXform(ctx, xf, rows, vocab, s, &f.xf)) return r;
-    f.logits = static_cast<const float*>(logits);
+    f.logits = logits;
+    f.dtype = dtype;
     f.row_stride = row_stride;
     f.rows = rows;
     f.vocab = vocab;
@@ -289,8 +290,18 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
                   int vocab, const mi355x_logits_xform* xf, mi355x_sample_params params,
                   const mi355x_sample_params* per_row_params, const double* uniforms, int32_t* out_tokens,
                   int32_t* kept_count, int32_t* kept_ids, float* kept_probs, int kept_capacity) {
+  return mi355x_sample_typed(ctx, stream, logits, MI355X_F32, row_stride, rows, vocab, xf, params, per_row_params,
+                             uniforms, out_tokens, kept_count, kept_ids, kept_probs, kept_capacity);
+}
+
+int mi355x_sample_typed(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype, int64_t row_stride,
+                        int rows, int vocab, const mi355x_logits_xform* xf, mi355x_sample_params params,
+                        const mi355x_sample_params* per_row_params, const double* uniforms, int32_t* out_tokens,
+                        int32_t* kept_count, int32_t* kept_ids, float* kept_probs, int kept_capacity) {
   if (int r = CheckRows(ctx, rows, vocab)) return r;
   if (!logits || !uniforms || !out_tokens) return Fail(MI355X_E_INVALID, "null logits, uniforms or output");
+  if (dtype != MI355X_F32 && dtype != MI355X_F16 && dtype != MI355X_BF16)
+    return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
   if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
   if ((kept_ids || kept_probs) && kept_capacity <= 0) return Fail(MI355X_E_INVALID, "kept_capacity must be positive");
   if (kept_probs && !kept_ids) return Fail(MI355X_E_INVALID, "kept_probs requires kept_ids");
@@ -327,6 +338,7 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
     if (int rc = check(params)) return rc;
   }
   a.logits = logits;
+  a.dtype = dtype;
   a.row_stride = row_stride;
   a.rows = rows;
   a.vocab = vocab;
@@ -354,29 +366,17 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
                        int rows, int vocab, int k, int32_t* out_tokens, float* out_scores) {
   if (int r = CheckRows(ctx, rows, vocab)) return r;
   if (!logits || !out_tokens || !out_scores) return Fail(MI355X_E_INVALID, "null logits or output");
-  if (dtype != MI355X_F32 && dtype != MI355X_F16) return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
+  if (dtype != MI355X_F32 && dtype != MI355X_F16 && dtype != MI355X_BF16)
+    return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
   if (k < 1 || k > 64 || k > vocab) return Fail(MI355X_E_INVALID, "k (%d) must be in [1, min(64, vocab)]", k);
   if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const float* src = static_cast<const float*>(logits);
-  if (dtype == MI355X_F16) {
-    // widened once into an fp32 scratch, as DeviceInterface::TopKScores does (src/cuda/interface.cpp:440-451)
-    const size_t need = static_cast<size_t>(rows) * vocab;
-    if (need > ctx->widen_elems) {
-      HIP_TRY(hipStreamSynchronize(s));
-      if (ctx->widen) (void)hipFree(ctx->widen);
-      ctx->widen = nullptr;
-      ctx->widen_elems = 0;
-      HIP_TRY(hipMalloc(reinterpret_cast<void**>(&ctx->widen), need * sizeof(float)));
-      ctx->widen_elems = need;
-    }
-    HIP_TRY(ms_launch_widen_f16(logits, row_stride, ctx->widen, vocab, rows, vocab, s));
-    src = ctx->widen;
-    row_stride = vocab;
-  }
+  // sixteen-bit rows are read as they are and widened in registers (DeviceInterface::TopKScores makes an fp32
+  // copy first, src/cuda/interface.cpp:440-451); the scores returned are the widened values
   ms::SampleArgs a{};
   if (int r = MakeXform(ctx, nullptr, rows, vocab, s, &a.xf)) return r;
-  a.logits = src;
+  a.logits = logits;
+  a.dtype = dtype;
   a.row_stride = row_stride;
   a.rows = rows;
   a.vocab = vocab;

@@ -150,11 +150,46 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
   return __uint_as_float(sign | __float_as_uint(mag));
 }
 
+// Eight fp16 values in a 16-byte vector, widened as above.  The hardware conversion is exact for zeros,
+// subnormals and normals; the rare vector that holds an exponent field of 31 is redone by the bit formula.
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void widen_half8(v4u q, float* o) {
+  const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+  uint32_t suspicious = 0u;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    o[2 * c] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w[c] & 0xffffu)));
+    o[2 * c + 1] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w[c] >> 16)));
+    suspicious |= ((w[c] & 0x7c007c00u) + 0x04000400u) & 0x80008000u;  // a half whose exponent bits are all ones
+  }
+  if (__builtin_expect(suspicious != 0u, 0)) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      o[2 * c] = half_bits_to_float(w[c] & 0xffffu);
+      o[2 * c + 1] = half_bits_to_float(w[c] >> 16);
+    }
+  }
+}
+
 // bfloat16 -> fp32 as BFloat16ToFloat32 does (src/models/utils.cpp:84-86 via :55-77): the bits moved to
 // the upper half, except that every NaN becomes the canonical quiet NaN.
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t h) {
   if ((h & 0x7f80u) == 0x7f80u && (h & 0x7fu) != 0u) return __uint_as_float(0x7fc00000u);
   return __uint_as_float(h << 16);
+}
+
+struct bf16_t {  // a bfloat16 bit pattern (uint16_t stands for IEEE binary16 throughout)
+  uint16_t bits;
+};
+// Eight bfloat16 values in a 16-byte vector.  NaNs keep their payload here (the canonical quiet NaN of
+// bf16_bits_to_float is only needed where a value is written out): selection only asks whether a value is a NaN.
+__device__ __forceinline__ void widen_bf16x8(v4u q, float* o) {
+  const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    o[2 * c] = __uint_as_float(w[c] << 16);
+    o[2 * c + 1] = __uint_as_float(w[c] & 0xffff0000u);
+  }
 }
 
 // fp32 -> fp16 with FastFloat32ToFloat16's arithmetic (src/models/utils.cpp:111-118): the rounding
@@ -329,6 +364,10 @@ __device__ __forceinline__ float load_one<float>(const float* row, int idx) { re
 template <>
 __device__ __forceinline__ float load_one<uint16_t>(const uint16_t* row, int idx) {
   return half_bits_to_float(row[idx]);
+}
+template <>
+__device__ __forceinline__ float load_one<bf16_t>(const bf16_t* row, int idx) {
+  return bf16_bits_to_float(row[idx].bits);
 }
 
 }  // namespace ms

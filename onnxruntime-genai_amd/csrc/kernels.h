@@ -41,9 +41,10 @@ struct InlineParams {
 };
 
 struct SampleArgs {
-  const float* logits;
+  const void* logits;   // rows of fp32, fp16 or bf16 values (dtype), row_stride elements apart
   int64_t row_stride;
   int rows, vocab, chunks;
+  int dtype;            // MI355X_F32 / MI355X_F16 / MI355X_BF16 (0 counts as fp32)
   Xform xf;
   mi355x_sample_params uniform;
   const mi355x_sample_params* per_row;  // device, or null
@@ -181,8 +182,6 @@ hipError_t ms_launch_greedy_tail(int32_t* next_tokens, int32_t* eos_seen, int ba
                                  int32_t pad, int32_t* sequences, int max_length, int current_length, int32_t* done,
                                  hipStream_t stream);
 hipError_t ms_launch_spec_verify_sparse(const ms::SpecSparseArgs* a, int batch, hipStream_t stream);
-hipError_t ms_launch_widen_f16(const void* in, int64_t in_stride, float* out, int64_t out_stride, int rows,
-                               int vocab, hipStream_t stream);
 hipError_t ms_launch_cast(const void* in, void* out, size_t count, int kind, hipStream_t stream);
 hipError_t ms_launch_logits_handoff(const void* raw, int kind, int rows, int seq_len, int vocab,
                                     const int32_t* token_index, float* out, int64_t out_stride, hipStream_t stream);

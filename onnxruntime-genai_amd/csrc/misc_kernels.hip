@@ -1,5 +1,5 @@
 // Softmax / log-softmax with the reference's sequential fp32 sum, the KV-cache beam gather, the
-// speculative-decoding verifier and the fp16 -> fp32 widening copy.
+// speculative-decoding verifier, casts and the logits hand-off.
 #include "kernels.h"
 #include "block_seq.h"
 #include "wave_select.h"
@@ -459,15 +459,6 @@ __global__ __launch_bounds__(256) void spec_verify_sparse_kernel(const SpecSpars
   }
 }
 
-// fp16 -> fp32 with the reference's FastFloat16ToFloat32 semantics (DeviceInterface::Cast).
-__global__ __launch_bounds__(256) void widen_f16_kernel(const uint16_t* in, int64_t in_stride, float* out,
-                                                        int64_t out_stride, int vocab) {
-  const uint16_t* src = in + static_cast<size_t>(blockIdx.y) * in_stride;
-  float* dst = out + static_cast<size_t>(blockIdx.y) * out_stride;
-  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < vocab; i += gridDim.x * blockDim.x)
-    dst[i] = half_bits_to_float(src[i]);
-}
-
 // ---- DeviceInterface::Cast (src/cpu/interface.cpp:74-106) -----------------------------------------
 // kind: 0 fp16->fp32, 1 bf16->fp32, 2 fp32->fp16, 3 fp32->bf16 (upper 16 bits), 4 int32->int64.
 __global__ __launch_bounds__(256) void cast_kernel(const void* in, void* out, size_t count, int kind) {
@@ -599,11 +590,3 @@ extern "C" hipError_t ms_launch_spec_verify_sparse(const ms::SpecSparseArgs* a, 
   return hipGetLastError();
 }
 
-extern "C" hipError_t ms_launch_widen_f16(const void* in, int64_t in_stride, float* out, int64_t out_stride, int rows,
-                                          int vocab, hipStream_t stream) {
-  int gx = (vocab + 255) / 256;
-  if (gx > 512) gx = 512;
-  hipLaunchKernelGGL(ms::widen_f16_kernel, dim3(gx, rows), dim3(256), 0, stream, static_cast<const uint16_t*>(in),
-                     in_stride, out, out_stride, vocab);
-  return hipGetLastError();
-}

@@ -1,894 +1,15 @@
-// Sampling kernels.
-//
-// sample_fused_kernel (top-k rows, k <= 64; one launch per step): every workgroup (512 threads x 64
-// logits) streams one 32K-logit chunk of one row with 128-bit non-temporal loads, logits processing
-// fused, keeps the chunk's best 64 candidates and publishes them sorted; the workgroup of a row's last
-// chunk polls for the other chunks' lists, merges them four at a time (bitonic merges in registers)
-// and runs the reference's scalar epilogue (softmax over the k, nucleus cut, categorical draw) in rank
-// order.  nucleus_stream_kernel (rows with k <= 1; 1024 threads x 32 logits per workgroup) compacts
-// every chunk's candidates into the row's key buffer; nucleus_finish_kernel sorts them and finishes.
-// Anything the fast paths decline (k > 64, heavy ties, tiny vocabularies, more history ids in a chunk
-// than its list holds) goes through general_row, an exact full sort.  Each streaming kernel exists
-// with and without the code of the logits processing (_xf) and with the per-row parameters in a
-// device table or inside the kernel arguments (_rows).
-#include "kernels.h"
-#include "block_seq.h"
-#include "wave_select.h"
+// Finish kernels of the nucleus / large-k sampling paths, the fp32 streaming kernels and the launch logic of
+// mi355x_sample (the streaming kernels of fp16 and bf16 rows are instantiated in sample_kernels_f16.hip and
+// sample_kernels_bf16.hip from the same templates).
+#include "sample_stream.h"
+
+extern "C" {
+hipError_t ms_launch_stream(const ms::SampleArgs* a, const ms::InlineParams* table, int which, hipStream_t stream);
+hipError_t ms_launch_stream_f16(const ms::SampleArgs* a, const ms::InlineParams* table, int which, hipStream_t stream);
+hipError_t ms_launch_stream_bf16(const ms::SampleArgs* a, const ms::InlineParams* table, int which, hipStream_t stream);
+}
 
 namespace ms {
-
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-// (k, p, T) of a row.  INLINE kernels carry a table as their second argument and read it through the
-// kernel-argument segment itself (constant address space, scalar loads): indexing the by-value
-// argument object with a run-time row would make the compiler copy the whole object to private memory.
-static_assert(sizeof(SampleArgs) % alignof(InlineParams) == 0, "the table follows the first argument without padding");
-template <bool INLINE>
-__device__ __forceinline__ mi355x_sample_params row_params(const SampleArgs& a, int row) {
-  if constexpr (INLINE) {
-    typedef __attribute__((address_space(4))) const char* KernargPtr;
-    const KernargPtr base = (KernargPtr)__builtin_amdgcn_kernarg_segment_ptr();
-    typedef __attribute__((address_space(4))) const mi355x_sample_params* TablePtr;
-    const TablePtr table = (TablePtr)(base + sizeof(SampleArgs));
-    mi355x_sample_params q;
-    q.k = __builtin_amdgcn_readfirstlane(table[row].k);
-    q.p = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(table[row].p)));
-    q.temperature = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(table[row].temperature)));
-    return q;
-  } else {
-    // The device table is read-only during the launch: read through the constant address space, its
-    // entries come by scalar loads like the uniform parameters from the kernel arguments, the row's mode
-    // is a scalar, and nothing here waits for a vector load before the logits are requested.
-    mi355x_sample_params q = a.uniform;
-    if (a.per_row) {
-      typedef __attribute__((address_space(4))) const mi355x_sample_params* TablePtr;
-      const TablePtr table = (TablePtr)a.per_row;
-      q.k = table[row].k;
-      q.p = table[row].p;
-      q.temperature = table[row].temperature;
-    }
-    return q;
-  }
-}
-
-__device__ __forceinline__ int next_pow2(int v) {
-  int p = 64;
-  while (p < v) p <<= 1;
-  return p;
-}
-
-__device__ __forceinline__ RowOutputs row_outputs(const SampleArgs& a, int row) {
-  return RowOutputs{a.out_tokens + row, a.kept_count ? a.kept_count + row : nullptr,
-                    a.kept_ids ? a.kept_ids + static_cast<size_t>(row) * a.kept_capacity : nullptr,
-                    a.kept_probs ? a.kept_probs + static_cast<size_t>(row) * a.kept_capacity : nullptr,
-                    a.kept_capacity};
-}
-
-// Exact general path for one row, any (k, p, T), any vocabulary size: rebuilds the processed row as
-// key64s in global scratch, sorts all of it, then runs the reference algorithm on the sorted row.
-// Run by one whole block.  scratch holds next_pow2(vocab) entries.
-struct SortInGlobalMemory {
-  __device__ void operator()(u64* keys, int n2, int) const { block_sort_desc(keys, n2); }
-};
-
-template <typename SortFn = SortInGlobalMemory>
-__device__ __forceinline__ void general_row(const SampleArgs& a, int row, const mi355x_sample_params prm, u64* scratch, SeqShared& sh,
-                                            SortFn sort_desc = SortFn{}) {
-  const int V = a.vocab;
-  const float* lrow = a.logits + static_cast<size_t>(row) * a.row_stride;
-  const int n2 = next_pow2(V);
-  const bool has_mask = a.xf.mask != nullptr;
-  const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
-  const int n_eos = a.xf.eos_count(row);
-  const uint32_t* ban_row = a.xf.ban_row(row, V);
-  for (int i = threadIdx.x; i < n2; i += blockDim.x) {
-    u64 k = 0;
-    if (i < V) {
-      const float x = xform_value(lrow[i], a.xf.penalty, a.xf.eos, i, has_mask ? mrow[i >> 5] : 0u, has_mask, false, n_eos, ban_row);
-      k = make_key64(order_key(x), static_cast<uint32_t>(i));
-      if (i == 0 && x != x && a.emit_topk == kEmitArgmax) k = ~0ull;  // ArgMax starts from id 0 and nothing compares above a NaN
-    }
-    scratch[i] = k;
-  }
-  __syncthreads();
-  if (a.xf.use_penalty()) {
-    const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
-    const int hlen = a.xf.hist_len(row);
-    for (int j = threadIdx.x; j < hlen; j += blockDim.x) {
-      const int tok = h[j];
-      if (tok < 0 || tok >= V) continue;
-      bool dup = false;
-      for (int jj = 0; jj < j && !dup; ++jj) dup = (h[jj] == tok);
-      if (dup) continue;
-      const float x = xform_value(lrow[tok], a.xf.penalty, a.xf.eos, tok, has_mask ? mrow[tok >> 5] : 0u, has_mask, true, n_eos, ban_row);
-      scratch[tok] = (tok == 0 && x != x && a.emit_topk == kEmitArgmax) ? ~0ull : make_key64(order_key(x), static_cast<uint32_t>(tok));
-    }
-    __syncthreads();
-  }
-  sort_desc(scratch, n2, V);  // descending; entries from V on are 0
-  if (a.emit_topk) {
-    const int kk = prm.k < V ? prm.k : V;
-    for (int j = threadIdx.x; j < kk; j += blockDim.x) {
-      const uint32_t id = key64_index(scratch[j]);
-      a.out_tokens[static_cast<size_t>(row) * prm.k + j] = static_cast<int32_t>(id);
-      if (a.out_scores) a.out_scores[static_cast<size_t>(row) * prm.k + j] = lrow[id];  // the value itself: keys do not tell -0 from +0
-    }
-    if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
-    return;
-  }
-  const float max_score = key_to_float(key64_okey(scratch[0]));
-  const float inv_temp = 1.0f / prm.temperature;
-  const RowOutputs out = row_outputs(a, row);
-  const u64* sc = scratch;
-  auto sorted = [=](int i) { return sc[i]; };
-  auto exps = [=](int i) { return em::expf_exact((key_to_float(key64_okey(sc[i])) - max_score) * inv_temp); };
-  block_sample_epilogue<4>(sorted, exps, V, V, prm, a.uniforms[row], out, sh);
-  if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
-}
-
-__device__ __forceinline__ int row_mode(mi355x_sample_params prm, int vocab, int chunks, int emit_topk = 0) {
-  if (vocab <= 64 || chunks * kSmallCap > kAllCap) return kModeGeneral;
-  if (emit_topk) return kModeTopkSmall;
-  if (prm.k > 1) {
-    const int kk = prm.k < vocab ? prm.k : vocab;
-    return kk <= 64 ? kModeTopkSmall : (kk <= kLargeKMax ? kModeTopkLarge : kModeGeneral);
-  }
-  return kModeNucleus;
-}
-
-// Depth below the row maximum (in score units) past which no element can lie strictly inside the
-// nucleus: once exp((s-max)/T) <= (1-p)/(p*V) -- with a margin of e^2 for fp32 rounding -- the stop
-// test prefix >= p*(prefix + (V-i-1)*e) of FindNucleus is certainly true, because prefix >= 1.
-__device__ __forceinline__ float nucleus_depth(mi355x_sample_params prm, int vocab) {
-  float d = 105.0f;  // exp underflows to exactly 0 below -103.98
-  if (prm.p <= 0.0f) d = 0.0f;
-  else if (prm.p < 0.999f) d = fminf(105.0f, logf(prm.p * static_cast<float>(vocab) / (1.0f - prm.p)) + 2.0f);
-  return d * prm.temperature;
-}
-
-// Values of a published candidate slot that are not keys (a key's low half is ~id, far above these).
-constexpr u64 kSlotEmpty = 1, kSlotOverflow = 2;
-constexpr int kWaveListCap = 128;  // hits one wave can list per chunk
-constexpr int kExtraCap = 2048;    // distinct history ids one chunk can hold; beyond, the row takes the exact path
-constexpr uint32_t kChunkCntOverflow = 0xffffffffu;  // chunk_cnt of a nucleus chunk that gave up
-
-// LDS of the fused kernel.
-struct FusedShared {
-  uint32_t hist_bits[kSChunk / 32];
-  uint32_t mask_bits[kSChunk / 32];
-  u64 wave_list[kSMaxWaves * kWaveListCap];  // each wave's hits of this chunk, before the sort
-  u64 list_hi[64];          // second half of a long list, sorted ascending
-  u64 own[64];              // the finishing workgroup's own list
-  u64 lists[kAllCap / 4];   // first-level results of the finishing workgroup's merge (rows of > 4 chunks)
-  uint32_t pool[64];
-  uint32_t wave_val[kSMaxWaves];
-  u64 wave_val64[kSMaxWaves];
-  uint32_t count, flag;
-  uint32_t nan0;  // the processed logit of id 0 is a NaN (set in chunk 0; used by the argmax output)
-  uint32_t n_extra;
-  float extra_val[kExtraCap];     // processed logits of the history ids of this chunk ...
-  uint32_t extra_idx[kExtraCap];  // ... and their ids
-  SeqShared seq;
-};
-
-template <int BLOCK>
-__device__ __forceinline__ int elem_index(int chunk, int j, int c) {
-  return chunk * kSChunk + (j * BLOCK + static_cast<int>(threadIdx.x)) * 4 + c;
-}
-
-// The 32-entry table of expf_core, one entry per lane (lane & 31), fetched by lane shuffle.
-struct LaneExp2Tab {
-  uint32_t lo, hi;
-  __device__ uint64_t operator()(uint32_t i) const {
-    const uint32_t l = __shfl(lo, static_cast<int>(i), 64);
-    const uint32_t h = __shfl(hi, static_cast<int>(i), 64);
-    return (static_cast<uint64_t>(h) << 32) | l;
-  }
-};
-
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ double dpp_from_below(double x) {
-  const u64 b = static_cast<u64>(__double_as_longlong(x));
-  const uint32_t lo = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b), CTRL, ROW_MASK, 0xf, false);
-  const uint32_t hi = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b >> 32), CTRL, ROW_MASK, 0xf, false);
-  return __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
-}
-
-// Inclusive prefix sums over the wave in tree order (lanes without a source add +0.0).
-__device__ __forceinline__ double wave_scan_add(double x) {
-  x += dpp_from_below<0x111, 0xf>(x);  // row_shr:1
-  x += dpp_from_below<0x112, 0xf>(x);  // row_shr:2
-  x += dpp_from_below<0x114, 0xf>(x);  // row_shr:4
-  x += dpp_from_below<0x118, 0xf>(x);  // row_shr:8
-  x += dpp_from_below<0x142, 0xa>(x);  // row_bcast:15 into rows 1 and 3
-  x += dpp_from_below<0x143, 0xc>(x);  // row_bcast:31 into rows 2 and 3
-  return x;
-}
-
-__device__ __forceinline__ float read_lane(float x, int l) {
-  return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(x), l));
-}
-__device__ __forceinline__ u64 read_lane(u64 x, int l) {
-  const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(x), l);
-  const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(x >> 32), l);
-  return (static_cast<u64>(hi) << 32) | lo;
-}
-__device__ __forceinline__ double read_lane(double x, int l) {
-  const u64 b = static_cast<u64>(__double_as_longlong(x));
-  const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(b), l);
-  const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(b >> 32), l);
-  return __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
-}
-
-// Epilogue for k <= 64 run by one wave: lane j holds the j-th best (key64), j < m.
-// Follows ComputeSampledCategorical's top-k branch (src/sampling_distribution.h:243-281) and
-// std::discrete_distribution literally: every fp32 sum is accumulated in rank order.  The fp64
-// cumulative distribution is first evaluated in tree order on the raw weights; only if the draw lies
-// within rounding distance of one of its values is it rebuilt with the reference's own sequence of
-// operations (division by the sum, sequential partial sums), so the chosen position is always the
-// sequential one.
-__device__ __forceinline__ void wave_topk_epilogue(u64 key, int m, mi355x_sample_params prm, double u,
-                                                   LaneExp2Tab tab, const RowOutputs& out) {
-  const int lane = lane_id();
-  m = __builtin_amdgcn_readfirstlane(m);
-  const float score = key_to_float(key64_okey(key));
-  const float max_score = read_lane(score, 0);
-  const float inv_temp = 1.0f / prm.temperature;
-  const float e_all = em::expf_core((score - max_score) * inv_temp, tab);
-  const float e = lane < m ? e_all : 0.0f;
-  const float sum = read_lane(wave_serial_prefix(e, m), m - 1);
-  const float pr = sum > 0.0f ? e / sum : e;
-  // cumulative probabilities, eight chain steps at a time; with a top-p cut the chain stops at the
-  // first group that contains the cut (lanes below the number of steps done hold final values)
-  const bool cut = prm.p > 0.0f && prm.p < 1.0f;
-  float cum = 0.0f;
-  int keep = m;
-  for (int t = 0; t < m; t += 8) {
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const float prev = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(cum), 0x138, 0xf, 0xf, false));
-      cum = prev + pr;
-    }
-    if (cut) {
-      const int f = first_lane(__ballot(lane < t + 8 && lane < m && cum >= prm.p));
-      if (f >= 0) {
-        keep = f + 1;
-        break;
-      }
-    }
-  }
-  keep = __builtin_amdgcn_readfirstlane(keep);
-  const float keep_sum = read_lane(cum, keep - 1);
-  const float inv = keep_sum > 0.0f ? 1.0f / keep_sum : 0.0f;
-  const float q = pr * inv;
-  int pos = 0;
-  if (keep >= 2) {
-    const double qd = lane < keep ? static_cast<double>(q) : 0.0;
-    const double w = wave_scan_add(qd);
-    const double total = read_lane(w, keep - 1);
-    const double target = u * total;
-    const double guard = 16.0 * static_cast<double>(keep) * 1.1102230246251565e-16 * total;
-    const bool risky = __ballot(lane < keep - 1 && fabs(w - target) <= guard) != 0ull;
-    if (!risky) {
-      pos = first_lane(__ballot(lane < keep && (lane == keep - 1 || w >= target)));
-    } else {
-      const double dsum = read_lane(wave_serial_prefix(qd, keep), keep - 1);
-      const double pn = qd / dsum;
-      double cp = wave_serial_prefix(pn, keep);
-      if (lane == keep - 1) cp = 1.0;
-      pos = first_lane(__ballot(lane < keep && cp >= u));
-    }
-    if (pos < 0) pos = keep - 1;
-    if (total != total) pos = 0;  // NaN weights: std::lower_bound over NaN quotients ends on 0
-  }
-  const uint32_t idx = key64_index(key);
-  const int32_t tok = static_cast<int32_t>(__builtin_amdgcn_readlane(idx, pos));
-  if (lane == 0) {
-    *out.token = tok;
-    if (out.kept_count) *out.kept_count = keep;
-  }
-  if (out.kept_ids && lane < keep && lane < out.kept_capacity) {
-    out.kept_ids[lane] = static_cast<int32_t>(idx);
-    if (out.kept_probs) out.kept_probs[lane] = q;
-  }
-}
-
-__device__ const uint64_t g_exp2_tab[32] = {
-    0x3ff0000000000000ULL, 0x3fefd9b0d3158574ULL, 0x3fefb5586cf9890fULL, 0x3fef9301d0125b51ULL,
-    0x3fef72b83c7d517bULL, 0x3fef54873168b9aaULL, 0x3fef387a6e756238ULL, 0x3fef1e9df51fdee1ULL,
-    0x3fef06fe0a31b715ULL, 0x3feef1a7373aa9cbULL, 0x3feedea64c123422ULL, 0x3feece086061892dULL,
-    0x3feebfdad5362a27ULL, 0x3feeb42b569d4f82ULL, 0x3feeab07dd485429ULL, 0x3feea47eb03a5585ULL,
-    0x3feea09e667f3bcdULL, 0x3fee9f75e8ec5f74ULL, 0x3feea11473eb0187ULL, 0x3feea589994cce13ULL,
-    0x3feeace5422aa0dbULL, 0x3feeb737b0cdc5e5ULL, 0x3feec49182a3f090ULL, 0x3feed503b23e255dULL,
-    0x3feee89f995ad3adULL, 0x3feeff76f2fb5e47ULL, 0x3fef199bdd85529cULL, 0x3fef3720dcef9069ULL,
-    0x3fef5818dcfba487ULL, 0x3fef7c97337b9b5fULL, 0x3fefa4afa2a490daULL, 0x3fefd0765b6e4540ULL,
-};
-
-// Workgroup barrier that orders LDS accesses only: unlike __syncthreads() it does not wait for the
-// global loads still in flight.
-__device__ __forceinline__ void lds_barrier() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-// block_max with barriers that do not wait for global memory.
-template <int kSWaves, typename T>
-__device__ __forceinline__ T block_max_lds(T v, T* scratch) {
-  v = wave_max(v);
-  const int lane = lane_id(), wave = threadIdx.x >> 6;
-  if (lane == 0) scratch[wave] = v;
-  lds_barrier();
-  T r = scratch[0];
-#pragma unroll
-  for (int w = 1; w < kSWaves; ++w) r = scratch[w] > r ? scratch[w] : r;
-  lds_barrier();
-  return r;
-}
-
-// Applies the two LDS bitmaps of a chunk to the registers of a thread: an id whose bit in `allowed` is
-// clear becomes kLowest, an id whose bit in `history` is set becomes NaN (its processed value lives in
-// the extras list).  Branch-free: the bit, spread over a word, selects between the two bit patterns.
-template <int kSBlock, bool ALLOWED, bool HISTORY>
-__device__ __forceinline__ void mask_registers(float (&v)[kSChunk / kSBlock], const uint32_t* allowed,
-                                               const uint32_t* history, int tid) {
-  constexpr int kSVec = kSChunk / (kSBlock * 4);
-#pragma unroll
-  for (int j = 0; j < kSVec; ++j) {
-    const int rel0 = (j * kSBlock + tid) * 4;
-    const uint32_t anib = ALLOWED ? allowed[rel0 >> 5] >> (rel0 & 31) : 0u;
-    const uint32_t hnib = HISTORY ? history[rel0 >> 5] >> (rel0 & 31) : 0u;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      uint32_t x = __float_as_uint(v[j * 4 + c]);
-      if (ALLOWED) {
-        uint32_t keep = static_cast<uint32_t>(static_cast<int32_t>(anib << (31 - c)) >> 31);
-        asm volatile("" : "+v"(keep));  // stays a bitwise select (one instruction) instead of compare + select
-        x = (x & keep) | (0xff7fffffu & ~keep);  // bits of kLowest
-      }
-      if (HISTORY) {
-        const uint32_t drop = static_cast<uint32_t>(static_cast<int32_t>(hnib << (31 - c)) >> 31);
-        x |= drop;  // all ones is a NaN
-      }
-      v[j * 4 + c] = __uint_as_float(x);
-    }
-    if ((j & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // at most eight bitmap words in registers at a time
-  }
-}
-
-// Streaming pass of one (row, chunk) of a top-k<=64 or nucleus row.  Returns true when this workgroup
-// must run the general path for the row (it was the last to arrive and the fast path declined).
-template <bool NUCLEUS, bool XFORM, bool LARGEK = false>
-__device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chunk, mi355x_sample_params prm,
-                                           FusedShared& sm) {
-  constexpr int kSBlock = NUCLEUS ? kNucleusBlock : kTopkBlock;  // threads of this workgroup
-  constexpr int kSWaves = kSBlock / 64;
-  constexpr int kSVec = kSChunk / (kSBlock * 4);  // 128-bit loads per thread
-  constexpr int kSElems = kSVec * 4;              // logits held in registers per thread
-  const int V = a.vocab;
-  const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
-  u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
-  const float* lrow = a.logits + static_cast<size_t>(row) * a.row_stride;
-  const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
-  const float kNaN = __uint_as_float(0x7fc00000u);  // marks ids >= vocab: never a maximum, never >= a bound
-  const uint32_t poison = *a.fallback_rows;  // needed after the streaming pass only
-  float v[kSElems];
-#pragma unroll
-  for (int j = 0; j < kSVec; ++j) {
-    const int i0 = elem_index<kSBlock>(chunk, j, 0);
-    if (aligned && i0 + 4 <= V) {
-      const v4f q = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(lrow + i0));
-      v[j * 4 + 0] = q.x;
-      v[j * 4 + 1] = q.y;
-      v[j * 4 + 2] = q.z;
-      v[j * 4 + 3] = q.w;
-    } else {
-#pragma unroll
-      for (int c = 0; c < 4; ++c) v[j * 4 + c] = (i0 + c < V) ? lrow[i0 + c] : kNaN;
-    }
-  }
-  // The arguments the phases after the streaming pass need are fetched now, while the logits are in
-  // flight, instead of one by one where they are first used.
-  const int n_chunks = arg_now(a.chunks);
-  u64* const cand_small = arg_now(a.cand_small);
-  const double* const uniforms = arg_now(a.uniforms);
-  const int emit_topk = arg_now(a.emit_topk);
-  const int poll_limit = arg_now(a.poll_limit);
-  const RowOutputs outputs = {arg_now(a.out_tokens) + row,
-                              arg_now(a.kept_count),
-                              arg_now(a.kept_ids),
-                              arg_now(a.kept_probs),
-                              arg_now(a.kept_capacity)};
-  // ---- logits processing ----------------------------------------------------------------------
-  // Grammar mask and min-length masking reach the registers as one LDS bitmap of allowed ids (a clear
-  // bit -> kLowest; ids past the vocabulary count as allowed and keep their NaN).  The ids of the row's
-  // history are few and their processing (a correctly rounded division, the n-gram ban) is long, so
-  // they leave the register arrays altogether: a second bitmap turns them into NaN there, and the
-  // threads that marked them compute their processed values into a short list in LDS, `extras`, which
-  // every later phase visits next to the registers.
-  // The bitmap words and the first history ids of this thread are requested before anything waits.
-  constexpr int kWordsPerThread = kSChunk / 32 / kSBlock;  // bitmap words a thread stages
-  static_assert(kWordsPerThread >= 1 && kSChunk / 32 == kWordsPerThread * kSBlock, "whole bitmap words per thread");
-  const bool active = XFORM && a.xf.active();  // kernels without logits processing carry none of its code
-  const bool pen = active && a.xf.use_penalty();
-  const bool has_mask = active && a.xf.mask != nullptr;
-  const int words = (V - 1) / 32 + 1;
-  const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * words : nullptr;
-  const int32_t* hist = pen ? a.xf.history + static_cast<size_t>(row) * a.xf.history_stride : nullptr;
-  const bool hist_ahead = pen && a.xf.history_lens == nullptr;  // the length is known without a load
-  int hist_pre[2] = {-1, -1};
-  uint32_t mask_pre[kWordsPerThread];
-#pragma unroll
-  for (int q = 0; q < 2; ++q)
-    if (hist_ahead && tid + q * kSBlock < a.xf.history_len) hist_pre[q] = hist[tid + q * kSBlock];
-#pragma unroll
-  for (int q = 0; q < kWordsPerThread; ++q) {
-    mask_pre[q] = ~0u;
-    if (has_mask) {
-      const int w = chunk * (kSChunk / 32) + tid + q * kSBlock;
-      mask_pre[q] = w < words ? mrow[w] : 0u;
-    }
-  }
-  uint32_t n_extra = 0u;
-  bool extra_overflow = false;
-  if (XFORM && active) {
-    const int n_eos = a.xf.eos_count(row);
-    if (tid == 0) {
-      sm.n_extra = 0u;
-      sm.nan0 = 0u;
-    }
-#pragma unroll
-    for (int q = 0; q < kWordsPerThread; ++q) {
-      const int i = tid + q * kSBlock;
-      const int w = chunk * (kSChunk / 32) + i;
-      uint32_t word = mask_pre[q];
-      for (int e = 0; e < n_eos; ++e)
-        if ((a.xf.eos[e] >> 5) == w) word &= ~(1u << (a.xf.eos[e] & 31));
-      const int n_real = V - w * 32;  // ids of this word inside the vocabulary
-      if (n_real < 32) word |= n_real <= 0 ? ~0u : (~0u << n_real);
-      sm.mask_bits[i] = word;
-      sm.hist_bits[i] = 0u;
-    }
-    lds_barrier();
-    if (pen) {
-      const int hlen = a.xf.hist_len(row);
-      const float penalty = a.xf.penalty;
-      const uint32_t* ban_row = a.xf.ban_row(row, V);
-      // the thread that is first to mark an id computes its processed value
-      auto visit = [&](int id) {
-        const int rel = id - chunk * kSChunk;
-        if (rel >= 0 && rel < kSChunk && id < V) {
-          const uint32_t bit = 1u << (rel & 31);
-          if (!(atomicOr(&sm.hist_bits[rel >> 5], bit) & bit)) {
-            const uint32_t slot = atomicAdd(&sm.n_extra, 1u);
-            if (slot < static_cast<uint32_t>(kExtraCap)) {
-              const uint32_t mw = has_mask ? mrow[id >> 5] : 0u;
-              const float val = xform_value(lrow[id], penalty, a.xf.eos, id, mw, has_mask, true, n_eos, ban_row);
-              sm.extra_val[slot] = val;
-              sm.extra_idx[slot] = static_cast<uint32_t>(id);
-              if (id == 0 && val != val) sm.nan0 = 1u;
-            }
-          }
-        }
-      };
-      int first = tid;
-      if (hist_ahead) {
-        if (tid < hlen) visit(hist_pre[0]);
-        if (tid + kSBlock < hlen) visit(hist_pre[1]);
-        first = tid + 2 * kSBlock;
-      }
-      for (int i = first; i < hlen; i += kSBlock) visit(hist[i]);
-      lds_barrier();
-      n_extra = sm.n_extra;
-      extra_overflow = n_extra > static_cast<uint32_t>(kExtraCap);  // the row takes the exact path
-      if (extra_overflow) n_extra = 0u;
-    }
-    mask_registers<kSBlock, true, true>(v, sm.mask_bits, sm.hist_bits, tid);
-  }
-  // per-thread maximum in the float domain (fmaxf skips NaN), keeping the maximum of every float4
-  float qm[kSVec];
-  float fm = -__builtin_inff();
-#pragma unroll
-  for (int j = 0; j < kSVec; ++j) {
-    qm[j] = fmaxf(fmaxf(v[j * 4], v[j * 4 + 1]), fmaxf(v[j * 4 + 2], v[j * 4 + 3]));
-    fm = fmaxf(fm, qm[j]);
-  }
-  for (uint32_t i = tid; i < n_extra; i += kSBlock) fm = fmaxf(fm, sm.extra_val[i]);
-  // 0: the thread holds no element
-  const uint32_t lmax = (elem_index<kSBlock>(chunk, 0, 0) < V || static_cast<uint32_t>(tid) < n_extra) ? order_key(fm) : 0u;
-  if (tid == 0) {
-    sm.count = 0u;
-    if constexpr (!NUCLEUS) {
-      // id 0's processed value is v[0] unless id 0 is in the history (then its owner has set the flag)
-      const bool in_history = XFORM && pen && (sm.hist_bits[0] & 1u) != 0u;
-      const bool is_nan = chunk == 0 && !in_history && v[0] != v[0];
-      if (!(XFORM && active)) sm.nan0 = is_nan ? 1u : 0u;
-      else if (is_nan) sm.nan0 = 1u;
-    }
-  }
-
-  if constexpr (NUCLEUS) {
-    // Everything within nucleus_depth of the chunk maximum goes to the row's key buffer, in no
-    // particular order (the finish kernel sorts).  A wave counts its candidates, reserves a range of
-    // the chunk's list with one LDS atomic and fills it; the slot of a candidate is the wave's running
-    // count plus the number of candidate lanes below.
-    // Rows with 64 < k <= kLargeKMax come here too: their candidates are the elements that reach the
-    // exact k-th best per-thread maximum of the chunk (at least k elements do; with fewer than k
-    // threads holding elements, all), which contain the chunk's k best.
-    static_assert(kLargeKMax <= kSBlock && kSMaxWaves * kWaveListCap >= kSBlock, "one offer per thread, sorted in the hit lists' LDS");
-    constexpr bool large_k = LARGEK;
-    const uint32_t cmax = block_max<uint32_t>(lmax, sm.wave_val);
-    float thr = -__builtin_inff();
-    if (large_k) {
-      u64* scratch = sm.wave_list;
-      scratch[tid] = static_cast<u64>(lmax);
-      __syncthreads();
-      block_sort_desc(scratch, kSBlock);
-      const uint32_t kth = static_cast<uint32_t>(scratch[(prm.k < V ? prm.k : V) - 1]);
-      if (kth != 0u) thr = key_to_float(kth);
-      __syncthreads();
-    } else if (cmax != 0u) {
-      thr = key_to_float(cmax) - nucleus_depth(prm, V);
-    }
-    // First pass: the wave's number of candidates.
-    uint32_t wcnt = 0u;
-#pragma unroll
-    for (int e = 0; e < kSElems; ++e) wcnt += static_cast<uint32_t>(__popcll(__ballot(v[e] >= thr)));  // false for NaN
-    for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
-      const uint32_t i = i0 + tid;
-      wcnt += static_cast<uint32_t>(__popcll(__ballot(i < n_extra && sm.extra_val[i] >= thr)));
-    }
-    uint32_t woff = 0u;
-    if (lane == 0) woff = atomicAdd(&sm.count, wcnt);
-    woff = __builtin_amdgcn_readfirstlane(woff);
-    // Second pass: the stores.  The list holds (raw float bits, ~id): the finish kernel turns the bits
-    // into order keys.  The compares are made afresh against a copy of the threshold the compiler
-    // cannot identify with the first one, so that the 64 lane masks of the first pass need not stay
-    // alive.  Nothing below waits for the stores.
-    char* const dst = reinterpret_cast<char*>(big_row + static_cast<size_t>(chunk) * kSChunk);
-    float thr2 = thr;
-    asm volatile("" : "+v"(thr2));
-    const uint32_t nid0 = ~static_cast<uint32_t>(elem_index<kSBlock>(chunk, 0, 0));  // ~(id0 + d) = ~id0 - d
-#pragma unroll
-    for (int e = 0; e < kSElems; ++e) {
-      const bool cand = v[e] >= thr2;
-      const u64 b = __ballot(cand);
-      if (cand) {
-        const uint32_t pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
-                                                       __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), woff));
-        const uint32_t nid = nid0 - static_cast<uint32_t>((e / 4) * kSBlock * 4 + (e % 4));
-        *reinterpret_cast<u64*>(dst + pos * 8u) = make_key64(__float_as_uint(v[e]), ~nid);
-      }
-      woff += static_cast<uint32_t>(__popcll(b));
-      __builtin_amdgcn_sched_barrier(0);  // keeps the keys of later elements from being built early
-    }
-    u64 extra_below = 0;  // the best of this thread's extras below the threshold, as a whole key
-    for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
-      const uint32_t i = i0 + tid;
-      const float ev = i < n_extra ? sm.extra_val[i] : kNaN;
-      const uint32_t ei = i < n_extra ? sm.extra_idx[i] : 0u;
-      const bool cand = ev >= thr2;
-      const u64 b = __ballot(cand);
-      if (cand) {
-        const uint32_t pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
-                                                       __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), woff));
-        *reinterpret_cast<u64*>(dst + pos * 8u) = make_key64(__float_as_uint(ev), ei);
-      }
-      woff += static_cast<uint32_t>(__popcll(b));
-      const u64 key = make_key64(order_key(ev), ei);
-      if (ev < thr2 && key > extra_below) extra_below = key;
-    }
-    // The best element below the threshold, first of equals: the block agrees on the best score, then
-    // the few threads that hold it look up its lowest id.
-    float thr3 = thr;
-    asm volatile("" : "+v"(thr3));
-    float fb = -__builtin_inff();
-#pragma unroll
-    for (int e = 0; e < kSElems; ++e) {
-      if (v[e] < thr3 && v[e] > fb) fb = v[e];  // compares are false for NaN
-      __builtin_amdgcn_sched_barrier(0);        // each lane mask is used at once
-    }
-    uint32_t fbk = 0u;  // 0: the thread has no element below the threshold
-    if (fb > -__builtin_inff()) {
-      fbk = order_key(fb);
-    } else if (thr3 > -__builtin_inff()) {  // an element equal to -inf is one, too
-      bool any = false;
-#pragma unroll
-      for (int e = 0; e < kSElems; ++e) any = any || v[e] == -__builtin_inff();
-      if (any) fbk = order_key(-__builtin_inff());
-    }
-    const uint32_t ebk = key64_okey(extra_below);
-    const uint32_t bbk = block_max_lds<kSWaves, uint32_t>(fbk > ebk ? fbk : ebk, sm.wave_val);
-    u64 best_below = ebk == bbk ? extra_below : 0;
-    if (bbk != 0u && fbk == bbk) {
-      const float bbf = key_to_float(bbk);
-      int fe = 0;
-#pragma unroll
-      for (int e = kSElems - 1; e >= 0; --e)
-        if (v[e] == bbf) fe = e;
-      const u64 key = make_key64(bbk, static_cast<uint32_t>(elem_index<kSBlock>(chunk, fe >> 2, fe & 3)));
-      best_below = key > best_below ? key : best_below;
-    }
-    best_below = block_max_lds<kSWaves, u64>(best_below, sm.wave_val64);  // its barriers also order the atomics on sm.count
-    if (tid == 0) {
-      const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
-      a.chunk_cnt[ci] = extra_overflow ? kChunkCntOverflow : sm.count;
-      a.chunk_max[ci] = cmax;
-      a.chunk_next[ci] = best_below;
-    }
-    return false;
-  }
-
-  // ---- top-k, k <= 64 ---------------------------------------------------------------------------
-  // A finishing workgroup that once gave up waiting may have left published lists behind; from then on
-  // (bit 31 of the fallback counter) every row takes the exact path, which reads no such state.
-  if (poison >> 31) return chunk == n_chunks - 1;
-  const int kk = prm.k < V ? prm.k : V;
-  int n_valid = V - chunk * kSChunk;
-  if (n_valid > kSChunk) n_valid = kSChunk;
-  int n_lanes = n_valid >= 4 * kSBlock ? kSBlock : (n_valid + 3) / 4;  // threads that hold elements
-  if (static_cast<uint32_t>(n_lanes) < n_extra) n_lanes = n_extra < static_cast<uint32_t>(kSBlock) ? static_cast<int>(n_extra) : kSBlock;
-  const size_t ci = static_cast<size_t>(row) * n_chunks + chunk;
-  u64* dst = cand_small + ci * kSmallCap;
-  uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool);
-  // The pooled bound is exact unless one wave holds more than its share of the best k; with k close to
-  // 64 it can sit low enough for the hits to overflow their lists, and in a short tail chunk it may
-  // find fewer than k offers (0).  Either way the exact k-th best of the per-thread maxima takes its
-  // place: about k + k*k/1024 elements reach that one.
-  static_assert(kSWaves * kWaveListCap >= kSBlock, "the hit lists double as the sort buffer of the exact bound");
-  uint32_t n_c = 0u, cnt[kSWaves];
-  bool overflow = false;
-  // exact k-th best of the per-thread maxima
-  auto exact_bound = [&]() {
-    u64* scratch = sm.wave_list;  // free until the hits are listed
-    scratch[tid] = static_cast<u64>(lmax);
-    __syncthreads();
-    block_sort_desc(scratch, kSBlock);
-    const uint32_t t = static_cast<uint32_t>(scratch[kk - 1]);
-    __syncthreads();
-    return t;
-  };
-  // Hits are rare (about k per chunk).  Every wave lists its own hits in a private LDS segment: the
-  // slot of a hit is the wave's running count (a scalar) plus the number of hitting lanes below, so
-  // no atomics, no second pass and no block-wide prefix are needed.  Ends with the per-wave counts.
-  auto list_hits = [&](uint32_t bound) {
-    // bound == 0: the chunk has fewer than k elements -- keep them all
-    const float tau_f = bound != 0u ? key_to_float(bound) : -__builtin_inff();
-    uint32_t woff = 0u;
-#pragma unroll
-    for (int j = 0; j < kSVec; ++j) {
-      if (__ballot(qm[j] >= tau_f) != 0ull) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const bool hit = v[j * 4 + c] >= tau_f;
-          const u64 b = __ballot(hit);
-          if (b == 0ull) continue;
-          if (hit) {
-            const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
-                                                                  __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), 0u));
-            // key64 of a real element is never 0 (its index half is ~idx != 0), so 0 marks an empty slot
-            // listed with the raw float bits; the few entries that survive get their order keys later
-            if (pos < kWaveListCap)
-              sm.wave_list[wave * kWaveListCap + pos] =
-                  make_key64(__float_as_uint(v[j * 4 + c]), static_cast<uint32_t>(elem_index<kSBlock>(chunk, j, c)));
-          }
-          woff += static_cast<uint32_t>(__popcll(b));
-        }
-      }
-    }
-    for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
-      const uint32_t i = i0 + tid;
-      const float ev = i < n_extra ? sm.extra_val[i] : kNaN;
-      const bool hit = ev >= tau_f;
-      const u64 b = __ballot(hit);
-      if (hit) {
-        const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32),
-                                                              __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), 0u));
-        if (pos < kWaveListCap) sm.wave_list[wave * kWaveListCap + pos] = make_key64(__float_as_uint(ev), sm.extra_idx[i]);
-      }
-      woff += static_cast<uint32_t>(__popcll(b));
-    }
-    if (lane == 0) sm.wave_val[wave] = woff;
-    __syncthreads();
-    n_c = 0u;
-    overflow = false;
-#pragma unroll
-    for (int w = 0; w < kSWaves; ++w) {
-      cnt[w] = sm.wave_val[w];
-      n_c += cnt[w];
-      overflow = overflow || cnt[w] > static_cast<uint32_t>(kWaveListCap);
-    }
-    overflow = overflow || n_c > static_cast<uint32_t>(kListCap);
-  };
-  const bool pooled = tau != 0u;
-  if (__builtin_expect(!pooled, 0)) tau = exact_bound();
-  list_hits(tau);
-  if (__builtin_expect(overflow && pooled, 0)) {  // rare: a second, separate copy of the listing code, with the exact bound
-    tau = exact_bound();
-    list_hits(tau);
-  }
-  overflow = overflow || extra_overflow;
-  // The chunk's best 64 candidates, sorted (best first): nothing ranked lower inside its own chunk can
-  // be among the row's k <= 64 best.  Waves 0 and 1 sort one half of the list each, wave 0 merges.
-  // The workgroup of the row's LAST chunk finishes the row; every other workgroup publishes its list
-  // and is done.  A published slot is never 0: kSlotEmpty pads a short list, kSlotOverflow replaces a
-  // list that did not fit.  The finishing workgroup polls the slots until all of them are non-zero and
-  // clears them again for the next launch; no counter, no wait for the stores and no second round
-  // trip lie between a chunk's sort and the row's merge.  Workgroups are dispatched in index order
-  // and a publishing workgroup never waits, so the lists a finishing workgroup polls for belong to
-  // workgroups that are running or done.
-  const bool two_halves = n_c > 64u;
-  const bool finisher = chunk == n_chunks - 1;
-  u64 mykey = 0;
-  if (wave < 2 && !overflow) {
-    // entry p of the concatenated wave lists: list w covers [start_w, start_w + count_w)
-    const uint32_t p = static_cast<uint32_t>(wave) * 64u + static_cast<uint32_t>(lane);
-    if (p < n_c) {
-      uint32_t start = 0u, w = 0u, off = 0u;
-#pragma unroll
-      for (int i = 0; i < kSWaves - 1; ++i) {
-        start += cnt[i];
-        if (p >= start) {
-          w = static_cast<uint32_t>(i) + 1u;
-          off = start;
-        }
-      }
-      const u64 raw = sm.wave_list[w * kWaveListCap + (p - off)];
-      mykey = (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw >> 32)))) << 32) |
-              (raw & 0xffffffffull);
-    }
-    if (wave == 0 || two_halves) mykey = wave_sort_desc_fast<u64>(mykey);
-    if (wave == 1 && two_halves) sm.list_hi[63 - lane] = mykey;
-  }
-  if (two_halves && !overflow) __syncthreads();
-  if (wave == 0) {
-    if (!overflow && two_halves) {
-      const u64 other = sm.list_hi[lane];  // ascending against descending: a bitonic pair
-      mykey = other > mykey ? other : mykey;
-      sort_merge<64, 32, u64>(mykey, lane);
-    }
-    // ArgMax starts from id 0 and nothing compares above a NaN (src/search.h:9-29): such a row's answer is 0
-    if (emit_topk == kEmitArgmax && chunk == 0 && lane == 0 && sm.nan0 != 0u) mykey = ~0ull;
-    const u64 slot = overflow ? kSlotOverflow : (mykey != 0 ? mykey : kSlotEmpty);
-    if (finisher) sm.own[lane] = slot;
-    else store_coherent(&dst[lane], slot);
-  }
-  if (!finisher) return false;
-
-  // ---- the row's finishing workgroup ---------------------------------------------------------------
-  LaneExp2Tab tab;
-  {
-    const uint64_t t = g_exp2_tab[lane & 31];  // issued now, consumed by the epilogue
-    tab.lo = static_cast<uint32_t>(t);
-    tab.hi = static_cast<uint32_t>(t >> 32);
-  }
-  const double u = emit_topk ? 0.0 : uniforms[row];
-  // sm.own is written by wave 0; with at most four chunks wave 0 alone reads it (a wave's LDS accesses execute in order)
-  if (n_chunks > 4) __syncthreads();
-  u64* seg = cand_small + static_cast<size_t>(row) * n_chunks * kSmallCap;
-  // Wave w merges the sorted lists of chunks 4w .. 4w+3 in registers, straight from global memory;
-  // rows of more than four chunks need a second level through LDS.  Wave 0 ends with the row's 64
-  // best, checks that there are k of them, and runs the epilogue while the other waves wait at the
-  // barrier that tells the workgroup whether the exact path is needed after all.
-  const int chunks = n_chunks;
-  const int groups = (chunks + 3) >> 2;
-  u64 final_key = 0;
-  bool bad = false;  // a list is missing (overflow, or the wait below gave up)
-  if (wave < groups) {
-    const int c0 = wave * 4;
-    // lane's four slots, in the orientation wave_merge4 wants them
-    const int cc[4] = {c0, c0 + 1, c0 + 2, c0 + 3};
-    const int ii[4] = {lane, 63 - lane, 63 - lane, lane};
-    u64 got[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (cc[q] >= chunks) got[q] = kSlotEmpty;
-      else if (cc[q] == chunks - 1) got[q] = sm.own[ii[q]];
-      else got[q] = 0;
-    }
-    int spins = 0;
-    while (true) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (got[q] == 0) got[q] = load_coherent(&seg[cc[q] * kSmallCap + ii[q]]);
-      if (__ballot(got[0] == 0 || got[1] == 0 || got[2] == 0 || got[3] == 0) == 0ull) break;
-      if (spins++ >= poll_limit) {
-        if (lane == 0) atomicOr(a.fallback_rows, 0x80000000u);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(2);
-    }
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (cc[q] < chunks - 1 && got[q] != 0) store_coherent(&seg[cc[q] * kSmallCap + ii[q]], 0);  // for the next launch
-      bad = bad || got[q] == 0 || got[q] == kSlotOverflow;
-      if (got[q] <= kSlotOverflow) got[q] = 0;
-    }
-    bad = __ballot(bad) != 0ull;
-    const u64* g4 = got;
-    final_key = wave_merge4([&](int c, int) -> u64 { return g4[c]; }, lane);
-    if (groups > 1) sm.lists[wave * kSmallCap + lane] = final_key;
-    if (bad && lane == 0) sm.count = 1u;  // zeroed by thread 0 before the barriers of the bound
-  }
-  if (groups > 1) {
-    __syncthreads();
-    if (wave == 0) {
-      const u64* l = sm.lists;
-      final_key = wave_merge4([&](int c, int i) -> u64 { return c < groups ? l[c * kSmallCap + i] : 0; }, lane);
-      bad = sm.count != 0u;
-    }
-  }
-  if (wave == 0) {
-    const u64 kth = read_lane(final_key, kk - 1);
-    const bool enough = !bad && kth != 0;  // otherwise NaNs are needed to fill k: the exact path decides
-    if (lane == 0) sm.flag = enough ? 1u : 0u;
-    if (enough) {
-      if (lane >= kk) final_key = 0;
-      if (emit_topk) {
-        if (lane < kk) {
-          const uint32_t id = key64_index(final_key);
-          a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(id);
-          if (emit_topk == 1)
-            a.out_scores[static_cast<size_t>(row) * prm.k + lane] =
-                a.logits[static_cast<size_t>(row) * a.row_stride + id];  // keys do not tell -0 from +0
-        }
-      } else {
-        {
-          RowOutputs out = outputs;  // pointers to this row's slots
-          out.kept_count = out.kept_count ? out.kept_count + row : nullptr;
-          out.kept_ids = out.kept_ids ? out.kept_ids + static_cast<size_t>(row) * out.kept_capacity : nullptr;
-          out.kept_probs = out.kept_probs ? out.kept_probs + static_cast<size_t>(row) * out.kept_capacity : nullptr;
-          wave_topk_epilogue(final_key, kk, prm, u, tab, out);
-        }
-      }
-    }
-  }
-  __syncthreads();
-  return sm.flag == 0u;
-}
-
-// Rows in nucleus mode and all other rows are streamed by kernels of their own (a launch may need
-// both): each kernel holds the code of its mode only, and a change to one path leaves the machine
-// code of the other as it was.
-template <bool INLINE, bool NUCLEUS, bool XFORM, bool LARGEK = false>
-__device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
-  const int row = blockIdx.y, chunk = blockIdx.x;
-  __shared__ FusedShared sm;
-  const mi355x_sample_params prm = row_params<INLINE>(a, row);
-  const int mode = row_mode(prm, a.vocab, a.chunks, a.emit_topk);
-  if constexpr (NUCLEUS) {
-    if (mode == (LARGEK ? kModeTopkLarge : kModeNucleus)) stream_row<true, XFORM, LARGEK>(a, row, chunk, prm, sm);
-  } else {
-    if (mode == kModeNucleus || mode == kModeTopkLarge) return;
-    if (mode == kModeGeneral) {
-      if (chunk != 0) return;
-    } else if (!stream_row<false, XFORM>(a, row, chunk, prm, sm)) {
-      return;
-    }
-    // Rows the fast paths decline end here, in the exact general path (a single inlined call site keeps
-    // the argument block in scalar registers instead of a scratch copy).
-    __syncthreads();
-    general_row(a, row, prm, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq);
-  }
-}
-
-// Kernel variants: per-row parameter table in the arguments or not (_rows); nucleus rows, top-k rows with
-// 64 < k <= kLargeKMax (largek) or all other rows; with or without the code of the logits processing (_xf).
-#define MS_STREAM_KERNEL(NAME, NUCLEUS, XFORM, LARGEK)                                                              \
-  __global__ __launch_bounds__(NUCLEUS ? kNucleusBlock : kTopkBlock) void NAME##_kernel(const SampleArgs a) {      \
-    sample_fused_body<false, NUCLEUS, XFORM, LARGEK>(a);                                                            \
-  }                                                                                                                 \
-  __global__ __launch_bounds__(NUCLEUS ? kNucleusBlock : kTopkBlock) void NAME##_rows_kernel(const SampleArgs a,   \
-                                                                                            const InlineParams) { \
-    sample_fused_body<true, NUCLEUS, XFORM, LARGEK>(a);                                                             \
-  }
-MS_STREAM_KERNEL(sample_fused, false, false, false)
-MS_STREAM_KERNEL(sample_fused_xf, false, true, false)
-MS_STREAM_KERNEL(nucleus_stream, true, false, false)
-MS_STREAM_KERNEL(nucleus_stream_xf, true, true, false)
-MS_STREAM_KERNEL(largek_stream, true, false, true)
-MS_STREAM_KERNEL(largek_stream_xf, true, true, true)
-#undef MS_STREAM_KERNEL
 
 // Sorts n keys (kFinishBlock < n <= kNucleusCap) in LDS, descending, by a block of kFinishBlock
 // threads: a counting pass over kSortBuckets buckets that are linear in the score (bucket 0 holds the
@@ -1277,7 +398,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   if (!ok) {
     __syncthreads();
     u64* const tile = lds_keys;
-    general_row(a, row, prm, big_row, seqsh, [=](u64* keys, int n2, int n_real) {
+    general_row<AnyDtype>(a, row, prm, big_row, seqsh, [=](u64* keys, int n2, int n_real) {
       if (n2 >= 2 * kNucleusCap) tiled_sort_desc(keys, n2, tile);
       else block_sort_desc(keys, n2);
     });
@@ -1295,46 +416,30 @@ __global__ __launch_bounds__(kFinishBlock) void largek_finish_rows_kernel(const 
 
 }  // namespace ms
 
+MS_STREAM_KERNELS(, float)  // the fp32 streaming kernels live here, next to the finish kernels
+
 extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_other,
                                        bool any_nucleus, bool any_large_k, hipStream_t stream) {
-  const dim3 grid(a->chunks, a->rows), block(ms::kTopkBlock), nblock(ms::kNucleusBlock);
   const dim3 fgrid(a->rows), fblock(ms::kFinishBlock);
-  const bool xf = a->xf.active();
+  auto launch_stream = a->dtype == MI355X_F16 ? ms_launch_stream_f16 : a->dtype == MI355X_BF16 ? ms_launch_stream_bf16 : ms_launch_stream;
   hipError_t e = hipSuccess;
   if (any_other) {
-    if (table) {
-      if (xf) hipLaunchKernelGGL(ms::sample_fused_xf_rows_kernel, grid, block, 0, stream, *a, *table);
-      else hipLaunchKernelGGL(ms::sample_fused_rows_kernel, grid, block, 0, stream, *a, *table);
-    } else {
-      if (xf) hipLaunchKernelGGL(ms::sample_fused_xf_kernel, grid, block, 0, stream, *a);
-      else hipLaunchKernelGGL(ms::sample_fused_kernel, grid, block, 0, stream, *a);
-    }
-    e = hipGetLastError();
+    e = launch_stream(a, table, 0, stream);
     if (e != hipSuccess) return e;
   }
   if (any_nucleus) {
-    if (table) {
-      if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_rows_kernel, grid, nblock, 0, stream, *a, *table);
-      else hipLaunchKernelGGL(ms::nucleus_stream_rows_kernel, grid, nblock, 0, stream, *a, *table);
-      hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
-    } else {
-      if (xf) hipLaunchKernelGGL(ms::nucleus_stream_xf_kernel, grid, nblock, 0, stream, *a);
-      else hipLaunchKernelGGL(ms::nucleus_stream_kernel, grid, nblock, 0, stream, *a);
-      hipLaunchKernelGGL(ms::nucleus_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
-    }
+    e = launch_stream(a, table, 1, stream);
+    if (e != hipSuccess) return e;
+    if (table) hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
+    else hipLaunchKernelGGL(ms::nucleus_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
   if (any_large_k) {
-    if (table) {
-      if (xf) hipLaunchKernelGGL(ms::largek_stream_xf_rows_kernel, grid, nblock, 0, stream, *a, *table);
-      else hipLaunchKernelGGL(ms::largek_stream_rows_kernel, grid, nblock, 0, stream, *a, *table);
-      hipLaunchKernelGGL(ms::largek_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
-    } else {
-      if (xf) hipLaunchKernelGGL(ms::largek_stream_xf_kernel, grid, nblock, 0, stream, *a);
-      else hipLaunchKernelGGL(ms::largek_stream_kernel, grid, nblock, 0, stream, *a);
-      hipLaunchKernelGGL(ms::largek_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
-    }
+    e = launch_stream(a, table, 2, stream);
+    if (e != hipSuccess) return e;
+    if (table) hipLaunchKernelGGL(ms::largek_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
+    else hipLaunchKernelGGL(ms::largek_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
     e = hipGetLastError();
   }
   return e;

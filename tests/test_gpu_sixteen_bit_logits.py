@@ -1,0 +1,160 @@
+"""fp16 / bf16 logits read directly by the sampling, top-k-scores and argmax entry points: results must equal
+the oracle run on the rows widened with the CPU path's conversions (Logits::Get casts before the search sees
+the scores, src/models/logits.cpp:72-76; FastFloat16ToFloat32 / BFloat16ToFloat32, src/models/utils.cpp:84-109).
+Token ids, kept ids and probability bits are compared exactly."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import make_mask, pkg, say
+
+pytestmark = pytest.mark.gpu
+
+KIND = {torch.float16: 0, torch.bfloat16: 1}
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = pkg().SearchContext(96, 201088)
+    yield c
+    c.close()
+
+
+def bits(a):
+    return np.asarray(a, np.float32).view(np.uint32)
+
+
+def to_bits16(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def widened(orc, t):
+    return orc.cast(to_bits16(t), KIND[t.dtype], np.float32)
+
+
+def check_sample(ctx, orc, x16, u, per_row, xf=None, proc=None, cap=1024):
+    rows = x16.shape[0]
+    tok, kc, ki, kp = ctx.sample(x16, torch.from_numpy(u).cuda(), per_row=per_row, xf=xf, kept_capacity=cap)
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    wide = widened(orc, x16) if proc is None else proc
+    for r in range(rows):
+        k, p, t = per_row[r]
+        idx, probs = orc.sampled_categorical(wide[r], k, p, t)
+        n = min(len(idx), cap)
+        assert kc[r] == len(idx), (r, per_row[r], kc[r], len(idx))
+        assert np.array_equal(ki[r, :n], idx[:n]), (r, per_row[r])
+        assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), (r, per_row[r])
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (r, per_row[r])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,vocab", [(64, 128256), (5, 40000 + 13), (3, 33000), (4, 70), (2, 201088)])
+def test_sample_reads_sixteen_bit_rows(ctx, orc, dtype, rows, vocab):
+    """Every selection mode on fp16 / bf16 rows, aligned and unaligned row starts, short last chunks."""
+    say("sample 16-bit", dtype, rows, vocab)
+    g = torch.Generator(device="cuda").manual_seed(vocab + rows)
+    x = (torch.randn(rows, vocab, generator=g, device="cuda") * 3).to(dtype)
+    rng = np.random.default_rng(vocab)
+    u = rng.random(rows)
+    menu = [(50, 0.9, 0.7), (1, 0.0, 1.0), (0, 0.9, 1.0), (64, 0.0, 1.3), (100, 0.95, 1.0), (0, 0.5, 0.6), (8, 1.0, 2.0),
+            (600, 0.9, 1.0)]
+    per_row = [menu[(r * 3 + r // 8) % len(menu)] for r in range(rows)]
+    check_sample(ctx, orc, x, u, per_row)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_sixteen_bit_ties_are_broken_by_lowest_id(ctx, orc, dtype):
+    """Sixteen-bit rows are full of equal values: the kept sets must follow score descending, id ascending."""
+    say("sample 16-bit ties", dtype)
+    rows, vocab = 6, 50000
+    g = torch.Generator(device="cuda").manual_seed(4)
+    x = torch.round(torch.randn(rows, vocab, generator=g, device="cuda") * 2).to(dtype)  # a few dozen distinct values
+    u = np.random.default_rng(1).random(rows)
+    check_sample(ctx, orc, x, u, [(50, 0.9, 0.7), (10, 0.0, 1.0), (64, 0.5, 1.0), (2, 0.0, 1.0), (1, 0.0, 1.0), (40, 1.0, 1.0)])
+
+
+def test_every_fp16_pattern_through_the_streaming_loads(ctx, orc):
+    """All 65536 fp16 bit patterns in one row (exponent field 31 decodes as an ordinary exponent, subnormals are
+    exact): the 64 best ids and their widened scores from mi355x_topk_scores equal a sort of the widened row."""
+    say("topk_scores over all fp16 patterns")
+    pat = np.arange(65536, dtype=np.uint16)
+    rng = np.random.default_rng(9)
+    rows = np.stack([pat, rng.permutation(pat), pat[::-1].copy()])
+    x = torch.from_numpy(rows.view(np.int16)).cuda().view(torch.float16)
+    tok, sc = ctx.topk_scores(x, 64)
+    wide = orc.cast(rows, 0, np.float32)
+    for r in range(3):
+        order = np.lexsort((np.arange(65536), -wide[r].astype(np.float64)))[:64]
+        assert np.array_equal(tok[r].cpu().numpy(), order)
+        assert np.array_equal(bits(sc[r].cpu().numpy()), bits(wide[r][order]))
+    assert wide[0].max() == np.float32(131008.0)  # 0x7fff decoded as 65536 * (1 + 1023/1024)
+    # and the sampler keeps exactly the ids whose widened value is largest
+    u = np.array([0.3, 0.6, 0.9])
+    check_sample(ctx, orc, x, u, [(64, 0.0, 30000.0), (20, 0.0, 5000.0), (50, 0.9, 20000.0)])
+
+
+def test_every_bf16_pattern_through_the_streaming_loads(ctx, orc):
+    """All 65536 bf16 patterns, NaNs and infinities included: NaNs order below every number, +inf wins."""
+    say("topk_scores over all bf16 patterns")
+    pat = np.arange(65536, dtype=np.uint16)
+    rows = np.stack([pat, np.random.default_rng(2).permutation(pat)])
+    x = torch.from_numpy(rows.view(np.int16)).cuda().view(torch.bfloat16)
+    tok, sc = ctx.topk_scores(x, 64)
+    wide = orc.cast(rows, 1, np.float32)
+    for r in range(2):
+        key = np.where(np.isnan(wide[r]), -np.inf, wide[r].astype(np.float64))
+        nan_last = np.isnan(wide[r]).astype(np.int64)
+        order = np.lexsort((np.arange(65536), -key, nan_last))[:64]
+        assert np.array_equal(tok[r].cpu().numpy(), order)
+        assert np.array_equal(bits(sc[r].cpu().numpy()), bits(wide[r][order]))
+    assert np.isinf(wide[0][tok[0, 0].item()])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_sixteen_bit_rows_with_logits_processing(ctx, orc, dtype):
+    """Grammar mask, min-length EOS masking and repetition penalty applied to the widened values."""
+    say("sample 16-bit xform", dtype)
+    rows, vocab = 6, 70001
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = (torch.randn(rows, vocab, generator=g, device="cuda") * 3).to(dtype)
+    rng = np.random.default_rng(12)
+    mask = make_mask(rng, rows, vocab, 0.3)
+    hist = rng.integers(0, vocab, (rows, 300)).astype(np.int32)
+    hist[:, 0] = x.float().argmax(dim=1).cpu().numpy()
+    eos = [5, 70000]
+    u = rng.random(rows)
+    xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                           repetition_penalty=1.3, eos_ids=eos, apply_min_length=True)
+    proc = orc.apply_mask(widened(orc, x), mask)
+    for r in range(rows):
+        proc[r, eos] = np.finfo(np.float32).min
+        proc[r] = orc.apply_repetition_penalty(proc[r], hist[r], 1.3)
+    check_sample(ctx, orc, x, u, [(50, 0.9, 0.7), (0, 0.9, 1.0), (1, 0.0, 1.0), (100, 0.0, 1.0), (0, 0.3, 0.5), (64, 0.95, 1.0)],
+                 xf=xf, proc=proc, cap=4096)
+    am = ctx.argmax(x, xf).cpu().numpy()
+    assert np.array_equal(am, orc.argmax_batch(proc))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_argmax_sixteen_bit_rows(ctx, orc, dtype):
+    say("argmax 16-bit", dtype)
+    g = torch.Generator(device="cuda").manual_seed(21)
+    x = (torch.randn(7, 151936, generator=g, device="cuda") * 2).to(dtype)
+    assert np.array_equal(ctx.argmax(x).cpu().numpy(), orc.argmax_batch(widened(orc, x)))
+    y = x[:, 3:100003]  # rows that start off a 16-byte boundary
+    assert np.array_equal(ctx.argmax(y).cpu().numpy(), orc.argmax_batch(widened(orc, y.contiguous())))
+
+
+def test_config2_shape_in_fp16_equals_fp32_on_the_widened_rows(ctx, orc):
+    """Benchmark configuration 2 with fp16 logits: identical tokens to the fp32 entry point fed the widened rows."""
+    say("config2 fp16")
+    rows, vocab = 64, 128256
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn(rows, vocab, generator=g, device="cuda") * 3
+    x.scatter_add_(1, torch.randint(0, vocab, (rows, 8), generator=g, device="cuda"), torch.full((rows, 8), 10.0, device="cuda"))
+    h = x.half()
+    u = torch.rand(rows, generator=g, device="cuda", dtype=torch.float64)
+    a = ctx.sample(h, u, k=50, p=0.9, temperature=0.7)
+    b = ctx.sample(torch.from_numpy(widened(orc, h)).cuda(), u, k=50, p=0.9, temperature=0.7)
+    assert torch.equal(a, b)
+    assert np.array_equal(a.cpu().numpy(), orc.sample_batch(widened(orc, h), 50, 0.9, 0.7, u.cpu().numpy()))
