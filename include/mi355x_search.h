@@ -7,6 +7,13 @@
  * unless stated otherwise.  Return value: 0 on success, a negative MI355X_E_* code on failure, with a
  * thread-local message available from mi355x_search_last_error().
  *
+ * Graph capture: every entry point only launches kernels on `stream`, with workspace from the context, and
+ * can be captured into a HIP graph -- except the synchronous ones (create / destroy, *_is_done,
+ * *_hypothesis, *_fallback_rows, *_wait_gave_up, beam_scorer_set_prompt) and the three that copy a caller's
+ * HOST array with an asynchronous copy (mi355x_sample* with per-row parameters for more than 64 rows,
+ * mi355x_logits_handoff with token_index, mi355x_kv_gather): those return MI355X_E_UNSUPPORTED on a
+ * capturing stream instead of recording a node that would read the caller's array at every replay.
+ *
  * Tie rule everywhere: equal scores are ordered by ascending index (lowest index wins).
  * -0.0 and +0.0 compare equal.  NaN scores order below every number, except in mi355x_argmax, which
  * reproduces the reference's strict '>' scan (a NaN at index 0 is never beaten).
@@ -141,7 +148,8 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
  *   params            used for every row when per_row_params is NULL.
  *   per_row_params    HOST [rows], heterogeneous parameters (copied by the call: up to 64 rows travel
  *                     inside the kernel arguments, larger batches through one asynchronous copy to a
- *                     table in the context).
+ *                     table in the context -- that copy reads the caller's array, so such a call fails
+ *                     with MI355X_E_UNSUPPORTED on a stream that is being captured into a graph).
  *   uniforms          device [rows] doubles in [0,1): row r's categorical draw, the value
  *                     std::discrete_distribution would take from generate_canonical<double,53>.
  *                     A row whose kept set has one token ignores its uniform.
@@ -166,6 +174,17 @@ int mi355x_sample_typed(mi355x_search_ctx* ctx, void* stream, const void* logits
                         mi355x_sample_params params, const mi355x_sample_params* per_row_params,
                         const double* uniforms, int32_t* out_tokens, int32_t* kept_count,
                         int32_t* kept_ids, float* kept_probs, int kept_capacity);
+
+/* mi355x_sample_typed on rows that do not lie at a constant stride: BatchedSampler::Sample receives one span per
+ * request (src/smartptrs.h:134-137; the CUDA sampler packs such rows with a kernel first,
+ * src/cuda/cuda_sampling.cu:390-449).  row_ptrs: HOST array of `rows` device pointers, one per row of `vocab`
+ * elements; they travel inside the kernel arguments (64 rows per launch), so nothing is packed or copied and
+ * the call can be captured into a graph.  Row r of mask / history / uniforms / outputs belongs to row_ptrs[r]. */
+int mi355x_sample_scattered(mi355x_search_ctx* ctx, void* stream, const void* const* row_ptrs, int dtype,
+                            int rows, int vocab, const mi355x_logits_xform* xf,
+                            mi355x_sample_params params, const mi355x_sample_params* per_row_params,
+                            const double* uniforms, int32_t* out_tokens, int32_t* kept_count,
+                            int32_t* kept_ids, float* kept_probs, int kept_capacity);
 
 /* Softmax / log-softmax with temperature, in place, one row per `vocab` floats:
  * Softmax and LogSoftMax (src/softmax.h:26-47).  Sums are accumulated in index order in fp32 exactly
@@ -216,7 +235,8 @@ int mi355x_beam_scorer_hypothesis(mi355x_beam_scorer* s, void* stream, int batch
  * for every tensor t and row j, past[t][j] = present[t][beam_indices[j]], blocks of block_bytes
  * bytes (any size; blocks and tensors aligned to 16 bytes move with 128-bit accesses, others with the
  * widest access they are aligned to).  present/past: HOST arrays of n_tensors device pointers (copied by the
- * call); beam_indices: device [rows]. */
+ * call with asynchronous copies that read the caller's arrays: on a stream that is being captured into a
+ * graph the call fails with MI355X_E_UNSUPPORTED); beam_indices: device [rows]. */
 int mi355x_kv_gather(mi355x_search_ctx* ctx, void* stream, const void* const* present,
                      void* const* past, int n_tensors, const int32_t* beam_indices, int rows,
                      size_t block_bytes);
@@ -291,7 +311,8 @@ int mi355x_cast(mi355x_search_ctx* ctx, void* stream, const void* in, int in_dty
 /* Logits hand-off before the path: Logits::Get (src/models/logits.cpp:33-82) copies the logits of each
  * row's last real token out of the model's [rows, seq_len, vocab] output and widens fp16/bf16 to fp32;
  * here both happen in one pass.  raw: device, dtype MI355X_F32 / MI355X_F16 / MI355X_BF16;
- * token_index: HOST [rows] positions inside seq_len (copied by the call), or NULL for seq_len - 1;
+ * token_index: HOST [rows] positions inside seq_len (copied by the call; with it the call cannot be captured
+ * into a graph and fails with MI355X_E_UNSUPPORTED on a capturing stream), or NULL for seq_len - 1;
  * out: device [rows] rows of vocab floats, row r at out + r*out_stride. */
 int mi355x_logits_handoff(mi355x_search_ctx* ctx, void* stream, const void* raw, int dtype, int rows,
                           int seq_len, int vocab, const int32_t* token_index, float* out,

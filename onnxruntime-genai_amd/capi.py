@@ -53,6 +53,8 @@ def load_library():
                                 C.POINTER(SampleParams), vp, vp, vp, vp, vp, i32]
     L.mi355x_sample_typed.argtypes = [vp, vp, vp, i32, i64, i32, i32, C.POINTER(LogitsXformC), SampleParams,
                                       C.POINTER(SampleParams), vp, vp, vp, vp, vp, i32]
+    L.mi355x_sample_scattered.argtypes = [vp, vp, C.POINTER(vp), i32, i32, i32, C.POINTER(LogitsXformC), SampleParams,
+                                          C.POINTER(SampleParams), vp, vp, vp, vp, vp, i32]
     L.mi355x_search_fallback_rows.argtypes = [vp, vp, C.POINTER(C.c_uint)]
     L.mi355x_search_wait_gave_up.argtypes = [vp, vp, C.POINTER(C.c_int)]
     L.mi355x_search_set_poll_limit.argtypes = [vp, C.c_int]
@@ -201,7 +203,16 @@ class SearchContext:
 
     def sample(self, logits, uniforms, k=0, p=0.0, temperature=1.0, per_row=None, xf=None, out=None,
                kept_capacity=0):
-        rows, vocab, stride = self._rows(logits)
+        """logits: a [rows, vocab] tensor, or a list of rows (1-D tensors of one dtype and length, anywhere in
+        device memory), which goes through mi355x_sample_scattered."""
+        scattered = isinstance(logits, (list, tuple))
+        if scattered:
+            row_list, logits = logits, logits[0].unsqueeze(0)
+            assert all(r.is_cuda and r.dim() == 1 and r.stride(0) == 1 and r.dtype == logits.dtype and
+                       r.numel() == logits.shape[1] for r in row_list)
+            rows, vocab, stride = len(row_list), logits.shape[1], logits.shape[1]
+        else:
+            rows, vocab, stride = self._rows(logits)
         assert uniforms.dtype == torch.float64 and uniforms.numel() >= rows
         if out is None:
             out = torch.empty(rows, dtype=torch.int32, device=logits.device)
@@ -216,7 +227,10 @@ class SearchContext:
         args = (stride, rows, vocab, C.byref(xf.c) if xf else None, SampleParams(int(k), float(p), float(temperature)),
                 pr, uniforms.data_ptr(), out.data_ptr(), kc.data_ptr() if kept_capacity else None,
                 ki.data_ptr() if kept_capacity else None, kp.data_ptr() if kept_capacity else None, kept_capacity)
-        if logits.dtype == torch.float32:
+        if scattered:
+            ptrs = (C.c_void_p * rows)(*[r.data_ptr() for r in row_list])
+            self._check(self.L.mi355x_sample_scattered(self.h, _stream(), ptrs, _DTYPE_CODES[logits.dtype], *args[1:]))
+        elif logits.dtype == torch.float32:
             self._check(self.L.mi355x_sample(self.h, _stream(), logits.data_ptr(), *args))
         else:  # fp16 / bf16 rows are read as they are
             self._check(self.L.mi355x_sample_typed(self.h, _stream(), logits.data_ptr(), _DTYPE_CODES[logits.dtype], *args))

@@ -190,7 +190,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->row_arrive, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->row_best, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->big, static_cast<size_t>(max_rows) * c->big_stride, false));
-  ok(c->Alloc(&c->fallback_rows, 1, true));
+  ok(c->Alloc(&c->fallback_rows, 2, true));  // [0] rows finished by the exact path, [1] a wait gave up
   ok(c->Alloc(&c->ban, static_cast<size_t>(max_rows) * ((max_vocab - 1) / 32 + 1), false));
   ok(c->Alloc(&c->params_dev, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->beam_row_scores, static_cast<size_t>(max_rows) * ms::kBeamMaxCand, false));
@@ -294,23 +294,26 @@ int mi355x_sample(mi355x_search_ctx* ctx, void* stream, const float* logits, int
                              uniforms, out_tokens, kept_count, kept_ids, kept_probs, kept_capacity);
 }
 
-int mi355x_sample_typed(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype, int64_t row_stride,
-                        int rows, int vocab, const mi355x_logits_xform* xf, mi355x_sample_params params,
-                        const mi355x_sample_params* per_row_params, const double* uniforms, int32_t* out_tokens,
-                        int32_t* kept_count, int32_t* kept_ids, float* kept_probs, int kept_capacity) {
-  if (int r = CheckRows(ctx, rows, vocab)) return r;
-  if (!logits || !uniforms || !out_tokens) return Fail(MI355X_E_INVALID, "null logits, uniforms or output");
-  if (dtype != MI355X_F32 && dtype != MI355X_F16 && dtype != MI355X_BF16)
-    return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
-  if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
-  if ((kept_ids || kept_probs) && kept_capacity <= 0) return Fail(MI355X_E_INVALID, "kept_capacity must be positive");
-  if (kept_probs && !kept_ids) return Fail(MI355X_E_INVALID, "kept_probs requires kept_ids");
-  hipStream_t s = static_cast<hipStream_t>(stream);
+namespace {
+
+// True while `s` records into a graph: an entry point that reads a caller's HOST array with an asynchronous copy
+// would leave a node that reads that array again at every replay.
+bool Capturing(hipStream_t s) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(s, &status) == hipSuccess && status != hipStreamCaptureStatusNone;
+}
+
+// One launch set of the sampling path.  Rows lie row_stride elements apart from `logits`, or -- row_ptrs not
+// null, at most kInlineParamRows rows -- start at the device pointers row_ptrs[0 .. rows).
+int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const void* const* row_ptrs, int dtype,
+               int64_t row_stride, int rows, int vocab, const mi355x_logits_xform* xf, mi355x_sample_params params,
+               const mi355x_sample_params* per_row_params, const double* uniforms, int32_t* out_tokens,
+               int32_t* kept_count, int32_t* kept_ids, float* kept_probs, int kept_capacity) {
   ms::SampleArgs a{};
   if (int r = MakeXform(ctx, xf, rows, vocab, s, &a.xf)) return r;
   bool any_nucleus = false, any_other = false, any_large_k = false;
   const int chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
-  ms::InlineParams table;
+  ms::InlineParams table{};
   bool use_table = false;
   auto check = [&](const mi355x_sample_params& p) -> int {
     if (!(p.temperature > 0.0f)) return Fail(MI355X_E_INVALID, "temperature must be positive (got %g)", p.temperature);
@@ -326,18 +329,25 @@ int mi355x_sample_typed(mi355x_search_ctx* ctx, void* stream, const void* logits
   if (per_row_params) {
     for (int r = 0; r < rows; ++r)
       if (int rc = check(per_row_params[r])) return rc;
-    if (rows <= ms::kInlineParamRows) {
-      for (int r = 0; r < rows; ++r) table.row[r] = per_row_params[r];
-      use_table = true;
-    } else {
-      HIP_TRY(hipMemcpyAsync(ctx->params_dev, per_row_params, sizeof(mi355x_sample_params) * rows,
-                             hipMemcpyHostToDevice, s));
-      a.per_row = ctx->params_dev;
-    }
   } else {
     if (int rc = check(params)) return rc;
   }
-  a.logits = logits;
+  if (row_ptrs || (per_row_params && rows <= ms::kInlineParamRows)) {
+    for (int r = 0; r < rows; ++r) {
+      table.row[r] = per_row_params ? per_row_params[r] : params;
+      table.row_ptr[r] = row_ptrs ? row_ptrs[r] : nullptr;
+    }
+    use_table = true;
+  } else if (per_row_params) {
+    if (Capturing(s))
+      return Fail(MI355X_E_UNSUPPORTED, "more than %d rows with per-row parameters are copied from the caller's host "
+                  "array and cannot be captured into a graph; call with at most %d rows", ms::kInlineParamRows,
+                  ms::kInlineParamRows);
+    HIP_TRY(hipMemcpyAsync(ctx->params_dev, per_row_params, sizeof(mi355x_sample_params) * rows,
+                           hipMemcpyHostToDevice, s));
+    a.per_row = ctx->params_dev;
+  }
+  a.logits = row_ptrs ? row_ptrs[0] : logits;
   a.dtype = dtype;
   a.row_stride = row_stride;
   a.rows = rows;
@@ -359,6 +369,60 @@ int mi355x_sample_typed(mi355x_search_ctx* ctx, void* stream, const void* logits
   a.fallback_rows = ctx->fallback_rows;
   a.poll_limit = ctx->poll_limit;
   HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_other, any_nucleus, any_large_k, s));
+  return MI355X_OK;
+}
+
+int CheckSampleArgs(int dtype, const double* uniforms, const int32_t* out_tokens, const int32_t* kept_ids,
+                    const float* kept_probs, int kept_capacity) {
+  if (!uniforms || !out_tokens) return Fail(MI355X_E_INVALID, "null logits, uniforms or output");
+  if (dtype != MI355X_F32 && dtype != MI355X_F16 && dtype != MI355X_BF16)
+    return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
+  if ((kept_ids || kept_probs) && kept_capacity <= 0) return Fail(MI355X_E_INVALID, "kept_capacity must be positive");
+  if (kept_probs && !kept_ids) return Fail(MI355X_E_INVALID, "kept_probs requires kept_ids");
+  return MI355X_OK;
+}
+
+}  // namespace
+
+int mi355x_sample_typed(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype, int64_t row_stride,
+                        int rows, int vocab, const mi355x_logits_xform* xf, mi355x_sample_params params,
+                        const mi355x_sample_params* per_row_params, const double* uniforms, int32_t* out_tokens,
+                        int32_t* kept_count, int32_t* kept_ids, float* kept_probs, int kept_capacity) {
+  if (int r = CheckRows(ctx, rows, vocab)) return r;
+  if (!logits) return Fail(MI355X_E_INVALID, "null logits, uniforms or output");
+  if (int r = CheckSampleArgs(dtype, uniforms, out_tokens, kept_ids, kept_probs, kept_capacity)) return r;
+  if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
+  return SampleImpl(ctx, static_cast<hipStream_t>(stream), logits, nullptr, dtype, row_stride, rows, vocab, xf, params,
+                    per_row_params, uniforms, out_tokens, kept_count, kept_ids, kept_probs, kept_capacity);
+}
+
+int mi355x_sample_scattered(mi355x_search_ctx* ctx, void* stream, const void* const* row_ptrs, int dtype, int rows,
+                            int vocab, const mi355x_logits_xform* xf, mi355x_sample_params params,
+                            const mi355x_sample_params* per_row_params, const double* uniforms, int32_t* out_tokens,
+                            int32_t* kept_count, int32_t* kept_ids, float* kept_probs, int kept_capacity) {
+  if (int r = CheckRows(ctx, rows, vocab)) return r;
+  if (!row_ptrs) return Fail(MI355X_E_INVALID, "null row pointer array");
+  for (int r = 0; r < rows; ++r)
+    if (!row_ptrs[r]) return Fail(MI355X_E_INVALID, "row %d has a null pointer", r);
+  if (int r = CheckSampleArgs(dtype, uniforms, out_tokens, kept_ids, kept_probs, kept_capacity)) return r;
+  const int words = (vocab - 1) / 32 + 1;
+  // the row pointers travel inside the kernel arguments, kInlineParamRows rows per launch
+  for (int r0 = 0; r0 < rows; r0 += ms::kInlineParamRows) {
+    const int n = rows - r0 < ms::kInlineParamRows ? rows - r0 : ms::kInlineParamRows;
+    mi355x_logits_xform part;
+    if (xf) {
+      part = *xf;
+      if (part.mask) part.mask += static_cast<size_t>(r0) * words;
+      if (part.history) part.history += static_cast<size_t>(r0) * part.history_stride;
+      if (part.history_lens) part.history_lens += r0;
+    }
+    if (int rc = SampleImpl(ctx, static_cast<hipStream_t>(stream), nullptr, row_ptrs + r0, dtype, vocab, n, vocab,
+                            xf ? &part : nullptr, params, per_row_params ? per_row_params + r0 : nullptr, uniforms + r0,
+                            out_tokens + r0, kept_count ? kept_count + r0 : nullptr,
+                            kept_ids ? kept_ids + static_cast<size_t>(r0) * kept_capacity : nullptr,
+                            kept_probs ? kept_probs + static_cast<size_t>(r0) * kept_capacity : nullptr, kept_capacity))
+      return rc;
+  }
   return MI355X_OK;
 }
 
@@ -571,6 +635,8 @@ int mi355x_logits_handoff(mi355x_search_ctx* ctx, void* stream, const void* raw,
     for (int r = 0; r < rows; ++r)
       if (token_index[r] < 0 || token_index[r] >= seq_len)
         return Fail(MI355X_E_INVALID, "token_index[%d] = %d outside [0, %d)", r, token_index[r], seq_len);
+    if (Capturing(s))
+      return Fail(MI355X_E_UNSUPPORTED, "token_index is copied from the caller's host array: not capturable into a graph");
     HIP_TRY(hipMemcpyAsync(ctx->row_index, token_index, sizeof(int32_t) * rows, hipMemcpyHostToDevice, s));
     index_dev = ctx->row_index;
   }
@@ -593,6 +659,8 @@ int mi355x_kv_gather(mi355x_search_ctx* ctx, void* stream, const void* const* pr
   int width = 16;
   while (align & static_cast<uintptr_t>(width - 1)) width >>= 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (Capturing(s))
+    return Fail(MI355X_E_UNSUPPORTED, "the tensor pointer tables are copied from the caller's host arrays: not capturable into a graph");
   HIP_TRY(hipMemcpyAsync(ctx->ptr_table, present, sizeof(void*) * n_tensors, hipMemcpyHostToDevice, s));
   HIP_TRY(hipMemcpyAsync(ctx->ptr_table + n_tensors, past, sizeof(void*) * n_tensors, hipMemcpyHostToDevice, s));
   HIP_TRY(ms_launch_kv_gather(ctx->ptr_table, ctx->ptr_table + n_tensors, n_tensors, beam_indices, rows, block_bytes, width, s));
@@ -615,17 +683,16 @@ int mi355x_search_fallback_rows(mi355x_search_ctx* ctx, void* stream, unsigned* 
   HIP_TRY(hipMemcpyAsync(rows, ctx->fallback_rows, sizeof(unsigned), hipMemcpyDeviceToHost,
                          static_cast<hipStream_t>(stream)));
   HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
-  *rows &= 0x7fffffffu;  // bit 31 is the flag mi355x_search_wait_gave_up reports
   return MI355X_OK;
 }
 
 int mi355x_search_wait_gave_up(mi355x_search_ctx* ctx, void* stream, int* gave_up) {
   if (!ctx || !gave_up) return Fail(MI355X_E_INVALID, "null argument");
   unsigned word = 0;
-  HIP_TRY(hipMemcpyAsync(&word, ctx->fallback_rows, sizeof(unsigned), hipMemcpyDeviceToHost,
+  HIP_TRY(hipMemcpyAsync(&word, ctx->fallback_rows + 1, sizeof(unsigned), hipMemcpyDeviceToHost,
                          static_cast<hipStream_t>(stream)));
   HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
-  *gave_up = static_cast<int>(word >> 31);
+  *gave_up = word != 0u;
   return MI355X_OK;
 }
 

@@ -38,6 +38,7 @@ constexpr int kLargeKMax = 512;
 constexpr int kInlineParamRows = 64;
 struct InlineParams {
   mi355x_sample_params row[kInlineParamRows];
+  const void* row_ptr[kInlineParamRows];  // where each row starts, for rows scattered over memory; null: row_stride apart
 };
 
 struct SampleArgs {
@@ -61,7 +62,7 @@ struct SampleArgs {
   u64* chunk_next;        // [rows][chunks]
   u64* big;               // [rows][big_stride]
   size_t big_stride;
-  uint32_t* fallback_rows;  // cumulative count of rows finished by the general path; bit 31: a wait gave up
+  uint32_t* fallback_rows;  // [0] cumulative count (modulo 2^32) of rows finished by the general path; [1] non-zero once a wait gave up
   int poll_limit;           // polls a finishing workgroup waits for another workgroup's list
   int emit_topk;            // 1: write the k best (id, raw score) per row instead of sampling; 2 (kEmitArgmax): the
                             // best id only, k = 1, with ArgMax's rule that a NaN at id 0 wins (src/search.h:9-29)

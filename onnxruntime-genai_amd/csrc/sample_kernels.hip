@@ -398,7 +398,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   if (!ok) {
     __syncthreads();
     u64* const tile = lds_keys;
-    general_row<AnyDtype>(a, row, prm, big_row, seqsh, [=](u64* keys, int n2, int n_real) {
+    general_row<AnyDtype>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, big_row, seqsh, [=](u64* keys, int n2, int n_real) {
       if (n2 >= 2 * kNucleusCap) tiled_sort_desc(keys, n2, tile);
       else block_sort_desc(keys, n2);
     });

@@ -72,23 +72,40 @@ struct AnyDtype {};
 template <typename InT>
 struct RowPtr {
   const InT* p;
-  __device__ __forceinline__ RowPtr(const SampleArgs& a, int row)
-      : p(static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride) {}
+  __device__ __forceinline__ RowPtr(const void* row0, int) : p(static_cast<const InT*>(row0)) {}
   __device__ __forceinline__ float operator[](int i) const { return load_one<InT>(p, i); }
 };
 template <>
 struct RowPtr<AnyDtype> {
-  const void* base;
-  size_t first;
+  const void* p;
   int dtype;
-  __device__ __forceinline__ RowPtr(const SampleArgs& a, int row)
-      : base(a.logits), first(static_cast<size_t>(row) * a.row_stride), dtype(a.dtype) {}
+  __device__ __forceinline__ RowPtr(const void* row0, int dtype_code) : p(row0), dtype(dtype_code) {}
   __device__ __forceinline__ float operator[](int i) const {
-    if (dtype == MI355X_F16) return half_bits_to_float(static_cast<const uint16_t*>(base)[first + i]);
-    if (dtype == MI355X_BF16) return bf16_bits_to_float(static_cast<const uint16_t*>(base)[first + i]);
-    return static_cast<const float*>(base)[first + i];
+    if (dtype == MI355X_F16) return half_bits_to_float(static_cast<const uint16_t*>(p)[i]);
+    if (dtype == MI355X_BF16) return bf16_bits_to_float(static_cast<const uint16_t*>(p)[i]);
+    return static_cast<const float*>(p)[i];
   }
 };
+
+// First element of row `row`.  Rows normally lie row_stride elements apart; the kernels that carry a table in
+// their arguments (INLINE) also take rows scattered over memory, one pointer per row in that table (null: not used).
+template <bool INLINE>
+__device__ __forceinline__ const void* row_start(const SampleArgs& a, int row, size_t elem_bytes) {
+  if constexpr (INLINE) {
+    typedef __attribute__((address_space(4))) const char* KernargPtr;
+    const KernargPtr base = (KernargPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    typedef __attribute__((address_space(4))) const unsigned long long* TablePtr;
+    const TablePtr table = (TablePtr)(base + sizeof(SampleArgs) + offsetof(InlineParams, row_ptr));
+    const unsigned long long ptr = table[row];
+    if (ptr != 0ull) {
+      const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(ptr));
+      const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(ptr >> 32));
+      return reinterpret_cast<const void*>((static_cast<unsigned long long>(hi) << 32) | lo);
+    }
+  }
+  return static_cast<const char*>(a.logits) + static_cast<size_t>(row) * a.row_stride * elem_bytes;
+}
+__device__ __forceinline__ size_t dtype_bytes(int dtype) { return (dtype == MI355X_F16 || dtype == MI355X_BF16) ? 2 : 4; }
 
 // Exact general path for one row, any (k, p, T), any vocabulary size: rebuilds the processed row as
 // key64s in global scratch, sorts all of it, then runs the reference algorithm on the sorted row.
@@ -98,10 +115,10 @@ struct SortInGlobalMemory {
 };
 
 template <typename InT, typename SortFn = SortInGlobalMemory>
-__device__ __forceinline__ void general_row(const SampleArgs& a, int row, const mi355x_sample_params prm, u64* scratch, SeqShared& sh,
-                                            SortFn sort_desc = SortFn{}) {
+__device__ __forceinline__ void general_row(const SampleArgs& a, int row, const void* row0, const mi355x_sample_params prm,
+                                            u64* scratch, SeqShared& sh, SortFn sort_desc = SortFn{}) {
   const int V = a.vocab;
-  const RowPtr<InT> lrow(a, row);
+  const RowPtr<InT> lrow(row0, a.dtype);
   const int n2 = next_pow2(V);
   const bool has_mask = a.xf.mask != nullptr;
   const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
@@ -392,8 +409,8 @@ __device__ __forceinline__ void mask_registers(float (&v)[kSChunk / kSBlock], co
 // Streaming pass of one (row, chunk) of a top-k<=64 or nucleus row.  Returns true when this workgroup
 // must run the general path for the row (it was the last to arrive and the fast path declined).
 template <typename InT, bool NUCLEUS, bool XFORM, bool LARGEK = false>
-__device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chunk, mi355x_sample_params prm,
-                                           FusedShared& sm) {
+__device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const void* row0, int chunk,
+                                           mi355x_sample_params prm, FusedShared& sm) {
   constexpr int kSBlock = NUCLEUS ? kNucleusBlock : kTopkBlock;  // threads of this workgroup
   constexpr int kSWaves = kSBlock / 64;
   constexpr int kSVec = kSChunk / (kSBlock * 4);  // quads of logits per thread (fp32 rows: its 128-bit loads)
@@ -403,10 +420,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
   const int V = a.vocab;
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
-  const InT* lrow = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
+  const InT* lrow = static_cast<const InT*>(row0);
   const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
   const float kNaN = __uint_as_float(0x7fc00000u);  // marks ids >= vocab: never a maximum, never >= a bound
-  const uint32_t poison = *a.fallback_rows;  // needed after the streaming pass only
+  const uint32_t poison = a.fallback_rows[1];  // needed after the streaming pass only
   float v[kSElems];
   if constexpr (VEC == 4) {
 #pragma unroll
@@ -681,8 +698,8 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
 
   // ---- top-k, k <= 64 ---------------------------------------------------------------------------
   // A finishing workgroup that once gave up waiting may have left published lists behind; from then on
-  // (bit 31 of the fallback counter) every row takes the exact path, which reads no such state.
-  if (poison >> 31) return chunk == n_chunks - 1;
+  // (the flag word next to the fallback counter) every row takes the exact path, which reads no such state.
+  if (poison != 0u) return chunk == n_chunks - 1;
   const int kk = prm.k < V ? prm.k : V;
   int n_valid = V - chunk * kSChunk;
   if (n_valid > kSChunk) n_valid = kSChunk;
@@ -853,7 +870,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
         if (got[q] == 0) got[q] = load_coherent(&seg[cc[q] * kSmallCap + ii[q]]);
       if (__ballot(got[0] == 0 || got[1] == 0 || got[2] == 0 || got[3] == 0) == 0ull) break;
       if (spins++ >= poll_limit) {
-        if (lane == 0) atomicOr(a.fallback_rows, 0x80000000u);
+        if (lane == 0) atomicOr(a.fallback_rows + 1, 1u);
         break;
       }
       __builtin_amdgcn_s_sleep(2);
@@ -889,7 +906,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, int chu
           const uint32_t id = key64_index(final_key);
           a.out_tokens[static_cast<size_t>(row) * prm.k + lane] = static_cast<int32_t>(id);
           if (emit_topk == 1)
-            a.out_scores[static_cast<size_t>(row) * prm.k + lane] = RowPtr<InT>(a, row)[id];  // keys do not tell -0 from +0
+            a.out_scores[static_cast<size_t>(row) * prm.k + lane] = RowPtr<InT>(row0, 0)[id];  // keys do not tell -0 from +0
         }
       } else {
         {
@@ -914,20 +931,21 @@ __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
   const int row = blockIdx.y, chunk = blockIdx.x;
   __shared__ FusedShared sm;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
+  const void* const row0 = row_start<INLINE>(a, row, sizeof(InT));
   const int mode = row_mode(prm, a.vocab, a.chunks, a.emit_topk);
   if constexpr (NUCLEUS) {
-    if (mode == (LARGEK ? kModeTopkLarge : kModeNucleus)) stream_row<InT, true, XFORM, LARGEK>(a, row, chunk, prm, sm);
+    if (mode == (LARGEK ? kModeTopkLarge : kModeNucleus)) stream_row<InT, true, XFORM, LARGEK>(a, row, row0, chunk, prm, sm);
   } else {
     if (mode == kModeNucleus || mode == kModeTopkLarge) return;
     if (mode == kModeGeneral) {
       if (chunk != 0) return;
-    } else if (!stream_row<InT, false, XFORM>(a, row, chunk, prm, sm)) {
+    } else if (!stream_row<InT, false, XFORM>(a, row, row0, chunk, prm, sm)) {
       return;
     }
     // Rows the fast paths decline end here, in the exact general path (a single inlined call site keeps
     // the argument block in scalar registers instead of a scratch copy).
     __syncthreads();
-    general_row<InT>(a, row, prm, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq);
+    general_row<InT>(a, row, row0, prm, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq);
   }
 }
 

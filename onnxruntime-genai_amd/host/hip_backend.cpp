@@ -111,12 +111,18 @@ struct HipSamplerState final : BatchedSamplerState {
 // BatchedSampler (src/smartptrs.h:121-138): one fused launch for all rows, heterogeneous (k, p, T),
 // a private random stream per request, transactions by counter snapshot.
 struct HipBatchedSampler final : BatchedSampler {
-  HipBatchedSampler(DeviceInterface& device, size_t max_batch, int vocab) : device_{device}, max_batch_{max_batch}, vocab_{vocab} {
+  HipBatchedSampler(DeviceInterface& device, size_t max_batch, int vocab) : max_batch_{max_batch}, vocab_{vocab} {
     AbiCheck(mi355x_search_create(0, static_cast<int>(max_batch), vocab, &ctx_));
     tokens_ = device.Allocate<int32_t>(max_batch);
-    uniforms_ = device.Allocate<double>(max_batch);
+    for (int i = 0; i < 2; ++i) {
+      uniforms_[i] = device.Allocate<double>(max_batch);
+      HIP_CHECK(hipEventCreateWithFlags(&copied_[i], hipEventDisableTiming));
+    }
   }
-  ~HipBatchedSampler() override { mi355x_search_destroy(ctx_); }
+  ~HipBatchedSampler() override {
+    for (hipEvent_t e : copied_) (void)hipEventDestroy(e);
+    mi355x_search_destroy(ctx_);
+  }
 
   std::unique_ptr<BatchedSamplerState> CreateState(int random_seed) override {
     auto s = std::make_unique<HipSamplerState>();
@@ -149,7 +155,7 @@ struct HipBatchedSampler final : BatchedSampler {
     if (rows == 0 || rows > max_batch_ || params.size() != rows || states.size() != rows)
       throw std::runtime_error("Batched sampler: row, parameter and state counts must match and fit the batch.");
     if (vocab_size != vocab_) throw std::runtime_error("Batched sampler: vocabulary size differs from the one it was created for.");
-    // rows at a constant stride are sampled in place; anything else is packed first
+    // rows at a constant stride are sampled in place; anything else goes by row pointers
     const float* base = scores[0].Span().data();
     ptrdiff_t stride = rows > 1 ? scores[1].Span().data() - base : vocab_size;
     bool strided = stride >= vocab_size;
@@ -157,24 +163,31 @@ struct HipBatchedSampler final : BatchedSampler {
       if (scores[r].size() != static_cast<size_t>(vocab_size)) throw std::runtime_error("Batched sampler: a row is not vocab_size long.");
       strided = scores[r].Span().data() == base + static_cast<ptrdiff_t>(r) * stride;
     }
-    if (!strided) {
-      if (packed_.empty()) packed_ = device_.Allocate<float>(max_batch_ * static_cast<size_t>(vocab_));
-      for (size_t r = 0; r < rows; ++r)
-        HIP_CHECK(hipMemcpyAsync(packed_.Span().data() + r * vocab_, scores[r].Span().data(), sizeof(float) * vocab_,
-                                 hipMemcpyDeviceToDevice, g_stream));
-      base = packed_.Span().data();
-      stride = vocab_;
-    }
     std::vector<mi355x_sample_params> prm(rows);
-    auto u = uniforms_.CpuSpan();
+    // two uniform buffers take turns: the host mirror about to be rewritten is the one whose copy to the device
+    // was issued two calls ago, and its event says when that copy has read it
+    const int slot = turn_;
+    turn_ ^= 1;
+    HIP_CHECK(hipEventSynchronize(copied_[slot]));
+    auto u = uniforms_[slot].CpuSpan();
     for (size_t r = 0; r < rows; ++r) {
       prm[r] = mi355x_sample_params{params[r].k, params[r].p, params[r].temperature};
       auto* s = Own(states[r]);
       u[r] = PhiloxUniform(s->seed, s->counter++);
     }
-    uniforms_.CopyCpuToDevice();
-    AbiCheck(mi355x_sample(ctx_, g_stream, base, stride, static_cast<int>(rows), vocab_, nullptr, prm[0], prm.data(),
-                           uniforms_.Span().data(), tokens_.Span().data(), nullptr, nullptr, nullptr, 0));
+    uniforms_[slot].CopyCpuToDevice();
+    HIP_CHECK(hipEventRecord(copied_[slot], g_stream));
+    if (strided) {
+      AbiCheck(mi355x_sample(ctx_, g_stream, base, stride, static_cast<int>(rows), vocab_, nullptr, prm[0], prm.data(),
+                             uniforms_[slot].Span().data(), tokens_.Span().data(), nullptr, nullptr, nullptr, 0));
+    } else {
+      // rows scattered over memory: their pointers travel inside the kernel arguments, nothing is packed
+      std::vector<const void*> ptrs(rows);
+      for (size_t r = 0; r < rows; ++r) ptrs[r] = scores[r].Span().data();
+      AbiCheck(mi355x_sample_scattered(ctx_, g_stream, ptrs.data(), MI355X_F32, static_cast<int>(rows), vocab_, nullptr,
+                                       prm[0], prm.data(), uniforms_[slot].Span().data(), tokens_.Span().data(), nullptr,
+                                       nullptr, nullptr, 0));
+    }
     return tokens_.subspan(0, rows);
   }
 
@@ -184,13 +197,13 @@ struct HipBatchedSampler final : BatchedSampler {
     if (!s || s->owner != this) throw std::runtime_error("Batched sampler state belongs to another sampler.");
     return s;
   }
-  DeviceInterface& device_;
   size_t max_batch_;
   int vocab_;
   mi355x_search_ctx* ctx_{};
   DeviceSpan<int32_t> tokens_;
-  DeviceSpan<double> uniforms_;
-  DeviceSpan<float> packed_;
+  DeviceSpan<double> uniforms_[2];
+  hipEvent_t copied_[2]{};
+  int turn_{};
   std::vector<std::pair<HipSamplerState*, uint64_t>> saved_;
 };
 

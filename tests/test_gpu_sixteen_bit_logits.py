@@ -158,3 +158,63 @@ def test_config2_shape_in_fp16_equals_fp32_on_the_widened_rows(ctx, orc):
     b = ctx.sample(torch.from_numpy(widened(orc, h)).cuda(), u, k=50, p=0.9, temperature=0.7)
     assert torch.equal(a, b)
     assert np.array_equal(a.cpu().numpy(), orc.sample_batch(widened(orc, h), 50, 0.9, 0.7, u.cpu().numpy()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_rows_scattered_over_memory(ctx, orc, dtype):
+    """mi355x_sample_scattered: 70 rows (two launches of at most 64) that live in separate allocations, at odd
+    offsets and in reverse order, give what mi355x_sample gives on the same rows packed into one matrix."""
+    say("scattered rows", dtype)
+    rows, vocab = 70, 50001
+    g = torch.Generator(device="cuda").manual_seed(70)
+    backing = [(torch.randn(vocab + 11, generator=g, device="cuda") * 3).to(dtype) for _ in range(rows)]
+    row_list = [backing[rows - 1 - r][(r % 5):(r % 5) + vocab] for r in range(rows)]
+    packed = torch.stack(row_list).contiguous()
+    rng = np.random.default_rng(7)
+    u = torch.from_numpy(rng.random(rows)).cuda()
+    menu = [(50, 0.9, 0.7), (1, 0.0, 1.0), (0, 0.9, 1.0), (100, 0.95, 1.0), (64, 0.0, 1.2)]
+    per_row = [menu[(r * 2 + r // 9) % len(menu)] for r in range(rows)]
+    mask = make_mask(rng, rows, vocab, 0.5)
+    hist = rng.integers(0, vocab, (rows, 40)).astype(np.int32)
+    xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                           repetition_penalty=1.25)
+    for use_xf in (None, xf):
+        a = ctx.sample(row_list, u, per_row=per_row, xf=use_xf, kept_capacity=128)
+        b = ctx.sample(packed, u, per_row=per_row, xf=use_xf, kept_capacity=128)
+        for got, want in zip(a, b):
+            assert torch.equal(got, want)
+    # uniform parameters, no per-row table from the caller
+    assert torch.equal(ctx.sample(row_list, u, k=50, p=0.9, temperature=0.7), ctx.sample(packed, u, k=50, p=0.9, temperature=0.7))
+    if dtype == torch.float32:
+        want = [orc.sample_row(packed[r].cpu().numpy(), *per_row[r], u[r].item()) for r in range(rows)]
+        assert ctx.sample(row_list, u, per_row=per_row).cpu().tolist() == want
+
+
+def test_calls_that_copy_host_arrays_refuse_graph_capture(ctx):
+    """Per-row parameters of more than 64 rows and the KV pointer tables are copied from the caller's host arrays:
+    under stream capture those calls fail with a clear error and record nothing; the 64-row forms are captured."""
+    say("capture refusal")
+    rows, vocab = 70, 4099
+    x = torch.randn(rows, vocab, device="cuda")
+    u = torch.rand(rows, device="cuda", dtype=torch.float64)
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    per_row = [(50, 0.9, 0.7)] * rows
+    present = [torch.randn(4, 64, device="cuda") for _ in range(2)]
+    past = [torch.zeros_like(p) for p in present]
+    idx = torch.tensor([1, 1, 0, 3], dtype=torch.int32, device="cuda")
+    eager = ctx.sample(x[:64], u, per_row=per_row[:64]).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            with pytest.raises(RuntimeError, match="captured"):
+                ctx.sample(x, u, per_row=per_row, out=out)
+            with pytest.raises(RuntimeError, match="not capturable"):
+                ctx.kv_gather(present, past, idx)
+            ctx.sample(x[:64], u, per_row=per_row[:64], out=out[:64])
+        out.zero_()
+        graph.replay()
+        side.synchronize()
+    assert torch.equal(out[:64], eager)
