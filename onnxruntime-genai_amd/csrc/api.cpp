@@ -63,6 +63,7 @@ struct mi355x_search_ctx {
   ms::u64* big{};
   size_t big_stride{};
   uint32_t* fallback_rows{};
+  uint32_t* row_done{};
   int poll_limit{ms::kDefaultPollLimit};
   uint32_t* ban{};  // [max_rows, mask words]: ids banned by the no-repeat-n-gram rule
   mi355x_sample_params* params_dev{};
@@ -190,6 +191,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->row_arrive, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->row_best, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->big, static_cast<size_t>(max_rows) * c->big_stride, false));
+  ok(c->Alloc(&c->row_done, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->fallback_rows, 2, true));  // [0] rows finished by the exact path, [1] a wait gave up
   ok(c->Alloc(&c->ban, static_cast<size_t>(max_rows) * ((max_vocab - 1) / 32 + 1), false));
   ok(c->Alloc(&c->params_dev, static_cast<size_t>(max_rows), false));
@@ -368,6 +370,7 @@ int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const 
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
   a.poll_limit = ctx->poll_limit;
+  a.row_done = ctx->row_done;
   HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_other, any_nucleus, any_large_k, s));
   return MI355X_OK;
 }

@@ -67,6 +67,7 @@ struct SampleArgs {
   int emit_topk;            // 1: write the k best (id, raw score) per row instead of sampling; 2 (kEmitArgmax): the
                             // best id only, k = 1, with ArgMax's rule that a NaN at id 0 wins (src/search.h:9-29)
   float* out_scores;        // [rows, k], emit_topk == 1 only (out_tokens is [rows, k] then)
+  uint32_t* row_done;       // [rows] or null: nucleus rows under a grammar mask that the sparse-mask kernel finished
 };
 
 struct ArgmaxArgs {

@@ -153,6 +153,61 @@ __device__ __forceinline__ void tiled_sort_desc(u64* g, int n2, u64* lds) {
   }
 }
 
+// The tail shared by the finish kernels: lds_keys[0 .. n_c) hold a row's candidates as key64s in any order,
+// best_below (0: none) is the best element of the row that is not among them.  Sorts them together in LDS,
+// caches the exponentials and runs the exact epilogue.  With cut_at_best_below the candidates that rank
+// after best_below are dropped first (they are not a prefix of the row's order).  rmax / thr: order keys of
+// the best and of (a bound below) the lowest candidate, which scale the buckets of the sort.  Returns false
+// when the row needs the exact path (the epilogue found no end of the nucleus among the elements given).
+__device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucket_start, uint32_t n_c, u64 best_below,
+                                                  uint32_t rmax, uint32_t thr, bool cut_at_best_below,
+                                                  mi355x_sample_params prm, int V, double u, const RowOutputs& out,
+                                                  SeqShared& seqsh, uint32_t* red32) {
+  const int tid = threadIdx.x;
+  if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
+  if (best_below != 0) n_c += 1;
+  __syncthreads();
+  bool sorted_done = false;
+  if (n_c > static_cast<uint32_t>(kFinishBlock) && rmax != 0u) {
+    sorted_done = bucket_sort_desc(lds_keys, bucket_start, static_cast<int>(n_c), key_to_float(rmax), key_to_float(thr), red32);
+  }
+  if (!sorted_done) {
+    const int n2 = next_pow2(static_cast<int>(n_c));
+    for (int p = static_cast<int>(n_c) + tid; p < n2; p += blockDim.x) lds_keys[p] = 0;
+    __syncthreads();
+    switch (n2 / kFinishBlock) {
+      case 0:
+      case 1: block_sort_desc(lds_keys, n2); break;
+      case 2: block_sort_desc_regs<2>(lds_keys); break;
+      case 4: block_sort_desc_regs<4>(lds_keys); break;
+      case 8: block_sort_desc_regs<8>(lds_keys); break;
+      default: block_sort_desc_regs<16>(lds_keys); break;
+    }
+  }
+  if (cut_at_best_below && best_below != 0) {
+    // keys are distinct: exactly one thread finds it
+    __shared__ uint32_t cut;
+    for (uint32_t i = tid; i < n_c; i += blockDim.x)
+      if (lds_keys[i] == best_below) cut = i + 1u;
+    __syncthreads();
+    n_c = cut;
+  }
+  // cache exp((s - max)/T) in the score half of every entry
+  const float max_score = key_to_float(key64_okey(lds_keys[0]));
+  __syncthreads();
+  const float inv_temp = 1.0f / prm.temperature;
+  for (uint32_t i = tid; i < n_c; i += blockDim.x) {
+    const u64 k64 = lds_keys[i];
+    const float e = em::expf_exact((key_to_float(key64_okey(k64)) - max_score) * inv_temp);
+    lds_keys[i] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k64 & 0xffffffffull);
+  }
+  __syncthreads();
+  const u64* lk = lds_keys;
+  auto sorted = [=](int i) { return lk[i]; };
+  auto exps = [=](int i) { return __uint_as_float(static_cast<uint32_t>(lk[i] >> 32)); };
+  return block_sample_epilogue<4>(sorted, exps, static_cast<int>(n_c), V, prm, u, out, seqsh);
+}
+
 // Per-row finish of the nucleus path: gathers the candidates the streaming pass left in `big`,
 // sorts them in LDS and runs the exact epilogue.  One block of kFinishBlock threads per row;
 // dynamic LDS: kNucleusCap key64s + the bucket table of the sort.
@@ -169,6 +224,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   const int tid = threadIdx.x;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
   if (row_mode(prm, V, a.chunks) != (LARGEK ? kModeTopkLarge : kModeNucleus)) return;
+  if (!LARGEK && a.xf.mask && a.row_done && a.row_done[row] != 0u) return;  // finished by the sparse-mask kernel
   constexpr bool large_k = LARGEK;  // then every listed element is a candidate and no element after them is needed
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
@@ -359,41 +415,8 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   bool ok = !gave_up && !trim_failed && n_c < kNucleusCap;  // room for the next-best element too
   if (large_k) thr = ~block_max<uint32_t>(~lowest, red32);  // the lowest candidate score: the sort scales its buckets by it
   if (ok) {
-    if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
-    if (best_below != 0) n_c += 1;
-    __syncthreads();
-    bool sorted_done = false;
-    if (n_c > static_cast<uint32_t>(kFinishBlock) && rmax != 0u) {
-      sorted_done = bucket_sort_desc(lds_keys, bucket_start, static_cast<int>(n_c), key_to_float(rmax),
-                                     key_to_float(thr), red32);
-    }
-    if (!sorted_done) {
-      const int n2 = next_pow2(static_cast<int>(n_c));
-      for (int p = static_cast<int>(n_c) + tid; p < n2; p += blockDim.x) lds_keys[p] = 0;
-      __syncthreads();
-      switch (n2 / kFinishBlock) {
-        case 0:
-        case 1: block_sort_desc(lds_keys, n2); break;
-        case 2: block_sort_desc_regs<2>(lds_keys); break;
-        case 4: block_sort_desc_regs<4>(lds_keys); break;
-        case 8: block_sort_desc_regs<8>(lds_keys); break;
-        default: block_sort_desc_regs<16>(lds_keys); break;
-      }
-    }
-    // cache exp((s - max)/T) in the score half of every entry
-    const float max_score = key_to_float(key64_okey(lds_keys[0]));
-    __syncthreads();
-    const float inv_temp = 1.0f / prm.temperature;
-    for (uint32_t i = tid; i < n_c; i += blockDim.x) {
-      const u64 k64 = lds_keys[i];
-      const float e = em::expf_exact((key_to_float(key64_okey(k64)) - max_score) * inv_temp);
-      lds_keys[i] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k64 & 0xffffffffull);
-    }
-    __syncthreads();
-    const u64* lk = lds_keys;
-    auto sorted = [=](int i) { return lk[i]; };
-    auto exps = [=](int i) { return __uint_as_float(static_cast<uint32_t>(lk[i] >> 32)); };
-    ok = block_sample_epilogue<4>(sorted, exps, static_cast<int>(n_c), V, prm, a.uniforms[row], row_outputs(a, row), seqsh);
+    ok = finish_candidates(lds_keys, bucket_start, n_c, best_below, rmax, thr, false, prm, V, a.uniforms[row],
+                           row_outputs(a, row), seqsh, red32);
   }
   if (!ok) {
     __syncthreads();
@@ -414,6 +437,209 @@ __global__ __launch_bounds__(kFinishBlock) void largek_finish_rows_kernel(const 
   nucleus_finish_body<true, true>(a);
 }
 
+// ---- nucleus rows under a sparse grammar mask ------------------------------------------------------------
+// A row whose mask lets through fewer ids than the finish kernels can sort needs none of its masked logits:
+// a masked id is lowest() whatever its logit was.  One workgroup per row enumerates the allowed ids from the
+// mask words, gathers exactly those logits, adds the row's history ids with their processed values (the
+// reference's order: mask, min-length, penalty, n-gram ban), applies the nucleus threshold and finishes the
+// row like the finish kernel does.  The best element outside the candidates is the better of the best listed
+// element below the threshold and the first masked id that is not in the history (every such id scores
+// lowest()).  row_done[row] tells the streaming and finish kernels launched afterwards whether the row is
+// finished (1) or theirs to do (0: the mask lets too many ids through, too many history ids, or the nucleus
+// did not close inside the candidates).
+constexpr int kSparseWords = 16;                              // mask words per thread: vocabularies up to 524288
+constexpr int kSparseIds = kNucleusCap / kFinishBlock;        // gathered ids per thread
+constexpr int kSparseExtras = (kSortBuckets + 1) / 2;         // distinct history ids (they use the bucket table's LDS)
+
+template <typename InT>
+__device__ __forceinline__ void sparse_gather(const void* row0, const uint32_t (&ids)[kSparseIds + 2], float (&x)[kSparseIds + 2]) {
+  const InT* const p = static_cast<const InT*>(row0);
+  InT raw[kSparseIds];
+#pragma unroll
+  for (int u = 0; u < kSparseIds; ++u) raw[u] = p[ids[u] != 0xffffffffu ? ids[u] : 0u];
+#pragma unroll
+  for (int u = 0; u < kSparseIds; ++u) x[u] = load_one<InT>(&raw[u], 0);
+}
+
+template <bool INLINE>
+__device__ __forceinline__ void nucleus_sparse_body(const SampleArgs& a) {
+  extern __shared__ u64 lds_keys[];
+  uint32_t* const bucket_start = reinterpret_cast<uint32_t*>(lds_keys + kNucleusCap);
+  uint32_t* const hist_bits = reinterpret_cast<uint32_t*>(lds_keys);                  // first half: history bitmap of the row
+  uint32_t* const id_list = reinterpret_cast<uint32_t*>(lds_keys + kNucleusCap / 2);  // second half: ids to gather
+  float* const extra_val = reinterpret_cast<float*>(bucket_start);
+  uint32_t* const extra_idx = bucket_start + kSparseExtras;
+  __shared__ SeqShared seqsh;
+  __shared__ uint32_t red32[16];
+  __shared__ u64 red64[16];
+  __shared__ uint32_t sh_total, sh_extra, sh_count;
+  const int row = blockIdx.x, tid = threadIdx.x, lane = lane_id();
+  const int V = a.vocab;
+  const mi355x_sample_params prm = row_params<INLINE>(a, row);
+  if (row_mode(prm, V, a.chunks) != kModeNucleus) return;
+  const int words = (V - 1) / 32 + 1;
+  auto leave = [&](bool done) {
+    if (tid == 0) a.row_done[row] = done ? 1u : 0u;
+  };
+  if (words > kFinishBlock * kSparseWords) return leave(false);
+  const uint32_t* mrow = a.xf.mask + static_cast<size_t>(row) * words;
+  const RowPtr<AnyDtype> lrow(row_start<INLINE>(a, row, dtype_bytes(a.dtype)), a.dtype);
+  const int n_eos = a.xf.eos_count(row);
+  const bool pen = a.xf.use_penalty();
+  // allowed ids of this thread's words: mask bits minus the EOS ids under min-length, nothing past the vocabulary
+  uint32_t w[kSparseWords], valid[kSparseWords];
+#pragma unroll
+  for (int q = 0; q < kSparseWords; ++q) {
+    const int wi = tid + q * kFinishBlock;
+    w[q] = 0u;
+    valid[q] = 0u;
+    if (q * kFinishBlock < words && wi < words) {
+      const int n_real = V - wi * 32;
+      valid[q] = n_real >= 32 ? ~0u : ((1u << n_real) - 1u);
+      uint32_t m = mrow[wi];
+      for (int e = 0; e < n_eos; ++e)
+        if ((a.xf.eos[e] >> 5) == wi) m &= ~(1u << (a.xf.eos[e] & 31));
+      w[q] = m & valid[q];
+    }
+  }
+  if (tid == 0) {
+    sh_total = 0u;
+    sh_extra = 0u;
+    sh_count = 0u;
+  }
+  // history ids: marked in a bitmap of the whole row; whoever marks an id first computes its processed value
+  if (pen) {
+    for (int i = tid; i < words; i += kFinishBlock) hist_bits[i] = 0u;
+    __syncthreads();
+    const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
+    const int hlen = a.xf.hist_len(row);
+    const uint32_t* ban_row = a.xf.ban_row(row, V);
+    for (int j = tid; j < hlen; j += kFinishBlock) {
+      const int tok = h[j];
+      if (tok < 0 || tok >= V) continue;
+      const uint32_t bit = 1u << (tok & 31);
+      if (atomicOr(&hist_bits[tok >> 5], bit) & bit) continue;
+      const uint32_t slot = atomicAdd(&sh_extra, 1u);
+      if (slot < static_cast<uint32_t>(kSparseExtras)) {
+        extra_val[slot] = xform_value(lrow[tok], a.xf.penalty, a.xf.eos, tok, mrow[tok >> 5], true, true, n_eos, ban_row);
+        extra_idx[slot] = static_cast<uint32_t>(tok);
+      }
+    }
+  }
+  __syncthreads();
+  // ids to gather (allowed, not in the history) and the first masked id outside the history
+  uint32_t count = 0u, first_masked = 0xffffffffu;
+#pragma unroll
+  for (int q = 0; q < kSparseWords; ++q) {
+    if (q * kFinishBlock < words) {
+      const int wi = tid + q * kFinishBlock;
+      const uint32_t hb = (pen && wi < words) ? hist_bits[wi] : 0u;
+      const uint32_t masked = ~w[q] & valid[q] & ~hb;
+      w[q] &= ~hb;
+      count += static_cast<uint32_t>(__popc(w[q]));
+      if (masked != 0u) {
+        const uint32_t id = static_cast<uint32_t>(wi) * 32u + static_cast<uint32_t>(__ffs(masked) - 1);
+        first_masked = id < first_masked ? id : first_masked;
+      }
+    }
+  }
+  uint32_t inc = count;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t y = __shfl_up(inc, d, 64);
+    if (lane >= d) inc += y;
+  }
+  uint32_t wave_base = 0u;
+  if (lane == 63) wave_base = atomicAdd(&sh_total, inc);
+  wave_base = __shfl(wave_base, 63, 64);
+  first_masked = ~block_max<uint32_t>(~first_masked, red32);  // its barriers also publish sh_total and sh_extra
+  const uint32_t n_allowed = sh_total, n_extra = sh_extra;
+  if (n_allowed + n_extra + 2u > static_cast<uint32_t>(kNucleusCap) || n_extra > static_cast<uint32_t>(kSparseExtras) ||
+      n_allowed + n_extra == 0u)
+    return leave(false);
+  uint32_t pos = wave_base + inc - count;
+#pragma unroll
+  for (int q = 0; q < kSparseWords; ++q) {
+    if (q * kFinishBlock < words) {
+      uint32_t m = w[q];
+      const uint32_t base_id = static_cast<uint32_t>(tid + q * kFinishBlock) * 32u;
+      while (m != 0u) {
+        id_list[pos++] = base_id + static_cast<uint32_t>(__ffs(m) - 1);
+        m &= m - 1u;
+      }
+    }
+  }
+  __syncthreads();
+  // gather: every load of a thread is requested before the first is used
+  uint32_t ids[kSparseIds + 2];
+  float x[kSparseIds + 2];
+#pragma unroll
+  for (int u = 0; u < kSparseIds; ++u) {
+    const uint32_t i = static_cast<uint32_t>(tid + u * kFinishBlock);
+    ids[u] = i < n_allowed ? id_list[i] : 0xffffffffu;
+  }
+  // (the element type is resolved once, outside the loads, so that they are plain loads issued back to back)
+  if (a.dtype == MI355X_F16) sparse_gather<uint16_t>(lrow.p, ids, x);
+  else if (a.dtype == MI355X_BF16) sparse_gather<bf16_t>(lrow.p, ids, x);
+  else sparse_gather<float>(lrow.p, ids, x);
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const uint32_t i = static_cast<uint32_t>(tid + u * kFinishBlock);
+    ids[kSparseIds + u] = i < n_extra ? extra_idx[i] : 0xffffffffu;
+    x[kSparseIds + u] = i < n_extra ? extra_val[i] : __uint_as_float(0x7fc00000u);
+  }
+  uint32_t kmax = 0u;
+#pragma unroll
+  for (int u = 0; u < kSparseIds + 2; ++u) {
+    const uint32_t k = ids[u] != 0xffffffffu ? order_key(x[u]) : 0u;
+    kmax = k > kmax ? k : kmax;
+  }
+  const uint32_t rmax = block_max<uint32_t>(kmax, red32);  // its barriers end every read of the id list and the extras
+  if (rmax == 0u) return leave(false);
+  const uint32_t thr = order_key(key_to_float(rmax) - nucleus_depth(prm, V));
+  if (thr <= order_key(kLowest)) return leave(false);  // masked ids would be candidates themselves
+  // candidates (at or above the threshold) go to the sort buffer at slots a wave reserves with one atomic per
+  // batch; the best of the others is kept
+  u64 best_below = first_masked != 0xffffffffu ? make_key64(order_key(kLowest), first_masked) : 0;
+#pragma unroll
+  for (int u0 = 0; u0 < kSparseIds + 2; u0 += 6) {
+    u64 hits[6];
+    uint32_t wcnt = 0u;
+#pragma unroll
+    for (int u = u0; u < u0 + 6 && u < kSparseIds + 2; ++u) {
+      const bool have = ids[u] != 0xffffffffu;
+      const uint32_t ok32 = have ? order_key(x[u]) : 0u;
+      const bool cand = have && ok32 >= thr;
+      hits[u - u0] = __ballot(cand);
+      wcnt += static_cast<uint32_t>(__popcll(hits[u - u0]));
+      if (have && !cand) {
+        const u64 k64 = make_key64(ok32, ids[u]);
+        best_below = k64 > best_below ? k64 : best_below;
+      }
+    }
+    uint32_t base = 0u;
+    if (lane == 0 && wcnt != 0u) base = atomicAdd(&sh_count, wcnt);
+    base = __builtin_amdgcn_readfirstlane(base);
+#pragma unroll
+    for (int u = u0; u < u0 + 6 && u < kSparseIds + 2; ++u) {
+      const u64 b = hits[u - u0];
+      const uint32_t p = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), base));
+      if ((b >> lane) & 1ull) lds_keys[p] = make_key64(order_key(x[u]), ids[u]);
+      base += static_cast<uint32_t>(__popcll(b));
+    }
+  }
+  best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
+  const uint32_t n_c = sh_count;
+  const bool ok = finish_candidates(lds_keys, bucket_start, n_c, best_below, rmax, thr, false, prm, V, a.uniforms[row],
+                                    row_outputs(a, row), seqsh, red32);
+  leave(ok);
+}
+
+__global__ __launch_bounds__(kFinishBlock) void nucleus_sparse_kernel(const SampleArgs a) { nucleus_sparse_body<false>(a); }
+__global__ __launch_bounds__(kFinishBlock) void nucleus_sparse_rows_kernel(const SampleArgs a, const InlineParams) {
+  nucleus_sparse_body<true>(a);
+}
+
 }  // namespace ms
 
 MS_STREAM_KERNELS(, float)  // the fp32 streaming kernels live here, next to the finish kernels
@@ -428,6 +654,12 @@ extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::Inline
     if (e != hipSuccess) return e;
   }
   if (any_nucleus) {
+    if (a->xf.mask && a->row_done) {  // rows under a sparse grammar mask are finished here; the next two kernels skip them
+      if (table) hipLaunchKernelGGL(ms::nucleus_sparse_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
+      else hipLaunchKernelGGL(ms::nucleus_sparse_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
+      e = hipGetLastError();
+      if (e != hipSuccess) return e;
+    }
     e = launch_stream(a, table, 1, stream);
     if (e != hipSuccess) return e;
     if (table) hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
@@ -449,7 +681,9 @@ extern "C" hipError_t ms_sample_init() {
   const void* finish[] = {reinterpret_cast<const void*>(ms::nucleus_finish_kernel),
                           reinterpret_cast<const void*>(ms::nucleus_finish_rows_kernel),
                           reinterpret_cast<const void*>(ms::largek_finish_kernel),
-                          reinterpret_cast<const void*>(ms::largek_finish_rows_kernel)};
+                          reinterpret_cast<const void*>(ms::largek_finish_rows_kernel),
+                          reinterpret_cast<const void*>(ms::nucleus_sparse_kernel),
+                          reinterpret_cast<const void*>(ms::nucleus_sparse_rows_kernel)};
   for (const void* f : finish) {
     const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, ms::kFinishLds);
     if (e != hipSuccess) return e;

@@ -934,7 +934,12 @@ __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
   const void* const row0 = row_start<INLINE>(a, row, sizeof(InT));
   const int mode = row_mode(prm, a.vocab, a.chunks, a.emit_topk);
   if constexpr (NUCLEUS) {
-    if (mode == (LARGEK ? kModeTopkLarge : kModeNucleus)) stream_row<InT, true, XFORM, LARGEK>(a, row, row0, chunk, prm, sm);
+    if (mode == (LARGEK ? kModeTopkLarge : kModeNucleus)) {
+      if constexpr (XFORM && !LARGEK) {
+        if (a.xf.mask && a.row_done && a.row_done[row] != 0u) return;  // finished by the sparse-mask kernel
+      }
+      stream_row<InT, true, XFORM, LARGEK>(a, row, row0, chunk, prm, sm);
+    }
   } else {
     if (mode == kModeNucleus || mode == kModeTopkLarge) return;
     if (mode == kModeGeneral) {

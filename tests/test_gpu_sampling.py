@@ -693,3 +693,58 @@ def test_greedy_tail_eos_pad_append(ctx, batch):
     before = d_seq.clone()
     ctx.greedy_tail(torch.zeros(batch, dtype=torch.int32, device="cuda"), d_seen, eos, pad, d_seq, max_length, d_done)
     assert torch.equal(before, d_seq)  # nothing is written beyond max_length
+
+
+@pytest.mark.parametrize("vocab,frac,penalty,p", [
+    (201088, 0.05, 1.2, 0.95),     # the sparse-mask kernel finishes the rows
+    (201088, 0.0005, 1.2, 0.95),   # a hundred allowed ids
+    (201088, 0.079, 0.8, 0.9),     # close to what the sort buffer holds; a penalty below one lifts masked history ids
+    (201088, 0.0816, 1.2, 0.9),    # around the capacity: some rows fit, some are left to the dense kernels
+    (201088, 0.5, 1.2, 0.95),      # dense: every row declined
+    (70001, 0.05, 1.3, 0.999),     # the nucleus takes nearly every allowed id
+    (70001, 0.02, 1.0, 0.3),       # no penalty: no history bitmap
+    (4099, 0.3, 1.1, 0.95),
+])
+def test_nucleus_rows_under_sparse_and_dense_masks(ctx, orc, vocab, frac, penalty, p):
+    """Rows in nucleus mode with a grammar mask of any density, min-length EOS masking, a history with ids that
+    are masked, ids that are allowed, repeats and out-of-range ids; a few allowed logits are -inf, NaN or
+    lowest().  Kept ids, probability bits and tokens equal the oracle's."""
+    say("nucleus under mask", vocab, frac, penalty, p)
+    rng = np.random.default_rng(int(vocab * 1000 + frac * 1e6))
+    rows = 6
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    mask = make_mask(rng, rows, vocab, frac)
+    allowed = np.unpackbits(mask.view(np.uint8), axis=1, bitorder="little")[:, :vocab].astype(bool)
+    for r in range(rows):
+        ids = np.flatnonzero(allowed[r])
+        if len(ids) > 8:  # special values among the allowed logits
+            x[r, ids[1]] = -np.inf
+            x[r, ids[3]] = np.nan if r % 2 else LOWEST
+            x[r, ids[5]] = x[r, ids[6]]  # a tie
+    hist = rng.integers(0, vocab, (rows, 200)).astype(np.int32)
+    hist[:, 7] = hist[:, 3]  # a repeat
+    hist[:, 9] = -1
+    for r in range(rows):
+        ids = np.flatnonzero(allowed[r])
+        hist[r, 0] = ids[0]                      # allowed ids in the history
+        hist[r, 1] = ids[len(ids) // 2]
+        hist[r, 2] = np.flatnonzero(~allowed[r])[0] if (~allowed[r]).any() else 0  # the first masked id is in the history
+    eos = [int(np.flatnonzero(allowed[0])[0]), 2]
+    u = rng.random(rows)
+    xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                           repetition_penalty=penalty, eos_ids=eos, apply_min_length=True)
+    cap = 20000
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=p, temperature=0.9,
+                                 xf=xf, kept_capacity=cap)
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    proc = orc.apply_mask(x, mask)
+    for r in range(rows):
+        row = proc[r].copy()
+        row[eos] = LOWEST
+        row = orc.apply_repetition_penalty(row, hist[r][(hist[r] >= 0)], penalty)
+        idx, probs = orc.sampled_categorical(row, 0, p, 0.9)
+        n = min(len(idx), cap)
+        assert kc[r] == len(idx), (r, kc[r], len(idx))
+        assert np.array_equal(ki[r, :n], idx[:n]), r
+        assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), r
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
