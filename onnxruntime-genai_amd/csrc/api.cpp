@@ -75,6 +75,7 @@ struct mi355x_search_ctx {
   uint32_t* seg_max{};
   double* seg_sum{};
   int4* seg_step{};
+  int4* sub_step{};
   float* row_max{};
   float* row_sum{};
   int32_t* row_index{};  // device copy of per-row host indices (logits hand-off)
@@ -202,6 +203,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->seg_sum, static_cast<size_t>(max_rows) * c->max_segs, false));
   ok(c->Alloc(&c->seg_cand, static_cast<size_t>(max_rows) * c->max_segs * ms::kBeamMaxCand, false));
   ok(c->Alloc(&c->seg_step, static_cast<size_t>(max_rows) * c->max_segs, false));
+  ok(c->Alloc(&c->sub_step, static_cast<size_t>(max_rows) * c->max_segs * ms::kSegSubs, false));
   ok(c->Alloc(&c->row_max, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->row_sum, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->row_index, static_cast<size_t>(max_rows), false));
@@ -480,6 +482,7 @@ static bool FillSeqSum(mi355x_search_ctx* ctx, const void* x, int64_t row_stride
   q->seg_max = ctx->seg_max;
   q->seg_sum = ctx->seg_sum;
   q->seg_step = ctx->seg_step;
+  q->sub_step = ctx->sub_step;
   q->e = reinterpret_cast<float*>(ctx->big);
   q->e_stride = ctx->big_stride * 2;
   q->out_max = ctx->row_max;
@@ -810,9 +813,8 @@ int mi355x_beam_scorer_step(mi355x_beam_scorer* s, void* stream, const float* ca
   if (!s || !cand_scores || !cand_tokens || !cand_beam_indices) return Fail(MI355X_E_INVALID, "null argument");
   if (s->length >= s->st.max_length) return Fail(MI355X_E_INVALID, "sequence already at max_length (%d)", s->st.max_length);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  HIP_TRY(ms_launch_scorer_process(&s->st, s->seq[s->cur], s->length, cand_scores, cand_tokens, cand_beam_indices, st));
-  HIP_TRY(ms_launch_beam_append(s->seq[s->cur], s->seq[1 - s->cur], s->st.batch * s->st.beams, s->st.max_length,
-                                s->length, s->st.next_indices, s->st.next_tokens, st));
+  HIP_TRY(ms_launch_scorer_step(&s->st, s->seq[s->cur], s->seq[1 - s->cur], s->length, cand_scores, cand_tokens,
+                                cand_beam_indices, st));
   s->cur = 1 - s->cur;
   s->length += 1;
   return MI355X_OK;

@@ -203,53 +203,75 @@ __device__ __forceinline__ void scorer_add(const ScorerState& s, int batch, cons
   __builtin_amdgcn_wave_barrier();
 }
 
-__global__ __launch_bounds__(64) void beam_scorer_process_kernel(const ScorerState s, const int32_t* sequences,
-                                                                 int sequence_length, const float* cand_scores,
-                                                                 const int32_t* cand_tokens, const int32_t* cand_indices) {
+// BeamSearchScorer::Process for one batch entry (one wave), then BeamSearch_Cpu::AppendNextTokensToSequences for
+// the entry's rows: lane i keeps the (token, source row) of beam row i, and the wave copies those rows of the
+// current sequences into the next buffer with the token appended.  A done entry's rows copy global row 0, as the
+// reference does with its index 0; nothing read here is written by another entry's wave in the same launch.
+__global__ __launch_bounds__(64) void beam_scorer_step_kernel(const ScorerState s, const int32_t* sequences,
+                                                              int32_t* sequences_next, int sequence_length,
+                                                              const float* cand_scores, const int32_t* cand_tokens,
+                                                              const int32_t* cand_indices) {
   const int batch = blockIdx.x, lane = lane_id();
   const int nb = s.beams, top_k = 2 * nb;
+  int my_tok = s.pad, my_src = 0;  // what a done entry emits
   if (s.done[batch]) {
     if (lane < nb) {
       s.next_scores[batch * nb + lane] = 0.0f;
       s.next_tokens[batch * nb + lane] = s.pad;
       s.next_indices[batch * nb + lane] = 0;
     }
-    return;
-  }
-  int beam_idx = 0;
-  for (int j = 0; j < top_k; ++j) {
-    const int tok = cand_tokens[batch * top_k + j];
-    const float score = cand_scores[batch * top_k + j];
-    const int bbi = batch * nb + cand_indices[batch * top_k + j];
-    if (scorer_is_eos(s, tok)) {
-      if (j >= nb) continue;
-      scorer_add(s, batch, sequences + static_cast<size_t>(bbi) * s.max_length, sequence_length, score);
-    } else {
-      if (lane == 0) {
-        s.next_scores[batch * nb + beam_idx] = score;
-        s.next_tokens[batch * nb + beam_idx] = tok;
-        s.next_indices[batch * nb + beam_idx] = bbi;
-      }
-      ++beam_idx;
+  } else {
+    // a beam row that gets no candidate this step (more EOS candidates than the reference expects) keeps the
+    // token and source row it had, as the reference's arrays do
+    if (lane < nb) {
+      my_tok = s.next_tokens[batch * nb + lane];
+      my_src = s.next_indices[batch * nb + lane];
     }
-    if (beam_idx == nb) break;
+    int beam_idx = 0;
+    for (int j = 0; j < top_k; ++j) {
+      const int tok = cand_tokens[batch * top_k + j];
+      const float score = cand_scores[batch * top_k + j];
+      const int bbi = batch * nb + cand_indices[batch * top_k + j];
+      if (scorer_is_eos(s, tok)) {
+        if (j >= nb) continue;
+        scorer_add(s, batch, sequences + static_cast<size_t>(bbi) * s.max_length, sequence_length, score);
+      } else {
+        if (lane == beam_idx) {
+          my_tok = tok;
+          my_src = bbi;
+          s.next_scores[batch * nb + beam_idx] = score;
+          s.next_tokens[batch * nb + beam_idx] = tok;
+          s.next_indices[batch * nb + beam_idx] = bbi;
+        }
+        ++beam_idx;
+      }
+      if (beam_idx == nb) break;
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (lane == 0 && s.hyp_used[batch] >= nb) {
+      bool can_improve = false;
+      if (!s.early_stopping) {
+        // The reference's window starts at batch*beams rather than batch*2*beams (:161); kept as is.
+        float best = cand_scores[batch * nb];
+        for (int i = 1; i < top_k; ++i) best = fmaxf(best, cand_scores[batch * nb + i]);
+        const float current = best / s.pow_table[sequence_length];
+        can_improve = s.hyp_score[batch * nb + nb - 1] < current;  // CanImprove
+      }
+      if (!can_improve) {
+        s.done[batch] = 1;
+        atomicSub(s.not_done, 1);
+      }
+    }
   }
-  __builtin_amdgcn_wave_barrier();
-  if (lane != 0) return;
-  if (s.hyp_used[batch] < nb) return;
-  if (!s.early_stopping) {
-    // The reference's window starts at batch*beams rather than batch*2*beams (:161); kept as is.
-    float best = cand_scores[batch * nb];
-    for (int i = 1; i < top_k; ++i) best = fmaxf(best, cand_scores[batch * nb + i]);
-    const float current = best / s.pow_table[sequence_length];
-    if (s.hyp_score[batch * nb + nb - 1] < current) return;  // CanImprove
+  for (int i = 0; i < nb; ++i) {
+    const int src_row = __shfl(my_src, i, 64), tok = __shfl(my_tok, i, 64);
+    const int32_t* src = sequences + static_cast<size_t>(src_row) * s.max_length;
+    int32_t* dst = sequences_next + static_cast<size_t>(batch * nb + i) * s.max_length;
+    for (int t = lane; t < sequence_length; t += 64) dst[t] = src[t];
+    if (lane == 0) dst[sequence_length] = tok;
   }
-  s.done[batch] = 1;
-  atomicSub(s.not_done, 1);
 }
 
-// BeamSearchScorer::Finalize (src/beam_search_scorer.cpp:173-196): open batch entries add their
-// current beams as hypotheses.
 __global__ __launch_bounds__(64) void beam_scorer_finalize_kernel(const ScorerState s, const int32_t* sequences,
                                                                   int sequence_length) {
   const int batch = blockIdx.x;
@@ -258,17 +280,6 @@ __global__ __launch_bounds__(64) void beam_scorer_finalize_kernel(const ScorerSt
     const int bbi = batch * s.beams + j;
     scorer_add(s, batch, sequences + static_cast<size_t>(bbi) * s.max_length, sequence_length, s.next_scores[bbi]);
   }
-}
-
-// BeamSearch_Cpu::AppendNextTokensToSequences (src/search.cpp:354-381).
-__global__ __launch_bounds__(256) void beam_append_kernel(const int32_t* seq, int32_t* seq_next, int max_length,
-                                                          int current_length, const int32_t* beam_indices,
-                                                          const int32_t* tokens) {
-  const int i = blockIdx.x;
-  const int32_t* src = seq + static_cast<size_t>(beam_indices[i]) * max_length;
-  int32_t* dst = seq_next + static_cast<size_t>(i) * max_length;
-  for (int t = threadIdx.x; t < current_length; t += blockDim.x) dst[t] = src[t];
-  if (threadIdx.x == 0) dst[current_length] = tokens[i];
 }
 
 
@@ -463,23 +474,16 @@ extern "C" hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hi
   return hipGetLastError();
 }
 
-extern "C" hipError_t ms_launch_scorer_process(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,
-                                               const float* cs, const int32_t* ct, const int32_t* ci, hipStream_t stream) {
-  hipLaunchKernelGGL(ms::beam_scorer_process_kernel, dim3(s->batch), dim3(64), 0, stream, *s, sequences, sequence_length,
-                     cs, ct, ci);
+extern "C" hipError_t ms_launch_scorer_step(const ms::ScorerState* s, const int32_t* sequences, int32_t* sequences_next,
+                                            int sequence_length, const float* cs, const int32_t* ct, const int32_t* ci,
+                                            hipStream_t stream) {
+  hipLaunchKernelGGL(ms::beam_scorer_step_kernel, dim3(s->batch), dim3(64), 0, stream, *s, sequences, sequences_next,
+                     sequence_length, cs, ct, ci);
   return hipGetLastError();
 }
-
 extern "C" hipError_t ms_launch_scorer_finalize(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,
                                                 hipStream_t stream) {
   hipLaunchKernelGGL(ms::beam_scorer_finalize_kernel, dim3(s->batch), dim3(64), 0, stream, *s, sequences, sequence_length);
   return hipGetLastError();
 }
 
-extern "C" hipError_t ms_launch_beam_append(const int32_t* seq, int32_t* seq_next, int rows, int max_length,
-                                            int current_length, const int32_t* beam_indices, const int32_t* tokens,
-                                            hipStream_t stream) {
-  hipLaunchKernelGGL(ms::beam_append_kernel, dim3(rows), dim3(256), 0, stream, seq, seq_next, max_length, current_length,
-                     beam_indices, tokens);
-  return hipGetLastError();
-}

@@ -84,6 +84,7 @@ constexpr int kBeamMaxCand = 32;  // 2 * beams, beams <= 16
 
 // Multi-workgroup exact sequential sum (seqsum_kernels.hip).
 constexpr int kSegElems = 4096;   // elements per segment
+constexpr int kSegSubs = 16;      // parts of a segment with composed steps of their own (256 elements each)
 constexpr int kMaxSegs = 1024;    // segments per row the walk kernel can hold
 constexpr int kSeqSumMinVocab = 16384;  // shorter rows are summed by one workgroup in one launch
 
@@ -94,7 +95,10 @@ struct SeqSumArgs {
   float inv_temp;
   uint32_t* seg_max;  // [rows][segs] order keys
   double* seg_sum;    // [rows][segs]
-  int4* seg_step;     // [rows][segs]: d0, d1, binade (-1: scan the segment), unused
+  int4* seg_step;     // [rows][segs]: d0, d1, binade, unused; binade -1: scan the segment; -2: one power of two may
+                      // fall inside the segment, the sixteen parts of the segment have records in sub_step and
+                      // the last field holds the binade before it
+  int4* sub_step;     // [rows][segs][kSegSubs]: (d0, d1) of a 256-element part under the lower binade, then under the next
   float* e;           // [rows][e_stride] exponentials
   size_t e_stride;
   float* out_max;     // [rows]
@@ -193,11 +197,9 @@ hipError_t ms_launch_beam_finish(const ms::BeamArgs* a, int dtype, hipStream_t s
 hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, int have_seg_max, hipStream_t stream);
 hipError_t ms_launch_softmax_apply(float* scores, int64_t row_stride, const ms::SeqSumArgs* a, int log_softmax,
                                    hipStream_t stream);
-hipError_t ms_launch_scorer_process(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,
-                                    const float* cs, const int32_t* ct, const int32_t* ci, hipStream_t stream);
+hipError_t ms_launch_scorer_step(const ms::ScorerState* s, const int32_t* sequences, int32_t* sequences_next,
+                                 int sequence_length, const float* cs, const int32_t* ct, const int32_t* ci,
+                                 hipStream_t stream);
 hipError_t ms_launch_scorer_finalize(const ms::ScorerState* s, const int32_t* sequences, int sequence_length,
                                      hipStream_t stream);
-hipError_t ms_launch_beam_append(const int32_t* seq, int32_t* seq_next, int rows, int max_length,
-                                 int current_length, const int32_t* beam_indices, const int32_t* tokens,
-                                 hipStream_t stream);
 }

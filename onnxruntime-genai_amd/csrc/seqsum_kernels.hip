@@ -50,19 +50,23 @@ template <typename InT>
 __global__ __launch_bounds__(kSegBlock) void seqsum_exp_kernel(const SeqSumArgs a) {
   __shared__ uint32_t red[4];
   __shared__ double dred[4];
+  __shared__ uint64_t exp_tab[32];  // the table of expf in LDS: a lookup per element from constant memory is a gather
   const int seg = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
   const InT* x = static_cast<const InT*>(a.x) + static_cast<size_t>(row) * a.row_stride;
   const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
   float v[kSegPer];
   seg_load<InT>(x, aligned, a.vocab, seg, 0.0f, v);
-  const float max_score = row_max_of_segments(a, row, red);
+  if (tid < 32) exp_tab[tid] = em::exp2_tab(static_cast<uint32_t>(tid));
+  const float max_score = row_max_of_segments(a, row, red);  // its barriers also publish the table
+  const uint64_t* const tab = exp_tab;
+  auto lds_tab = [=](uint32_t i) { return tab[i]; };
   float* erow = a.e + static_cast<size_t>(row) * a.e_stride;
   double part = 0.0;
 #pragma unroll
   for (int e = 0; e < kSegPer; ++e) {
     const int idx = seg_index<InT>(seg, e);
     if (idx < a.vocab) {
-      const float ex = em::expf_exact((v[e] - max_score) * a.inv_temp);
+      const float ex = em::expf_core((v[e] - max_score) * a.inv_temp, lds_tab);
       erow[idx] = ex;
       part += static_cast<double>(ex);
     }
@@ -98,16 +102,39 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs
   const double lo = before * (1.0 - seq_drift(first));
   const double hi = (before + sums[seg]) * (1.0 + seq_drift(first + n));
   const float lo_f = __double2float_rd(lo), hi_f = __double2float_ru(hi);
-  const int se = seq_decompose(lo_f).se;
+  const int se = seq_decompose(lo_f).se, se_hi = seq_decompose(hi_f).se;
   int4* rec = a.seg_step + static_cast<size_t>(row) * a.segs + seg;
-  const bool known = lo_f > 0.0f && hi_f < 3.0e38f && seq_decompose(hi_f).se == se;
-  if (!known) {  // a power of two may fall inside the segment: the walk scans it
+  const bool in_range = lo_f > 0.0f && hi_f < 3.0e38f;
+  const bool known = in_range && se_hi == se;
+  if (!known && !(in_range && se_hi == se + 1)) {  // several powers of two may fall inside the segment: the walk scans it
     if (tid == 0) *rec = make_int4(0, 0, -1, 0);
     return;
   }
   const float* erow = a.e + static_cast<size_t>(row) * a.e_stride + first;
   float ev[kSegPer];
   window_fetch<kSegPer>(ev, 0, n, [=](int i) { return erow[i]; }, stage);
+  if (!known) {
+    // One power of two may fall inside the segment.  Each of its sixteen 256-element parts (sixteen lanes of
+    // sixteen elements) gets a composed step under the binade before that power and one under the binade after
+    // it: the walk applies the first kind up to the part where the sum leaves the binade, adds that part
+    // element by element, and goes on with the second kind.
+    static_assert(kSegSubs * 16 * kSegPer == kSegElems && kSegBlock == kSegSubs * 16, "a part is sixteen lanes");
+    Step lo_step{0u, 0u}, hi_step{0u, 0u};
+#pragma unroll
+    for (int j = 0; j < kSegPer; ++j) {
+      lo_step = step_compose(lo_step, seq_make_step(ev[j], se));
+      hi_step = step_compose(hi_step, seq_make_step(ev[j], se + 1));
+    }
+    lo_step = row_scan_steps(lo_step);
+    hi_step = row_scan_steps(hi_step);
+    if ((lane & 15) == 15) {
+      int4* sub = a.sub_step + (static_cast<size_t>(row) * a.segs + seg) * kSegSubs;
+      sub[tid >> 4] = make_int4(static_cast<int>(lo_step.d0), static_cast<int>(lo_step.d1), static_cast<int>(hi_step.d0),
+                                static_cast<int>(hi_step.d1));
+    }
+    if (tid == 0) *rec = make_int4(0, 0, -2, se);
+    return;
+  }
   Step agg{0u, 0u};
 #pragma unroll
   for (int j = 0; j < kSegPer; ++j) agg = step_compose(agg, seq_make_step(ev[j], se));
@@ -127,6 +154,7 @@ __global__ __launch_bounds__(kWalkBlock) void seqsum_walk_kernel(const SeqSumArg
   __shared__ SeqShared sh;
   __shared__ uint32_t red[16];
   __shared__ int4 recs[kMaxSegs];
+  __shared__ int4 subs[kSegSubs];
   __shared__ __align__(16) float stage[kSegElems];
   const int row = blockIdx.x, tid = threadIdx.x;
   for (int s = tid; s < a.segs; s += kWalkBlock) recs[s] = a.seg_step[static_cast<size_t>(row) * a.segs + s];
@@ -149,6 +177,32 @@ __global__ __launch_bounds__(kWalkBlock) void seqsum_walk_kernel(const SeqSumArg
     const int n = a.vocab - first < kSegElems ? a.vocab - first : kSegElems;
     const float* e = erow + first;
     int dummy;
+    if (r.z == -2) {
+      // part by part: a part's composed step under the binade the sum is in, or -- where the sum leaves the
+      // binade, or is in neither of the two binades the records were made for -- the part's elements one by one
+      const int4* sub = a.sub_step + (static_cast<size_t>(row) * a.segs + seg) * kSegSubs;
+      __syncthreads();  // the previous segment's readers of subs are done
+      if (tid < kSegSubs) subs[tid] = sub[tid];
+      __syncthreads();
+      constexpr int kPart = kSegElems / kSegSubs;
+      for (int j = 0; j * kPart < n; ++j) {
+        const SeqState st = seq_decompose(s);
+        const int4 q = subs[j];
+        if (st.se == r.w || st.se == r.w + 1) {
+          const Step f = st.se == r.w ? Step{static_cast<uint32_t>(q.x), static_cast<uint32_t>(q.y)}
+                                      : Step{static_cast<uint32_t>(q.z), static_cast<uint32_t>(q.w)};
+          const uint32_t n2 = step_apply(st.n, f);
+          if (n2 < kMantLimit) {
+            s = seq_recompose(n2, st.se);
+            continue;
+          }
+        }
+        const float* ep = e + j * kPart;
+        const int np = n - j * kPart < kPart ? n - j * kPart : kPart;
+        s = block_seq_sum<kPart / kWalkBlock>(s, np, [=](int i) { return ep[i]; }, NoStop{}, &dummy, sh, nullptr, kPart);  // one wave's chain
+      }
+      continue;
+    }
     s = block_seq_sum<kSegElems / kWalkBlock>(s, n, [=](int i) { return e[i]; }, NoStop{}, &dummy, sh, stage,
                                                  seg == 0 ? 1024 : 0);
   }
