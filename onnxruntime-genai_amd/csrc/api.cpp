@@ -76,6 +76,7 @@ struct mi355x_search_ctx {
   double* seg_sum{};
   int4* seg_step{};
   int4* sub_step{};
+  int* sub_se{};
   float* row_max{};
   float* row_sum{};
   int32_t* row_index{};  // device copy of per-row host indices (logits hand-off)
@@ -204,6 +205,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->seg_cand, static_cast<size_t>(max_rows) * c->max_segs * ms::kBeamMaxCand, false));
   ok(c->Alloc(&c->seg_step, static_cast<size_t>(max_rows) * c->max_segs, false));
   ok(c->Alloc(&c->sub_step, static_cast<size_t>(max_rows) * c->max_segs * ms::kSegSubs, false));
+  ok(c->Alloc(&c->sub_se, static_cast<size_t>(max_rows) * c->max_segs * ms::kSegSubs, false));
   ok(c->Alloc(&c->row_max, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->row_sum, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->row_index, static_cast<size_t>(max_rows), false));
@@ -483,6 +485,7 @@ static bool FillSeqSum(mi355x_search_ctx* ctx, const void* x, int64_t row_stride
   q->seg_sum = ctx->seg_sum;
   q->seg_step = ctx->seg_step;
   q->sub_step = ctx->sub_step;
+  q->sub_se = ctx->sub_se;
   q->e = reinterpret_cast<float*>(ctx->big);
   q->e_stride = ctx->big_stride * 2;
   q->out_max = ctx->row_max;

@@ -78,12 +78,10 @@ __device__ __forceinline__ Step wave_scan_steps(Step x) {
   return x;
 }
 
-// The same scan inside every row of sixteen lanes only: lanes 15, 31, 47 and 63 end with their row's composition.
-__device__ __forceinline__ Step row_scan_steps(Step x) {
+// Composition over groups of four lanes: lanes 3, 7, 11, ... end with the composition of their group.
+__device__ __forceinline__ Step quad_scan_steps(Step x) {
   x = step_compose(step_from_below<0x111, 0xf>(x), x);  // row_shr:1
   x = step_compose(step_from_below<0x112, 0xf>(x), x);  // row_shr:2
-  x = step_compose(step_from_below<0x114, 0xf>(x), x);  // row_shr:4
-  x = step_compose(step_from_below<0x118, 0xf>(x), x);  // row_shr:8
   return x;
 }
 

@@ -84,7 +84,7 @@ constexpr int kBeamMaxCand = 32;  // 2 * beams, beams <= 16
 
 // Multi-workgroup exact sequential sum (seqsum_kernels.hip).
 constexpr int kSegElems = 4096;   // elements per segment
-constexpr int kSegSubs = 16;      // parts of a segment with composed steps of their own (256 elements each)
+constexpr int kSegSubs = 64;      // parts of a segment with composed steps of their own (64 elements each)
 constexpr int kMaxSegs = 1024;    // segments per row the walk kernel can hold
 constexpr int kSeqSumMinVocab = 16384;  // shorter rows are summed by one workgroup in one launch
 
@@ -95,10 +95,10 @@ struct SeqSumArgs {
   float inv_temp;
   uint32_t* seg_max;  // [rows][segs] order keys
   double* seg_sum;    // [rows][segs]
-  int4* seg_step;     // [rows][segs]: d0, d1, binade, unused; binade -1: scan the segment; -2: one power of two may
-                      // fall inside the segment, the sixteen parts of the segment have records in sub_step and
-                      // the last field holds the binade before it
-  int4* sub_step;     // [rows][segs][kSegSubs]: (d0, d1) of a 256-element part under the lower binade, then under the next
+  int4* seg_step;     // [rows][segs]: d0, d1, binade, unused; binade -2: powers of two may fall inside the segment and
+                      // its parts have records of their own
+  int4* sub_step;     // [rows][segs][kSegSubs]: (d0, d1) of a 64-element part under the binade in sub_se, then under the next
+  int* sub_se;        // [rows][segs][kSegSubs]: that binade; -1: the walk adds the part element by element
   float* e;           // [rows][e_stride] exponentials
   size_t e_stride;
   float* out_max;     // [rows]

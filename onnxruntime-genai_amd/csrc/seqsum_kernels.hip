@@ -10,10 +10,11 @@
 //   3. seqsum_step:  from the double prefix sums a segment knows the binade its running sum will be
 //                    in -- unless a power of two may fall inside it -- and composes the step functions
 //                    of its elements under that binade into one (d0, d1) pair.
-//   4. seqsum_walk:  one workgroup per row walks the segments in order: a composed step is applied
-//                    after checking that the running sum really is in the assumed binade and stays
-//                    in it (then the composition is exactly the sequential result); every other
-//                    segment is summed with the exact in-order scan of block_seq.h.
+//   4. seqsum_walk:  one wave per row walks the segments in order: composed steps are applied after
+//                    checking that the running sum really is in the assumed binade and stays in it
+//                    (then the composition is exactly the sequential result); a segment that may hold
+//                    a power of two is walked through the composed steps of its 64 parts, and a
+//                    part that fails the check is added element by element.
 // The check in step 4 makes the result independent of the estimate in step 3: a wrong guess only
 // costs a scan.
 #include "kernels.h"
@@ -102,37 +103,53 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs
   const double lo = before * (1.0 - seq_drift(first));
   const double hi = (before + sums[seg]) * (1.0 + seq_drift(first + n));
   const float lo_f = __double2float_rd(lo), hi_f = __double2float_ru(hi);
-  const int se = seq_decompose(lo_f).se, se_hi = seq_decompose(hi_f).se;
+  const int se = seq_decompose(lo_f).se;
   int4* rec = a.seg_step + static_cast<size_t>(row) * a.segs + seg;
-  const bool in_range = lo_f > 0.0f && hi_f < 3.0e38f;
-  const bool known = in_range && se_hi == se;
-  if (!known && !(in_range && se_hi == se + 1)) {  // several powers of two may fall inside the segment: the walk scans it
-    if (tid == 0) *rec = make_int4(0, 0, -1, 0);
-    return;
-  }
+  const bool known = lo_f > 0.0f && hi_f < 3.0e38f && seq_decompose(hi_f).se == se;
   const float* erow = a.e + static_cast<size_t>(row) * a.e_stride + first;
   float ev[kSegPer];
   window_fetch<kSegPer>(ev, 0, n, [=](int i) { return erow[i]; }, stage);
   if (!known) {
-    // One power of two may fall inside the segment.  Each of its sixteen 256-element parts (sixteen lanes of
-    // sixteen elements) gets a composed step under the binade before that power and one under the binade after
-    // it: the walk applies the first kind up to the part where the sum leaves the binade, adds that part
-    // element by element, and goes on with the second kind.
-    static_assert(kSegSubs * 16 * kSegPer == kSegElems && kSegBlock == kSegSubs * 16, "a part is sixteen lanes");
-    Step lo_step{0u, 0u}, hi_step{0u, 0u};
+    // Powers of two may fall inside the segment.  Each of its 64-element parts (four lanes of sixteen elements)
+    // estimates the binade the sum has where the part begins, from the double sums of the parts before it, and
+    // gets a composed step under that binade and one under the next: the walk applies the one that matches the
+    // sum it holds, and adds a part element by element where the sum leaves its binade inside the part or the
+    // estimate was wrong.
+    constexpr int kPart = kSegElems / kSegSubs;
+    static_assert(kPart == 4 * kSegPer && kSegBlock == kSegSubs * 4, "a part is four lanes");
+    __shared__ double part_sum[kSegSubs];
+    double mine = 0.0;
 #pragma unroll
-    for (int j = 0; j < kSegPer; ++j) {
-      lo_step = step_compose(lo_step, seq_make_step(ev[j], se));
-      hi_step = step_compose(hi_step, seq_make_step(ev[j], se + 1));
+    for (int j = 0; j < kSegPer; ++j) mine += static_cast<double>(ev[j]);
+    mine += __shfl_xor(mine, 1, 64);
+    mine += __shfl_xor(mine, 2, 64);  // all four lanes of a part hold its sum
+    const int part = tid >> 2;
+    if ((lane & 3) == 0) part_sum[part] = mine;
+    __syncthreads();
+    double start = before;
+    for (int q = 0; q < part; ++q) start += part_sum[q];
+    const int p_first = first + part * kPart;
+    const float plo = __double2float_rd(start * (1.0 - seq_drift(p_first)));
+    const float phi = __double2float_ru((start + mine) * (1.0 + seq_drift(p_first + kPart)));
+    int pse = seq_decompose(plo).se;
+    if (!(plo > 0.0f && phi < 3.0e38f && seq_decompose(phi).se <= pse + 1)) pse = -1;  // the walk adds this part itself
+    Step lo_step{0u, 0u}, hi_step{0u, 0u};
+    if (pse >= 0) {
+#pragma unroll
+      for (int j = 0; j < kSegPer; ++j) {
+        lo_step = step_compose(lo_step, seq_make_step(ev[j], pse));
+        hi_step = step_compose(hi_step, seq_make_step(ev[j], pse + 1));
+      }
     }
-    lo_step = row_scan_steps(lo_step);
-    hi_step = row_scan_steps(hi_step);
-    if ((lane & 15) == 15) {
-      int4* sub = a.sub_step + (static_cast<size_t>(row) * a.segs + seg) * kSegSubs;
-      sub[tid >> 4] = make_int4(static_cast<int>(lo_step.d0), static_cast<int>(lo_step.d1), static_cast<int>(hi_step.d0),
-                                static_cast<int>(hi_step.d1));
+    lo_step = quad_scan_steps(lo_step);
+    hi_step = quad_scan_steps(hi_step);
+    if ((lane & 3) == 3) {
+      const size_t at = (static_cast<size_t>(row) * a.segs + seg) * kSegSubs + part;
+      a.sub_step[at] = make_int4(static_cast<int>(lo_step.d0), static_cast<int>(lo_step.d1), static_cast<int>(hi_step.d0),
+                                 static_cast<int>(hi_step.d1));
+      a.sub_se[at] = pse;
     }
-    if (tid == 0) *rec = make_int4(0, 0, -2, se);
+    if (tid == 0) *rec = make_int4(0, 0, -2, 0);
     return;
   }
   Step agg{0u, 0u};
@@ -148,65 +165,170 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs
   }
 }
 
-constexpr int kWalkBlock = 256;
+// ---- the walk: one wave per row, no barriers -----------------------------------------------------------
+// Steps compose associatively as long as the sum stays in one binade, so the wave does not visit the segments
+// one by one: lane l takes the record of segment seg + l, the wave scans the compositions, and every lane
+// checks whether the sum would still be inside the binade after its segment.  All lanes before the first one
+// that fails are exact; the failing segment is handled through the records of its 64 parts in the same way,
+// a part that fails is added element by element (a chain of lane-shifted float additions), and the wave goes on
+// behind it with the binade the sum then has.
+constexpr Step kStepIdentity{0u, 0u};
+constexpr Step kStepLeaves{kStepSat, kStepSat};  // composed with anything, it still says "left the binade"
+constexpr int kWalkSpecials = 16;                 // segments per group of 64 whose part records are cached in LDS
 
-__global__ __launch_bounds__(kWalkBlock) void seqsum_walk_kernel(const SeqSumArgs a) {
-  __shared__ SeqShared sh;
-  __shared__ uint32_t red[16];
-  __shared__ int4 recs[kMaxSegs];
-  __shared__ int4 subs[kSegSubs];
-  __shared__ __align__(16) float stage[kSegElems];
-  const int row = blockIdx.x, tid = threadIdx.x;
-  for (int s = tid; s < a.segs; s += kWalkBlock) recs[s] = a.seg_step[static_cast<size_t>(row) * a.segs + s];
-  const float max_score = row_max_of_segments(a, row, red);  // its barriers also publish recs
+// Applies the steps f (one per lane; identity below `from`, kStepLeaves where no valid record exists) to the sum
+// s in lane order and returns the number of leading lanes from `from` on, below `limit`, whose results are exact;
+// s becomes the sum behind the last of them.
+__device__ __forceinline__ int wave_apply_steps(float& s, Step f, int from, int limit) {
+  const int lane = lane_id();
+  const SeqState st = seq_decompose(s);
+  const Step p = wave_scan_steps(f);
+  const uint32_t n2 = step_apply(st.n, p);
+  const unsigned long long bad = __ballot(lane >= from && lane < limit && n2 >= kMantLimit);
+  const int stop = bad != 0ull ? __ffsll(static_cast<long long>(bad)) - 1 : limit;
+  if (stop > from) s = seq_recompose(__shfl(n2, stop - 1, 64), st.se);
+  return stop;
+}
+
+constexpr int kWalkAhead = 8;  // parts per cached segment whose elements are fetched ahead into LDS
+
+__global__ __launch_bounds__(64) void seqsum_walk_kernel(const SeqSumArgs a) {
+  static_assert(kSegSubs == 64, "one part per lane");
+  constexpr int kPart = kSegElems / kSegSubs;
+  static_assert(kPart == 64, "a part is one round of the addition chain");
+  __shared__ int4 part_rec[kWalkSpecials][kSegSubs];
+  __shared__ int part_se[kWalkSpecials][kSegSubs];
+  __shared__ float ahead[kWalkSpecials][kWalkAhead][kPart];
+  __shared__ int ahead_part[kWalkSpecials][kWalkAhead];
+  __shared__ int items[kWalkSpecials * kWalkAhead];
+  const int row = blockIdx.x, lane = threadIdx.x;
+  const size_t rbase = static_cast<size_t>(row) * a.segs;
+  uint32_t m = 0u;
+  for (int sg = lane; sg < a.segs; sg += 64) {
+    const uint32_t k = a.seg_max[rbase + sg];
+    m = k > m ? k : m;
+  }
+  const float max_score = key_to_float(wave_max<uint32_t>(m));
   const float* erow = a.e + static_cast<size_t>(row) * a.e_stride;
   float s = 0.0f;
-  for (int seg = 0; seg < a.segs; ++seg) {
-    const int4 r = recs[seg];
-    if (r.z >= 0) {
-      const SeqState st = seq_decompose(s);
-      if (st.se == r.z) {
-        const uint32_t n2 = step_apply(st.n, Step{static_cast<uint32_t>(r.x), static_cast<uint32_t>(r.y)});
-        if (n2 < kMantLimit) {  // stayed inside the binade: the composed step is the sequential result
-          s = seq_recompose(n2, st.se);
-          continue;
+  for (int g0 = 0; g0 < a.segs; g0 += 64) {  // groups of 64 segments, one per lane
+    const int g_n = a.segs - g0 < 64 ? a.segs - g0 : 64;
+    const int4 r = lane < g_n ? a.seg_step[rbase + g0 + lane] : make_int4(0, 0, -3, 0);
+    // The part records of the group's first segments that have any are fetched now, all together, and with
+    // them the elements of the parts that will most likely be added one by one: those whose estimated binade
+    // differs from the next part's, and those without an estimate.
+    __syncthreads();  // (one wave: orders the LDS accesses of the previous group before these stores)
+    const unsigned long long special = __ballot(lane < g_n && r.z == -2);
+    const int n_special = __popcll(special) < kWalkSpecials ? __popcll(special) : kWalkSpecials;
+    // (all record loads are requested before the first is used, then all element loads)
+    int4 rec_q[kWalkSpecials];
+    int rec_se[kWalkSpecials];
+    int seg_of[kWalkSpecials];
+    {
+      unsigned long long left = special;
+#pragma unroll
+      for (int slot = 0; slot < kWalkSpecials; ++slot) {
+        seg_of[slot] = -1;
+        rec_q[slot] = make_int4(0, 0, 0, 0);
+        rec_se[slot] = -1;
+        if (slot < n_special) {
+          seg_of[slot] = __ffsll(static_cast<long long>(left)) - 1;
+          left &= left - 1ull;
+          const size_t at = (rbase + g0 + seg_of[slot]) * kSegSubs;
+          rec_q[slot] = a.sub_step[at + lane];
+          rec_se[slot] = a.sub_se[at + lane];
         }
       }
     }
-    const int first = seg * kSegElems;
-    const int n = a.vocab - first < kSegElems ? a.vocab - first : kSegElems;
-    const float* e = erow + first;
-    int dummy;
-    if (r.z == -2) {
-      // part by part: a part's composed step under the binade the sum is in, or -- where the sum leaves the
-      // binade, or is in neither of the two binades the records were made for -- the part's elements one by one
-      const int4* sub = a.sub_step + (static_cast<size_t>(row) * a.segs + seg) * kSegSubs;
-      __syncthreads();  // the previous segment's readers of subs are done
-      if (tid < kSegSubs) subs[tid] = sub[tid];
-      __syncthreads();
-      constexpr int kPart = kSegElems / kSegSubs;
-      for (int j = 0; j * kPart < n; ++j) {
-        const SeqState st = seq_decompose(s);
-        const int4 q = subs[j];
-        if (st.se == r.w || st.se == r.w + 1) {
-          const Step f = st.se == r.w ? Step{static_cast<uint32_t>(q.x), static_cast<uint32_t>(q.y)}
-                                      : Step{static_cast<uint32_t>(q.z), static_cast<uint32_t>(q.w)};
-          const uint32_t n2 = step_apply(st.n, f);
-          if (n2 < kMantLimit) {
-            s = seq_recompose(n2, st.se);
-            continue;
+    int n_items = 0;  // (slot, position, part) of every part fetched ahead, listed in LDS
+#pragma unroll
+    for (int slot = 0; slot < kWalkSpecials; ++slot) {
+      if (slot < n_special) {
+        part_rec[slot][lane] = rec_q[slot];
+        part_se[slot][lane] = rec_se[slot];
+        const int next_se = __shfl_down(rec_se[slot], 1, 64);
+        unsigned long long want = __ballot(rec_se[slot] < 0 || (lane < 63 && next_se != rec_se[slot]));
+        for (int c = 0; c < kWalkAhead; ++c) {
+          int p = -1;
+          if (want != 0ull) {
+            p = __ffsll(static_cast<long long>(want)) - 1;
+            want &= want - 1ull;
+            if (lane == 0) items[n_items] = (seg_of[slot] << 16) | (slot << 10) | (c << 6) | p;
+            ++n_items;
           }
+          if (lane == 0) ahead_part[slot][c] = p;
         }
-        const float* ep = e + j * kPart;
-        const int np = n - j * kPart < kPart ? n - j * kPart : kPart;
-        s = block_seq_sum<kPart / kWalkBlock>(s, np, [=](int i) { return ep[i]; }, NoStop{}, &dummy, sh, nullptr, kPart);  // one wave's chain
       }
-      continue;
     }
-    s = block_seq_sum<kSegElems / kWalkBlock>(s, n, [=](int i) { return e[i]; }, NoStop{}, &dummy, sh, stage,
-                                                 seg == 0 ? 1024 : 0);
+    __syncthreads();
+    for (int i0 = 0; i0 < n_items; i0 += 8) {
+      float val[8];
+      int item[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        item[u] = i0 + u < n_items ? items[i0 + u] : -1;
+        val[u] = 0.0f;
+        if (item[u] >= 0) {
+          const int sg = item[u] >> 16, p = item[u] & 63;
+          const int idx = (g0 + sg) * kSegElems + p * kPart + lane;
+          if (idx < a.vocab) val[u] = erow[idx];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (item[u] >= 0) ahead[(item[u] >> 10) & 63][(item[u] >> 6) & 15][lane] = val[u];
+    }
+    __syncthreads();
+    int seg = 0;  // inside the group
+    while (seg < g_n) {
+      // the run of whole segments that are in the binade the sum is in now
+      const int se = seq_decompose(s).se;
+      const Step f = lane < seg ? kStepIdentity : (r.z == se ? Step{static_cast<uint32_t>(r.x), static_cast<uint32_t>(r.y)} : kStepLeaves);
+      seg = wave_apply_steps(s, f, seg, g_n);
+      if (seg >= g_n) break;
+      // segment `seg` part by part
+      const int first = (g0 + seg) * kSegElems;
+      const int n = a.vocab - first < kSegElems ? a.vocab - first : kSegElems;
+      const int n_parts = (n + kPart - 1) / kPart;
+      const int z = __shfl(r.z, seg, 64);
+      const int slot = __popcll(special & ((1ull << seg) - 1ull));
+      const bool cached = z == -2 && slot < kWalkSpecials;
+      int4 q = make_int4(0, 0, 0, 0);
+      int pse = -1;
+      if (cached) {
+        q = part_rec[slot][lane];
+        pse = part_se[slot][lane];
+      } else if (z == -2) {
+        q = a.sub_step[(rbase + g0 + seg) * kSegSubs + lane];
+        pse = a.sub_se[(rbase + g0 + seg) * kSegSubs + lane];
+      }
+      int part = 0;
+      while (part < n_parts) {
+        const int pe = seq_decompose(s).se;
+        Step pf = kStepLeaves;
+        if (lane < part) pf = kStepIdentity;
+        else if (pse >= 0 && pse == pe) pf = Step{static_cast<uint32_t>(q.x), static_cast<uint32_t>(q.y)};
+        else if (pse >= 0 && pse + 1 == pe) pf = Step{static_cast<uint32_t>(q.z), static_cast<uint32_t>(q.w)};
+        part = wave_apply_steps(s, pf, part, n_parts);
+        if (part < n_parts) {
+          // this part's elements one by one, from LDS where they were fetched ahead
+          const int np = n - part * kPart < kPart ? n - part * kPart : kPart;
+          const float* src = erow + first + part * kPart;
+          int hit = -1;
+          if (cached) {
+#pragma unroll
+            for (int c = 0; c < kWalkAhead; ++c)
+              if (ahead_part[slot][c] == part) hit = c;
+          }
+          const float x = hit >= 0 ? ahead[slot][hit][lane] : (lane < np ? src[lane] : 0.0f);
+          s = __shfl(wave_serial_prefix(lane == 0 ? s + x : x, 64), 63, 64);
+          ++part;
+        }
+      }
+      ++seg;
+    }
   }
-  if (tid == 0) {
+  if (lane == 0) {
     a.out_sum[row] = s;
     a.out_max[row] = max_score;
   }
@@ -250,7 +372,7 @@ extern "C" hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, int h
     hipLaunchKernelGGL(ms::seqsum_exp_kernel<float>, grid, block, 0, stream, *a);
   }
   hipLaunchKernelGGL(ms::seqsum_step_kernel, grid, block, 0, stream, *a);
-  hipLaunchKernelGGL(ms::seqsum_walk_kernel, dim3(a->rows), dim3(ms::kWalkBlock), 0, stream, *a);
+  hipLaunchKernelGGL(ms::seqsum_walk_kernel, dim3(a->rows), dim3(64), 0, stream, *a);
   return hipGetLastError();
 }
 
