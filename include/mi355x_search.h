@@ -68,6 +68,12 @@ typedef struct mi355x_search_ctx mi355x_search_ctx;
  *            history ids gets lowest(), after the penalty (ApplyNoRepeatNgramToLogits,
  *            src/sampling_distribution.h:64-79; Search_Cpu::ApplyNoRepeatNgram,
  *            src/search.cpp:432-469).  Needs history.
+ *   mask_allowed_max  optional promise about `mask`: no row's mask has more than this many bits set
+ *            (0 = unknown).  The grammar engine builds the mask on the host (ComputeMask,
+ *            src/constrained_logits_processor.cpp:157-188), where the count is one popcount pass.  When the
+ *            bound fits the sort buffer of the sparse-mask kernel (about 16000 ids together with the history),
+ *            nucleus rows are finished by that one kernel and the dense kernels are not launched at all; a row
+ *            that breaks the promise is still sampled correctly, by the exact path (slowly).
  */
 typedef struct mi355x_logits_xform {
   const uint32_t* mask;
@@ -81,6 +87,7 @@ typedef struct mi355x_logits_xform {
   const int32_t* history_lens;
   int32_t min_length;
   int32_t no_repeat_ngram_size;
+  int32_t mask_allowed_max;
 } mi355x_logits_xform;
 
 /* (k, p, temperature) of one row: BatchedSamplingParams, src/smartptrs.h:113-117.  Meaning as in

@@ -20,7 +20,7 @@ class LogitsXformC(C.Structure):
     _fields_ = [("mask", C.c_void_p), ("history", C.c_void_p), ("history_stride", C.c_int32),
                 ("history_len", C.c_int32), ("repetition_penalty", C.c_float), ("apply_min_length", C.c_int32),
                 ("n_eos", C.c_int32), ("eos_ids", C.c_int32 * MAX_EOS), ("history_lens", C.c_void_p),
-                ("min_length", C.c_int32), ("no_repeat_ngram_size", C.c_int32)]
+                ("min_length", C.c_int32), ("no_repeat_ngram_size", C.c_int32), ("mask_allowed_max", C.c_int32)]
 
 
 class SampleParams(C.Structure):
@@ -98,7 +98,7 @@ class LogitsXform:
 
     def __init__(self, mask=None, history=None, history_len=None, repetition_penalty=1.0, eos_ids=(),
                  apply_min_length=False, history_lens=None, min_length=0, no_repeat_ngram_size=0,
-                 shared_history=False):
+                 shared_history=False, mask_allowed_max=0):
         self.mask, self.history, self.history_lens = mask, history, history_lens
         c = self.c = LogitsXformC()
         c.mask = mask.data_ptr() if mask is not None else None
@@ -116,6 +116,7 @@ class LogitsXform:
         c.apply_min_length = int(apply_min_length)
         c.min_length = min_length
         c.no_repeat_ngram_size = no_repeat_ngram_size
+        c.mask_allowed_max = mask_allowed_max
         c.n_eos = len(eos_ids)
         for i, e in enumerate(eos_ids):
             c.eos_ids[i] = e

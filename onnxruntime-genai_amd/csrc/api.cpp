@@ -375,6 +375,12 @@ int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const 
   a.fallback_rows = ctx->fallback_rows;
   a.poll_limit = ctx->poll_limit;
   a.row_done = ctx->row_done;
+  // a caller that bounds the number of allowed ids per row lets the sparse-mask kernel work alone
+  if (xf && xf->mask && xf->mask_allowed_max > 0) {
+    const int hist = a.xf.history_lens ? a.xf.history_stride : a.xf.history_len;
+    const int64_t listed = static_cast<int64_t>(xf->mask_allowed_max) + (a.xf.use_penalty() ? hist : 0) + 2;
+    a.sparse_only = listed <= ms::kNucleusCap && hist <= 2048;  // (what the kernel can list; beyond, all three kernels)
+  }
   HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_other, any_nucleus, any_large_k, s));
   return MI355X_OK;
 }

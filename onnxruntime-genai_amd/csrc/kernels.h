@@ -68,6 +68,8 @@ struct SampleArgs {
                             // best id only, k = 1, with ArgMax's rule that a NaN at id 0 wins (src/search.h:9-29)
   float* out_scores;        // [rows, k], emit_topk == 1 only (out_tokens is [rows, k] then)
   uint32_t* row_done;       // [rows] or null: nucleus rows under a grammar mask that the sparse-mask kernel finished
+  int sparse_only;          // the sparse-mask kernel is the only one launched for nucleus rows: a row it cannot
+                            // finish goes to the exact path inside it
 };
 
 struct ArgmaxArgs {

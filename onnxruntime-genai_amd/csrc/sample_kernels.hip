@@ -461,8 +461,9 @@ __device__ __forceinline__ void sparse_gather(const void* row0, const uint32_t (
   for (int u = 0; u < kSparseIds; ++u) x[u] = load_one<InT>(&raw[u], 0);
 }
 
+// Returns 1 when the row is finished, 0 when it is not, -1 when it is not a nucleus row.
 template <bool INLINE>
-__device__ __forceinline__ void nucleus_sparse_body(const SampleArgs& a) {
+__device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   extern __shared__ u64 lds_keys[];
   uint32_t* const bucket_start = reinterpret_cast<uint32_t*>(lds_keys + kNucleusCap);
   uint32_t* const hist_bits = reinterpret_cast<uint32_t*>(lds_keys);                  // first half: history bitmap of the row
@@ -476,14 +477,14 @@ __device__ __forceinline__ void nucleus_sparse_body(const SampleArgs& a) {
   const int row = blockIdx.x, tid = threadIdx.x, lane = lane_id();
   const int V = a.vocab;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
-  if (row_mode(prm, V, a.chunks) != kModeNucleus) return;
+  if (row_mode(prm, V, a.chunks) != kModeNucleus) return -1;
   const int words = (V - 1) / 32 + 1;
-  auto leave = [&](bool done) {
-    if (tid == 0) a.row_done[row] = done ? 1u : 0u;
-  };
+  const RowPtr<AnyDtype> lrow(row_start<INLINE>(a, row, dtype_bytes(a.dtype)), a.dtype);
+  // A row this kernel cannot finish is left to the dense kernels launched after it -- or, when the caller's
+  // bound on the mask made this the only kernel, to the exact path (the caller of this function sees to that).
+  auto leave = [&](bool done) { return done ? 1 : 0; };
   if (words > kFinishBlock * kSparseWords) return leave(false);
   const uint32_t* mrow = a.xf.mask + static_cast<size_t>(row) * words;
-  const RowPtr<AnyDtype> lrow(row_start<INLINE>(a, row, dtype_bytes(a.dtype)), a.dtype);
   const int n_eos = a.xf.eos_count(row);
   const bool pen = a.xf.use_penalty();
   // allowed ids of this thread's words: mask bits minus the EOS ids under min-length, nothing past the vocabulary
@@ -632,12 +633,32 @@ __device__ __forceinline__ void nucleus_sparse_body(const SampleArgs& a) {
   const uint32_t n_c = sh_count;
   const bool ok = finish_candidates(lds_keys, bucket_start, n_c, best_below, rmax, thr, false, prm, V, a.uniforms[row],
                                     row_outputs(a, row), seqsh, red32);
-  leave(ok);
+  return leave(ok);
 }
 
-__global__ __launch_bounds__(kFinishBlock) void nucleus_sparse_kernel(const SampleArgs a) { nucleus_sparse_body<false>(a); }
+template <bool INLINE>
+__device__ __forceinline__ void nucleus_sparse_entry(const SampleArgs& a) {
+  int done = nucleus_sparse_body<INLINE>(a);
+  if (done < 0) return;
+  const int row = blockIdx.x;
+  if (done == 0 && a.sparse_only) {  // no dense kernels follow: the exact path, here
+    extern __shared__ u64 lds_keys[];
+    __shared__ SeqShared exact_sh;
+    __syncthreads();
+    u64* const tile = lds_keys;
+    general_row<AnyDtype>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), row_params<INLINE>(a, row),
+                          a.big + static_cast<size_t>(row) * a.big_stride, exact_sh, [=](u64* keys, int n2, int) {
+                            if (n2 >= 2 * kNucleusCap) tiled_sort_desc(keys, n2, tile);
+                            else block_sort_desc(keys, n2);
+                          });
+    done = 1;
+  }
+  if (threadIdx.x == 0) a.row_done[row] = static_cast<uint32_t>(done);
+}
+
+__global__ __launch_bounds__(kFinishBlock) void nucleus_sparse_kernel(const SampleArgs a) { nucleus_sparse_entry<false>(a); }
 __global__ __launch_bounds__(kFinishBlock) void nucleus_sparse_rows_kernel(const SampleArgs a, const InlineParams) {
-  nucleus_sparse_body<true>(a);
+  nucleus_sparse_entry<true>(a);
 }
 
 }  // namespace ms
@@ -660,12 +681,14 @@ extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::Inline
       e = hipGetLastError();
       if (e != hipSuccess) return e;
     }
-    e = launch_stream(a, table, 1, stream);
-    if (e != hipSuccess) return e;
-    if (table) hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
-    else hipLaunchKernelGGL(ms::nucleus_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
-    e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (!(a->xf.mask && a->row_done && a->sparse_only)) {
+      e = launch_stream(a, table, 1, stream);
+      if (e != hipSuccess) return e;
+      if (table) hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
+      else hipLaunchKernelGGL(ms::nucleus_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
+      e = hipGetLastError();
+      if (e != hipSuccess) return e;
+    }
   }
   if (any_large_k) {
     e = launch_stream(a, table, 2, stream);

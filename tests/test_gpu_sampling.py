@@ -734,17 +734,24 @@ def test_nucleus_rows_under_sparse_and_dense_masks(ctx, orc, vocab, frac, penalt
     xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
                            repetition_penalty=penalty, eos_ids=eos, apply_min_length=True)
     cap = 20000
-    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=p, temperature=0.9,
-                                 xf=xf, kept_capacity=cap)
-    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
     proc = orc.apply_mask(x, mask)
+    want = []
     for r in range(rows):
         row = proc[r].copy()
         row[eos] = LOWEST
         row = orc.apply_repetition_penalty(row, hist[r][(hist[r] >= 0)], penalty)
-        idx, probs = orc.sampled_categorical(row, 0, p, 0.9)
-        n = min(len(idx), cap)
-        assert kc[r] == len(idx), (r, kc[r], len(idx))
-        assert np.array_equal(ki[r, :n], idx[:n]), r
-        assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), r
-        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+        want.append(orc.sampled_categorical(row, 0, p, 0.9))
+    # without a promise about the mask, with the true bound on the allowed ids per row, and with a promise
+    # that the rows break (they are still sampled correctly, by the exact path)
+    for promise in (0, int(allowed.sum(axis=1).max()), 3):
+        xf.c.mask_allowed_max = promise
+        tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=p, temperature=0.9,
+                                     xf=xf, kept_capacity=cap)
+        tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+        for r in range(rows):
+            idx, probs = want[r]
+            n = min(len(idx), cap)
+            assert kc[r] == len(idx), (promise, r, kc[r], len(idx))
+            assert np.array_equal(ki[r, :n], idx[:n]), (promise, r)
+            assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), (promise, r)
+            assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (promise, r)
