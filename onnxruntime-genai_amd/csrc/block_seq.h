@@ -404,14 +404,15 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float
 }
 
 // In-place bitonic sort, descending, of n (a power of two) keys in LDS or global memory.
-__device__ __forceinline__ void block_sort_desc(u64* a, int n) {
+template <typename Key>
+__device__ __forceinline__ void block_sort_desc(Key* a, int n) {
   for (int k = 2; k <= n; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
       for (int t = threadIdx.x; t < (n >> 1); t += blockDim.x) {
         const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1));
         const int hi = lo | j;
         const bool desc = (lo & k) == 0;
-        const u64 x = a[lo], y = a[hi];
+        const Key x = a[lo], y = a[hi];
         if ((x < y) == desc) {
           a[lo] = y;
           a[hi] = x;

@@ -28,9 +28,11 @@ constexpr int kModeTopkSmall = 0;
 constexpr int kModeNucleus = 1;
 constexpr int kModeGeneral = 2;
 constexpr int kModeTopkLarge = 3;  // 64 < k <= kLargeKMax: streamed and finished by the nucleus kernels
-// The per-chunk bound of such rows is the k-th best of the 1024 per-thread maxima of a nucleus workgroup; up to half
-// the threads it stays tight (about 1.4 k elements reach it), towards all of them it lets a third of the chunk through.
-constexpr int kLargeKMax = 512;
+// The per-chunk bound of such rows is the k-th best of what the 1024 threads of a nucleus workgroup offer: their
+// maxima up to k = 512 (tight up to half the threads: about 1.4 k elements reach it), their four best elements
+// each beyond that (about 1.1 k elements reach the k-th best of those 4096).
+constexpr int kLargeKMax = 2048;
+constexpr int kLargeKOneOffer = 512;  // up to here one offer per thread is enough
 
 // Heterogeneous (k, p, T) of a batch of at most kInlineParamRows rows travel inside the kernel
 // arguments, as a second argument of kernel variants of their own, so that no copy to the device

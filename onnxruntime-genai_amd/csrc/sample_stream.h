@@ -592,18 +592,49 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     // Rows with 64 < k <= kLargeKMax come here too: their candidates are the elements that reach the
     // exact k-th best per-thread maximum of the chunk (at least k elements do; with fewer than k
     // threads holding elements, all), which contain the chunk's k best.
-    static_assert(kLargeKMax <= kSBlock && kSMaxWaves * kWaveListCap >= kSBlock, "one offer per thread, sorted in the hit lists' LDS");
+    static_assert(kLargeKOneOffer <= kSBlock && kSMaxWaves * kWaveListCap >= kSBlock, "one offer per thread, sorted in the hit lists' LDS");
+    static_assert(kLargeKMax <= 4 * kSBlock && kSMaxWaves * kWaveListCap * sizeof(u64) >= 4 * kSBlock * sizeof(uint32_t),
+                  "four offers per thread, sorted as 32-bit keys in the hit lists' LDS");
     constexpr bool large_k = LARGEK;
     const uint32_t cmax = block_max<uint32_t>(lmax, sm.wave_val);
     float thr = -__builtin_inff();
     if (large_k) {
-      u64* scratch = sm.wave_list;
-      scratch[tid] = static_cast<u64>(lmax);
-      __syncthreads();
-      block_sort_desc(scratch, kSBlock);
-      const uint32_t kth = static_cast<uint32_t>(scratch[(prm.k < V ? prm.k : V) - 1]);
-      if (kth != 0u) thr = key_to_float(kth);
-      __syncthreads();
+      const int kk = prm.k < V ? prm.k : V;
+      if (kk <= kLargeKOneOffer) {
+        u64* scratch = sm.wave_list;
+        scratch[tid] = static_cast<u64>(lmax);
+        __syncthreads();
+        block_sort_desc(scratch, kSBlock);
+        const uint32_t kth = static_cast<uint32_t>(scratch[kk - 1]);
+        if (kth != 0u) thr = key_to_float(kth);
+        __syncthreads();
+      } else {
+        // the four best elements of every thread (registers and its share of the history ids' list), as order
+        // keys: at least k elements reach the k-th best of those offers, or fewer than k exist and all are kept
+        uint32_t best[4] = {0u, 0u, 0u, 0u};
+        auto offer = [&](float x) {
+          uint32_t key = order_key(x);  // 0 for NaN: no element
+          if (key > best[3]) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const uint32_t hi = key > best[q] ? key : best[q];
+              key = key > best[q] ? best[q] : key;
+              best[q] = hi;
+            }
+          }
+        };
+#pragma unroll
+        for (int e = 0; e < kSElems; ++e) offer(v[e]);
+        for (uint32_t i = tid; i < n_extra; i += kSBlock) offer(sm.extra_val[i]);
+        uint32_t* offers = reinterpret_cast<uint32_t*>(sm.wave_list);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) offers[tid * 4 + q] = best[q];
+        __syncthreads();
+        block_sort_desc(offers, 4 * kSBlock);
+        const uint32_t kth = offers[kk - 1];
+        if (kth != 0u) thr = key_to_float(kth);
+        __syncthreads();
+      }
     } else if (cmax != 0u) {
       thr = key_to_float(cmax) - nucleus_depth(prm, V);
     }
