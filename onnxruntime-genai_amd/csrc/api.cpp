@@ -61,6 +61,7 @@ struct mi355x_search_ctx {
   uint32_t* row_arrive{};
   ms::u64* row_best{};
   ms::u64* big{};
+  ms::u64* big2{};
   size_t big_stride{};
   uint32_t* fallback_rows{};
   uint32_t* row_done{};
@@ -193,6 +194,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->row_arrive, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->row_best, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->big, static_cast<size_t>(max_rows) * c->big_stride, false));
+  ok(c->Alloc(&c->big2, static_cast<size_t>(max_rows) * c->big_stride, false));
   ok(c->Alloc(&c->row_done, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->fallback_rows, 2, true));  // [0] rows finished by the exact path, [1] a wait gave up
   ok(c->Alloc(&c->ban, static_cast<size_t>(max_rows) * ((max_vocab - 1) / 32 + 1), false));
@@ -317,7 +319,7 @@ int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const 
                int32_t* kept_count, int32_t* kept_ids, float* kept_probs, int kept_capacity) {
   ms::SampleArgs a{};
   if (int r = MakeXform(ctx, xf, rows, vocab, s, &a.xf)) return r;
-  bool any_nucleus = false, any_other = false, any_large_k = false;
+  bool any_nucleus = false, any_other = false, any_large_k = false, any_exact = false;
   const int chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
   ms::InlineParams table{};
   bool use_table = false;
@@ -326,10 +328,12 @@ int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const 
     // the kernels' own rule (row_mode) decides; these flags only have to cover it
     const int kk = p.k < vocab ? p.k : vocab;
     const bool fits = vocab > 64 && chunks * ms::kSmallCap <= ms::kAllCap;
-    const bool nucleus = p.k <= 1, large_k = p.k > 1 && kk > 64 && kk <= ms::kLargeKMax;
+    const bool whole = p.k <= 1 && !(p.p < 1.0f);  // no top-k and no nucleus: the whole vocabulary
+    const bool nucleus = p.k <= 1 && !whole, large_k = p.k > 1 && kk > 64 && kk <= ms::kLargeKMax;
     if (nucleus && vocab > 64) any_nucleus = true;
     if (large_k && vocab > 64) any_large_k = true;
-    if (!((nucleus || large_k) && fits)) any_other = true;
+    if (vocab > 64 && (!fits || whole || (p.k > 1 && kk > ms::kLargeKMax))) any_exact = true;
+    else if (!((nucleus || large_k) && fits)) any_other = true;
     return MI355X_OK;
   };
   if (per_row_params) {
@@ -371,10 +375,12 @@ int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const 
   a.chunk_max = ctx->chunk_max;
   a.chunk_next = ctx->chunk_next;
   a.big = ctx->big;
+  a.big2 = ctx->big2;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
   a.poll_limit = ctx->poll_limit;
   a.row_done = ctx->row_done;
+  a.exact_kernel = any_exact ? 1 : 0;
   // a caller that bounds the number of allowed ids per row lets the sparse-mask kernel work alone
   if (xf && xf->mask && xf->mask_allowed_max > 0) {
     const int hist = a.xf.history_lens ? a.xf.history_stride : a.xf.history_len;

@@ -217,17 +217,17 @@ struct Xform {
   const int32_t* history_lens;  // per-row number of valid history ids, or null (history_len for every row)
   int min_length;               // with history_lens: only rows shorter than this get the EOS masking
   const uint32_t* ban;          // per-row bitmap (mask layout) of ids the no-repeat-n-gram rule bans, or null
-  __host__ __device__ bool active() const { return mask || use_penalty() || n_eos > 0; }
+  __host__ __device__ __forceinline__ bool active() const { return mask || use_penalty() || n_eos > 0; }
   // true when elements must be tested against the row's history: a penalty to apply or banned ids to
   // look up (a banned id always occurs in the history; a penalty of 1.0f leaves a value unchanged)
-  __host__ __device__ bool use_penalty() const {
+  __host__ __device__ __forceinline__ bool use_penalty() const {
     return history && (history_lens || history_len > 0) && (penalty != 1.0f || ban);
   }
-  __device__ int hist_len(int row) const { return history_lens ? history_lens[row] : history_len; }
-  __device__ int eos_count(int row) const {
+  __device__ __forceinline__ int hist_len(int row) const { return history_lens ? history_lens[row] : history_len; }
+  __device__ __forceinline__ int eos_count(int row) const {
     return (history_lens && min_length > 0 && history_lens[row] >= min_length) ? 0 : n_eos;
   }
-  __device__ const uint32_t* ban_row(int row, int vocab) const {
+  __device__ __forceinline__ const uint32_t* ban_row(int row, int vocab) const {
     return ban ? ban + static_cast<size_t>(row) * ((vocab - 1) / 32 + 1) : nullptr;
   }
 };

@@ -63,6 +63,7 @@ struct SampleArgs {
   uint32_t* chunk_max;    // [rows][chunks]
   u64* chunk_next;        // [rows][chunks]
   u64* big;               // [rows][big_stride]
+  u64* big2;              // [rows][big_stride] second buffer of the exact path's radix sort, or null
   size_t big_stride;
   uint32_t* fallback_rows;  // [0] cumulative count (modulo 2^32) of rows finished by the general path; [1] non-zero once a wait gave up
   int poll_limit;           // polls a finishing workgroup waits for another workgroup's list
@@ -72,6 +73,7 @@ struct SampleArgs {
   uint32_t* row_done;       // [rows] or null: nucleus rows under a grammar mask that the sparse-mask kernel finished
   int sparse_only;          // the sparse-mask kernel is the only one launched for nucleus rows: a row it cannot
                             // finish goes to the exact path inside it
+  int exact_kernel;         // rows whose parameters alone send them to the exact path have a kernel of their own
 };
 
 struct ArgmaxArgs {
@@ -172,7 +174,8 @@ extern "C" {
 hipError_t ms_sample_init();
 // `table`, when not null, holds the parameters of rows 0 .. a->rows-1 (a->rows <= kInlineParamRows).
 // any_nucleus / any_large_k / any_other: some row may be in nucleus mode / a top-k row with
-// 64 < k <= kLargeKMax / in another mode (each mode has kernels of its own).
+// 64 < k <= kLargeKMax / in another mode (each mode has kernels of its own); a->exact_kernel: some row's
+// parameters send it to the exact path.
 hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_other, bool any_nucleus,
                             bool any_large_k, hipStream_t stream);
 hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipStream_t stream);

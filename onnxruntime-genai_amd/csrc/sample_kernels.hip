@@ -153,6 +153,210 @@ __device__ __forceinline__ void tiled_sort_desc(u64* g, int n2, u64* lds) {
   }
 }
 
+// Sorts n distinct keys in global memory, descending, by a block of kFinishBlock threads that has kFinishLds
+// bytes of LDS, with a second global buffer `alt` of n keys: a most-significant-digit radix sort with
+// kRadixDigits digits.  The first level's digit is linear in the score between the row's largest and smallest
+// ordinary value (everything at or below lowest() and every NaN lands in the last digit), which spreads a
+// smooth distribution evenly; a refinement level's digit is linear in the 64-bit key between the largest and
+// smallest key of its range.  Per level: one pass counts the keys per digit, one scatters them into `alt`
+// digit by digit, then runs of consecutive digits that fit the LDS tile are loaded, every key finds its rank
+// among the keys of its digit by comparing, and goes to its final place.  A digit of more than kRankCap keys
+// goes back unsorted and is refined over its own, narrower key range.  Every key moves through memory three
+// times per level (the seventeen levels of a sorting network over a 128K row move it forty times).  All
+// inline: an out-of-line call in here makes the calling kernels use scratch memory.  Returns false, with
+// `keys` some permutation of its input, when more ranges need refinement than the list holds.
+constexpr int kRadixDigits = 16384;
+constexpr int kRadixTile = static_cast<int>(kFinishLds / sizeof(u64)) - (kRadixDigits + 2) / 2;  // keys of a run
+constexpr int kRankCap = 512;
+constexpr int kRadixStack = 32;
+static_assert(kRadixTile * sizeof(u64) >= kRadixDigits * sizeof(uint32_t), "the scatter cursors use the tile");
+
+// Runs BODY with K = SRC[I] for I in [0, CNT), eight loads per thread in flight.  A macro: closures that capture
+// the loop's state by reference end up in scratch memory here.
+#define MS_FOR_KEYS(SRC, CNT, K, I, BODY)                                                                   \
+  for (uint32_t i0_ = threadIdx.x; i0_ < (CNT); i0_ += 8 * kFinishBlock) {                                  \
+    u64 kb_[8];                                                                                             \
+    _Pragma("unroll") for (int u_ = 0; u_ < 8; ++u_)                                                        \
+        kb_[u_] = i0_ + u_ * kFinishBlock < (CNT) ? (SRC)[i0_ + u_ * kFinishBlock] : 0;                     \
+    _Pragma("unroll") for (int u_ = 0; u_ < 8; ++u_) {                                                      \
+      if (i0_ + u_ * kFinishBlock < (CNT)) {                                                                \
+        const u64 K = kb_[u_];                                                                              \
+        const uint32_t I = i0_ + u_ * kFinishBlock;                                                         \
+        BODY                                                                                                \
+      }                                                                                                     \
+    }                                                                                                       \
+  }
+
+__device__ __forceinline__ bool radix_rank_sort_desc(u64* keys, u64* alt, int n, u64* lds, uint32_t* red32, u64* red64) {
+  __shared__ uint32_t stack_pos[kRadixStack], stack_cnt[kRadixStack];
+  __shared__ int stack_n, failed;
+  const int tid = threadIdx.x;
+  uint32_t* const hist = reinterpret_cast<uint32_t*>(lds);  // kRadixDigits + 1 running totals
+  u64* const tile = lds + (kRadixDigits + 2) / 2;
+  uint32_t* const cursor = reinterpret_cast<uint32_t*>(tile);  // while a range is scattered
+  if (tid == 0) {
+    stack_n = 1;
+    stack_pos[0] = 0u;
+    stack_cnt[0] = static_cast<uint32_t>(n);
+    failed = 0;
+  }
+  for (int level = 0; level < 64 * kRadixStack; ++level) {
+    __syncthreads();
+    const int sn = stack_n;
+    if (sn == 0 || failed) break;
+    const uint32_t pos = stack_pos[sn - 1], cnt = stack_cnt[sn - 1];
+    __syncthreads();
+    if (tid == 0) stack_n = sn - 1;
+    u64* const src = keys + pos;
+    u64* const dst = alt + pos;
+    // the range of the keys, and of the ordinary scores among them
+    const uint32_t ordinary = order_key(-1e30f);
+    u64 kmin = ~0ull, kmax = 0ull;
+    uint32_t omin = 0xffffffffu;
+    MS_FOR_KEYS(src, cnt, k, i, {
+      (void)i;
+      kmin = k < kmin ? k : kmin;
+      kmax = k > kmax ? k : kmax;
+      const uint32_t o = key64_okey(k);
+      omin = (o > ordinary && o < omin) ? o : omin;
+    })
+    kmax = block_max<u64>(kmax, red64);
+    kmin = ~block_max<u64>(~kmin, red64);
+    omin = ~block_max<uint32_t>(~omin, red32);
+    const u64 span = kmax - kmin;
+    if (span == 0ull && cnt > 1u) {  // equal keys cannot be told apart: not a row of (score, id) keys
+      if (tid == 0) failed = 1;
+      continue;
+    }
+    const float fmax = key_to_float(key64_okey(kmax));
+    const float fmin = key_to_float(omin);
+    const float fspan = fmax - fmin;
+    const bool by_score = level == 0 && fmax < 3.0e38f && omin != 0xffffffffu && fspan > 0.0f && fspan < 3.0e38f;
+    const float scale = by_score ? static_cast<float>(kRadixDigits) / fspan : 0.0f;
+    const int bits = span != 0ull ? 64 - __clzll(span) : 0;
+    const int shift = bits > 14 ? bits - 14 : 0;  // (kmax - k) >> shift < kRadixDigits
+    static_assert(kRadixDigits == 1 << 14, "the shift above");
+    auto digit = [=](u64 k) -> uint32_t {
+      if (by_score) {
+        float bf = (fmax - key_to_float(key64_okey(k))) * scale;
+        bf = bf < static_cast<float>(kRadixDigits - 1) ? bf : static_cast<float>(kRadixDigits - 1);  // also NaN-safe
+        return bf > 0.0f ? static_cast<uint32_t>(bf) : 0u;
+      }
+      return static_cast<uint32_t>((kmax - k) >> shift);
+    };
+    for (int b = tid; b <= kRadixDigits; b += kFinishBlock) hist[b] = 0u;
+    __syncthreads();
+    const bool one_digit = cnt <= static_cast<uint32_t>(kRankCap);
+    if (one_digit) {
+      if (tid == 0) hist[0] = cnt;  // one digit holds the whole range
+    } else {
+      MS_FOR_KEYS(src, cnt, k, i, {
+        (void)i;
+        atomicAdd(&hist[digit(k)], 1u);
+      })
+    }
+    __syncthreads();
+    {  // exclusive scan of the digit counts: wave w owns kPer * 64 consecutive digits, 64 at a time; oversize
+       // digits join the list
+      constexpr int kPer = kRadixDigits / kFinishBlock;
+      const int lane = tid & 63, wave = tid >> 6;
+      uint32_t own = 0u;
+#pragma unroll 4
+      for (int i = 0; i < kPer; ++i) own += hist[(wave * kPer + i) * 64 + lane];
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) own += __shfl_xor(own, d, 64);
+      if (lane == 0) red32[wave] = own;
+      __syncthreads();
+      uint32_t run = 0u;
+      for (int w = 0; w < wave; ++w) run += red32[w];
+#pragma unroll 2
+      for (int i = 0; i < kPer; ++i) {
+        const int d0 = (wave * kPer + i) * 64 + lane;
+        const uint32_t c = hist[d0];
+        uint32_t inc = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const uint32_t y = __shfl_up(inc, d, 64);
+          if (lane >= d) inc += y;
+        }
+        const uint32_t base = run + inc - c;
+        hist[d0] = base;
+        cursor[d0] = base;
+        if (c > static_cast<uint32_t>(kRankCap)) {
+          const int at = atomicAdd(&stack_n, 1);
+          if (at < kRadixStack) {
+            stack_pos[at] = pos + base;
+            stack_cnt[at] = c;
+          } else {
+            failed = 1;
+          }
+        }
+        run += __shfl(inc, 63, 64);
+      }
+      if (tid == kFinishBlock - 1) hist[kRadixDigits] = run;
+    }
+    __syncthreads();
+    if (failed) break;  // nothing has moved yet
+    MS_FOR_KEYS(src, cnt, k, i, { dst[one_digit ? i : atomicAdd(&cursor[digit(k)], 1u)] = k; })
+    __syncthreads();
+    int b0 = 0;
+    while (b0 < kRadixDigits) {
+      const uint32_t base = hist[b0];
+      int lo = b0, hi = kRadixDigits;  // the last digit boundary up to which the keys from b0 on fit the tile
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (hist[mid] - base <= static_cast<uint32_t>(kRadixTile)) lo = mid;
+        else hi = mid - 1;
+      }
+      if (lo == b0) {  // a digit larger than the tile: back unsorted (it is on the list)
+        const uint32_t c = hist[b0 + 1] - base;
+        MS_FOR_KEYS(dst + base, c, k, i, { src[base + i] = k; })
+        b0 += 1;
+        continue;
+      }
+      const uint32_t c = hist[lo] - base;
+      if (c != 0u) {
+        MS_FOR_KEYS(dst + base, c, k, i, { tile[i] = k; })
+        __syncthreads();
+        for (uint32_t i = tid; i < c; i += kFinishBlock) {
+          const u64 k = tile[i];
+          const uint32_t d = one_digit ? 0u : digit(k);
+          const uint32_t first = hist[d], last = hist[d + 1];
+          uint32_t at = base + i;  // an oversize digit stays where it is
+          if (last - first <= static_cast<uint32_t>(kRankCap)) {
+            uint32_t rank = 0u, j = first - base;
+            const uint32_t end = last - base;
+            for (; j + 4 <= end; j += 4) {  // four independent reads in flight
+              const u64 x0 = tile[j], x1 = tile[j + 1], x2 = tile[j + 2], x3 = tile[j + 3];
+              rank += (x0 > k ? 1u : 0u) + (x1 > k ? 1u : 0u) + (x2 > k ? 1u : 0u) + (x3 > k ? 1u : 0u);
+            }
+            for (; j < end; ++j) rank += tile[j] > k ? 1u : 0u;
+            at = first + rank;
+          }
+          src[at] = k;
+        }
+        __syncthreads();
+      }
+      b0 = lo;
+    }
+  }
+  __syncthreads();
+  return failed == 0;
+}
+
+// The sort of the exact path in kernels that have the finish kernels' LDS: the radix sort above, else the network.
+struct SortWithTile {
+  u64* alt;
+  u64* tile;  // the kernel's dynamic LDS (kFinishLds bytes)
+  uint32_t* red32;
+  u64* red64;
+  __device__ __forceinline__ void operator()(u64* keys, int n2, int n_real) const {
+    if (alt != nullptr && radix_rank_sort_desc(keys, alt, n_real, tile, red32, red64)) return;
+    if (n2 >= 2 * kNucleusCap) tiled_sort_desc(keys, n2, tile);
+    else block_sort_desc(keys, n2);
+  }
+};
+
 // The tail shared by the finish kernels: lds_keys[0 .. n_c) hold a row's candidates as key64s in any order,
 // best_below (0: none) is the best element of the row that is not among them.  Sorts them together in LDS,
 // caches the exponentials and runs the exact epilogue.  With cut_at_best_below the candidates that rank
@@ -420,11 +624,8 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   }
   if (!ok) {
     __syncthreads();
-    u64* const tile = lds_keys;
-    general_row<AnyDtype>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, big_row, seqsh, [=](u64* keys, int n2, int n_real) {
-      if (n2 >= 2 * kNucleusCap) tiled_sort_desc(keys, n2, tile);
-      else block_sort_desc(keys, n2);
-    });
+    general_row<AnyDtype>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, big_row, seqsh,
+                          SortWithTile{a.big2 ? a.big2 + static_cast<size_t>(row) * a.big_stride : nullptr, lds_keys, red32, red64});
   }
 }
 
@@ -644,13 +845,13 @@ __device__ __forceinline__ void nucleus_sparse_entry(const SampleArgs& a) {
   if (done == 0 && a.sparse_only) {  // no dense kernels follow: the exact path, here
     extern __shared__ u64 lds_keys[];
     __shared__ SeqShared exact_sh;
+    __shared__ uint32_t exact_red32[16];
+    __shared__ u64 exact_red64[16];
     __syncthreads();
-    u64* const tile = lds_keys;
     general_row<AnyDtype>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), row_params<INLINE>(a, row),
-                          a.big + static_cast<size_t>(row) * a.big_stride, exact_sh, [=](u64* keys, int n2, int) {
-                            if (n2 >= 2 * kNucleusCap) tiled_sort_desc(keys, n2, tile);
-                            else block_sort_desc(keys, n2);
-                          });
+                          a.big + static_cast<size_t>(row) * a.big_stride, exact_sh,
+                          SortWithTile{a.big2 ? a.big2 + static_cast<size_t>(row) * a.big_stride : nullptr, lds_keys, exact_red32,
+                                       exact_red64});
     done = 1;
   }
   if (threadIdx.x == 0) a.row_done[row] = static_cast<uint32_t>(done);
@@ -660,6 +861,25 @@ __global__ __launch_bounds__(kFinishBlock) void nucleus_sparse_kernel(const Samp
 __global__ __launch_bounds__(kFinishBlock) void nucleus_sparse_rows_kernel(const SampleArgs a, const InlineParams) {
   nucleus_sparse_entry<true>(a);
 }
+
+// Rows whose parameters alone put them on the exact path (k above kLargeKMax, more chunks than a finishing
+// workgroup ranks): one workgroup per row with the finish kernels' LDS, so that the row is sorted by the radix
+// sort instead of a sorting network in global memory.
+template <bool INLINE>
+__device__ __forceinline__ void exact_rows_body(const SampleArgs& a) {
+  extern __shared__ u64 lds_keys[];
+  __shared__ SeqShared seqsh;
+  __shared__ uint32_t red32[16];
+  __shared__ u64 red64[16];
+  const int row = blockIdx.x;
+  const mi355x_sample_params prm = row_params<INLINE>(a, row);
+  if (row_mode(prm, a.vocab, a.chunks) != kModeGeneral) return;
+  general_row<AnyDtype>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, a.big + static_cast<size_t>(row) * a.big_stride,
+                        seqsh,
+                        SortWithTile{a.big2 ? a.big2 + static_cast<size_t>(row) * a.big_stride : nullptr, lds_keys, red32, red64});
+}
+__global__ __launch_bounds__(kFinishBlock) void exact_rows_kernel(const SampleArgs a) { exact_rows_body<false>(a); }
+__global__ __launch_bounds__(kFinishBlock) void exact_rows_rows_kernel(const SampleArgs a, const InlineParams) { exact_rows_body<true>(a); }
 
 }  // namespace ms
 
@@ -696,6 +916,12 @@ extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::Inline
     if (table) hipLaunchKernelGGL(ms::largek_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
     else hipLaunchKernelGGL(ms::largek_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
     e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  if (a->exact_kernel) {
+    if (table) hipLaunchKernelGGL(ms::exact_rows_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
+    else hipLaunchKernelGGL(ms::exact_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
+    e = hipGetLastError();
   }
   return e;
 }
@@ -706,7 +932,9 @@ extern "C" hipError_t ms_sample_init() {
                           reinterpret_cast<const void*>(ms::largek_finish_kernel),
                           reinterpret_cast<const void*>(ms::largek_finish_rows_kernel),
                           reinterpret_cast<const void*>(ms::nucleus_sparse_kernel),
-                          reinterpret_cast<const void*>(ms::nucleus_sparse_rows_kernel)};
+                          reinterpret_cast<const void*>(ms::nucleus_sparse_rows_kernel),
+                          reinterpret_cast<const void*>(ms::exact_rows_kernel),
+                          reinterpret_cast<const void*>(ms::exact_rows_rows_kernel)};
   for (const void* f : finish) {
     const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, ms::kFinishLds);
     if (e != hipSuccess) return e;

@@ -124,14 +124,28 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const 
   const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * ((V - 1) / 32 + 1) : nullptr;
   const int n_eos = a.xf.eos_count(row);
   const uint32_t* ban_row = a.xf.ban_row(row, V);
-  for (int i = threadIdx.x; i < n2; i += blockDim.x) {
-    u64 k = 0;
-    if (i < V) {
-      const float x = xform_value(lrow[i], a.xf.penalty, a.xf.eos, i, has_mask ? mrow[i >> 5] : 0u, has_mask, false, n_eos, ban_row);
-      k = make_key64(order_key(x), static_cast<uint32_t>(i));
-      if (i == 0 && x != x && a.emit_topk == kEmitArgmax) k = ~0ull;  // ArgMax starts from id 0 and nothing compares above a NaN
+  constexpr int kLoads = 4;  // loads a thread has in flight
+  for (int i0 = threadIdx.x; i0 < n2; i0 += kLoads * blockDim.x) {
+    float raw[kLoads];
+    uint32_t mw[kLoads];
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const int i = i0 + u * blockDim.x;
+      raw[u] = i < V ? lrow[i] : 0.0f;
+      mw[u] = (has_mask && i < V) ? mrow[i >> 5] : 0u;
     }
-    scratch[i] = k;
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const int i = i0 + u * blockDim.x;
+      if (i >= n2) continue;
+      u64 k = 0;
+      if (i < V) {
+        const float x = xform_value(raw[u], a.xf.penalty, a.xf.eos, i, mw[u], has_mask, false, n_eos, ban_row);
+        k = make_key64(order_key(x), static_cast<uint32_t>(i));
+        if (i == 0 && x != x && a.emit_topk == kEmitArgmax) k = ~0ull;  // ArgMax starts from id 0 and nothing compares above a NaN
+      }
+      scratch[i] = k;
+    }
   }
   __syncthreads();
   if (a.xf.use_penalty()) {
@@ -176,6 +190,7 @@ __device__ __forceinline__ int row_mode(mi355x_sample_params prm, int vocab, int
     const int kk = prm.k < vocab ? prm.k : vocab;
     return kk <= 64 ? kModeTopkSmall : (kk <= kLargeKMax ? kModeTopkLarge : kModeGeneral);
   }
+  if (!(prm.p < 1.0f)) return kModeGeneral;  // sampling from the whole vocabulary: every element is a candidate
   return kModeNucleus;
 }
 
@@ -974,7 +989,7 @@ __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
   } else {
     if (mode == kModeNucleus || mode == kModeTopkLarge) return;
     if (mode == kModeGeneral) {
-      if (chunk != 0) return;
+      if (chunk != 0 || a.exact_kernel) return;  // exact_kernel: the exact-rows kernel sorts such rows much faster
     } else if (!stream_row<InT, false, XFORM>(a, row, row0, chunk, prm, sm)) {
       return;
     }

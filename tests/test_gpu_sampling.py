@@ -759,3 +759,63 @@ def test_nucleus_rows_under_sparse_and_dense_masks(ctx, orc, vocab, frac, penalt
             assert np.array_equal(ki[r, :n], idx[:n]), (promise, r)
             assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), (promise, r)
             assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (promise, r)
+
+
+def exact_path_rows(name, rng, vocab):
+    if name == "gaussian":
+        return (rng.standard_normal((2, vocab)) * 3).astype(np.float32)
+    if name == "constant":
+        return np.full((2, vocab), 1.5, np.float32)
+    if name == "rounded":  # thirteen distinct scores: every digit of the sort's first level overflows
+        return np.round(rng.standard_normal((2, vocab)) * 2).astype(np.float32)
+    if name == "peaked":  # nearly every score inside a sliver of the row's range
+        x = (5.0 + rng.random((2, vocab)) * 1e-3).astype(np.float32)
+        x[:, rng.integers(0, vocab, 6)] = [100.0, -100.0, 50.0, 7.0, 5.0005, -3.0]
+        return x
+    if name == "mostly_lowest":  # what a grammar mask leaves behind
+        x = (rng.standard_normal((2, vocab)) * 3).astype(np.float32)
+        x[rng.random((2, vocab)) < 0.95] = LOWEST
+        return x
+    if name == "specials":
+        x = (rng.standard_normal((2, vocab)) * 3).astype(np.float32)
+        x[0, rng.integers(0, vocab, 9)] = [np.inf, -np.inf, np.nan, -np.inf, np.inf, 0.0, -0.0, LOWEST, np.nan]
+        x[1, rng.integers(0, vocab, 4)] = [-np.inf, -np.inf, LOWEST, LOWEST]
+        return x
+    raise KeyError(name)
+
+
+@pytest.mark.parametrize("vocab", [65, 511, 513, 4100, 10239, 10241, 16384, 70001, 128256, 201088])
+@pytest.mark.parametrize("name", ["gaussian", "constant", "rounded", "peaked", "mostly_lowest", "specials"])
+def test_exact_path_orders_whole_rows(ctx, orc, name, vocab):
+    """k above the candidate-list bound and sampling from the whole vocabulary (k = 0, p = 1) take the exact
+    path, which sorts the entire row; the kept ids are that order, checked to the last element."""
+    if vocab > 70001 and name in ("constant", "peaked"):
+        pytest.skip("covered at the smaller sizes")
+    say("exact path", name, vocab)
+    rng = np.random.default_rng(vocab + len(name))
+    x = exact_path_rows(name, rng, vocab)
+    u = rng.random(2)
+    before = ctx.fallback_rows()
+    sample_and_check(ctx, orc, x, u, vocab, 0.0, 0.9, cap=vocab)
+    sample_and_check(ctx, orc, x, u, 0, 1.0, 1.1, cap=vocab)
+    if vocab > 2048:
+        sample_and_check(ctx, orc, x, u, 2049, 0.97, 1.0, cap=2049)
+    # k <= 2048 goes through the candidate lists, which hand rows with ties or NaNs at their bound to the exact path too
+    assert ctx.fallback_rows() - before >= (6 if vocab > 2048 else 2)
+
+
+def test_exact_path_sixteen_bit_rows(ctx, orc):
+    """fp16 rows hold a few thousand distinct scores: long runs of ties through the exact path's sort."""
+    say("exact path fp16")
+    rng = np.random.default_rng(16)
+    x16 = (rng.standard_normal((2, 128256)) * 3).astype(np.float16)
+    u = rng.random(2)
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x16).cuda(), torch.from_numpy(u).cuda(), k=0, p=1.0, temperature=1.0,
+                                 kept_capacity=128256)
+    x = x16.astype(np.float32)
+    for r in range(2):
+        idx, probs = orc.sampled_categorical(x[r], 0, 1.0, 1.0)
+        assert kc[r].item() == len(idx)
+        assert np.array_equal(ki[r, :len(idx)].cpu().numpy(), idx), r
+        assert np.array_equal(bits(kp[r, :len(idx)].cpu().numpy()), bits(probs)), r
+        assert tok[r].item() == idx[orc.discrete_draw(probs, u[r])], r
