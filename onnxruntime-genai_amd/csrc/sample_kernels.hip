@@ -72,15 +72,22 @@ __device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n,
   }
   if (t == kFinishBlock - 1) start[kSortBuckets] = base;
   __syncthreads();
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-    if (r * kFinishBlock + t < n) keys[start[info[r] >> 8] + (info[r] & 255u)] = k[r];
-  __syncthreads();
+  // info becomes: where the bucket starts | keys in the bucket << 16 (a bucket holds at most kBucketCap keys)
+  static_assert(kBucketCap < 256 && kNucleusCap <= 65536, "the packing of info");
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (r * kFinishBlock + t < n) {
       const uint32_t b = info[r] >> 8;
-      const uint32_t lo = start[b], hi = start[b + 1];
+      const uint32_t lo = start[b];
+      keys[lo + (info[r] & 255u)] = k[r];
+      info[r] = lo | ((start[b + 1] - lo) << 16);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (r * kFinishBlock + t < n) {
+      const uint32_t lo = info[r] & 0xffffu, hi = lo + (info[r] >> 16);
       uint32_t rank = 0u;
       for (uint32_t j = lo; j < hi; ++j) rank += keys[j] > k[r] ? 1u : 0u;
       info[r] = lo + rank;
