@@ -423,7 +423,7 @@ __device__ __forceinline__ void mask_registers(float (&v)[kSChunk / kSBlock], co
 
 // Streaming pass of one (row, chunk) of a top-k<=64 or nucleus row.  Returns true when this workgroup
 // must run the general path for the row (it was the last to arrive and the fast path declined).
-template <typename InT, bool NUCLEUS, bool XFORM, bool LARGEK = false>
+template <typename InT, bool NUCLEUS, bool XFORM, bool LARGEK = false, bool ARGMAX = false>
 __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const void* row0, int chunk,
                                            mi355x_sample_params prm, FusedShared& sm) {
   constexpr int kSBlock = NUCLEUS ? kNucleusBlock : kTopkBlock;  // threads of this workgroup
@@ -742,10 +742,69 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     return false;
   }
 
-  // ---- top-k, k <= 64 ---------------------------------------------------------------------------
   // A finishing workgroup that once gave up waiting may have left published lists behind; from then on
   // (the flag word next to the fallback counter) every row takes the exact path, which reads no such state.
   if (poison != 0u) return chunk == n_chunks - 1;
+  if constexpr (ARGMAX) {
+    // ---- argmax ---------------------------------------------------------------------------------
+    // ArgMax (src/search.h:9-29) keeps id 0 unless a later value compares greater: the largest value, the
+    // lowest id among equals, NaNs never win, and a NaN at id 0 wins outright.  A thread's candidate is
+    // the first of its elements that equals its maximum; the key (order key, ~id) orders candidates the
+    // same way, so the row's answer is the largest key: no bound, no lists, no sort.  Every chunk
+    // publishes its best key in the first entry of its candidate slots; the workgroup of the row's last
+    // chunk polls for them, as the top-k rows do for their lists.
+    uint32_t best_idx = 0xffffffffu;
+#pragma unroll
+    for (int j = kSVec - 1; j >= 0; --j) {
+      if (qm[j] == fm) {
+#pragma unroll
+        for (int c = 3; c >= 0; --c)
+          if (v[j * 4 + c] == fm) best_idx = static_cast<uint32_t>(elem_index<kSBlock, VEC>(chunk, j, c));
+      }
+    }
+    for (uint32_t i = tid; i < n_extra; i += kSBlock)
+      if (sm.extra_val[i] == fm && sm.extra_idx[i] < best_idx) best_idx = sm.extra_idx[i];
+    u64 key = best_idx != 0xffffffffu ? make_key64(order_key(fm), best_idx) : 0;
+    key = wave_max(key);
+    if (lane == 0) sm.list_hi[wave] = key;
+    lds_barrier();
+    const bool finisher = chunk == n_chunks - 1;
+    if (wave != 0 && !finisher) return false;
+    if (wave == 0) {
+      key = lane < kSWaves ? sm.list_hi[lane] : 0;
+      key = wave_max(key);
+      if (chunk == 0 && sm.nan0 != 0u) key = ~0ull;
+      const size_t ci = static_cast<size_t>(row) * n_chunks + chunk;
+      const u64 slot = extra_overflow ? kSlotOverflow : (key != 0 ? key : kSlotEmpty);
+      if (!finisher) {
+        if (lane == 0) store_coherent(&cand_small[ci * kSmallCap], slot);
+        return false;
+      }
+      u64* seg = cand_small + static_cast<size_t>(row) * n_chunks * kSmallCap;
+      u64 got = lane < n_chunks - 1 ? 0 : (lane == n_chunks - 1 ? slot : kSlotEmpty);
+      int spins = 0;
+      while (true) {
+        if (got == 0) got = load_coherent(&seg[lane * kSmallCap]);
+        if (__ballot(got == 0) == 0ull) break;
+        if (spins++ >= poll_limit) {
+          if (lane == 0) atomicOr(a.fallback_rows + 1, 1u);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      if (lane < n_chunks - 1 && got != 0) store_coherent(&seg[lane * kSmallCap], 0);  // for the next launch
+      const bool bad = __ballot(got == 0 || got == kSlotOverflow) != 0ull;
+      const u64 best = wave_max(got <= kSlotOverflow ? 0 : got);
+      const bool found = !bad && best != 0;  // otherwise the exact path decides (an overflowing history, a wait that gave up)
+      if (lane == 0) {
+        sm.flag = found ? 1u : 0u;
+        if (found) outputs.token[0] = static_cast<int32_t>(key64_index(best));
+      }
+    }
+    __syncthreads();
+    return sm.flag == 0u;
+  }
+  // ---- top-k, k <= 64 ---------------------------------------------------------------------------
   const int kk = prm.k < V ? prm.k : V;
   int n_valid = V - chunk * kSChunk;
   if (n_valid > kSChunk) n_valid = kSChunk;
@@ -972,7 +1031,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
 // Rows in nucleus mode and all other rows are streamed by kernels of their own (a launch may need
 // both): each kernel holds the code of its mode only, and a change to one path leaves the machine
 // code of the other as it was.
-template <typename InT, bool INLINE, bool NUCLEUS, bool XFORM, bool LARGEK = false>
+template <typename InT, bool INLINE, bool NUCLEUS, bool XFORM, bool LARGEK = false, bool ARGMAX = false>
 __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
   const int row = blockIdx.y, chunk = blockIdx.x;
   __shared__ FusedShared sm;
@@ -990,7 +1049,7 @@ __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
     if (mode == kModeNucleus || mode == kModeTopkLarge) return;
     if (mode == kModeGeneral) {
       if (chunk != 0 || a.exact_kernel) return;  // exact_kernel: the exact-rows kernel sorts such rows much faster
-    } else if (!stream_row<InT, false, XFORM>(a, row, row0, chunk, prm, sm)) {
+    } else if (!stream_row<InT, false, XFORM, false, ARGMAX>(a, row, row0, chunk, prm, sm)) {
       return;
     }
     // Rows the fast paths decline end here, in the exact general path (a single inlined call site keeps
@@ -1012,8 +1071,9 @@ __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
     sample_fused_body<InT, true, NUCLEUS, XFORM, LARGEK>(a);                                                             \
   }
 
-// Defines the twelve streaming kernels of one element type and ms_launch_stream##SUFFIX, which launches the one
-// a call needs: which = 0 rows of every other mode, 1 nucleus rows, 2 rows with 64 < k <= kLargeKMax.
+// Defines the streaming kernels of one element type (twelve for sampling, two for argmax) and
+// ms_launch_stream##SUFFIX, which launches the one a call needs: which = 0 rows of every other mode (argmax
+// calls: the argmax kernels), 1 nucleus rows, 2 rows with 64 < k <= kLargeKMax.
 #define MS_STREAM_KERNELS(SUFFIX, InT)                                                                                   \
   namespace ms {                                                                                                         \
   MS_STREAM_KERNEL(sample_fused, SUFFIX, InT, false, false, false)                                                       \
@@ -1022,12 +1082,21 @@ __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
   MS_STREAM_KERNEL(nucleus_stream_xf, SUFFIX, InT, true, true, false)                                                    \
   MS_STREAM_KERNEL(largek_stream, SUFFIX, InT, true, false, true)                                                        \
   MS_STREAM_KERNEL(largek_stream_xf, SUFFIX, InT, true, true, true)                                                      \
+  __global__ __launch_bounds__(kTopkBlock) void argmax_stream##SUFFIX##_kernel(const SampleArgs a) {                     \
+    sample_fused_body<InT, false, false, false, false, true>(a);                                                         \
+  }                                                                                                                      \
+  __global__ __launch_bounds__(kTopkBlock) void argmax_stream_xf##SUFFIX##_kernel(const SampleArgs a) {                  \
+    sample_fused_body<InT, false, false, true, false, true>(a);                                                          \
+  }                                                                                                                      \
   }                                                                                                                      \
   extern "C" hipError_t ms_launch_stream##SUFFIX(const ms::SampleArgs* a, const ms::InlineParams* table, int which,      \
                                                  hipStream_t stream) {                                                   \
     const dim3 grid(a->chunks, a->rows), block(which == 0 ? ms::kTopkBlock : ms::kNucleusBlock);                         \
     const bool xf = a->xf.active();                                                                                      \
-    if (table) {                                                                                                         \
+    if (which == 0 && a->emit_topk == ms::kEmitArgmax && !table) {                                                       \
+      hipLaunchKernelGGL(xf ? ms::argmax_stream_xf##SUFFIX##_kernel : ms::argmax_stream##SUFFIX##_kernel, grid, block, 0, \
+                         stream, *a);                                                                                    \
+    } else if (table) {                                                                                                         \
       auto* f = which == 0   ? (xf ? ms::sample_fused_xf##SUFFIX##_rows_kernel : ms::sample_fused##SUFFIX##_rows_kernel) \
                 : which == 1 ? (xf ? ms::nucleus_stream_xf##SUFFIX##_rows_kernel : ms::nucleus_stream##SUFFIX##_rows_kernel) \
                              : (xf ? ms::largek_stream_xf##SUFFIX##_rows_kernel : ms::largek_stream##SUFFIX##_rows_kernel); \
