@@ -11,10 +11,11 @@ import torch
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per step from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these same commands, scaled by a
-# known-size copy (profiles/beam_step_kernels_config3.md, profiles/nucleus_kernels_config5.md); counters
-# cannot be read from inside the process.  None where no counter run exists.
-MEASURED_TRAFFIC = {"c3": 6_222_000_000 + 82_000_000, "c5": 289_000_000}
-
+# known-size copy; counters cannot be read from inside the process, so these are offline profile constants.
+# c3: KV gather 6.22 GB + selection kernels 0.06 GB; c5: the one sparse-mask kernel.  None where no counter run exists.
+MEASURED_TRAFFIC = {"c3": 6_222_000_000 + 62_000_000, "c5": 204_000_000}
+TRAFFIC_SOURCE = {"c3": "offline profile constant: profiles/beam_step_kernels_config3.md",
+                  "c5": "offline profile constant: profiles/nucleus_sparse_kernel_config5.md"}
 
 def _timed(fn_step, K, W, graph=True):
     """Runs W warm-up steps, then K steps between two events; with graph=True the K steps are
@@ -56,6 +57,7 @@ def _line(args, metric, unit, value, ms_total, K, W, dtype, workload, extra, alg
         "config": dict({"workload": workload}, **extra),
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "traffic_source": TRAFFIC_SOURCE.get(args.workload),
                      "algorithmic_bytes_per_step": algo_bytes},
         "cpu_baseline": cpu,
     }
