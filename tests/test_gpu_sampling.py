@@ -23,7 +23,7 @@ def bits(a):
     return np.asarray(a, np.float32).view(np.uint32)
 
 
-@pytest.mark.parametrize("rows,vocab", [(1, 32064), (3, 33), (4, 8192), (2, 8193), (5, 50257), (64, 128256)])
+@pytest.mark.parametrize("rows,vocab", [(1, 32064), (3, 33), (4, 8192), (2, 8193), (5, 50257), (64, 128256), (3, 201088)])
 def test_argmax_matches_oracle(ctx, orc, rows, vocab):
     say("argmax", rows, vocab)
     rng = np.random.default_rng(rows * 1000 + vocab)
@@ -47,6 +47,51 @@ def test_argmax_special_values(ctx, orc):
     x[5, 999] = np.inf
     got = ctx.argmax(torch.from_numpy(x).cuda()).cpu().numpy()
     assert np.array_equal(got, orc.argmax_batch(x))
+
+
+@pytest.mark.parametrize("vocab", [40000, 131072, 201088])
+def test_argmax_special_values_across_chunks(ctx, orc, vocab):
+    """Rows of several 32768-id chunks: equal maxima in different chunks (the lowest id wins), a maximum in the last
+    partial chunk, NaN at id 0 (wins outright), NaN elsewhere (never wins), rows without a finite value."""
+    say("argmax special, chunks", vocab)
+    rng = np.random.default_rng(vocab)
+    x = (rng.standard_normal((10, vocab)) * 2).astype(np.float32)
+    x[0, [vocab - 1, 33000, 5]] = 50.0
+    x[1, [vocab - 1, 33000]] = 50.0
+    x[2, vocab - 1] = 50.0
+    x[3, 0] = np.nan
+    x[3, 35000] = 60.0
+    x[4, 35000] = np.nan
+    x[4, 36000] = np.nan
+    x[5, :] = -np.inf
+    x[6, :] = np.nan
+    x[7, :] = -np.inf
+    x[7, 39999] = LOWEST
+    x[8, :] = 3.0
+    x[9, :] = np.nan
+    x[9, 0] = 1.0
+    x[9, 39000] = 1.0
+    want = orc.argmax_batch(x)
+    assert np.array_equal(ctx.argmax(torch.from_numpy(x).cuda()).cpu().numpy(), want)
+    xf = pkg().LogitsXform(history=torch.from_numpy(np.tile(np.array([[5, 33000, 35000, 0]], np.int32), (10, 1))).cuda(),
+                           repetition_penalty=1.3)
+    proc = np.stack([orc.apply_repetition_penalty(x[r], np.array([5, 33000, 35000, 0], np.int32), 1.3) for r in range(10)])
+    assert np.array_equal(ctx.argmax(torch.from_numpy(x).cuda(), xf=xf).cpu().numpy(), orc.argmax_batch(proc))
+    with np.errstate(over="ignore"):  # lowest() becomes -inf in fp16
+        h = x.astype(np.float16)
+    assert np.array_equal(ctx.argmax(torch.from_numpy(h).cuda()).cpu().numpy(), orc.argmax_batch(orc.fp16_to_fp32(h)))
+
+
+def test_argmax_of_rows_longer_than_the_chunked_path_holds(orc):
+    """More than 16 chunks per row (vocabulary above 524288): the exact path answers; exactly 16: the chunked one."""
+    say("argmax very long rows")
+    rng = np.random.default_rng(77)
+    for vocab in (524288, 524289 + 4096):
+        ctx = pkg().SearchContext(2, vocab)
+        x = (rng.standard_normal((2, vocab)) * 2).astype(np.float32)
+        x[1, vocab - 1] = 40.0
+        assert np.array_equal(ctx.argmax(torch.from_numpy(x).cuda()).cpu().numpy(), orc.argmax_batch(x))
+        ctx.close()
 
 
 def test_argmax_fp16(ctx, orc):
