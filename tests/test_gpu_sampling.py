@@ -520,34 +520,48 @@ def test_sample_randomised_shapes_and_parameters(ctx, orc, seed):
         x = (np.round(x * 2) / 2).astype(np.float32)  # heavy ties
     if seed % 5 == 0:
         x[0, :] = 1.25  # a constant row
-    say("sample random", seed, rows, vocab, scale)
+    # the logits as fp32, fp16 or bf16 (the oracle sees the widened values)
+    kind = ("f32", "f16", "bf16")[seed % 7 % 3]
+    if kind == "f16":
+        with np.errstate(over="ignore"):
+            x_dev = torch.from_numpy(x.astype(np.float16)).cuda()
+        x = x_dev.float().cpu().numpy()
+    elif kind == "bf16":
+        x_dev = torch.from_numpy(x).to(torch.bfloat16).cuda()
+        x = x_dev.float().cpu().numpy()
+    else:
+        x_dev = torch.from_numpy(x).cuda()
+    say("sample random", seed, rows, vocab, scale, kind)
     xf, proc = None, x
     if seed % 4 in (1, 2):
         mask = make_mask(rng, rows, vocab, float(rng.choice([0.02, 0.5, 0.98])))
         hist = rng.integers(0, vocab, (rows, int(rng.integers(1, 200)))).astype(np.int32)
         pen = float(rng.choice([1.0, 1.3, 0.8]))
         eos = [int(rng.integers(0, vocab))]
+        allowed = int(np.unpackbits(mask.view(np.uint8)).reshape(rows, -1).sum(axis=1).max())
+        promise = int(rng.choice([0, allowed, 3]))  # none, the true bound, a broken promise (still exact)
         xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
-                               repetition_penalty=pen, eos_ids=eos, apply_min_length=bool(seed % 8 == 1))
+                               repetition_penalty=pen, eos_ids=eos, apply_min_length=bool(seed % 8 == 1),
+                               mask_allowed_max=promise)
         proc = orc.apply_mask(x, mask)
         proc = np.stack([orc.apply_repetition_penalty(orc.apply_min_length(proc[r], 0, 1 if seed % 8 == 1 else 0, eos),
                                                        hist[r], pen) for r in range(rows)])
     u = rng.random(rows)
 
     def params():
-        k = int(rng.choice([0, 1, 2, 5, 40, 50, 64, 65, 200, vocab, vocab + 7]))
+        k = int(rng.choice([0, 1, 2, 5, 40, 50, 64, 65, 200, 513, 2048, 2049, vocab, vocab + 7]))
         p = float(rng.choice([0.0, 0.1, 0.5, 0.9, 0.999, 1.0]))
         return k, p, float(rng.uniform(0.3, 2.0))
 
     if seed % 2:  # heterogeneous rows
         per_row = [params() for _ in range(rows)]
-        tok = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), per_row=per_row, xf=xf).cpu().numpy()
+        tok = ctx.sample(x_dev, torch.from_numpy(u).cuda(), per_row=per_row, xf=xf).cpu().numpy()
         for r, (k, p, t) in enumerate(per_row):
             assert tok[r] == orc.sample_row(proc[r], k, p, t, u[r]), (r, k, p, t)
     else:
         k, p, t = params()
         cap = 256
-        tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=k, p=p, temperature=t,
+        tok, kc, ki, kp = ctx.sample(x_dev, torch.from_numpy(u).cuda(), k=k, p=p, temperature=t,
                                      xf=xf, kept_capacity=cap)
         tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
         for r in range(rows):
