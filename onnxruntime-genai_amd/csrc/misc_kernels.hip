@@ -28,7 +28,11 @@ __global__ __launch_bounds__(1024) void softmax_kernel(float* scores, int64_t ro
     const float lse = em::logf_exact(sum);
 #pragma unroll 8
     for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-      const float s = (x[i] - max_score) * inv_temp;
+      // The maximum went through an order key, which holds +0 for either zero, while the reference subtracts the
+      // row's own first maximal element.  The sign of a zero difference only shows when lse is 0, that is when the
+      // maximum is a single element -- and that element minus itself is +0 -- so +0 is right wherever it matters.
+      const float d = x[i] - max_score;
+      const float s = (d == 0.0f ? 0.0f : d) * inv_temp;
       x[i] = s - lse;
     }
   } else {

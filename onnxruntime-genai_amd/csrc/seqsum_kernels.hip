@@ -350,7 +350,9 @@ __global__ __launch_bounds__(kSegBlock) void softmax_apply_kernel(float* scores,
     const int i = seg * kSegElems + j * kSegBlock + static_cast<int>(threadIdx.x);
     if (i < a.vocab) {
       if (LOG) {
-        x[i] = (x[i] - max_score) * a.inv_temp - lse;
+        // x - max is never -0 where it shows (see softmax_kernel): the maximum here lost the sign of its zero
+        const float d = x[i] - max_score;
+        x[i] = (d == 0.0f ? 0.0f : d) * a.inv_temp - lse;
       } else {
         const float ex = erow[i];
         x[i] = sum > 0.0f ? ex * inv_sum : ex;

@@ -66,6 +66,28 @@ def test_log_softmax_extreme_rows(ctx, orc):
         assert np.array_equal(bits(got[r]), bits(orc.log_softmax(x[r], 1.0))), r
 
 
+@pytest.mark.parametrize("vocab", [3, 5000, 20000, 70000])
+def test_softmax_rows_whose_maximum_is_a_signed_zero(ctx, orc, vocab):
+    """The reference subtracts the row's own first maximal element, -0.0 included: a single -0.0 maximum above
+    values whose exponentials vanish gives log-softmax +0.0, not -0.0; mixed zeros give -log(count)."""
+    say("softmax signed zeros", vocab)
+    x = np.full((6, vocab), -np.inf, np.float32)
+    x[0, 0] = -0.0
+    x[1, :] = -300.0
+    x[1, vocab // 2] = -0.0
+    x[2, 0], x[2, 1] = 0.0, -0.0
+    x[3, 0], x[3, 1] = -0.0, 0.0
+    x[4, :] = -0.0
+    x[5, :] = -300.0
+    x[5, vocab - 1] = 0.0
+    for t in (1.0, 0.05):
+        for log in (True, False):
+            got = ctx.softmax(torch.from_numpy(x.copy()).cuda(), t, log=log).cpu().numpy()
+            for r in range(6):
+                want = orc.log_softmax(x[r], t) if log else orc.softmax(x[r], t)
+                assert np.array_equal(bits(got[r]), bits(want)), (r, t, log)
+
+
 @pytest.mark.parametrize("batch,beams,vocab,dtype", [(2, 3, 1000, np.float32), (8, 4, 151936, np.float16),
                                                      (1, 16, 5000, np.float32), (3, 2, 2, np.float32),
                                                      (2, 4, 3000, np.float16)])
