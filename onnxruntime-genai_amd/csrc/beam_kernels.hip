@@ -399,16 +399,83 @@ __global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a) {
     j += dj;
     if (j >= m) j -= m;
   }
-  u64 last = ~0ull;
-  for (int j = 0; j < m; ++j) {
-    u64 best = 0ull;
+  // The m best keys, best first.  Every wave lists its keys that reach the m-th best of its 64 per-lane maxima (at
+  // least m of its keys do, so the wave's m best are among them; with fewer than m lanes holding keys, all keys), the
+  // four lists together usually hold fewer than 64 keys, and wave 0 sorts those.
+  __shared__ u64 hit[4][64];
+  __shared__ uint32_t hit_n[4];
+  __shared__ u64 wave_best[4 * kBeamMaxCand];
+  const int lane = tid & 63, wave = tid >> 6;
+  {
+    u64 lane_best = 0ull;
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      if (r < nr && key[r] < last && key[r] > best) best = key[r];
-    best = block_max<u64>(best, red64);
-    if (tid == 0) best_list[j] = best;
-    last = best;  // 0 once nothing is left: later rounds find nothing either
+      if (r < nr && key[r] > lane_best) lane_best = key[r];
+    const u64 tau = __shfl(wave_sort_desc_fast<u64>(lane_best), m - 1, 64);
+    uint32_t woff = 0u;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const bool cand = r < nr && key[r] != 0ull && key[r] >= tau;
+      const u64 bal = __ballot(cand);
+      if (bal == 0ull) continue;
+      if (cand) {
+        const uint32_t pos = woff + __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(bal >> 32),
+                                                              __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(bal), 0u));
+        if (pos < 64u) hit[wave][pos] = key[r];
+      }
+      woff += static_cast<uint32_t>(__popcll(bal));
+    }
+    if (lane == 0) hit_n[wave] = woff;
   }
+  __syncthreads();
+  const uint32_t n0 = hit_n[0], n1 = hit_n[1], n2 = hit_n[2], n3 = hit_n[3];
+  u64 last = ~0ull;
+  if (n0 + n1 + n2 + n3 <= 64u) {
+    if (wave == 0) {
+      const uint32_t p = static_cast<uint32_t>(lane);
+      u64 k = 0ull;
+      if (p < n0) k = hit[0][p];
+      else if (p < n0 + n1) k = hit[1][p - n0];
+      else if (p < n0 + n1 + n2) k = hit[2][p - n0 - n1];
+      else if (p < n0 + n1 + n2 + n3) k = hit[3][p - n0 - n1 - n2];
+      k = wave_sort_desc_fast<u64>(k);
+      if (lane < m) best_list[lane] = k;
+    }
+  } else {
+    // More than one wave's worth of listed keys (many beams, or ties at a bound): every wave extracts the m best of
+    // its own keys, each the largest key below the previous one, then wave 0 extracts the m best of the four lists.
+    for (int j = 0; j < m; ++j) {
+      u64 best = 0ull;
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (r < nr && key[r] < last && key[r] > best) best = key[r];
+      best = wave_max(best);
+      if (lane == 0) wave_best[wave * kBeamMaxCand + j] = best;
+      last = best;  // 0 once nothing is left: later rounds find nothing either
+    }
+    __syncthreads();
+    if (wave == 0) {
+      // entries j < m of the four lists: two per lane (4 m <= 128)
+      u64 mine[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int e = lane + 64 * h;
+        mine[h] = e < 4 * m ? wave_best[(e / m) * kBeamMaxCand + e % m] : 0ull;
+      }
+      last = ~0ull;
+      for (int j = 0; j < m; ++j) {
+        u64 best = 0ull;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          if (mine[h] < last && mine[h] > best) best = mine[h];
+        best = wave_max(best);
+        if (lane == 0) best_list[j] = best;
+        last = best;
+      }
+    }
+  }
+  __syncthreads();
+  last = best_list[m - 1];
   const uint32_t cut = key64_okey(last);
   const uint32_t reach = block_max<uint32_t>(full_reach, red);
   if (cut == 0u || reach >= cut) {
