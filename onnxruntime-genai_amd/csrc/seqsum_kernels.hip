@@ -63,13 +63,25 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_kernel(const SeqSumArgs 
   auto lds_tab = [=](uint32_t i) { return tab[i]; };
   float* erow = a.e + static_cast<size_t>(row) * a.e_stride;
   double part = 0.0;
+  // four consecutive exponentials per store (the row of exponentials starts 16-byte aligned and a thread's ids come
+  // in aligned groups of four); a group that crosses the end of the row is stored element by element
 #pragma unroll
-  for (int e = 0; e < kSegPer; ++e) {
-    const int idx = seg_index<InT>(seg, e);
-    if (idx < a.vocab) {
-      const float ex = em::expf_core((v[e] - max_score) * a.inv_temp, lds_tab);
-      erow[idx] = ex;
-      part += static_cast<double>(ex);
+  for (int e0 = 0; e0 < kSegPer; e0 += 4) {
+    const int idx = seg_index<InT>(seg, e0);
+    float ex[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      ex[c] = idx + c < a.vocab ? em::expf_core((v[e0 + c] - max_score) * a.inv_temp, lds_tab) : 0.0f;
+      part += static_cast<double>(ex[c]);
+    }
+    if (idx + 4 <= a.vocab) {
+      v4f q;
+      q.x = ex[0], q.y = ex[1], q.z = ex[2], q.w = ex[3];
+      *reinterpret_cast<v4f*>(erow + idx) = q;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (idx + c < a.vocab) erow[idx + c] = ex[c];
     }
   }
   part = wave_sum<double>(part);
