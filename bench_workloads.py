@@ -145,10 +145,10 @@ def c3(args, pkg, orc, orc_lib, dev):
     scorer = new_scorer()
 
     def select_step(i):
-        sc, tok, idx = ctx.beam_select(logits[i % pool], B, NB, scorer.next_scores)
-        scorer.step(sc, tok, idx)
+        scorer.search_step(logits[i % pool])  # BeamSearch_Cpu::SelectTop in one call: selection + scorer step
 
-    ms_sel = _timed(select_step, K, W, graph=False)  # the scorer step is not capturable
+    # launched eagerly, as a host loop does: the scorer's step takes the sequence length by value
+    ms_sel = _timed(select_step, K, W, graph=False)
     beam_idx = scorer.next_indices.clone()
     # ---- phase 2: KV gather ------------------------------------------------------------------------
     shape = (BB, 4, 2048, 128)

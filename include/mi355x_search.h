@@ -223,6 +223,12 @@ int mi355x_beam_scorer_set_prompt(mi355x_beam_scorer* s, void* stream, const int
  * mi355x_beam_select (device [batch, 2*beams]). */
 int mi355x_beam_scorer_step(mi355x_beam_scorer* s, void* stream, const float* cand_scores,
                             const int32_t* cand_tokens, const int32_t* cand_beam_indices);
+/* BeamSearch_Cpu::SelectTop as one call (src/search.cpp:101-176: log-softmax of every beam's row plus its running
+ * score, the 2*beams best candidates per batch entry, BeamSearchScorer::Process, AppendNextTokensToSequences):
+ * mi355x_beam_select with the scorer's own next scores as beam scores and candidate buffers of its own, then
+ * mi355x_beam_scorer_step.  logits: device [batch*beams, row_stride], fp32 or fp16. */
+int mi355x_beam_search_step(mi355x_beam_scorer* s, void* stream, const void* logits, int dtype,
+                            int64_t row_stride, int vocab);
 /* Device views valid until the next step: next beam scores [batch*beams], tokens, indices
  * (GetNextScores/GetNextTokens/GetNextIndices, src/beam_search_scorer.h:52-54). */
 const float* mi355x_beam_scorer_next_scores(const mi355x_beam_scorer* s);

@@ -65,6 +65,7 @@ def load_library():
         "mi355x_beam_scorer_create": [vp, i32, i32, i32, i32, C.POINTER(C.c_int32), i32, f32, i32, C.POINTER(vp)],
         "mi355x_beam_scorer_set_prompt": [vp, vp, C.POINTER(C.c_int32), i32],
         "mi355x_beam_scorer_step": [vp, vp, vp, vp, vp],
+        "mi355x_beam_search_step": [vp, vp, vp, i32, i64, i32],
         "mi355x_beam_scorer_is_done": [vp, vp, C.POINTER(C.c_int)],
         "mi355x_beam_scorer_hypothesis": [vp, vp, i32, i32, C.POINTER(C.c_int32), i32, C.POINTER(C.c_int),
                                           C.POINTER(C.c_float)],
@@ -411,6 +412,12 @@ class BeamScorer:
     def step(self, cand_scores, cand_tokens, cand_indices):
         self.ctx._check(self.L.mi355x_beam_scorer_step(self.h, _stream(), cand_scores.data_ptr(),
                                                        cand_tokens.data_ptr(), cand_indices.data_ptr()))
+
+    def search_step(self, logits):
+        """Selection and scorer step in one call (BeamSearch_Cpu::SelectTop): logits [batch*beams, vocab] fp32 or fp16."""
+        assert logits.dim() == 2 and logits.stride(1) == 1 and logits.shape[0] == self.batch * self.beams
+        self.ctx._check(self.L.mi355x_beam_search_step(self.h, _stream(), logits.data_ptr(), _DTYPE_CODES[logits.dtype],
+                                                       logits.stride(0), logits.shape[1]))
 
     def _copy(self, ptr, dtype, count):
         out = torch.empty(count, dtype=dtype, device=self.ctx.device)

@@ -734,6 +734,9 @@ struct mi355x_beam_scorer {
   int length{};
   bool finalized{};
   float* pow_dev{};
+  float* cand_scores{};    // [batch, 2*beams]: the candidates of mi355x_beam_search_step
+  int32_t* cand_tokens{};
+  int32_t* cand_beams{};
 };
 
 int mi355x_beam_scorer_create(mi355x_search_ctx* ctx, int batch, int beams, int max_length, int pad_token_id,
@@ -779,6 +782,9 @@ int mi355x_beam_scorer_create(mi355x_search_ctx* ctx, int batch, int beams, int 
   alloc(reinterpret_cast<void**>(&s->pow_dev), (static_cast<size_t>(max_length) + 1) * sizeof(float));
   alloc(reinterpret_cast<void**>(&s->seq[0]), bb * max_length * sizeof(int32_t));
   alloc(reinterpret_cast<void**>(&s->seq[1]), bb * max_length * sizeof(int32_t));
+  alloc(reinterpret_cast<void**>(&s->cand_scores), 2 * bb * sizeof(float));
+  alloc(reinterpret_cast<void**>(&s->cand_tokens), 2 * bb * sizeof(int32_t));
+  alloc(reinterpret_cast<void**>(&s->cand_beams), 2 * bb * sizeof(int32_t));
   if (e == hipSuccess) {
     // initial beam scores 0, -1e9, -1e9, ... per batch entry (src/beam_search_scorer.cpp:76-81); rank -> row
     // identity; pow(length, length_penalty) from the host libm, the function the reference calls.
@@ -833,6 +839,16 @@ int mi355x_beam_scorer_step(mi355x_beam_scorer* s, void* stream, const float* ca
   s->cur = 1 - s->cur;
   s->length += 1;
   return MI355X_OK;
+}
+
+int mi355x_beam_search_step(mi355x_beam_scorer* s, void* stream, const void* logits, int dtype, int64_t row_stride,
+                            int vocab) {
+  if (!s) return Fail(MI355X_E_INVALID, "null argument");
+  if (s->length >= s->st.max_length) return Fail(MI355X_E_INVALID, "sequence already at max_length (%d)", s->st.max_length);
+  if (int r = mi355x_beam_select(s->ctx, stream, logits, dtype, row_stride, s->st.batch, s->st.beams, vocab, s->st.next_scores,
+                                 s->cand_scores, s->cand_tokens, s->cand_beams))
+    return r;
+  return mi355x_beam_scorer_step(s, stream, s->cand_scores, s->cand_tokens, s->cand_beams);
 }
 
 const float* mi355x_beam_scorer_next_scores(const mi355x_beam_scorer* s) { return s ? s->st.next_scores : nullptr; }

@@ -662,11 +662,7 @@ void BeamSearch_Hip::ApplyNoRepeatNgram(int ngram_size) {
 
 void BeamSearch_Hip::SelectTop() {
   const int vocab = params_->config.model.vocab_size;
-  AbiCheck(mi355x_beam_select(ctx_, g_stream, next_token_scores_.Span().data(), MI355X_F32, vocab, params_->search.batch_size,
-                              params_->search.num_beams, vocab, mi355x_beam_scorer_next_scores(scorer_),
-                              cand_scores_.Span().data(), cand_tokens_.Span().data(), cand_indices_.Span().data()));
-  AbiCheck(mi355x_beam_scorer_step(scorer_, g_stream, cand_scores_.Span().data(), cand_tokens_.Span().data(),
-                                   cand_indices_.Span().data()));
+  AbiCheck(mi355x_beam_search_step(scorer_, g_stream, next_token_scores_.Span().data(), MI355X_F32, vocab, vocab));
   ++length_;
   sequences_.RewindTo(length_);  // keeps Search::GetSequenceLength() in step with the device store
 }

@@ -66,6 +66,31 @@ def test_log_softmax_extreme_rows(ctx, orc):
         assert np.array_equal(bits(got[r]), bits(orc.log_softmax(x[r], 1.0))), r
 
 
+@pytest.mark.parametrize("batch,beams,vocab,dtype", [(3, 4, 50001, np.float16), (2, 3, 900, np.float32)])
+def test_beam_search_step_is_select_plus_scorer_step(ctx, batch, beams, vocab, dtype):
+    """mi355x_beam_search_step (BeamSearch_Cpu::SelectTop in one call) against mi355x_beam_select +
+    mi355x_beam_scorer_step on a second scorer: same next scores, tokens, indices and sequences after every step."""
+    say("beam_search_step", batch, beams, vocab)
+    rng = np.random.default_rng(vocab)
+    one = pkg().BeamScorer(ctx, batch, beams, 12, 0, [7], 0.8, False)
+    two = pkg().BeamScorer(ctx, batch, beams, 12, 0, [7], 0.8, False)
+    prompt = rng.integers(1, vocab, (batch, 2)).astype(np.int32)
+    one.set_prompt(prompt)
+    two.set_prompt(prompt)
+    for step in range(8):
+        x = torch.from_numpy((rng.standard_normal((batch * beams, vocab)) * 2).astype(dtype)).cuda()
+        if step % 3 == 1:
+            x[:, 7] += 6.0  # EOS candidates
+        one.search_step(x)
+        sc, tok, idx = ctx.beam_select(x, batch, beams, two.next_scores)
+        two.step(sc, tok, idx)
+        assert torch.equal(one.next_scores.view(torch.int32), two.next_scores.view(torch.int32)), step
+        assert torch.equal(one.next_tokens, two.next_tokens) and torch.equal(one.next_indices, two.next_indices), step
+        assert torch.equal(one.sequences()[0], two.sequences()[0]), step
+    one.close()
+    two.close()
+
+
 @pytest.mark.parametrize("vocab", [3, 5000, 20000, 70000])
 def test_softmax_rows_whose_maximum_is_a_signed_zero(ctx, orc, vocab):
     """The reference subtracts the row's own first maximal element, -0.0 included: a single -0.0 maximum above
