@@ -234,8 +234,18 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
       if (lane == 63) sh.wave_tot[par][wave] = inc;
       __syncthreads();
       Step ex = step_from_below<0x138, 0xf>(inc);  // wave_shr:1, identity into lane 0
+      // composition of the waves before this one: lane l takes wave l's total, four scan levels cover the at most
+      // 16 waves, and this wave reads lane wave - 1
+      Step wt = lane < nw ? sh.wave_tot[par][lane] : Step{0u, 0u};
+      wt = step_compose(step_from_below<0x111, 0xf>(wt), wt);  // row_shr:1
+      wt = step_compose(step_from_below<0x112, 0xf>(wt), wt);  // row_shr:2
+      wt = step_compose(step_from_below<0x114, 0xf>(wt), wt);  // row_shr:4
+      wt = step_compose(step_from_below<0x118, 0xf>(wt), wt);  // row_shr:8
       Step wp{0u, 0u};
-      for (int w = 0; w < wave; ++w) wp = step_compose(wp, sh.wave_tot[par][w]);
+      if (wave > 0) {
+        wp.d0 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wt.d0), wave - 1));
+        wp.d1 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(wt.d1), wave - 1));
+      }
       ex = step_compose(wp, ex);
       uint32_t nn = step_apply(st.n, ex);
       uint32_t key = kNone;
@@ -276,16 +286,11 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
         sh.ev_b[par][wave] = pb;
       }
       __syncthreads();
-      uint32_t gk = kNone;
-      float ga = 0.0f, gb = 0.0f;
-      for (int w = 0; w < nw; ++w) {
-        const uint32_t k2 = sh.ev_key[par][w];
-        if (k2 < gk) {
-          gk = k2;
-          ga = sh.ev_a[par][w];
-          gb = sh.ev_b[par][w];
-        }
-      }
+      // the first event of the block: lane l looks at wave l's (event keys are distinct: they carry the index)
+      const uint32_t k2 = lane < nw ? sh.ev_key[par][lane] : kNone;
+      const uint32_t gk = wave_min_u32(k2);
+      const int from = __ffsll(static_cast<long long>(__ballot(k2 == gk))) - 1;  // 0 when there is no event
+      const float ga = sh.ev_a[par][from], gb = sh.ev_b[par][from];
       const uint32_t n_last = sh.n_last[par];
       par ^= 1;
       if (gk == kNone) {  // the rest of the window stayed inside the binade

@@ -416,7 +416,7 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
   const u64* lk = lds_keys;
   auto sorted = [=](int i) { return lk[i]; };
   auto exps = [=](int i) { return __uint_as_float(static_cast<uint32_t>(lk[i] >> 32)); };
-  return block_sample_epilogue<4>(sorted, exps, static_cast<int>(n_c), V, prm, u, out, seqsh);
+  return block_sample_epilogue<8>(sorted, exps, static_cast<int>(n_c), V, prm, u, out, seqsh);
 }
 
 // Per-row finish of the nucleus path: gathers the candidates the streaming pass left in `big`,
