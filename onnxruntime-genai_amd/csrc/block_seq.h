@@ -328,21 +328,25 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float
   if (n < 2) return 0;
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6, nw = blockDim.x >> 6;
   const int span = static_cast<int>(blockDim.x) * ITEMS;
-  // total
-  double part = 0.0;
-#pragma unroll 8
-  for (int i = tid; i < n; i += blockDim.x) part += static_cast<double>(w(i));
-  part = wave_sum<double>(part);
-  if (lane == 0) sh.dred[wave] = part;
-  __syncthreads();
+  // The total comes first unless the whole distribution fits one window: then the window's own scan supplies it
+  // (any summation order will do: the guard band below covers the difference).
+  const bool single = n <= span;
   double total = 0.0;
-  for (int k = 0; k < nw; ++k) total += sh.dred[k];
-  __syncthreads();
-  // A NaN weight (a row of -inf logits gives exp(-inf - -inf)) makes every quotient w/sum NaN; the
-  // binary search of std::discrete_distribution over NaNs and the forced final 1.0 ends on 0.
-  if (total != total) return 0;
-  const double guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16 * total;
-  const double target = u * total;
+  if (!single) {
+    double part = 0.0;
+#pragma unroll 8
+    for (int i = tid; i < n; i += blockDim.x) part += static_cast<double>(w(i));
+    part = wave_sum<double>(part);
+    if (lane == 0) sh.dred[wave] = part;
+    __syncthreads();
+    for (int k = 0; k < nw; ++k) total += sh.dred[k];
+    __syncthreads();
+    // A NaN weight (a row of -inf logits gives exp(-inf - -inf)) makes every quotient w/sum NaN; the
+    // binary search of std::discrete_distribution over NaNs and the forced final 1.0 ends on 0.
+    if (total != total) return 0;
+  }
+  double guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16 * total;
+  double target = u * total;
   double carry = 0.0;
   int first = kIntMax;
   int risky = 0;
@@ -367,10 +371,21 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float
     }
     if (lane == 63) sh.dscan[wave] = inc;
     __syncthreads();
-    double wp = carry;
-    for (int k = 0; k < wave; ++k) wp += sh.dscan[k];
-    double block_total = 0.0;
-    for (int k = 0; k < nw; ++k) block_total += sh.dscan[k];
+    // sums of the waves before this one and of the whole window: lane k takes wave k's sum, four scan levels
+    double ws = lane < nw ? sh.dscan[lane] : 0.0;
+#pragma unroll
+    for (int d = 1; d < 16; d <<= 1) {
+      const double y = __shfl_up(ws, d, 64);
+      if (lane >= d) ws += y;
+    }
+    const double block_total = __shfl(ws, nw - 1, 64);
+    const double wp = carry + (wave > 0 ? __shfl(ws, wave - 1, 64) : 0.0);
+    if (single) {
+      total = block_total;
+      if (total != total) return 0;  // NaN weights, as above (every thread holds the same total)
+      guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16 * total;
+      target = u * total;
+    }
     double run = wp + (inc - loc);
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
