@@ -695,6 +695,12 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   const uint32_t* mrow = a.xf.mask + static_cast<size_t>(row) * words;
   const int n_eos = a.xf.eos_count(row);
   const bool pen = a.xf.use_penalty();
+  // The thread's first history id is requested before anything else, its logit and mask word right after the
+  // mask words below: three dependent round trips to memory (id, logit, then the gather) would otherwise follow
+  // one another behind the barriers.
+  const int32_t* const h = pen ? a.xf.history + static_cast<size_t>(row) * a.xf.history_stride : nullptr;
+  const int hlen = pen ? a.xf.hist_len(row) : 0;
+  const int tok0 = (pen && tid < hlen) ? h[tid] : -1;
   // allowed ids of this thread's words: mask bits minus the EOS ids under min-length, nothing past the vocabulary
   uint32_t w[kSparseWords], valid[kSparseWords];
 #pragma unroll
@@ -711,6 +717,9 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
       w[q] = m & valid[q];
     }
   }
+  const bool tok0_ok = tok0 >= 0 && tok0 < V;
+  const float raw0 = tok0_ok ? lrow[tok0] : 0.0f;
+  const uint32_t mw0 = tok0_ok ? mrow[tok0 >> 5] : 0u;
   if (tid == 0) {
     sh_total = 0u;
     sh_extra = 0u;
@@ -720,17 +729,17 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   if (pen) {
     for (int i = tid; i < words; i += kFinishBlock) hist_bits[i] = 0u;
     __syncthreads();
-    const int32_t* h = a.xf.history + static_cast<size_t>(row) * a.xf.history_stride;
-    const int hlen = a.xf.hist_len(row);
     const uint32_t* ban_row = a.xf.ban_row(row, V);
     for (int j = tid; j < hlen; j += kFinishBlock) {
-      const int tok = h[j];
+      const bool ahead = j == tid;  // fetched above
+      const int tok = ahead ? tok0 : h[j];
       if (tok < 0 || tok >= V) continue;
       const uint32_t bit = 1u << (tok & 31);
       if (atomicOr(&hist_bits[tok >> 5], bit) & bit) continue;
       const uint32_t slot = atomicAdd(&sh_extra, 1u);
       if (slot < static_cast<uint32_t>(kSparseExtras)) {
-        extra_val[slot] = xform_value(lrow[tok], a.xf.penalty, a.xf.eos, tok, mrow[tok >> 5], true, true, n_eos, ban_row);
+        extra_val[slot] = xform_value(ahead ? raw0 : lrow[tok], a.xf.penalty, a.xf.eos, tok, ahead ? mw0 : mrow[tok >> 5], true, true,
+                                      n_eos, ban_row);
         extra_idx[slot] = static_cast<uint32_t>(tok);
       }
     }
