@@ -403,19 +403,24 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
     __syncthreads();
     n_c = cut;
   }
-  // cache exp((s - max)/T) in the score half of every entry
+  // cache exp((s - max)/T) in the score half of every entry.  The epilogue's threads each read eight consecutive
+  // entries, 64 bytes apart from lane to lane; entry i therefore moves inside its group of eight to slot
+  // (i ^ (i >> 4)) & 7, which spreads those reads over all banks.  A group is read and rewritten by eight
+  // neighbouring lanes in one pass of the loop, so the exchange happens in place.
   const float max_score = key_to_float(key64_okey(lds_keys[0]));
   __syncthreads();
   const float inv_temp = 1.0f / prm.temperature;
-  for (uint32_t i = tid; i < n_c; i += blockDim.x) {
-    const u64 k64 = lds_keys[i];
+  auto slot_of = [](uint32_t i) { return (i & ~7u) | ((i ^ (i >> 4)) & 7u); };
+  static_assert(kFinishBlock % 8 == 0 && kNucleusCap % 8 == 0, "whole groups per pass");
+  for (uint32_t i = tid; i < ((n_c + 7u) & ~7u); i += blockDim.x) {
+    const u64 k64 = i < n_c ? lds_keys[i] : 0;
     const float e = em::expf_exact((key_to_float(key64_okey(k64)) - max_score) * inv_temp);
-    lds_keys[i] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k64 & 0xffffffffull);
+    lds_keys[slot_of(i)] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k64 & 0xffffffffull);
   }
   __syncthreads();
   const u64* lk = lds_keys;
-  auto sorted = [=](int i) { return lk[i]; };
-  auto exps = [=](int i) { return __uint_as_float(static_cast<uint32_t>(lk[i] >> 32)); };
+  auto sorted = [=](int i) { return lk[slot_of(static_cast<uint32_t>(i))]; };
+  auto exps = [=](int i) { return __uint_as_float(static_cast<uint32_t>(lk[slot_of(static_cast<uint32_t>(i))] >> 32)); };
   return block_sample_epilogue<8>(sorted, exps, static_cast<int>(n_c), V, prm, u, out, seqsh);
 }
 
