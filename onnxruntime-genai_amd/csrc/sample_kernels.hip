@@ -17,7 +17,7 @@ namespace ms {
 // keys.  The bucket of a score is a monotone function of it, so the result is the exact key order.
 // Returns false -- keys untouched in value, possibly permuted -- when a bucket holds more than
 // kBucketCap keys (heavy ties); the caller then uses the sorting network.
-constexpr int kSortBuckets = 4096;
+constexpr int kSortBuckets = 7168;  // what fits next to the keys in 160 KB of LDS; a multiple of kFinishBlock
 constexpr int kBucketCap = 64;
 constexpr size_t kFinishLds = kNucleusCap * sizeof(u64) + (kSortBuckets + 1) * sizeof(uint32_t);
 
