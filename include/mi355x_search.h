@@ -299,6 +299,21 @@ int mi355x_spec_verify_sparse(mi355x_search_ctx* ctx, void* stream, const int32_
                               const float* accept_u, const double* sample_u, int batch, int K, int mode,
                               int32_t* accepted_len, int32_t* final_token, int32_t* engine_draws);
 
+/* The draws of a batch in the order ONE engine serves them: GreedySearch_Cpu::SampleTopK/TopP/TopKTopP walk the
+ * rows in order and call SampleCategoricalToken with the search's single std::mt19937 (src/search.cpp:207-243,
+ * src/sampling_distribution.h:218-227); std::discrete_distribution consumes one canonical double per row -- none
+ * for a row whose kept set holds one token, and finished rows are not sampled at all.  The caller computes the
+ * next `rows` canonical doubles of (a copy of) its engine into uniform_pool; row r draws with
+ * uniform_pool[number of consuming rows before r] from the kept set mi355x_sample left on the device
+ * (kept_count [rows], kept_ids / kept_probs [rows, kept_capacity], kept_capacity >= every count), and
+ * *draws_used (device int32, may be null) tells the caller how many doubles to discard from the real engine
+ * (two mt19937 outputs each).  skip_rows: device [rows] int32, non-zero = finished row (consumes nothing; its
+ * token is its best id), or null.  out_tokens device [rows]. */
+int mi355x_draw_in_order(mi355x_search_ctx* ctx, void* stream, const int32_t* kept_count,
+                         const int32_t* kept_ids, const float* kept_probs, int kept_capacity, int rows,
+                         const int32_t* skip_rows, const double* uniform_pool, int32_t* out_tokens,
+                         int32_t* draws_used);
+
 /* Tail of a greedy / sampling step on the device: Launch_CheckForEOSAndPad followed by
  * Launch_AppendNextTokensToSequences (src/cuda/search_cuda.cu:33-48,80-117), i.e. PadIfAlreadyEOS,
  * SetNextToken and AppendNextTokensToSequences of the CPU search (src/search.cpp:194-201,256-296):

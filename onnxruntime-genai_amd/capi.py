@@ -64,6 +64,7 @@ def load_library():
         "mi355x_beam_select": [vp, vp, vp, i32, i64, i32, i32, i32, vp, vp, vp, vp],
         "mi355x_beam_scorer_create": [vp, i32, i32, i32, i32, C.POINTER(C.c_int32), i32, f32, i32, C.POINTER(vp)],
         "mi355x_beam_scorer_set_prompt": [vp, vp, C.POINTER(C.c_int32), i32],
+        "mi355x_draw_in_order": [vp, vp, vp, vp, vp, i32, i32, vp, vp, vp, vp],
         "mi355x_beam_scorer_step": [vp, vp, vp, vp, vp],
         "mi355x_beam_search_step": [vp, vp, vp, i32, i64, i32],
         "mi355x_beam_scorer_is_done": [vp, vp, C.POINTER(C.c_int)],
@@ -348,6 +349,22 @@ def _greedy_tail(self, next_tokens, eos_seen, eos_ids, pad, sequences, current_l
 
 
 
+def _draw_in_order(self, kept_count, kept_ids, kept_probs, uniform_pool, skip_rows=None):
+    """SampleCategoricalToken for a batch served by one engine, rows in order: returns (tokens [rows], draws used)."""
+    rows, cap = kept_ids.shape
+    assert kept_count.dtype == torch.int32 and kept_ids.dtype == torch.int32 and kept_probs.dtype == torch.float32
+    assert uniform_pool.dtype == torch.float64 and uniform_pool.numel() >= rows
+    for t in (kept_count, kept_ids, kept_probs, uniform_pool):
+        assert t.is_cuda and t.is_contiguous()
+    out = torch.empty(rows, dtype=torch.int32, device=self.device)
+    used = torch.zeros(1, dtype=torch.int32, device=self.device)
+    self._check(self.L.mi355x_draw_in_order(self.h, _stream(), kept_count.data_ptr(), kept_ids.data_ptr(),
+                                            kept_probs.data_ptr(), cap, rows,
+                                            skip_rows.data_ptr() if skip_rows is not None else None,
+                                            uniform_pool.data_ptr(), out.data_ptr(), used.data_ptr()))
+    return out, used
+
+
 def _cast(self, src, dtype):
     """DeviceInterface::Cast: returns a new tensor of `dtype` with the reference CPU path's conversion."""
     assert src.is_cuda and src.is_contiguous()
@@ -376,6 +393,7 @@ SearchContext.cast = _cast
 SearchContext.logits_handoff = _logits_handoff
 SearchContext.topk_scores = _topk_scores
 SearchContext.softmax = _softmax
+SearchContext.draw_in_order = _draw_in_order
 SearchContext.beam_select = _beam_select
 SearchContext.spec_verify_sparse = _spec_verify_sparse
 SearchContext.greedy_tail = _greedy_tail

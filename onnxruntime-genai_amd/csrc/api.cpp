@@ -611,6 +611,17 @@ int mi355x_spec_verify_sparse(mi355x_search_ctx* ctx, void* stream, const int32_
   return MI355X_OK;
 }
 
+int mi355x_draw_in_order(mi355x_search_ctx* ctx, void* stream, const int32_t* kept_count, const int32_t* kept_ids,
+                         const float* kept_probs, int kept_capacity, int rows, const int32_t* skip_rows,
+                         const double* uniform_pool, int32_t* out_tokens, int32_t* draws_used) {
+  if (!ctx || !kept_count || !kept_ids || !kept_probs || !uniform_pool || !out_tokens)
+    return Fail(MI355X_E_INVALID, "null argument");
+  if (rows <= 0 || kept_capacity <= 0) return Fail(MI355X_E_INVALID, "rows and kept_capacity must be positive");
+  HIP_TRY(ms_launch_draw_in_order(kept_count, kept_ids, kept_probs, kept_capacity, rows, skip_rows, uniform_pool, out_tokens,
+                                  draws_used, static_cast<hipStream_t>(stream)));
+  return MI355X_OK;
+}
+
 int mi355x_greedy_tail(mi355x_search_ctx* ctx, void* stream, int32_t* next_tokens, int32_t* eos_seen, int batch,
                        const int32_t* eos_ids, int n_eos, int32_t pad_token_id, int32_t* sequences, int max_length,
                        int current_length, int32_t* done) {

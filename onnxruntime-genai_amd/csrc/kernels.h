@@ -185,6 +185,9 @@ hipError_t ms_launch_softmax(float* scores, int64_t row_stride, int rows, int vo
                              int log_softmax, hipStream_t stream);
 // Writes, for every row, the bitmap of ids the no-repeat-n-gram rule bans (mask layout) into `ban`.
 hipError_t ms_launch_ngram_ban(const ms::Xform* xf, int rows, int vocab, int ngram, uint32_t* ban, hipStream_t stream);
+hipError_t ms_launch_draw_in_order(const int32_t* kept_count, const int32_t* kept_ids, const float* kept_probs, int cap, int rows,
+                                    const int32_t* skip, const double* pool, int32_t* out_tokens, int32_t* draws_used,
+                                    hipStream_t stream);
 hipError_t ms_launch_kv_gather(const void* const* present_dev, void* const* past_dev, int n_tensors,
                                const int32_t* beam_indices, int rows, size_t block_bytes, int width,
                                hipStream_t stream);

@@ -45,6 +45,47 @@ __global__ __launch_bounds__(1024) void softmax_kernel(float* scores, int64_t ro
   }
 }
 
+// ---- categorical draws of a batch in the order one engine serves them --------------------------------------
+// GreedySearch_Cpu draws row after row from one std::mt19937 (src/search.cpp:207-243, SampleCategoricalToken
+// src/sampling_distribution.h:218-227): a row whose kept set holds one token consumes nothing
+// (std::discrete_distribution over a single weight returns 0 without touching the engine), nor does a finished
+// row.  The caller precomputes the next `rows` canonical doubles of its engine; row r takes the one whose index is
+// the number of consuming rows before it.  One workgroup per row; row 0 also reports how many were consumed.
+__global__ __launch_bounds__(256) void draw_in_order_kernel(const int32_t* kept_count, const int32_t* kept_ids,
+                                                            const float* kept_probs, int cap, int rows, const int32_t* skip,
+                                                            const double* pool, int32_t* out_tokens, int32_t* draws_used) {
+  __shared__ SeqShared sh;
+  __shared__ int red_before[4], red_total[4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  int before = 0, total = 0;
+  for (int r = tid; r < rows; r += 256) {
+    const int c = (!(skip && skip[r] != 0) && kept_count[r] >= 2) ? 1 : 0;
+    total += c;
+    before += r < row ? c : 0;
+  }
+  before = wave_sum<int>(before);
+  total = wave_sum<int>(total);
+  if ((tid & 63) == 0) {
+    red_before[tid >> 6] = before;
+    red_total[tid >> 6] = total;
+  }
+  __syncthreads();
+  before = (red_before[0] + red_before[1]) + (red_before[2] + red_before[3]);
+  total = (red_total[0] + red_total[1]) + (red_total[2] + red_total[3]);
+  int n = kept_count[row];
+  n = n < cap ? n : cap;
+  const bool consumes = !(skip && skip[row] != 0) && n >= 2;
+  int pos = 0;
+  if (consumes) {
+    const float* pr = kept_probs + static_cast<size_t>(row) * cap;
+    pos = block_discrete_draw<4>(n, [=](int i) { return pr[i]; }, pool[before], sh);
+  }
+  if (tid == 0) {
+    out_tokens[row] = kept_ids[static_cast<size_t>(row) * cap + pos];
+    if (row == 0 && draws_used) *draws_used = total;
+  }
+}
+
 // ---- no-repeat-n-gram bans (src/sampling_distribution.h:64-79, src/search.cpp:432-469) -------------------
 // One workgroup per row.  Every earlier occurrence of the row's last ngram-1 history ids marks the id
 // that followed it.  The row's bitmap is assembled in LDS, one window of kBanWindow ids at a time,
@@ -525,6 +566,14 @@ extern "C" hipError_t ms_launch_softmax(float* scores, int64_t row_stride, int r
     hipLaunchKernelGGL(ms::softmax_kernel<true>, dim3(rows), dim3(1024), 0, stream, scores, row_stride, vocab, temperature);
   else
     hipLaunchKernelGGL(ms::softmax_kernel<false>, dim3(rows), dim3(1024), 0, stream, scores, row_stride, vocab, temperature);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t ms_launch_draw_in_order(const int32_t* kept_count, const int32_t* kept_ids, const float* kept_probs,
+                                               int cap, int rows, const int32_t* skip, const double* pool,
+                                               int32_t* out_tokens, int32_t* draws_used, hipStream_t stream) {
+  hipLaunchKernelGGL(ms::draw_in_order_kernel, dim3(rows), dim3(256), 0, stream, kept_count, kept_ids, kept_probs, cap, rows,
+                     skip, pool, out_tokens, draws_used);
   return hipGetLastError();
 }
 

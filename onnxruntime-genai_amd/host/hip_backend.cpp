@@ -346,6 +346,8 @@ GreedySearch_Hip::GreedySearch_Hip(const GeneratorParams& params) : Search{param
   sequence_lengths_.Zero();
   uniforms_ = dev.Allocate<double>(batch);
   uniforms_.Zero();
+  draws_used_ = dev.Allocate<int32_t>(1);
+  draws_used_.Zero();
   kept_count_ = dev.Allocate<int32_t>(batch);
   state_ = dev.Allocate<int32_t>(batch + 1);
   state_.Zero();
@@ -503,36 +505,30 @@ void GreedySearch_Hip::Sample(int k, float p, float temperature, std::mt19937& r
     kept_probs_ = params_->p_device->Allocate<float>(static_cast<size_t>(batch) * cap);
     kept_capacity_ = cap;
   }
+  // The next `batch` canonical doubles of the caller's engine, taken from a copy of it: std::discrete_distribution
+  // consumes one per row, none for a row that keeps a single token or is finished, so how many this step uses is
+  // only known once the kept sets are.
+  {
+    std::mt19937 peek = rng;
+    auto u = uniforms_.CpuSpan();
+    for (int b = 0; b < batch; ++b) u[b] = std::generate_canonical<double, std::numeric_limits<double>::digits>(peek);
+    uniforms_.CopyCpuToDevice();
+  }
   AbiCheck(mi355x_sample(ctx_, g_stream, next_token_scores_.Span().data(), vocab, batch, vocab, PendingXform(),
                          mi355x_sample_params{k, p, temperature}, nullptr, uniforms_.Span().data(),
                          next_tokens_.Span().data(), kept_count_.Span().data(), kept_ids_.Span().data(),
                          kept_probs_.Span().data(), kept_capacity_));
   ClearPending();
-  const std::vector<int32_t> counts = [&] {
-    auto h = kept_count_.CopyDeviceToCpu();
-    return std::vector<int32_t>(h.begin(), h.end());
-  }();
-  const std::vector<int32_t> finished = [&] {
-    auto h = state_.CopyDeviceToCpu();
-    return std::vector<int32_t>(h.begin(), h.begin() + batch);
-  }();
-  std::vector<int32_t> ids;
-  std::vector<float> probs;
-  for (size_t b = 0; b < static_cast<size_t>(batch); ++b) {
-    if (finished[b]) continue;  // a finished row consumes no draw, as in the CPU loop; the tail pads it
-    const int n = counts[b];
-    ids.resize(n);
-    probs.resize(n);
-    HIP_CHECK(hipMemcpyAsync(ids.data(), kept_ids_.Span().data() + b * kept_capacity_, sizeof(int32_t) * n, hipMemcpyDeviceToHost, g_stream));
-    HIP_CHECK(hipMemcpyAsync(probs.data(), kept_probs_.Span().data() + b * kept_capacity_, sizeof(float) * n, hipMemcpyDeviceToHost, g_stream));
-    HIP_CHECK(hipStreamSynchronize(g_stream));
-    // SampleCategoricalToken (src/sampling_distribution.h:218-227): same distribution object, same engine
-    std::discrete_distribution<int> distribution(probs.begin(), probs.end());
-    next_tokens_.CpuSpan()[b] = ids[static_cast<size_t>(distribution(rng))];
-  }
-  next_tokens_.CopyCpuToDevice();
+  // SampleCategoricalToken for every row in the order the CPU loop serves them from `rng`, on the device: which
+  // of the doubles prepared above a row takes depends on the kept counts of the rows before it.
+  AbiCheck(mi355x_draw_in_order(ctx_, g_stream, kept_count_.Span().data(), kept_ids_.Span().data(), kept_probs_.Span().data(),
+                                kept_capacity_, batch, state_.Span().data(), uniforms_.Span().data(),
+                                next_tokens_.Span().data(), draws_used_.Span().data()));
   LaunchTail(next_tokens_.Span().data());
-  FinishStep();
+  HIP_CHECK(hipMemcpyAsync(draws_used_.CpuSpan().data(), draws_used_.Span().data(), sizeof(int32_t), hipMemcpyDeviceToHost, g_stream));
+  FinishStep();  // synchronises
+  // the engine ends where std::discrete_distribution would have left it: two outputs per consumed double
+  rng.discard(2ull * static_cast<unsigned long long>(draws_used_.CpuSpan()[0]));
 }
 
 void GreedySearch_Hip::AppendTokens(DeviceSpan<int32_t>& next_tokens) {

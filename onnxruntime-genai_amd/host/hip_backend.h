@@ -21,10 +21,11 @@ void Philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t ou
 double PhiloxUniform(uint64_t seed, uint64_t counter);
 
 // GreedySearch_Cpu's device counterpart (src/search.h:202-240, src/search.cpp:178-324).
-// Token selection runs on the GPU; EOS / padding / done bookkeeping is host state, as in the CPU
-// class.  Sampling matches the CPU class draw for draw: the kernels return each row's kept
-// distribution and the draw is made on the host by std::discrete_distribution with the caller's
-// std::mt19937, so both token and engine state equal the CPU path's.
+// Token selection, the draws and the EOS / padding / append tail run on the GPU; a step synchronises once.
+// Sampling matches the CPU class draw for draw: the host prepares the next canonical doubles of (a copy of) the
+// caller's std::mt19937, the device hands them to the rows in the order std::discrete_distribution would have
+// consumed them (a row with one kept token and a finished row take none) and reports how many were used, and the
+// caller's engine is advanced by exactly that many, so both token and engine state equal the CPU path's.
 struct GreedySearch_Hip : Search {
   explicit GreedySearch_Hip(const GeneratorParams& params);
   ~GreedySearch_Hip() override;
@@ -76,6 +77,7 @@ struct GreedySearch_Hip : Search {
   DeviceSpan<int32_t> kept_count_, kept_ids_;
   DeviceSpan<float> kept_probs_;
   DeviceSpan<double> uniforms_;
+  DeviceSpan<int32_t> draws_used_;
   int kept_capacity_{};
   DeviceSpan<int32_t> state_, tx_state_;  // per-row EOS flags followed by the all-rows-finished flag
   std::vector<int32_t> eos_ids_;

@@ -878,3 +878,32 @@ def test_exact_path_sixteen_bit_rows(ctx, orc):
         assert np.array_equal(ki[r, :len(idx)].cpu().numpy(), idx), r
         assert np.array_equal(bits(kp[r, :len(idx)].cpu().numpy()), bits(probs)), r
         assert tok[r].item() == idx[orc.discrete_draw(probs, u[r])], r
+
+
+@pytest.mark.parametrize("rows,cap", [(1, 8), (9, 64), (70, 300), (5, 20000)])
+def test_draw_in_order_follows_one_engine(ctx, orc, rows, cap):
+    """mi355x_draw_in_order: rows take the prepared canonical doubles in the order one std::mt19937 would serve them:
+    a row with a single kept token and a finished row consume none, every other row the next one."""
+    say("draw_in_order", rows, cap)
+    rng = np.random.default_rng(rows * 7 + cap)
+    counts = rng.integers(1, cap + 1, rows).astype(np.int32)
+    counts[rng.random(rows) < 0.3] = 1
+    skip = (rng.random(rows) < 0.25).astype(np.int32)
+    ids = rng.integers(0, 1 << 20, (rows, cap)).astype(np.int32)
+    probs = rng.random((rows, cap)).astype(np.float32)
+    for r in range(rows):
+        probs[r, :counts[r]] /= probs[r, :counts[r]].sum(dtype=np.float32)
+    pool = rng.random(rows)
+    for use_skip in (True, False):
+        tok, used = ctx.draw_in_order(torch.from_numpy(counts).cuda(), torch.from_numpy(ids).cuda(),
+                                      torch.from_numpy(probs).cuda(), torch.from_numpy(pool).cuda(),
+                                      torch.from_numpy(skip).cuda() if use_skip else None)
+        tok = tok.cpu().numpy()
+        d = 0
+        for r in range(rows):
+            if (use_skip and skip[r]) or counts[r] < 2:
+                assert tok[r] == ids[r, 0], r
+                continue
+            assert tok[r] == ids[r, orc.discrete_draw(probs[r, :counts[r]], pool[d])], (r, d)
+            d += 1
+        assert used.item() == d
