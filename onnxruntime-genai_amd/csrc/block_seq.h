@@ -194,7 +194,7 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
       for (int r0 = 0; r0 < n_head && fnd < 0; r0 += 64) {
         const float x = x_next;
         const int idx = r0 + lane;
-        x_next = idx + 64 < n_head ? get(idx + 64) : 0.0f;  // in flight during this round's chain
+        x_next = idx + 64 < n_head ? get(idx + 64) : 0.0f;  // in flight during the chain of the current 64 elements
         const float sp = wave_serial_prefix(lane == 0 ? carry + x : x, 64);
         const unsigned long long hit = __ballot(idx < n_head && stop(sp, x, idx));
         if (hit != 0ull) {
