@@ -636,7 +636,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   }
   if (!ok) {
     __syncthreads();
-    general_row<AnyDtype>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, big_row, seqsh,
+    general_row<AnyDtype, SortWithTile>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, big_row, seqsh,
                           SortWithTile{a.big2 ? a.big2 + static_cast<size_t>(row) * a.big_stride : nullptr, lds_keys, red32, red64});
   }
 }
@@ -869,7 +869,7 @@ __device__ __forceinline__ void nucleus_sparse_entry(const SampleArgs& a) {
     __shared__ uint32_t exact_red32[16];
     __shared__ u64 exact_red64[16];
     __syncthreads();
-    general_row<AnyDtype>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), row_params<INLINE>(a, row),
+    general_row<AnyDtype, SortWithTile>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), row_params<INLINE>(a, row),
                           a.big + static_cast<size_t>(row) * a.big_stride, exact_sh,
                           SortWithTile{a.big2 ? a.big2 + static_cast<size_t>(row) * a.big_stride : nullptr, lds_keys, exact_red32,
                                        exact_red64});
@@ -895,7 +895,7 @@ __device__ __forceinline__ void exact_rows_body(const SampleArgs& a) {
   const int row = blockIdx.x;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
   if (row_mode(prm, a.vocab, a.chunks) != kModeGeneral) return;
-  general_row<AnyDtype>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, a.big + static_cast<size_t>(row) * a.big_stride,
+  general_row<AnyDtype, SortWithTile, 8>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, a.big + static_cast<size_t>(row) * a.big_stride,
                         seqsh,
                         SortWithTile{a.big2 ? a.big2 + static_cast<size_t>(row) * a.big_stride : nullptr, lds_keys, red32, red64});
 }

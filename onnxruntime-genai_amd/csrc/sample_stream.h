@@ -114,7 +114,7 @@ struct SortInGlobalMemory {
   __device__ void operator()(u64* keys, int n2, int) const { block_sort_desc(keys, n2); }
 };
 
-template <typename InT, typename SortFn = SortInGlobalMemory>
+template <typename InT, typename SortFn = SortInGlobalMemory, int EPI_ITEMS = 4>
 __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const void* row0, const mi355x_sample_params prm,
                                             u64* scratch, SeqShared& sh, SortFn sort_desc = SortFn{}) {
   const int V = a.vocab;
@@ -179,7 +179,7 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const 
   const u64* sc = scratch;
   auto sorted = [=](int i) { return sc[i]; };
   auto exps = [=](int i) { return em::expf_exact((key_to_float(key64_okey(sc[i])) - max_score) * inv_temp); };
-  block_sample_epilogue<4>(sorted, exps, V, V, prm, a.uniforms[row], out, sh);
+  block_sample_epilogue<EPI_ITEMS>(sorted, exps, V, V, prm, a.uniforms[row], out, sh);
   if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
 }
 
