@@ -28,14 +28,7 @@ struct SeqShared {
   double bcast_d;
 };
 
-__device__ __forceinline__ int wave_min_i(int v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) {
-    const int o = __shfl_xor(v, m, 64);
-    v = o < v ? o : v;
-  }
-  return v;
-}
+__device__ __forceinline__ int wave_min_i(int v) { return -1 - wave_max<int>(-1 - v); }  // ~v reverses the order of ints
 
 // Minimum of two ints over the block (both reduced at once).  Contains two barriers.
 __device__ __forceinline__ void block_min2(int& a, int& b, SeqShared& sh) {
@@ -85,14 +78,7 @@ __device__ __forceinline__ Step quad_scan_steps(Step x) {
   return x;
 }
 
-__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) {
-    const uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), m, 64));
-    v = o < v ? o : v;
-  }
-  return v;
-}
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) { return ~wave_max<uint32_t>(~v); }
 
 // Fetches the ITEMS consecutive addends thread t owns in the window [w0, wend): indices
 // w0 + t*ITEMS + j.  Asking get() for them directly makes every lane walk its own 4*ITEMS-byte strip of
@@ -316,6 +302,25 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
   return s;
 }
 
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_from_below(double x) {
+  const u64 b = static_cast<u64>(__double_as_longlong(x));
+  const uint32_t lo = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b), CTRL, ROW_MASK, 0xf, false);
+  const uint32_t hi = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b >> 32), CTRL, ROW_MASK, 0xf, false);
+  return __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
+}
+
+// Inclusive prefix sums over the wave in tree order (lanes without a source add +0.0).
+__device__ __forceinline__ double wave_scan_add(double x) {
+  x += dpp_from_below<0x111, 0xf>(x);  // row_shr:1
+  x += dpp_from_below<0x112, 0xf>(x);  // row_shr:2
+  x += dpp_from_below<0x114, 0xf>(x);  // row_shr:4
+  x += dpp_from_below<0x118, 0xf>(x);  // row_shr:8
+  x += dpp_from_below<0x142, 0xa>(x);  // row_bcast:15 into rows 1 and 3
+  x += dpp_from_below<0x143, 0xc>(x);  // row_bcast:31 into rows 2 and 3
+  return x;
+}
+
 // Position std::discrete_distribution would return for weights w(0..n-1) and canonical draw u
 // (libstdc++ random.tcc: normalise by the double sum, partial sums in double, last forced to 1,
 // lower_bound).  The reference divides every weight by the sum and accumulates the quotients
@@ -363,23 +368,13 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float
         loc += pv[j];
       }
     }
-    double inc = loc;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const double y = __shfl_up(inc, d, 64);
-      if (lane >= d) inc += y;
-    }
+    const double inc = wave_scan_add(loc);  // lane-shifting additions: the general lane shuffles go through LDS
     if (lane == 63) sh.dscan[wave] = inc;
     __syncthreads();
-    // sums of the waves before this one and of the whole window: lane k takes wave k's sum, four scan levels
-    double ws = lane < nw ? sh.dscan[lane] : 0.0;
-#pragma unroll
-    for (int d = 1; d < 16; d <<= 1) {
-      const double y = __shfl_up(ws, d, 64);
-      if (lane >= d) ws += y;
-    }
-    const double block_total = __shfl(ws, nw - 1, 64);
-    const double wp = carry + (wave > 0 ? __shfl(ws, wave - 1, 64) : 0.0);
+    // sums of the waves before this one and of the whole window: lane k takes wave k's sum
+    const double ws = wave_scan_add(lane < nw ? sh.dscan[lane] : 0.0);
+    const double block_total = wave_read_lane(ws, nw - 1);
+    const double wp = carry + (wave > 0 ? wave_read_lane(ws, wave - 1) : 0.0);
     if (single) {
       total = block_total;
       if (total != total) return 0;  // NaN weights, as above (every thread holds the same total)

@@ -62,21 +62,62 @@ __device__ __forceinline__ u64 shfl_t<u64>(u64 v, int lane) {
   return (static_cast<u64>(hi) << 32) | lo;
 }
 
+// The value `d` lanes below (row_shr inside a row of 16 lanes, then the row broadcasts), `old` where there is
+// no such lane; 4- and 8-byte types.  These lane-shifting moves are register operations; the general lane
+// shuffles (__shfl*) go through the LDS crossbar and take several times as long.
+template <int CTRL, int ROW_MASK, typename T>
+__device__ __forceinline__ T dpp_from_below_or(T old, T x) {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit values");
+  if constexpr (sizeof(T) == 4) {
+    const uint32_t r = __builtin_amdgcn_update_dpp(__builtin_bit_cast(uint32_t, old), __builtin_bit_cast(uint32_t, x), CTRL,
+                                                   ROW_MASK, 0xf, false);
+    return __builtin_bit_cast(T, r);
+  } else {
+    const u64 o = __builtin_bit_cast(u64, old), b = __builtin_bit_cast(u64, x);
+    const uint32_t lo = __builtin_amdgcn_update_dpp(static_cast<uint32_t>(o), static_cast<uint32_t>(b), CTRL, ROW_MASK, 0xf, false);
+    const uint32_t hi = __builtin_amdgcn_update_dpp(static_cast<uint32_t>(o >> 32), static_cast<uint32_t>(b >> 32), CTRL,
+                                                   ROW_MASK, 0xf, false);
+    return __builtin_bit_cast(T, (static_cast<u64>(hi) << 32) | lo);
+  }
+}
+
+// Value of x in lane l (l uniform over the wave).
+template <typename T>
+__device__ __forceinline__ T wave_read_lane(T x, int l) {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit values");
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), l));
+  } else {
+    const u64 b = __builtin_bit_cast(u64, x);
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(b)), l));
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(b >> 32)), l));
+    return __builtin_bit_cast(T, (static_cast<u64>(hi) << 32) | lo);
+  }
+}
+
+// Reductions over the wave; every lane gets the result.  Six lane-shifting steps leave it in lane 63.
 template <typename T>
 __device__ __forceinline__ T wave_max(T v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) {
-    const T o = shfl_xor_t<T>(v, m);
-    v = o > v ? o : v;
+#define MS_STEP(CTRL, MASK)                                  \
+  {                                                          \
+    const T o = dpp_from_below_or<CTRL, MASK, T>(v, v);      \
+    v = o > v ? o : v;                                       \
   }
-  return v;
+  MS_STEP(0x111, 0xf) MS_STEP(0x112, 0xf) MS_STEP(0x114, 0xf) MS_STEP(0x118, 0xf) MS_STEP(0x142, 0xa) MS_STEP(0x143, 0xc)
+#undef MS_STEP
+  return wave_read_lane(v, 63);
 }
 
 template <typename T>
 __device__ __forceinline__ T wave_sum(T v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_t<T>(v, m);
-  return v;
+  const T zero = T(0);
+  v += dpp_from_below_or<0x111, 0xf, T>(zero, v);  // row_shr:1
+  v += dpp_from_below_or<0x112, 0xf, T>(zero, v);  // row_shr:2
+  v += dpp_from_below_or<0x114, 0xf, T>(zero, v);  // row_shr:4
+  v += dpp_from_below_or<0x118, 0xf, T>(zero, v);  // row_shr:8
+  v += dpp_from_below_or<0x142, 0xa, T>(zero, v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_from_below_or<0x143, 0xc, T>(zero, v);  // row_bcast:31 into rows 2 and 3
+  return wave_read_lane(v, 63);
 }
 
 // Bitonic sort of one value per lane, descending by lane index (lane 0 ends with the maximum).

@@ -171,16 +171,37 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
   *all_zero = false;
   float wv[WINDOWS][ITEMS];
   double part = 0.0;
+  {
+    // Every weight is requested before the first barrier (a barrier waits for the loads in flight, so fetching
+    // window by window would pay the memory latency once per window), consecutive lanes on consecutive indices;
+    // then each window is transposed through LDS so that a thread holds ITEMS consecutive weights.
+    const int bd = static_cast<int>(blockDim.x);
+    float raw[WINDOWS][ITEMS];
 #pragma unroll
-  for (int c = 0; c < WINDOWS; ++c) {
-    const int i0 = c * span;
+    for (int c = 0; c < WINDOWS; ++c)
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) wv[c][j] = 0.0f;
-    if (i0 < n) {
-      window_fetch<ITEMS>(wv[c], i0, (n - i0 < span) ? n : i0 + span, w, stage);
-      __syncthreads();  // the staging buffer is rewritten by the next window
+      for (int j = 0; j < ITEMS; ++j) {
+        const int idx = c * span + j * bd + tid;
+        raw[c][j] = idx < n ? w(idx) : 0.0f;
+      }
 #pragma unroll
-      for (int j = 0; j < ITEMS; ++j) part += static_cast<double>(wv[c][j]);
+    for (int c = 0; c < WINDOWS; ++c) {
+#pragma unroll
+      for (int j = 0; j < ITEMS; ++j) wv[c][j] = 0.0f;
+      if (c * span < n) {
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) stage[j * bd + tid] = raw[c][j];
+        __syncthreads();
+        static_assert(ITEMS % 4 == 0, "whole float4 reads");
+#pragma unroll
+        for (int j = 0; j < ITEMS; j += 4) {
+          const float4 q = *reinterpret_cast<const float4*>(stage + tid * ITEMS + j);
+          wv[c][j] = q.x, wv[c][j + 1] = q.y, wv[c][j + 2] = q.z, wv[c][j + 3] = q.w;
+        }
+        __syncthreads();  // the staging buffer is rewritten by the next window
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) part += static_cast<double>(wv[c][j]);
+      }
     }
   }
   part = wave_sum<double>(part);
@@ -208,18 +229,13 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
       double loc = 0.0;
 #pragma unroll
       for (int j = 0; j < ITEMS; ++j) loc += static_cast<double>(wv[c][j]);
-      double inc = loc;
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const double y = __shfl_up(inc, d, 64);
-        if (lane >= d) inc += y;
-      }
+      const double inc = wave_scan_add(loc);
       if (lane == 63) sh.dscan[wave] = inc;
       __syncthreads();
-      double wp = carry;
-      for (int k = 0; k < wave; ++k) wp += sh.dscan[k];
-      double block_total = 0.0;
-      for (int k = 0; k < nw; ++k) block_total += sh.dscan[k];
+      // sums of the waves before this one and of the whole window: lane k takes wave k's sum
+      const double ws = wave_scan_add(lane < nw ? sh.dscan[lane] : 0.0);
+      const double block_total = wave_read_lane(ws, nw - 1);
+      const double wp = carry + (wave > 0 ? wave_read_lane(ws, wave - 1) : 0.0);
       double run = wp + (inc - loc);
 #pragma unroll
       for (int j = 0; j < ITEMS; ++j) {

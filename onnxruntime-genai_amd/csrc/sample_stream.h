@@ -251,25 +251,6 @@ struct LaneExp2Tab {
   }
 };
 
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ double dpp_from_below(double x) {
-  const u64 b = static_cast<u64>(__double_as_longlong(x));
-  const uint32_t lo = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b), CTRL, ROW_MASK, 0xf, false);
-  const uint32_t hi = __builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(b >> 32), CTRL, ROW_MASK, 0xf, false);
-  return __longlong_as_double(static_cast<long long>((static_cast<u64>(hi) << 32) | lo));
-}
-
-// Inclusive prefix sums over the wave in tree order (lanes without a source add +0.0).
-__device__ __forceinline__ double wave_scan_add(double x) {
-  x += dpp_from_below<0x111, 0xf>(x);  // row_shr:1
-  x += dpp_from_below<0x112, 0xf>(x);  // row_shr:2
-  x += dpp_from_below<0x114, 0xf>(x);  // row_shr:4
-  x += dpp_from_below<0x118, 0xf>(x);  // row_shr:8
-  x += dpp_from_below<0x142, 0xa>(x);  // row_bcast:15 into rows 1 and 3
-  x += dpp_from_below<0x143, 0xc>(x);  // row_bcast:31 into rows 2 and 3
-  return x;
-}
-
 __device__ __forceinline__ float read_lane(float x, int l) {
   return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(x), l));
 }
