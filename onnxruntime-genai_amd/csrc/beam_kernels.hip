@@ -264,7 +264,7 @@ __global__ __launch_bounds__(64) void beam_scorer_step_kernel(const ScorerState 
     }
   }
   for (int i = 0; i < nb; ++i) {
-    const int src_row = __shfl(my_src, i, 64), tok = __shfl(my_tok, i, 64);
+    const int src_row = wave_read_lane(my_src, i), tok = wave_read_lane(my_tok, i);
     const int32_t* src = sequences + static_cast<size_t>(src_row) * s.max_length;
     int32_t* dst = sequences_next + static_cast<size_t>(batch * nb + i) * s.max_length;
     for (int t = lane; t < sequence_length; t += 64) dst[t] = src[t];
@@ -411,7 +411,7 @@ __global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a) {
 #pragma unroll
     for (int r = 0; r < R; ++r)
       if (r < nr && key[r] > lane_best) lane_best = key[r];
-    const u64 tau = __shfl(wave_sort_desc_fast<u64>(lane_best), m - 1, 64);
+    const u64 tau = wave_read_lane(wave_sort_desc_fast<u64>(lane_best), m - 1);
     uint32_t woff = 0u;
 #pragma unroll
     for (int r = 0; r < R; ++r) {

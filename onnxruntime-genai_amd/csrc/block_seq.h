@@ -186,9 +186,9 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
         if (hit != 0ull) {
           const int l = __ffsll(static_cast<long long>(hit)) - 1;
           fnd = r0 + l;
-          carry = __shfl(sp, l, 64);
+          carry = wave_read_lane(sp, l);
         } else {
-          carry = __shfl(sp, 63, 64);  // lanes past the end added zeros
+          carry = wave_read_lane(sp, 63);  // lanes past the end added zeros
         }
       }
       if (lane == 0) {

@@ -120,6 +120,19 @@ __device__ __forceinline__ T wave_sum(T v) {
   return wave_read_lane(v, 63);
 }
 
+// Inclusive prefix sums over the wave (tree order).
+template <typename T>
+__device__ __forceinline__ T wave_prefix_sum(T v) {
+  const T zero = T(0);
+  v += dpp_from_below_or<0x111, 0xf, T>(zero, v);  // row_shr:1
+  v += dpp_from_below_or<0x112, 0xf, T>(zero, v);  // row_shr:2
+  v += dpp_from_below_or<0x114, 0xf, T>(zero, v);  // row_shr:4
+  v += dpp_from_below_or<0x118, 0xf, T>(zero, v);  // row_shr:8
+  v += dpp_from_below_or<0x142, 0xa, T>(zero, v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_from_below_or<0x143, 0xc, T>(zero, v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // Bitonic sort of one value per lane, descending by lane index (lane 0 ends with the maximum).
 template <typename T>
 __device__ __forceinline__ T wave_sort_desc(T x) {

@@ -53,12 +53,7 @@ __device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n,
     local += cnt[i];
     big |= cnt[i] > static_cast<uint32_t>(kBucketCap) ? 1u : 0u;
   }
-  uint32_t inc = local;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const uint32_t y = __shfl_up(inc, d, 64);
-    if ((t & 63) >= d) inc += y;
-  }
+  uint32_t inc = wave_prefix_sum<uint32_t>(local);
   const uint32_t any_big = block_max<uint32_t>(big, red);
   if ((t & 63) == 63) red[t >> 6] = inc;
   __syncthreads();
@@ -270,8 +265,7 @@ __device__ __forceinline__ bool radix_rank_sort_desc(u64* keys, u64* alt, int n,
       uint32_t own = 0u;
 #pragma unroll 4
       for (int i = 0; i < kPer; ++i) own += hist[(wave * kPer + i) * 64 + lane];
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) own += __shfl_xor(own, d, 64);
+      own = wave_sum<uint32_t>(own);
       if (lane == 0) red32[wave] = own;
       __syncthreads();
       uint32_t run = 0u;
@@ -280,12 +274,7 @@ __device__ __forceinline__ bool radix_rank_sort_desc(u64* keys, u64* alt, int n,
       for (int i = 0; i < kPer; ++i) {
         const int d0 = (wave * kPer + i) * 64 + lane;
         const uint32_t c = hist[d0];
-        uint32_t inc = c;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-          const uint32_t y = __shfl_up(inc, d, 64);
-          if (lane >= d) inc += y;
-        }
+        uint32_t inc = wave_prefix_sum<uint32_t>(c);
         const uint32_t base = run + inc - c;
         hist[d0] = base;
         cursor[d0] = base;
@@ -298,7 +287,7 @@ __device__ __forceinline__ bool radix_rank_sort_desc(u64* keys, u64* alt, int n,
             failed = 1;
           }
         }
-        run += __shfl(inc, 63, 64);
+        run += wave_read_lane(inc, 63);
       }
       if (tid == kFinishBlock - 1) hist[kRadixDigits] = run;
     }
@@ -545,12 +534,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       const uint32_t limit = static_cast<uint32_t>(kNucleusCap - 2);
       uint32_t own = 0u;
       for (int i = 0; i < kPer; ++i) own += bucket_start[tid * kPer + i];
-      uint32_t inc = own;
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t y = __shfl_up(inc, d, 64);
-        if (lane >= d) inc += y;
-      }
+      uint32_t inc = wave_prefix_sum<uint32_t>(own);
       const int crossing = first_lane(__ballot(inc > limit));  // -1: everything fits
       if (crossing < 0) {
         if (tid == 0) sh_trim = kSortBuckets - 1;
@@ -766,15 +750,10 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
       }
     }
   }
-  uint32_t inc = count;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const uint32_t y = __shfl_up(inc, d, 64);
-    if (lane >= d) inc += y;
-  }
+  uint32_t inc = wave_prefix_sum<uint32_t>(count);
   uint32_t wave_base = 0u;
   if (lane == 63) wave_base = atomicAdd(&sh_total, inc);
-  wave_base = __shfl(wave_base, 63, 64);
+  wave_base = wave_read_lane(wave_base, 63);
   first_masked = ~block_max<uint32_t>(~first_masked, red32);  // its barriers also publish sh_total and sh_extra
   const uint32_t n_allowed = sh_total, n_extra = sh_extra;
   if (n_allowed + n_extra + 2u > static_cast<uint32_t>(kNucleusCap) || n_extra > static_cast<uint32_t>(kSparseExtras) ||

@@ -198,7 +198,7 @@ __device__ __forceinline__ int wave_apply_steps(float& s, Step f, int from, int 
   const uint32_t n2 = step_apply(st.n, p);
   const unsigned long long bad = __ballot(lane >= from && lane < limit && n2 >= kMantLimit);
   const int stop = bad != 0ull ? __ffsll(static_cast<long long>(bad)) - 1 : limit;
-  if (stop > from) s = seq_recompose(__shfl(n2, stop - 1, 64), st.se);
+  if (stop > from) s = seq_recompose(wave_read_lane(n2, stop - 1), st.se);
   return stop;
 }
 
@@ -302,7 +302,7 @@ __global__ __launch_bounds__(64) void seqsum_walk_kernel(const SeqSumArgs a) {
       const int first = (g0 + seg) * kSegElems;
       const int n = a.vocab - first < kSegElems ? a.vocab - first : kSegElems;
       const int n_parts = (n + kPart - 1) / kPart;
-      const int z = __shfl(r.z, seg, 64);
+      const int z = wave_read_lane(r.z, seg);
       const int slot = __popcll(special & ((1ull << seg) - 1ull));
       const bool cached = z == -2 && slot < kWalkSpecials;
       int4 q = make_int4(0, 0, 0, 0);
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(64) void seqsum_walk_kernel(const SeqSumArgs a) {
               if (ahead_part[slot][c] == part) hit = c;
           }
           const float x = hit >= 0 ? ahead[slot][hit][lane] : (lane < np ? src[lane] : 0.0f);
-          s = __shfl(wave_serial_prefix(lane == 0 ? s + x : x, 64), 63, 64);
+          s = wave_read_lane(wave_serial_prefix(lane == 0 ? s + x : x, 64), 63);
           ++part;
         }
       }

@@ -111,7 +111,7 @@ __device__ __forceinline__ uint32_t wave_slot(bool pred, uint32_t* counter) {
   const int leader = __ffsll(static_cast<long long>(b)) - 1;
   uint32_t base = 0u;
   if (lane == leader) base = atomicAdd(counter, static_cast<uint32_t>(__popcll(b)));
-  base = __shfl(base, leader, 64);
+  base = wave_read_lane(base, leader);
   return base + static_cast<uint32_t>(__popcll(b & ((1ull << lane) - 1ull)));
 }
 
