@@ -164,14 +164,35 @@ __global__ __launch_bounds__(256) void kv_gather_narrow_kernel(const void* const
 // registers between the pass that sums them and the pass that scans them.  Reports weights that sum to
 // exactly 0 through all_zero instead of drawing from them.  Same arithmetic and the same sequential
 // replay near a boundary as block_discrete_draw.
-template <int ITEMS, int WINDOWS, typename GetW>
-__device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u, SeqShared& sh, float* stage, bool* all_zero) {
+struct NoVectorLoads {};  // block_discrete_draw_once without a loader of whole groups of weights
+
+template <int ITEMS, int WINDOWS, typename GetW, typename GetGroup = NoVectorLoads>
+__device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u, SeqShared& sh, float* stage, bool* all_zero,
+                                                        GetGroup group = GetGroup{}) {
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6, nw = blockDim.x >> 6;
   const int span = static_cast<int>(blockDim.x) * ITEMS;
   *all_zero = false;
   float wv[WINDOWS][ITEMS];
   double part = 0.0;
-  {
+  if constexpr (!std::is_same<GetGroup, NoVectorLoads>::value) {
+    // group(i, out) loads the ITEMS weights i .. i + ITEMS - 1 (i a multiple of ITEMS, all below n) with wide
+    // loads: a thread reads its own consecutive weights directly, neighbouring lanes neighbouring groups, and no
+    // transposition through LDS (two barriers per window) is needed.
+#pragma unroll
+    for (int c = 0; c < WINDOWS; ++c) {
+      const int i0 = c * span + tid * ITEMS;
+      if (i0 + ITEMS <= n) {
+        group(i0, wv[c]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) wv[c][j] = i0 + j < n ? w(i0 + j) : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < WINDOWS; ++c)
+#pragma unroll
+      for (int j = 0; j < ITEMS; ++j) part += static_cast<double>(wv[c][j]);
+  } else {
     // Every weight is requested before the first barrier (a barrier waits for the loads in flight, so fetching
     // window by window would pay the memory latency once per window), consecutive lanes on consecutive indices;
     // then each window is transposed through LDS so that a thread holds ITEMS consecutive weights.
@@ -316,6 +337,8 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
   // to four windows are read once per draw.
   constexpr int kItems = 8, kWindows = 4;
   const bool once = vocab <= kWindows * kItems * 1024;
+  // both rows start on a 16-byte boundary: their weights can be read eight at a time
+  const bool rows_aligned = ((reinterpret_cast<uintptr_t>(pt) | reinterpret_cast<uintptr_t>(pd)) & 15u) == 0;
   int pos = 0;
   bool from_target = n >= K;
   if (!from_target) {
@@ -323,7 +346,20 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
       const float d = pt[i] - pd[i];
       return d > 0.0f ? d : 0.0f;
     };
-    if (once) {
+    auto w8 = [=](int i, float (&out)[kItems]) {
+      const float4 t0 = *reinterpret_cast<const float4*>(pt + i), t1 = *reinterpret_cast<const float4*>(pt + i + 4);
+      const float4 d0 = *reinterpret_cast<const float4*>(pd + i), d1 = *reinterpret_cast<const float4*>(pd + i + 4);
+      const float t[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+      const float d[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float r = t[j] - d[j];
+        out[j] = r > 0.0f ? r : 0.0f;
+      }
+    };
+    if (once && rows_aligned) {
+      pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &from_target, w8);
+    } else if (once) {
       pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &from_target);
     } else {
       int any = 0;
@@ -336,9 +372,14 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
   }
   if (from_target) {
     auto w = [=](int i) { return pt[i]; };
+    auto w8 = [=](int i, float (&out)[kItems]) {
+      const float4 t0 = *reinterpret_cast<const float4*>(pt + i), t1 = *reinterpret_cast<const float4*>(pt + i + 4);
+      out[0] = t0.x, out[1] = t0.y, out[2] = t0.z, out[3] = t0.w, out[4] = t1.x, out[5] = t1.y, out[6] = t1.z, out[7] = t1.w;
+    };
     bool unused;
-    pos = once ? block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &unused)
-               : block_discrete_draw<kItems>(vocab, w, sample_u[b], sh, stage);
+    if (once && rows_aligned) pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &unused, w8);
+    else if (once) pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &unused);
+    else pos = block_discrete_draw<kItems>(vocab, w, sample_u[b], sh, stage);
   }
   if (threadIdx.x == 0) {
     accepted_len[b] = n;
