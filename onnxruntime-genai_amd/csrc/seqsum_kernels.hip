@@ -100,7 +100,6 @@ __device__ __forceinline__ double seq_drift(int count) {
 
 __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs a) {
   __shared__ double dred[4];
-  __shared__ __align__(16) float stage[kSegElems];
   __shared__ Step wave_tot[4];
   const int seg = blockIdx.x, row = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const double* sums = a.seg_sum + static_cast<size_t>(row) * a.segs;
@@ -119,8 +118,20 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs
   int4* rec = a.seg_step + static_cast<size_t>(row) * a.segs + seg;
   const bool known = lo_f > 0.0f && hi_f < 3.0e38f && seq_decompose(hi_f).se == se;
   const float* erow = a.e + static_cast<size_t>(row) * a.e_stride + first;
+  // thread t continues with elements 16 t .. 16 t + 15 of the segment: four 128-bit loads (the rows of
+  // exponentials and the segments start 16-byte aligned); only a segment cut short by the end of the row goes
+  // element by element.  (Requesting them before the sums above are waited for measured slower.)
   float ev[kSegPer];
-  window_fetch<kSegPer>(ev, 0, n, [=](int i) { return erow[i]; }, stage);
+  if (n == kSegElems) {
+#pragma unroll
+    for (int j = 0; j < kSegPer; j += 4) {
+      const float4 q = *reinterpret_cast<const float4*>(erow + tid * kSegPer + j);
+      ev[j] = q.x, ev[j + 1] = q.y, ev[j + 2] = q.z, ev[j + 3] = q.w;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < kSegPer; ++j) ev[j] = tid * kSegPer + j < n ? erow[tid * kSegPer + j] : 0.0f;
+  }
   if (!known) {
     // Powers of two may fall inside the segment.  Each of its 64-element parts (four lanes of sixteen elements)
     // estimates the binade the sum has where the part begins, from the double sums of the parts before it, and
