@@ -239,6 +239,18 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
   if (n < 2) return 0;
   const double guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16 * total;
   const double target = u * total;
+  // The windows' scans are independent until their totals chain up: all of them run before the one barrier.
+  __shared__ double win_scan[WINDOWS][16];
+  double loc[WINDOWS], inc[WINDOWS];
+#pragma unroll
+  for (int c = 0; c < WINDOWS; ++c) {
+    loc[c] = 0.0;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) loc[c] += static_cast<double>(wv[c][j]);
+    inc[c] = wave_scan_add(loc[c]);
+    if (lane == 63) win_scan[c][wave] = inc[c];
+  }
+  __syncthreads();
   double carry = 0.0;
   int first = kIntMax;
   int risky = 0;
@@ -247,17 +259,11 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
     const int i0 = c * span;
     if (i0 < n) {
       const int base = i0 + tid * ITEMS;
-      double loc = 0.0;
-#pragma unroll
-      for (int j = 0; j < ITEMS; ++j) loc += static_cast<double>(wv[c][j]);
-      const double inc = wave_scan_add(loc);
-      if (lane == 63) sh.dscan[wave] = inc;
-      __syncthreads();
       // sums of the waves before this one and of the whole window: lane k takes wave k's sum
-      const double ws = wave_scan_add(lane < nw ? sh.dscan[lane] : 0.0);
+      const double ws = wave_scan_add(lane < nw ? win_scan[c][lane] : 0.0);
       const double block_total = wave_read_lane(ws, nw - 1);
       const double wp = carry + (wave > 0 ? wave_read_lane(ws, wave - 1) : 0.0);
-      double run = wp + (inc - loc);
+      double run = wp + (inc[c] - loc[c]);
 #pragma unroll
       for (int j = 0; j < ITEMS; ++j) {
         const int idx = base + j;
@@ -268,7 +274,6 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
         }
       }
       carry += block_total;
-      __syncthreads();
     }
   }
   int a = first, b = risky ? 0 : 1;
