@@ -413,6 +413,122 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
   return block_sample_epilogue<8>(sorted, exps, static_cast<int>(n_c), V, prm, u, out, seqsh);
 }
 
+// Drops the candidates that certainly lie past the end of the nucleus, so that only the rest is sorted.
+// FindNucleus stops at the first element i (in rank order) with prefix_i >= p * (prefix_i + (V - i - 1) * e_i).  A
+// histogram of the candidates over the sort's score-linear buckets bounds both sides: after all elements of buckets
+// 0 .. b the prefix is at least the sum of count * exp(lower edge), and the element that ends bucket b is at most
+// exp(upper edge of b), so once  lower_bound(prefix) * (1 - p) >= p * (V - count so far) * exp(upper edge)  -- with 2 %
+// to spare for the rounding of the reference's fp32 sums and of this estimate -- the stop lies at or before the end of
+// bucket b.  Candidates of later buckets are dropped (the best of them becomes the element after the candidates),
+// and thr rises to the lowest score of the buckets kept.  Only an estimate is at stake: the epilogue still decides
+// on exact values and reports when the nucleus does not end among the elements it is given (then the exact path
+// takes the row).  lds_keys[0 .. n_c) are the candidates in any order; table: kSortBuckets words.
+constexpr uint32_t kTrimMin = 2048;  // shorter lists are sorted whole
+
+__device__ __forceinline__ void trim_to_nucleus(u64* lds_keys, uint32_t* table, uint32_t& n_c, u64& best_below, uint32_t rmax,
+                                                uint32_t& thr, mi355x_sample_params prm, int V, uint32_t* red32, u64* red64,
+                                                uint32_t* counter) {
+  if (n_c < kTrimMin || !(prm.p > 0.0f && prm.p < 1.0f)) return;
+  constexpr int R = kNucleusCap / kFinishBlock;
+  __shared__ int cut_bucket;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const float fmax = key_to_float(rmax), fthr = key_to_float(thr);
+  const float span = fmax - fthr;
+  if (!(span > 0.0f) || !(span < 3.0e38f)) return;
+  const float scale = static_cast<float>(kSortBuckets) / span;
+  auto bucket_of = [=](float x) {
+    float bf = (fmax - x) * scale;
+    bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);
+    return bf > 0.0f ? static_cast<int>(bf) : 0;
+  };
+  for (int b = tid; b < kSortBuckets; b += kFinishBlock) table[b] = 0u;
+  if (tid == 0) cut_bucket = kSortBuckets;
+  __syncthreads();
+  if (tid == 0) *counter = 0u;  // (after the barrier: every thread has read the count of the list it came with)
+  u64 k[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t i = static_cast<uint32_t>(r * kFinishBlock + tid);
+    k[r] = i < n_c ? lds_keys[i] : 0;
+    if (i < n_c) atomicAdd(&table[bucket_of(key_to_float(key64_okey(k[r])))], 1u);
+  }
+  __syncthreads();
+  {
+    // thread t owns buckets t * kPer .. (t + 1) * kPer - 1; bucket b spans scores fmax - (b + 1) / scale .. fmax - b / scale
+    constexpr int kPer = kSortBuckets / kFinishBlock;
+    __shared__ double scan_cnt[16], scan_mass[16];
+    const int wave = tid >> 6;
+    const float step = (1.0f / prm.temperature) / scale;  // exponent per bucket; the hardware's exp2 is exact enough for bounds
+    const double p = static_cast<double>(prm.p);
+    double cb[kPer], mb[kPer], cnt = 0.0, mass = 0.0;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int b = tid * kPer + i;
+      cb[i] = static_cast<double>(table[b]);
+      mb[i] = cb[i] * static_cast<double>(__expf(-static_cast<float>(b + 1) * step));
+      cnt += cb[i];
+      mass += mb[i];
+    }
+    const double cnt_inc = wave_scan_add(cnt), mass_inc = wave_scan_add(mass);
+    if (lane == 63) {
+      scan_cnt[wave] = cnt_inc;
+      scan_mass[wave] = mass_inc;
+    }
+    __syncthreads();
+    const double wc = wave_scan_add(lane < kFinishBlock / 64 ? scan_cnt[lane] : 0.0);
+    const double wm = wave_scan_add(lane < kFinishBlock / 64 ? scan_mass[lane] : 0.0);
+    double c = (wave > 0 ? wave_read_lane(wc, wave - 1) : 0.0) + (cnt_inc - cnt);
+    double m = (wave > 0 ? wave_read_lane(wm, wave - 1) : 0.0) + (mass_inc - mass);
+    uint32_t mine = static_cast<uint32_t>(kSortBuckets);
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int b = tid * kPer + i;
+      c += cb[i];
+      m += mb[i];
+      // the stop lies at or before the end of bucket b
+      const bool closed = m * (1.0 - p) >= 1.02 * p * (static_cast<double>(V) - c) * static_cast<double>(__expf(-static_cast<float>(b) * step));
+      if (closed && mine == static_cast<uint32_t>(kSortBuckets)) mine = static_cast<uint32_t>(b);
+    }
+    const uint32_t first_closed = ~block_max<uint32_t>(~mine, red32);
+    if (tid == 0) cut_bucket = static_cast<int>(first_closed);
+  }
+  __syncthreads();
+  const int last_bucket = cut_bucket;
+  if (last_bucket >= kSortBuckets - 1) return;  // nothing to drop
+  // the lowest score whose bucket is still kept: the bucket is a non-increasing function of the score
+  uint32_t lo = thr, hi = rmax;
+  while (lo < hi) {
+    const uint32_t mid = lo + ((hi - lo) >> 1);
+    if (bucket_of(key_to_float(mid)) <= last_bucket) hi = mid;
+    else lo = mid + 1u;
+  }
+  const uint32_t thr2 = hi;
+  // compaction: the candidates at or above thr2 go back to the front of the list (a wave reserves its range with
+  // one atomic), the best of the others is kept
+  uint32_t wave_total = 0u;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const bool have = k[r] != 0;
+    const bool cand = have && key64_okey(k[r]) >= thr2;
+    wave_total += static_cast<uint32_t>(__popcll(__ballot(cand)));
+    if (have && !cand) best_below = k[r] > best_below ? k[r] : best_below;
+  }
+  uint32_t base = 0u;
+  if (lane == 0 && wave_total != 0u) base = atomicAdd(counter, wave_total);
+  base = __builtin_amdgcn_readfirstlane(base);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const bool cand = k[r] != 0 && key64_okey(k[r]) >= thr2;
+    const u64 bal = __ballot(cand);
+    const uint32_t pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(bal >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(bal), base));
+    if (cand) lds_keys[pos] = k[r];
+    base += static_cast<uint32_t>(__popcll(bal));
+  }
+  best_below = block_max<u64>(best_below, red64);  // its barriers also publish the counter and the list
+  n_c = *counter;
+  thr = thr2;
+}
+
 // Per-row finish of the nucleus path: gathers the candidates the streaming pass left in `big`,
 // sorts them in LDS and runs the exact epilogue.  One block of kFinishBlock threads per row;
 // dynamic LDS: kNucleusCap key64s + the bucket table of the sort.
@@ -614,6 +730,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   uint32_t n_c = sh_count;
   bool ok = !gave_up && !trim_failed && n_c < kNucleusCap;  // room for the next-best element too
   if (large_k) thr = ~block_max<uint32_t>(~lowest, red32);  // the lowest candidate score: the sort scales its buckets by it
+  if (ok && !large_k) trim_to_nucleus(lds_keys, bucket_start, n_c, best_below, rmax, thr, prm, V, red32, red64, &sh_count);
   if (ok) {
     ok = finish_candidates(lds_keys, bucket_start, n_c, best_below, rmax, thr, false, prm, V, a.uniforms[row],
                            row_outputs(a, row), seqsh, red32);
