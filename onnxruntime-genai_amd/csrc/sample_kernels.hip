@@ -495,14 +495,10 @@ __device__ __forceinline__ void trim_to_nucleus(u64* lds_keys, uint32_t* table, 
   __syncthreads();
   const int last_bucket = cut_bucket;
   if (last_bucket >= kSortBuckets - 1) return;  // nothing to drop
-  // the lowest score whose bucket is still kept: the bucket is a non-increasing function of the score
-  uint32_t lo = thr, hi = rmax;
-  while (lo < hi) {
-    const uint32_t mid = lo + ((hi - lo) >> 1);
-    if (bucket_of(key_to_float(mid)) <= last_bucket) hi = mid;
-    else lo = mid + 1u;
-  }
-  const uint32_t thr2 = hi;
+  // Everything down to half a bucket below the last kept bucket stays (a few keys more than needed: what matters is
+  // that no key of a kept bucket is dropped, whatever the rounding of the bucket function).
+  const uint32_t edge = order_key(fmax - (static_cast<float>(last_bucket) + 1.5f) / scale);
+  const uint32_t thr2 = edge > thr ? edge : thr;
   // compaction: the candidates at or above thr2 go back to the front of the list (a wave reserves its range with
   // one atomic), the best of the others is kept
   uint32_t wave_total = 0u;
