@@ -200,7 +200,7 @@ int mi355x_softmax(mi355x_search_ctx* ctx, void* stream, float* scores, int64_t 
                    int vocab, float temperature, int log_softmax);
 
 /* Beam-search candidate selection: BeamSearch_Cpu::SelectTop up to the scorer call
- * (src/search.cpp:101-164).  logits: device [batch*beams] rows (fp32 or fp16); beam_scores: device
+ * (src/search.cpp:101-164).  logits: device [batch*beams] rows (fp32, fp16 or bf16); beam_scores: device
  * [batch*beams].  Per batch entry the 2*beams best of the beams*vocab values
  * log_softmax(row)+beam_score, best first: out_scores/out_tokens/out_beam_indices device
  * [batch, 2*beams] (beam index relative to the batch entry).  beams <= 16. */
@@ -226,7 +226,7 @@ int mi355x_beam_scorer_step(mi355x_beam_scorer* s, void* stream, const float* ca
 /* BeamSearch_Cpu::SelectTop as one call (src/search.cpp:101-176: log-softmax of every beam's row plus its running
  * score, the 2*beams best candidates per batch entry, BeamSearchScorer::Process, AppendNextTokensToSequences):
  * mi355x_beam_select with the scorer's own next scores as beam scores and candidate buffers of its own, then
- * mi355x_beam_scorer_step.  logits: device [batch*beams, row_stride], fp32 or fp16. */
+ * mi355x_beam_scorer_step.  logits: device [batch*beams, row_stride], fp32, fp16 or bf16. */
 int mi355x_beam_search_step(mi355x_beam_scorer* s, void* stream, const void* logits, int dtype,
                             int64_t row_stride, int vocab);
 /* Device views valid until the next step: next beam scores [batch*beams], tokens, indices

@@ -432,7 +432,7 @@ class BeamScorer:
                                                        cand_tokens.data_ptr(), cand_indices.data_ptr()))
 
     def search_step(self, logits):
-        """Selection and scorer step in one call (BeamSearch_Cpu::SelectTop): logits [batch*beams, vocab] fp32 or fp16."""
+        """Selection and scorer step in one call (BeamSearch_Cpu::SelectTop): logits [batch*beams, vocab] fp32, fp16 or bf16."""
         assert logits.dim() == 2 and logits.stride(1) == 1 and logits.shape[0] == self.batch * self.beams
         self.ctx._check(self.L.mi355x_beam_search_step(self.h, _stream(), logits.data_ptr(), _DTYPE_CODES[logits.dtype],
                                                        logits.stride(0), logits.shape[1]))

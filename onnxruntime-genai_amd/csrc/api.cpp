@@ -531,7 +531,8 @@ int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits,
   if (int r = CheckRows(ctx, batch * beams, vocab)) return r;
   if (!logits || !beam_scores || !out_scores || !out_tokens || !out_beam_indices)
     return Fail(MI355X_E_INVALID, "null argument");
-  if (dtype != MI355X_F32 && dtype != MI355X_F16) return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
+  if (dtype != MI355X_F32 && dtype != MI355X_F16 && dtype != MI355X_BF16)
+    return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
   if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
   if (static_cast<long long>(beams) * vocab < 2LL * beams)
     return Fail(MI355X_E_INVALID, "beam search requires num_beams * vocab_size (%lld) >= 2 * num_beams (%d)",

@@ -31,8 +31,8 @@ __device__ __forceinline__ void row_for_each(const InT* x, int V, Fn fn) {
         } else {
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
-            v[r][2 * c] = half_bits_to_float(w[c] & 0xffffu);
-            v[r][2 * c + 1] = half_bits_to_float(w[c] >> 16);
+            v[r][2 * c] = narrow_bits_to_float<InT>(w[c] & 0xffffu);
+            v[r][2 * c + 1] = narrow_bits_to_float<InT>(w[c] >> 16);
           }
         }
       } else {
@@ -513,6 +513,8 @@ extern "C" hipError_t ms_launch_beam_segments(const ms::BeamArgs* a, int dtype, 
   const dim3 grid(a->segs, a->batch * a->beams), block(ms::kSegBlock);
   if (dtype == MI355X_F16)
     hipLaunchKernelGGL(ms::beam_seg_kernel<uint16_t>, grid, block, 0, stream, *a);
+  else if (dtype == MI355X_BF16)
+    hipLaunchKernelGGL(ms::beam_seg_kernel<ms::bf16_t>, grid, block, 0, stream, *a);
   else
     hipLaunchKernelGGL(ms::beam_seg_kernel<float>, grid, block, 0, stream, *a);
   return hipGetLastError();
@@ -521,18 +523,19 @@ extern "C" hipError_t ms_launch_beam_segments(const ms::BeamArgs* a, int dtype, 
 extern "C" hipError_t ms_launch_beam_finish(const ms::BeamArgs* a, int dtype, hipStream_t stream) {
   if (dtype == MI355X_F16)
     hipLaunchKernelGGL(ms::beam_fin_kernel<uint16_t>, dim3(a->batch), dim3(256), 0, stream, *a);
+  else if (dtype == MI355X_BF16)
+    hipLaunchKernelGGL(ms::beam_fin_kernel<ms::bf16_t>, dim3(a->batch), dim3(256), 0, stream, *a);
   else
     hipLaunchKernelGGL(ms::beam_fin_kernel<float>, dim3(a->batch), dim3(256), 0, stream, *a);
   return hipGetLastError();
 }
 
-namespace ms {
-}  // namespace ms
-
 extern "C" hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hipStream_t stream) {
   const int rows = a->batch * a->beams;
   if (dtype == MI355X_F16)
     hipLaunchKernelGGL(ms::beam_row_kernel<uint16_t>, dim3(rows), dim3(1024), 0, stream, *a);
+  else if (dtype == MI355X_BF16)
+    hipLaunchKernelGGL(ms::beam_row_kernel<ms::bf16_t>, dim3(rows), dim3(1024), 0, stream, *a);
   else
     hipLaunchKernelGGL(ms::beam_row_kernel<float>, dim3(rows), dim3(1024), 0, stream, *a);
   hipError_t e = hipGetLastError();

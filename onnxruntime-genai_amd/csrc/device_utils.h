@@ -235,6 +235,12 @@ __device__ __forceinline__ float bf16_bits_to_float(uint32_t h) {
 struct bf16_t {  // a bfloat16 bit pattern (uint16_t stands for IEEE binary16 throughout)
   uint16_t bits;
 };
+// One 16-bit element as fp32: binary16 for uint16_t, bfloat16 for bf16_t.
+template <typename InT>
+__device__ __forceinline__ float narrow_bits_to_float(uint32_t bits) {
+  if constexpr (sizeof(InT) == sizeof(bf16_t) && !__is_same(InT, uint16_t)) return bf16_bits_to_float(bits);
+  else return half_bits_to_float(bits);
+}
 // Eight bfloat16 values in a 16-byte vector.  NaNs keep their payload here (the canonical quiet NaN of
 // bf16_bits_to_float is only needed where a value is written out): selection only asks whether a value is a NaN.
 __device__ __forceinline__ void widen_bf16x8(v4u q, float* o) {

@@ -13,7 +13,7 @@ constexpr int kSegBlock = 256;
 constexpr int kSegPer = kSegElems / kSegBlock;  // 16 elements per thread
 
 // Loads the 16 elements of thread t in segment `seg`: for j, the VEC consecutive ids starting at
-// seg*kSegElems + (j*256 + t)*VEC (VEC = 4 for fp32, 8 for fp16).  Ids >= vocab yield `fill`.
+// seg*kSegElems + (j*256 + t)*VEC (VEC = 4 for fp32, 8 for fp16 and bf16).  Ids >= vocab yield `fill`.
 template <typename InT>
 __device__ __forceinline__ void seg_load(const InT* row, bool aligned, int vocab, int seg, float fill,
                                          float (&v)[kSegPer]) {
@@ -31,8 +31,8 @@ __device__ __forceinline__ void seg_load(const InT* row, bool aligned, int vocab
         const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-          v[j * 8 + 2 * c] = half_bits_to_float(w[c] & 0xffffu);
-          v[j * 8 + 2 * c + 1] = half_bits_to_float(w[c] >> 16);
+          v[j * 8 + 2 * c] = narrow_bits_to_float<InT>(w[c] & 0xffffu);
+          v[j * 8 + 2 * c + 1] = narrow_bits_to_float<InT>(w[c] >> 16);
         }
       }
     } else {

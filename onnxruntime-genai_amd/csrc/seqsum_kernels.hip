@@ -392,6 +392,9 @@ extern "C" hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, int h
   if (dtype == MI355X_F16) {
     if (!have_seg_max) hipLaunchKernelGGL(ms::seqsum_max_kernel<uint16_t>, grid, block, 0, stream, *a);
     hipLaunchKernelGGL(ms::seqsum_exp_kernel<uint16_t>, grid, block, 0, stream, *a);
+  } else if (dtype == MI355X_BF16) {
+    if (!have_seg_max) hipLaunchKernelGGL(ms::seqsum_max_kernel<ms::bf16_t>, grid, block, 0, stream, *a);
+    hipLaunchKernelGGL(ms::seqsum_exp_kernel<ms::bf16_t>, grid, block, 0, stream, *a);
   } else {
     if (!have_seg_max) hipLaunchKernelGGL(ms::seqsum_max_kernel<float>, grid, block, 0, stream, *a);
     hipLaunchKernelGGL(ms::seqsum_exp_kernel<float>, grid, block, 0, stream, *a);

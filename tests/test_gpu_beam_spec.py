@@ -66,7 +66,8 @@ def test_log_softmax_extreme_rows(ctx, orc):
         assert np.array_equal(bits(got[r]), bits(orc.log_softmax(x[r], 1.0))), r
 
 
-@pytest.mark.parametrize("batch,beams,vocab,dtype", [(3, 4, 50001, np.float16), (2, 3, 900, np.float32)])
+@pytest.mark.parametrize("batch,beams,vocab,dtype", [(3, 4, 50001, torch.float16), (2, 3, 900, torch.float32),
+                                                     (2, 4, 33000, torch.bfloat16)])
 def test_beam_search_step_is_select_plus_scorer_step(ctx, batch, beams, vocab, dtype):
     """mi355x_beam_search_step (BeamSearch_Cpu::SelectTop in one call) against mi355x_beam_select +
     mi355x_beam_scorer_step on a second scorer: same next scores, tokens, indices and sequences after every step."""
@@ -78,7 +79,7 @@ def test_beam_search_step_is_select_plus_scorer_step(ctx, batch, beams, vocab, d
     one.set_prompt(prompt)
     two.set_prompt(prompt)
     for step in range(8):
-        x = torch.from_numpy((rng.standard_normal((batch * beams, vocab)) * 2).astype(dtype)).cuda()
+        x = torch.from_numpy((rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float32)).to(dtype).cuda()
         if step % 3 == 1:
             x[:, 7] += 6.0  # EOS candidates
         one.search_step(x)
@@ -115,15 +116,21 @@ def test_softmax_rows_whose_maximum_is_a_signed_zero(ctx, orc, vocab):
 
 @pytest.mark.parametrize("batch,beams,vocab,dtype", [(2, 3, 1000, np.float32), (8, 4, 151936, np.float16),
                                                      (1, 16, 5000, np.float32), (3, 2, 2, np.float32),
-                                                     (2, 4, 3000, np.float16)])
+                                                     (2, 4, 3000, np.float16), (2, 4, 3001, "bf16"),
+                                                     (8, 4, 151936, "bf16"), (1, 3, 40000, "bf16")])
 def test_beam_select(ctx, orc, batch, beams, vocab, dtype):
-    say("beam_select", batch, beams, vocab, dtype.__name__)
+    say("beam_select", batch, beams, vocab, getattr(dtype, "__name__", dtype))
     rng = np.random.default_rng(vocab + beams)
-    x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(dtype)
     bs = (rng.standard_normal(batch * beams) * 3).astype(np.float32)
     bs[1::beams] = -1e9
-    sc, tok, idx = ctx.beam_select(torch.from_numpy(x).cuda(), batch, beams, torch.from_numpy(bs).cuda())
-    xf = orc.fp16_to_fp32(x) if dtype == np.float16 else x
+    if dtype == "bf16":  # rows of bfloat16 are read as they lie; the oracle sees the widened values
+        x_dev = torch.from_numpy((rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float32)).to(torch.bfloat16).cuda()
+        xf = x_dev.float().cpu().numpy()
+    else:
+        x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(dtype)
+        x_dev = torch.from_numpy(x).cuda()
+        xf = orc.fp16_to_fp32(x) if dtype == np.float16 else x
+    sc, tok, idx = ctx.beam_select(x_dev, batch, beams, torch.from_numpy(bs).cuda())
     osc, otok, oidx, _ = orc.beam_select_top(xf, batch, beams, bs)
     assert np.array_equal(tok.cpu().numpy(), otok)
     assert np.array_equal(idx.cpu().numpy(), oidx)
@@ -143,9 +150,12 @@ def test_beam_select_constant_rows(ctx, orc):
 
 
 def _check_beam_select(ctx, orc, x, batch, beams, bs):
-    dev_x = torch.from_numpy(x).cuda()
+    if isinstance(x, torch.Tensor):  # bfloat16 rows: the oracle sees the widened values
+        dev_x, xf = x.cuda(), x.float().numpy()
+    else:
+        dev_x = torch.from_numpy(x).cuda()
+        xf = orc.fp16_to_fp32(x) if x.dtype == np.float16 else x
     sc, tok, idx = ctx.beam_select(dev_x, batch, beams, torch.from_numpy(bs).cuda())
-    xf = orc.fp16_to_fp32(x) if x.dtype == np.float16 else x
     osc, otok, oidx, _ = orc.beam_select_top(xf, batch, beams, bs)
     assert np.array_equal(tok.cpu().numpy(), otok)
     assert np.array_equal(idx.cpu().numpy(), oidx)
@@ -153,7 +163,8 @@ def _check_beam_select(ctx, orc, x, batch, beams, bs):
 
 
 @pytest.mark.parametrize("case", ["random_fp32", "beams16", "constant", "one_segment", "equal_finals_spread",
-                                  "equal_finals_dense", "minus_inf", "ragged_fp16", "strided_fp32"])
+                                  "equal_finals_dense", "minus_inf", "ragged_fp16", "strided_fp32", "ragged_bf16",
+                                  "coarse_bf16"])
 def test_beam_select_long_rows_through_segment_lists(ctx, orc, case):
     """Rows of at least 16384 logits: every 4096-element segment lists its 2*beams largest logits and one
     workgroup per batch entry scores them.  The cases force the lists' limits: all candidates of an entry inside
@@ -199,6 +210,13 @@ def test_beam_select_long_rows_through_segment_lists(ctx, orc, case):
     elif case == "ragged_fp16":
         batch, beams, vocab = 2, 3, 16384 + 4099
         x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float16)  # odd row length: unaligned rows
+    elif case == "ragged_bf16":
+        batch, beams, vocab = 2, 3, 16384 + 4099
+        x = torch.from_numpy((rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float32)).to(torch.bfloat16)
+    elif case == "coarse_bf16":
+        # values near 8 carry three fraction bits in bfloat16: most of the row's best logits are equal
+        batch, beams, vocab = 2, 4, 70000
+        x = torch.from_numpy((8 + rng.random((batch * beams, vocab))).astype(np.float32)).to(torch.bfloat16)
     else:
         batch, beams, vocab = 2, 2, 24001
         full = (rng.standard_normal((batch * beams, vocab + 7)) * 2).astype(np.float32)
