@@ -523,9 +523,12 @@ int mi355x_softmax(mi355x_search_ctx* ctx, void* stream, float* scores, int64_t 
   return MI355X_OK;
 }
 
-int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype, int64_t row_stride,
-                       int batch, int beams, int vocab, const float* beam_scores, float* out_scores,
-                       int32_t* out_tokens, int32_t* out_beam_indices) {
+namespace {
+// mi355x_beam_select; with `step`, the launch that finishes the selection also does the scorer step where the
+// path taken has such a launch (*fused says whether it did).
+int BeamSelectImpl(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype, int64_t row_stride,
+                   int batch, int beams, int vocab, const float* beam_scores, float* out_scores,
+                   int32_t* out_tokens, int32_t* out_beam_indices, const ms::ScorerStep* step, bool* fused) {
   if (batch <= 0 || beams <= 0) return Fail(MI355X_E_INVALID, "batch and beams must be positive");
   if (beams > ms::kBeamMaxCand / 2) return Fail(MI355X_E_UNSUPPORTED, "beams (%d) above the supported %d", beams, ms::kBeamMaxCand / 2);
   if (int r = CheckRows(ctx, batch * beams, vocab)) return r;
@@ -563,13 +566,22 @@ int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits,
       a.segs = q.segs;
       HIP_TRY(ms_launch_beam_segments(&a, dtype, static_cast<hipStream_t>(stream)));
       HIP_TRY(ms_launch_seqsum(&q, dtype, 1, static_cast<hipStream_t>(stream)));
-      HIP_TRY(ms_launch_beam_finish(&a, dtype, static_cast<hipStream_t>(stream)));
+      HIP_TRY(ms_launch_beam_finish(&a, dtype, step, static_cast<hipStream_t>(stream)));
+      if (fused) *fused = step != nullptr;
       return MI355X_OK;
     }
     HIP_TRY(ms_launch_seqsum(&q, dtype, 0, static_cast<hipStream_t>(stream)));
   }
   HIP_TRY(ms_launch_beam_select(&a, dtype, static_cast<hipStream_t>(stream)));
   return MI355X_OK;
+}
+}  // namespace
+
+int mi355x_beam_select(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype, int64_t row_stride,
+                       int batch, int beams, int vocab, const float* beam_scores, float* out_scores,
+                       int32_t* out_tokens, int32_t* out_beam_indices) {
+  return BeamSelectImpl(ctx, stream, logits, dtype, row_stride, batch, beams, vocab, beam_scores, out_scores, out_tokens,
+                        out_beam_indices, nullptr, nullptr);
 }
 
 int mi355x_spec_verify_sparse(mi355x_search_ctx* ctx, void* stream, const int32_t* target_count,
@@ -791,6 +803,8 @@ int mi355x_beam_scorer_create(mi355x_search_ctx* ctx, int batch, int beams, int 
   alloc(reinterpret_cast<void**>(&st.hyp_used), batch * sizeof(int));
   alloc(reinterpret_cast<void**>(&st.done), batch * sizeof(int));
   alloc(reinterpret_cast<void**>(&st.not_done), sizeof(int));
+  alloc(reinterpret_cast<void**>(&st.pending), batch * sizeof(int));
+  alloc(reinterpret_cast<void**>(&st.arrive), sizeof(unsigned));
   alloc(reinterpret_cast<void**>(&s->pow_dev), (static_cast<size_t>(max_length) + 1) * sizeof(float));
   alloc(reinterpret_cast<void**>(&s->seq[0]), bb * max_length * sizeof(int32_t));
   alloc(reinterpret_cast<void**>(&s->seq[1]), bb * max_length * sizeof(int32_t));
@@ -857,10 +871,15 @@ int mi355x_beam_search_step(mi355x_beam_scorer* s, void* stream, const void* log
                             int vocab) {
   if (!s) return Fail(MI355X_E_INVALID, "null argument");
   if (s->length >= s->st.max_length) return Fail(MI355X_E_INVALID, "sequence already at max_length (%d)", s->st.max_length);
-  if (int r = mi355x_beam_select(s->ctx, stream, logits, dtype, row_stride, s->st.batch, s->st.beams, vocab, s->st.next_scores,
-                                 s->cand_scores, s->cand_tokens, s->cand_beams))
+  ms::ScorerStep step{s->st, s->seq[s->cur], s->seq[1 - s->cur], s->length};
+  bool fused = false;
+  if (int r = BeamSelectImpl(s->ctx, stream, logits, dtype, row_stride, s->st.batch, s->st.beams, vocab, s->st.next_scores,
+                             s->cand_scores, s->cand_tokens, s->cand_beams, &step, &fused))
     return r;
-  return mi355x_beam_scorer_step(s, stream, s->cand_scores, s->cand_tokens, s->cand_beams);
+  if (!fused) return mi355x_beam_scorer_step(s, stream, s->cand_scores, s->cand_tokens, s->cand_beams);
+  s->cur = 1 - s->cur;
+  s->length += 1;
+  return MI355X_OK;
 }
 
 const float* mi355x_beam_scorer_next_scores(const mi355x_beam_scorer* s) { return s ? s->st.next_scores : nullptr; }

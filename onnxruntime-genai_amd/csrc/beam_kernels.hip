@@ -169,14 +169,15 @@ __device__ __forceinline__ bool scorer_is_eos(const ScorerState& s, int tok) {
 
 // BeamHypotheses::Add (src/beam_search_scorer.cpp:19-39).  Hypotheses live in beams+1 token rows per
 // batch entry; `slot` maps rank -> row, so inserting shifts ranks, not tokens.
+// `used`: the entry's hypothesis count, which the caller holds (the same in all lanes) and this keeps up to date.
 __device__ __forceinline__ void scorer_add(const ScorerState& s, int batch, const int32_t* seq, int length,
-                                           float sum_logprobs) {
+                                           float sum_logprobs, int& used) {
   const int nb = s.beams, lane = lane_id();
   float* hs = s.hyp_score + batch * nb;
   int* hl = s.hyp_len + batch * nb;
   int* slot = s.hyp_slot + batch * (nb + 1);
   const float score = sum_logprobs / s.pow_table[length];
-  int index = s.hyp_used[batch];
+  int index = used;
   int row;
   if (index == nb) {
     if (score <= hs[nb - 1]) return;
@@ -184,6 +185,7 @@ __device__ __forceinline__ void scorer_add(const ScorerState& s, int batch, cons
     row = slot[nb - 1];  // the evicted hypothesis' row is reused
   } else {
     row = slot[index];
+    used = index + 1;
     if (lane == 0) s.hyp_used[batch] = index + 1;
   }
   int32_t* dst = s.hyp_tokens + (static_cast<size_t>(batch) * (nb + 1) + row) * s.max_length;
@@ -203,18 +205,61 @@ __device__ __forceinline__ void scorer_add(const ScorerState& s, int batch, cons
   __builtin_amdgcn_wave_barrier();
 }
 
-// BeamSearchScorer::Process for one batch entry (one wave), then BeamSearch_Cpu::AppendNextTokensToSequences for
-// the entry's rows: lane i keeps the (token, source row) of beam row i, and the wave copies those rows of the
-// current sequences into the next buffer with the token appended.  A done entry's rows copy global row 0, as the
-// reference does with its index 0; nothing read here is written by another entry's wave in the same launch.
-__global__ __launch_bounds__(64) void beam_scorer_step_kernel(const ScorerState s, const int32_t* sequences,
-                                                              int32_t* sequences_next, int sequence_length,
-                                                              const float* cand_scores, const int32_t* cand_tokens,
-                                                              const int32_t* cand_indices) {
-  const int batch = blockIdx.x, lane = lane_id();
+// Reads through to memory that other workgroups of the same launch have written (after a fence on both sides).
+__device__ __forceinline__ float load_agent(const float* p) {
+  return __uint_as_float(__hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+__device__ __forceinline__ int load_agent(const int* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The end of BeamSearchScorer::Process for an entry that holds `beams` hypotheses and does not stop early
+// (src/beam_search_scorer.cpp:155-170): done unless the best candidate could still improve on the worst kept
+// hypothesis.  The reference's window over the candidates starts at batch*beams rather than batch*2*beams (:161),
+// so it looks at other entries' candidates; kept as is, which is why this runs once all entries' candidates exist.
+__device__ __forceinline__ void scorer_check_done(const ScorerState& s, int batch, const float* all_scores,
+                                                  int sequence_length) {
+  const int nb = s.beams, top_k = 2 * nb;
+  float best = load_agent(all_scores + batch * nb);
+  for (int i = 1; i < top_k; ++i) best = fmaxf(best, load_agent(all_scores + batch * nb + i));
+  const float current = best / s.pow_table[sequence_length];
+  const bool can_improve = load_agent(s.hyp_score + batch * nb + nb - 1) < current;  // CanImprove
+  if (!can_improve) {
+    s.done[batch] = 1;
+    atomicSub(s.not_done, 1);
+  }
+}
+
+// What a scorer step reads of the entry's state before it looks at the candidates; asked for early, the loads
+// are back by the time the candidates are.
+struct ScorerEntryState {
+  int done, used;   // the same in all lanes
+  int tok, src;     // lane i < beams: token and source row that beam row i holds from the step before
+};
+__device__ __forceinline__ ScorerEntryState scorer_entry_state(const ScorerState& s, int batch) {
+  const int lane = lane_id(), nb = s.beams;
+  ScorerEntryState e;
+  e.done = s.done[batch];
+  e.used = s.hyp_used[batch];
+  e.tok = lane < nb ? s.next_tokens[batch * nb + lane] : s.pad;
+  e.src = lane < nb ? s.next_indices[batch * nb + lane] : 0;
+  return e;
+}
+
+// BeamSearchScorer::Process for one batch entry (one wave); scorer_append follows it: lane i keeps the (token,
+// source row) of beam row i in `next`, and the wave then copies those rows of the current sequences into the next
+// buffer with the token appended.  A done entry's rows copy global row 0, as the reference does with its index 0;
+// nothing read here is written by another entry's wave in the same launch.  cand_*: the entry's own 2*beams
+// candidates.  Returns (the same in all lanes) whether scorer_check_done still has to run for the entry.
+__device__ __forceinline__ bool scorer_entry(const ScorerState& s, int batch, const ScorerEntryState& st,
+                                             const int32_t* sequences, int sequence_length, const float* cand_scores,
+                                             const int32_t* cand_tokens, const int32_t* cand_indices,
+                                             ScorerEntryState& next) {
+  const int lane = lane_id();
   const int nb = s.beams, top_k = 2 * nb;
   int my_tok = s.pad, my_src = 0;  // what a done entry emits
-  if (s.done[batch]) {
+  bool check = false;
+  if (st.done) {
     if (lane < nb) {
       s.next_scores[batch * nb + lane] = 0.0f;
       s.next_tokens[batch * nb + lane] = s.pad;
@@ -223,18 +268,17 @@ __global__ __launch_bounds__(64) void beam_scorer_step_kernel(const ScorerState 
   } else {
     // a beam row that gets no candidate this step (more EOS candidates than the reference expects) keeps the
     // token and source row it had, as the reference's arrays do
-    if (lane < nb) {
-      my_tok = s.next_tokens[batch * nb + lane];
-      my_src = s.next_indices[batch * nb + lane];
-    }
+    my_tok = st.tok;
+    my_src = st.src;
+    int used = st.used;
     int beam_idx = 0;
     for (int j = 0; j < top_k; ++j) {
-      const int tok = cand_tokens[batch * top_k + j];
-      const float score = cand_scores[batch * top_k + j];
-      const int bbi = batch * nb + cand_indices[batch * top_k + j];
+      const int tok = cand_tokens[j];
+      const float score = cand_scores[j];
+      const int bbi = batch * nb + cand_indices[j];
       if (scorer_is_eos(s, tok)) {
         if (j >= nb) continue;
-        scorer_add(s, batch, sequences + static_cast<size_t>(bbi) * s.max_length, sequence_length, score);
+        scorer_add(s, batch, sequences + static_cast<size_t>(bbi) * s.max_length, sequence_length, score, used);
       } else {
         if (lane == beam_idx) {
           my_tok = tok;
@@ -247,38 +291,74 @@ __global__ __launch_bounds__(64) void beam_scorer_step_kernel(const ScorerState 
       }
       if (beam_idx == nb) break;
     }
-    __builtin_amdgcn_wave_barrier();
-    if (lane == 0 && s.hyp_used[batch] >= nb) {
-      bool can_improve = false;
-      if (!s.early_stopping) {
-        // The reference's window starts at batch*beams rather than batch*2*beams (:161); kept as is.
-        float best = cand_scores[batch * nb];
-        for (int i = 1; i < top_k; ++i) best = fmaxf(best, cand_scores[batch * nb + i]);
-        const float current = best / s.pow_table[sequence_length];
-        can_improve = s.hyp_score[batch * nb + nb - 1] < current;  // CanImprove
-      }
-      if (!can_improve) {
-        s.done[batch] = 1;
-        atomicSub(s.not_done, 1);
+    if (used >= nb) {
+      if (s.early_stopping) {
+        if (lane == 0) {
+          s.done[batch] = 1;
+          atomicSub(s.not_done, 1);
+        }
+      } else {
+        check = true;
       }
     }
   }
-  for (int i = 0; i < nb; ++i) {
-    const int src_row = wave_read_lane(my_src, i), tok = wave_read_lane(my_tok, i);
-    const int32_t* src = sequences + static_cast<size_t>(src_row) * s.max_length;
-    int32_t* dst = sequences_next + static_cast<size_t>(batch * nb + i) * s.max_length;
-    for (int t = lane; t < sequence_length; t += 64) dst[t] = src[t];
-    if (lane == 0) dst[sequence_length] = tok;
+  next.tok = my_tok;
+  next.src = my_src;
+  return check;
+}
+
+// BeamSearch_Cpu::AppendNextTokensToSequences for the entry's rows, from what scorer_entry left in `next`.
+__device__ __forceinline__ void scorer_append(const ScorerState& s, int batch, const ScorerEntryState& next,
+                                              const int32_t* sequences, int32_t* sequences_next, int sequence_length) {
+  const int lane = lane_id(), nb = s.beams;
+  const int my_tok = next.tok, my_src = next.src;
+  // the rows four at a time: their loads are all under way before the first store waits for one
+  for (int i0 = 0; i0 < nb; i0 += 4) {
+    const int32_t* src[4];
+    int32_t* dst[4];
+    int tok[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u < nb ? i0 + u : nb - 1;  // (a row past the end repeats the last one)
+      src[u] = sequences + static_cast<size_t>(wave_read_lane(my_src, i)) * s.max_length;
+      dst[u] = sequences_next + static_cast<size_t>(batch * nb + i) * s.max_length;
+      tok[u] = wave_read_lane(my_tok, i);
+    }
+    for (int t = lane; t < sequence_length; t += 64) {
+      int32_t v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = src[u][t];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) dst[u][t] = v[u];
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) dst[u][sequence_length] = tok[u];
+    }
   }
+}
+
+__global__ __launch_bounds__(64) void beam_scorer_step_kernel(const ScorerState s, const int32_t* sequences,
+                                                              int32_t* sequences_next, int sequence_length,
+                                                              const float* cand_scores, const int32_t* cand_tokens,
+                                                              const int32_t* cand_indices) {
+  const int batch = blockIdx.x, top_k = 2 * s.beams;
+  const ScorerEntryState st = scorer_entry_state(s, batch);
+  ScorerEntryState next{};
+  const bool check = scorer_entry(s, batch, st, sequences, sequence_length, cand_scores + batch * top_k,
+                                  cand_tokens + batch * top_k, cand_indices + batch * top_k, next);
+  scorer_append(s, batch, next, sequences, sequences_next, sequence_length);
+  if (check && lane_id() == 0) scorer_check_done(s, batch, cand_scores, sequence_length);
 }
 
 __global__ __launch_bounds__(64) void beam_scorer_finalize_kernel(const ScorerState s, const int32_t* sequences,
                                                                   int sequence_length) {
   const int batch = blockIdx.x;
   if (s.done[batch]) return;
+  int used = s.hyp_used[batch];
   for (int j = 0; j < s.beams; ++j) {
     const int bbi = batch * s.beams + j;
-    scorer_add(s, batch, sequences + static_cast<size_t>(bbi) * s.max_length, sequence_length, s.next_scores[bbi]);
+    scorer_add(s, batch, sequences + static_cast<size_t>(bbi) * s.max_length, sequence_length, s.next_scores[bbi], used);
   }
 }
 
@@ -350,8 +430,10 @@ __global__ __launch_bounds__(kSegBlock) void beam_seg_kernel(const BeamArgs a) {
   if (tid < m) out[tid] = list[tid];
 }
 
-template <typename InT>
-__global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a) {
+// SCORER: the entry's workgroup goes on with the entry's scorer step (scorer_entry, by its first wave, from the
+// candidates in LDS); the tests that need every entry's candidates are left to the workgroup that gets through last.
+template <typename InT, bool SCORER>
+__global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a, const ScorerStep sp) {
   constexpr int R = kBeamFinCap / 256;
   __shared__ u64 red64[4];
   __shared__ uint32_t red[4];
@@ -365,6 +447,10 @@ __global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a) {
   u64 raw[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) raw[r] = (r < nr && tid + r * 256 < n) ? cand[tid + r * 256] : 0ull;
+  ScorerEntryState entry_state{};
+  if constexpr (SCORER) {
+    if (tid < 64) entry_state = scorer_entry_state(sp.s, b);
+  }
   bool odd = false;  // a row whose maximum is not a finite number: its scores need not follow the logit order
   if (tid < a.beams) {
     const int row = b * a.beams + tid;
@@ -498,12 +584,38 @@ __global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a) {
     }
   }
   __syncthreads();
+  __shared__ float c_scores[kBeamMaxCand];
+  __shared__ int32_t c_tokens[kBeamMaxCand], c_beams[kBeamMaxCand];
   if (tid < m) {
     const u64 k = best_list[tid];
     const uint32_t flat = key64_index(k);
-    a.out_scores[b * m + tid] = key_to_float(key64_okey(k));
-    a.out_tokens[b * m + tid] = static_cast<int32_t>(flat % static_cast<uint32_t>(V));
-    a.out_beams[b * m + tid] = static_cast<int32_t>(flat / static_cast<uint32_t>(V));
+    const float score = key_to_float(key64_okey(k));
+    const int32_t tok = static_cast<int32_t>(flat % static_cast<uint32_t>(V));
+    const int32_t beam = static_cast<int32_t>(flat / static_cast<uint32_t>(V));
+    a.out_scores[b * m + tid] = score;
+    a.out_tokens[b * m + tid] = tok;
+    a.out_beams[b * m + tid] = beam;
+    if constexpr (SCORER) c_scores[tid] = score, c_tokens[tid] = tok, c_beams[tid] = beam;
+  }
+  if constexpr (SCORER) {
+    __syncthreads();
+    if (wave != 0) return;
+    const ScorerState& s = sp.s;
+    ScorerEntryState next{};
+    const bool check = scorer_entry(s, b, entry_state, sp.sequences, sp.sequence_length, c_scores, c_tokens, c_beams, next);
+    if (lane == 0) s.pending[b] = check ? 1 : 0;
+    // Everything the tests below read of this workgroup is out before it counts itself through, and the last one
+    // through sees all of it; the sequences, which those tests do not read, are extended while the count travels.
+    __threadfence();
+    unsigned ticket = 0u;
+    if (lane == 0) ticket = atomicAdd(s.arrive, 1u);
+    scorer_append(s, b, next, sp.sequences, sp.sequences_next, sp.sequence_length);
+    if (wave_read_lane(ticket, 0) != gridDim.x - 1u) return;
+    __threadfence();
+    if (lane == 0) *s.arrive = 0u;
+    for (int e = lane; e < s.batch; e += 64) {
+      if (load_agent(s.pending + e) != 0) scorer_check_done(s, e, a.out_scores, sp.sequence_length);
+    }
   }
 }
 
@@ -520,13 +632,21 @@ extern "C" hipError_t ms_launch_beam_segments(const ms::BeamArgs* a, int dtype, 
   return hipGetLastError();
 }
 
-extern "C" hipError_t ms_launch_beam_finish(const ms::BeamArgs* a, int dtype, hipStream_t stream) {
-  if (dtype == MI355X_F16)
-    hipLaunchKernelGGL(ms::beam_fin_kernel<uint16_t>, dim3(a->batch), dim3(256), 0, stream, *a);
-  else if (dtype == MI355X_BF16)
-    hipLaunchKernelGGL(ms::beam_fin_kernel<ms::bf16_t>, dim3(a->batch), dim3(256), 0, stream, *a);
+namespace {
+template <typename InT>
+void launch_beam_finish(const ms::BeamArgs* a, const ms::ScorerStep* step, hipStream_t stream) {
+  if (step)
+    hipLaunchKernelGGL((ms::beam_fin_kernel<InT, true>), dim3(a->batch), dim3(256), 0, stream, *a, *step);
   else
-    hipLaunchKernelGGL(ms::beam_fin_kernel<float>, dim3(a->batch), dim3(256), 0, stream, *a);
+    hipLaunchKernelGGL((ms::beam_fin_kernel<InT, false>), dim3(a->batch), dim3(256), 0, stream, *a, ms::ScorerStep{});
+}
+}  // namespace
+
+extern "C" hipError_t ms_launch_beam_finish(const ms::BeamArgs* a, int dtype, const ms::ScorerStep* step,
+                                            hipStream_t stream) {
+  if (dtype == MI355X_F16) launch_beam_finish<uint16_t>(a, step, stream);
+  else if (dtype == MI355X_BF16) launch_beam_finish<ms::bf16_t>(a, step, stream);
+  else launch_beam_finish<float>(a, step, stream);
   return hipGetLastError();
 }
 

@@ -166,6 +166,16 @@ struct ScorerState {
   int* done;              // [batch]
   int* not_done;          // [1]
   const float* pow_table; // [max_length+1]: powf(length, length_penalty), computed by the host libm
+  int* pending;           // [batch]: entries whose "can a later candidate still improve" test waits for all entries' candidates
+  unsigned* arrive;       // [1]: workgroups of a fused selection + scorer launch that are through; 0 between launches
+};
+
+// What one scorer step works on besides its state: the sequences as they are, the buffer the extended ones go to.
+struct ScorerStep {
+  ScorerState s;
+  const int32_t* sequences;
+  int32_t* sequences_next;
+  int sequence_length;
 };
 
 }  // namespace ms
@@ -203,7 +213,8 @@ hipError_t ms_launch_logits_handoff(const void* raw, int kind, int rows, int seq
                                     const int32_t* token_index, float* out, int64_t out_stride, hipStream_t stream);
 hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hipStream_t stream);
 hipError_t ms_launch_beam_segments(const ms::BeamArgs* a, int dtype, hipStream_t stream);
-hipError_t ms_launch_beam_finish(const ms::BeamArgs* a, int dtype, hipStream_t stream);
+// step != null: every batch entry's workgroup goes on with the entry's scorer step (ms_launch_scorer_step's work).
+hipError_t ms_launch_beam_finish(const ms::BeamArgs* a, int dtype, const ms::ScorerStep* step, hipStream_t stream);
 hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, int have_seg_max, hipStream_t stream);
 hipError_t ms_launch_softmax_apply(float* scores, int64_t row_stride, const ms::SeqSumArgs* a, int log_softmax,
                                    hipStream_t stream);

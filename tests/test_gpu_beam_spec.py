@@ -92,6 +92,54 @@ def test_beam_search_step_is_select_plus_scorer_step(ctx, batch, beams, vocab, d
     two.close()
 
 
+@pytest.mark.parametrize("batch,beams,vocab,early,dtype", [(70, 2, 20000, False, torch.float32),
+                                                           (5, 4, 17000, True, torch.float16),
+                                                           (8, 4, 151936, False, torch.float16),
+                                                           (3, 3, 16384, False, torch.bfloat16)])
+def test_search_step_finishes_entries_like_the_two_calls(ctx, batch, beams, vocab, early, dtype):
+    """Rows long enough for the launch that finishes the selection to do the scorer step as well: entries collect
+    hypotheses and become done at different steps (the "can it still improve" test reads other entries' candidates),
+    and next scores, tokens, indices, sequences, the done state and every hypothesis equal those of
+    mi355x_beam_select + mi355x_beam_scorer_step on a second scorer."""
+    say("search_step done entries", batch, beams, vocab, early)
+    rng = np.random.default_rng(batch * 131 + beams)
+    big = pkg().SearchContext(batch * beams, vocab)
+    one = pkg().BeamScorer(big, batch, beams, 14, 0, [7, 9], 1.3, early)
+    two = pkg().BeamScorer(big, batch, beams, 14, 0, [7, 9], 1.3, early)
+    prompt = rng.integers(10, vocab, (batch, 3)).astype(np.int32)
+    one.set_prompt(prompt)
+    two.set_prompt(prompt)
+    base = torch.from_numpy((rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float32))
+    for step in range(11):
+        x = base.roll(step * 37 + 1, 1).clone()
+        rows = rng.random(batch * beams) < 0.4
+        x[torch.from_numpy(rows), 7 if step % 2 else 9] += 9.0  # EOS candidates in some rows
+        x = x.to(dtype).cuda()
+        one.search_step(x)
+        sc, tok, idx = big.beam_select(x, batch, beams, two.next_scores)
+        two.step(sc, tok, idx)
+        assert torch.equal(one.next_scores.view(torch.int32), two.next_scores.view(torch.int32)), step
+        assert torch.equal(one.next_tokens, two.next_tokens) and torch.equal(one.next_indices, two.next_indices), step
+        assert torch.equal(one.sequences()[0], two.sequences()[0]), step
+        assert one.is_done() == two.is_done(), step
+    finished = 0
+    for b in range(batch):
+        for i in range(beams):
+            try:
+                h1 = one.hypothesis(b, i)
+            except RuntimeError:
+                with pytest.raises(RuntimeError):
+                    two.hypothesis(b, i)
+                continue
+            h2 = two.hypothesis(b, i)
+            assert h1[0] == h2[0] and np.float32(h1[1]).view(np.int32) == np.float32(h2[1]).view(np.int32), (b, i)
+            finished += 1
+    assert finished > 0
+    one.close()
+    two.close()
+    big.close()
+
+
 @pytest.mark.parametrize("vocab", [3, 5000, 20000, 70000])
 def test_softmax_rows_whose_maximum_is_a_signed_zero(ctx, orc, vocab):
     """The reference subtracts the row's own first maximal element, -0.0 included: a single -0.0 maximum above
