@@ -282,7 +282,7 @@ def test_beam_select_long_rows_through_segment_lists(ctx, orc, case):
 
 
 def run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, length_penalty, early_stopping, seed,
-                    dtype=np.float16, eos_boost=0.0):
+                    dtype=np.float16, eos_boost=0.0, fused=False):
     rng = np.random.default_rng(seed)
     prompt = rng.integers(0, vocab, (batch, 3)).astype(np.int32)
     dev = pkg().BeamScorer(ctx, batch, beams, max_length, 0, eos, length_penalty, early_stopping)
@@ -298,8 +298,11 @@ def run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, lengt
             x[:, e] += eos_boost
         xf = orc.fp16_to_fp32(x) if dtype == np.float16 else x
         # device
-        dsc, dtok, didx = ctx.beam_select(torch.from_numpy(x).cuda(), batch, beams, dev.next_scores)
-        dev.step(dsc, dtok, didx)
+        if fused:  # selection and scorer step in one call: only the state after the step shows
+            dev.search_step(torch.from_numpy(x).cuda())
+        else:
+            dsc, dtok, didx = ctx.beam_select(torch.from_numpy(x).cuda(), batch, beams, dev.next_scores)
+            dev.step(dsc, dtok, didx)
         # oracle
         osc, otok, oidx, _ = orc.beam_select_top(xf, batch, beams, ref.next_scores)
         ref.process(seq, length, osc, otok, oidx)
@@ -307,8 +310,9 @@ def run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, lengt
         orc.lib.orc_beam_append(seq.reshape(-1), nxt.reshape(-1), batch * beams, max_length, length,
                                 ref.next_indices, ref.next_tokens)
         seq, length = nxt, length + 1
-        assert np.array_equal(dtok.cpu().numpy(), otok) and np.array_equal(didx.cpu().numpy(), oidx)
-        assert np.array_equal(bits(dsc.cpu().numpy()), bits(osc))
+        if not fused:
+            assert np.array_equal(dtok.cpu().numpy(), otok) and np.array_equal(didx.cpu().numpy(), oidx)
+            assert np.array_equal(bits(dsc.cpu().numpy()), bits(osc))
         assert np.array_equal(dev.next_tokens.cpu().numpy(), ref.next_tokens)
         assert np.array_equal(dev.next_indices.cpu().numpy(), ref.next_indices)
         assert np.array_equal(bits(dev.next_scores.cpu().numpy()), bits(ref.next_scores))

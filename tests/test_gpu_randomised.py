@@ -4,7 +4,8 @@ verification, KV gather) through the C ABI against the CPU oracle.  Shapes are d
 kernels' internal edges (64-lane waves, 4096-element sum segments, the 16384-logit switch to the
 multi-workgroup sum, 32768-logit chunks); values include ties, -inf, lowest() and constant rows.
 Integer results and fp32 results must be bit-identical (NaNs compare equal to NaNs).
-MI355X_RANDOM_CASES scales the number of seeds per test (default 300 -> 40 .. 100 per test)."""
+MI355X_RANDOM_CASES scales the number of seeds per test (default 300 -> 40 .. 100 per test);
+MI355X_RANDOM_FIRST is the first seed (default 0)."""
 import os
 
 import numpy as np
@@ -18,6 +19,7 @@ from test_gpu_beam_spec import run_beam_search
 pytestmark = pytest.mark.gpu
 
 CASES = int(os.environ.get("MI355X_RANDOM_CASES", "300"))
+FIRST = int(os.environ.get("MI355X_RANDOM_FIRST", "0"))
 EDGES = [1, 2, 3, 63, 64, 65, 255, 256, 257, 1023, 1025, 4095, 4096, 4097, 8191, 8193, 16383, 16384, 16385, 20480,
          32767, 32768, 32769, 65535, 65537, 98304, 131073, 151936, 201088]
 
@@ -51,7 +53,7 @@ def random_logits(rng, rows, vocab, seed):
     return x
 
 
-@pytest.mark.parametrize("seed", range(max(CASES // 3, 1)))
+@pytest.mark.parametrize("seed", range(FIRST, FIRST + max(CASES // 3, 1)))
 def test_softmax_randomised(ctx, orc, seed):
     rng = np.random.default_rng(2000 + seed)
     vocab = int(rng.choice(EDGES)) if seed % 2 else int(rng.integers(1, 70000))
@@ -66,7 +68,7 @@ def test_softmax_randomised(ctx, orc, seed):
         assert same_bits(lsm[r], orc.log_softmax(x[r], t)), r
 
 
-@pytest.mark.parametrize("seed", range(max(CASES // 3, 1)))
+@pytest.mark.parametrize("seed", range(FIRST, FIRST + max(CASES // 3, 1)))
 def test_argmax_and_topk_scores_randomised(ctx, orc, seed):
     rng = np.random.default_rng(3000 + seed)
     vocab = int(rng.choice(EDGES)) if seed % 2 else int(rng.integers(1, 140000))
@@ -101,7 +103,7 @@ def test_argmax_and_topk_scores_randomised(ctx, orc, seed):
             assert same_bits(tsc[r], proc[r][order]), r
 
 
-@pytest.mark.parametrize("seed", range(max(CASES // 3, 1)))
+@pytest.mark.parametrize("seed", range(FIRST, FIRST + max(CASES // 3, 1)))
 def test_beam_select_randomised(ctx, orc, seed):
     rng = np.random.default_rng(4000 + seed)
     beams = int(rng.choice([1, 2, 3, 4, 5, 8, 16]))
@@ -128,12 +130,12 @@ def test_beam_select_randomised(ctx, orc, seed):
     assert same_bits(sc.cpu().numpy(), osc)
 
 
-@pytest.mark.parametrize("seed", range(max(CASES // 8, 1)))
+@pytest.mark.parametrize("seed", range(FIRST, FIRST + max(CASES // 8, 1)))
 def test_beam_search_randomised(ctx, orc, seed):
     rng = np.random.default_rng(5000 + seed)
     beams = int(rng.choice([2, 3, 4, 6]))
     batch = int(rng.integers(1, 5))
-    vocab = int(rng.choice([2 * beams + 1, 50, 300, 20000]))
+    vocab = int(rng.choice([2 * beams + 1, 50, 300, 20000, 33001]))
     n_eos = int(rng.integers(1, 3))
     eos = sorted(set(int(v) for v in rng.integers(0, vocab, n_eos)))
     steps = int(rng.integers(2, 12))
@@ -141,7 +143,8 @@ def test_beam_search_randomised(ctx, orc, seed):
     lp = float(rng.choice([1.0, 0.6, 2.0, 0.0]))
     say("beam search random", seed, batch, beams, vocab, eos, steps, max_length, lp)
     run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, lp, bool(seed % 2), 6000 + seed,
-                    dtype=np.float32 if seed % 3 else np.float16, eos_boost=float(rng.choice([0.0, 2.5, 6.0])))
+                    dtype=np.float32 if seed % 3 else np.float16, eos_boost=float(rng.choice([0.0, 2.5, 6.0])),
+                    fused=bool((seed // 2) % 2))
 
 
 def random_distributions(rng, shape, vocab, sparse):
@@ -154,7 +157,7 @@ def random_distributions(rng, shape, vocab, sparse):
     return (e / e.sum(-1, keepdims=True)).astype(np.float32)
 
 
-@pytest.mark.parametrize("seed", range(max(CASES // 4, 1)))
+@pytest.mark.parametrize("seed", range(FIRST, FIRST + max(CASES // 4, 1)))
 def test_spec_verify_randomised(ctx, orc, seed):
     rng = np.random.default_rng(7000 + seed)
     batch = int(rng.integers(1, 17))
@@ -186,7 +189,7 @@ def test_spec_verify_randomised(ctx, orc, seed):
     assert np.array_equal(tok.cpu().numpy(), otok)
 
 
-@pytest.mark.parametrize("seed", range(max(CASES // 10, 1)))
+@pytest.mark.parametrize("seed", range(FIRST, FIRST + max(CASES // 10, 1)))
 def test_kv_gather_randomised(ctx, orc, seed):
     rng = np.random.default_rng(8000 + seed)
     rows = int(rng.integers(1, 33))
@@ -241,7 +244,7 @@ def random_round(rng, orc, vocab, K, big):
     return proposal, target, draft
 
 
-@pytest.mark.parametrize("seed", range(max(CASES // 4, 1)))
+@pytest.mark.parametrize("seed", range(FIRST, FIRST + max(CASES // 4, 1)))
 def test_spec_verify_sparse_randomised(ctx, orc, seed):
     """The three modes of mi355x_spec_verify_sparse on kept sets (top-k sized, and nucleus sized for every
     fourth seed) against orc_spec_verify_sparse / orc_verify_deterministic: accepted length, final token

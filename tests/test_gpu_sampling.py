@@ -504,7 +504,9 @@ def test_sample_heterogeneous_rows(ctx, orc, rows, vocab):
     assert tok[0] == orc.argmax(x[0])
 
 
-@pytest.mark.parametrize("seed", range(int(os.environ.get("MI355X_RANDOM_CASES", "300"))))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("MI355X_RANDOM_FIRST", "0")),
+                                        int(os.environ.get("MI355X_RANDOM_FIRST", "0")) +
+                                        int(os.environ.get("MI355X_RANDOM_CASES", "300"))))
 def test_sample_randomised_shapes_and_parameters(ctx, orc, seed):
     """Differential test over random shapes (vocabularies around the 32768-logit chunk edges included),
     per-row (k, p, T) mixes, logit scales, coarse grids (ties), grammar masks, repetition penalties and
