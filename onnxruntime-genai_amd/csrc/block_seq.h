@@ -71,6 +71,27 @@ __device__ __forceinline__ Step wave_scan_steps(Step x) {
   return x;
 }
 
+// The same scan, starting afresh at the lanes that hold their own index in h (the others hold -1; lane 0 must
+// start a run): x ends as the composition from the run's first lane up to this lane, h as that first lane.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ void segscan_level(Step& x, int& h) {
+  const Step below = step_from_below<CTRL, ROW_MASK>(x);
+  const int h_below = dpp_from_below_or<CTRL, ROW_MASK, int>(-1, h);
+  const Step joined = step_compose(below, x);
+  const bool starts = h >= 0;  // the lanes covered so far already hold a run's first lane
+  x.d0 = starts ? x.d0 : joined.d0;
+  x.d1 = starts ? x.d1 : joined.d1;
+  h = starts ? h : h_below;
+}
+__device__ __forceinline__ void wave_segscan_steps(Step& x, int& h) {
+  segscan_level<0x111, 0xf>(x, h);  // row_shr:1
+  segscan_level<0x112, 0xf>(x, h);  // row_shr:2
+  segscan_level<0x114, 0xf>(x, h);  // row_shr:4
+  segscan_level<0x118, 0xf>(x, h);  // row_shr:8
+  segscan_level<0x142, 0xa>(x, h);  // row_bcast:15 into rows 1 and 3
+  segscan_level<0x143, 0xc>(x, h);  // row_bcast:31 into rows 2 and 3
+}
+
 // Composition over groups of four lanes: lanes 3, 7, 11, ... end with the composition of their group.
 __device__ __forceinline__ Step quad_scan_steps(Step x) {
   x = step_compose(step_from_below<0x111, 0xf>(x), x);  // row_shr:1

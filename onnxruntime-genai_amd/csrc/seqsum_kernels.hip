@@ -188,16 +188,25 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs
   }
 }
 
-// ---- the walk: one wave per row, no barriers -----------------------------------------------------------
-// Steps compose associatively as long as the sum stays in one binade, so the wave does not visit the segments
-// one by one: lane l takes the record of segment seg + l, the wave scans the compositions, and every lane
-// checks whether the sum would still be inside the binade after its segment.  All lanes before the first one
-// that fails are exact; the failing segment is handled through the records of its 64 parts in the same way,
-// a part that fails is added element by element (a chain of lane-shifted float additions), and the wave goes on
-// behind it with the binade the sum then has.
+// ---- the walk: one wave per row walks, fifteen more prepare its way ------------------------------------
+// Steps compose associatively as long as the sum stays in one binade, so the walking wave does not visit the
+// segments one by one: lane l takes the record of segment seg + l, the compositions over lanes are scanned, and
+// every lane checks whether the sum would still be inside the binade after its segment.  All lanes before the
+// first one that fails are exact; the failing segment is handled through the records of its 64 parts in the same
+// way, a part that fails is added element by element (a chain of lane-shifted float additions), and the wave goes
+// on behind it with the binade the sum then has.
+//
+// Which records compose with which is known before the sum is: a record says for which binade it holds, so the
+// lanes fall into runs of equal binade, and the composition of a run from its first lane up to every lane of it
+// (a scan that starts afresh at every run) does not depend on the sum.  The workgroup's other waves prepare
+// these scans -- one wave for the segments' records, one per segment whose parts are needed -- and fetch the
+// elements of the parts that will most likely be added one by one, all at the same time; the walking wave then
+// only applies a prepared composition to the sum it holds wherever it stands at the first lane of a run in the
+// binade the run expects, and falls back to a scan of its own anywhere else.
 constexpr Step kStepIdentity{0u, 0u};
 constexpr Step kStepLeaves{kStepSat, kStepSat};  // composed with anything, it still says "left the binade"
 constexpr int kWalkSpecials = 16;                 // segments per group of 64 whose part records are cached in LDS
+constexpr int kWalkWaves = 16;
 
 // Applies the steps f (one per lane; identity below `from`, kStepLeaves where no valid record exists) to the sum
 // s in lane order and returns the number of leading lanes from `from` on, below `limit`, whose results are exact;
@@ -213,145 +222,193 @@ __device__ __forceinline__ int wave_apply_steps(float& s, Step f, int from, int 
   return stop;
 }
 
+// A prepared run: `run` composes the steps from lane `head` up to this lane; `se` is the binade they hold for
+// (negative: none).  Applied to the sum s standing at lane `from`: the number of leading lanes from `from` on that
+// are exact (from itself if the run does not start there or expects another binade); s moves behind them.
+// *same_run: the lane it stopped at belongs to the run too, so the sum leaves the binade inside that lane's share.
+__device__ __forceinline__ int wave_apply_run(float& s, uint2 run, int head, int se, int from, int limit, bool* same_run) {
+  const int lane = lane_id();
+  const SeqState st = seq_decompose(s);
+  const uint32_t n2 = step_apply(st.n, Step{run.x, run.y});
+  const bool mine = lane >= from && lane < limit && head == from && se == st.se;
+  const unsigned long long in_run = __ballot(mine);
+  const unsigned long long not_good = ~__ballot(mine && n2 < kMantLimit) & (~0ull << from);
+  const int stop = not_good != 0ull ? __ffsll(static_cast<long long>(not_good)) - 1 : 64;
+  if (stop > from) s = seq_recompose(wave_read_lane(n2, stop - 1), st.se);
+  *same_run = stop < 64 && ((in_run >> stop) & 1ull) != 0ull;
+  return stop;
+}
+
+// Scan of steps that starts afresh at every lane whose `se` differs from the lane's below (and at every lane
+// without a valid step): the composition from the run's first lane up to each lane, and that first lane.
+__device__ __forceinline__ void wave_prepare_runs(Step st, int se, uint2* run, int* head) {
+  const int lane = lane_id();
+  const int below = dpp_from_below_or<0x138, 0xf, int>(-4, se);  // wave_shr:1; lane 0 sees a value no lane holds
+  int h = (lane == 0 || se < 0 || se != below) ? lane : -1;
+  wave_segscan_steps(st, h);
+  *run = make_uint2(st.d0, st.d1);
+  *head = h;
+}
+
 constexpr int kWalkAhead = 8;  // parts per cached segment whose elements are fetched ahead into LDS
 
-__global__ __launch_bounds__(64) void seqsum_walk_kernel(const SeqSumArgs a) {
+__global__ __launch_bounds__(64 * kWalkWaves) void seqsum_walk_kernel(const SeqSumArgs a) {
   static_assert(kSegSubs == 64, "one part per lane");
   constexpr int kPart = kSegElems / kSegSubs;
   static_assert(kPart == 64, "a part is one round of the addition chain");
   __shared__ int4 part_rec[kWalkSpecials][kSegSubs];
   __shared__ int part_se[kWalkSpecials][kSegSubs];
+  __shared__ uint2 part_run[kWalkSpecials][kSegSubs];
+  __shared__ unsigned char part_head[kWalkSpecials][kSegSubs];
   __shared__ float ahead[kWalkSpecials][kWalkAhead][kPart];
   __shared__ int ahead_part[kWalkSpecials][kWalkAhead];
-  __shared__ int items[kWalkSpecials * kWalkAhead];
-  const int row = blockIdx.x, lane = threadIdx.x;
+  __shared__ uint2 seg_run[64];
+  __shared__ int seg_head[64];
+  const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const size_t rbase = static_cast<size_t>(row) * a.segs;
-  uint32_t m = 0u;
-  for (int sg = lane; sg < a.segs; sg += 64) {
-    const uint32_t k = a.seg_max[rbase + sg];
-    m = k > m ? k : m;
+  float max_score = 0.0f;
+  if (wave == 0) {
+    uint32_t m = 0u;
+    for (int sg = lane; sg < a.segs; sg += 64) {
+      const uint32_t k = a.seg_max[rbase + sg];
+      m = k > m ? k : m;
+    }
+    max_score = key_to_float(wave_max<uint32_t>(m));
   }
-  const float max_score = key_to_float(wave_max<uint32_t>(m));
   const float* erow = a.e + static_cast<size_t>(row) * a.e_stride;
   float s = 0.0f;
   for (int g0 = 0; g0 < a.segs; g0 += 64) {  // groups of 64 segments, one per lane
     const int g_n = a.segs - g0 < 64 ? a.segs - g0 : 64;
     const int4 r = lane < g_n ? a.seg_step[rbase + g0 + lane] : make_int4(0, 0, -3, 0);
-    // The part records of the group's first segments that have any are fetched now, all together, and with
-    // them the elements of the parts that will most likely be added one by one: those whose estimated binade
-    // differs from the next part's, and those without an estimate.
-    __syncthreads();  // (one wave: orders the LDS accesses of the previous group before these stores)
     const unsigned long long special = __ballot(lane < g_n && r.z == -2);
     const int n_special = __popcll(special) < kWalkSpecials ? __popcll(special) : kWalkSpecials;
-    // (all record loads are requested before the first is used, then all element loads)
-    int4 rec_q[kWalkSpecials];
-    int rec_se[kWalkSpecials];
-    int seg_of[kWalkSpecials];
-    {
+    __syncthreads();  // the walk through the previous group is over
+    // task 0: the runs of the segments' records; task 1 + slot: the parts of the slot-th segment that has part
+    // records -- its runs and the elements of the parts that will most likely be added one by one (those whose
+    // estimated binade differs from the next part's, and those without an estimate)
+    for (int task = wave; task <= n_special; task += kWalkWaves) {
+      if (task == 0) {
+        uint2 run;
+        int head;
+        wave_prepare_runs(r.z >= 0 ? Step{static_cast<uint32_t>(r.x), static_cast<uint32_t>(r.y)} : kStepLeaves, r.z, &run,
+                          &head);
+        seg_run[lane] = run;
+        seg_head[lane] = head;
+        continue;
+      }
+      const int slot = task - 1;
       unsigned long long left = special;
+      for (int i = 0; i < slot; ++i) left &= left - 1ull;
+      const int sg = __ffsll(static_cast<long long>(left)) - 1;
+      const size_t at = (rbase + g0 + sg) * kSegSubs;
+      const int4 q = a.sub_step[at + lane];
+      const int pse = a.sub_se[at + lane];
+      part_rec[slot][lane] = q;
+      part_se[slot][lane] = pse;
+      const int next_se = __shfl_down(pse, 1, 64);
+      unsigned long long want = __ballot(pse < 0 || (lane < 63 && next_se != pse));
+      int pp[kWalkAhead];
+      float val[kWalkAhead];
 #pragma unroll
-      for (int slot = 0; slot < kWalkSpecials; ++slot) {
-        seg_of[slot] = -1;
-        rec_q[slot] = make_int4(0, 0, 0, 0);
-        rec_se[slot] = -1;
-        if (slot < n_special) {
-          seg_of[slot] = __ffsll(static_cast<long long>(left)) - 1;
-          left &= left - 1ull;
-          const size_t at = (rbase + g0 + seg_of[slot]) * kSegSubs;
-          rec_q[slot] = a.sub_step[at + lane];
-          rec_se[slot] = a.sub_se[at + lane];
+      for (int c = 0; c < kWalkAhead; ++c) {
+        pp[c] = -1;
+        val[c] = 0.0f;
+        if (want != 0ull) {
+          pp[c] = __ffsll(static_cast<long long>(want)) - 1;
+          want &= want - 1ull;
+          const int idx = (g0 + sg) * kSegElems + pp[c] * kPart + lane;
+          if (idx < a.vocab) val[c] = erow[idx];
         }
       }
-    }
-    int n_items = 0;  // (slot, position, part) of every part fetched ahead, listed in LDS
+      uint2 run;
+      int head;
+      wave_prepare_runs(pse >= 0 ? Step{static_cast<uint32_t>(q.x), static_cast<uint32_t>(q.y)} : kStepLeaves, pse, &run, &head);
+      part_run[slot][lane] = run;
+      part_head[slot][lane] = static_cast<unsigned char>(head);
 #pragma unroll
-    for (int slot = 0; slot < kWalkSpecials; ++slot) {
-      if (slot < n_special) {
-        part_rec[slot][lane] = rec_q[slot];
-        part_se[slot][lane] = rec_se[slot];
-        const int next_se = __shfl_down(rec_se[slot], 1, 64);
-        unsigned long long want = __ballot(rec_se[slot] < 0 || (lane < 63 && next_se != rec_se[slot]));
-        for (int c = 0; c < kWalkAhead; ++c) {
-          int p = -1;
-          if (want != 0ull) {
-            p = __ffsll(static_cast<long long>(want)) - 1;
-            want &= want - 1ull;
-            if (lane == 0) items[n_items] = (seg_of[slot] << 16) | (slot << 10) | (c << 6) | p;
-            ++n_items;
-          }
-          if (lane == 0) ahead_part[slot][c] = p;
-        }
+      for (int c = 0; c < kWalkAhead; ++c) {
+        if (lane == 0) ahead_part[slot][c] = pp[c];
+        if (pp[c] >= 0) ahead[slot][c][lane] = val[c];
       }
     }
     __syncthreads();
-    for (int i0 = 0; i0 < n_items; i0 += 8) {
-      float val[8];
-      int item[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        item[u] = i0 + u < n_items ? items[i0 + u] : -1;
-        val[u] = 0.0f;
-        if (item[u] >= 0) {
-          const int sg = item[u] >> 16, p = item[u] & 63;
-          const int idx = (g0 + sg) * kSegElems + p * kPart + lane;
-          if (idx < a.vocab) val[u] = erow[idx];
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (item[u] >= 0) ahead[(item[u] >> 10) & 63][(item[u] >> 6) & 15][lane] = val[u];
-    }
-    __syncthreads();
+    if (wave != 0) continue;
+    const uint2 s_run = seg_run[lane];
+    const int s_head = seg_head[lane];
     int seg = 0;  // inside the group
     while (seg < g_n) {
-      // the run of whole segments that are in the binade the sum is in now
-      const int se = seq_decompose(s).se;
-      const Step f = lane < seg ? kStepIdentity : (r.z == se ? Step{static_cast<uint32_t>(r.x), static_cast<uint32_t>(r.y)} : kStepLeaves);
-      seg = wave_apply_steps(s, f, seg, g_n);
-      if (seg >= g_n) break;
+      bool same_run;
+      // the prepared run of whole segments, if one starts here in the binade the sum is in now
+      const int ahead_seg = wave_apply_run(s, s_run, s_head, r.z, seg, g_n, &same_run);
+      if (ahead_seg > seg) {
+        seg = ahead_seg;
+        continue;
+      }
+      const int z = wave_read_lane(r.z, seg);
+      if (z != -2) {
+        // a segment with a record of its own that the prepared runs did not take: the scan from here
+        const int se = seq_decompose(s).se;
+        const Step f = lane < seg ? kStepIdentity : (r.z == se ? Step{static_cast<uint32_t>(r.x), static_cast<uint32_t>(r.y)} : kStepLeaves);
+        const int next = wave_apply_steps(s, f, seg, g_n);
+        if (next > seg) {
+          seg = next;
+          continue;
+        }
+      }
       // segment `seg` part by part
       const int first = (g0 + seg) * kSegElems;
       const int n = a.vocab - first < kSegElems ? a.vocab - first : kSegElems;
       const int n_parts = (n + kPart - 1) / kPart;
-      const int z = wave_read_lane(r.z, seg);
       const int slot = __popcll(special & ((1ull << seg) - 1ull));
       const bool cached = z == -2 && slot < kWalkSpecials;
       int4 q = make_int4(0, 0, 0, 0);
       int pse = -1;
+      uint2 p_run = make_uint2(0u, 0u);
+      int p_head = -1;
       if (cached) {
         q = part_rec[slot][lane];
         pse = part_se[slot][lane];
+        p_run = part_run[slot][lane];
+        p_head = part_head[slot][lane];
       } else if (z == -2) {
         q = a.sub_step[(rbase + g0 + seg) * kSegSubs + lane];
         pse = a.sub_se[(rbase + g0 + seg) * kSegSubs + lane];
       }
       int part = 0;
       while (part < n_parts) {
-        const int pe = seq_decompose(s).se;
-        Step pf = kStepLeaves;
-        if (lane < part) pf = kStepIdentity;
-        else if (pse >= 0 && pse == pe) pf = Step{static_cast<uint32_t>(q.x), static_cast<uint32_t>(q.y)};
-        else if (pse >= 0 && pse + 1 == pe) pf = Step{static_cast<uint32_t>(q.z), static_cast<uint32_t>(q.w)};
-        part = wave_apply_steps(s, pf, part, n_parts);
-        if (part < n_parts) {
-          // this part's elements one by one, from LDS where they were fetched ahead
-          const int np = n - part * kPart < kPart ? n - part * kPart : kPart;
-          const float* src = erow + first + part * kPart;
-          int hit = -1;
-          if (cached) {
-#pragma unroll
-            for (int c = 0; c < kWalkAhead; ++c)
-              if (ahead_part[slot][c] == part) hit = c;
-          }
-          const float x = hit >= 0 ? ahead[slot][hit][lane] : (lane < np ? src[lane] : 0.0f);
-          s = wave_read_lane(wave_serial_prefix(lane == 0 ? s + x : x, 64), 63);
-          ++part;
+        // the prepared run of parts, if one starts here in the binade the sum is in now; where it ends inside
+        // its own run, the sum leaves the binade in that part
+        const int ahead_part_n = wave_apply_run(s, p_run, p_head, pse, part, n_parts, &same_run);
+        if (ahead_part_n > part) {
+          part = ahead_part_n;
+          if (part >= n_parts) break;
+          if (!same_run) continue;
+        } else {
+          const int pe = seq_decompose(s).se;
+          Step pf = kStepLeaves;
+          if (lane < part) pf = kStepIdentity;
+          else if (pse >= 0 && pse == pe) pf = Step{static_cast<uint32_t>(q.x), static_cast<uint32_t>(q.y)};
+          else if (pse >= 0 && pse + 1 == pe) pf = Step{static_cast<uint32_t>(q.z), static_cast<uint32_t>(q.w)};
+          part = wave_apply_steps(s, pf, part, n_parts);
+          if (part >= n_parts) break;
         }
+        // this part's elements one by one, from LDS where they were fetched ahead
+        const int np = n - part * kPart < kPart ? n - part * kPart : kPart;
+        const float* src = erow + first + part * kPart;
+        int hit = -1;
+        if (cached) {
+#pragma unroll
+          for (int c = 0; c < kWalkAhead; ++c)
+            if (ahead_part[slot][c] == part) hit = c;
+        }
+        const float x = hit >= 0 ? ahead[slot][hit][lane] : (lane < np ? src[lane] : 0.0f);
+        s = wave_read_lane(wave_serial_prefix(lane == 0 ? s + x : x, 64), 63);
+        ++part;
       }
       ++seg;
     }
   }
-  if (lane == 0) {
+  if (wave == 0 && lane == 0) {
     a.out_sum[row] = s;
     a.out_max[row] = max_score;
   }
@@ -400,7 +457,7 @@ extern "C" hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, int h
     hipLaunchKernelGGL(ms::seqsum_exp_kernel<float>, grid, block, 0, stream, *a);
   }
   hipLaunchKernelGGL(ms::seqsum_step_kernel, grid, block, 0, stream, *a);
-  hipLaunchKernelGGL(ms::seqsum_walk_kernel, dim3(a->rows), dim3(64), 0, stream, *a);
+  hipLaunchKernelGGL(ms::seqsum_walk_kernel, dim3(a->rows), dim3(64 * ms::kWalkWaves), 0, stream, *a);
   return hipGetLastError();
 }
 
