@@ -204,6 +204,8 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   c->max_segs = (max_vocab + ms::kSegElems - 1) / ms::kSegElems;
   ok(c->Alloc(&c->seg_max, static_cast<size_t>(max_rows) * c->max_segs, false));
   ok(c->Alloc(&c->seg_sum, static_cast<size_t>(max_rows) * c->max_segs, false));
+  // "not written yet" everywhere (all bits set): the state the exact-sum kernels expect and leave behind
+  if (c->seg_sum) ok(hipMemset(c->seg_sum, 0xff, static_cast<size_t>(max_rows) * c->max_segs * sizeof(double)));
   ok(c->Alloc(&c->seg_cand, static_cast<size_t>(max_rows) * c->max_segs * ms::kBeamMaxCand, false));
   ok(c->Alloc(&c->seg_step, static_cast<size_t>(max_rows) * c->max_segs, false));
   ok(c->Alloc(&c->sub_step, static_cast<size_t>(max_rows) * c->max_segs * ms::kSegSubs, false));

@@ -3,19 +3,19 @@
 // The reference adds the exponentials of a row one by one into a float (LogSoftMax / Softmax,
 // src/softmax.h:26-47); block_seq.h reproduces that with a scan of step functions, but one workgroup
 // per row leaves most of the chip idle when there are few, long rows (beam search: 32 rows of 152K).
-// Here a row is cut into segments of kSegElems elements and four small kernels share the work:
-//   1. seqsum_max:   segment maxima.
-//   2. seqsum_exp:   e_i = expf((x_i - rowmax) * inv_T) (exact), stored as fp32, plus the segment's
-//                    sum in double.
-//   3. seqsum_step:  from the double prefix sums a segment knows the binade its running sum will be
-//                    in -- unless a power of two may fall inside it -- and composes the step functions
-//                    of its elements under that binade into one (d0, d1) pair.
-//   4. seqsum_walk:  one wave per row walks the segments in order: composed steps are applied after
-//                    checking that the running sum really is in the assumed binade and stays in it
-//                    (then the composition is exactly the sequential result); a segment that may hold
-//                    a power of two is walked through the composed steps of its 64 parts, and a
-//                    part that fails the check is added element by element.
-// The check in step 4 makes the result independent of the estimate in step 3: a wrong guess only
+// Here a row is cut into segments of kSegElems elements and three launches share the work:
+//   1. seqsum_max:      segment maxima.
+//   2. seqsum_exp_step: e_i = expf((x_i - rowmax) * inv_T) (exact), stored as fp32, plus the segment's
+//                       sum in double; then, from the double sums of the segments before it, a segment
+//                       knows the binade its running sum will be in -- unless a power of two may fall
+//                       inside it -- and composes the step functions of its elements under that binade
+//                       into one (d0, d1) pair.
+//   3. seqsum_walk:     one wave per row walks the segments in order: composed steps are applied after
+//                       checking that the running sum really is in the assumed binade and stays in it
+//                       (then the composition is exactly the sequential result); a segment that may hold
+//                       a power of two is walked through the composed steps of its 64 parts, and a
+//                       part that fails the check is added element by element.
+// The check in step 3 makes the result independent of the estimate in step 2: a wrong guess only
 // costs a scan.
 #include "kernels.h"
 #include "block_seq.h"
@@ -47,12 +47,40 @@ __device__ __forceinline__ float row_max_of_segments(const SeqSumArgs& a, int ro
   return key_to_float(block_max<uint32_t>(m, red));
 }
 
+// A segment sum that has not been written yet: all bits set, a NaN no sum can be (sums of exponentials are
+// finite, and a NaN that came in through the logits keeps zeros in its low bits when widened to double).  The
+// buffer holds this value everywhere between launches: the walk puts it back.
+constexpr unsigned long long kSumNotReady = ~0ull;
+constexpr int kSumPollLimit = 1 << 15;
+
+__device__ __forceinline__ unsigned long long load_sum_bits(const double* p) {
+  return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_sum_bits(double* p, unsigned long long bits) {
+  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Expected relative distance between the float the reference holds after adding `count` non-negative
+// terms one by one and their exact sum: roundings mostly cancel, so it grows like sqrt(count) * 2^-24
+// (the worst case grows like count * 2^-24).  Only an estimate is needed: a segment classified on a
+// wrong estimate fails the walk's check and is scanned.
+__device__ __forceinline__ double seq_drift(int count) {
+  return (8.0 * sqrt(static_cast<double>(count)) + 8.0) * 6.0e-8;
+}
+
+// Steps 2 and 3 in one launch.  A segment's workgroup writes its exponentials and publishes their double sum;
+// then it waits for the sums of the row's earlier segments, which earlier workgroups of the same launch publish
+// (workgroups start in index order and a row's segments are consecutive indices, so whatever a workgroup waits for
+// is running or done), and goes on with its step record from the exponentials it still holds.  A wait that gives
+// up only costs time: the segment is recorded as one whose parts the walk adds element by element.
 template <typename InT>
-__global__ __launch_bounds__(kSegBlock) void seqsum_exp_kernel(const SeqSumArgs a) {
+__global__ __launch_bounds__(kSegBlock) void seqsum_exp_step_kernel(const SeqSumArgs a) {
   __shared__ uint32_t red[4];
   __shared__ double dred[4];
   __shared__ uint64_t exp_tab[32];  // the table of expf in LDS: a lookup per element from constant memory is a gather
-  const int seg = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
+  __shared__ __align__(16) float stage[kSegElems];  // the segment's exponentials in element order
+  __shared__ Step wave_tot[4];
+  const int seg = blockIdx.x, row = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const InT* x = static_cast<const InT*>(a.x) + static_cast<size_t>(row) * a.row_stride;
   const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
   float v[kSegPer];
@@ -62,6 +90,7 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_kernel(const SeqSumArgs 
   const uint64_t* const tab = exp_tab;
   auto lds_tab = [=](uint32_t i) { return tab[i]; };
   float* erow = a.e + static_cast<size_t>(row) * a.e_stride;
+  const int first = seg * kSegElems;
   double part = 0.0;
   // four consecutive exponentials per store (the row of exponentials starts 16-byte aligned and a thread's ids come
   // in aligned groups of four); a group that crosses the end of the row is stored element by element
@@ -74,9 +103,10 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_kernel(const SeqSumArgs 
       ex[c] = idx + c < a.vocab ? em::expf_core((v[e0 + c] - max_score) * a.inv_temp, lds_tab) : 0.0f;
       part += static_cast<double>(ex[c]);
     }
+    v4f q;
+    q.x = ex[0], q.y = ex[1], q.z = ex[2], q.w = ex[3];
+    *reinterpret_cast<v4f*>(stage + (idx - first)) = q;
     if (idx + 4 <= a.vocab) {
-      v4f q;
-      q.x = ex[0], q.y = ex[1], q.z = ex[2], q.w = ex[3];
       *reinterpret_cast<v4f*>(erow + idx) = q;
     } else {
 #pragma unroll
@@ -85,52 +115,46 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_kernel(const SeqSumArgs 
     }
   }
   part = wave_sum<double>(part);
-  if ((tid & 63) == 0) dred[tid >> 6] = part;
-  __syncthreads();
-  if (tid == 0) a.seg_sum[static_cast<size_t>(row) * a.segs + seg] = (dred[0] + dred[1]) + (dred[2] + dred[3]);
-}
-
-// Expected relative distance between the float the reference holds after adding `count` non-negative
-// terms one by one and their exact sum: roundings mostly cancel, so it grows like sqrt(count) * 2^-24
-// (the worst case grows like count * 2^-24).  Only an estimate is needed: a segment classified on a
-// wrong estimate fails the walk's check and is scanned.
-__device__ __forceinline__ double seq_drift(int count) {
-  return (8.0 * sqrt(static_cast<double>(count)) + 8.0) * 6.0e-8;
-}
-
-__global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs a) {
-  __shared__ double dred[4];
-  __shared__ Step wave_tot[4];
-  const int seg = blockIdx.x, row = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const double* sums = a.seg_sum + static_cast<size_t>(row) * a.segs;
+  if (lane == 0) dred[wave] = part;
+  __syncthreads();  // (the staged exponentials are complete, too)
+  const double own = (dred[0] + dred[1]) + (dred[2] + dred[3]);
+  double* sums = a.seg_sum + static_cast<size_t>(row) * a.segs;
+  if (tid == 0) store_sum_bits(sums + seg, static_cast<unsigned long long>(__double_as_longlong(own)));
+  // the sums of the segments before this one
   double before = 0.0;
-  for (int s = tid; s < seg; s += kSegBlock) before += sums[s];
+  bool gave_up = false;
+  for (int sg = tid; sg < seg; sg += kSegBlock) {
+    unsigned long long bits = load_sum_bits(sums + sg);
+    for (int spins = 0; bits == kSumNotReady && spins < kSumPollLimit; ++spins) {
+      __builtin_amdgcn_s_sleep(1);
+      bits = load_sum_bits(sums + sg);
+    }
+    if (bits == kSumNotReady) gave_up = true;
+    else before += __longlong_as_double(static_cast<long long>(bits));
+  }
+  gave_up = __syncthreads_or(gave_up ? 1 : 0) != 0;  // (also: every thread has read dred)
   before = wave_sum<double>(before);
   if (lane == 0) dred[wave] = before;
   __syncthreads();
   before = (dred[0] + dred[1]) + (dred[2] + dred[3]);
-  const int first = seg * kSegElems;
   const int n = a.vocab - first < kSegElems ? a.vocab - first : kSegElems;
+  int4* rec = a.seg_step + static_cast<size_t>(row) * a.segs + seg;
+  if (gave_up) {
+    if (tid < kSegSubs) a.sub_se[(static_cast<size_t>(row) * a.segs + seg) * kSegSubs + tid] = -1;
+    if (tid == 0) *rec = make_int4(0, 0, -2, 0);
+    return;
+  }
   const double lo = before * (1.0 - seq_drift(first));
-  const double hi = (before + sums[seg]) * (1.0 + seq_drift(first + n));
+  const double hi = (before + own) * (1.0 + seq_drift(first + n));
   const float lo_f = __double2float_rd(lo), hi_f = __double2float_ru(hi);
   const int se = seq_decompose(lo_f).se;
-  int4* rec = a.seg_step + static_cast<size_t>(row) * a.segs + seg;
   const bool known = lo_f > 0.0f && hi_f < 3.0e38f && seq_decompose(hi_f).se == se;
-  const float* erow = a.e + static_cast<size_t>(row) * a.e_stride + first;
-  // thread t continues with elements 16 t .. 16 t + 15 of the segment: four 128-bit loads (the rows of
-  // exponentials and the segments start 16-byte aligned); only a segment cut short by the end of the row goes
-  // element by element.  (Requesting them before the sums above are waited for measured slower.)
+  // thread t continues with elements 16 t .. 16 t + 15 of the segment (zeros past the end of the row)
   float ev[kSegPer];
-  if (n == kSegElems) {
 #pragma unroll
-    for (int j = 0; j < kSegPer; j += 4) {
-      const float4 q = *reinterpret_cast<const float4*>(erow + tid * kSegPer + j);
-      ev[j] = q.x, ev[j + 1] = q.y, ev[j + 2] = q.z, ev[j + 3] = q.w;
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < kSegPer; ++j) ev[j] = tid * kSegPer + j < n ? erow[tid * kSegPer + j] : 0.0f;
+  for (int j = 0; j < kSegPer; j += 4) {
+    const float4 q = *reinterpret_cast<const float4*>(stage + tid * kSegPer + j);
+    ev[j] = q.x, ev[j + 1] = q.y, ev[j + 2] = q.z, ev[j + 3] = q.w;
   }
   if (!known) {
     // Powers of two may fall inside the segment.  Each of its 64-element parts (four lanes of sixteen elements)
@@ -140,18 +164,21 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs
     // estimate was wrong.
     constexpr int kPart = kSegElems / kSegSubs;
     static_assert(kPart == 4 * kSegPer && kSegBlock == kSegSubs * 4, "a part is four lanes");
-    __shared__ double part_sum[kSegSubs];
+    __shared__ double wave_parts[4];
     double mine = 0.0;
 #pragma unroll
     for (int j = 0; j < kSegPer; ++j) mine += static_cast<double>(ev[j]);
     mine += __shfl_xor(mine, 1, 64);
     mine += __shfl_xor(mine, 2, 64);  // all four lanes of a part hold its sum
-    const int part = tid >> 2;
-    if ((lane & 3) == 0) part_sum[part] = mine;
+    const int part_i = tid >> 2;
+    // the sum of the parts before this one: a prefix over the wave's sixteen parts and the totals of the waves before
+    const double upto = wave_prefix_sum<double>((lane & 3) == 0 ? mine : 0.0);
+    if (lane == 63) wave_parts[wave] = upto;
     __syncthreads();
     double start = before;
-    for (int q = 0; q < part; ++q) start += part_sum[q];
-    const int p_first = first + part * kPart;
+    for (int w = 0; w < wave; ++w) start += wave_parts[w];
+    start += upto - mine;
+    const int p_first = first + part_i * kPart;
     const float plo = __double2float_rd(start * (1.0 - seq_drift(p_first)));
     const float phi = __double2float_ru((start + mine) * (1.0 + seq_drift(p_first + kPart)));
     int pse = seq_decompose(plo).se;
@@ -167,7 +194,7 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_step_kernel(const SeqSumArgs
     lo_step = quad_scan_steps(lo_step);
     hi_step = quad_scan_steps(hi_step);
     if ((lane & 3) == 3) {
-      const size_t at = (static_cast<size_t>(row) * a.segs + seg) * kSegSubs + part;
+      const size_t at = (static_cast<size_t>(row) * a.segs + seg) * kSegSubs + part_i;
       a.sub_step[at] = make_int4(static_cast<int>(lo_step.d0), static_cast<int>(lo_step.d1), static_cast<int>(hi_step.d0),
                                  static_cast<int>(hi_step.d1));
       a.sub_se[at] = pse;
@@ -275,6 +302,9 @@ __global__ __launch_bounds__(64 * kWalkWaves) void seqsum_walk_kernel(const SeqS
     }
     max_score = key_to_float(wave_max<uint32_t>(m));
   }
+  // (the row's segment sums have served: back to "not written" for the next launch)
+  for (int sg = static_cast<int>(threadIdx.x) - 64; sg >= 0 && sg < a.segs; sg += 64 * (kWalkWaves - 1))
+    store_sum_bits(a.seg_sum + rbase + sg, kSumNotReady);
   const float* erow = a.e + static_cast<size_t>(row) * a.e_stride;
   float s = 0.0f;
   for (int g0 = 0; g0 < a.segs; g0 += 64) {  // groups of 64 segments, one per lane
@@ -448,15 +478,14 @@ extern "C" hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, int h
   const dim3 grid(a->segs, a->rows), block(ms::kSegBlock);
   if (dtype == MI355X_F16) {
     if (!have_seg_max) hipLaunchKernelGGL(ms::seqsum_max_kernel<uint16_t>, grid, block, 0, stream, *a);
-    hipLaunchKernelGGL(ms::seqsum_exp_kernel<uint16_t>, grid, block, 0, stream, *a);
+    hipLaunchKernelGGL(ms::seqsum_exp_step_kernel<uint16_t>, grid, block, 0, stream, *a);
   } else if (dtype == MI355X_BF16) {
     if (!have_seg_max) hipLaunchKernelGGL(ms::seqsum_max_kernel<ms::bf16_t>, grid, block, 0, stream, *a);
-    hipLaunchKernelGGL(ms::seqsum_exp_kernel<ms::bf16_t>, grid, block, 0, stream, *a);
+    hipLaunchKernelGGL(ms::seqsum_exp_step_kernel<ms::bf16_t>, grid, block, 0, stream, *a);
   } else {
     if (!have_seg_max) hipLaunchKernelGGL(ms::seqsum_max_kernel<float>, grid, block, 0, stream, *a);
-    hipLaunchKernelGGL(ms::seqsum_exp_kernel<float>, grid, block, 0, stream, *a);
+    hipLaunchKernelGGL(ms::seqsum_exp_step_kernel<float>, grid, block, 0, stream, *a);
   }
-  hipLaunchKernelGGL(ms::seqsum_step_kernel, grid, block, 0, stream, *a);
   hipLaunchKernelGGL(ms::seqsum_walk_kernel, dim3(a->rows), dim3(64 * ms::kWalkWaves), 0, stream, *a);
   return hipGetLastError();
 }
