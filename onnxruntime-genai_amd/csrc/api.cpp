@@ -517,7 +517,7 @@ int mi355x_softmax(mi355x_search_ctx* ctx, void* stream, float* scores, int64_t 
   ms::SeqSumArgs q{};
   if (FillSeqSum(ctx, scores, row_stride, rows, vocab, 1.0f / temperature, &q)) {
     // long rows: the exact sum is spread over the whole GPU, then an element-wise pass finishes
-    HIP_TRY(ms_launch_seqsum(&q, MI355X_F32, 0, s));
+    HIP_TRY(ms_launch_seqsum(&q, MI355X_F32, s));
     HIP_TRY(ms_launch_softmax_apply(scores, row_stride, &q, log_softmax, s));
   } else {
     HIP_TRY(ms_launch_softmax(scores, row_stride, rows, vocab, temperature, log_softmax, s));
@@ -561,18 +561,19 @@ int BeamSelectImpl(mi355x_search_ctx* ctx, void* stream, const void* logits, int
     a.row_max = q.out_max;
     a.row_sum = q.out_sum;
     if (static_cast<long long>(beams) * q.segs * 2 * beams <= ms::kBeamFinCap) {
-      // long rows: the segments list their best logits while the maxima are taken, the exact sums follow,
-      // and one workgroup per batch entry scores the listed candidates
+      // long rows: the segments list their best logits inside the launch that writes their exponentials, the
+      // exact sums follow, and one workgroup per batch entry scores the listed candidates
       a.seg_cand = ctx->seg_cand;
       a.seg_max = q.seg_max;
       a.segs = q.segs;
-      HIP_TRY(ms_launch_beam_segments(&a, dtype, static_cast<hipStream_t>(stream)));
-      HIP_TRY(ms_launch_seqsum(&q, dtype, 1, static_cast<hipStream_t>(stream)));
+      HIP_TRY(ms_launch_seqsum_max(&q, dtype, static_cast<hipStream_t>(stream)));
+      HIP_TRY(ms_launch_beam_exp_step(&q, &a, dtype, static_cast<hipStream_t>(stream)));
+      HIP_TRY(ms_launch_seqsum_walk(&q, static_cast<hipStream_t>(stream)));
       HIP_TRY(ms_launch_beam_finish(&a, dtype, step, static_cast<hipStream_t>(stream)));
       if (fused) *fused = step != nullptr;
       return MI355X_OK;
     }
-    HIP_TRY(ms_launch_seqsum(&q, dtype, 0, static_cast<hipStream_t>(stream)));
+    HIP_TRY(ms_launch_seqsum(&q, dtype, static_cast<hipStream_t>(stream)));
   }
   HIP_TRY(ms_launch_beam_select(&a, dtype, static_cast<hipStream_t>(stream)));
   return MI355X_OK;

@@ -4,6 +4,7 @@
 #include "block_seq.h"
 #include "wave_select.h"
 #include "seg_io.h"
+#include "seqsum_exp_step.h"
 
 namespace ms {
 
@@ -367,8 +368,8 @@ __global__ __launch_bounds__(64) void beam_scorer_finalize_kernel(const ScorerSt
 //
 // The final score ((x - max) - log(sum)) + beam_score is a non-decreasing function of the logit x, so the
 // 2*beams best final scores of a batch entry belong to elements that are among the 2*beams largest logits of
-// their own segment.  beam_seg_kernel lists those per segment (and writes the segment maxima the exact sum
-// needs, which saves that kernel's own pass); beam_fin_kernel scores the listed elements and keeps the best by
+// their own segment.  SegmentLists lists those per segment (inside the exact sum's launch that holds the
+// segment's logits in registers anyway); beam_fin_kernel scores the listed elements and keeps the best by
 // (final score desc, beam * vocab + token asc), the order of the flat partial_sort of src/search.cpp:148-163.
 // Rounding can give different logits the same final score, and then the lowest index wins, which the logit
 // order does not know.  A segment whose list is full (it may hold more elements of the same final score as its
@@ -378,57 +379,67 @@ __global__ __launch_bounds__(64) void beam_scorer_finalize_kernel(const ScorerSt
 constexpr int kSegCandCap = 512;        // candidates a segment may list before it reports an overflow
 constexpr u64 kSegOverflow = ~0ull;     // first entry of a segment that listed more than kSegCandCap
 
+// Runs inside the launch that writes the exponentials, while a segment's workgroup waits for the sums of the
+// segments before it: v are the segment's logits as that launch loaded them (zeros past the end of the row).
 template <typename InT>
-__global__ __launch_bounds__(kSegBlock) void beam_seg_kernel(const BeamArgs a) {
-  __shared__ u64 list[kSegCandCap];
-  __shared__ uint32_t pool[64];
-  __shared__ uint32_t red[4];
-  __shared__ uint32_t count;
-  const int seg = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
-  const int V = a.vocab, m = 2 * a.beams;
-  const InT* x = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
-  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
-  float v[kSegPer];
-  seg_load<InT>(x, aligned, V, seg, -__builtin_inff(), v);
-  float fm = -__builtin_inff();
+struct SegmentLists {
+  BeamArgs a;
+  __device__ __forceinline__ void operator()(const float (&v)[kSegPer], int seg, int row) const {
+    __shared__ u64 list[kSegCandCap];
+    __shared__ uint32_t pool[64];
+    __shared__ uint32_t count;
+    const int tid = threadIdx.x;
+    const int V = a.vocab, m = 2 * a.beams;
+    float fm = -__builtin_inff();
 #pragma unroll
-  for (int e = 0; e < kSegPer; ++e) fm = fmaxf(fm, v[e]);
-  const uint32_t mkey = order_key(fm);
-  const uint32_t smax = block_max<uint32_t>(mkey, red);
-  if (tid == 0) a.seg_max[static_cast<size_t>(row) * a.segs + seg] = smax;
-  const uint32_t offer = seg_index<InT>(seg, 0) < V ? mkey : 0u;  // threads past the end of the row offer nothing
-  const uint32_t tau = block_pool_bound(offer, m, kSegBlock / 64, pool);
-  if (tid == 0) count = 0u;
-  __syncthreads();
+    for (int e = 0; e < kSegPer; ++e)
+      if (seg_index<InT>(seg, e) < V) fm = fmaxf(fm, v[e]);
+    const uint32_t offer = seg_index<InT>(seg, 0) < V ? order_key(fm) : 0u;  // threads past the end of the row offer nothing
+    const uint32_t tau = block_pool_bound(offer, m, kSegBlock / 64, pool);
+    if (tid == 0) count = 0u;
+    __syncthreads();
+    // a thread's candidates are counted first, so that a wave asks for its list positions once
+    uint32_t mine = 0u;
 #pragma unroll
-  for (int e = 0; e < kSegPer; ++e) {
-    const int idx = seg_index<InT>(seg, e);
-    const uint32_t k = order_key(v[e]);
-    const bool cand = idx < V && (tau == 0u || k >= tau);  // tau == 0: fewer than m offers, list everything
-    const uint32_t pos = wave_slot(cand, &count);
-    if (cand && pos < kSegCandCap) list[pos] = make_key64(k, static_cast<uint32_t>(idx));
-  }
-  __syncthreads();
-  const int n = static_cast<int>(count);
-  u64* out = a.seg_cand + (static_cast<size_t>(row) * a.segs + seg) * m;
-  if (n > kSegCandCap) {
-    if (tid < m) out[tid] = tid == 0 ? kSegOverflow : 0ull;
-    return;
-  }
-  if (n <= 64) {  // the usual case: one wave sorts the list in registers
-    if (tid < 64) {
-      const u64 k = wave_sort_desc_fast<u64>(tid < n ? list[tid] : 0ull);
-      if (tid < m) out[tid] = k;
+    for (int e = 0; e < kSegPer; ++e) {
+      const bool cand = seg_index<InT>(seg, e) < V && (tau == 0u || order_key(v[e]) >= tau);  // tau == 0: fewer than m offers, list everything
+      mine |= cand ? 1u << e : 0u;
     }
-    return;
+    const uint32_t n_mine = static_cast<uint32_t>(__popc(mine));
+    const uint32_t upto = wave_prefix_sum<uint32_t>(n_mine);
+    const uint32_t n_wave = wave_read_lane(upto, 63);
+    uint32_t pos = 0u;
+    if (n_wave != 0u) {
+      if ((tid & 63) == 0) pos = atomicAdd(&count, n_wave);
+      pos = wave_read_lane(pos, 0) + upto - n_mine;
+    }
+#pragma unroll
+    for (int e = 0; e < kSegPer; ++e) {
+      if ((mine >> e) & 1u) {
+        if (pos < kSegCandCap) list[pos] = make_key64(order_key(v[e]), static_cast<uint32_t>(seg_index<InT>(seg, e)));
+        ++pos;
+      }
+    }
+    __syncthreads();
+    const int n = static_cast<int>(count);
+    u64* out = a.seg_cand + (static_cast<size_t>(row) * a.segs + seg) * m;
+    if (n > kSegCandCap) {
+      if (tid < m) out[tid] = tid == 0 ? kSegOverflow : 0ull;
+    } else if (n <= 64) {  // the usual case: one wave sorts the list in registers
+      if (tid < 64) {
+        const u64 k = wave_sort_desc_fast<u64>(tid < n ? list[tid] : 0ull);
+        if (tid < m) out[tid] = k;
+      }
+    } else {
+      int n2 = 128;
+      while (n2 < n) n2 <<= 1;
+      for (int p = n + tid; p < n2; p += kSegBlock) list[p] = 0ull;
+      __syncthreads();
+      block_sort_desc(list, n2);
+      if (tid < m) out[tid] = list[tid];
+    }
   }
-  int n2 = 128;
-  while (n2 < n) n2 <<= 1;
-  for (int p = n + tid; p < n2; p += kSegBlock) list[p] = 0ull;
-  __syncthreads();
-  block_sort_desc(list, n2);
-  if (tid < m) out[tid] = list[tid];
-}
+};
 
 // SCORER: the entry's workgroup goes on with the entry's scorer step (scorer_entry, by its first wave, from the
 // candidates in LDS); the tests that need every entry's candidates are left to the workgroup that gets through last.
@@ -621,14 +632,18 @@ __global__ __launch_bounds__(256) void beam_fin_kernel(const BeamArgs a, const S
 
 }  // namespace ms
 
-extern "C" hipError_t ms_launch_beam_segments(const ms::BeamArgs* a, int dtype, hipStream_t stream) {
-  const dim3 grid(a->segs, a->batch * a->beams), block(ms::kSegBlock);
+// The exact sums' second launch (exponentials, step records) with the segments' candidate lists built in it.
+extern "C" hipError_t ms_launch_beam_exp_step(const ms::SeqSumArgs* q, const ms::BeamArgs* a, int dtype, hipStream_t stream) {
+  const dim3 grid(q->segs, q->rows), block(ms::kSegBlock);
   if (dtype == MI355X_F16)
-    hipLaunchKernelGGL(ms::beam_seg_kernel<uint16_t>, grid, block, 0, stream, *a);
+    hipLaunchKernelGGL((ms::seqsum_exp_step_kernel<uint16_t, ms::SegmentLists<uint16_t>>), grid, block, 0, stream, *q,
+                       ms::SegmentLists<uint16_t>{*a});
   else if (dtype == MI355X_BF16)
-    hipLaunchKernelGGL(ms::beam_seg_kernel<ms::bf16_t>, grid, block, 0, stream, *a);
+    hipLaunchKernelGGL((ms::seqsum_exp_step_kernel<ms::bf16_t, ms::SegmentLists<ms::bf16_t>>), grid, block, 0, stream, *q,
+                       ms::SegmentLists<ms::bf16_t>{*a});
   else
-    hipLaunchKernelGGL(ms::beam_seg_kernel<float>, grid, block, 0, stream, *a);
+    hipLaunchKernelGGL((ms::seqsum_exp_step_kernel<float, ms::SegmentLists<float>>), grid, block, 0, stream, *q,
+                       ms::SegmentLists<float>{*a});
   return hipGetLastError();
 }
 

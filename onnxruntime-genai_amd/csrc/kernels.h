@@ -212,10 +212,12 @@ hipError_t ms_launch_cast(const void* in, void* out, size_t count, int kind, hip
 hipError_t ms_launch_logits_handoff(const void* raw, int kind, int rows, int seq_len, int vocab,
                                     const int32_t* token_index, float* out, int64_t out_stride, hipStream_t stream);
 hipError_t ms_launch_beam_select(const ms::BeamArgs* a, int dtype, hipStream_t stream);
-hipError_t ms_launch_beam_segments(const ms::BeamArgs* a, int dtype, hipStream_t stream);
+hipError_t ms_launch_beam_exp_step(const ms::SeqSumArgs* q, const ms::BeamArgs* a, int dtype, hipStream_t stream);
 // step != null: every batch entry's workgroup goes on with the entry's scorer step (ms_launch_scorer_step's work).
 hipError_t ms_launch_beam_finish(const ms::BeamArgs* a, int dtype, const ms::ScorerStep* step, hipStream_t stream);
-hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, int have_seg_max, hipStream_t stream);
+hipError_t ms_launch_seqsum(const ms::SeqSumArgs* a, int dtype, hipStream_t stream);  // its three launches
+hipError_t ms_launch_seqsum_max(const ms::SeqSumArgs* a, int dtype, hipStream_t stream);
+hipError_t ms_launch_seqsum_walk(const ms::SeqSumArgs* a, hipStream_t stream);
 hipError_t ms_launch_softmax_apply(float* scores, int64_t row_stride, const ms::SeqSumArgs* a, int log_softmax,
                                    hipStream_t stream);
 hipError_t ms_launch_scorer_step(const ms::ScorerState* s, const int32_t* sequences, int32_t* sequences_next,
