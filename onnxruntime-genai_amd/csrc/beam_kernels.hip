@@ -29,6 +29,10 @@ __device__ __forceinline__ void row_for_each(const InT* x, int V, Fn fn) {
         if constexpr (VEC == 4) {
 #pragma unroll
           for (int c = 0; c < 4; ++c) v[r][c] = __uint_as_float(w[c]);
+        } else if constexpr (__is_same(InT, uint16_t)) {
+          v4u qq;
+          qq.x = q.x, qq.y = q.y, qq.z = q.z, qq.w = q.w;
+          widen_half8(qq, v[r]);
         } else {
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
@@ -384,25 +388,37 @@ constexpr u64 kSegOverflow = ~0ull;     // first entry of a segment that listed 
 template <typename InT>
 struct SegmentLists {
   BeamArgs a;
-  __device__ __forceinline__ void operator()(const float (&v)[kSegPer], int seg, int row) const {
-    __shared__ u64 list[kSegCandCap];
-    __shared__ uint32_t pool[64];
-    __shared__ uint32_t count;
+  struct Shared {
+    u64 list[kSegCandCap];
+    uint32_t wave_bound[kSegBlock / 64];
+    uint32_t count;
+  };
+  template <bool FULL>
+  __device__ __forceinline__ void run(Shared& sh, const float (&v)[kSegPer], int seg, int row) const {
+    u64* const list = sh.list;
+    uint32_t* const wave_bound = sh.wave_bound;
+    uint32_t& count = sh.count;
     const int tid = threadIdx.x;
     const int V = a.vocab, m = 2 * a.beams;
     float fm = -__builtin_inff();
 #pragma unroll
     for (int e = 0; e < kSegPer; ++e)
-      if (seg_index<InT>(seg, e) < V) fm = fmaxf(fm, v[e]);
-    const uint32_t offer = seg_index<InT>(seg, 0) < V ? order_key(fm) : 0u;  // threads past the end of the row offer nothing
-    const uint32_t tau = block_pool_bound(offer, m, kSegBlock / 64, pool);
+      if (FULL || seg_index<InT>(seg, e) < V) fm = fmaxf(fm, v[e]);
+    const uint32_t offer = (FULL || seg_index<InT>(seg, 0) < V) ? order_key(fm) : 0u;  // threads past the end of the row offer nothing
+    // A wave's m-th best thread maximum (0 with fewer than m offers) has m of the wave's elements at or above it;
+    // so has the largest of the four, and with it everything that can be among the segment's m best.
+    const uint32_t mth = wave_read_lane(wave_sort_desc_fast<uint32_t>(offer), m - 1);
+    if ((tid & 63) == 0) wave_bound[tid >> 6] = mth;
     if (tid == 0) count = 0u;
     __syncthreads();
+    uint32_t tau = wave_bound[0];
+#pragma unroll
+    for (int w = 1; w < kSegBlock / 64; ++w) tau = wave_bound[w] > tau ? wave_bound[w] : tau;
     // a thread's candidates are counted first, so that a wave asks for its list positions once
     uint32_t mine = 0u;
 #pragma unroll
     for (int e = 0; e < kSegPer; ++e) {
-      const bool cand = seg_index<InT>(seg, e) < V && (tau == 0u || order_key(v[e]) >= tau);  // tau == 0: fewer than m offers, list everything
+      const bool cand = (FULL || seg_index<InT>(seg, e) < V) && (tau == 0u || order_key(v[e]) >= tau);  // tau == 0: fewer than m offers, list everything
       mine |= cand ? 1u << e : 0u;
     }
     const uint32_t n_mine = static_cast<uint32_t>(__popc(mine));

@@ -28,11 +28,15 @@ __device__ __forceinline__ void seg_load(const InT* row, bool aligned, int vocab
         v[j * 4] = q.x, v[j * 4 + 1] = q.y, v[j * 4 + 2] = q.z, v[j * 4 + 3] = q.w;
       } else {
         const v4u q = *reinterpret_cast<const v4u*>(row + i0);
-        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        if constexpr (__is_same(InT, uint16_t)) {
+          widen_half8(q, &v[j * 8]);  // the hardware conversion, redone by the bit formula where it differs
+        } else {
+          const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          v[j * 8 + 2 * c] = narrow_bits_to_float<InT>(w[c] & 0xffffu);
-          v[j * 8 + 2 * c + 1] = narrow_bits_to_float<InT>(w[c] >> 16);
+          for (int c = 0; c < 4; ++c) {
+            v[j * 8 + 2 * c] = narrow_bits_to_float<InT>(w[c] & 0xffffu);
+            v[j * 8 + 2 * c + 1] = narrow_bits_to_float<InT>(w[c] >> 16);
+          }
         }
       }
     } else {

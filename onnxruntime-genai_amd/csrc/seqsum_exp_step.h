@@ -46,22 +46,37 @@ __device__ __forceinline__ double seq_drift(int count) {
 // `between(v, seg, row)` runs, in all threads, after the sum is out and before the earlier sums are needed: work
 // on the segment's elements v (as loaded: zeros past the end of the row) that would otherwise wait for a launch of
 // its own.
+// FULL: the segment lies inside the row (all but a row's last segment do), so nothing has to ask where the row ends.
+// `Shared` is what it needs of LDS (declared once, by the kernel, for both forms of the body).
 struct NothingBetween {
-  __device__ __forceinline__ void operator()(const float (&)[kSegPer], int, int) const {}
+  struct Shared {};
+  template <bool FULL>
+  __device__ __forceinline__ void run(Shared&, const float (&)[kSegPer], int, int) const {}
 };
 
-template <typename InT, typename Between>
-__global__ __launch_bounds__(kSegBlock) void seqsum_exp_step_kernel(const SeqSumArgs a, const Between between) {
-  __shared__ uint32_t red[4];
-  __shared__ double dred[4];
-  __shared__ uint64_t exp_tab[32];  // the table of expf in LDS: a lookup per element from constant memory is a gather
-  __shared__ __align__(16) float stage[kSegElems];  // the segment's exponentials in element order
-  __shared__ Step wave_tot[4];
+struct ExpStepShared {
+  uint32_t red[4];
+  double dred[4];
+  uint64_t exp_tab[32];  // the table of expf in LDS: a lookup per element from constant memory is a gather
+  __align__(16) float stage[kSegElems];  // the segment's exponentials in element order
+  Step wave_tot[4];
+  double wave_parts[4];
+};
+
+template <typename InT, typename Between, bool FULL>
+__device__ __forceinline__ void seqsum_exp_step_body(const SeqSumArgs& a, const Between& between, ExpStepShared& sh,
+                                                     typename Between::Shared& between_sh) {
+  uint32_t* const red = sh.red;
+  double* const dred = sh.dred;
+  uint64_t* const exp_tab = sh.exp_tab;
+  float* const stage = sh.stage;
+  Step* const wave_tot = sh.wave_tot;
+  double* const wave_parts = sh.wave_parts;
   const int seg = blockIdx.x, row = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const InT* x = static_cast<const InT*>(a.x) + static_cast<size_t>(row) * a.row_stride;
   const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
   float v[kSegPer];
-  seg_load<InT>(x, aligned, a.vocab, seg, 0.0f, v);
+  seg_load<InT>(x, aligned, FULL ? (seg + 1) * kSegElems : a.vocab, seg, 0.0f, v);
   if (tid < 32) exp_tab[tid] = em::exp2_tab(static_cast<uint32_t>(tid));
   const float max_score = row_max_of_segments(a, row, red);  // its barriers also publish the table
   const uint64_t* const tab = exp_tab;
@@ -77,13 +92,13 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_step_kernel(const SeqSum
     float ex[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      ex[c] = idx + c < a.vocab ? em::expf_core((v[e0 + c] - max_score) * a.inv_temp, lds_tab) : 0.0f;
+      ex[c] = (FULL || idx + c < a.vocab) ? em::expf_core((v[e0 + c] - max_score) * a.inv_temp, lds_tab) : 0.0f;
       part += static_cast<double>(ex[c]);
     }
     v4f q;
     q.x = ex[0], q.y = ex[1], q.z = ex[2], q.w = ex[3];
     *reinterpret_cast<v4f*>(stage + (idx - first)) = q;
-    if (idx + 4 <= a.vocab) {
+    if (FULL || idx + 4 <= a.vocab) {
       *reinterpret_cast<v4f*>(erow + idx) = q;
     } else {
 #pragma unroll
@@ -97,7 +112,7 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_step_kernel(const SeqSum
   const double own = (dred[0] + dred[1]) + (dred[2] + dred[3]);
   double* sums = a.seg_sum + static_cast<size_t>(row) * a.segs;
   if (tid == 0) store_sum_bits(sums + seg, static_cast<unsigned long long>(__double_as_longlong(own)));
-  between(v, seg, row);
+  between.template run<FULL>(between_sh, v, seg, row);
   // the sums of the segments before this one
   double before = 0.0;
   bool gave_up = false;
@@ -115,7 +130,7 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_step_kernel(const SeqSum
   if (lane == 0) dred[wave] = before;
   __syncthreads();
   before = (dred[0] + dred[1]) + (dred[2] + dred[3]);
-  const int n = a.vocab - first < kSegElems ? a.vocab - first : kSegElems;
+  const int n = FULL ? kSegElems : a.vocab - first;
   int4* rec = a.seg_step + static_cast<size_t>(row) * a.segs + seg;
   if (gave_up) {
     if (tid < kSegSubs) a.sub_se[(static_cast<size_t>(row) * a.segs + seg) * kSegSubs + tid] = -1;
@@ -142,7 +157,6 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_step_kernel(const SeqSum
     // estimate was wrong.
     constexpr int kPart = kSegElems / kSegSubs;
     static_assert(kPart == 4 * kSegPer && kSegBlock == kSegSubs * 4, "a part is four lanes");
-    __shared__ double wave_parts[4];
     double mine = 0.0;
 #pragma unroll
     for (int j = 0; j < kSegPer; ++j) mine += static_cast<double>(ev[j]);
@@ -191,6 +205,16 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_exp_step_kernel(const SeqSum
     for (int w = 1; w < 4; ++w) t = step_compose(t, wave_tot[w]);
     *rec = make_int4(static_cast<int>(t.d0), static_cast<int>(t.d1), se, 0);
   }
+}
+
+template <typename InT, typename Between>
+__global__ __launch_bounds__(kSegBlock) void seqsum_exp_step_kernel(const SeqSumArgs a, const Between between) {
+  __shared__ ExpStepShared sh;
+  __shared__ typename Between::Shared between_sh;
+  if ((static_cast<int>(blockIdx.x) + 1) * kSegElems <= a.vocab)
+    seqsum_exp_step_body<InT, Between, true>(a, between, sh, between_sh);
+  else
+    seqsum_exp_step_body<InT, Between, false>(a, between, sh, between_sh);
 }
 
 }  // namespace ms
