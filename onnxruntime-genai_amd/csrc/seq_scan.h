@@ -83,4 +83,28 @@ EM_HD Step seq_make_step(float e, int se) {
   return f;
 }
 
+// The composition of the step functions of e[0..count) (finite, >= 0) under the unit 2^(se-150), read off real
+// float additions in one go: within a binade the rounding of an addition depends only on the addend and on the
+// parity of the sum's mantissa integer, so all even sums of the binade run through the same sequence of
+// parities and increments as its first even value does, and all odd ones as its first odd value does.  The two
+// are added up for real; where such a sum lands in a higher binade (it cannot come back: the addends are not
+// negative) the composition is reported as saturated, which the composition of the single steps would carry to
+// 2^24 or beyond from every start of that parity as well.
+EM_HD Step seq_compose_run(const float* e, int count, int se) {
+  const uint32_t b0 = static_cast<uint32_t>(se) << 23;
+  const uint32_t b1 = b0 | 1u;
+  float f0 = em::as_float(b0), f1 = em::as_float(b1);
+#pragma unroll
+  for (int j = 0; j < count; ++j) {
+    f0 = f0 + e[j];
+    f1 = f1 + e[j];
+  }
+  const uint32_t r0 = em::as_u32(f0), r1 = em::as_u32(f1);
+  const uint32_t lim = b0 + 0x800000u;  // first bit pattern of the next binade
+  Step f;
+  f.d0 = r0 < lim ? r0 - b0 : kStepSat;
+  f.d1 = r1 < lim ? r1 - b1 : kStepSat;
+  return f;
+}
+
 }  // namespace ms

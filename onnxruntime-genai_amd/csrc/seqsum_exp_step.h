@@ -177,11 +177,8 @@ __device__ __forceinline__ void seqsum_exp_step_body(const SeqSumArgs& a, const 
     if (!(plo > 0.0f && phi < 3.0e38f && seq_decompose(phi).se <= pse + 1)) pse = -1;  // the walk adds this part itself
     Step lo_step{0u, 0u}, hi_step{0u, 0u};
     if (pse >= 0) {
-#pragma unroll
-      for (int j = 0; j < kSegPer; ++j) {
-        lo_step = step_compose(lo_step, seq_make_step(ev[j], pse));
-        hi_step = step_compose(hi_step, seq_make_step(ev[j], pse + 1));
-      }
+      lo_step = seq_compose_run(ev, kSegPer, pse);
+      hi_step = seq_compose_run(ev, kSegPer, pse + 1);
     }
     lo_step = quad_scan_steps(lo_step);
     hi_step = quad_scan_steps(hi_step);
@@ -194,9 +191,7 @@ __device__ __forceinline__ void seqsum_exp_step_body(const SeqSumArgs& a, const 
     if (tid == 0) *rec = make_int4(0, 0, -2, 0);
     return;
   }
-  Step agg{0u, 0u};
-#pragma unroll
-  for (int j = 0; j < kSegPer; ++j) agg = step_compose(agg, seq_make_step(ev[j], se));
+  const Step agg = seq_compose_run(ev, kSegPer, se);
   const Step inc = wave_scan_steps(agg);
   if (lane == 63) wave_tot[wave] = inc;
   __syncthreads();

@@ -55,6 +55,48 @@ static bool run_case(const std::vector<float>& e, float s0, int window, bool tre
   return true;
 }
 
+// The same with every `group` consecutive addends turned into one step function by seq_compose_run (real float
+// additions from the binade's first even and first odd value), as the kernels that only need a thread's aggregate do:
+// checked where a group ends; a group in which the sum leaves the binade is added element by element.
+static bool run_case_groups(const std::vector<float>& e, float s0, int window, int group) {
+  const int n = (int)e.size();
+  std::vector<float> want(n);
+  {
+    volatile float s = s0;
+    for (int i = 0; i < n; ++i) { s = s + e[i]; want[i] = s; }
+  }
+  float s = s0;
+  int i0 = 0;
+  while (i0 < n) {
+    const int cnt = std::min(window * group, n - i0);
+    const int groups = (cnt + group - 1) / group;
+    const SeqState st = seq_decompose(s);
+    Step acc{0, 0};
+    int cross = -1;
+    uint32_t before = st.n;
+    for (int g = 0; g < groups; ++g) {
+      const int len = std::min(group, cnt - g * group);
+      acc = step_compose(acc, seq_compose_run(&e[i0 + g * group], len, st.se));
+      const uint32_t na = step_apply(st.n, acc);
+      if (na >= kMantLimit) { cross = g; break; }
+      if (em::as_u32(seq_recompose(na, st.se)) != em::as_u32(want[i0 + g * group + len - 1])) return false;
+      before = na;
+    }
+    if (cross < 0) {
+      s = seq_recompose(before, st.se);
+      i0 += cnt;
+    } else {
+      volatile float t = cross ? seq_recompose(before, st.se) : s;
+      const int len = std::min(group, cnt - cross * group);
+      for (int j = 0; j < len; ++j) t = t + e[i0 + cross * group + j];
+      s = t;
+      if (em::as_u32(s) != em::as_u32(want[i0 + cross * group + len - 1])) return false;
+      i0 += cross * group + len;
+    }
+  }
+  return true;
+}
+
 int main() {
   std::mt19937_64 rng(12345);
   std::normal_distribution<float> nd(0.f, 1.f);
@@ -82,7 +124,8 @@ int main() {
     const int window = 1 + (int)(rng() % 700);
     bad += !run_case(e, s0, window, false);
     bad += !run_case(e, s0, window, true);
-    cases += 2;
+    bad += !run_case_groups(e, s0, 1 + window % 64, rep % 3 == 0 ? 16 : 1 + (int)(rng() % 40));
+    cases += 3;
   }
   printf("%ld %ld\n", bad, cases);
   return 0;
