@@ -1,7 +1,8 @@
 """Every benchmark configuration at its FULL size, one step each, through the C ABI against the CPU oracle
 (configuration 2 and the selection phase of 3 are covered at full size in test_gpu_sampling.py /
 test_gpu_beam_spec.py; here: all 256 rows of configuration 5, a heterogeneous batch of more than 64 rows
-at a 128K vocabulary, and the 56-tensor KV gather of configuration 3)."""
+at a 128K vocabulary, exact sums over more segments than the GPU runs at once, and the 56-tensor KV gather of
+configuration 3)."""
 import numpy as np
 import pytest
 import torch
@@ -71,6 +72,32 @@ def test_heterogeneous_batch_of_96_rows_at_128k_vocab(orc):
         assert np.array_equal(ki[r, :n], idx[:n]), (r, per_row[r])
         assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), (r, per_row[r])
         assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (r, per_row[r])
+    ctx.close()
+
+
+def test_exact_sums_of_more_segments_than_the_gpu_runs_at_once(orc):
+    """Log-softmax of 256 rows x 151936: 9728 segment workgroups in one launch, several times what the GPU holds
+    at once, each waiting for the sums of its row's earlier segments that the same launch publishes.  The rows repeat
+    six distinct ones (softmax-like, constant, sparse with -inf, tiny and huge spreads), so six oracle rows pin all
+    256; a second call on the same context checks the state the first one left behind."""
+    say("softmax 256 x 151936")
+    rng = np.random.default_rng(77)
+    rows, vocab = 256, 151936
+    ctx = pkg().SearchContext(rows, vocab)
+    base = np.empty((6, vocab), np.float32)
+    base[0] = rng.standard_normal(vocab) * 2
+    base[1] = -1.25
+    base[2] = np.where(rng.random(vocab) < 0.8, -np.inf, rng.standard_normal(vocab) * 4).astype(np.float32)
+    base[3] = rng.standard_normal(vocab) * 1e-4
+    base[4] = rng.standard_normal(vocab) * 40
+    base[5] = np.linspace(-30, 0, vocab)
+    want = [orc.log_softmax(base[i], 1.0) for i in range(6)]
+    pick = rng.integers(0, 6, rows)
+    x = torch.from_numpy(base[pick]).cuda()
+    for call in range(2):
+        got = ctx.softmax(x.clone(), 1.0, log=True).cpu().numpy()
+        for r in range(rows):
+            assert np.array_equal(bits(got[r]), bits(want[pick[r]])), (call, r, int(pick[r]))
     ctx.close()
 
 
