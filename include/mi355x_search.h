@@ -359,6 +359,12 @@ int mi355x_search_fallback_rows(mi355x_search_ctx* ctx, void* stream, unsigned* 
  * recovery: 0 lets every wait that is not satisfied at once give up. */
 int mi355x_search_wait_gave_up(mi355x_search_ctx* ctx, void* stream, int* gave_up);
 int mi355x_search_set_poll_limit(mi355x_search_ctx* ctx, int polls);
+/* The exact sums of long rows (mi355x_softmax, mi355x_beam_select from 16384 logits per row on) have a bounded
+ * wait of their own: a 4096-logit segment's workgroup polls, under the same limit, for the sums of the row's
+ * earlier segments, which workgroups of the same launch publish.  A wait that gives up costs time only: the
+ * segment is then added element by element, and the result is the same.  *segments = how many segments that has
+ * happened to on this context (synchronises `stream`; no counterpart in the reference). */
+int mi355x_search_sum_waits_gave_up(mi355x_search_ctx* ctx, void* stream, unsigned* segments);
 
 #ifdef __cplusplus
 }

@@ -58,6 +58,7 @@ def load_library():
     L.mi355x_search_fallback_rows.argtypes = [vp, vp, C.POINTER(C.c_uint)]
     L.mi355x_search_wait_gave_up.argtypes = [vp, vp, C.POINTER(C.c_int)]
     L.mi355x_search_set_poll_limit.argtypes = [vp, C.c_int]
+    L.mi355x_search_sum_waits_gave_up.argtypes = [vp, vp, C.POINTER(C.c_uint)]
     for name, args in {
         "mi355x_topk_scores": [vp, vp, vp, i32, i64, i32, i32, i32, vp, vp],
         "mi355x_softmax": [vp, vp, vp, i64, i32, i32, f32, i32],
@@ -179,6 +180,11 @@ class SearchContext:
         g = C.c_int()
         self._check(self.L.mi355x_search_wait_gave_up(self.h, _stream(), C.byref(g)))
         return bool(g.value)
+
+    def sum_waits_gave_up(self):
+        n = C.c_uint()
+        self._check(self.L.mi355x_search_sum_waits_gave_up(self.h, _stream(), C.byref(n)))
+        return n.value
 
     def set_poll_limit(self, polls):
         self._check(self.L.mi355x_search_set_poll_limit(self.h, int(polls)))

@@ -196,7 +196,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->big, static_cast<size_t>(max_rows) * c->big_stride, false));
   ok(c->Alloc(&c->big2, static_cast<size_t>(max_rows) * c->big_stride, false));
   ok(c->Alloc(&c->row_done, static_cast<size_t>(max_rows), true));
-  ok(c->Alloc(&c->fallback_rows, 2, true));  // [0] rows finished by the exact path, [1] a wait gave up
+  ok(c->Alloc(&c->fallback_rows, 4, true));  // [0] rows finished by the exact path, [1] a wait gave up, [2] exact-sum segments whose wait gave up
   ok(c->Alloc(&c->ban, static_cast<size_t>(max_rows) * ((max_vocab - 1) / 32 + 1), false));
   ok(c->Alloc(&c->params_dev, static_cast<size_t>(max_rows), false));
   ok(c->Alloc(&c->beam_row_scores, static_cast<size_t>(max_rows) * ms::kBeamMaxCand, false));
@@ -504,6 +504,8 @@ static bool FillSeqSum(mi355x_search_ctx* ctx, const void* x, int64_t row_stride
   q->e_stride = ctx->big_stride * 2;
   q->out_max = ctx->row_max;
   q->out_sum = ctx->row_sum;
+  q->poll_limit = ctx->poll_limit;
+  q->gave_up = ctx->fallback_rows + 2;
   return true;
 }
 
@@ -741,6 +743,14 @@ int mi355x_search_wait_gave_up(mi355x_search_ctx* ctx, void* stream, int* gave_u
                          static_cast<hipStream_t>(stream)));
   HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   *gave_up = word != 0u;
+  return MI355X_OK;
+}
+
+int mi355x_search_sum_waits_gave_up(mi355x_search_ctx* ctx, void* stream, unsigned* segments) {
+  if (!ctx || !segments) return Fail(MI355X_E_INVALID, "null argument");
+  HIP_TRY(hipMemcpyAsync(segments, ctx->fallback_rows + 2, sizeof(unsigned), hipMemcpyDeviceToHost,
+                         static_cast<hipStream_t>(stream)));
+  HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   return MI355X_OK;
 }
 

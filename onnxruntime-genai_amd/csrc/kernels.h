@@ -109,6 +109,8 @@ struct SeqSumArgs {
   size_t e_stride;
   float* out_max;     // [rows]
   float* out_sum;     // [rows]
+  int poll_limit;     // polls a segment's workgroup spends on an earlier segment's sum before it gives up
+  uint32_t* gave_up;  // counts the segments whose wait gave up
 };
 
 struct SpecSparseArgs {

@@ -20,7 +20,6 @@ __device__ __forceinline__ float row_max_of_segments(const SeqSumArgs& a, int ro
 // finite, and a NaN that came in through the logits keeps zeros in its low bits when widened to double).  The
 // buffer holds this value everywhere between launches: the walk puts it back.
 constexpr unsigned long long kSumNotReady = ~0ull;
-constexpr int kSumPollLimit = 1 << 15;
 
 __device__ __forceinline__ unsigned long long load_sum_bits(const double* p) {
   return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -118,7 +117,7 @@ __device__ __forceinline__ void seqsum_exp_step_body(const SeqSumArgs& a, const 
   bool gave_up = false;
   for (int sg = tid; sg < seg; sg += kSegBlock) {
     unsigned long long bits = load_sum_bits(sums + sg);
-    for (int spins = 0; bits == kSumNotReady && spins < kSumPollLimit; ++spins) {
+    for (int spins = 0; bits == kSumNotReady && spins < a.poll_limit; ++spins) {
       __builtin_amdgcn_s_sleep(1);
       bits = load_sum_bits(sums + sg);
     }
@@ -134,7 +133,10 @@ __device__ __forceinline__ void seqsum_exp_step_body(const SeqSumArgs& a, const 
   int4* rec = a.seg_step + static_cast<size_t>(row) * a.segs + seg;
   if (gave_up) {
     if (tid < kSegSubs) a.sub_se[(static_cast<size_t>(row) * a.segs + seg) * kSegSubs + tid] = -1;
-    if (tid == 0) *rec = make_int4(0, 0, -2, 0);
+    if (tid == 0) {
+      *rec = make_int4(0, 0, -2, 0);
+      atomicAdd(a.gave_up, 1u);
+    }
     return;
   }
   const double lo = before * (1.0 - seq_drift(first));

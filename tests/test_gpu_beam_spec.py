@@ -140,6 +140,44 @@ def test_search_step_finishes_entries_like_the_two_calls(ctx, batch, beams, voca
     big.close()
 
 
+def test_exact_sums_whose_waits_give_up(orc):
+    """Failure handling of the exact sums' look-back, forced from the host: with a poll limit of 0 a segment's
+    workgroup gives up on every earlier sum that has not arrived yet and its segment is added element by element.
+    Log-softmax and beam selection must come out bit-identical, the context must count the event, and with the
+    limit restored the same calls must be right again (and count nothing new)."""
+    say("exact sums, poll limit 0")
+    rng = np.random.default_rng(78)
+    rows, vocab, batch, beams = 24, 151936, 6, 4
+    c = pkg().SearchContext(rows, vocab)
+    try:
+        x = (rng.standard_normal((rows, vocab)) * 2).astype(np.float32)
+        bs = (rng.standard_normal(rows) * 3).astype(np.float32)
+        want = [orc.log_softmax(x[r], 1.0) for r in range(rows)]
+        wsc, wtok, widx, _ = orc.beam_select_top(x, batch, beams, bs)
+        xd, bd = torch.from_numpy(x).cuda(), torch.from_numpy(bs).cuda()
+
+        def check():
+            got = c.softmax(xd.clone(), 1.0, log=True).cpu().numpy()
+            for r in range(rows):
+                assert np.array_equal(bits(got[r]), bits(want[r])), r
+            sc, tok, idx = c.beam_select(xd, batch, beams, bd)
+            assert np.array_equal(tok.cpu().numpy(), wtok) and np.array_equal(idx.cpu().numpy(), widx)
+            assert np.array_equal(bits(sc.cpu().numpy()), bits(wsc))
+
+        check()
+        assert c.sum_waits_gave_up() == 0
+        c.set_poll_limit(0)
+        check()
+        gave_up = c.sum_waits_gave_up()
+        assert gave_up > 0
+        c.set_poll_limit(1 << 21)
+        check()
+        assert c.sum_waits_gave_up() == gave_up
+        assert not c.wait_gave_up()  # the sampling paths' own flag is untouched
+    finally:
+        c.close()
+
+
 @pytest.mark.parametrize("vocab", [3, 5000, 20000, 70000])
 def test_softmax_rows_whose_maximum_is_a_signed_zero(ctx, orc, vocab):
     """The reference subtracts the row's own first maximal element, -0.0 included: a single -0.0 maximum above
