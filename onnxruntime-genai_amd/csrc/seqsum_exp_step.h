@@ -4,6 +4,7 @@
 #include "kernels.h"
 #include "block_seq.h"
 #include "seg_io.h"
+#include "wave_select.h"
 
 namespace ms {
 
@@ -162,8 +163,9 @@ __device__ __forceinline__ void seqsum_exp_step_body(const SeqSumArgs& a, const 
     double mine = 0.0;
 #pragma unroll
     for (int j = 0; j < kSegPer; ++j) mine += static_cast<double>(ev[j]);
-    mine += __shfl_xor(mine, 1, 64);
-    mine += __shfl_xor(mine, 2, 64);  // all four lanes of a part hold its sum
+    mine += __longlong_as_double(static_cast<long long>(lane_xor64<1>(static_cast<u64>(__double_as_longlong(mine)))));
+    mine += __longlong_as_double(static_cast<long long>(lane_xor64<2>(static_cast<u64>(__double_as_longlong(mine)))));
+    // (all four lanes of a part hold its sum)
     const int part_i = tid >> 2;
     // the sum of the parts before this one: a prefix over the wave's sixteen parts and the totals of the waves before
     const double upto = wave_prefix_sum<double>((lane & 3) == 0 ? mine : 0.0);

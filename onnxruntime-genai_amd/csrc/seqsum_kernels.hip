@@ -159,7 +159,7 @@ __global__ __launch_bounds__(64 * kWalkWaves) void seqsum_walk_kernel(const SeqS
       const int pse = a.sub_se[at + lane];
       part_rec[slot][lane] = q;
       part_se[slot][lane] = pse;
-      const int next_se = __shfl_down(pse, 1, 64);
+      const int next_se = static_cast<int>(__builtin_amdgcn_update_dpp(0u, static_cast<uint32_t>(pse), 0x130, 0xf, 0xf, false));  // wave_shl:1: the lane above
       unsigned long long want = __ballot(pse < 0 || (lane < 63 && next_se != pse));
       int pp[kWalkAhead];
       float val[kWalkAhead];
