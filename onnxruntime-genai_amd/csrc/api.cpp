@@ -217,6 +217,8 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->ptr_table, c->ptr_table_cap, false));
   if (e == hipSuccess) e = ms_sample_init();
   if (e == hipSuccess) e = ms_static_scratch_setup();  // set-up of mi355x_argmax_static on this device
+  // the fills above ran on the null stream: done before a caller's stream, which need not wait for it, uses them
+  if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
   if (e != hipSuccess) {
     mi355x_search_destroy(c);
     return Fail(MI355X_E_HIP, "workspace allocation failed: %s", hipGetErrorString(e));
@@ -837,6 +839,7 @@ int mi355x_beam_scorer_create(mi355x_search_ctx* ctx, int batch, int beams, int 
     if (e == hipSuccess) e = hipMemcpy(st.hyp_slot, slots.data(), slots.size() * sizeof(int), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemcpy(s->pow_dev, powt.data(), powt.size() * sizeof(float), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemcpy(st.not_done, &batch, sizeof(int), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);  // the fills are done before any stream uses the state
     st.pow_table = s->pow_dev;
   }
   if (e != hipSuccess) {

@@ -140,6 +140,36 @@ def test_search_step_finishes_entries_like_the_two_calls(ctx, batch, beams, voca
     big.close()
 
 
+def test_first_calls_of_a_new_context_on_a_side_stream(orc):
+    """A context (and a scorer) used right after creation on a stream that does not wait for the null stream:
+    the workspace's initial fills must be complete by then.  Long rows, so the exact sums read their "not
+    written" pattern."""
+    say("new context on a side stream")
+    rng = np.random.default_rng(5)
+    batch, beams, vocab = 3, 2, 40000
+    x = (rng.standard_normal((batch * beams, vocab)) * 2).astype(np.float32)
+    want = [orc.log_softmax(x[r], 1.0) for r in range(batch * beams)]
+    xd = torch.from_numpy(x).cuda()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    for attempt in range(3):
+        with torch.cuda.stream(side):
+            c = pkg().SearchContext(batch * beams, vocab)
+            got = c.softmax(xd.clone(), 1.0, log=True)
+            scorer = pkg().BeamScorer(c, batch, beams, 8, 0, [1], 1.0, False)
+            scorer.set_prompt(np.full((batch, 2), 5, np.int32))
+            scorer.search_step(xd)
+            osc, otok, oidx, _ = orc.beam_select_top(x, batch, beams, np.tile(np.array([0.0, -1e9], np.float32), batch))
+            side.synchronize()
+            got = got.cpu().numpy()
+            for r in range(batch * beams):
+                assert np.array_equal(bits(got[r]), bits(want[r])), (attempt, r)
+            assert np.array_equal(scorer.next_tokens.cpu().numpy().reshape(batch, beams), otok[:, :beams]), attempt
+            assert c.sum_waits_gave_up() == 0
+            scorer.close()
+            c.close()
+
+
 def test_exact_sums_whose_waits_give_up(orc):
     """Failure handling of the exact sums' look-back, forced from the host: with a poll limit of 0 a segment's
     workgroup gives up on every earlier sum that has not arrived yet and its segment is added element by element.
