@@ -342,6 +342,36 @@ __device__ __forceinline__ double wave_scan_add(double x) {
   return x;
 }
 
+// One thread's share of the search for the first cumulative value that reaches `target`: its weights pv follow a
+// cumulative value of `before` and sum to `loc`.  first = the lowest index whose cumulative value reaches the target
+// (the last index always does: its value is forced to 1); risky = some cumulative value other than the last lies
+// within `guard` of the target.  Most threads lie entirely on one side of the target by more than the guard and
+// settle that from their two end values: the additions of a thread's weights in another order differ from these
+// by less than the guard (it counts sixteen roundings per weight of the whole distribution), hence the factor two.
+template <int ITEMS>
+__device__ __forceinline__ void draw_scan_thread(const double (&pv)[ITEMS], double before, double loc, int base, int n,
+                                                 double target, double guard, int& first, int& risky) {
+  if (base >= n) return;
+  if (before + loc < target - 2.0 * guard) {  // all below the target
+    if (base + ITEMS >= n && n - 1 < first) first = n - 1;
+    return;
+  }
+  if (before > target + 2.0 * guard) {  // all above it
+    if (base < first) first = base;
+    return;
+  }
+  double run = before;
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const int idx = base + j;
+    if (idx < n) {
+      run += pv[j];
+      if (idx != n - 1 && fabs(run - target) <= guard) risky = 1;
+      if ((idx == n - 1 || run >= target) && idx < first) first = idx;  // the last value is forced to 1
+    }
+  }
+}
+
 // Position std::discrete_distribution would return for weights w(0..n-1) and canonical draw u
 // (libstdc++ random.tcc: normalise by the double sum, partial sums in double, last forced to 1,
 // lower_bound).  The reference divides every weight by the sum and accumulates the quotients
@@ -402,16 +432,7 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float
       guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16 * total;
       target = u * total;
     }
-    double run = wp + (inc - loc);
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-      const int idx = base + j;
-      if (idx < n) {
-        run += pv[j];
-        if (idx != n - 1 && fabs(run - target) <= guard) risky = 1;
-        if ((idx == n - 1 || run >= target) && idx < first) first = idx;  // the last value is forced to 1
-      }
-    }
+    draw_scan_thread<ITEMS>(pv, wp + (inc - loc), loc, base, n, target, guard, first, risky);
     carry += block_total;
     __syncthreads();
   }

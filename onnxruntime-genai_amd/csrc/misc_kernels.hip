@@ -173,7 +173,6 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
   const int span = static_cast<int>(blockDim.x) * ITEMS;
   *all_zero = false;
   float wv[WINDOWS][ITEMS];
-  double part = 0.0;
   if constexpr (!std::is_same<GetGroup, NoVectorLoads>::value) {
     // group(i, out) loads the ITEMS weights i .. i + ITEMS - 1 (i a multiple of ITEMS, all below n) with wide
     // loads: a thread reads its own consecutive weights directly, neighbouring lanes neighbouring groups, and no
@@ -188,10 +187,6 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
         for (int j = 0; j < ITEMS; ++j) wv[c][j] = i0 + j < n ? w(i0 + j) : 0.0f;
       }
     }
-#pragma unroll
-    for (int c = 0; c < WINDOWS; ++c)
-#pragma unroll
-      for (int j = 0; j < ITEMS; ++j) part += static_cast<double>(wv[c][j]);
   } else {
     // Every weight is requested before the first barrier (a barrier waits for the loads in flight, so fetching
     // window by window would pay the memory latency once per window), consecutive lanes on consecutive indices;
@@ -220,17 +215,34 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
           wv[c][j] = q.x, wv[c][j + 1] = q.y, wv[c][j + 2] = q.z, wv[c][j + 3] = q.w;
         }
         __syncthreads();  // the staging buffer is rewritten by the next window
-#pragma unroll
-        for (int j = 0; j < ITEMS; ++j) part += static_cast<double>(wv[c][j]);
       }
     }
   }
-  part = wave_sum<double>(part);
-  if (lane == 0) sh.dred[wave] = part;
+  // The windows' scans are independent until their totals chain up: all of them run before the one barrier, and
+  // the total of the distribution comes out of them (any summation order will do: the guard band covers it).
+  __shared__ double win_scan[WINDOWS][16];
+  double pv[WINDOWS][ITEMS], loc[WINDOWS], inc[WINDOWS];
+#pragma unroll
+  for (int c = 0; c < WINDOWS; ++c) {
+    loc[c] = 0.0;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      pv[c][j] = static_cast<double>(wv[c][j]);
+      loc[c] += pv[c][j];
+    }
+    inc[c] = wave_scan_add(loc[c]);
+    if (lane == 63) win_scan[c][wave] = inc[c];
+  }
   __syncthreads();
+  // sums of the waves before this one and of every window: lane k takes wave k's sum
+  double ws[WINDOWS], window_total[WINDOWS];
   double total = 0.0;
-  for (int k = 0; k < nw; ++k) total += sh.dred[k];
-  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < WINDOWS; ++c) {
+    ws[c] = wave_scan_add(lane < nw ? win_scan[c][lane] : 0.0);
+    window_total[c] = wave_read_lane(ws[c], nw - 1);
+    total += window_total[c];
+  }
   if (total != total) return 0;  // NaN weights: see block_discrete_draw
   if (total == 0.0) {
     *all_zero = true;
@@ -239,42 +251,14 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
   if (n < 2) return 0;
   const double guard = 16.0 * static_cast<double>(n) * 1.1102230246251565e-16 * total;
   const double target = u * total;
-  // The windows' scans are independent until their totals chain up: all of them run before the one barrier.
-  __shared__ double win_scan[WINDOWS][16];
-  double loc[WINDOWS], inc[WINDOWS];
-#pragma unroll
-  for (int c = 0; c < WINDOWS; ++c) {
-    loc[c] = 0.0;
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) loc[c] += static_cast<double>(wv[c][j]);
-    inc[c] = wave_scan_add(loc[c]);
-    if (lane == 63) win_scan[c][wave] = inc[c];
-  }
-  __syncthreads();
   double carry = 0.0;
   int first = kIntMax;
   int risky = 0;
 #pragma unroll
   for (int c = 0; c < WINDOWS; ++c) {
-    const int i0 = c * span;
-    if (i0 < n) {
-      const int base = i0 + tid * ITEMS;
-      // sums of the waves before this one and of the whole window: lane k takes wave k's sum
-      const double ws = wave_scan_add(lane < nw ? win_scan[c][lane] : 0.0);
-      const double block_total = wave_read_lane(ws, nw - 1);
-      const double wp = carry + (wave > 0 ? wave_read_lane(ws, wave - 1) : 0.0);
-      double run = wp + (inc[c] - loc[c]);
-#pragma unroll
-      for (int j = 0; j < ITEMS; ++j) {
-        const int idx = base + j;
-        if (idx < n) {
-          run += static_cast<double>(wv[c][j]);
-          if (idx != n - 1 && fabs(run - target) <= guard) risky = 1;
-          if ((idx == n - 1 || run >= target) && idx < first) first = idx;  // the last value is forced to 1
-        }
-      }
-      carry += block_total;
-    }
+    const double wp = carry + (wave > 0 ? wave_read_lane(ws[c], wave - 1) : 0.0);
+    draw_scan_thread<ITEMS>(pv[c], wp + (inc[c] - loc[c]), loc[c], c * span + tid * ITEMS, n, target, guard, first, risky);
+    carry += window_total[c];
   }
   int a = first, b = risky ? 0 : 1;
   block_min2(a, b, sh);
