@@ -342,6 +342,15 @@ __device__ __forceinline__ double wave_scan_add(double x) {
   return x;
 }
 
+// Inclusive prefix sums inside every row of sixteen lanes (enough where only the first sixteen lanes hold values).
+__device__ __forceinline__ double row_scan_add(double x) {
+  x += dpp_from_below<0x111, 0xf>(x);  // row_shr:1
+  x += dpp_from_below<0x112, 0xf>(x);  // row_shr:2
+  x += dpp_from_below<0x114, 0xf>(x);  // row_shr:4
+  x += dpp_from_below<0x118, 0xf>(x);  // row_shr:8
+  return x;
+}
+
 // One thread's share of the search for the first cumulative value that reaches `target`: its weights pv follow a
 // cumulative value of `before` and sum to `loc`.  first = the lowest index whose cumulative value reaches the target
 // (the last index always does: its value is forced to 1); risky = some cumulative value other than the last lies
@@ -423,7 +432,7 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float
     if (lane == 63) sh.dscan[wave] = inc;
     __syncthreads();
     // sums of the waves before this one and of the whole window: lane k takes wave k's sum
-    const double ws = wave_scan_add(lane < nw ? sh.dscan[lane] : 0.0);
+    const double ws = row_scan_add(lane < nw ? sh.dscan[lane] : 0.0);
     const double block_total = wave_read_lane(ws, nw - 1);
     const double wp = carry + (wave > 0 ? wave_read_lane(ws, wave - 1) : 0.0);
     if (single) {

@@ -234,13 +234,17 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
     if (lane == 63) win_scan[c][wave] = inc[c];
   }
   __syncthreads();
-  // sums of the waves before this one and of every window: lane k takes wave k's sum
-  double ws[WINDOWS], window_total[WINDOWS];
+  // sums of the waves before this one and of every window, all windows in one scan: row c of sixteen lanes takes
+  // window c's wave sums, and the lane shifts inside rows scan the four rows at once
+  static_assert(WINDOWS <= 4, "one row of sixteen lanes per window");
+  const int my_window = (lane >> 4) < WINDOWS ? (lane >> 4) : 0;
+  double ws = ((lane >> 4) < WINDOWS && (lane & 15) < nw) ? win_scan[my_window][lane & 15] : 0.0;
+  ws = row_scan_add(ws);
+  double window_total[WINDOWS];
   double total = 0.0;
 #pragma unroll
   for (int c = 0; c < WINDOWS; ++c) {
-    ws[c] = wave_scan_add(lane < nw ? win_scan[c][lane] : 0.0);
-    window_total[c] = wave_read_lane(ws[c], nw - 1);
+    window_total[c] = wave_read_lane(ws, c * 16 + 15);
     total += window_total[c];
   }
   if (total != total) return 0;  // NaN weights: see block_discrete_draw
@@ -256,7 +260,7 @@ __device__ __forceinline__ int block_discrete_draw_once(int n, GetW w, double u,
   int risky = 0;
 #pragma unroll
   for (int c = 0; c < WINDOWS; ++c) {
-    const double wp = carry + (wave > 0 ? wave_read_lane(ws[c], wave - 1) : 0.0);
+    const double wp = carry + (wave > 0 ? wave_read_lane(ws, c * 16 + wave - 1) : 0.0);
     draw_scan_thread<ITEMS>(pv[c], wp + (inc[c] - loc[c]), loc[c], c * span + tid * ITEMS, n, target, guard, first, risky);
     carry += window_total[c];
   }

@@ -475,8 +475,8 @@ __device__ __forceinline__ void trim_to_nucleus(u64* lds_keys, uint32_t* table, 
       scan_mass[wave] = mass_inc;
     }
     __syncthreads();
-    const double wc = wave_scan_add(lane < kFinishBlock / 64 ? scan_cnt[lane] : 0.0);
-    const double wm = wave_scan_add(lane < kFinishBlock / 64 ? scan_mass[lane] : 0.0);
+    const double wc = row_scan_add(lane < kFinishBlock / 64 ? scan_cnt[lane] : 0.0);
+    const double wm = row_scan_add(lane < kFinishBlock / 64 ? scan_mass[lane] : 0.0);
     double c = (wave > 0 ? wave_read_lane(wc, wave - 1) : 0.0) + (cnt_inc - cnt);
     double m = (wave > 0 ? wave_read_lane(wm, wave - 1) : 0.0) + (mass_inc - mass);
     uint32_t mine = static_cast<uint32_t>(kSortBuckets);
