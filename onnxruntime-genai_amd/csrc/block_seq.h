@@ -3,6 +3,7 @@
 // an in-place bitonic sort, and the exact sampling epilogue shared by the nucleus and general paths.
 #pragma once
 #include <type_traits>
+#include <utility>
 #include "device_utils.h"
 #include "seq_scan.h"
 #include "wave_select.h"
@@ -167,6 +168,40 @@ struct NoStop {
   __device__ bool operator()(float, float, int) const { return false; }
 };
 
+// A stop predicate may also say that it holds nowhere in a run of consecutive addends, judged at the run's last
+// element: bool nowhere_in_run_ending(prefix, addend, index).  It must only say so when that is certain.
+template <typename StopFn, typename = void>
+struct StopSettlesRuns : std::false_type {};
+template <typename StopFn>
+struct StopSettlesRuns<StopFn, decltype(void(std::declval<const StopFn&>().nowhere_in_run_ending(0.0f, 0.0f, 0)))>
+    : std::true_type {};
+
+// Stops at the first prefix that reaches a fixed mass.  Prefixes do not decrease, so a run whose last prefix is
+// below the mass holds no stop.
+struct StopAtMass {
+  float mass;
+  __device__ __forceinline__ bool operator()(float pf, float, int) const { return pf >= mass; }
+  __device__ __forceinline__ bool nowhere_in_run_ending(float pf, float, int) const { return pf < mass; }
+};
+
+// FindNucleus' stop (src/sampling_distribution.h:164-174) over addends in descending order: the prefix reaches
+// p times (prefix + the bound (vocab - i - 1) * addend on what follows).  In exact arithmetic prefix - p * (prefix +
+// bound) does not decrease along the row (prefixes do not decrease, addends and counts do not increase); the
+// float evaluation is within a few 2^-24 of it, so a run whose last element misses the stop by more than 2^-18 of
+// the right-hand side holds none.
+struct StopAtNucleus {
+  float p;
+  int vocab, offset;  // the addend's rank in the row is its index + offset
+  __device__ __forceinline__ bool operator()(float pf, float e, int i) const {
+    const float tail = static_cast<float>(vocab - (i + offset) - 1) * e;
+    return pf >= p * (pf + tail);
+  }
+  __device__ __forceinline__ bool nowhere_in_run_ending(float pf, float e, int i) const {
+    const float tail = static_cast<float>(vocab - (i + offset) - 1) * e;
+    return pf < (p * (pf + tail)) * 0.99999619f;  // 1 - 2^-18
+  }
+};
+
 // Exact value of (((s0 + e(0)) + e(1)) + ... ) in fp32 over i < n, computed by the whole block
 // (every thread must call with identical arguments; every thread gets the result).
 // If stop(prefix_i, e(i), i) holds for some i -- prefix_i being the sum including e(i) -- the scan
@@ -229,14 +264,11 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
     int start = w0;  // first index not yet folded into s
     while (true) {
       const SeqState st = seq_decompose(s);
-      Step f[ITEMS];
-      Step agg{0u, 0u};
+      // the thread's addends that are still to be folded in (the others count as zeros), composed into one step
+      float live[ITEMS];
 #pragma unroll
-      for (int j = 0; j < ITEMS; ++j) {
-        const int idx = base + j;
-        f[j] = (idx >= start && idx < wend) ? seq_make_step(ev[j], st.se) : Step{0u, 0u};
-        agg = step_compose(agg, f[j]);
-      }
+      for (int j = 0; j < ITEMS; ++j) live[j] = (base + j >= start && base + j < wend) ? ev[j] : 0.0f;
+      const Step agg = seq_compose_run(live, ITEMS, st.se);
       const Step inc = wave_scan_steps(agg);
       if (lane == 63) sh.wave_tot[par][wave] = inc;
       __syncthreads();
@@ -260,14 +292,38 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
       // Without a stop predicate only a binade change is of interest, and a thread whose last
       // prefix is still inside the binade (prefixes never decrease) has none among its elements.
       constexpr bool kPlain = std::is_same<StopFn, NoStop>::value;
-      if (kPlain && step_apply(nn, agg) < kMantLimit) {
-        nn = step_apply(nn, agg);
-      } else {
+      const uint32_t nn_end = step_apply(nn, agg);
+      bool walk = true;
+      if (nn_end < kMantLimit) {
+        if constexpr (kPlain) {
+          nn = nn_end;
+          walk = false;
+        } else if constexpr (StopSettlesRuns<StopFn>::value) {
+          // A thread whose addends are all live and stay inside the binade asks its predicate about the run as a
+          // whole: nowhere true (judged at the run's last element), or true at its first element already, which
+          // is then the thread's event; only the thread in which the predicate turns true walks its elements.
+          if (base >= start && base + ITEMS <= wend) {
+            if (stop.nowhere_in_run_ending(seq_recompose(nn_end, st.se), ev[ITEMS - 1], base + ITEMS - 1)) {
+              nn = nn_end;
+              walk = false;
+            } else {
+              const float p1 = seq_recompose(step_apply(nn, seq_make_step(ev[0], st.se)), st.se);
+              if (stop(p1, ev[0], base)) {
+                key = static_cast<uint32_t>(base) << 1;
+                pa = p1;
+                nn = nn_end;
+                walk = false;
+              }
+            }
+          }
+        }
+      }
+      if (walk) {
 #pragma unroll
         for (int j = 0; j < ITEMS; ++j) {
           const int idx = base + j;
           if (idx >= start && idx < wend) {
-            const uint32_t nn2 = step_apply(nn, f[j]);
+            const uint32_t nn2 = step_apply(nn, seq_make_step(ev[j], st.se));
             if (key == kNone) {
               if (nn2 >= kMantLimit) {  // leaves the binade here (or an earlier thread's element did)
                 key = (static_cast<uint32_t>(idx) << 1) | 1u;
@@ -607,7 +663,7 @@ __device__ __forceinline__ bool block_sample_epilogue(Sorted sorted, Exps exps, 
     if (prm.p > 0.0f && prm.p < 1.0f) {
       const float p = prm.p;
       int si;
-      keep_sum = block_seq_sum<ITEMS>(0.0f, m, pr, [=](float pf, float, int) { return pf >= p; }, &si, sh, nullptr, kEpiHead);
+      keep_sum = block_seq_sum<ITEMS>(0.0f, m, pr, StopAtMass{p}, &si, sh, nullptr, kEpiHead);
       if (si >= 0) keep = si + 1;
     } else {
       keep_sum = block_seq_sum<ITEMS>(0.0f, m, pr, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead);
@@ -628,13 +684,8 @@ __device__ __forceinline__ bool block_sample_epilogue(Sorted sorted, Exps exps, 
     for (;;) {
       const int b = base;
       int si;
-      prefix = block_seq_sum<ITEMS>(
-          prefix, limit - b, [=](int i) { return exps(i + b); },
-          [=](float pf, float e, int i) {
-            const float tail = static_cast<float>(V - (i + b) - 1) * e;
-            return pf >= p * (pf + tail);
-          },
-          &si, sh, nullptr, b == 0 ? kEpiHead : 0);
+      prefix = block_seq_sum<ITEMS>(prefix, limit - b, [=](int i) { return exps(i + b); }, StopAtNucleus{p, V, b}, &si, sh,
+                                    nullptr, b == 0 ? kEpiHead : 0);
       if (si < 0) {
         if (limit != vocab) return false;
         cutoff = vocab;
@@ -650,9 +701,7 @@ __device__ __forceinline__ bool block_sample_epilogue(Sorted sorted, Exps exps, 
       if (n_sorted < vocab) return false;
       const float global = block_seq_sum<ITEMS>(0.0f, vocab, exps, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead);
       int sj;
-      const float c = block_seq_sum<ITEMS>(0.0f, vocab, exps,
-                                           [=](float pf, float, int) { return pf >= p * global; }, &sj, sh,
-                                           nullptr, kEpiHead);
+      const float c = block_seq_sum<ITEMS>(0.0f, vocab, exps, StopAtMass{p * global}, &sj, sh, nullptr, kEpiHead);
       (void)c;
       if (sj >= 0) {
         cutoff = sj + 1;
