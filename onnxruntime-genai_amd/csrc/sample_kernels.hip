@@ -759,10 +759,12 @@ __global__ __launch_bounds__(kFinishBlock) void largek_finish_rows_kernel(const 
 // did not close inside the candidates).
 constexpr int kSparseWords = 16;                              // mask words per thread: vocabularies up to 524288
 constexpr int kSparseIds = kNucleusCap / kFinishBlock;        // gathered ids per thread
-constexpr int kSparseExtras = (kSortBuckets + 1) / 2;         // distinct history ids (they use the bucket table's LDS)
+constexpr int kSparseExtraRegs = 2;                           // processed history ids a thread takes on as candidates
+constexpr int kSparseExtras = kSparseExtraRegs * kFinishBlock;  // distinct history ids (their list uses the bucket table's LDS)
+static_assert(2 * kSparseExtras <= kSortBuckets + 1, "the list of processed history ids fits the bucket table");
 
 template <typename InT>
-__device__ __forceinline__ void sparse_gather(const void* row0, const uint32_t (&ids)[kSparseIds + 2], float (&x)[kSparseIds + 2]) {
+__device__ __forceinline__ void sparse_gather(const void* row0, const uint32_t (&ids)[kSparseIds + kSparseExtraRegs], float (&x)[kSparseIds + kSparseExtraRegs]) {
   const InT* const p = static_cast<const InT*>(row0);
   InT raw[kSparseIds];
 #pragma unroll
@@ -886,8 +888,8 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   }
   __syncthreads();
   // gather: every load of a thread is requested before the first is used
-  uint32_t ids[kSparseIds + 2];
-  float x[kSparseIds + 2];
+  uint32_t ids[kSparseIds + kSparseExtraRegs];
+  float x[kSparseIds + kSparseExtraRegs];
 #pragma unroll
   for (int u = 0; u < kSparseIds; ++u) {
     const uint32_t i = static_cast<uint32_t>(tid + u * kFinishBlock);
@@ -898,14 +900,14 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   else if (a.dtype == MI355X_BF16) sparse_gather<bf16_t>(lrow.p, ids, x);
   else sparse_gather<float>(lrow.p, ids, x);
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
+  for (int u = 0; u < kSparseExtraRegs; ++u) {
     const uint32_t i = static_cast<uint32_t>(tid + u * kFinishBlock);
     ids[kSparseIds + u] = i < n_extra ? extra_idx[i] : 0xffffffffu;
     x[kSparseIds + u] = i < n_extra ? extra_val[i] : __uint_as_float(0x7fc00000u);
   }
   uint32_t kmax = 0u;
 #pragma unroll
-  for (int u = 0; u < kSparseIds + 2; ++u) {
+  for (int u = 0; u < kSparseIds + kSparseExtraRegs; ++u) {
     const uint32_t k = ids[u] != 0xffffffffu ? order_key(x[u]) : 0u;
     kmax = k > kmax ? k : kmax;
   }
@@ -917,11 +919,11 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   // batch; the best of the others is kept
   u64 best_below = first_masked != 0xffffffffu ? make_key64(order_key(kLowest), first_masked) : 0;
 #pragma unroll
-  for (int u0 = 0; u0 < kSparseIds + 2; u0 += 6) {
+  for (int u0 = 0; u0 < kSparseIds + kSparseExtraRegs; u0 += 6) {
     u64 hits[6];
     uint32_t wcnt = 0u;
 #pragma unroll
-    for (int u = u0; u < u0 + 6 && u < kSparseIds + 2; ++u) {
+    for (int u = u0; u < u0 + 6 && u < kSparseIds + kSparseExtraRegs; ++u) {
       const bool have = ids[u] != 0xffffffffu;
       const uint32_t ok32 = have ? order_key(x[u]) : 0u;
       const bool cand = have && ok32 >= thr;
@@ -936,7 +938,7 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
     if (lane == 0 && wcnt != 0u) base = atomicAdd(&sh_count, wcnt);
     base = __builtin_amdgcn_readfirstlane(base);
 #pragma unroll
-    for (int u = u0; u < u0 + 6 && u < kSparseIds + 2; ++u) {
+    for (int u = u0; u < u0 + 6 && u < kSparseIds + kSparseExtraRegs; ++u) {
       const u64 b = hits[u - u0];
       const uint32_t p = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), base));
       if ((b >> lane) & 1ull) lds_keys[p] = make_key64(order_key(x[u]), ids[u]);

@@ -463,6 +463,41 @@ def test_sample_long_and_dense_histories(ctx, orc, vocab, hist_len, span, k, p):
     assert (took_exact > 0) == (span == 2500), took_exact  # only the overflowing lists go to the exact path
 
 
+@pytest.mark.parametrize("hist_len", [1500, 2500, 3400, 5000])
+def test_sparse_mask_rows_with_thousands_of_distinct_history_ids(orc, hist_len):
+    """Nucleus rows under a sparse grammar mask whose history holds more distinct ids than the sparse-mask kernel's
+    threads take on as processed candidates (two each): such rows must leave that kernel, not lose ids.  Half of
+    the history ids are allowed and strong, so that every one of them is inside the nucleus."""
+    say("sparse mask, long history", hist_len)
+    rng = np.random.default_rng(hist_len)
+    rows, vocab = 2, 201088
+    c = pkg().SearchContext(rows, vocab)
+    try:
+        x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+        mask = make_mask(rng, rows, vocab, 0.04)
+        hist = np.stack([rng.choice(vocab, hist_len, replace=False) for _ in range(rows)]).astype(np.int32)
+        for r in range(rows):
+            ids = hist[r, :hist_len // 2]
+            np.bitwise_or.at(mask.reshape(rows, -1)[r], ids >> 5, np.uint32(1) << (ids & 31).astype(np.uint32))
+            x[r, ids] += 6.0
+        u = rng.random(rows)
+        xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                               repetition_penalty=1.2)
+        tok, kc, ki, kp = c.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=0.95, temperature=1.0,
+                                   xf=xf, kept_capacity=16384)
+        tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+        proc = orc.apply_mask(x, mask)
+        for r in range(rows):
+            row = orc.apply_repetition_penalty(proc[r], hist[r], 1.2)
+            idx, probs = orc.sampled_categorical(row, 0, 0.95, 1.0)
+            assert kc[r] == len(idx), r
+            assert np.array_equal(ki[r, :len(idx)], idx), r
+            assert np.array_equal(bits(kp[r, :len(idx)]), bits(probs)), r
+            assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+    finally:
+        c.close()
+
+
 @pytest.mark.parametrize("vocab", [5000, 70001])
 def test_nucleus_with_minus_infinity_below_the_threshold(ctx, orc, vocab):
     """Rows whose elements outside the candidate range are all -inf: the element after the nucleus, which a
