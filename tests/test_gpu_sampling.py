@@ -572,7 +572,8 @@ def test_sample_randomised_shapes_and_parameters(ctx, orc, seed):
     xf, proc = None, x
     if seed % 4 in (1, 2):
         mask = make_mask(rng, rows, vocab, float(rng.choice([0.02, 0.5, 0.98])))
-        hist = rng.integers(0, vocab, (rows, int(rng.integers(1, 200)))).astype(np.int32)
+        hist_len = int(rng.integers(1, 200)) if seed % 9 else int(rng.integers(1500, 6000))  # now and then a long one
+        hist = rng.integers(0, vocab, (rows, hist_len)).astype(np.int32)
         pen = float(rng.choice([1.0, 1.3, 0.8]))
         eos = [int(rng.integers(0, vocab))]
         allowed = int(np.unpackbits(mask.view(np.uint8)).reshape(rows, -1).sum(axis=1).max())
