@@ -13,7 +13,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per step from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of these same commands, scaled by a
 # known-size copy; counters cannot be read from inside the process, so these are offline profile constants.
 # c3: KV gather 6.22 GB + selection kernels 0.04 GB; c5: the one sparse-mask kernel.  None where no counter run exists.
-MEASURED_TRAFFIC = {"c3": 6_222_000_000 + 42_000_000, "c5": 204_350_000}
+MEASURED_TRAFFIC = {"c3": 6_222_000_000 + 42_000_000, "c5": 204_200_000}
 TRAFFIC_SOURCE = {"c3": "offline profile constant: profiles/beam_step_kernels_config3.md",
                   "c5": "offline profile constant: profiles/nucleus_sparse_kernel_config5.md"}
 
