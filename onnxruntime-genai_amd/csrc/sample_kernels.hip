@@ -21,8 +21,10 @@ constexpr int kSortBuckets = 7168;  // what fits next to the keys in 160 KB of L
 constexpr int kBucketCap = 64;
 constexpr size_t kFinishLds = kNucleusCap * sizeof(u64) + (kSortBuckets + 1) * sizeof(uint32_t);
 
-__device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n, float fmax, float fthr, uint32_t* red) {
-  constexpr int R = kNucleusCap / kFinishBlock;
+// R: keys per thread the code provides for (n <= R * kFinishBlock); a list of a quarter or half of the capacity
+// gets code whose unrolled loops are that much shorter.
+template <int R>
+__device__ __noinline__ bool bucket_sort_desc_sized(u64* keys, uint32_t* start, int n, float fmax, float fthr, uint32_t* red) {
   const int t = threadIdx.x;
   u64 k[R];
   uint32_t info[R];  // bucket << 8 | slot inside the bucket, later the final position
@@ -94,6 +96,13 @@ __device__ __noinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n,
     if (r * kFinishBlock + t < n) keys[info[r]] = k[r];
   __syncthreads();
   return true;
+}
+
+__device__ __forceinline__ bool bucket_sort_desc(u64* keys, uint32_t* start, int n, float fmax, float fthr, uint32_t* red) {
+  constexpr int kFull = kNucleusCap / kFinishBlock;
+  if (n <= kFull / 4 * kFinishBlock) return bucket_sort_desc_sized<kFull / 4>(keys, start, n, fmax, fthr, red);
+  if (n <= kFull / 2 * kFinishBlock) return bucket_sort_desc_sized<kFull / 2>(keys, start, n, fmax, fthr, red);
+  return bucket_sort_desc_sized<kFull>(keys, start, n, fmax, fthr, red);
 }
 
 // Sorts n2 keys (a power of two, at least two tiles) in global memory, descending, by a block of
