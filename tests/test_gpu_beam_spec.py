@@ -398,6 +398,21 @@ def run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, lengt
     dev.close()
 
 
+@pytest.mark.parametrize("batch,beams,vocab", [(2, 8, 131072), (2, 8, 131073), (1, 16, 16384), (40, 4, 16385)])
+def test_beam_search_at_the_edges_of_the_segment_route(orc, batch, beams, vocab):
+    """Whole searches through mi355x_beam_search_step where the long-row route changes: beams x segments x 2 beams
+    exactly at the finishing kernel's capacity and one segment over (which takes the row-wise kernels), sixteen beams
+    at the shortest long row, forty batch entries whose rows end one logit into a segment."""
+    say("beam search edges", batch, beams, vocab)
+    c = pkg().SearchContext(batch * beams, vocab)
+    try:
+        for early in (False, True):
+            run_beam_search(c, orc, batch, beams, vocab, 5, [3, vocab - 1], 10, 1.1, early, 1000 + batch + beams,
+                            dtype=np.float16 if beams == 8 else np.float32, eos_boost=5.0, fused=True)
+    finally:
+        c.close()
+
+
 def test_config3_beam_search_steps(ctx, orc):
     """Benchmark configuration 3 shape (batch 8, beams 4, vocab 151936 fp16, length_penalty 1.0), 6 of the 64
     steps: selection, scorer state, beam-reordered sequences and final hypotheses match the oracle."""
