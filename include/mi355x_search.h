@@ -118,7 +118,7 @@ int mi355x_process_logits(mi355x_search_ctx* ctx, void* stream, float* logits, i
 /* Greedy argmax per row: GreedySearch_Cpu::SelectTop / ArgMax (src/search.cpp:178-192,
  * src/search.h:9-29) and DeviceInterface::ArgMaxDevice (src/smartptrs.h:258).  dtype MI355X_F32,
  * MI355X_F16 (widened exactly like FastFloat16ToFloat32, src/models/utils.cpp:103-109) or MI355X_BF16
- * (BFloat16ToFloat32, :84-86; rows of 65 to 524288 logits only).
+ * (BFloat16ToFloat32, :84-86).
  * xf may be NULL.  out_tokens: device [rows] int32. */
 int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype,
                   int64_t row_stride, int rows, int vocab, const mi355x_logits_xform* xf,

@@ -138,7 +138,7 @@ def argmax_static(logits, out, xf=None):
     L = load_library()
     assert logits.is_cuda and logits.dim() == 2 and logits.stride(1) == 1
     assert out.is_cuda and out.dtype == torch.int32 and out.numel() >= logits.shape[0] and out.is_contiguous()
-    dtype = {torch.float32: MI355X_F32, torch.float16: MI355X_F16}[logits.dtype]
+    dtype = _DTYPE_CODES[logits.dtype]
     rc = L.mi355x_argmax_static(_stream(), logits.data_ptr(), dtype, logits.stride(0), logits.shape[0], logits.shape[1],
                                 C.byref(xf.c) if xf else None, out.data_ptr())
     if rc != 0:

@@ -258,8 +258,6 @@ int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int 
   // rows of more than 64 logits go through the fused selection kernel (k = 1, ids only), whatever their type
   const int fused_chunks = (vocab + ms::kSChunk - 1) / ms::kSChunk;
   const bool fused = vocab > 64 && fused_chunks * ms::kSmallCap <= ms::kAllCap && rows * fused_chunks >= ms::kArgmaxFusedMinBlocks;
-  if (dtype == MI355X_BF16 && !fused)
-    return Fail(MI355X_E_UNSUPPORTED, "bf16 rows need 64 < vocab <= %d", ms::kAllCap / ms::kSmallCap * ms::kSChunk);
   if (fused) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     ms::SampleArgs f{};

@@ -98,8 +98,8 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
           const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
-            v[j][2 * c] = half_bits_to_float(w[c] & 0xffffu);
-            v[j][2 * c + 1] = half_bits_to_float(w[c] >> 16);
+            v[j][2 * c] = narrow_bits_to_float<InT>(w[c] & 0xffffu);
+            v[j][2 * c + 1] = narrow_bits_to_float<InT>(w[c] >> 16);
           }
         }
       } else {
@@ -175,6 +175,8 @@ extern "C" hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipSt
   if (a->vocab <= ms::kRowKernelMaxVocab && a->rows * a->chunks < 256) {
     if (dtype == MI355X_F16)
       hipLaunchKernelGGL(ms::argmax_row_kernel<uint16_t>, dim3(a->rows), dim3(1024), 0, stream, *a);
+    else if (dtype == MI355X_BF16)
+      hipLaunchKernelGGL(ms::argmax_row_kernel<ms::bf16_t>, dim3(a->rows), dim3(1024), 0, stream, *a);
     else
       hipLaunchKernelGGL(ms::argmax_row_kernel<float>, dim3(a->rows), dim3(1024), 0, stream, *a);
     return hipGetLastError();
@@ -182,6 +184,8 @@ extern "C" hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipSt
   dim3 grid(a->chunks, a->rows);
   if (dtype == MI355X_F16)
     hipLaunchKernelGGL(ms::argmax_kernel<uint16_t>, grid, dim3(ms::kBlock), 0, stream, *a);
+  else if (dtype == MI355X_BF16)
+    hipLaunchKernelGGL(ms::argmax_kernel<ms::bf16_t>, grid, dim3(ms::kBlock), 0, stream, *a);
   else
     hipLaunchKernelGGL(ms::argmax_kernel<float>, grid, dim3(ms::kBlock), 0, stream, *a);
   return hipGetLastError();

@@ -363,33 +363,38 @@ struct Loader<float> {
   }
 };
 
-template <>
-struct Loader<uint16_t> {  // IEEE binary16 bit patterns
+template <typename T16>
+struct Loader16 {  // sixteen-bit elements: IEEE binary16 bit patterns (uint16_t) or bfloat16 (bf16_t)
   static constexpr int VEC = 8;
   static constexpr int NV = kElems / VEC;
   __device__ static __forceinline__ int index_of(int chunk, int j, int c) {
     return chunk * kChunk + (j * kBlock + static_cast<int>(threadIdx.x)) * VEC + c;
   }
-  __device__ static __forceinline__ void load(const uint16_t* row, bool aligned, int vocab, int chunk,
+  __device__ static __forceinline__ void load(const T16* row, bool aligned, int vocab, int chunk,
                                               float (&v)[kElems]) {
+    const uint16_t* const bits = reinterpret_cast<const uint16_t*>(row);
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int i0 = index_of(chunk, j, 0);
       if (aligned && i0 + VEC <= vocab) {
-        const uint4 q = *reinterpret_cast<const uint4*>(row + i0);
+        const uint4 q = *reinterpret_cast<const uint4*>(bits + i0);
         const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-          v[j * 8 + 2 * c] = half_bits_to_float(w[c] & 0xffffu);
-          v[j * 8 + 2 * c + 1] = half_bits_to_float(w[c] >> 16);
+          v[j * 8 + 2 * c] = narrow_bits_to_float<T16>(w[c] & 0xffffu);
+          v[j * 8 + 2 * c + 1] = narrow_bits_to_float<T16>(w[c] >> 16);
         }
       } else {
 #pragma unroll
-        for (int c = 0; c < VEC; ++c) v[j * 8 + c] = (i0 + c < vocab) ? half_bits_to_float(row[i0 + c]) : 0.0f;
+        for (int c = 0; c < VEC; ++c) v[j * 8 + c] = (i0 + c < vocab) ? narrow_bits_to_float<T16>(bits[i0 + c]) : 0.0f;
       }
     }
   }
 };
+template <>
+struct Loader<uint16_t> : Loader16<uint16_t> {};
+template <>
+struct Loader<bf16_t> : Loader16<bf16_t> {};
 
 // Applies the logits processing to the registers loaded by Loader<InT>::load.
 template <typename InT>

@@ -63,7 +63,8 @@ extern "C" int mi355x_argmax_static(void* stream, const void* logits, int dtype,
     return FailHere(MI355X_E_CAPACITY, "rows (%d) exceed the %d rows the static scratch holds; use mi355x_argmax", rows,
                     kStaticMaxRows);
   if (!logits || !out_tokens) return FailHere(MI355X_E_INVALID, "null logits or output");
-  if (dtype != MI355X_F32 && dtype != MI355X_F16) return FailHere(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
+  if (dtype != MI355X_F32 && dtype != MI355X_F16 && dtype != MI355X_BF16)
+    return FailHere(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
   if (row_stride < vocab) return FailHere(MI355X_E_INVALID, "row_stride smaller than vocab");
   hipStream_t s = static_cast<hipStream_t>(stream);
   ms::ArgmaxArgs a{};

@@ -143,6 +143,14 @@ def test_argmax_sixteen_bit_rows(ctx, orc, dtype):
     assert np.array_equal(ctx.argmax(x).cpu().numpy(), orc.argmax_batch(widened(orc, x)))
     y = x[:, 3:100003]  # rows that start off a 16-byte boundary
     assert np.array_equal(ctx.argmax(y).cpu().numpy(), orc.argmax_batch(widened(orc, y.contiguous())))
+    for width in (1, 7, 64):  # rows too short for the streaming kernel take the small kernels
+        z = x[:, 5:5 + width].contiguous()
+        assert np.array_equal(ctx.argmax(z).cpu().numpy(), orc.argmax_batch(widened(orc, z))), width
+    # the entry point without a context: the chunked kernel (rows x chunks >= 256) and the row kernel
+    for rows, vocab in ((40, 70001), (3, 5000)):
+        w = (torch.randn(rows, vocab, generator=g, device="cuda") * 2).to(dtype)
+        out = torch.empty(rows, dtype=torch.int32, device="cuda")
+        assert np.array_equal(pkg().argmax_static(w, out).cpu().numpy(), orc.argmax_batch(widened(orc, w))), (rows, vocab)
 
 
 def test_config2_shape_in_fp16_equals_fp32_on_the_widened_rows(ctx, orc):

@@ -14,7 +14,8 @@ def test_static_argmax_matches_context_argmax_twice():
     ctx = p.SearchContext(64, 151936)
     g = torch.Generator(device="cuda").manual_seed(7)
     # both shapes take the chunked kernel, the one that uses the scratch (rows x chunks >= 256)
-    for rows, vocab, dtype in ((64, 151936, torch.float16), (40, 70001, torch.float16), (33, 100003, torch.float32)):
+    for rows, vocab, dtype in ((64, 151936, torch.float16), (40, 70001, torch.float16), (33, 100003, torch.float32),
+                               (36, 66000, torch.bfloat16)):
         say("argmax_static", rows, vocab, dtype)
         x = (torch.randn(rows, vocab, generator=g, device="cuda") * 3).to(dtype)
         x[3, vocab - 1] = 40.0  # a winner in the last, partial chunk
