@@ -339,6 +339,48 @@ __device__ __forceinline__ void wave_topk_epilogue(u64 key, int m, mi355x_sample
   }
 }
 
+// The token alone, for calls that ask for nothing else: k <= 64, lane j holds the j-th best, j < m.
+// Every decision of wave_topk_epilogue -- where the top-p cut falls, which position the draw selects -- compares
+// a sequentially rounded fp32 or fp64 sum with a fixed number.  Here both are taken from ONE fp64 prefix sum of
+// the exponentials in tree order: S_j / S_{m-1} differs from the reference's cumulative probability by less than
+// 2 * 63 * 2^-24 + 2^-23 < 8e-6 (two sequential fp32 sums of at most 64 positive terms and one division), and
+// S_j / S_{keep-1} from its fp64 cumulative distribution by less than 3e-7 (the common factors cancel; two fp32
+// roundings per weight remain).  A comparison that falls inside those bands decides nothing: the function then
+// returns false and the caller runs wave_topk_epilogue, so the token is always the sequential one.
+__device__ __forceinline__ bool wave_topk_token_fast(u64 key, int m, mi355x_sample_params prm, float inv_temp, double u,
+                                                     LaneExp2Tab tab, int32_t* token) {
+  const int lane = lane_id();
+  m = __builtin_amdgcn_readfirstlane(m);
+  const float score = key_to_float(key64_okey(key));
+  const float max_score = read_lane(score, 0);
+  const float e_all = em::expf_core((score - max_score) * inv_temp, tab);
+  const double ed = lane < m ? static_cast<double>(e_all) : 0.0;
+  const double S = wave_scan_add(ed);
+  const double total = read_lane(S, m - 1);
+  bool decided = total >= 1.0 && total <= 128.0;  // the best element weighs exp(0) = 1; false for NaN weights
+  int keep = m;
+  if (prm.p > 0.0f && prm.p < 1.0f) {
+    const double mass = static_cast<double>(prm.p) * total;
+    const bool in_band = lane < m && fabs(S - mass) <= 1e-5 * total;
+    decided = decided && __ballot(in_band) == 0ull;
+    const int f = first_lane(__ballot(lane < m && S >= mass));
+    if (f >= 0) keep = f + 1;
+  }
+  int pos = 0;
+  if (keep >= 2) {
+    const double kept_total = read_lane(S, keep - 1);
+    const double target = u * kept_total;
+    const bool in_band = lane < keep - 1 && fabs(S - target) <= 1e-6 * kept_total;
+    decided = decided && __ballot(in_band) == 0ull;
+    pos = first_lane(__ballot(lane == keep - 1 || S >= target));
+  }
+  if (!decided) return false;
+  const uint32_t idx = key64_index(key);
+  const int32_t tok = static_cast<int32_t>(__builtin_amdgcn_readlane(idx, pos));
+  if (lane == 0) *token = tok;
+  return true;
+}
+
 static __device__ const uint64_t g_exp2_tab[32] = {
     0x3ff0000000000000ULL, 0x3fefd9b0d3158574ULL, 0x3fefb5586cf9890fULL, 0x3fef9301d0125b51ULL,
     0x3fef72b83c7d517bULL, 0x3fef54873168b9aaULL, 0x3fef387a6e756238ULL, 0x3fef1e9df51fdee1ULL,
@@ -926,6 +968,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     tab.hi = static_cast<uint32_t>(t >> 32);
   }
   const double u = emit_topk ? 0.0 : uniforms[row];
+  const float inv_temp = 1.0f / prm.temperature;
   // sm.own is written by wave 0; with at most four chunks wave 0 alone reads it (a wave's LDS accesses execute in order)
   if (n_chunks > 4) __syncthreads();
   u64* seg = cand_small + static_cast<size_t>(row) * n_chunks * kSmallCap;
@@ -997,10 +1040,13 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       } else {
         {
           RowOutputs out = outputs;  // pointers to this row's slots
-          out.kept_count = out.kept_count ? out.kept_count + row : nullptr;
-          out.kept_ids = out.kept_ids ? out.kept_ids + static_cast<size_t>(row) * out.kept_capacity : nullptr;
-          out.kept_probs = out.kept_probs ? out.kept_probs + static_cast<size_t>(row) * out.kept_capacity : nullptr;
-          wave_topk_epilogue(final_key, kk, prm, u, tab, out);
+          const bool token_only = !out.kept_count && !out.kept_ids && !out.kept_probs;
+          if (!(token_only && wave_topk_token_fast(final_key, kk, prm, inv_temp, u, tab, out.token))) {
+            out.kept_count = out.kept_count ? out.kept_count + row : nullptr;
+            out.kept_ids = out.kept_ids ? out.kept_ids + static_cast<size_t>(row) * out.kept_capacity : nullptr;
+            out.kept_probs = out.kept_probs ? out.kept_probs + static_cast<size_t>(row) * out.kept_capacity : nullptr;
+            wave_topk_epilogue(final_key, kk, prm, u, tab, out);
+          }
         }
       }
     }

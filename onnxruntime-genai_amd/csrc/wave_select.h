@@ -35,13 +35,38 @@ __device__ __forceinline__ u64 lane_xor64(u64 x) {
 }
 __device__ __forceinline__ uint32_t lane_xor_any(uint32_t x, int m) { return __shfl_xor(x, m, 64); }
 
+// The pair (own key, key of the lane J away) of a compare-exchange step on 32-bit keys, in an order that suits the
+// hardware: the two results of a permlane swap already are the pair's two members in every lane.
+template <int J>
+__device__ __forceinline__ void lane_pair(uint32_t x, uint32_t& a, uint32_t& b) {
+  if constexpr (J == 16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+    a = r[0];
+    b = r[1];
+  } else if constexpr (J == 32) {
+    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    a = r[0];
+    b = r[1];
+  } else {
+    a = x;
+    b = lane_xor<J>(x);
+  }
+}
+
 template <int K, int J, typename T>
 __device__ __forceinline__ void sort_merge(T& x, int lane) {
-  T y;
-  if constexpr (sizeof(T) == 8) y = lane_xor64<J>(x);
-  else y = lane_xor<J>(x);
   const bool keep_max = (((lane & K) == 0) == ((lane & J) == 0));
-  x = ((y > x) == keep_max) ? y : x;
+  if constexpr (sizeof(T) == 8) {
+    const T y = lane_xor64<J>(x);
+    x = ((y > x) == keep_max) ? y : x;
+  } else {
+    // maximum and minimum of the pair (the lane exchange folds into both instructions as a DPP operand), then
+    // one select on a lane mask that does not depend on the data
+    uint32_t a, b;
+    lane_pair<J>(x, a, b);
+    const uint32_t mx = a > b ? a : b, mn = a > b ? b : a;
+    x = keep_max ? mx : mn;
+  }
   if constexpr (J > 1) sort_merge<K, J / 2, T>(x, lane);
 }
 
