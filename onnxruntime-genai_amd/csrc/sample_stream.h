@@ -219,6 +219,8 @@ struct FusedShared {
   u64 own[64];              // the finishing workgroup's own list
   u64 lists[kAllCap / 4];   // first-level results of the finishing workgroup's merge (rows of > 4 chunks)
   uint32_t pool[64];
+  uint32_t n_hits;                // hits of the chunk on the ranking route of the top-k rows
+  uint32_t rank_failed;           // a wave or the chunk holds more hits than the ranking route provides for
   uint32_t wave_val[kSMaxWaves];
   u64 wave_val64[kSMaxWaves];
   uint32_t count, flag;
@@ -835,6 +837,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   if (static_cast<uint32_t>(n_lanes) < n_extra) n_lanes = n_extra < static_cast<uint32_t>(kSBlock) ? static_cast<int>(n_extra) : kSBlock;
   const size_t ci = static_cast<size_t>(row) * n_chunks + chunk;
   u64* dst = cand_small + ci * kSmallCap;
+  if (tid == 64) {  // ordered before the ranking route's atomics by the barrier of the bound
+    sm.n_hits = 0u;
+    sm.rank_failed = 0u;
+  }
   uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool);
   // The pooled bound is exact unless one wave holds more than its share of the best k; with k close to
   // 64 it can sit low enough for the hits to overflow their lists, and in a short tail chunk it may
@@ -906,6 +912,143 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     overflow = overflow || n_c > static_cast<uint32_t>(kListCap);
   };
   const bool pooled = tau != 0u;
+  const bool finisher = chunk == n_chunks - 1;
+  // ---- the ranking route ------------------------------------------------------------------------------
+  // A hit's place in the chunk's sorted list is the number of hits with a larger key, and with about sixty hits
+  // that is cheaper to count than to sort for.  Each wave walks its hits with scalar code (the lane's value is
+  // read into a scalar register, value and id are collected in lanes), reserves room in the chunk's list with
+  // one LDS atomic and appends its keys.  After a barrier every wave holds the whole list, a key per lane, and
+  // ranks an eighth of it: one 64-bit compare over the wave and a population count per hit -- exact whatever the
+  // ties, because the keys are distinct.  After a second barrier wave 0 publishes the ranked list.  More than 64
+  // hits in a wave or more than kListCap in the chunk: the listing and sorting route below does the chunk instead.
+  bool placed = false;
+  if (__builtin_expect(pooled && emit_topk != kEmitArgmax && !extra_overflow, 1)) {
+    const float tau_f = key_to_float(tau);
+    u64 qb[kSVec];
+#pragma unroll
+    for (int j = 0; j < kSVec; ++j) {
+      qb[j] = __ballot(qm[j] >= tau_f);
+      asm volatile("" : "+s"(qb[j]));  // all compares are issued before the first mask is looked at
+    }
+    uint32_t hx = 0u, hid = 0u;  // lane h: value bits and id of the wave's h-th hit
+    int n = 0;
+    // The hits of one register, whose lanes hold consecutive runs of ids (lane 0: id_lane0), or of one round over
+    // the history ids' list (LISTED: the ids come in `ids`).  Per hit: its lane, the lane's value into a scalar
+    // register, value and id into lane n of hx / hid (a lane number beyond 63 wraps; n > 64 is noticed below).
+    auto take = [&](u64 b, float val, uint32_t id_lane0, auto listed, uint32_t ids) {
+      while (b != 0ull) {
+        int l;
+        uint32_t xb, id;
+        if constexpr (decltype(listed)::value) {
+          asm volatile(
+              "s_ff1_i32_b64 %[l], %[b]\n\t"
+              "s_bitset0_b64 %[b], %[l]\n\t"
+              "v_readlane_b32 %[x], %[val], %[l]\n\t"
+              "v_readlane_b32 %[id], %[ids], %[l]\n\t"
+              "s_mov_b32 m0, %[n]\n\t"
+              "s_add_i32 %[n], %[n], 1\n\t"
+              "v_writelane_b32 %[hx], %[x], m0\n\t"
+              "v_writelane_b32 %[hid], %[id], m0"
+              : [b] "+s"(b), [n] "+s"(n), [hx] "+v"(hx), [hid] "+v"(hid), [l] "=&s"(l), [x] "=&s"(xb), [id] "=&s"(id)
+              : [val] "v"(val), [ids] "v"(ids)
+              : "m0", "scc");
+        } else if constexpr (VEC == 4) {
+          asm volatile(
+              "s_ff1_i32_b64 %[l], %[b]\n\t"
+              "s_bitset0_b64 %[b], %[l]\n\t"
+              "v_readlane_b32 %[x], %[val], %[l]\n\t"
+              "s_lshl2_add_u32 %[id], %[l], %[id0]\n\t"
+              "s_mov_b32 m0, %[n]\n\t"
+              "s_add_i32 %[n], %[n], 1\n\t"
+              "v_writelane_b32 %[hx], %[x], m0\n\t"
+              "v_writelane_b32 %[hid], %[id], m0"
+              : [b] "+s"(b), [n] "+s"(n), [hx] "+v"(hx), [hid] "+v"(hid), [l] "=&s"(l), [x] "=&s"(xb), [id] "=&s"(id)
+              : [val] "v"(val), [id0] "s"(id_lane0)
+              : "m0", "scc");
+        } else {
+          asm volatile(
+              "s_ff1_i32_b64 %[l], %[b]\n\t"
+              "s_bitset0_b64 %[b], %[l]\n\t"
+              "v_readlane_b32 %[x], %[val], %[l]\n\t"
+              "s_lshl3_add_u32 %[id], %[l], %[id0]\n\t"
+              "s_mov_b32 m0, %[n]\n\t"
+              "s_add_i32 %[n], %[n], 1\n\t"
+              "v_writelane_b32 %[hx], %[x], m0\n\t"
+              "v_writelane_b32 %[hid], %[id], m0"
+              : [b] "+s"(b), [n] "+s"(n), [hx] "+v"(hx), [hid] "+v"(hid), [l] "=&s"(l), [x] "=&s"(xb), [id] "=&s"(id)
+              : [val] "v"(val), [id0] "s"(id_lane0)
+              : "m0", "scc");
+        }
+      }
+    };
+    static_assert(VEC == 4 || VEC == 8, "a lane's run of ids is a shift of its number");
+    const uint32_t wave_id0 = static_cast<uint32_t>(chunk) * kSChunk +
+                              static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(wave)) * 64u * VEC;
+#pragma unroll
+    for (int j = 0; j < kSVec; ++j) {
+      if (qb[j] != 0ull) {
+        u64 eb[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) eb[c] = __ballot(v[j * 4 + c] >= tau_f);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          take(eb[c], v[j * 4 + c], wave_id0 + static_cast<uint32_t>(elem_offset<kSBlock, VEC>(j * 4 + c)), std::false_type{}, 0u);
+      }
+    }
+    for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
+      const uint32_t i = i0 + tid;
+      const float ev = i < n_extra ? sm.extra_val[i] : kNaN;
+      const uint32_t ei = i < n_extra ? sm.extra_idx[i] : 0u;
+      take(__ballot(ev >= tau_f), ev, 0u, std::true_type{}, ei);
+    }
+    u64* const hits = sm.wave_list;  // the chunk's hits as keys, in no order
+    uint32_t base = 0u;
+    if (lane == 0) base = atomicAdd(&sm.n_hits, static_cast<uint32_t>(n));
+    base = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(base)));
+    if (n > 64 || base + static_cast<uint32_t>(n) > static_cast<uint32_t>(kListCap)) {
+      if (lane == 0) sm.rank_failed = 1u;
+    } else if (lane < n) {
+      hits[base + lane] = make_key64(order_key(__uint_as_float(hx)), hid);
+    }
+    __syncthreads();
+    const uint32_t total = sm.n_hits;
+    placed = sm.rank_failed == 0u;
+    if (placed) {
+      // lane l holds hit l (and hit 64 + l of a long list); wave w ranks hits 8w .. 8w+7 (16w .. 16w+15), lane i the i-th
+      const bool wide = total > 64u;
+      const int per = wide ? 16 : 8;
+      const uint32_t first = static_cast<uint32_t>(wave * per);
+      const u64 mine0 = static_cast<uint32_t>(lane) < total ? hits[lane] : 0;
+      const u64 mykey = (lane < per && first + lane < total) ? hits[first + lane] : 0;
+      uint32_t myrank = 0u;
+      if (!wide) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const u64 key = read_lane(mine0, wave * 8 + i);
+          const int r = __popcll(__ballot(mine0 > key));
+          asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(myrank) : "s"(r), "n"(i));
+        }
+      } else {
+        const u64 mine1 = static_cast<uint32_t>(lane) + 64u < total ? hits[lane + 64] : 0;
+        const u64 src = wave < 4 ? mine0 : mine1;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const u64 key = read_lane(src, (wave * 16 + i) & 63);
+          const int r = __popcll(__ballot(mine0 > key)) + __popcll(__ballot(mine1 > key));
+          asm volatile("v_writelane_b32 %0, %1, %2" : "+v"(myrank) : "s"(r), "n"(i));
+        }
+      }
+      if (mykey != 0 && myrank < static_cast<uint32_t>(kSmallCap)) sm.own[myrank] = mykey;
+      __syncthreads();
+      if (wave == 0) {
+        const u64 slot = static_cast<uint32_t>(lane) < total ? sm.own[lane] : kSlotEmpty;
+        if (finisher) sm.own[lane] = slot;
+        else store_coherent(&dst[lane], slot);
+      }
+      if (!finisher) return false;
+    }
+  }
+  if (!placed) {
   if (__builtin_expect(!pooled, 0)) tau = exact_bound();
   list_hits(tau);
   if (__builtin_expect(overflow && pooled, 0)) {  // rare: a second, separate copy of the listing code, with the exact bound
@@ -923,7 +1066,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   // and a publishing workgroup never waits, so the lists a finishing workgroup polls for belong to
   // workgroups that are running or done.
   const bool two_halves = n_c > 64u;
-  const bool finisher = chunk == n_chunks - 1;
   u64 mykey = 0;
   if (wave < 2 && !overflow) {
     // entry p of the concatenated wave lists: list w covers [start_w, start_w + count_w)
@@ -958,6 +1100,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     if (finisher) sm.own[lane] = slot;
     else store_coherent(&dst[lane], slot);
   }
+  }  // !placed
   if (!finisher) return false;
 
   // ---- the row's finishing workgroup ---------------------------------------------------------------

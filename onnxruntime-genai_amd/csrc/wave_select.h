@@ -70,16 +70,71 @@ __device__ __forceinline__ void sort_merge(T& x, int lane) {
   if constexpr (J > 1) sort_merge<K, J / 2, T>(x, lane);
 }
 
+// The two members of the pair (lane, lane ^ J) of a compare-exchange step on 64-bit keys: lo = the key of the lane
+// whose bit J is clear, hi = the other one, both in both lanes.  For J = 16 and 32 the two results of a permlane
+// swap are exactly that; for the shorter distances a lane reads its partner and sorts out which is which.
+template <int J>
+__device__ __forceinline__ void lane_pair64(u64 x, int lane, u64& lo, u64& hi) {
+  const uint32_t x0 = static_cast<uint32_t>(x), x1 = static_cast<uint32_t>(x >> 32);
+  if constexpr (J == 16) {
+    const auto r0 = __builtin_amdgcn_permlane16_swap(x0, x0, false, false);
+    const auto r1 = __builtin_amdgcn_permlane16_swap(x1, x1, false, false);
+    lo = (static_cast<u64>(r1[0]) << 32) | r0[0];
+    hi = (static_cast<u64>(r1[1]) << 32) | r0[1];
+  } else if constexpr (J == 32) {
+    const auto r0 = __builtin_amdgcn_permlane32_swap(x0, x0, false, false);
+    const auto r1 = __builtin_amdgcn_permlane32_swap(x1, x1, false, false);
+    lo = (static_cast<u64>(r1[0]) << 32) | r0[0];
+    hi = (static_cast<u64>(r1[1]) << 32) | r0[1];
+  } else {
+    const u64 y = lane_xor64<J>(x);
+    const bool upper = (lane & J) != 0;
+    lo = upper ? y : x;
+    hi = upper ? x : y;
+  }
+}
+
 // Bitonic merge of a bitonic sequence held one key per lane: the result is sorted by lane, descending,
 // or ascending if ASC.
 template <int J, bool ASC, typename T>
 __device__ __forceinline__ void bitonic_merge(T& x, int lane) {
-  T y;
-  if constexpr (sizeof(T) == 8) y = lane_xor64<J>(x);
-  else y = lane_xor<J>(x);
-  const bool keep_max = ((lane & J) == 0) != ASC;
-  x = ((y > x) == keep_max) ? y : x;
+  if constexpr (sizeof(T) == 8 && J >= 16) {
+    u64 lo, hi;
+    lane_pair64<J>(x, lane, lo, hi);
+    const bool upper = (lane & J) != 0;
+    x = ((hi > lo) != (upper != ASC)) ? hi : lo;  // descending: the lower lane keeps the larger key
+  } else {
+    T y;
+    if constexpr (sizeof(T) == 8) y = lane_xor64<J>(x);
+    else y = lane_xor<J>(x);
+    const bool keep_max = ((lane & J) == 0) != ASC;
+    x = ((y > x) == keep_max) ? y : x;
+  }
   if constexpr (J > 1) bitonic_merge<J / 2, ASC, T>(x, lane);
+}
+
+// The same for two independent sequences at once, a descending and b ascending: the two dependent chains
+// are written step by step side by side, so that the instructions of one fill the waits of the other.
+template <int J>
+__device__ __forceinline__ void bitonic_merge_two(u64& a, u64& b, int lane) {
+  const bool upper = (lane & J) != 0;
+  if constexpr (J >= 16) {
+    u64 alo, ahi, blo, bhi;
+    lane_pair64<J>(a, lane, alo, ahi);
+    lane_pair64<J>(b, lane, blo, bhi);
+    const bool ta = (ahi > alo) != upper;
+    const bool tb = (bhi > blo) == upper;
+    a = ta ? ahi : alo;
+    b = tb ? bhi : blo;
+  } else {
+    const u64 ya = lane_xor64<J>(a);
+    const u64 yb = lane_xor64<J>(b);
+    const bool ta = (ya > a) != upper;
+    const bool tb = (yb > b) == upper;
+    a = ta ? ya : a;
+    b = tb ? yb : b;
+  }
+  if constexpr (J > 1) bitonic_merge_two<J / 2>(a, b, lane);
 }
 
 // The 64 largest of four lists of 64 keys, each sorted descending (list(c, i) = i-th best of list c, 0 for
@@ -91,8 +146,7 @@ __device__ __forceinline__ u64 wave_merge4(List list, int lane) {
   const u64 a0 = list(0, lane), a1 = list(1, 63 - lane), b0 = list(2, 63 - lane), b1 = list(3, lane);
   u64 a = a1 > a0 ? a1 : a0;
   u64 b = b1 > b0 ? b1 : b0;
-  bitonic_merge<32, false, u64>(a, lane);
-  bitonic_merge<32, true, u64>(b, lane);
+  bitonic_merge_two<32>(a, b, lane);
   u64 g = b > a ? b : a;
   bitonic_merge<32, false, u64>(g, lane);
   return g;
