@@ -25,7 +25,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 // argument object with a run-time row would make the compiler copy the whole object to private memory.
 static_assert(sizeof(SampleArgs) % alignof(InlineParams) == 0, "the table follows the first argument without padding");
 template <bool INLINE>
-__device__ __forceinline__ mi355x_sample_params row_params(const SampleArgs& a, int row) {
+__device__ __forceinline__ mi355x_sample_params row_params(const SampleArgs& a, int row, mi355x_sample_params uniform) {
   if constexpr (INLINE) {
     typedef __attribute__((address_space(4))) const char* KernargPtr;
     const KernargPtr base = (KernargPtr)__builtin_amdgcn_kernarg_segment_ptr();
@@ -40,7 +40,7 @@ __device__ __forceinline__ mi355x_sample_params row_params(const SampleArgs& a, 
     // The device table is read-only during the launch: read through the constant address space, its
     // entries come by scalar loads like the uniform parameters from the kernel arguments, the row's mode
     // is a scalar, and nothing here waits for a vector load before the logits are requested.
-    mi355x_sample_params q = a.uniform;
+    mi355x_sample_params q = uniform;
     if (a.per_row) {
       typedef __attribute__((address_space(4))) const mi355x_sample_params* TablePtr;
       const TablePtr table = (TablePtr)a.per_row;
@@ -50,6 +50,10 @@ __device__ __forceinline__ mi355x_sample_params row_params(const SampleArgs& a, 
     }
     return q;
   }
+}
+template <bool INLINE>
+__device__ __forceinline__ mi355x_sample_params row_params(const SampleArgs& a, int row) {
+  return row_params<INLINE>(a, row, a.uniform);
 }
 
 __device__ __forceinline__ int next_pow2(int v) {
@@ -219,6 +223,7 @@ struct FusedShared {
   u64 own[64];              // the finishing workgroup's own list
   u64 lists[kAllCap / 4];   // first-level results of the finishing workgroup's merge (rows of > 4 chunks)
   uint32_t pool[64];
+  uint32_t poisoned;              // the workgroup's copy of the flag that sends every row to the exact path
   uint32_t n_hits;                // hits of the chunk on the ranking route of the top-k rows
   uint32_t rank_failed;           // a wave or the chunk holds more hits than the ranking route provides for
   uint32_t wave_val[kSMaxWaves];
@@ -463,9 +468,21 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   const InT* lrow = static_cast<const InT*>(row0);
   const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
   const float kNaN = __uint_as_float(0x7fc00000u);  // marks ids >= vocab: never a maximum, never >= a bound
-  const uint32_t poison = a.fallback_rows[1];  // needed after the streaming pass only
   float v[kSElems];
+  // a chunk that lies inside an aligned row requests its loads without a test between them
+  const bool whole_chunk = aligned && (chunk + 1) * kSChunk <= V;
   if constexpr (VEC == 4) {
+    if (whole_chunk) {
+      const v4f* src = reinterpret_cast<const v4f*>(lrow + static_cast<size_t>(chunk) * kSChunk) + tid;
+#pragma unroll
+      for (int j = 0; j < kSLoads; ++j) {
+        const v4f q = __builtin_nontemporal_load(src + j * kSBlock);
+        v[j * 4 + 0] = q.x;
+        v[j * 4 + 1] = q.y;
+        v[j * 4 + 2] = q.z;
+        v[j * 4 + 3] = q.w;
+      }
+    } else
 #pragma unroll
     for (int j = 0; j < kSLoads; ++j) {
       const int i0 = elem_index<kSBlock, VEC>(chunk, j, 0);
@@ -504,6 +521,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       }
     }
   }
+  // One thread reads the flag that sends every row to the exact path, and the workgroup looks at that copy behind
+  // its first barrier: read by every wave for itself, at its own time, a flag raised in between would send some
+  // waves of a workgroup one way and the rest the other, with barriers waiting on both sides.
+  if (tid == 0) sm.poisoned = a.fallback_rows[1];
   // The arguments the phases after the streaming pass need are fetched now, while the logits are in
   // flight, instead of one by one where they are first used.
   const int n_chunks = arg_now(a.chunks);
@@ -768,8 +789,8 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   }
 
   // A finishing workgroup that once gave up waiting may have left published lists behind; from then on
-  // (the flag word next to the fallback counter) every row takes the exact path, which reads no such state.
-  if (poison != 0u) return chunk == n_chunks - 1;
+  // (the flag word next to the fallback counter, copied to sm.poisoned) every row takes the exact path, which
+  // reads no such state.
   if constexpr (ARGMAX) {
     // ---- argmax ---------------------------------------------------------------------------------
     // ArgMax (src/search.h:9-29) keeps id 0 unless a later value compares greater: the largest value, the
@@ -794,6 +815,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     if (lane == 0) sm.list_hi[wave] = key;
     lds_barrier();
     const bool finisher = chunk == n_chunks - 1;
+    if (sm.poisoned != 0u) return finisher;
     if (wave != 0 && !finisher) return false;
     if (wave == 0) {
       key = lane < kSWaves ? sm.list_hi[lane] : 0;
@@ -842,6 +864,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     sm.rank_failed = 0u;
   }
   uint32_t tau = block_pool_bound(lmax, kk, (n_lanes + 63) / 64, sm.pool);
+  if (sm.poisoned != 0u) return chunk == n_chunks - 1;
   // The pooled bound is exact unless one wave holds more than its share of the best k; with k close to
   // 64 it can sit low enough for the hits to overflow their lists, and in a short tail chunk it may
   // find fewer than k offers (0).  Either way the exact k-th best of the per-thread maxima takes its
@@ -1201,11 +1224,35 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
 // Rows in nucleus mode and all other rows are streamed by kernels of their own (a launch may need
 // both): each kernel holds the code of its mode only, and a change to one path leaves the machine
 // code of the other as it was.
+// The arguments a streaming kernel reads before it requests its logits, fetched together.  Kernel arguments come by
+// scalar loads that return out of order, so every wait for one of them waits for all that are under way, and a
+// value first needed behind a branch is requested behind that branch: left alone, five such round trips (per-row
+// table? shape, mode, row pointer, flag word) stood in front of the first logits request of every wave.
+// Returns the uniform (k, p, T) as values that exist before the first branch.
+__device__ __forceinline__ mi355x_sample_params args_up_front(const SampleArgs& a) {
+  const void* logits = a.logits;
+  int64_t row_stride = a.row_stride;
+  int vocab = a.vocab, chunks = a.chunks, k = a.uniform.k, emit_topk = a.emit_topk, exact_kernel = a.exact_kernel;
+  float p = a.uniform.p, temperature = a.uniform.temperature;
+  const mi355x_sample_params* per_row = a.per_row;
+  uint32_t* fallback_rows = a.fallback_rows;
+  uint32_t* row_done = a.row_done;
+  asm volatile(""
+               : "+s"(logits), "+s"(row_stride), "+s"(vocab), "+s"(chunks), "+s"(k), "+s"(p), "+s"(temperature), "+s"(per_row),
+                 "+s"(emit_topk), "+s"(exact_kernel), "+s"(fallback_rows), "+s"(row_done));
+  mi355x_sample_params q;
+  q.k = k;
+  q.p = p;
+  q.temperature = temperature;
+  return q;
+}
+
 template <typename InT, bool INLINE, bool NUCLEUS, bool XFORM, bool LARGEK = false, bool ARGMAX = false>
 __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
+  const mi355x_sample_params uniform_prm = args_up_front(a);
   const int row = blockIdx.y, chunk = blockIdx.x;
   __shared__ FusedShared sm;
-  const mi355x_sample_params prm = row_params<INLINE>(a, row);
+  const mi355x_sample_params prm = row_params<INLINE>(a, row, uniform_prm);
   const void* const row0 = row_start<INLINE>(a, row, sizeof(InT));
   const int mode = row_mode(prm, a.vocab, a.chunks, a.emit_topk);
   if constexpr (NUCLEUS) {
