@@ -28,6 +28,11 @@ MEASURED_TRAFFIC_BYTES = 33_460_000
 TRAFFIC_SOURCE = "offline profile constant: profiles/sample_fused_kernel_config2_pmc.md"
 
 
+def replays_for(K):
+    """Replays of a K-step graph inside one timed region: at least 8, and at least 1024 steps in all."""
+    return max(8, -(-1024 // K))
+
+
 def time_fp16_steps(torch, np, orc, ctx, side, logits, uniforms, u_host, W, K, pool, n_cpu):
     """The same K steps on fp16 copies of the logits, read directly by the sampling kernel (no widening pass):
     graph replay between two events as for the fp32 run; the tokens of the first n_cpu steps must equal the CPU
@@ -48,9 +53,11 @@ def time_fp16_steps(torch, np, orc, ctx, side, logits, uniforms, u_host, W, K, p
                 step16(i)
         g16.replay()
         side.synchronize()
+        R = replays_for(K)
         s16, e16 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         s16.record(side)
-        g16.replay()
+        for _ in range(R):
+            g16.replay()
         e16.record(side)
         side.synchronize()
     torch.cuda.synchronize()
@@ -60,7 +67,7 @@ def time_fp16_steps(torch, np, orc, ctx, side, logits, uniforms, u_host, W, K, p
         want = orc.sample_batch(wide, TOP_K, TOP_P, TEMP, u_host[W + i])
         if not np.array_equal(tok16[W + i].cpu().numpy(), want):
             sys.exit("PARITY FAILURE: tokens sampled from fp16 logits differ from the CPU oracle on the widened rows")
-    return s16.elapsed_time(e16), n
+    return s16.elapsed_time(e16) / R, n
 
 
 def time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, tokens, pool, W, K):
@@ -87,15 +94,17 @@ def time_batches_in_flight(torch, pkg, ctx, side, n_streams, logits, uniforms, t
                 side.wait_stream(s)
         graph3.replay()
         side.synchronize()
+        R = replays_for(K)
         start3, end3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start3.record(side)
-        graph3.replay()
+        for _ in range(R):
+            graph3.replay()
         end3.record(side)
         side.synchronize()
     torch.cuda.synchronize()
     if not torch.equal(tokens[W:W + K], seq_tokens):
         sys.exit("PARITY FAILURE: tokens differ between the sequential run and the run with several batches in flight")
-    overlapped_ms = start3.elapsed_time(end3)
+    overlapped_ms = start3.elapsed_time(end3) / R
     for c in ctxs[1:]:
         c.close()
     return overlapped_ms
@@ -157,6 +166,9 @@ def main():
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
                     help="c2 (default) is the headline configuration; the others time the remaining "
                          "configurations with the same JSON shape")
+    ap.add_argument("--other-configs", type=int, default=1,
+                    help="c2 only: 1 (default) also runs configurations 1, 3, 4 and 5 after the headline measurement and "
+                         "reports them under config.other_configs; 0 skips them")
     ap.add_argument("--batches-in-flight", type=int, default=3,
                     help="c2 only: after the timed sequential run, also time the same steps spread over this many "
                          "streams and contexts (informational field of the JSON line; 0 skips it, which keeps a "
@@ -225,13 +237,17 @@ def main():
                 step(i)
         graph.replay()  # first replay untimed (graph upload)
         side.synchronize()
+        # The K-step graph is replayed R times between the two events and the time divided by R: what one replay
+        # pays for being launched is spread over R * K steps, so the figure does not depend on K.
+        R = replays_for(K)
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record(side)
-        graph.replay()
+        for _ in range(R):
+            graph.replay()
         end.record(side)
         side.synchronize()
     torch.cuda.synchronize()
-    gpu_ms = start.elapsed_time(end)
+    gpu_ms = start.elapsed_time(end) / R
     got = tokens[W:W + n_cpu].cpu().numpy()
     cpu_in = [logits[(W + i) % pool].cpu().numpy() for i in range(n_cpu)]
     t0 = time.perf_counter()
@@ -279,6 +295,25 @@ def main():
 
     fp16_ms, fp16_checked = time_fp16_steps(torch, np, orc, ctx, side, logits, uniforms, u_host, W, K, pool, n_cpu)
     copy_gbps = hbm_copy_probe(torch, dev)
+    ctx.close()
+    del logits, uniforms, tokens
+    torch.cuda.empty_cache()
+    # ---- the other four configurations, each with its own parity gate (informational, not `value`) ---------
+    other = {}
+    if args.other_configs:
+        import bench_workloads
+        for name in ("c1", "c3", "c4", "c5"):
+            sub = argparse.Namespace(**vars(args))
+            sub.workload = name
+            line = bench_workloads.run(sub, pkg, orc, orc_lib, dev)
+            other[name] = {"us_per_step": line["ms_per_step"] * 1e3, "steps": line["steps"],
+                           "value": line["value"], "unit": line["unit"],
+                           "roofline_frac": line["roofline"]["frac"] if name in ("c3", "c5") else None,
+                           "parity": line["config"]["parity"]}
+            for key in ("select_ms_per_step", "kv_gather_ms_per_step", "kv_gather_frac_of_peak"):
+                if key in line["config"]:
+                    other[name][key] = line["config"][key]
+            torch.cuda.empty_cache()
     ms_per_step = gpu_ms / K
     algo_bytes = ROWS * VOCAB * 4 + ROWS * 8 + ROWS * 4  # logits once + uniforms + tokens
     achieved = algo_bytes / (ms_per_step * 1e-3) / 1e9
@@ -307,6 +342,9 @@ def main():
                                "logits buffers" % (K, pool),
                    "rows": ROWS, "vocab": VOCAB, "top_k": TOP_K, "top_p": TOP_P, "temperature": TEMP,
                    "parity": parity,
+                   "timed_region": "%d replays of the %d-step graph between two HIP events; ms_per_step = time / "
+                                   "(%d * %d)" % (replays_for(K), K, replays_for(K), K),
+                   "other_configs": other,
                    "general_path_rows": fallback,
                    "single_step_latency": latency,
                    "fp16_logits": {

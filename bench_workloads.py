@@ -26,6 +26,7 @@ def _timed(fn_step, K, W, graph=True):
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    R = 1
     with torch.cuda.stream(side):
         if graph:
             g = torch.cuda.CUDAGraph()
@@ -34,8 +35,10 @@ def _timed(fn_step, K, W, graph=True):
                     fn_step(i)
             g.replay()
             side.synchronize()
+            R = max(8, -(-1024 // K))  # replays inside the timed region, as in the headline run
             start.record(side)
-            g.replay()
+            for _ in range(R):
+                g.replay()
             end.record(side)
         else:
             start.record(side)
@@ -44,7 +47,7 @@ def _timed(fn_step, K, W, graph=True):
             end.record(side)
         side.synchronize()
     torch.cuda.synchronize()
-    return start.elapsed_time(end)
+    return start.elapsed_time(end) / R
 
 
 def _line(args, metric, unit, value, ms_total, K, W, dtype, workload, extra, algo_bytes, cpu):
@@ -107,7 +110,7 @@ def c3(args, pkg, orc, orc_lib, dev):
     [32, 4, 2048, 128] fp16 per step."""
     B, NB, V, L2, MAXLEN = 8, 4, 151936, 56, 96
     BB = B * NB
-    K = args.steps if args.steps != 128 else 64
+    K = min(args.steps, 88) if args.steps != 128 else 64  # the sequences hold 96 tokens: prompt 3 + warm-up 4 + K
     W = min(args.warmup, 4)
     g = torch.Generator(device=dev).manual_seed(3)
     pool = 16
