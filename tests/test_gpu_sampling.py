@@ -216,6 +216,74 @@ def test_draw_on_cdf_boundaries(ctx, orc, vocab, k, p, t):
     sample_and_check(ctx, orc, x, us, k, p, t, cap=64)
 
 
+def tokens_only(ctx, x, u, k, p, t):
+    """A call that asks for the tokens alone (no kept sets): the route the benchmark times."""
+    return ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(np.asarray(u, np.float64)).cuda(), k=k, p=p,
+                      temperature=t).cpu().numpy()
+
+
+@pytest.mark.parametrize("rows,vocab,k,p,t", [
+    (64, 128256, 50, 0.9, 0.7), (32, 128256, 64, 0.95, 1.0), (16, 201088, 40, 0.5, 1.3), (8, 4099, 50, 0.0, 1.0),
+    (8, 32064, 2, 0.9, 0.25), (8, 70001, 17, 1.0, 2.0), (4, 300, 50, 0.9, 1.0),
+])
+def test_token_only_calls_match_the_oracle(ctx, orc, rows, vocab, k, p, t):
+    """Calls without kept-set outputs decide the nucleus cut and the draw from one fp64 prefix sum with guard
+    bands; the tokens must be the ones the sequential arithmetic of the reference yields."""
+    say("token only", rows, vocab, k, p, t)
+    rng = np.random.default_rng(vocab * 7 + k)
+    for rep in range(3):
+        x = (rng.standard_normal((rows, vocab)) * (1.0 + 2.0 * rep)).astype(np.float32)
+        if rep == 2:
+            x = np.round(x * 4) / 4  # heavy ties
+        u = rng.random(rows)
+        got = tokens_only(ctx, x, u, k, p, t)
+        assert np.array_equal(got, orc.sample_batch(x, k, p, t, u)), rep
+
+
+@pytest.mark.parametrize("vocab,k,t", [(128256, 50, 0.7), (5000, 30, 1.0), (40000, 64, 1.5)])
+def test_token_only_calls_on_the_edges_of_their_guard_bands(ctx, orc, vocab, k, t):
+    """Token-only calls with draws placed on, just below and just above the values of the cumulative
+    distribution, and with top-p masses placed on, just below and just above the fp32 cumulative probabilities
+    of the reference's cut loop: none of these can be decided from the prefix sum in tree order, so the kernel
+    must notice and run the sequential epilogue."""
+    say("token only edges", vocab, k, t)
+    rng = np.random.default_rng(vocab + k)
+    base = (rng.standard_normal(vocab) * 3).astype(np.float32)
+    # draws on the boundaries of the final distribution, for a cut in the middle and for no cut
+    for p in (0.9, 0.0):
+        idx, probs = orc.sampled_categorical(base, k, p, t)
+        assert len(idx) >= 3
+        total = 0.0
+        for q in probs:
+            total += float(q)
+        cp, run = [], 0.0
+        for q in probs[:-1]:
+            run += float(q) / total
+            cp.append(run)
+        us = []
+        for j in sorted({0, 1, len(cp) // 2, len(cp) - 1}):
+            us += [cp[j], np.nextafter(cp[j], 0.0), np.nextafter(cp[j], 1.0)]
+        us = np.array([v for v in us if 0.0 <= v < 1.0], np.float64)
+        x = np.tile(base, (len(us), 1))
+        assert np.array_equal(tokens_only(ctx, x, us, k, p, t), orc.sample_batch(x, k, p, t, us))
+    # masses on the boundaries of the cut: the reference adds the fp32 probabilities in rank order
+    _, pr = orc.sampled_categorical(base, k, 0.0, t)
+    cum, run = [], np.float32(0.0)
+    for q in pr:
+        run = np.float32(run + q)
+        cum.append(run)
+    u = rng.random(8)
+    x = np.tile(base, (len(u), 1))
+    for j in sorted({0, 1, len(cum) // 3, len(cum) // 2, len(cum) - 2}):
+        for mass in (cum[j], np.nextafter(cum[j], np.float32(0)), np.nextafter(cum[j], np.float32(1))):
+            mass = float(mass)
+            if not 0.0 < mass < 1.0:
+                continue
+            kept = len(orc.sampled_categorical(base, k, mass, t)[0])
+            assert kept in (j + 1, j + 2), (j, mass, kept)  # the cut really falls where the mass was placed
+            assert np.array_equal(tokens_only(ctx, x, u, k, mass, t), orc.sample_batch(x, k, mass, t, u)), (j, mass)
+
+
 def test_config2_topk_topp_batch64(ctx, orc):
     """Benchmark configuration 2 at full size: batch 64, vocab 128256, N(0,3^2) logits + 8 peaks/row at +10,
     T=0.7, k=50, p=0.9, shared uniforms; 4 of the 128 steps."""
