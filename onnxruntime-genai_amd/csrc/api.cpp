@@ -453,7 +453,7 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   if (!logits || !out_tokens || !out_scores) return Fail(MI355X_E_INVALID, "null logits or output");
   if (dtype != MI355X_F32 && dtype != MI355X_F16 && dtype != MI355X_BF16)
     return Fail(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
-  if (k < 1 || k > 64 || k > vocab) return Fail(MI355X_E_INVALID, "k (%d) must be in [1, min(64, vocab)]", k);
+  if (k < 1 || k > vocab) return Fail(MI355X_E_INVALID, "k (%d) must be in [1, vocab]", k);
   if (row_stride < vocab) return Fail(MI355X_E_INVALID, "row_stride smaller than vocab");
   hipStream_t s = static_cast<hipStream_t>(stream);
   // sixteen-bit rows are read as they are and widened in registers (DeviceInterface::TopKScores makes an fp32
@@ -475,10 +475,18 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   a.chunk_max = ctx->chunk_max;
   a.chunk_next = ctx->chunk_next;
   a.big = ctx->big;
+  a.big2 = ctx->big2;
   a.big_stride = ctx->big_stride;
   a.fallback_rows = ctx->fallback_rows;
   a.poll_limit = ctx->poll_limit;
-  HIP_TRY(ms_launch_sample(&a, nullptr, true, false, false, s));
+  // up to 64: the fused kernel's sorted candidate lists; up to kLargeKMax: the candidate lists of the large-k
+  // sampling route with an epilogue that emits instead of drawing; beyond (and for rows of more chunks than a
+  // finishing workgroup ranks): the exact path's whole-row sort.  The kernels' own rule (row_mode) decides.
+  const bool fits = vocab > 64 && a.chunks * ms::kSmallCap <= ms::kAllCap;
+  const bool large_k = fits && k > 64 && k <= ms::kLargeKMax;
+  const bool exact = vocab > 64 && (!fits || k > ms::kLargeKMax);
+  a.exact_kernel = exact ? 1 : 0;
+  HIP_TRY(ms_launch_sample(&a, nullptr, !large_k && !exact, false, large_k, s));
   return MI355X_OK;
 }
 

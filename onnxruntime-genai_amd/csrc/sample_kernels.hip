@@ -371,7 +371,8 @@ struct SortWithTile {
 __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucket_start, uint32_t n_c, u64 best_below,
                                                   uint32_t rmax, uint32_t thr, bool cut_at_best_below,
                                                   mi355x_sample_params prm, int V, double u, const RowOutputs& out,
-                                                  SeqShared& seqsh, uint32_t* red32) {
+                                                  SeqShared& seqsh, uint32_t* red32, const SampleArgs* emit = nullptr,
+                                                  int emit_row = 0, const void* emit_row0 = nullptr) {
   const int tid = threadIdx.x;
   if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
   if (best_below != 0) n_c += 1;
@@ -392,6 +393,19 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
       case 8: block_sort_desc_regs<8>(lds_keys); break;
       default: block_sort_desc_regs<16>(lds_keys); break;
     }
+  }
+  if (emit) {
+    // DeviceInterface::TopKScores: the k best ids and their raw scores, best first (the value itself is read again:
+    // keys do not tell -0 from +0); fewer than k numbers among the candidates: the exact path decides
+    const int kk = prm.k < V ? prm.k : V;
+    if (n_c < static_cast<uint32_t>(kk) || lds_keys[kk - 1] == 0) return false;
+    const RowPtr<AnyDtype> lrow(emit_row0, emit->dtype);
+    for (int j = tid; j < kk; j += blockDim.x) {
+      const uint32_t id = key64_index(lds_keys[j]);
+      emit->out_tokens[static_cast<size_t>(emit_row) * prm.k + j] = static_cast<int32_t>(id);
+      emit->out_scores[static_cast<size_t>(emit_row) * prm.k + j] = lrow[id];
+    }
+    return true;
   }
   if (cut_at_best_below && best_below != 0) {
     // keys are distinct: exactly one thread finds it
@@ -549,7 +563,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   const int V = a.vocab;
   const int tid = threadIdx.x;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
-  if (row_mode(prm, V, a.chunks) != (LARGEK ? kModeTopkLarge : kModeNucleus)) return;
+  if (row_mode(prm, V, a.chunks, a.emit_topk) != (LARGEK ? kModeTopkLarge : kModeNucleus)) return;
   if (!LARGEK && a.xf.mask && a.row_done && a.row_done[row] != 0u) return;  // finished by the sparse-mask kernel
   constexpr bool large_k = LARGEK;  // then every listed element is a candidate and no element after them is needed
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
@@ -737,8 +751,10 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   if (large_k) thr = ~block_max<uint32_t>(~lowest, red32);  // the lowest candidate score: the sort scales its buckets by it
   if (ok && !large_k) trim_to_nucleus(lds_keys, bucket_start, n_c, best_below, rmax, thr, prm, V, red32, red64, &sh_count);
   if (ok) {
-    ok = finish_candidates(lds_keys, bucket_start, n_c, best_below, rmax, thr, false, prm, V, a.uniforms[row],
-                           row_outputs(a, row), seqsh, red32);
+    const bool emit = large_k && a.emit_topk == 1;
+    ok = finish_candidates(lds_keys, bucket_start, n_c, best_below, rmax, thr, false, prm, V, emit ? 0.0 : a.uniforms[row],
+                           row_outputs(a, row), seqsh, red32, emit ? &a : nullptr, row,
+                           emit ? row_start<INLINE>(a, row, dtype_bytes(a.dtype)) : nullptr);
   }
   if (!ok) {
     __syncthreads();
@@ -997,7 +1013,7 @@ __device__ __forceinline__ void exact_rows_body(const SampleArgs& a) {
   __shared__ u64 red64[16];
   const int row = blockIdx.x;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
-  if (row_mode(prm, a.vocab, a.chunks) != kModeGeneral) return;
+  if (row_mode(prm, a.vocab, a.chunks, a.emit_topk) != kModeGeneral) return;
   general_row<AnyDtype, SortWithTile, 8>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, a.big + static_cast<size_t>(row) * a.big_stride,
                         seqsh,
                         SortWithTile{a.big2 ? a.big2 + static_cast<size_t>(row) * a.big_stride : nullptr, lds_keys, red32, red64});

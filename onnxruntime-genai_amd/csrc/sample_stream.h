@@ -189,8 +189,8 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const 
 
 __device__ __forceinline__ int row_mode(mi355x_sample_params prm, int vocab, int chunks, int emit_topk = 0) {
   if (vocab <= 64 || chunks * kSmallCap > kAllCap) return kModeGeneral;
-  if (emit_topk) return kModeTopkSmall;
-  if (prm.k > 1) {
+  if (emit_topk == kEmitArgmax) return kModeTopkSmall;
+  if (prm.k > 1 || emit_topk) {
     const int kk = prm.k < vocab ? prm.k : vocab;
     return kk <= 64 ? kModeTopkSmall : (kk <= kLargeKMax ? kModeTopkLarge : kModeGeneral);
   }

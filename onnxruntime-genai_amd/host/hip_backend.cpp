@@ -284,7 +284,7 @@ struct HipInterface final : DeviceInterface {
   bool TopKScores(const void* logits, ONNXTensorElementDataType type, int num_rows, int vocab_size, int k,
                   int32_t* out_tokens, float* out_scores) override {
     const int dt = DtypeCode(type);
-    if (!dt || k < 1 || k > 64 || k > vocab_size) return false;
+    if (!dt || k < 1 || k > vocab_size) return false;  // any k, as the CUDA add-on's (src/cuda/interface.cpp:503-553)
     std::lock_guard<std::mutex> lock(mutex_);
     EnsureSmall(static_cast<size_t>(num_rows) * k);
     AbiCheck(mi355x_topk_scores(Scratch(num_rows, vocab_size), g_stream, logits, dt, vocab_size, num_rows, vocab_size, k,
@@ -298,11 +298,18 @@ struct HipInterface final : DeviceInterface {
  private:
   mi355x_search_ctx* Scratch(int rows, int vocab) {
     if (!scratch_ || rows > scratch_rows_ || vocab > scratch_vocab_) {
+      // The workspace grows in steps (rows to the next power of two from 16, the vocabulary to the next multiple of
+      // 64K ids from 256K), so that a caller whose shapes creep up -- one more row of a speculative round, a larger
+      // model -- pays for a new context (a synchronisation, hipFree and hipMalloc) a few times, not at every call.
       HIP_CHECK(hipStreamSynchronize(g_stream));
       if (scratch_) mi355x_search_destroy(scratch_);
       scratch_ = nullptr;
-      scratch_rows_ = std::max(rows, scratch_rows_);
-      scratch_vocab_ = std::max(vocab, scratch_vocab_);
+      int want_rows = std::max(16, scratch_rows_);
+      while (want_rows < rows) want_rows *= 2;
+      int want_vocab = std::max(262144, scratch_vocab_);
+      while (want_vocab < vocab) want_vocab += 65536;
+      scratch_rows_ = want_rows;
+      scratch_vocab_ = want_vocab;
       AbiCheck(mi355x_search_create(0, scratch_rows_, scratch_vocab_, &scratch_));
     }
     return scratch_;

@@ -279,7 +279,25 @@ void DeviceFastPaths() {
       EXPECT_EQ(top_scores[r * k + j], row[order[j]]);
     }
   }
-  EXPECT(!Device()->TopKScores(half_logits.Span().data(), ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16, rows, vocab, 65,
+  // k beyond 64 (an MTP / speculative caller with top_k 100, src/mtp_generator.cpp:386-397) stays on the device
+  {
+    constexpr int k2 = 100;
+    std::vector<int32_t> tokens2(rows * k2);
+    std::vector<float> scores2(rows * k2);
+    EXPECT(Device()->TopKScores(half_logits.Span().data(), ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16, rows, vocab, k2,
+                                tokens2.data(), scores2.data()));
+    for (int r = 0; r < rows; ++r) {
+      std::vector<int32_t> order(vocab);
+      std::iota(order.begin(), order.end(), 0);
+      const float* row = widened.data() + r * vocab;
+      std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return row[a] > row[b]; });
+      for (int j = 0; j < k2; ++j) {
+        EXPECT_EQ(tokens2[r * k2 + j], order[j]);
+        EXPECT_EQ(scores2[r * k2 + j], row[order[j]]);
+      }
+    }
+  }
+  EXPECT(!Device()->TopKScores(half_logits.Span().data(), ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16, rows, vocab, vocab + 1,
                                top_tokens.data(), top_scores.data()));
   // DeviceInterface::Cast: fp16 -> fp32 on the device equals the host-side widening used above
   auto widened_dev = Device()->Allocate<float>(values.size());

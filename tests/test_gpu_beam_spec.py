@@ -39,6 +39,45 @@ def test_topk_scores(ctx, orc, rows, vocab, k, dtype):
         assert np.array_equal(sc[r], xf[r][order])
 
 
+@pytest.mark.parametrize("rows", [1, 4, 32])
+@pytest.mark.parametrize("vocab", [200, 2000, 20000, 200000])
+def test_topk_scores_on_the_reference_grid(ctx, orc, rows, vocab):
+    """The parity grid of the reference's own top-k tests (test/cuda/cuda_topk_tests.cpp:199-201: batch 1 / 4 / 32,
+    vocabulary 200 ... 200000, k up to 256), extended past the large-k route's limit: every k goes through the one
+    entry point (up to 64: the fused kernel, up to 2048: the candidate lists, beyond: the whole-row sort) and must
+    give the ids and raw scores of a stable sort by (score descending, id ascending)."""
+    say("topk_scores grid", rows, vocab)
+    rng = np.random.default_rng(rows * 7 + vocab)
+    x = (rng.standard_normal((rows, vocab)) * 2).astype(np.float32)
+    x[0, : min(vocab, 300)] = np.round(x[0, : min(vocab, 300)])  # ties among the best
+    xd = torch.from_numpy(x).cuda()
+    order = [np.lexsort((np.arange(vocab), -x[r].astype(np.float64))) for r in range(rows)]
+    ks = [1, 2, 5, 8, 16, 50, 64, 65, 100, 128, 200, 256, 512, 1000, 2048, 2049, 3000]
+    for k in [k for k in ks if k <= vocab]:
+        tok, sc = ctx.topk_scores(xd, k)
+        tok, sc = tok.cpu().numpy(), sc.cpu().numpy()
+        for r in range(rows):
+            assert np.array_equal(tok[r], order[r][:k]), (k, r)
+            assert np.array_equal(bits(sc[r]), bits(x[r][order[r][:k]])), (k, r)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_topk_scores_large_k_of_sixteen_bit_rows(ctx, orc, dtype):
+    """k beyond 64 on fp16 / bf16 rows read as they are: long runs of equal values, ids in ascending order inside a run."""
+    say("topk_scores large k", dtype)
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(3, 70001, generator=g) * 2).to(dtype)
+    wide = x.float().numpy()
+    xd = x.cuda()
+    for k in (100, 700, 2048):
+        tok, sc = ctx.topk_scores(xd, k)
+        tok, sc = tok.cpu().numpy(), sc.cpu().numpy()
+        for r in range(3):
+            order = np.lexsort((np.arange(wide.shape[1]), -wide[r].astype(np.float64)))[:k]
+            assert np.array_equal(tok[r], order), (k, r)
+            assert np.array_equal(bits(sc[r]), bits(wide[r][order])), (k, r)
+
+
 @pytest.mark.parametrize("rows,vocab,t", [(4, 1000, 1.0), (3, 151936, 1.0), (2, 32064, 0.7), (2, 7, 2.0)])
 def test_softmax_bit_exact(ctx, orc, rows, vocab, t):
     say("softmax", rows, vocab, t)
