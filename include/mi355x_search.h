@@ -162,7 +162,12 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
  *   uniforms          device [rows] doubles in [0,1): row r's categorical draw, the value
  *                     std::discrete_distribution would take from generate_canonical<double,53>.
  *                     A row whose kept set has one token ignores its uniform.
- *   out_tokens        device [rows] int32.
+ *   out_tokens        device [rows] int32 -- or pinned host memory the device can address (hipHostMalloc): the
+ *                     kernel stores every row's token there itself, as the reference mirrors its results through
+ *                     pinned memory (src/cuda/interface.cpp:51-60), so no copy follows the launch; a host that
+ *                     filled the buffer with -1 sees the tokens arrive without synchronising the stream.  The
+ *                     same holds for the out_tokens of mi355x_argmax and for next_tokens / done of
+ *                     mi355x_greedy_tail.
  *   kept_count/kept_ids/kept_probs  optional device outputs [rows], [rows,kept_capacity] x2: the
  *                     kept distribution (ids best first, renormalised fp32 probabilities), truncated
  *                     to kept_capacity entries per row; kept_count holds the untruncated size.

@@ -343,10 +343,12 @@ def _spec_verify_sparse(self, target, draft, proposal, accept_u, sample_u, mode=
     return acc, tok, used
 
 
-def _greedy_tail(self, next_tokens, eos_seen, eos_ids, pad, sequences, current_length, done):
-    """EOS padding / marking, append at column current_length, all-rows-finished flag; all in place."""
+def _greedy_tail(self, next_tokens, eos_seen, eos_ids, pad, sequences, current_length, done, allow_host=False):
+    """EOS padding / marking, append at column current_length, all-rows-finished flag; all in place.
+    allow_host: next_tokens and done may be pinned host tensors, which the kernel reads and writes in place."""
     for t in (next_tokens, eos_seen, sequences, done):
-        assert t.is_cuda and t.is_contiguous() and t.dtype == torch.int32
+        assert t.is_contiguous() and t.dtype == torch.int32
+        assert t.is_cuda or (allow_host and t.is_pinned())
     eos = (C.c_int32 * max(len(eos_ids), 1))(*eos_ids)
     self._check(self.L.mi355x_greedy_tail(self.h, _stream(), next_tokens.data_ptr(), eos_seen.data_ptr(),
                                           next_tokens.numel(), eos, len(eos_ids), pad, sequences.data_ptr(),

@@ -284,6 +284,48 @@ def test_token_only_calls_on_the_edges_of_their_guard_bands(ctx, orc, vocab, k, 
             assert np.array_equal(tokens_only(ctx, x, u, k, mass, t), orc.sample_batch(x, k, mass, t, u)), (j, mass)
 
 
+def test_results_written_straight_to_pinned_host_memory(ctx, orc):
+    """The output pointers may name pinned host memory that the device can address (the reference mirrors its
+    results through pinned memory, src/cuda/interface.cpp:51-60): the kernels store the tokens there themselves, no
+    copy follows, and a host that has filled the buffer with -1 sees a step's tokens arrive without synchronising the
+    stream.  Sampling, argmax and the EOS / append tail."""
+    import time
+    say("pinned outputs")
+    rng = np.random.default_rng(404)
+    rows, vocab = 64, 128256
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    u = rng.random(rows)
+    xd, ud = torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda()
+    torch.cuda.synchronize()
+    out = torch.full((rows,), -1, dtype=torch.int32).pin_memory()
+    view = out.numpy()
+
+    def wait_for_tokens():
+        t0 = time.perf_counter()
+        while (view < 0).any():
+            assert time.perf_counter() - t0 < 10.0, "tokens never arrived in pinned memory"
+
+    ctx.sample(xd, ud, k=50, p=0.9, temperature=0.7, out=out)
+    wait_for_tokens()  # no synchronisation: the kernel's own stores are what the host sees
+    assert np.array_equal(view, orc.sample_batch(x, 50, 0.9, 0.7, u))
+    torch.cuda.synchronize()
+    view[:] = -1
+    ctx.argmax(xd, out=out)
+    wait_for_tokens()
+    assert np.array_equal(view, orc.argmax_batch(x))
+    torch.cuda.synchronize()
+    # the tail of a greedy step with its tokens and its all-finished flag in pinned memory
+    eos, pad, max_len, cur = [7, 9], 0, 8, 3
+    tokens = torch.tensor([5, 7, 9, 11], dtype=torch.int32).pin_memory()
+    done = torch.zeros(1, dtype=torch.int32).pin_memory()
+    seen = torch.tensor([0, 0, 1, 1], dtype=torch.int32).cuda()
+    seqs = torch.zeros((4, max_len), dtype=torch.int32).cuda()
+    pkg().SearchContext.greedy_tail(ctx, tokens, seen, eos, pad, seqs, cur, done, allow_host=True)
+    torch.cuda.synchronize()
+    assert tokens.tolist() == [5, 7, pad, pad] and seen.cpu().tolist() == [0, 1, 1, 1] and done.item() == 0
+    assert seqs[:, cur].cpu().tolist() == [5, 7, pad, pad]
+
+
 def test_config2_topk_topp_batch64(ctx, orc):
     """Benchmark configuration 2 at full size: batch 64, vocab 128256, N(0,3^2) logits + 8 peaks/row at +10,
     T=0.7, k=50, p=0.9, shared uniforms; 4 of the 128 steps."""
