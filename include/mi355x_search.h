@@ -9,10 +9,18 @@
  *
  * Graph capture: every entry point only launches kernels on `stream`, with workspace from the context, and
  * can be captured into a HIP graph -- except the synchronous ones (create / destroy, *_is_done,
- * *_hypothesis, *_fallback_rows, *_wait_gave_up, beam_scorer_set_prompt) and the three that copy a caller's
- * HOST array with an asynchronous copy (mi355x_sample* with per-row parameters for more than 64 rows,
- * mi355x_logits_handoff with token_index, mi355x_kv_gather): those return MI355X_E_UNSUPPORTED on a
- * capturing stream instead of recording a node that would read the caller's array at every replay.
+ * *_hypothesis, *_fallback_rows, *_wait_gave_up, beam_scorer_set_prompt) and the two that advance a scorer's
+ * host-side state (mi355x_beam_scorer_step, mi355x_beam_search_step: the sequence length and the buffer the
+ * sequences live in are part of the launch, so a replay would repeat one step; they return
+ * MI355X_E_UNSUPPORTED on a capturing stream).  The three calls that take a table from a caller's HOST array
+ * (mi355x_sample* with per-row parameters for more than 64 rows, mi355x_logits_handoff with token_index,
+ * mi355x_kv_gather) copy it into pinned memory of the context when they are called and record a copy from
+ * there, so the caller's array is not read again at a replay; every such call captured takes one of the
+ * context's 56 permanent staging slots (MI355X_E_UNSUPPORTED once they are used up).
+ *
+ * Versions: MI355X_ABI_VERSION names the layout of the structures below and the set of entry points;
+ * mi355x_search_abi_version() returns the value the loaded library was built with, so a caller built
+ * against another header can tell before it passes a structure.
  *
  * Tie rule everywhere: equal scores are ordered by ascending index (lowest index wins).
  * -0.0 and +0.0 compare equal.  NaN scores order below every number, except in mi355x_argmax, which
@@ -35,6 +43,9 @@ extern "C" {
 #define MI355X_E_UNSUPPORTED (-4) /* valid request this build does not implement */
 
 #define MI355X_MAX_EOS 16
+
+#define MI355X_ABI_VERSION 3
+int mi355x_search_abi_version(void);
 
 /* Element type of a logits / KV tensor (values follow ONNXTensorElementDataType where one exists:
  * FLOAT = 1, FLOAT16 = 10, the types DeviceInterface::ArgMax/TopKScores accept, src/smartptrs.h:249). */
@@ -136,7 +147,8 @@ int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int 
  * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
  * threads) race; calls on one stream, or otherwise ordered, are safe.  The call itself clears the slots
  * it is about to use (with a kernel, no memset node) and calls neither hipMalloc nor hipFree.
- * The array's address is looked up once per device, by mi355x_search_create or by the first call. */
+ * The array's address is looked up once per device, by mi355x_search_create or by the first call; a first call
+ * on a stream that records a graph is refused (MI355X_E_UNSUPPORTED), later ones can be captured. */
 #define MI355X_ARGMAX_STATIC_MAX_ROWS 4096
 int mi355x_argmax_static(void* stream, const void* logits, int dtype, int64_t row_stride, int rows,
                          int vocab, const mi355x_logits_xform* xf, int32_t* out_tokens);
@@ -156,9 +168,8 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
  * (src/smartptrs.h:134-137).
  *   params            used for every row when per_row_params is NULL.
  *   per_row_params    HOST [rows], heterogeneous parameters (copied by the call: up to 64 rows travel
- *                     inside the kernel arguments, larger batches through one asynchronous copy to a
- *                     table in the context -- that copy reads the caller's array, so such a call fails
- *                     with MI355X_E_UNSUPPORTED on a stream that is being captured into a graph).
+ *                     inside the kernel arguments, larger batches through pinned staging memory of the
+ *                     context and one asynchronous copy to a table in it).
  *   uniforms          device [rows] doubles in [0,1): row r's categorical draw, the value
  *                     std::discrete_distribution would take from generate_canonical<double,53>.
  *                     A row whose kept set has one token ignores its uniform.
@@ -255,8 +266,8 @@ int mi355x_beam_scorer_hypothesis(mi355x_beam_scorer* s, void* stream, int batch
  * for every tensor t and row j, past[t][j] = present[t][beam_indices[j]], blocks of block_bytes
  * bytes (any size; blocks and tensors aligned to 16 bytes move with 128-bit accesses, others with the
  * widest access they are aligned to).  present/past: HOST arrays of n_tensors device pointers (copied by the
- * call with asynchronous copies that read the caller's arrays: on a stream that is being captured into a
- * graph the call fails with MI355X_E_UNSUPPORTED); beam_indices: device [rows]. */
+ * call into pinned staging memory of the context, from where one asynchronous copy takes them to the device);
+ * beam_indices: device [rows]. */
 int mi355x_kv_gather(mi355x_search_ctx* ctx, void* stream, const void* const* present,
                      void* const* past, int n_tensors, const int32_t* beam_indices, int rows,
                      size_t block_bytes);
@@ -314,7 +325,8 @@ int mi355x_spec_verify_sparse(mi355x_search_ctx* ctx, void* stream, const int32_
  * uniform_pool[number of consuming rows before r] from the kept set mi355x_sample left on the device
  * (kept_count [rows], kept_ids / kept_probs [rows, kept_capacity], kept_capacity >= every count), and
  * *draws_used (device int32, may be null) tells the caller how many doubles to discard from the real engine
- * (two mt19937 outputs each).  skip_rows: device [rows] int32, non-zero = finished row (consumes nothing; its
+ * (two mt19937 outputs each); it is -1 when some kept_count exceeds kept_capacity (a row would then draw from a
+ * truncated set: the tokens of such a call must not be used).  skip_rows: device [rows] int32, non-zero = finished row (consumes nothing; its
  * token is its best id), or null.  out_tokens device [rows]. */
 int mi355x_draw_in_order(mi355x_search_ctx* ctx, void* stream, const int32_t* kept_count,
                          const int32_t* kept_ids, const float* kept_probs, int kept_capacity, int rows,
@@ -346,8 +358,8 @@ int mi355x_cast(mi355x_search_ctx* ctx, void* stream, const void* in, int in_dty
 /* Logits hand-off before the path: Logits::Get (src/models/logits.cpp:33-82) copies the logits of each
  * row's last real token out of the model's [rows, seq_len, vocab] output and widens fp16/bf16 to fp32;
  * here both happen in one pass.  raw: device, dtype MI355X_F32 / MI355X_F16 / MI355X_BF16;
- * token_index: HOST [rows] positions inside seq_len (copied by the call; with it the call cannot be captured
- * into a graph and fails with MI355X_E_UNSUPPORTED on a capturing stream), or NULL for seq_len - 1;
+ * token_index: HOST [rows] positions inside seq_len (copied by the call, through pinned staging memory of the
+ * context), or NULL for seq_len - 1;
  * out: device [rows] rows of vocab floats, row r at out + r*out_stride. */
 int mi355x_logits_handoff(mi355x_search_ctx* ctx, void* stream, const void* raw, int dtype, int rows,
                           int seq_len, int vocab, const int32_t* token_index, float* out,

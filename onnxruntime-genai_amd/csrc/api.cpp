@@ -82,6 +82,17 @@ struct mi355x_search_ctx {
   float* row_sum{};
   int32_t* row_index{};  // device copy of per-row host indices (logits hand-off)
   int32_t* beam_row_tokens{};
+  // Pinned host staging for the calls that take a table from a caller's HOST array (per-row parameters of more
+  // than 64 rows, the KV gather's pointer tables, token_index): the call copies the array into a slot here and
+  // records a copy from the slot to the device table.  Slots of the ring are reused once the copy that read them
+  // is done (an event per slot); a call on a capturing stream gets a slot of its own that is never reused, so the
+  // copy node of its graph reads the same bytes at every replay.
+  static constexpr int kStageRing = 8, kStageCaptured = 56;
+  char* stage{};
+  size_t stage_slot_bytes{};
+  hipEvent_t stage_event[kStageRing]{};
+  bool stage_pending[kStageRing]{};
+  int stage_next{}, stage_captured{};
 
   template <typename T>
   hipError_t Alloc(T** p, size_t count, bool zero) {
@@ -215,6 +226,15 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->row_index, static_cast<size_t>(max_rows), false));
   c->ptr_table_cap = 4096;
   ok(c->Alloc(&c->ptr_table, c->ptr_table_cap, false));
+  c->stage_slot_bytes = std::max(c->ptr_table_cap * sizeof(void*), static_cast<size_t>(max_rows) * sizeof(mi355x_sample_params));
+  c->stage_slot_bytes = (c->stage_slot_bytes + 255) & ~static_cast<size_t>(255);
+  if (e == hipSuccess) {
+    void* pinned = nullptr;
+    e = hipHostMalloc(&pinned, c->stage_slot_bytes * (mi355x_search_ctx::kStageRing + mi355x_search_ctx::kStageCaptured), hipHostMallocDefault);
+    c->stage = static_cast<char*>(pinned);
+  }
+  for (int i = 0; i < mi355x_search_ctx::kStageRing && e == hipSuccess; ++i)
+    e = hipEventCreateWithFlags(&c->stage_event[i], hipEventDisableTiming);
   if (e == hipSuccess) e = ms_sample_init();
   if (e == hipSuccess) e = ms_static_scratch_setup();  // set-up of mi355x_argmax_static on this device
   // the fills above ran on the null stream: done before a caller's stream, which need not wait for it, uses them
@@ -231,10 +251,15 @@ void mi355x_search_destroy(mi355x_search_ctx* ctx) {
   if (!ctx) return;
   (void)hipSetDevice(ctx->device);
   for (void* p : ctx->allocs) (void)hipFree(p);
+  for (hipEvent_t ev : ctx->stage_event)
+    if (ev) (void)hipEventDestroy(ev);
+  if (ctx->stage) (void)hipHostFree(ctx->stage);
   delete ctx;
 }
 
 size_t mi355x_search_workspace_bytes(const mi355x_search_ctx* ctx) { return ctx ? ctx->bytes : 0; }
+
+int mi355x_search_abi_version(void) { return MI355X_ABI_VERSION; }
 
 int mi355x_process_logits(mi355x_search_ctx* ctx, void* stream, float* logits, int64_t row_stride, int rows,
                           int vocab, const mi355x_logits_xform* xf) {
@@ -313,6 +338,32 @@ bool Capturing(hipStream_t s) {
   return hipStreamIsCapturing(s, &status) == hipSuccess && status != hipStreamCaptureStatusNone;
 }
 
+// Records a copy of `bytes` bytes of the caller's host array `src` to the device table `dst` on stream s, through a
+// pinned staging slot of the context (see mi355x_search_ctx::stage).
+int StageToDevice(mi355x_search_ctx* ctx, hipStream_t s, void* dst, const void* src, size_t bytes) {
+  if (bytes > ctx->stage_slot_bytes) return Fail(MI355X_E_CAPACITY, "a host table of %zu bytes exceeds the staging slot", bytes);
+  const bool capturing = Capturing(s);
+  int slot;
+  if (capturing) {
+    if (ctx->stage_captured == mi355x_search_ctx::kStageCaptured)
+      return Fail(MI355X_E_UNSUPPORTED, "this context has staged %d host tables for graph capture, all it provides for",
+                  mi355x_search_ctx::kStageCaptured);
+    slot = mi355x_search_ctx::kStageRing + ctx->stage_captured++;
+  } else {
+    slot = ctx->stage_next;
+    ctx->stage_next = (slot + 1) % mi355x_search_ctx::kStageRing;
+    if (ctx->stage_pending[slot]) HIP_TRY(hipEventSynchronize(ctx->stage_event[slot]));
+  }
+  char* pinned = ctx->stage + static_cast<size_t>(slot) * ctx->stage_slot_bytes;
+  std::memcpy(pinned, src, bytes);
+  HIP_TRY(hipMemcpyAsync(dst, pinned, bytes, hipMemcpyHostToDevice, s));
+  if (!capturing) {
+    HIP_TRY(hipEventRecord(ctx->stage_event[slot], s));
+    ctx->stage_pending[slot] = true;
+  }
+  return MI355X_OK;
+}
+
 // One launch set of the sampling path.  Rows lie row_stride elements apart from `logits`, or -- row_ptrs not
 // null, at most kInlineParamRows rows -- start at the device pointers row_ptrs[0 .. rows).
 int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const void* const* row_ptrs, int dtype,
@@ -351,12 +402,7 @@ int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const 
     }
     use_table = true;
   } else if (per_row_params) {
-    if (Capturing(s))
-      return Fail(MI355X_E_UNSUPPORTED, "more than %d rows with per-row parameters are copied from the caller's host "
-                  "array and cannot be captured into a graph; call with at most %d rows", ms::kInlineParamRows,
-                  ms::kInlineParamRows);
-    HIP_TRY(hipMemcpyAsync(ctx->params_dev, per_row_params, sizeof(mi355x_sample_params) * rows,
-                           hipMemcpyHostToDevice, s));
+    if (int rc = StageToDevice(ctx, s, ctx->params_dev, per_row_params, sizeof(mi355x_sample_params) * rows)) return rc;
     a.per_row = ctx->params_dev;
   }
   a.logits = row_ptrs ? row_ptrs[0] : logits;
@@ -693,9 +739,7 @@ int mi355x_logits_handoff(mi355x_search_ctx* ctx, void* stream, const void* raw,
     for (int r = 0; r < rows; ++r)
       if (token_index[r] < 0 || token_index[r] >= seq_len)
         return Fail(MI355X_E_INVALID, "token_index[%d] = %d outside [0, %d)", r, token_index[r], seq_len);
-    if (Capturing(s))
-      return Fail(MI355X_E_UNSUPPORTED, "token_index is copied from the caller's host array: not capturable into a graph");
-    HIP_TRY(hipMemcpyAsync(ctx->row_index, token_index, sizeof(int32_t) * rows, hipMemcpyHostToDevice, s));
+    if (int rc = StageToDevice(ctx, s, ctx->row_index, token_index, sizeof(int32_t) * rows)) return rc;
     index_dev = ctx->row_index;
   }
   HIP_TRY(ms_launch_logits_handoff(raw, kind, rows, seq_len, vocab, index_dev, out, out_stride, s));
@@ -717,10 +761,12 @@ int mi355x_kv_gather(mi355x_search_ctx* ctx, void* stream, const void* const* pr
   int width = 16;
   while (align & static_cast<uintptr_t>(width - 1)) width >>= 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (Capturing(s))
-    return Fail(MI355X_E_UNSUPPORTED, "the tensor pointer tables are copied from the caller's host arrays: not capturable into a graph");
-  HIP_TRY(hipMemcpyAsync(ctx->ptr_table, present, sizeof(void*) * n_tensors, hipMemcpyHostToDevice, s));
-  HIP_TRY(hipMemcpyAsync(ctx->ptr_table + n_tensors, past, sizeof(void*) * n_tensors, hipMemcpyHostToDevice, s));
+  {
+    std::vector<const void*> both(static_cast<size_t>(n_tensors) * 2);  // one table: present pointers, then past pointers
+    std::copy_n(present, n_tensors, both.begin());
+    std::copy_n(past, n_tensors, both.begin() + n_tensors);
+    if (int rc = StageToDevice(ctx, s, ctx->ptr_table, both.data(), sizeof(void*) * both.size())) return rc;
+  }
   HIP_TRY(ms_launch_kv_gather(ctx->ptr_table, ctx->ptr_table + n_tensors, n_tensors, beam_indices, rows, block_bytes, width, s));
   return MI355X_OK;
 }
@@ -882,6 +928,8 @@ int mi355x_beam_scorer_step(mi355x_beam_scorer* s, void* stream, const float* ca
   if (!s || !cand_scores || !cand_tokens || !cand_beam_indices) return Fail(MI355X_E_INVALID, "null argument");
   if (s->length >= s->st.max_length) return Fail(MI355X_E_INVALID, "sequence already at max_length (%d)", s->st.max_length);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (Capturing(st))
+    return Fail(MI355X_E_UNSUPPORTED, "a scorer step carries the sequence length and buffer of this very step: a graph replay would repeat it");
   HIP_TRY(ms_launch_scorer_step(&s->st, s->seq[s->cur], s->seq[1 - s->cur], s->length, cand_scores, cand_tokens,
                                 cand_beam_indices, st));
   s->cur = 1 - s->cur;
@@ -893,6 +941,8 @@ int mi355x_beam_search_step(mi355x_beam_scorer* s, void* stream, const void* log
                             int vocab) {
   if (!s) return Fail(MI355X_E_INVALID, "null argument");
   if (s->length >= s->st.max_length) return Fail(MI355X_E_INVALID, "sequence already at max_length (%d)", s->st.max_length);
+  if (Capturing(static_cast<hipStream_t>(stream)))
+    return Fail(MI355X_E_UNSUPPORTED, "a search step carries the sequence length and buffer of this very step: a graph replay would repeat it");
   ms::ScorerStep step{s->st, s->seq[s->cur], s->seq[1 - s->cur], s->length};
   bool fused = false;
   if (int r = BeamSelectImpl(s->ctx, stream, logits, dtype, row_stride, s->st.batch, s->st.beams, vocab, s->st.next_scores,

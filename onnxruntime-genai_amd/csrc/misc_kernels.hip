@@ -57,21 +57,29 @@ __global__ __launch_bounds__(256) void draw_in_order_kernel(const int32_t* kept_
   __shared__ SeqShared sh;
   __shared__ int red_before[4], red_total[4];
   const int row = blockIdx.x, tid = threadIdx.x;
-  int before = 0, total = 0;
+  // A row consumes a draw when the kept set it is given holds two tokens or more: the count as this kernel uses
+  // it, cut to the capacity of the lists.  A count beyond the capacity breaks the caller's contract (the row
+  // would draw from a truncated set): *draws_used then reports -1 instead of a number of draws.
+  int before = 0, total = 0, broken = 0;
   for (int r = tid; r < rows; r += 256) {
-    const int c = (!(skip && skip[r] != 0) && kept_count[r] >= 2) ? 1 : 0;
+    const int listed = kept_count[r] < cap ? kept_count[r] : cap;
+    const int c = (!(skip && skip[r] != 0) && listed >= 2) ? 1 : 0;
+    broken |= kept_count[r] > cap ? 1 : 0;
     total += c;
     before += r < row ? c : 0;
   }
   before = wave_sum<int>(before);
   total = wave_sum<int>(total);
+  broken = wave_sum<int>(broken);
   if ((tid & 63) == 0) {
     red_before[tid >> 6] = before;
-    red_total[tid >> 6] = total;
+    red_total[tid >> 6] = broken != 0 ? -1 : total;
   }
   __syncthreads();
   before = (red_before[0] + red_before[1]) + (red_before[2] + red_before[3]);
-  total = (red_total[0] + red_total[1]) + (red_total[2] + red_total[3]);
+  total = (red_total[0] < 0 || red_total[1] < 0 || red_total[2] < 0 || red_total[3] < 0)
+              ? -1
+              : (red_total[0] + red_total[1]) + (red_total[2] + red_total[3]);
   int n = kept_count[row];
   n = n < cap ? n : cap;
   const bool consumes = !(skip && skip[row] != 0) && n >= 2;

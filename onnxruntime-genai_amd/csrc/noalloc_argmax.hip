@@ -25,13 +25,16 @@ int FailHere(int code, const char* fmt, ...) {
   return code;
 }
 
-hipError_t ScratchOfCurrentDevice(void** out) {
+// The array's address on the calling thread's current device; looked up on first use unless `lookup_allowed` is
+// false (then an unknown address reports hipErrorNotReady).
+hipError_t ScratchOfCurrentDevice(void** out, bool lookup_allowed = true) {
   int device = 0;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return e;
   if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
   std::lock_guard<std::mutex> lock(g_mu);
   if (!g_scratch_ptr[device]) {
+    if (!lookup_allowed) return hipErrorNotReady;
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return e;
@@ -67,10 +70,22 @@ extern "C" int mi355x_argmax_static(void* stream, const void* logits, int dtype,
     return FailHere(MI355X_E_UNSUPPORTED, "dtype %d not supported", dtype);
   if (row_stride < vocab) return FailHere(MI355X_E_INVALID, "row_stride smaller than vocab");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // every GPU has its own copy of the array: the stream must belong to the device whose copy is used
+  int current = 0, of_stream = 0;
+  if (s != nullptr && hipGetDevice(&current) == hipSuccess && hipStreamGetDevice(s, &of_stream) == hipSuccess &&
+      of_stream != current)
+    return FailHere(MI355X_E_INVALID, "the stream belongs to device %d, the calling thread's current device is %d", of_stream,
+                    current);
   ms::ArgmaxArgs a{};
   if (int r = ms_make_xform(nullptr, xf, rows, vocab, s, &a.xf)) return r;
+  // the first use on a device looks the array's address up, which is no work for a stream that records a graph
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  const bool capturing = hipStreamIsCapturing(s, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone;
   void* base = nullptr;
-  hipError_t e = ScratchOfCurrentDevice(&base);
+  hipError_t e = ScratchOfCurrentDevice(&base, !capturing);
+  if (e == hipErrorNotReady)
+    return FailHere(MI355X_E_UNSUPPORTED, "the first call on a device cannot be captured into a graph: call once outside "
+                    "the capture (or create a context on the device) first");
   if (e != hipSuccess) return FailHere(MI355X_E_HIP, "static scratch lookup failed: %s", hipGetErrorString(e));
   a.logits = logits;
   a.row_stride = row_stride;

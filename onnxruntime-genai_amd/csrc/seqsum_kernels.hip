@@ -36,7 +36,13 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_max_kernel(const SeqSumArgs 
 #pragma unroll
   for (int e = 0; e < kSegPer; ++e) fm = fmaxf(fm, v[e]);
   const uint32_t m = block_max<uint32_t>(order_key(fm), red);
-  if (threadIdx.x == 0) a.seg_max[static_cast<size_t>(row) * a.segs + seg] = m;
+  if (threadIdx.x == 0) {
+    a.seg_max[static_cast<size_t>(row) * a.segs + seg] = m;
+    // This launch comes first in every sequence: it marks the segment's sum as not written, so that the look-back
+    // of the next launch never takes a sum left by an earlier call for this one's (the walk puts the mark back too,
+    // but a sequence that was cut short after its second launch would otherwise leave finite sums behind).
+    store_sum_bits(a.seg_sum + static_cast<size_t>(row) * a.segs + seg, kSumNotReady);
+  }
 }
 
 // ---- the walk: one wave per row walks, fifteen more prepare its way ------------------------------------

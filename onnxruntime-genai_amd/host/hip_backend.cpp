@@ -534,6 +534,7 @@ void GreedySearch_Hip::Sample(int k, float p, float temperature, std::mt19937& r
   LaunchTail(next_tokens_.Span().data());
   HIP_CHECK(hipMemcpyAsync(draws_used_.CpuSpan().data(), draws_used_.Span().data(), sizeof(int32_t), hipMemcpyDeviceToHost, g_stream));
   FinishStep();  // synchronises
+  if (draws_used_.CpuSpan()[0] < 0) throw std::runtime_error("a row's kept set outgrew the lists it was sampled from");
   // the engine ends where std::discrete_distribution would have left it: two outputs per consumed double
   rng.discard(2ull * static_cast<unsigned long long>(draws_used_.CpuSpan()[0]));
 }

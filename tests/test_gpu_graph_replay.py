@@ -67,3 +67,84 @@ def test_graph_replays_match_eager_calls(orc):
         for name in eager:
             assert torch.equal(again[name].view(torch.int32), eager[name].view(torch.int32)), (replay, name, "eager")
     ctx.close()
+
+
+def test_host_tables_are_staged_for_graph_capture(orc):
+    """Calls that take a table from a host array -- per-row parameters of more than 64 rows, the KV gather's pointer
+    tables -- copy it into pinned memory of the context when they are called, so their graph nodes do not read the
+    caller's array again: a 96-row heterogeneous batch and a KV gather captured into one graph, the host arrays
+    overwritten afterwards, four replays with eager calls between them."""
+    say("graph replay of staged host tables")
+    rows, vocab = 96, 50000
+    ctx = pkg().SearchContext(rows, vocab)
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn(rows, vocab, generator=g, device="cuda") * 3
+    u = torch.rand(rows, generator=g, device="cuda", dtype=torch.float64)
+    rng = np.random.default_rng(3)
+    params = [(int(rng.choice([0, 1, 5, 50, 64, 100])), float(rng.choice([0.0, 0.5, 0.9, 1.0])), float(rng.choice([0.7, 1.0, 1.5])))
+              for _ in range(rows)]
+    layers = [torch.randint(-30000, 30000, (8, 2, 16, 64), generator=g, device="cuda", dtype=torch.int16) for _ in range(6)]
+    past = [torch.zeros_like(t) for t in layers]
+    beam_idx = torch.tensor([3, 3, 0, 1, 7, 6, 6, 2], dtype=torch.int32, device="cuda")
+    xh, uh = x.cpu().numpy(), u.cpu().numpy()
+    want = np.array([orc.sample_row(xh[r], *params[r], uh[r]) for r in range(rows)], np.int32)
+    eager = ctx.sample(x, u, per_row=params)
+    torch.cuda.synchronize()
+    assert np.array_equal(eager.cpu().numpy(), want)
+
+    out = torch.zeros(rows, dtype=torch.int32, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            ctx.sample(x, u, per_row=params, out=out)
+            ctx.kv_gather(layers, past, beam_idx)
+    torch.cuda.synchronize()
+    for replay in range(4):
+        out.zero_()
+        for t in past:
+            t.zero_()
+        with torch.cuda.stream(side):
+            graph.replay()
+        side.synchronize()
+        assert np.array_equal(out.cpu().numpy(), want), replay
+        for t, src in zip(past, layers):
+            assert torch.equal(t, src[beam_idx.long()]), replay
+        # eager calls with other tables between the replays: they use other staging slots
+        other = [(50, 0.9, 0.7)] * rows
+        got = ctx.sample(x, u, per_row=other)
+        ctx.kv_gather(layers[:3], past[:3], torch.flip(beam_idx, [0]))
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy(), orc.sample_batch(xh, 50, 0.9, 0.7, uh)), replay
+    ctx.close()
+
+
+def test_scorer_steps_refuse_a_capturing_stream():
+    """The scorer's steps carry host-side state (sequence length, which of two buffers holds the sequences):
+    recording one into a graph would replay the same step, so they decline on a capturing stream."""
+    say("scorer step under capture")
+    batch, beams, vocab = 2, 2, 5000
+    ctx = pkg().SearchContext(batch * beams, vocab)
+    scorer = pkg().BeamScorer(ctx, batch, beams, 16, 0, [vocab - 1], 1.0, True)
+    scorer.set_prompt(np.zeros((batch, 2), np.int32))
+    x = torch.randn(batch * beams, vocab, device="cuda")
+    scorer.search_step(x)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    refused = False
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            try:
+                scorer.search_step(x)
+            except RuntimeError as e:
+                refused = "replay" in str(e)
+            ctx.argmax(x)  # the capture itself stays usable
+    torch.cuda.synchronize()
+    assert refused
+    scorer.search_step(x)  # and the scorer carries on eagerly
+    torch.cuda.synchronize()
+    scorer.close()
+    ctx.close()

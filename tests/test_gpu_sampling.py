@@ -996,8 +996,6 @@ def exact_path_rows(name, rng, vocab):
 def test_exact_path_orders_whole_rows(ctx, orc, name, vocab):
     """k above the candidate-list bound and sampling from the whole vocabulary (k = 0, p = 1) take the exact
     path, which sorts the entire row; the kept ids are that order, checked to the last element."""
-    if vocab > 70001 and name in ("constant", "peaked"):
-        pytest.skip("covered at the smaller sizes")
     say("exact path", name, vocab)
     rng = np.random.default_rng(vocab + len(name))
     x = exact_path_rows(name, rng, vocab)
@@ -1055,3 +1053,9 @@ def test_draw_in_order_follows_one_engine(ctx, orc, rows, cap):
             assert tok[r] == ids[r, orc.discrete_draw(probs[r, :counts[r]], pool[d])], (r, d)
             d += 1
         assert used.item() == d
+    # a kept-set size beyond the capacity of the lists breaks the contract: the call says so instead of counting
+    broken = counts.copy()
+    broken[rows // 2] = cap + 3
+    _, used = ctx.draw_in_order(torch.from_numpy(broken).cuda(), torch.from_numpy(ids).cuda(),
+                                torch.from_numpy(probs).cuda(), torch.from_numpy(pool).cuda(), None)
+    assert used.item() == -1

@@ -198,10 +198,12 @@ def test_rows_scattered_over_memory(ctx, orc, dtype):
         assert ctx.sample(row_list, u, per_row=per_row).cpu().tolist() == want
 
 
-def test_calls_that_copy_host_arrays_refuse_graph_capture(ctx):
-    """Per-row parameters of more than 64 rows and the KV pointer tables are copied from the caller's host arrays:
-    under stream capture those calls fail with a clear error and record nothing; the 64-row forms are captured."""
-    say("capture refusal")
+def test_captured_calls_with_host_tables_use_up_staging_slots():
+    """Per-row parameters of more than 64 rows and the KV pointer tables are copied from the caller's host arrays into
+    pinned staging memory of the context; a call captured into a graph keeps its slot for good, so a context
+    serves a bounded number of such captured calls (56) and says so when they are used up."""
+    say("staging slots under capture")
+    c = pkg().SearchContext(80, 4099)
     rows, vocab = 70, 4099
     x = torch.randn(rows, vocab, device="cuda")
     u = torch.rand(rows, device="cuda", dtype=torch.float64)
@@ -210,19 +212,26 @@ def test_calls_that_copy_host_arrays_refuse_graph_capture(ctx):
     present = [torch.randn(4, 64, device="cuda") for _ in range(2)]
     past = [torch.zeros_like(p) for p in present]
     idx = torch.tensor([1, 1, 0, 3], dtype=torch.int32, device="cuda")
-    eager = ctx.sample(x[:64], u, per_row=per_row[:64]).clone()
+    eager = c.sample(x, u, per_row=per_row).clone()
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):
-            with pytest.raises(RuntimeError, match="captured"):
-                ctx.sample(x, u, per_row=per_row, out=out)
-            with pytest.raises(RuntimeError, match="not capturable"):
-                ctx.kv_gather(present, past, idx)
-            ctx.sample(x[:64], u, per_row=per_row[:64], out=out[:64])
+            c.sample(x, u, per_row=per_row, out=out)
+            for _ in range(55):
+                c.kv_gather(present, past, idx)
+            with pytest.raises(RuntimeError, match="staged 56"):
+                c.kv_gather(present, past, idx)
         out.zero_()
         graph.replay()
         side.synchronize()
-    assert torch.equal(out[:64], eager)
+    assert torch.equal(out, eager)
+    for t, src in zip(past, present):
+        assert torch.equal(t, src[idx.long()])
+    # eager calls are not affected: they go through the ring
+    for _ in range(20):
+        c.kv_gather(present, past, idx)
+    torch.cuda.synchronize()
+    c.close()
