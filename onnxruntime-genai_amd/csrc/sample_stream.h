@@ -468,6 +468,31 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   const InT* lrow = static_cast<const InT*>(row0);
   const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
   const float kNaN = __uint_as_float(0x7fc00000u);  // marks ids >= vocab: never a maximum, never >= a bound
+  // The bitmap words and the first history ids of this thread are requested before the logits: loads come back in
+  // the order they were asked for, and the history has a chain of its own to start (mark the ids, read their logits
+  // again, penalise them) that should run while the logits arrive, not after them.
+  constexpr int kWordsPerThread = kSChunk / 32 / kSBlock;  // bitmap words a thread stages
+  static_assert(kWordsPerThread >= 1 && kSChunk / 32 == kWordsPerThread * kSBlock, "whole bitmap words per thread");
+  const bool active = XFORM && a.xf.active();  // kernels without logits processing carry none of its code
+  const bool pen = active && a.xf.use_penalty();
+  const bool has_mask = active && a.xf.mask != nullptr;
+  const int words = (V - 1) / 32 + 1;
+  const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * words : nullptr;
+  const int32_t* hist = pen ? a.xf.history + static_cast<size_t>(row) * a.xf.history_stride : nullptr;
+  const bool hist_ahead = pen && a.xf.history_lens == nullptr;  // the length is known without a load
+  int hist_pre[2] = {-1, -1};
+  uint32_t mask_pre[kWordsPerThread];
+#pragma unroll
+  for (int q = 0; q < 2; ++q)
+    if (hist_ahead && tid + q * kSBlock < a.xf.history_len) hist_pre[q] = hist[tid + q * kSBlock];
+#pragma unroll
+  for (int q = 0; q < kWordsPerThread; ++q) {
+    mask_pre[q] = ~0u;
+    if (has_mask) {
+      const int w = chunk * (kSChunk / 32) + tid + q * kSBlock;
+      mask_pre[q] = w < words ? mrow[w] : 0u;
+    }
+  }
   float v[kSElems];
   // a chunk that lies inside an aligned row requests its loads without a test between them
   const bool whole_chunk = aligned && (chunk + 1) * kSChunk <= V;
@@ -482,17 +507,39 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
         v[j * 4 + 2] = q.z;
         v[j * 4 + 3] = q.w;
       }
-    } else
+    } else if (aligned) {
+      // The row's last chunk.  Every register is set to NaN before the first load is requested and the loads that
+      // lie inside the row are requested back to back: a register written after a load into it was requested
+      // (even by other lanes) makes the compiler wait for that load first, which strings the sixteen loads of a
+      // thread out one memory round trip after the other.  The one load that straddles the row's end follows.
 #pragma unroll
-    for (int j = 0; j < kSLoads; ++j) {
-      const int i0 = elem_index<kSBlock, VEC>(chunk, j, 0);
-      if (aligned && i0 + 4 <= V) {
-        const v4f q = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(lrow + i0));
-        v[j * 4 + 0] = q.x;
-        v[j * 4 + 1] = q.y;
-        v[j * 4 + 2] = q.z;
-        v[j * 4 + 3] = q.w;
-      } else {
+      for (int e = 0; e < kSElems; ++e) asm volatile("v_mov_b32 %0, 0x7fc00000" : "=v"(v[e]));
+#pragma unroll
+      for (int j = 0; j < kSLoads; ++j) {
+        const int i0 = elem_index<kSBlock, VEC>(chunk, j, 0);
+        if (i0 + 4 <= V) {
+          const v4f q = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(lrow + i0));
+          v[j * 4 + 0] = q.x;
+          v[j * 4 + 1] = q.y;
+          v[j * 4 + 2] = q.z;
+          v[j * 4 + 3] = q.w;
+        }
+      }
+      if ((V & 3) != 0) {
+#pragma unroll
+        for (int j = 0; j < kSLoads; ++j) {
+          const int i0 = elem_index<kSBlock, VEC>(chunk, j, 0);
+          if (i0 < V && i0 + 4 > V) {
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+              if (i0 + c < V) v[j * 4 + c] = load_one<InT>(lrow, i0 + c);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kSLoads; ++j) {
+        const int i0 = elem_index<kSBlock, VEC>(chunk, j, 0);
 #pragma unroll
         for (int c = 0; c < 4; ++c) v[j * 4 + c] = (i0 + c < V) ? load_one<InT>(lrow, i0 + c) : kNaN;
       }
@@ -544,29 +591,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   // they leave the register arrays altogether: a second bitmap turns them into NaN there, and the
   // threads that marked them compute their processed values into a short list in LDS, `extras`, which
   // every later phase visits next to the registers.
-  // The bitmap words and the first history ids of this thread are requested before anything waits.
-  constexpr int kWordsPerThread = kSChunk / 32 / kSBlock;  // bitmap words a thread stages
-  static_assert(kWordsPerThread >= 1 && kSChunk / 32 == kWordsPerThread * kSBlock, "whole bitmap words per thread");
-  const bool active = XFORM && a.xf.active();  // kernels without logits processing carry none of its code
-  const bool pen = active && a.xf.use_penalty();
-  const bool has_mask = active && a.xf.mask != nullptr;
-  const int words = (V - 1) / 32 + 1;
-  const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * words : nullptr;
-  const int32_t* hist = pen ? a.xf.history + static_cast<size_t>(row) * a.xf.history_stride : nullptr;
-  const bool hist_ahead = pen && a.xf.history_lens == nullptr;  // the length is known without a load
-  int hist_pre[2] = {-1, -1};
-  uint32_t mask_pre[kWordsPerThread];
-#pragma unroll
-  for (int q = 0; q < 2; ++q)
-    if (hist_ahead && tid + q * kSBlock < a.xf.history_len) hist_pre[q] = hist[tid + q * kSBlock];
-#pragma unroll
-  for (int q = 0; q < kWordsPerThread; ++q) {
-    mask_pre[q] = ~0u;
-    if (has_mask) {
-      const int w = chunk * (kSChunk / 32) + tid + q * kSBlock;
-      mask_pre[q] = w < words ? mrow[w] : 0u;
-    }
-  }
   uint32_t n_extra = 0u;
   bool extra_overflow = false;
   if (XFORM && active) {
@@ -621,7 +645,9 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       extra_overflow = n_extra > static_cast<uint32_t>(kExtraCap);  // the row takes the exact path
       if (extra_overflow) n_extra = 0u;
     }
-    mask_registers<kSBlock, VEC, true, true>(v, sm.mask_bits, sm.hist_bits, tid);
+    // without a grammar mask and without EOS masking every id is allowed (ids past the vocabulary are NaN already)
+    if (has_mask || n_eos > 0) mask_registers<kSBlock, VEC, true, true>(v, sm.mask_bits, sm.hist_bits, tid);
+    else mask_registers<kSBlock, VEC, false, true>(v, sm.mask_bits, sm.hist_bits, tid);
   }
   // per-thread maximum in the float domain (fmaxf skips NaN), keeping the maximum of every float4
   float qm[kSVec];
@@ -799,28 +825,63 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     // same way, so the row's answer is the largest key: no bound, no lists, no sort.  Every chunk
     // publishes its best key in the first entry of its candidate slots; the workgroup of the row's last
     // chunk polls for them, as the top-k rows do for their lists.
-    uint32_t best_idx = 0xffffffffu;
-#pragma unroll
-    for (int j = kSVec - 1; j >= 0; --j) {
-      if (qm[j] == fm) {
-#pragma unroll
-        for (int c = 3; c >= 0; --c)
-          if (v[j * 4 + c] == fm) best_idx = static_cast<uint32_t>(elem_index<kSBlock, VEC>(chunk, j, c));
-      }
-    }
-    for (uint32_t i = tid; i < n_extra; i += kSBlock)
-      if (sm.extra_val[i] == fm && sm.extra_idx[i] < best_idx) best_idx = sm.extra_idx[i];
-    u64 key = best_idx != 0xffffffffu ? make_key64(order_key(fm), best_idx) : 0;
-    key = wave_max(key);
-    if (lane == 0) sm.list_hi[wave] = key;
-    lds_barrier();
+    // Two rounds: the workgroup agrees on the chunk's largest value first (a 32-bit reduction), then only the
+    // lanes that hold it look for its place -- with scalar tests of whole-wave compare masks, since hardly any
+    // lane does -- and the lowest id wins a second reduction.  (Every thread finding the place of its own
+    // maximum, as a single reduction over (value, id) keys needs, costs each wave some 150 instructions.)
+    const uint32_t cmax = block_max_lds<kSWaves, uint32_t>(lmax, sm.wave_val);
     const bool finisher = chunk == n_chunks - 1;
     if (sm.poisoned != 0u) return finisher;
+    uint32_t widx = 0xffffffffu;  // lowest id of the wave's elements that equal the chunk's maximum
+    if (cmax != 0u) {
+      const float cf = key_to_float(cmax);
+      if (__ballot(fm == cf) != 0ull) {
+        const uint32_t wave_id0 = static_cast<uint32_t>(chunk) * kSChunk +
+                                  static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(wave)) * 64u * VEC;
+        u64 qe[kSVec];
+#pragma unroll
+        for (int j = 0; j < kSVec; ++j) {
+          qe[j] = __ballot(qm[j] == cf);
+          asm volatile("" : "+s"(qe[j]));
+        }
+#pragma unroll
+        for (int j = 0; j < kSVec; ++j) {
+          if (qe[j] != 0ull) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              const u64 m = __ballot(v[j * 4 + c] == cf);
+              if (m != 0ull) {
+                const uint32_t id = wave_id0 + static_cast<uint32_t>(elem_offset<kSBlock, VEC>(j * 4 + c)) +
+                                    static_cast<uint32_t>(__builtin_ctzll(m)) * VEC;
+                widx = id < widx ? id : widx;
+              }
+            }
+          }
+        }
+        for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
+          const uint32_t i = i0 + tid;
+          const bool hit = i < n_extra && sm.extra_val[i] == cf;
+          const uint32_t id = wave_max<uint32_t>(hit ? ~sm.extra_idx[i] : 0u);
+          if (id != 0u && ~id < widx) widx = ~id;
+        }
+      }
+    }
+    if (lane == 0) sm.wave_val[wave] = ~widx;  // (the reduction above ended with a barrier: the slots are free)
+    lds_barrier();
     if (wave != 0 && !finisher) return false;
     if (wave == 0) {
-      key = lane < kSWaves ? sm.list_hi[lane] : 0;
-      key = wave_max(key);
+      uint32_t best = 0u;  // ~id of the lowest id
+#pragma unroll
+      for (int w = 0; w < kSWaves; ++w) best = sm.wave_val[w] > best ? sm.wave_val[w] : best;
+      u64 key = best != 0u ? (static_cast<u64>(cmax) << 32) | best : 0;
       if (chunk == 0 && sm.nan0 != 0u) key = ~0ull;
+      if (n_chunks == 1) {  // the row is this chunk: nothing to hand over
+        const bool found = !extra_overflow && key != 0;
+        if (lane == 0) {
+          sm.flag = found ? 1u : 0u;
+          if (found) outputs.token[0] = static_cast<int32_t>(key64_index(key));
+        }
+      } else {
       const size_t ci = static_cast<size_t>(row) * n_chunks + chunk;
       const u64 slot = extra_overflow ? kSlotOverflow : (key != 0 ? key : kSlotEmpty);
       if (!finisher) {
@@ -846,6 +907,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       if (lane == 0) {
         sm.flag = found ? 1u : 0u;
         if (found) outputs.token[0] = static_cast<int32_t>(key64_index(best));
+      }
       }
     }
     __syncthreads();
@@ -1229,7 +1291,18 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
 // value first needed behind a branch is requested behind that branch: left alone, five such round trips (per-row
 // table? shape, mode, row pointer, flag word) stood in front of the first logits request of every wave.
 // Returns the uniform (k, p, T) as values that exist before the first branch.
+template <bool XFORM>
 __device__ __forceinline__ mi355x_sample_params args_up_front(const SampleArgs& a) {
+  if constexpr (XFORM) {  // what the logits processing reads before the logits are requested, in the same round trip
+    const uint32_t* mask = a.xf.mask;
+    const int32_t* history = a.xf.history;
+    const int32_t* history_lens = a.xf.history_lens;
+    const uint32_t* ban = a.xf.ban;
+    int history_stride = a.xf.history_stride, history_len = a.xf.history_len, n_eos = a.xf.n_eos;
+    float penalty = a.xf.penalty;
+    asm volatile("" : "+s"(mask), "+s"(history), "+s"(history_lens), "+s"(ban), "+s"(history_stride), "+s"(history_len),
+                 "+s"(n_eos), "+s"(penalty));
+  }
   const void* logits = a.logits;
   int64_t row_stride = a.row_stride;
   int vocab = a.vocab, chunks = a.chunks, k = a.uniform.k, emit_topk = a.emit_topk, exact_kernel = a.exact_kernel;
@@ -1249,7 +1322,7 @@ __device__ __forceinline__ mi355x_sample_params args_up_front(const SampleArgs& 
 
 template <typename InT, bool INLINE, bool NUCLEUS, bool XFORM, bool LARGEK = false, bool ARGMAX = false>
 __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
-  const mi355x_sample_params uniform_prm = args_up_front(a);
+  const mi355x_sample_params uniform_prm = args_up_front<XFORM>(a);
   const int row = blockIdx.y, chunk = blockIdx.x;
   __shared__ FusedShared sm;
   const mi355x_sample_params prm = row_params<INLINE>(a, row, uniform_prm);
