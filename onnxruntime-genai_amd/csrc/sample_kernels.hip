@@ -362,18 +362,29 @@ struct SortWithTile {
   }
 };
 
+// Where entry i of the sorted list lives once its exponential is cached in it: the epilogue's threads each read
+// eight consecutive entries, 64 bytes apart from lane to lane, so entry i moves inside its group of eight to slot
+// (i ^ (i >> 4)) & 7, which spreads those reads over all banks.
+__device__ __forceinline__ uint32_t exp_slot(uint32_t i) { return (i & ~7u) | ((i ^ (i >> 4)) & 7u); }
+
 // The tail shared by the finish kernels: lds_keys[0 .. n_c) hold a row's candidates as key64s in any order,
 // best_below (0: none) is the best element of the row that is not among them.  Sorts them together in LDS,
 // caches the exponentials and runs the exact epilogue.  With cut_at_best_below the candidates that rank
 // after best_below are dropped first (they are not a prefix of the row's order).  rmax / thr: order keys of
 // the best and of (a bound below) the lowest candidate, which scale the buckets of the sort.  Returns false
 // when the row needs the exact path (the epilogue found no end of the nucleus among the elements given).
+// presorted: lds_keys[0 .. n_c) are sorted and hold their exponentials already (sort_gathered), only the epilogue is left.
 __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucket_start, uint32_t n_c, u64 best_below,
                                                   uint32_t rmax, uint32_t thr, bool cut_at_best_below,
                                                   mi355x_sample_params prm, int V, double u, const RowOutputs& out,
                                                   SeqShared& seqsh, uint32_t* red32, const SampleArgs* emit = nullptr,
-                                                  int emit_row = 0, const void* emit_row0 = nullptr) {
+                                                  int emit_row = 0, const void* emit_row0 = nullptr, bool presorted = false) {
   const int tid = threadIdx.x;
+  const u64* lk = lds_keys;
+  auto sorted = [=](int i) { return lk[exp_slot(static_cast<uint32_t>(i))]; };
+  auto exps = [=](int i) { return __uint_as_float(static_cast<uint32_t>(lk[exp_slot(static_cast<uint32_t>(i))] >> 32)); };
+  // (presorted: the list is sorted and carries its exponentials already; one call of the epilogue serves both cases)
+  if (!presorted) {
   if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
   if (best_below != 0) n_c += 1;
   __syncthreads();
@@ -422,7 +433,7 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
   const float max_score = key_to_float(key64_okey(lds_keys[0]));
   __syncthreads();
   const float inv_temp = 1.0f / prm.temperature;
-  auto slot_of = [](uint32_t i) { return (i & ~7u) | ((i ^ (i >> 4)) & 7u); };
+  auto slot_of = [](uint32_t i) { return exp_slot(i); };
   static_assert(kFinishBlock % 8 == 0 && kNucleusCap % 8 == 0, "whole groups per pass");
   for (uint32_t i = tid; i < ((n_c + 7u) & ~7u); i += blockDim.x) {
     const u64 k64 = i < n_c ? lds_keys[i] : 0;
@@ -430,9 +441,7 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
     lds_keys[slot_of(i)] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k64 & 0xffffffffull);
   }
   __syncthreads();
-  const u64* lk = lds_keys;
-  auto sorted = [=](int i) { return lk[slot_of(static_cast<uint32_t>(i))]; };
-  auto exps = [=](int i) { return __uint_as_float(static_cast<uint32_t>(lk[slot_of(static_cast<uint32_t>(i))] >> 32)); };
+  }
   return block_sample_epilogue<8>(sorted, exps, static_cast<int>(n_c), V, prm, u, out, seqsh);
 }
 
@@ -788,14 +797,165 @@ constexpr int kSparseExtraRegs = 2;                           // processed histo
 constexpr int kSparseExtras = kSparseExtraRegs * kFinishBlock;  // distinct history ids (their list uses the bucket table's LDS)
 static_assert(2 * kSparseExtras <= kSortBuckets + 1, "the list of processed history ids fits the bucket table");
 
-template <typename InT>
-__device__ __forceinline__ void sparse_gather(const void* row0, const uint32_t (&ids)[kSparseIds + kSparseExtraRegs], float (&x)[kSparseIds + kSparseExtraRegs]) {
-  const InT* const p = static_cast<const InT*>(row0);
-  InT raw[kSparseIds];
+// A logit as the bits it is stored in (fp32: the word, 16-bit types: the half word), so that the loads of a gather
+// are plain loads issued back to back whatever the type, and the value of such bits.
+__device__ __forceinline__ uint32_t logit_bits(const void* row0, int dtype, uint32_t i) {
+  return dtype == MI355X_F32 ? static_cast<const uint32_t*>(row0)[i] : static_cast<uint32_t>(static_cast<const uint16_t*>(row0)[i]);
+}
+__device__ __forceinline__ float logit_of_bits(uint32_t bits, int dtype) {
+  if (dtype == MI355X_F16) return half_bits_to_float(static_cast<uint16_t>(bits));
+  if (dtype == MI355X_BF16) return bf16_bits_to_float(static_cast<uint16_t>(bits));
+  return __uint_as_float(bits);
+}
+
+constexpr int kSparseRegs = kSparseIds + kSparseExtraRegs;
+constexpr uint32_t kSparseDirectMin = 2 * kFinishBlock;  // shorter lists take the general tail (a sorting network)
+
+// The sort, the trimming and the exponentials of a row whose elements the block's threads hold in registers
+// (ids[u] / x[u], 0xffffffff: no element): the same bucket sort as bucket_sort_desc, fed from the registers instead
+// of a list in LDS, with the histogram of its counting pass also deciding where the nucleus certainly ends (the
+// bound of trim_to_nucleus, in fp32: it only has to be a bound, the epilogue decides on exact values), so that the
+// buckets past that point are neither placed nor ranked.  `start` (kSortBuckets + 1 words) must be zero on entry.
+// Leaves the sorted entries in `keys` the way the epilogue reads them (exponential << 32 | id at exp_slot(rank)) and
+// returns their number; 0: a bucket holds more than kBucketCap keys, nothing but `start` was written, ids[u] of
+// candidates carry a mark above their low 20 bits (the others are 0), the caller takes the general tail.
+// best_below: the best element of the row that is not a candidate, as far as this thread knows (0: none); on return
+// with 0 the thread's own elements below the threshold have been added to it.
+__device__ __forceinline__ uint32_t sort_gathered(u64* keys, uint32_t* start, uint32_t (&ids)[kSparseRegs],
+                                                  const float (&x)[kSparseRegs], uint32_t rmax, uint32_t thr, u64& best_below,
+                                                  mi355x_sample_params prm, int V, uint32_t* red32, u64* red64) {
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const float fmax = key_to_float(rmax);
+  const float span = fmax - key_to_float(thr);
+  const float scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
+  auto bucket_of = [=](uint32_t okey) {
+    float bf = (fmax - key_to_float(okey)) * scale;
+    bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);  // also NaN-safe
+    return bf > 0.0f ? static_cast<uint32_t>(bf) : 0u;
+  };
+  // counting pass; a candidate's slot inside its bucket rides on its id from here on (ids stay below 1 << 20)
+  constexpr uint32_t kIdBits = 20, kIdMask = (1u << kIdBits) - 1u, kIsCand = 1u << 31;
+  static_assert(kFinishBlock * kSparseWords * 32 <= (1 << kIdBits) && kBucketCap < 255, "the packing of id and slot");
 #pragma unroll
-  for (int u = 0; u < kSparseIds; ++u) raw[u] = p[ids[u] != 0xffffffffu ? ids[u] : 0u];
+  for (int u = 0; u < kSparseRegs; ++u) {
+    const bool have = ids[u] != 0xffffffffu;
+    const uint32_t ok32 = order_key(x[u]);
+    if (have && ok32 >= thr) {
+      const uint32_t slot = atomicAdd(&start[bucket_of(ok32)], 1u);
+      ids[u] |= kIsCand | ((slot < 255u ? slot : 255u) << kIdBits);
+    } else if (have) {
+      const u64 k64 = make_key64(ok32, ids[u]);
+      best_below = k64 > best_below ? k64 : best_below;
+      ids[u] = 0u;
+    } else {
+      ids[u] = 0u;
+    }
+  }
+  __syncthreads();
+  // exclusive scan of the counts (consecutive buckets per thread) with the lower bound of the mass next to it
+  constexpr int kPer = kSortBuckets / kFinishBlock;
+  const float inv_temp = 1.0f / prm.temperature;
+  const float step = scale > 0.0f ? inv_temp / scale : 0.0f;  // exponent per bucket
+  const bool trim = prm.p > 0.0f && prm.p < 1.0f && scale > 0.0f;
+  uint32_t cnt[kPer], local = 0u, big = 0u;
+  float mb[kPer], mass = 0.0f;
 #pragma unroll
-  for (int u = 0; u < kSparseIds; ++u) x[u] = load_one<InT>(&raw[u], 0);
+  for (int i = 0; i < kPer; ++i) {
+    const int b = t * kPer + i;
+    cnt[i] = start[b];
+    local += cnt[i];
+    big |= cnt[i] > static_cast<uint32_t>(kBucketCap) ? 1u : 0u;
+    mb[i] = static_cast<float>(cnt[i]) * __expf(-static_cast<float>(b + 1) * step);
+    mass += mb[i];
+  }
+  const uint32_t inc = wave_prefix_sum<uint32_t>(local);
+  const float minc = wave_prefix_sum<float>(mass);
+  if (lane == 63) red64[wave] = (static_cast<u64>(__float_as_uint(minc)) << 32) | inc;
+  __syncthreads();
+  const u64 of_wave = lane < kFinishBlock / 64 ? red64[lane] : 0;
+  const uint32_t cw = wave_prefix_sum<uint32_t>(static_cast<uint32_t>(of_wave));
+  const float mw = wave_prefix_sum<float>(__uint_as_float(static_cast<uint32_t>(of_wave >> 32)));
+  const uint32_t n_cand = wave_read_lane(cw, kFinishBlock / 64 - 1);
+  uint32_t c = (wave > 0 ? wave_read_lane(cw, wave - 1) : 0u) + inc - local;
+  float m = (wave > 0 ? wave_read_lane(mw, wave - 1) : 0.0f) + (minc - mass);
+  // The stop of the nucleus search lies at or before the last element of bucket b once
+  //   mass(0..b) * (1 - p) >= p * (V - count(0..b)) * exp(upper edge of b)
+  // (2 % to spare for the roundings); when b is empty the element that satisfies the rule is the first one of the
+  // next bucket that is not.  So the first non-empty bucket that follows a bucket with that property is the last
+  // one the sort keeps.
+  uint32_t mine = static_cast<uint32_t>(kSortBuckets);
+  const float pf = prm.p;
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int b = t * kPer + i;
+    if (trim && cnt[i] != 0u && b > 0 && mine == static_cast<uint32_t>(kSortBuckets)) {
+      const bool closed_before =
+          m * (1.0f - pf) >= 1.02f * pf * static_cast<float>(static_cast<uint32_t>(V) - c) * __expf(-static_cast<float>(b - 1) * step);
+      if (closed_before) mine = static_cast<uint32_t>(b);
+    }
+    start[b] = c;
+    c += cnt[i];
+    m += mb[i];
+  }
+  if (t == kFinishBlock - 1) start[kSortBuckets] = c;
+  const uint32_t red = block_max<uint32_t>(big ? 0xffffffffu : ~mine, red32);  // its barriers also publish the starts
+  if (red == 0xffffffffu) return 0u;
+  const uint32_t last_bucket = ~red;  // kSortBuckets: every bucket is kept
+  uint32_t n_sorted = n_cand, n = n_cand;
+  if (last_bucket < static_cast<uint32_t>(kSortBuckets)) {
+    n_sorted = n = start[last_bucket + 1u];
+    best_below = 0;
+  } else {
+    best_below = block_max<u64>(best_below, red64);  // ranks after every candidate
+    n += best_below != 0 ? 1u : 0u;
+  }
+  // every kept key to its bucket, in the order of arrival
+#pragma unroll
+  for (int u = 0; u < kSparseRegs; ++u) {
+    if (ids[u] & kIsCand) {
+      const uint32_t ok32 = order_key(x[u]);
+      const uint32_t b = bucket_of(ok32);
+      if (b <= last_bucket) keys[start[b] + ((ids[u] >> kIdBits) & 255u)] = make_key64(ok32, ids[u] & kIdMask);
+    }
+  }
+  __syncthreads();
+  // The list is read back position by position (a thread's neighbours hold the neighbouring positions, so the lanes
+  // of a wave look at the same few buckets); a key's rank inside its bucket comes from comparing whole keys.
+  constexpr int R = kNucleusCap / kFinishBlock;
+  const uint32_t n_pad = (n + 7u) & ~7u;
+  u64 k[R];
+  uint32_t fin[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (static_cast<uint32_t>(r * kFinishBlock) < n_pad) {
+      const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + t);
+      k[r] = pos == n_sorted && pos < n ? best_below : 0;
+      fin[r] = pos;
+      if (pos < n_sorted) {
+        k[r] = keys[pos];
+        const uint32_t b = bucket_of(key64_okey(k[r]));
+        const uint32_t lo = start[b], hi = start[b + 1u];
+        uint32_t rank = 0u;
+        for (uint32_t j = lo; j < hi; ++j) rank += keys[j] > k[r] ? 1u : 0u;
+        fin[r] = lo + rank;
+      }
+    }
+  }
+  __syncthreads();
+  // final places, with exp((s - max) / T) cached in the score half of every entry (the last group of eight is
+  // filled up with empty entries)
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (static_cast<uint32_t>(r * kFinishBlock) < n_pad) {
+      const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + t);
+      if (pos < n_pad) {
+        const float e = em::expf_exact((key_to_float(key64_okey(k[r])) - fmax) * inv_temp);
+        keys[exp_slot(fin[r])] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k[r] & 0xffffffffull);
+      }
+    }
+  }
+  __syncthreads();
+  return n;
 }
 
 // Returns 1 when the row is finished, 0 when it is not, -1 when it is not a nucleus row.
@@ -804,19 +964,21 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   extern __shared__ u64 lds_keys[];
   uint32_t* const bucket_start = reinterpret_cast<uint32_t*>(lds_keys + kNucleusCap);
   uint32_t* const hist_bits = reinterpret_cast<uint32_t*>(lds_keys);                  // first half: history bitmap of the row
+  constexpr int kStashWords = kNucleusCap / 2;  // rows of up to that many mask words also keep their allowed ids as bits there
+  uint32_t* const allowed_bits = hist_bits + kStashWords;
   uint32_t* const id_list = reinterpret_cast<uint32_t*>(lds_keys + kNucleusCap / 2);  // second half: ids to gather
   float* const extra_val = reinterpret_cast<float*>(bucket_start);
   uint32_t* const extra_idx = bucket_start + kSparseExtras;
   __shared__ SeqShared seqsh;
   __shared__ uint32_t red32[16];
   __shared__ u64 red64[16];
-  __shared__ uint32_t sh_total, sh_extra, sh_count;
-  const int row = blockIdx.x, tid = threadIdx.x, lane = lane_id();
+  __shared__ uint32_t sh_extra, sh_count;
+  const int row = blockIdx.x, tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
   const int V = a.vocab;
   const mi355x_sample_params prm = row_params<INLINE>(a, row);
   if (row_mode(prm, V, a.chunks) != kModeNucleus) return -1;
   const int words = (V - 1) / 32 + 1;
-  const RowPtr<AnyDtype> lrow(row_start<INLINE>(a, row, dtype_bytes(a.dtype)), a.dtype);
+  const void* const row0 = row_start<INLINE>(a, row, dtype_bytes(a.dtype));
   // A row this kernel cannot finish is left to the dense kernels launched after it -- or, when the caller's
   // bound on the mask made this the only kernel, to the exact path (the caller of this function sees to that).
   auto leave = [&](bool done) { return done ? 1 : 0; };
@@ -824,87 +986,61 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   const uint32_t* mrow = a.xf.mask + static_cast<size_t>(row) * words;
   const int n_eos = a.xf.eos_count(row);
   const bool pen = a.xf.use_penalty();
-  // The thread's first history id is requested before anything else, its logit and mask word right after the
-  // mask words below: three dependent round trips to memory (id, logit, then the gather) would otherwise follow
-  // one another behind the barriers.
+  // The gather of the allowed ids' logits is what takes the time, so it starts as early as it can: straight after
+  // the mask words, with the history's ids still among the ids it fetches.  The history (ids, their logits and
+  // mask words: dependent round trips to memory) is worked through while the gather is in flight; an id found in
+  // it then leaves the gathered ones, its processed value joins as a candidate of its own.
   const int32_t* const h = pen ? a.xf.history + static_cast<size_t>(row) * a.xf.history_stride : nullptr;
   const int hlen = pen ? a.xf.hist_len(row) : 0;
   const int tok0 = (pen && tid < hlen) ? h[tid] : -1;
   // allowed ids of this thread's words: mask bits minus the EOS ids under min-length, nothing past the vocabulary
-  uint32_t w[kSparseWords], valid[kSparseWords];
+  uint32_t w[kSparseWords];
 #pragma unroll
   for (int q = 0; q < kSparseWords; ++q) {
     const int wi = tid + q * kFinishBlock;
     w[q] = 0u;
-    valid[q] = 0u;
-    if (q * kFinishBlock < words && wi < words) {
-      const int n_real = V - wi * 32;
-      valid[q] = n_real >= 32 ? ~0u : ((1u << n_real) - 1u);
-      uint32_t m = mrow[wi];
-      for (int e = 0; e < n_eos; ++e)
-        if ((a.xf.eos[e] >> 5) == wi) m &= ~(1u << (a.xf.eos[e] & 31));
-      w[q] = m & valid[q];
-    }
+    if (q * kFinishBlock < words && wi < words) w[q] = mrow[wi];
   }
-  const bool tok0_ok = tok0 >= 0 && tok0 < V;
-  const float raw0 = tok0_ok ? lrow[tok0] : 0.0f;
-  const uint32_t mw0 = tok0_ok ? mrow[tok0 >> 5] : 0u;
+  auto valid_bits = [&](int wi) {
+    const int n_real = V - wi * 32;
+    return wi >= words ? 0u : n_real >= 32 ? ~0u : ((1u << n_real) - 1u);
+  };
+  if (pen)
+    for (int i = tid; i < words; i += kFinishBlock) hist_bits[i] = 0u;
   if (tid == 0) {
-    sh_total = 0u;
     sh_extra = 0u;
     sh_count = 0u;
   }
-  // history ids: marked in a bitmap of the whole row; whoever marks an id first computes its processed value
-  if (pen) {
-    for (int i = tid; i < words; i += kFinishBlock) hist_bits[i] = 0u;
-    __syncthreads();
-    const uint32_t* ban_row = a.xf.ban_row(row, V);
-    for (int j = tid; j < hlen; j += kFinishBlock) {
-      const bool ahead = j == tid;  // fetched above
-      const int tok = ahead ? tok0 : h[j];
-      if (tok < 0 || tok >= V) continue;
-      const uint32_t bit = 1u << (tok & 31);
-      if (atomicOr(&hist_bits[tok >> 5], bit) & bit) continue;
-      const uint32_t slot = atomicAdd(&sh_extra, 1u);
-      if (slot < static_cast<uint32_t>(kSparseExtras)) {
-        extra_val[slot] = xform_value(ahead ? raw0 : lrow[tok], a.xf.penalty, a.xf.eos, tok, ahead ? mw0 : mrow[tok >> 5], true, true,
-                                      n_eos, ban_row);
-        extra_idx[slot] = static_cast<uint32_t>(tok);
-      }
-    }
-  }
-  __syncthreads();
-  // ids to gather (allowed, not in the history) and the first masked id outside the history
-  uint32_t count = 0u, first_masked = 0xffffffffu;
+  uint32_t count = 0u;
 #pragma unroll
   for (int q = 0; q < kSparseWords; ++q) {
     if (q * kFinishBlock < words) {
       const int wi = tid + q * kFinishBlock;
-      const uint32_t hb = (pen && wi < words) ? hist_bits[wi] : 0u;
-      const uint32_t masked = ~w[q] & valid[q] & ~hb;
-      w[q] &= ~hb;
+      uint32_t m = w[q];
+      for (int e = 0; e < n_eos; ++e)
+        if ((a.xf.eos[e] >> 5) == wi) m &= ~(1u << (a.xf.eos[e] & 31));
+      w[q] = m & valid_bits(wi);
       count += static_cast<uint32_t>(__popc(w[q]));
-      if (masked != 0u) {
-        const uint32_t id = static_cast<uint32_t>(wi) * 32u + static_cast<uint32_t>(__ffs(masked) - 1);
-        first_masked = id < first_masked ? id : first_masked;
-      }
     }
   }
-  uint32_t inc = wave_prefix_sum<uint32_t>(count);
-  uint32_t wave_base = 0u;
-  if (lane == 63) wave_base = atomicAdd(&sh_total, inc);
-  wave_base = wave_read_lane(wave_base, 63);
-  first_masked = ~block_max<uint32_t>(~first_masked, red32);  // its barriers also publish sh_total and sh_extra
-  const uint32_t n_allowed = sh_total, n_extra = sh_extra;
-  if (n_allowed + n_extra + 2u > static_cast<uint32_t>(kNucleusCap) || n_extra > static_cast<uint32_t>(kSparseExtras) ||
-      n_allowed + n_extra == 0u)
-    return leave(false);
+  // (the thread's first history id has arrived with the mask words: its logit and mask word are requested now)
+  const bool tok0_ok = tok0 >= 0 && tok0 < V;
+  const uint32_t mw0 = tok0_ok ? mrow[tok0 >> 5] : 0u;
+  const uint32_t raw0 = tok0_ok ? logit_bits(row0, a.dtype, static_cast<uint32_t>(tok0)) : 0u;
+  const uint32_t inc = wave_prefix_sum<uint32_t>(count);
+  if (lane == 63) red32[wave] = inc;
+  __syncthreads();
+  const uint32_t per_wave = wave_prefix_sum<uint32_t>(lane < kFinishBlock / 64 ? red32[lane] : 0u);
+  const uint32_t n_allowed = wave_read_lane(per_wave, kFinishBlock / 64 - 1);
+  const uint32_t wave_base = wave > 0 ? wave_read_lane(per_wave, wave - 1) : 0u;
+  if (n_allowed + 2u > static_cast<uint32_t>(kNucleusCap)) return leave(false);
   uint32_t pos = wave_base + inc - count;
 #pragma unroll
   for (int q = 0; q < kSparseWords; ++q) {
     if (q * kFinishBlock < words) {
       uint32_t m = w[q];
       const uint32_t base_id = static_cast<uint32_t>(tid + q * kFinishBlock) * 32u;
+      if (words <= kStashWords && tid + q * kFinishBlock < words) allowed_bits[tid + q * kFinishBlock] = m;  // (for this thread)
       while (m != 0u) {
         id_list[pos++] = base_id + static_cast<uint32_t>(__ffs(m) - 1);
         m &= m - 1u;
@@ -914,6 +1050,7 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   __syncthreads();
   // gather: every load of a thread is requested before the first is used
   uint32_t ids[kSparseIds + kSparseExtraRegs];
+  uint32_t raw[kSparseIds];
   float x[kSparseIds + kSparseExtraRegs];
 #pragma unroll
   for (int u = 0; u < kSparseIds; ++u) {
@@ -921,15 +1058,79 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
     ids[u] = i < n_allowed ? id_list[i] : 0xffffffffu;
   }
   // (the element type is resolved once, outside the loads, so that they are plain loads issued back to back)
-  if (a.dtype == MI355X_F16) sparse_gather<uint16_t>(lrow.p, ids, x);
-  else if (a.dtype == MI355X_BF16) sparse_gather<bf16_t>(lrow.p, ids, x);
-  else sparse_gather<float>(lrow.p, ids, x);
+  if (a.dtype == MI355X_F32) {
+#pragma unroll
+    for (int u = 0; u < kSparseIds; ++u) raw[u] = static_cast<const uint32_t*>(row0)[ids[u] != 0xffffffffu ? ids[u] : 0u];
+  } else {
+#pragma unroll
+    for (int u = 0; u < kSparseIds; ++u) raw[u] = static_cast<const uint16_t*>(row0)[ids[u] != 0xffffffffu ? ids[u] : 0u];
+  }
+  // history ids: marked in a bitmap of the whole row; whoever marks an id first computes its processed value
+  if (pen) {
+    const RowPtr<AnyDtype> lrow(row0, a.dtype);
+    const uint32_t* ban_row = a.xf.ban_row(row, V);
+    for (int j = tid; j < hlen; j += kFinishBlock) {
+      const bool ahead = j == tid;  // fetched above
+      const int tok = ahead ? tok0 : h[j];
+      if (tok < 0 || tok >= V) continue;
+      const uint32_t bit = 1u << (tok & 31);
+      if (atomicOr(&hist_bits[tok >> 5], bit) & bit) continue;
+      const uint32_t slot = atomicAdd(&sh_extra, 1u);
+      if (slot < static_cast<uint32_t>(kSparseExtras)) {
+        extra_val[slot] = xform_value(ahead ? logit_of_bits(raw0, a.dtype) : lrow[tok], a.xf.penalty, a.xf.eos, tok,
+                                      ahead ? mw0 : mrow[tok >> 5], true, true, n_eos, ban_row);
+        extra_idx[slot] = static_cast<uint32_t>(tok);
+      }
+    }
+  }
+  __syncthreads();
+  const uint32_t n_extra = sh_extra;
+  if (n_allowed + n_extra + 2u > static_cast<uint32_t>(kNucleusCap) || n_extra > static_cast<uint32_t>(kSparseExtras) ||
+      n_allowed + n_extra == 0u)
+    return leave(false);
+  // the gathered ids that are in the history leave; the first masked id outside the history
+  uint32_t first_masked = 0xffffffffu;
+  if (pen) {
+#pragma unroll
+    for (int u = 0; u < kSparseIds; ++u) {
+      const uint32_t id = ids[u] != 0xffffffffu ? ids[u] : 0u;
+      if ((hist_bits[id >> 5] >> (id & 31u)) & 1u) ids[u] = 0xffffffffu;
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < kSparseWords; ++q) {
+    if (q * kFinishBlock < words) {
+      const int wi = tid + q * kFinishBlock;
+      const uint32_t hb = (pen && wi < words) ? hist_bits[wi] : 0u;
+      uint32_t allowed = 0u;
+      if (wi < words) {
+        if (words <= kStashWords) {
+          allowed = allowed_bits[wi];
+        } else {  // (no room to keep them: the mask word once more, behind the gather)
+          allowed = mrow[wi];
+          for (int e = 0; e < n_eos; ++e)
+            if ((a.xf.eos[e] >> 5) == wi) allowed &= ~(1u << (a.xf.eos[e] & 31));
+        }
+      }
+      const uint32_t masked = ~allowed & valid_bits(wi) & ~hb;
+      if (masked != 0u) {
+        const uint32_t id = static_cast<uint32_t>(wi) * 32u + static_cast<uint32_t>(__ffs(masked) - 1);
+        first_masked = id < first_masked ? id : first_masked;
+      }
+    }
+  }
 #pragma unroll
   for (int u = 0; u < kSparseExtraRegs; ++u) {
     const uint32_t i = static_cast<uint32_t>(tid + u * kFinishBlock);
     ids[kSparseIds + u] = i < n_extra ? extra_idx[i] : 0xffffffffu;
     x[kSparseIds + u] = i < n_extra ? extra_val[i] : __uint_as_float(0x7fc00000u);
   }
+  first_masked = ~block_max<uint32_t>(~first_masked, red32);  // (its barriers: every thread has read its extras)
+  const bool direct = n_allowed + n_extra > kSparseDirectMin;
+  if (direct)
+    for (int b = tid; b <= kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;  // while the gather is in flight
+#pragma unroll
+  for (int u = 0; u < kSparseIds; ++u) x[u] = logit_of_bits(raw[u], a.dtype);
   uint32_t kmax = 0u;
 #pragma unroll
   for (int u = 0; u < kSparseIds + kSparseExtraRegs; ++u) {
@@ -940,9 +1141,19 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   if (rmax == 0u) return leave(false);
   const uint32_t thr = order_key(key_to_float(rmax) - nucleus_depth(prm, V));
   if (thr <= order_key(kLowest)) return leave(false);  // masked ids would be candidates themselves
+  u64 best_below = first_masked != 0xffffffffu ? make_key64(order_key(kLowest), first_masked) : 0;
+  uint32_t n_c = 0u;
+  if (direct) {
+    n_c = sort_gathered(lds_keys, bucket_start, ids, x, rmax, thr, best_below, prm, V, red32, red64);
+    if (n_c == 0u) {  // heavy ties: the general tail, the candidates as they were
+#pragma unroll
+      for (int u = 0; u < kSparseRegs; ++u) ids[u] = (ids[u] >> 31) ? (ids[u] & 0xfffffu) : 0xffffffffu;
+    }
+  }
+  const bool presorted = n_c != 0u;
+  if (!presorted) {
   // candidates (at or above the threshold) go to the sort buffer at slots a wave reserves with one atomic per
   // batch; the best of the others is kept
-  u64 best_below = first_masked != 0xffffffffu ? make_key64(order_key(kLowest), first_masked) : 0;
 #pragma unroll
   for (int u0 = 0; u0 < kSparseIds + kSparseExtraRegs; u0 += 6) {
     u64 hits[6];
@@ -971,9 +1182,10 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
     }
   }
   best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
-  const uint32_t n_c = sh_count;
-  const bool ok = finish_candidates(lds_keys, bucket_start, n_c, best_below, rmax, thr, false, prm, V, a.uniforms[row],
-                                    row_outputs(a, row), seqsh, red32);
+  n_c = sh_count;
+  }
+  const bool ok = finish_candidates(lds_keys, bucket_start, n_c, presorted ? 0 : best_below, rmax, thr, false, prm, V, a.uniforms[row],
+                                    row_outputs(a, row), seqsh, red32, nullptr, 0, nullptr, presorted);
   return leave(ok);
 }
 
