@@ -19,7 +19,7 @@ struct SeqShared {
   float ev_a[2][16], ev_b[2][16];
   uint32_t n_last[2];
   float head_sum;
-  int head_found;
+  int head_found, head_n;
   // block_discrete_draw / block_min2
   int red_a[16];
   int red_b[16];
@@ -225,13 +225,15 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
   __syncthreads();  // a previous call's readers are done with the parity-0 buffers
   // A sum that starts from nothing changes binade every few additions, and each change costs a pass
   // of the scan below.  The first `head` elements are therefore added for real, 64 at a time, by a
-  // chain of lane-shifted float additions in wave 0 (about ten cycles per element).
+  // chain of lane-shifted float additions in wave 0 (about ten cycles per element).  The head ends early once 64
+  // elements have added less than an eighth to the sum: from there on a binade is left rarely, and the other waves
+  // wait while the head runs.
   int n_head = 0;
   if (head > 0) {
     n_head = head < n ? head : n;
     if (wave == 0) {
       float carry = s0;
-      int fnd = -1;
+      int fnd = -1, done = n_head;
       float x_next = lane < n_head ? get(lane) : 0.0f;
       for (int r0 = 0; r0 < n_head && fnd < 0; r0 += 64) {
         const float x = x_next;
@@ -244,17 +246,24 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
           fnd = r0 + l;
           carry = wave_read_lane(sp, l);
         } else {
+          const float before = carry;
           carry = wave_read_lane(sp, 63);  // lanes past the end added zeros
+          if (carry - before <= 0.125f * carry && r0 + 64 < n_head) {
+            done = r0 + 64;
+            break;
+          }
         }
       }
       if (lane == 0) {
         sh.head_sum = carry;
         sh.head_found = fnd;
+        sh.head_n = done;
       }
     }
     __syncthreads();
     s = sh.head_sum;
     found = sh.head_found;
+    n_head = sh.head_n;
   }
   for (int w0 = n_head; w0 < n && found < 0; w0 += span) {
     const int base = w0 + tid * ITEMS;

@@ -809,64 +809,92 @@ __device__ __forceinline__ float logit_of_bits(uint32_t bits, int dtype) {
 }
 
 constexpr int kSparseRegs = kSparseIds + kSparseExtraRegs;
+// Slot u of the threads' registers holds elements at all (the same answer for every thread: whole slots are skipped):
+// gathered ids fill the first kSparseIds slots thread by thread, processed history ids the slots after them.
+__device__ __forceinline__ bool sparse_slot_used(int u, uint32_t n_gathered, uint32_t n_extra) {
+  return u < kSparseIds ? static_cast<uint32_t>(u * kFinishBlock) < n_gathered
+                        : static_cast<uint32_t>((u - kSparseIds) * kFinishBlock) < n_extra;
+}
 constexpr uint32_t kSparseDirectMin = 2 * kFinishBlock;  // shorter lists take the general tail (a sorting network)
 
-// The sort, the trimming and the exponentials of a row whose elements the block's threads hold in registers
-// (ids[u] / x[u], 0xffffffff: no element): the same bucket sort as bucket_sort_desc, fed from the registers instead
-// of a list in LDS, with the histogram of its counting pass also deciding where the nucleus certainly ends (the
-// bound of trim_to_nucleus, in fp32: it only has to be a bound, the epilogue decides on exact values), so that the
-// buckets past that point are neither placed nor ranked.  `start` (kSortBuckets + 1 words) must be zero on entry.
-// Leaves the sorted entries in `keys` the way the epilogue reads them (exponential << 32 | id at exp_slot(rank)) and
-// returns their number; 0: a bucket holds more than kBucketCap keys, nothing but `start` was written, ids[u] of
-// candidates carry a mark above their low 20 bits (the others are 0), the caller takes the general tail.
-// best_below: the best element of the row that is not a candidate, as far as this thread knows (0: none); on return
-// with 0 the thread's own elements below the threshold have been added to it.
-__device__ __forceinline__ uint32_t sort_gathered(u64* keys, uint32_t* start, uint32_t (&ids)[kSparseRegs],
-                                                  const float (&x)[kSparseRegs], uint32_t rmax, uint32_t thr, u64& best_below,
-                                                  mi355x_sample_params prm, int V, uint32_t* red32, u64* red64) {
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const float fmax = key_to_float(rmax);
-  const float span = fmax - key_to_float(thr);
-  const float scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
-  auto bucket_of = [=](uint32_t okey) {
-    float bf = (fmax - key_to_float(okey)) * scale;
+// The bucket sort of bucket_sort_desc for a row whose elements the block's threads hold in registers (ids[u] with the
+// order key ok[u] of its score; 0xffffffff: no element; n_gathered / n_extra as for sparse_slot_used), in two parts.
+// The buckets are linear in the score below `top`, the score of order key rtop; scores above it share bucket 0 (the
+// whole keys are compared inside a bucket, so any monotone assignment sorts exactly).
+struct GatheredBuckets {
+  float top, scale;  // bucket = (top - score) * scale, within 0 .. kSortBuckets - 1
+  __device__ __forceinline__ GatheredBuckets(uint32_t rtop, uint32_t thr) {
+    top = key_to_float(rtop);
+    const float span = top - key_to_float(thr);
+    scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
+  }
+  __device__ __forceinline__ uint32_t operator()(uint32_t okey) const {
+    float bf = (top - key_to_float(okey)) * scale;
     bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);  // also NaN-safe
     return bf > 0.0f ? static_cast<uint32_t>(bf) : 0u;
-  };
-  // counting pass; a candidate's slot inside its bucket rides on its id from here on (ids stay below 1 << 20)
-  constexpr uint32_t kIdBits = 20, kIdMask = (1u << kIdBits) - 1u, kIsCand = 1u << 31;
-  static_assert(kFinishBlock * kSparseWords * 32 <= (1 << kIdBits) && kBucketCap < 255, "the packing of id and slot");
+  }
+};
+constexpr uint32_t kGatheredIdBits = 20, kGatheredIdMask = (1u << kGatheredIdBits) - 1u, kGatheredIsCand = 1u << 31;
+static_assert(kFinishBlock * kSparseWords * 32 <= (1 << kGatheredIdBits) && kBucketCap < 255, "the packing of id and slot");
+
+// Part one, for the slots U0 .. U1 - 1: a candidate (order key at or above thr) takes a slot in its bucket's count
+// (`start`, kSortBuckets + 1 words, zero before the first call), which rides on its id from here on (ids stay below
+// 1 << 20), with a mark; the others leave (id 0) after updating best_below, the thread's best element below the
+// threshold.  Slots can be counted as soon as their values are there, while later ones are still on their way.
+template <int U0, int U1>
+__device__ __forceinline__ void count_gathered(uint32_t* start, uint32_t (&ids)[kSparseRegs], const uint32_t (&ok)[kSparseRegs],
+                                               const GatheredBuckets& bucket_of, uint32_t thr, u64& best_below,
+                                               uint32_t n_gathered, uint32_t n_extra) {
 #pragma unroll
-  for (int u = 0; u < kSparseRegs; ++u) {
-    const bool have = ids[u] != 0xffffffffu;
-    const uint32_t ok32 = order_key(x[u]);
-    if (have && ok32 >= thr) {
-      const uint32_t slot = atomicAdd(&start[bucket_of(ok32)], 1u);
-      ids[u] |= kIsCand | ((slot < 255u ? slot : 255u) << kIdBits);
-    } else if (have) {
-      const u64 k64 = make_key64(ok32, ids[u]);
-      best_below = k64 > best_below ? k64 : best_below;
+  for (int u = U0; u < U1; ++u) {
+    if (!sparse_slot_used(u, n_gathered, n_extra)) {
       ids[u] = 0u;
+      continue;
+    }
+    const bool have = ids[u] != 0xffffffffu;
+    if (have && ok[u] >= thr) {
+      const uint32_t slot = atomicAdd(&start[bucket_of(ok[u])], 1u);
+      ids[u] |= kGatheredIsCand | ((slot < 255u ? slot : 255u) << kGatheredIdBits);
     } else {
+      if (have) {
+        const u64 k64 = make_key64(ok[u], ids[u]);
+        best_below = k64 > best_below ? k64 : best_below;
+      }
       ids[u] = 0u;
     }
   }
+}
+
+// Part two, once every slot is counted: the scan of the counts, the trimming, the places and the exponentials.  The
+// histogram of the counting pass also bounds where the nucleus certainly ends (the bound of trim_to_nucleus, in
+// fp32 and per thread's run of buckets: it only has to be a bound, the epilogue decides on exact values), so that
+// the buckets past that point are neither placed nor ranked.  Leaves the sorted entries in `keys` the way the
+// epilogue reads them (exp((score - max) / T) << 32 | id at exp_slot(rank), rmax: order key of the row's maximum)
+// and returns their number; 0: a bucket holds more than kBucketCap keys, nothing but `start` was written, the caller
+// takes the general tail.  best_below: the thread's best element below the threshold (0: none).
+__device__ __forceinline__ uint32_t sort_counted(u64* keys, uint32_t* start, const uint32_t (&ids)[kSparseRegs],
+                                                 const uint32_t (&ok)[kSparseRegs], const GatheredBuckets& bucket_of, uint32_t rmax,
+                                                 u64 best_below, uint32_t n_gathered, uint32_t n_extra, mi355x_sample_params prm,
+                                                 int V, uint32_t* red32, u64* red64) {
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   __syncthreads();
-  // exclusive scan of the counts (consecutive buckets per thread) with the lower bound of the mass next to it
+  // exclusive scan of the counts (consecutive buckets per thread) with a lower bound of the mass next to it: every
+  // key of bucket b weighs at least exp(-(b + 1) * step) times the weight of `top`
   constexpr int kPer = kSortBuckets / kFinishBlock;
   const float inv_temp = 1.0f / prm.temperature;
-  const float step = scale > 0.0f ? inv_temp / scale : 0.0f;  // exponent per bucket
-  const bool trim = prm.p > 0.0f && prm.p < 1.0f && scale > 0.0f;
+  const float step = bucket_of.scale > 0.0f ? inv_temp / bucket_of.scale : 0.0f;  // exponent per bucket
+  const bool trim = prm.p > 0.0f && prm.p < 1.0f && bucket_of.scale > 0.0f;
+  const float ratio = __expf(-step);
+  float edge = __expf(-static_cast<float>(t * kPer + 1) * step);
   uint32_t cnt[kPer], local = 0u, big = 0u;
-  float mb[kPer], mass = 0.0f;
+  float mass = 0.0f;
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
-    const int b = t * kPer + i;
-    cnt[i] = start[b];
+    cnt[i] = start[t * kPer + i];
     local += cnt[i];
     big |= cnt[i] > static_cast<uint32_t>(kBucketCap) ? 1u : 0u;
-    mb[i] = static_cast<float>(cnt[i]) * __expf(-static_cast<float>(b + 1) * step);
-    mass += mb[i];
+    mass += static_cast<float>(cnt[i]) * edge;
+    edge *= ratio;
   }
   const uint32_t inc = wave_prefix_sum<uint32_t>(local);
   const float minc = wave_prefix_sum<float>(mass);
@@ -877,32 +905,32 @@ __device__ __forceinline__ uint32_t sort_gathered(u64* keys, uint32_t* start, ui
   const float mw = wave_prefix_sum<float>(__uint_as_float(static_cast<uint32_t>(of_wave >> 32)));
   const uint32_t n_cand = wave_read_lane(cw, kFinishBlock / 64 - 1);
   uint32_t c = (wave > 0 ? wave_read_lane(cw, wave - 1) : 0u) + inc - local;
-  float m = (wave > 0 ? wave_read_lane(mw, wave - 1) : 0.0f) + (minc - mass);
+  const float m = (wave > 0 ? wave_read_lane(mw, wave - 1) : 0.0f) + (minc - mass);
   // The stop of the nucleus search lies at or before the last element of bucket b once
   //   mass(0..b) * (1 - p) >= p * (V - count(0..b)) * exp(upper edge of b)
-  // (2 % to spare for the roundings); when b is empty the element that satisfies the rule is the first one of the
-  // next bucket that is not.  So the first non-empty bucket that follows a bucket with that property is the last
-  // one the sort keeps.
-  uint32_t mine = static_cast<uint32_t>(kSortBuckets);
-  const float pf = prm.p;
+  // (2 % to spare for the roundings); when b is empty, the element that satisfies the rule is the first one of the
+  // next bucket that is not.  A thread tests the bucket before its own: the first thread that finds the property
+  // there and has a key of its own owns the last buckets the sort keeps.  (Bucket 0 may hold keys above its upper
+  // edge: the test starts with thread 1.)
+  uint32_t mine = static_cast<uint32_t>(kFinishBlock);
+  if (trim && t > 0 && local != 0u) {
+    const float pf = prm.p;
+    if (m * (1.0f - pf) >= 1.02f * pf * static_cast<float>(static_cast<uint32_t>(V) - c) * __expf(-static_cast<float>(t * kPer - 1) * step))
+      mine = static_cast<uint32_t>(t);
+  }
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
-    const int b = t * kPer + i;
-    if (trim && cnt[i] != 0u && b > 0 && mine == static_cast<uint32_t>(kSortBuckets)) {
-      const bool closed_before =
-          m * (1.0f - pf) >= 1.02f * pf * static_cast<float>(static_cast<uint32_t>(V) - c) * __expf(-static_cast<float>(b - 1) * step);
-      if (closed_before) mine = static_cast<uint32_t>(b);
-    }
-    start[b] = c;
+    start[t * kPer + i] = c;
     c += cnt[i];
-    m += mb[i];
   }
   if (t == kFinishBlock - 1) start[kSortBuckets] = c;
   const uint32_t red = block_max<uint32_t>(big ? 0xffffffffu : ~mine, red32);  // its barriers also publish the starts
   if (red == 0xffffffffu) return 0u;
-  const uint32_t last_bucket = ~red;  // kSortBuckets: every bucket is kept
+  const uint32_t last_thread = ~red;
+  const bool all_kept = last_thread >= static_cast<uint32_t>(kFinishBlock);
+  const uint32_t last_bucket = all_kept ? static_cast<uint32_t>(kSortBuckets) : last_thread * kPer + (kPer - 1);
   uint32_t n_sorted = n_cand, n = n_cand;
-  if (last_bucket < static_cast<uint32_t>(kSortBuckets)) {
+  if (!all_kept) {
     n_sorted = n = start[last_bucket + 1u];
     best_below = 0;
   } else {
@@ -912,10 +940,9 @@ __device__ __forceinline__ uint32_t sort_gathered(u64* keys, uint32_t* start, ui
   // every kept key to its bucket, in the order of arrival
 #pragma unroll
   for (int u = 0; u < kSparseRegs; ++u) {
-    if (ids[u] & kIsCand) {
-      const uint32_t ok32 = order_key(x[u]);
-      const uint32_t b = bucket_of(ok32);
-      if (b <= last_bucket) keys[start[b] + ((ids[u] >> kIdBits) & 255u)] = make_key64(ok32, ids[u] & kIdMask);
+    if (sparse_slot_used(u, n_gathered, n_extra) && (ids[u] & kGatheredIsCand)) {
+      const uint32_t b = bucket_of(ok[u]);
+      if (b <= last_bucket) keys[start[b] + ((ids[u] >> kGatheredIdBits) & 255u)] = make_key64(ok[u], ids[u] & kGatheredIdMask);
     }
   }
   __syncthreads();
@@ -936,7 +963,10 @@ __device__ __forceinline__ uint32_t sort_gathered(u64* keys, uint32_t* start, ui
         const uint32_t b = bucket_of(key64_okey(k[r]));
         const uint32_t lo = start[b], hi = start[b + 1u];
         uint32_t rank = 0u;
-        for (uint32_t j = lo; j < hi; ++j) rank += keys[j] > k[r] ? 1u : 0u;
+        for (uint32_t j = lo; j < hi; j += 2u) {  // (two reads in flight)
+          const u64 first = keys[j], second = keys[j + 1u];  // (the list is followed by the bucket table: a read past it is harmless)
+          rank += (first > k[r] ? 1u : 0u) + ((j + 1u < hi && second > k[r]) ? 1u : 0u);
+        }
         fin[r] = lo + rank;
       }
     }
@@ -944,6 +974,7 @@ __device__ __forceinline__ uint32_t sort_gathered(u64* keys, uint32_t* start, ui
   __syncthreads();
   // final places, with exp((s - max) / T) cached in the score half of every entry (the last group of eight is
   // filled up with empty entries)
+  const float fmax = key_to_float(rmax);
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (static_cast<uint32_t>(r * kFinishBlock) < n_pad) {
@@ -998,8 +1029,9 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
 #pragma unroll
   for (int q = 0; q < kSparseWords; ++q) {
     const int wi = tid + q * kFinishBlock;
-    w[q] = 0u;
-    if (q * kFinishBlock < words && wi < words) w[q] = mrow[wi];
+    uint32_t word = 0u;
+    if (q * kFinishBlock < words) word = mrow[wi < words ? wi : 0];
+    w[q] = wi < words ? word : 0u;
   }
   auto valid_bits = [&](int wi) {
     const int n_real = V - wi * 32;
@@ -1050,21 +1082,31 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   __syncthreads();
   // gather: every load of a thread is requested before the first is used
   uint32_t ids[kSparseIds + kSparseExtraRegs];
-  uint32_t raw[kSparseIds];
-  float x[kSparseIds + kSparseExtraRegs];
+  uint32_t ok[kSparseRegs];  // the bits of a gathered logit, then the order key of the score (0: not a number, or no element)
 #pragma unroll
   for (int u = 0; u < kSparseIds; ++u) {
     const uint32_t i = static_cast<uint32_t>(tid + u * kFinishBlock);
     ids[u] = i < n_allowed ? id_list[i] : 0xffffffffu;
   }
-  // (the element type is resolved once, outside the loads, so that they are plain loads issued back to back)
-  if (a.dtype == MI355X_F32) {
+  // (The element type is resolved once, outside the loads, so that they are plain loads issued back to back; slots
+  // without an id load element 0, so that the number of loads in flight does not depend on the row.)
+  auto gather_slots = [&](auto first, auto last) {
+    if (a.dtype == MI355X_F32) {
 #pragma unroll
-    for (int u = 0; u < kSparseIds; ++u) raw[u] = static_cast<const uint32_t*>(row0)[ids[u] != 0xffffffffu ? ids[u] : 0u];
-  } else {
+      for (int u = decltype(first)::value; u < decltype(last)::value; ++u)
+        ok[u] = static_cast<const uint32_t*>(row0)[ids[u] != 0xffffffffu ? ids[u] : 0u];
+    } else {
 #pragma unroll
-    for (int u = 0; u < kSparseIds; ++u) raw[u] = static_cast<const uint16_t*>(row0)[ids[u] != 0xffffffffu ? ids[u] : 0u];
-  }
+      for (int u = decltype(first)::value; u < decltype(last)::value; ++u)
+        ok[u] = static_cast<const uint16_t*>(row0)[ids[u] != 0xffffffffu ? ids[u] : 0u];
+    }
+  };
+  // The first loads keep the memory system busy for longer than the history takes: the rest follows after it.  (All
+  // at once would have every wave wait at its load instructions, the queues being full, and reach the history
+  // only when the gather is nearly over.)
+  constexpr int kFirstLoads = 6;
+  gather_slots(std::integral_constant<int, 0>{}, std::integral_constant<int, kFirstLoads>{});
+  asm volatile("" ::: "memory");
   // history ids: marked in a bitmap of the whole row; whoever marks an id first computes its processed value
   if (pen) {
     const RowPtr<AnyDtype> lrow(row0, a.dtype);
@@ -1093,8 +1135,10 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   if (pen) {
 #pragma unroll
     for (int u = 0; u < kSparseIds; ++u) {
-      const uint32_t id = ids[u] != 0xffffffffu ? ids[u] : 0u;
-      if ((hist_bits[id >> 5] >> (id & 31u)) & 1u) ids[u] = 0xffffffffu;
+      if (static_cast<uint32_t>(u * kFinishBlock) < n_allowed) {
+        const uint32_t id = ids[u] != 0xffffffffu ? ids[u] : 0u;
+        if ((hist_bits[id >> 5] >> (id & 31u)) & 1u) ids[u] = 0xffffffffu;
+      }
     }
   }
 #pragma unroll
@@ -1123,31 +1167,61 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   for (int u = 0; u < kSparseExtraRegs; ++u) {
     const uint32_t i = static_cast<uint32_t>(tid + u * kFinishBlock);
     ids[kSparseIds + u] = i < n_extra ? extra_idx[i] : 0xffffffffu;
-    x[kSparseIds + u] = i < n_extra ? extra_val[i] : __uint_as_float(0x7fc00000u);
+    ok[kSparseIds + u] = i < n_extra ? order_key(extra_val[i]) : 0u;
   }
   first_masked = ~block_max<uint32_t>(~first_masked, red32);  // (its barriers: every thread has read its extras)
   const bool direct = n_allowed + n_extra > kSparseDirectMin;
   if (direct)
     for (int b = tid; b <= kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;  // while the gather is in flight
+  asm volatile("" ::: "memory");
+  gather_slots(std::integral_constant<int, kFirstLoads>{}, std::integral_constant<int, kSparseIds>{});
+  // The slots of the first loads and the processed history ids are there before the rest: their maximum stands in
+  // for the row's where only a reference point is needed (the threshold below it, the buckets of the sort), so that
+  // they are counted into their buckets while the other loads are still on their way.
+  auto keys_of_slots = [&](auto first, auto last) {
+    uint32_t kmax = 0u;
 #pragma unroll
-  for (int u = 0; u < kSparseIds; ++u) x[u] = logit_of_bits(raw[u], a.dtype);
-  uint32_t kmax = 0u;
+    for (int u = decltype(first)::value; u < decltype(last)::value; ++u) {
+      const uint32_t bits = ok[u];
+      ok[u] = 0u;
+      if (sparse_slot_used(u, n_allowed, n_extra)) {
+        ok[u] = ids[u] != 0xffffffffu ? order_key(logit_of_bits(bits, a.dtype)) : 0u;
+        kmax = ok[u] > kmax ? ok[u] : kmax;
+      }
+    }
+    return kmax;
+  };
+  uint32_t kmax = keys_of_slots(std::integral_constant<int, 0>{}, std::integral_constant<int, kFirstLoads>{});
 #pragma unroll
-  for (int u = 0; u < kSparseIds + kSparseExtraRegs; ++u) {
-    const uint32_t k = ids[u] != 0xffffffffu ? order_key(x[u]) : 0u;
-    kmax = k > kmax ? k : kmax;
-  }
-  const uint32_t rmax = block_max<uint32_t>(kmax, red32);  // its barriers end every read of the id list and the extras
-  if (rmax == 0u) return leave(false);
-  const uint32_t thr = order_key(key_to_float(rmax) - nucleus_depth(prm, V));
+  for (int u = kSparseIds; u < kSparseRegs; ++u) kmax = ok[u] > kmax ? ok[u] : kmax;
+  const uint32_t rtop = block_max<uint32_t>(kmax, red32);  // its barriers end every read of the id list and the extras
+  if (rtop == 0u) return leave(false);
+  const uint32_t thr = order_key(key_to_float(rtop) - nucleus_depth(prm, V));
   if (thr <= order_key(kLowest)) return leave(false);  // masked ids would be candidates themselves
   u64 best_below = first_masked != 0xffffffffu ? make_key64(order_key(kLowest), first_masked) : 0;
+  const GatheredBuckets bucket_of(rtop, thr);
+  if (direct) {
+    count_gathered<0, kFirstLoads>(bucket_start, ids, ok, bucket_of, thr, best_below, n_allowed, n_extra);
+    count_gathered<kSparseIds, kSparseRegs>(bucket_start, ids, ok, bucket_of, thr, best_below, n_allowed, n_extra);
+  }
+  uint32_t rmax = rtop;
+  if (static_cast<uint32_t>(kFirstLoads * kFinishBlock) < n_allowed) {
+    const uint32_t rest = block_max<uint32_t>(keys_of_slots(std::integral_constant<int, kFirstLoads>{}, std::integral_constant<int, kSparseIds>{}), red32);
+    rmax = rest > rmax ? rest : rmax;
+    if (direct) count_gathered<kFirstLoads, kSparseIds>(bucket_start, ids, ok, bucket_of, thr, best_below, n_allowed, n_extra);
+  } else {
+#pragma unroll
+    for (int u = kFirstLoads; u < kSparseIds; ++u) {
+      ok[u] = 0u;
+      if (direct) ids[u] = 0u;
+    }
+  }
   uint32_t n_c = 0u;
   if (direct) {
-    n_c = sort_gathered(lds_keys, bucket_start, ids, x, rmax, thr, best_below, prm, V, red32, red64);
+    n_c = sort_counted(lds_keys, bucket_start, ids, ok, bucket_of, rmax, best_below, n_allowed, n_extra, prm, V, red32, red64);
     if (n_c == 0u) {  // heavy ties: the general tail, the candidates as they were
 #pragma unroll
-      for (int u = 0; u < kSparseRegs; ++u) ids[u] = (ids[u] >> 31) ? (ids[u] & 0xfffffu) : 0xffffffffu;
+      for (int u = 0; u < kSparseRegs; ++u) ids[u] = (ids[u] >> 31) ? (ids[u] & kGatheredIdMask) : 0xffffffffu;
     }
   }
   const bool presorted = n_c != 0u;
@@ -1161,7 +1235,7 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
 #pragma unroll
     for (int u = u0; u < u0 + 6 && u < kSparseIds + kSparseExtraRegs; ++u) {
       const bool have = ids[u] != 0xffffffffu;
-      const uint32_t ok32 = have ? order_key(x[u]) : 0u;
+      const uint32_t ok32 = have ? ok[u] : 0u;
       const bool cand = have && ok32 >= thr;
       hits[u - u0] = __ballot(cand);
       wcnt += static_cast<uint32_t>(__popcll(hits[u - u0]));
@@ -1177,16 +1251,15 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
     for (int u = u0; u < u0 + 6 && u < kSparseIds + kSparseExtraRegs; ++u) {
       const u64 b = hits[u - u0];
       const uint32_t p = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), base));
-      if ((b >> lane) & 1ull) lds_keys[p] = make_key64(order_key(x[u]), ids[u]);
+      if ((b >> lane) & 1ull) lds_keys[p] = make_key64(ok[u], ids[u]);
       base += static_cast<uint32_t>(__popcll(b));
     }
   }
   best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
   n_c = sh_count;
   }
-  const bool ok = finish_candidates(lds_keys, bucket_start, n_c, presorted ? 0 : best_below, rmax, thr, false, prm, V, a.uniforms[row],
-                                    row_outputs(a, row), seqsh, red32, nullptr, 0, nullptr, presorted);
-  return leave(ok);
+  return leave(finish_candidates(lds_keys, bucket_start, n_c, presorted ? 0 : best_below, rmax, thr, false, prm, V, a.uniforms[row],
+                                 row_outputs(a, row), seqsh, red32, nullptr, 0, nullptr, presorted));
 }
 
 template <bool INLINE>
