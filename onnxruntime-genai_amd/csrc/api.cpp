@@ -57,6 +57,7 @@ struct mi355x_search_ctx {
   ms::u64* cand_small{};
   uint32_t* chunk_cnt{};
   uint32_t* chunk_max{};
+  uint32_t* chunk_thr{};
   ms::u64* chunk_next{};
   uint32_t* row_arrive{};
   ms::u64* row_best{};
@@ -201,6 +202,7 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   ok(c->Alloc(&c->cand_small, sc * ms::kSmallCap, true));  // all-zero between launches
   ok(c->Alloc(&c->chunk_cnt, rc, true));
   ok(c->Alloc(&c->chunk_max, rc, true));
+  ok(c->Alloc(&c->chunk_thr, rc, true));
   ok(c->Alloc(&c->chunk_next, rc, true));
   ok(c->Alloc(&c->row_arrive, static_cast<size_t>(max_rows), true));
   ok(c->Alloc(&c->row_best, static_cast<size_t>(max_rows), true));
@@ -299,6 +301,7 @@ int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int 
     f.cand_small = ctx->cand_small;
     f.chunk_cnt = ctx->chunk_cnt;
     f.chunk_max = ctx->chunk_max;
+    f.chunk_thr = ctx->chunk_thr;
     f.chunk_next = ctx->chunk_next;
     f.big = ctx->big;
     f.big_stride = ctx->big_stride;
@@ -421,6 +424,7 @@ int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const 
   a.cand_small = ctx->cand_small;
   a.chunk_cnt = ctx->chunk_cnt;
   a.chunk_max = ctx->chunk_max;
+  a.chunk_thr = ctx->chunk_thr;
   a.chunk_next = ctx->chunk_next;
   a.big = ctx->big;
   a.big2 = ctx->big2;
@@ -519,6 +523,7 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   a.cand_small = ctx->cand_small;
   a.chunk_cnt = ctx->chunk_cnt;
   a.chunk_max = ctx->chunk_max;
+  a.chunk_thr = ctx->chunk_thr;
   a.chunk_next = ctx->chunk_next;
   a.big = ctx->big;
   a.big2 = ctx->big2;

@@ -61,6 +61,7 @@ struct SampleArgs {
   u64* cand_small;        // [rows][chunks][kSmallCap]; zero between launches (published, then cleared by the finisher)
   uint32_t* chunk_cnt;    // [rows][chunks]
   uint32_t* chunk_max;    // [rows][chunks]
+  uint32_t* chunk_thr;    // [rows][chunks]: order key of the score below which a nucleus chunk listed nothing
   u64* chunk_next;        // [rows][chunks]
   u64* big;               // [rows][big_stride]
   u64* big2;              // [rows][big_stride] second buffer of the exact path's radix sort, or null

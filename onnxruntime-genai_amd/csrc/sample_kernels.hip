@@ -557,6 +557,155 @@ __device__ __forceinline__ void trim_to_nucleus(u64* lds_keys, uint32_t* table, 
   thr = thr2;
 }
 
+// ---- the bucket sort in parts, with the trimming inside ---------------------------------------------------------
+// The buckets of bucket_sort_desc, linear in the score below `top` (the score of order key rtop) down to the score of
+// thr; scores above `top` share bucket 0 (whole keys are compared inside a bucket, so any monotone assignment sorts
+// exactly).
+struct ScoreBuckets {
+  float top, scale;  // bucket = (top - score) * scale, within 0 .. kSortBuckets - 1
+  __device__ __forceinline__ ScoreBuckets(uint32_t rtop, uint32_t thr) {
+    top = key_to_float(rtop);
+    const float span = top - key_to_float(thr);
+    scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
+  }
+  __device__ __forceinline__ uint32_t operator()(uint32_t okey) const {
+    float bf = (top - key_to_float(okey)) * scale;
+    bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);  // also NaN-safe
+    return bf > 0.0f ? static_cast<uint32_t>(bf) : 0u;
+  }
+};
+
+// What the scan keeps: the keys of buckets 0 .. last_bucket, n_sorted of them, in a list of n entries (one more
+// when best_below, the best element below every candidate, follows them).  n = 0: a bucket holds more than
+// kBucketCap keys (or the first thread's buckets alone overflow the room), the caller sorts another way.
+struct TrimmedBuckets {
+  uint32_t last_bucket, n_sorted, n;
+  u64 best_below;
+};
+
+// After a counting pass has left the number of candidates per bucket in start[0 .. kSortBuckets): turns the counts
+// into the buckets' first places (start[kSortBuckets] = their total) and decides how many buckets the sort keeps.
+// The histogram bounds where the nucleus certainly ends (the bound of trim_to_nucleus, in fp32 and per thread's run
+// of buckets: it only has to be a bound, the epilogue decides on exact values and reports a nucleus that does not end
+// among the entries it is given), so the buckets past that point need neither places nor ranks; and no more buckets
+// are kept than fill room - 2 entries.  best_below: this thread's best element below the threshold (0: none); when
+// every bucket is kept, the block's best such element follows the candidates.  Contains barriers; every thread gets
+// the same result.
+__device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start, const ScoreBuckets& bucket_of, u64 best_below,
+                                                                mi355x_sample_params prm, int V, int room, uint32_t* red32,
+                                                                u64* red64) {
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  // exclusive scan of the counts (consecutive buckets per thread) with a lower bound of the mass next to it: every
+  // key of bucket b weighs at least exp(-(b + 1) * step) times the weight of `top`
+  constexpr int kPer = kSortBuckets / kFinishBlock;
+  const float step = bucket_of.scale > 0.0f ? (1.0f / prm.temperature) / bucket_of.scale : 0.0f;  // exponent per bucket
+  const bool trim = prm.p > 0.0f && prm.p < 1.0f && bucket_of.scale > 0.0f;
+  const float ratio = __expf(-step);
+  float edge = __expf(-static_cast<float>(t * kPer + 1) * step);
+  uint32_t cnt[kPer], local = 0u, big = 0u;
+  float mass = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    cnt[i] = start[t * kPer + i];
+    local += cnt[i];
+    big |= cnt[i] > static_cast<uint32_t>(kBucketCap) ? 1u : 0u;
+    mass += static_cast<float>(cnt[i]) * edge;
+    edge *= ratio;
+  }
+  const uint32_t inc = wave_prefix_sum<uint32_t>(local);
+  const float minc = wave_prefix_sum<float>(mass);
+  if (lane == 63) red64[wave] = (static_cast<u64>(__float_as_uint(minc)) << 32) | inc;
+  __syncthreads();
+  const u64 of_wave = lane < kFinishBlock / 64 ? red64[lane] : 0;
+  const uint32_t cw = wave_prefix_sum<uint32_t>(static_cast<uint32_t>(of_wave));
+  const float mw = wave_prefix_sum<float>(__uint_as_float(static_cast<uint32_t>(of_wave >> 32)));
+  const uint32_t n_cand = wave_read_lane(cw, kFinishBlock / 64 - 1);
+  uint32_t c = (wave > 0 ? wave_read_lane(cw, wave - 1) : 0u) + inc - local;
+  const float m = (wave > 0 ? wave_read_lane(mw, wave - 1) : 0.0f) + (minc - mass);
+  // The stop of the nucleus search lies at or before the last element of bucket b once
+  //   mass(0..b) * (1 - p) >= p * (V - count(0..b)) * exp(upper edge of b)
+  // (2 % to spare for the roundings); when b is empty, the element that satisfies the rule is the first one of the
+  // next bucket that is not.  A thread tests the bucket before its own: the first thread that finds the property
+  // there and has a key of its own owns the last buckets the sort keeps.  (Bucket 0 may hold keys above its upper
+  // edge: the test starts with thread 1.)  A thread whose buckets end beyond the room ends the kept ones before it.
+  uint32_t mine = static_cast<uint32_t>(kFinishBlock);
+  if (trim && t > 0 && local != 0u) {
+    const float pf = prm.p;
+    if (m * (1.0f - pf) >= 1.02f * pf * static_cast<float>(static_cast<uint32_t>(V) - c) * __expf(-static_cast<float>(t * kPer - 1) * step))
+      mine = static_cast<uint32_t>(t);
+  }
+  if (c + local > static_cast<uint32_t>(room - 2)) {
+    if (t == 0) big = 1u;
+    else mine = static_cast<uint32_t>(t - 1) < mine ? static_cast<uint32_t>(t - 1) : mine;
+  }
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    start[t * kPer + i] = c;
+    c += cnt[i];
+  }
+  if (t == kFinishBlock - 1) start[kSortBuckets] = c;
+  const uint32_t red = block_max<uint32_t>(big ? 0xffffffffu : ~mine, red32);  // its barriers also publish the starts
+  TrimmedBuckets r{static_cast<uint32_t>(kSortBuckets), n_cand, 0u, 0};
+  if (red == 0xffffffffu) return r;
+  const uint32_t last_thread = ~red;
+  if (last_thread < static_cast<uint32_t>(kFinishBlock)) {
+    r.last_bucket = last_thread * kPer + (kPer - 1);
+    r.n_sorted = r.n = start[r.last_bucket + 1u];
+    if (r.n == 0u) r.n_sorted = r.n = 0u;  // (cannot be: the first thread's buckets hold the maximum)
+  } else {
+    r.best_below = block_max<u64>(best_below, red64);  // ranks after every candidate
+    r.n = n_cand + (r.best_below != 0 ? 1u : 0u);
+  }
+  return r;
+}
+
+// The last part, once every kept key lies somewhere inside its bucket's places: the list is read back position by
+// position (a thread's neighbours hold the neighbouring positions, so the lanes of a wave look at the same few
+// buckets), a key's rank inside its bucket comes from comparing whole keys, and the pass that writes the final places
+// caches exp((score - max) / T) in the score half of every entry, at exp_slot(rank), the way the epilogue reads the
+// list (rmax: order key of the row's maximum).  SHIFTED: the keys were placed by counting start[b] up, so bucket b
+// now lies between start[b - 1] and start[b]; otherwise between start[b] and start[b + 1].
+template <bool SHIFTED>
+__device__ __forceinline__ void rank_and_cache_exps(u64* keys, const uint32_t* start, const ScoreBuckets& bucket_of,
+                                                    const TrimmedBuckets& kept, uint32_t rmax, float inv_temp) {
+  const int t = threadIdx.x;
+  constexpr int R = kNucleusCap / kFinishBlock;
+  const uint32_t n_pad = (kept.n + 7u) & ~7u;
+  u64 k[R];
+  uint32_t fin[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (static_cast<uint32_t>(r * kFinishBlock) < n_pad) {
+      const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + t);
+      k[r] = pos == kept.n_sorted && pos < kept.n ? kept.best_below : 0;
+      fin[r] = pos;
+      if (pos < kept.n_sorted) {
+        k[r] = keys[pos];
+        const uint32_t b = bucket_of(key64_okey(k[r]));
+        const uint32_t lo = SHIFTED ? (b > 0u ? start[b - 1u] : 0u) : start[b];
+        const uint32_t hi = SHIFTED ? start[b] : start[b + 1u];
+        uint32_t rank = 0u;
+        for (uint32_t j = lo; j < hi; ++j) rank += keys[j] > k[r] ? 1u : 0u;
+        fin[r] = lo + rank;
+      }
+    }
+  }
+  __syncthreads();
+  // (the last group of eight is filled up with empty entries)
+  const float fmax = key_to_float(rmax);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (static_cast<uint32_t>(r * kFinishBlock) < n_pad) {
+      const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + t);
+      if (pos < n_pad) {
+        const float e = em::expf_exact((key_to_float(key64_okey(k[r])) - fmax) * inv_temp);
+        keys[exp_slot(fin[r])] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k[r] & 0xffffffffull);
+      }
+    }
+  }
+  __syncthreads();
+}
+
 // Per-row finish of the nucleus path: gathers the candidates the streaming pass left in `big`,
 // sorts them in LDS and runs the exact epilogue.  One block of kFinishBlock threads per row;
 // dynamic LDS: kNucleusCap key64s + the bucket table of the sort.
@@ -595,19 +744,23 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // their prefix sums
   __shared__ int sh_trim;
   __shared__ uint32_t sh_head, sh_all;
-  uint32_t m = 0u;
+  uint32_t m = 0u, cthr = 0u;
   u64 best_below = 0;
   if (tid < a.chunks) {
     const uint32_t cnt = a.chunk_cnt[cbase + tid];
     m = cnt == kChunkCntOverflow ? 0xffffffffu : a.chunk_max[cbase + tid];  // above every key: the exact path
+    cthr = large_k ? 0u : a.chunk_thr[cbase + tid];
     best_below = large_k ? 0 : a.chunk_next[cbase + tid];
     sh_cnt[tid] = cnt;
   }
   if (tid == 0) sh_count = 0u;
   const uint32_t rmax = block_max<uint32_t>(m, red32);
   const bool gave_up = rmax == 0xffffffffu;
+  // Every chunk's threshold holds for the whole row (no element of the row below it lies strictly inside the
+  // nucleus), so the highest one is the row's: every element at or above it is in its chunk's list.
   uint32_t thr = 0u;
-  if (rmax != 0u && !large_k) thr = order_key(key_to_float(rmax) - nucleus_depth(prm, V));
+  if (!large_k) thr = block_max<uint32_t>(cthr, red32);
+  if (rmax == 0u) thr = 0u;  // (no number in the row)
   if (tid == 0) {
     uint32_t all = 0u;
     for (int c = 0; c < a.chunks; ++c) all += gave_up ? 0u : sh_cnt[c];
@@ -651,6 +804,74 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // score-linear buckets.  The nucleus test of the epilogue only looks at the elements it is given, in
   // rank order, and reports when they do not contain the nucleus; only then does the row need the
   // exact path.
+  // The entries of the head (in registers) and then of the rest of the lists, in batches: fn(entries, valid).
+  auto listed_batches = [&](auto fn) {
+    if (head != 0u) {
+#pragma unroll
+      for (int b = 0; b < kAheadChunks * kAhead / kGather; ++b) {
+        if (b * kGather / kAhead < a.chunks) {
+          u64 raw[kGather];
+          bool valid[kGather];
+#pragma unroll
+          for (int u = 0; u < kGather; ++u) {
+            const int q = b * kGather + u, c = q / kAhead;
+            raw[u] = pre[q];
+            valid[u] = c < a.chunks && static_cast<uint32_t>((q % kAhead) * kFinishBlock + tid) < sh_cnt[c < a.chunks ? c : 0];
+          }
+          fn(raw, valid);
+        }
+      }
+    }
+    flat_batches(fn);
+  };
+  // A nucleus row's usual way: a counting sort over the lists where they lie.  A first pass over them counts the
+  // candidates (at or above the row's threshold) into the sort's buckets; the histogram tells how many buckets the
+  // nucleus can reach at all (and how many fit the sort); a second pass gives every key of those buckets a place in
+  // LDS.  However long the lists are, only what is kept has to fit.  A bucket with too many keys (heavy ties) leaves
+  // the row to the steps below: the list in LDS, trimmed, and the sorting network.
+  bool presorted = false, ok = false;
+  uint32_t n_c = 0u;
+  if (!large_k && !gave_up && rmax != 0u) {
+    const ScoreBuckets bucket_of(rmax, thr);
+    for (int b = tid; b <= kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;
+    __syncthreads();
+    u64 below = best_below;
+    listed_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
+#pragma unroll
+      for (int u = 0; u < kGather; ++u) {
+        if (valid[u]) {
+          const uint32_t ok32 = order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)));
+          if (ok32 >= thr) {
+            atomicAdd(&bucket_start[bucket_of(ok32)], 1u);
+          } else {
+            const u64 k64 = (static_cast<u64>(ok32) << 32) | (raw[u] & 0xffffffffull);
+            below = k64 > below ? k64 : below;
+          }
+        }
+      }
+    });
+    __syncthreads();
+    const TrimmedBuckets kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, kNucleusCap, red32, red64);
+    if (kept.n != 0u) {
+      listed_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
+#pragma unroll
+        for (int u = 0; u < kGather; ++u) {
+          if (valid[u]) {
+            const uint32_t ok32 = order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)));
+            if (ok32 >= thr) {
+              const uint32_t b = bucket_of(ok32);
+              if (b <= kept.last_bucket) lds_keys[atomicAdd(&bucket_start[b], 1u)] = (static_cast<u64>(ok32) << 32) | (raw[u] & 0xffffffffull);
+            }
+          }
+        }
+      });
+      __syncthreads();
+      rank_and_cache_exps<true>(lds_keys, bucket_start, bucket_of, kept, rmax, 1.0f / prm.temperature);
+      presorted = ok = true;
+      n_c = kept.n;
+    }
+  }
+  if (!presorted) {
   bool trim_failed = false;
   if (!large_k && sh_all >= static_cast<uint32_t>(kNucleusCap)) {  // head == 0 here
     const float fmax = key_to_float(rmax), fthr = key_to_float(thr);
@@ -737,33 +958,18 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       base += static_cast<uint32_t>(__popcll(hits[u]));
     }
   };
-  if (head != 0u) {
-#pragma unroll
-    for (int b = 0; b < kAheadChunks * kAhead / kGather; ++b) {
-      if (b * kGather / kAhead < a.chunks) {
-        u64 raw[kGather];
-        bool valid[kGather];
-#pragma unroll
-        for (int u = 0; u < kGather; ++u) {
-          const int q = b * kGather + u, c = q / kAhead;
-          raw[u] = pre[q];
-          valid[u] = c < a.chunks && static_cast<uint32_t>((q % kAhead) * kFinishBlock + tid) < sh_cnt[c < a.chunks ? c : 0];
-        }
-        consume(raw, valid);
-      }
-    }
-  }
-  flat_batches(consume);
+  listed_batches(consume);
   best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
-  uint32_t n_c = sh_count;
-  bool ok = !gave_up && !trim_failed && n_c < kNucleusCap;  // room for the next-best element too
+  n_c = sh_count;
+  ok = !gave_up && !trim_failed && n_c < kNucleusCap;  // room for the next-best element too
   if (large_k) thr = ~block_max<uint32_t>(~lowest, red32);  // the lowest candidate score: the sort scales its buckets by it
   if (ok && !large_k) trim_to_nucleus(lds_keys, bucket_start, n_c, best_below, rmax, thr, prm, V, red32, red64, &sh_count);
+  }
   if (ok) {
     const bool emit = large_k && a.emit_topk == 1;
-    ok = finish_candidates(lds_keys, bucket_start, n_c, best_below, rmax, thr, false, prm, V, emit ? 0.0 : a.uniforms[row],
-                           row_outputs(a, row), seqsh, red32, emit ? &a : nullptr, row,
-                           emit ? row_start<INLINE>(a, row, dtype_bytes(a.dtype)) : nullptr);
+    ok = finish_candidates(lds_keys, bucket_start, n_c, presorted ? 0 : best_below, rmax, thr, false, prm, V,
+                           emit ? 0.0 : a.uniforms[row], row_outputs(a, row), seqsh, red32, emit ? &a : nullptr, row,
+                           emit ? row_start<INLINE>(a, row, dtype_bytes(a.dtype)) : nullptr, presorted);
   }
   if (!ok) {
     __syncthreads();
@@ -817,23 +1023,9 @@ __device__ __forceinline__ bool sparse_slot_used(int u, uint32_t n_gathered, uin
 }
 constexpr uint32_t kSparseDirectMin = 2 * kFinishBlock;  // shorter lists take the general tail (a sorting network)
 
-// The bucket sort of bucket_sort_desc for a row whose elements the block's threads hold in registers (ids[u] with the
-// order key ok[u] of its score; 0xffffffff: no element; n_gathered / n_extra as for sparse_slot_used), in two parts.
-// The buckets are linear in the score below `top`, the score of order key rtop; scores above it share bucket 0 (the
-// whole keys are compared inside a bucket, so any monotone assignment sorts exactly).
-struct GatheredBuckets {
-  float top, scale;  // bucket = (top - score) * scale, within 0 .. kSortBuckets - 1
-  __device__ __forceinline__ GatheredBuckets(uint32_t rtop, uint32_t thr) {
-    top = key_to_float(rtop);
-    const float span = top - key_to_float(thr);
-    scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
-  }
-  __device__ __forceinline__ uint32_t operator()(uint32_t okey) const {
-    float bf = (top - key_to_float(okey)) * scale;
-    bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);  // also NaN-safe
-    return bf > 0.0f ? static_cast<uint32_t>(bf) : 0u;
-  }
-};
+// The bucket sort of a row whose elements the block's threads hold in registers (ids[u] with the order key ok[u] of
+// its score; 0xffffffff: no element; n_gathered / n_extra as for sparse_slot_used): counted slot by slot, then
+// scanned, placed and ranked.
 constexpr uint32_t kGatheredIdBits = 20, kGatheredIdMask = (1u << kGatheredIdBits) - 1u, kGatheredIsCand = 1u << 31;
 static_assert(kFinishBlock * kSparseWords * 32 <= (1 << kGatheredIdBits) && kBucketCap < 255, "the packing of id and slot");
 
@@ -843,7 +1035,7 @@ static_assert(kFinishBlock * kSparseWords * 32 <= (1 << kGatheredIdBits) && kBuc
 // threshold.  Slots can be counted as soon as their values are there, while later ones are still on their way.
 template <int U0, int U1>
 __device__ __forceinline__ void count_gathered(uint32_t* start, uint32_t (&ids)[kSparseRegs], const uint32_t (&ok)[kSparseRegs],
-                                               const GatheredBuckets& bucket_of, uint32_t thr, u64& best_below,
+                                               const ScoreBuckets& bucket_of, uint32_t thr, u64& best_below,
                                                uint32_t n_gathered, uint32_t n_extra) {
 #pragma unroll
   for (int u = U0; u < U1; ++u) {
@@ -865,128 +1057,28 @@ __device__ __forceinline__ void count_gathered(uint32_t* start, uint32_t (&ids)[
   }
 }
 
-// Part two, once every slot is counted: the scan of the counts, the trimming, the places and the exponentials.  The
-// histogram of the counting pass also bounds where the nucleus certainly ends (the bound of trim_to_nucleus, in
-// fp32 and per thread's run of buckets: it only has to be a bound, the epilogue decides on exact values), so that
-// the buckets past that point are neither placed nor ranked.  Leaves the sorted entries in `keys` the way the
-// epilogue reads them (exp((score - max) / T) << 32 | id at exp_slot(rank), rmax: order key of the row's maximum)
-// and returns their number; 0: a bucket holds more than kBucketCap keys, nothing but `start` was written, the caller
-// takes the general tail.  best_below: the thread's best element below the threshold (0: none).
+// Part two, once every slot is counted: scan and trimming, the places, ranks and exponentials.  Returns the number
+// of sorted entries `keys` then holds, the way the epilogue reads them; 0: a bucket holds more than kBucketCap keys,
+// nothing but `start` was written, the caller takes the general tail.  rmax: order key of the row's maximum;
+// best_below: the thread's best element below the threshold (0: none).
 __device__ __forceinline__ uint32_t sort_counted(u64* keys, uint32_t* start, const uint32_t (&ids)[kSparseRegs],
-                                                 const uint32_t (&ok)[kSparseRegs], const GatheredBuckets& bucket_of, uint32_t rmax,
+                                                 const uint32_t (&ok)[kSparseRegs], const ScoreBuckets& bucket_of, uint32_t rmax,
                                                  u64 best_below, uint32_t n_gathered, uint32_t n_extra, mi355x_sample_params prm,
                                                  int V, uint32_t* red32, u64* red64) {
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   __syncthreads();
-  // exclusive scan of the counts (consecutive buckets per thread) with a lower bound of the mass next to it: every
-  // key of bucket b weighs at least exp(-(b + 1) * step) times the weight of `top`
-  constexpr int kPer = kSortBuckets / kFinishBlock;
-  const float inv_temp = 1.0f / prm.temperature;
-  const float step = bucket_of.scale > 0.0f ? inv_temp / bucket_of.scale : 0.0f;  // exponent per bucket
-  const bool trim = prm.p > 0.0f && prm.p < 1.0f && bucket_of.scale > 0.0f;
-  const float ratio = __expf(-step);
-  float edge = __expf(-static_cast<float>(t * kPer + 1) * step);
-  uint32_t cnt[kPer], local = 0u, big = 0u;
-  float mass = 0.0f;
-#pragma unroll
-  for (int i = 0; i < kPer; ++i) {
-    cnt[i] = start[t * kPer + i];
-    local += cnt[i];
-    big |= cnt[i] > static_cast<uint32_t>(kBucketCap) ? 1u : 0u;
-    mass += static_cast<float>(cnt[i]) * edge;
-    edge *= ratio;
-  }
-  const uint32_t inc = wave_prefix_sum<uint32_t>(local);
-  const float minc = wave_prefix_sum<float>(mass);
-  if (lane == 63) red64[wave] = (static_cast<u64>(__float_as_uint(minc)) << 32) | inc;
-  __syncthreads();
-  const u64 of_wave = lane < kFinishBlock / 64 ? red64[lane] : 0;
-  const uint32_t cw = wave_prefix_sum<uint32_t>(static_cast<uint32_t>(of_wave));
-  const float mw = wave_prefix_sum<float>(__uint_as_float(static_cast<uint32_t>(of_wave >> 32)));
-  const uint32_t n_cand = wave_read_lane(cw, kFinishBlock / 64 - 1);
-  uint32_t c = (wave > 0 ? wave_read_lane(cw, wave - 1) : 0u) + inc - local;
-  const float m = (wave > 0 ? wave_read_lane(mw, wave - 1) : 0.0f) + (minc - mass);
-  // The stop of the nucleus search lies at or before the last element of bucket b once
-  //   mass(0..b) * (1 - p) >= p * (V - count(0..b)) * exp(upper edge of b)
-  // (2 % to spare for the roundings); when b is empty, the element that satisfies the rule is the first one of the
-  // next bucket that is not.  A thread tests the bucket before its own: the first thread that finds the property
-  // there and has a key of its own owns the last buckets the sort keeps.  (Bucket 0 may hold keys above its upper
-  // edge: the test starts with thread 1.)
-  uint32_t mine = static_cast<uint32_t>(kFinishBlock);
-  if (trim && t > 0 && local != 0u) {
-    const float pf = prm.p;
-    if (m * (1.0f - pf) >= 1.02f * pf * static_cast<float>(static_cast<uint32_t>(V) - c) * __expf(-static_cast<float>(t * kPer - 1) * step))
-      mine = static_cast<uint32_t>(t);
-  }
-#pragma unroll
-  for (int i = 0; i < kPer; ++i) {
-    start[t * kPer + i] = c;
-    c += cnt[i];
-  }
-  if (t == kFinishBlock - 1) start[kSortBuckets] = c;
-  const uint32_t red = block_max<uint32_t>(big ? 0xffffffffu : ~mine, red32);  // its barriers also publish the starts
-  if (red == 0xffffffffu) return 0u;
-  const uint32_t last_thread = ~red;
-  const bool all_kept = last_thread >= static_cast<uint32_t>(kFinishBlock);
-  const uint32_t last_bucket = all_kept ? static_cast<uint32_t>(kSortBuckets) : last_thread * kPer + (kPer - 1);
-  uint32_t n_sorted = n_cand, n = n_cand;
-  if (!all_kept) {
-    n_sorted = n = start[last_bucket + 1u];
-    best_below = 0;
-  } else {
-    best_below = block_max<u64>(best_below, red64);  // ranks after every candidate
-    n += best_below != 0 ? 1u : 0u;
-  }
+  const TrimmedBuckets kept = scan_buckets_and_trim(start, bucket_of, best_below, prm, V, kNucleusCap, red32, red64);
+  if (kept.n == 0u) return 0u;
   // every kept key to its bucket, in the order of arrival
 #pragma unroll
   for (int u = 0; u < kSparseRegs; ++u) {
     if (sparse_slot_used(u, n_gathered, n_extra) && (ids[u] & kGatheredIsCand)) {
       const uint32_t b = bucket_of(ok[u]);
-      if (b <= last_bucket) keys[start[b] + ((ids[u] >> kGatheredIdBits) & 255u)] = make_key64(ok[u], ids[u] & kGatheredIdMask);
+      if (b <= kept.last_bucket) keys[start[b] + ((ids[u] >> kGatheredIdBits) & 255u)] = make_key64(ok[u], ids[u] & kGatheredIdMask);
     }
   }
   __syncthreads();
-  // The list is read back position by position (a thread's neighbours hold the neighbouring positions, so the lanes
-  // of a wave look at the same few buckets); a key's rank inside its bucket comes from comparing whole keys.
-  constexpr int R = kNucleusCap / kFinishBlock;
-  const uint32_t n_pad = (n + 7u) & ~7u;
-  u64 k[R];
-  uint32_t fin[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    if (static_cast<uint32_t>(r * kFinishBlock) < n_pad) {
-      const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + t);
-      k[r] = pos == n_sorted && pos < n ? best_below : 0;
-      fin[r] = pos;
-      if (pos < n_sorted) {
-        k[r] = keys[pos];
-        const uint32_t b = bucket_of(key64_okey(k[r]));
-        const uint32_t lo = start[b], hi = start[b + 1u];
-        uint32_t rank = 0u;
-        for (uint32_t j = lo; j < hi; j += 2u) {  // (two reads in flight)
-          const u64 first = keys[j], second = keys[j + 1u];  // (the list is followed by the bucket table: a read past it is harmless)
-          rank += (first > k[r] ? 1u : 0u) + ((j + 1u < hi && second > k[r]) ? 1u : 0u);
-        }
-        fin[r] = lo + rank;
-      }
-    }
-  }
-  __syncthreads();
-  // final places, with exp((s - max) / T) cached in the score half of every entry (the last group of eight is
-  // filled up with empty entries)
-  const float fmax = key_to_float(rmax);
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    if (static_cast<uint32_t>(r * kFinishBlock) < n_pad) {
-      const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + t);
-      if (pos < n_pad) {
-        const float e = em::expf_exact((key_to_float(key64_okey(k[r])) - fmax) * inv_temp);
-        keys[exp_slot(fin[r])] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k[r] & 0xffffffffull);
-      }
-    }
-  }
-  __syncthreads();
-  return n;
+  rank_and_cache_exps<false>(keys, start, bucket_of, kept, rmax, 1.0f / prm.temperature);
+  return kept.n;
 }
 
 // Returns 1 when the row is finished, 0 when it is not, -1 when it is not a nucleus row.
@@ -1199,7 +1291,7 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   const uint32_t thr = order_key(key_to_float(rtop) - nucleus_depth(prm, V));
   if (thr <= order_key(kLowest)) return leave(false);  // masked ids would be candidates themselves
   u64 best_below = first_masked != 0xffffffffu ? make_key64(order_key(kLowest), first_masked) : 0;
-  const GatheredBuckets bucket_of(rtop, thr);
+  const ScoreBuckets bucket_of(rtop, thr);
   if (direct) {
     count_gathered<0, kFirstLoads>(bucket_start, ids, ok, bucket_of, thr, best_below, n_allowed, n_extra);
     count_gathered<kSparseIds, kSparseRegs>(bucket_start, ids, ok, bucket_of, thr, best_below, n_allowed, n_extra);

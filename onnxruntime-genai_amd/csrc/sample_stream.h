@@ -208,6 +208,20 @@ __device__ __forceinline__ float nucleus_depth(mi355x_sample_params prm, int voc
   return d * prm.temperature;
 }
 
+// The same depth when more is known about the prefix than that it holds the maximum: `mass` is (a lower bound of) the
+// sum of exp((s - max)/T) over the elements within kDepthMassReach exponent units of the maximum.  An element deeper
+// than those follows all of them in rank order, so its prefix is at least `mass` and the stop test holds once
+// exp((s-max)/T) <= mass * (1-p)/(p*V), with a margin of e^0.5 for the roundings on both sides (of the reference's
+// fp32 prefix, of this sum).  The depth never ends above the reach, or the sum would count elements that follow.
+constexpr float kDepthMassReach = 6.0f;
+__device__ __forceinline__ float nucleus_depth(mi355x_sample_params prm, int vocab, float mass) {
+  float d = 105.0f;
+  if (prm.p <= 0.0f) d = 0.0f;
+  else if (prm.p < 0.999f)
+    d = fminf(105.0f, fmaxf(kDepthMassReach, logf(prm.p * static_cast<float>(vocab) / (1.0f - prm.p)) - logf(fmaxf(mass, 1.0f))) + 0.5f);
+  return d * prm.temperature;
+}
+
 // Values of a published candidate slot that are not keys (a key's low half is ~id, far above these).
 constexpr u64 kSlotEmpty = 1, kSlotOverflow = 2;
 constexpr int kWaveListCap = 128;  // hits one wave can list per chunk
@@ -723,7 +737,28 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
         __syncthreads();
       }
     } else if (cmax != 0u) {
-      thr = key_to_float(cmax) - nucleus_depth(prm, V);
+      // the chunk's own elements near its maximum bound the prefix of everything deeper (any element of the row that
+      // lies deeper than this chunk's threshold follows them in rank order), which moves the threshold up
+      const float fcmax = key_to_float(cmax), inv_t = 1.0f / prm.temperature;
+      float near = 0.0f;
+#pragma unroll
+      for (int e = 0; e < kSElems; ++e) {
+        const float d = (v[e] - fcmax) * inv_t;
+        near += d >= -kDepthMassReach ? __expf(d) : 0.0f;  // (false for NaN)
+      }
+      for (uint32_t i = tid; i < n_extra; i += kSBlock) {
+        const float d = (sm.extra_val[i] - fcmax) * inv_t;
+        near += d >= -kDepthMassReach ? __expf(d) : 0.0f;
+      }
+      near = wave_sum<float>(near);
+      float* const wave_part = reinterpret_cast<float*>(sm.wave_val);
+      if (lane == 0) wave_part[wave] = near;
+      lds_barrier();
+      float mass = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kSWaves; ++w) mass += wave_part[w];
+      lds_barrier();
+      thr = fcmax - nucleus_depth(prm, V, mass);
     }
     // First pass: the wave's number of candidates.
     uint32_t wcnt = 0u;
@@ -809,6 +844,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
       a.chunk_cnt[ci] = extra_overflow ? kChunkCntOverflow : sm.count;
       a.chunk_max[ci] = cmax;
+      a.chunk_thr[ci] = order_key(thr);
       a.chunk_next[ci] = best_below;
     }
     return false;
