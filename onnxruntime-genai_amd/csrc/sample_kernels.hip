@@ -568,11 +568,12 @@ struct ScoreBuckets {
     const float span = top - key_to_float(thr);
     scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
   }
-  __device__ __forceinline__ uint32_t operator()(uint32_t okey) const {
-    float bf = (top - key_to_float(okey)) * scale;
+  __device__ __forceinline__ uint32_t of_score(float score) const {  // (-0 and +0 share a bucket, as they share an order key)
+    float bf = (top - score) * scale;
     bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);  // also NaN-safe
     return bf > 0.0f ? static_cast<uint32_t>(bf) : 0u;
   }
+  __device__ __forceinline__ uint32_t operator()(uint32_t okey) const { return of_score(key_to_float(okey)); }
 };
 
 // What the scan keeps: the keys of buckets 0 .. last_bucket, n_sorted of them, in a list of n entries (one more
@@ -651,7 +652,6 @@ __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start,
   if (last_thread < static_cast<uint32_t>(kFinishBlock)) {
     r.last_bucket = last_thread * kPer + (kPer - 1);
     r.n_sorted = r.n = start[r.last_bucket + 1u];
-    if (r.n == 0u) r.n_sorted = r.n = 0u;  // (cannot be: the first thread's buckets hold the maximum)
   } else {
     r.best_below = block_max<u64>(best_below, red64);  // ranks after every candidate
     r.n = n_cand + (r.best_below != 0 ? 1u : 0u);
@@ -726,19 +726,23 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   constexpr bool large_k = LARGEK;  // then every listed element is a candidate and no element after them is needed
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const size_t cbase = static_cast<size_t>(row) * a.chunks;
-  // The head of every chunk's list (kAhead entries per thread) is requested before the counts are
+  // The head of every chunk's list (a few entries per thread) is requested before the counts are
   // known -- whatever lies past a list's end is discarded later -- so that these loads overlap the
   // round trip for the counts.  Rows of more than kAheadChunks chunks, and rows whose lists hold more
   // than the sort has room for, read everything afterwards.
-  constexpr int kGather = 8, kAheadChunks = 8, kAhead = 2;  // kGather: entries a thread has in flight
-  static_assert((kAheadChunks * kAhead) % kGather == 0, "the head is consumed in whole batches");
-  u64 pre[kAheadChunks * kAhead];
+  constexpr int kGather = 8, kAheadChunks = 8, kHeadSlots = 16;  // kGather: entries a thread has in flight
+  static_assert(kHeadSlots % kGather == 0 && kHeadSlots >= 2 * kAheadChunks, "the head is consumed in whole batches");
+  // (the fewer chunks, the more of each list fits the head: slot q holds entry (q & (per - 1)) * kFinishBlock + tid
+  // of chunk q >> head_shift, per = 1 << head_shift)
+  const int head_shift = a.chunks <= 1 ? 4 : a.chunks <= 2 ? 3 : a.chunks <= 4 ? 2 : 1;
+  u64 pre[kHeadSlots];
 #pragma unroll
-  for (int c = 0; c < kAheadChunks; ++c)
-#pragma unroll
-    for (int u = 0; u < kAhead; ++u)
-      pre[c * kAhead + u] =
-          (a.chunks <= kAheadChunks && c < a.chunks) ? big_row[static_cast<size_t>(c) * kSChunk + u * kFinishBlock + tid] : 0;
+  for (int q = 0; q < kHeadSlots; ++q) {
+    const int c = q >> head_shift, u = q & ((1 << head_shift) - 1);
+    pre[q] = (a.chunks <= kAheadChunks && c < a.chunks) ? big_row[static_cast<size_t>(c) * kSChunk + u * kFinishBlock + tid] : 0;
+  }
+  if (!large_k)  // the sort's table, while the loads are on their way
+    for (int b = tid; b <= kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;
   // Thread c reads everything chunk c left behind; the barriers of the first reduction publish the counts.
   __shared__ uint32_t sh_cnt[kAllCap / kSmallCap];       // candidates per chunk
   __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // their prefix sums
@@ -765,7 +769,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     uint32_t all = 0u;
     for (int c = 0; c < a.chunks; ++c) all += gave_up ? 0u : sh_cnt[c];
     const uint32_t head =
-        (a.chunks <= kAheadChunks && all < static_cast<uint32_t>(kNucleusCap)) ? kAhead * kFinishBlock : 0u;
+        (a.chunks <= kAheadChunks && all < static_cast<uint32_t>(kNucleusCap)) ? static_cast<uint32_t>(kFinishBlock) << head_shift : 0u;
     uint32_t run = 0u;
     for (int c = 0; c < a.chunks; ++c) {
       sh_first[c] = run;
@@ -777,7 +781,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   }
   __syncthreads();
   const int lane = lane_id();
-  // Calls fn(entries, valid) for batches of kGather entries per thread of the flat sequence made of the
+  // Calls fn(entries, valid, used) for batches of kGather entries per thread (bit u of `used` clear: slot u is empty in every thread) of the flat sequence made of the
   // chunks' lists past their heads (sh_first[c] = such entries of the chunks before c).
   const uint32_t head = sh_head;
   auto flat_batches = [&](auto fn) {
@@ -785,18 +789,21 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     for (uint32_t f0 = 0; f0 < total; f0 += kGather * blockDim.x) {
       u64 raw[kGather];
       bool valid[kGather];
+      const uint32_t left = (total - f0 + blockDim.x - 1u) / blockDim.x;
+      const int n_slots = left < static_cast<uint32_t>(kGather) ? static_cast<int>(left) : kGather;  // no thread has an entry beyond
+      const uint32_t used = (1u << n_slots) - 1u;
 #pragma unroll
       for (int u = 0; u < kGather; ++u) {
         const uint32_t f = f0 + u * blockDim.x + tid;
         raw[u] = 0;
-        valid[u] = f < total;
-        if (valid[u]) {
+        valid[u] = u < n_slots && f < total;
+        if (u < n_slots && valid[u]) {
           int c = 0;
           for (int cc = 1; cc < a.chunks; ++cc) c += f >= sh_first[cc] ? 1 : 0;
           raw[u] = big_row[static_cast<size_t>(c) * kSChunk + head + (f - sh_first[c])];
         }
       }
-      fn(raw, valid);
+      fn(raw, valid, used);
     }
   };
   // More candidates listed than the sort holds (a flat distribution): the threshold is raised to the
@@ -804,21 +811,26 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // score-linear buckets.  The nucleus test of the epilogue only looks at the elements it is given, in
   // rank order, and reports when they do not contain the nucleus; only then does the row need the
   // exact path.
-  // The entries of the head (in registers) and then of the rest of the lists, in batches: fn(entries, valid).
+  // The entries of the head (in registers) and then of the rest of the lists, in batches: fn(entries, valid, used),
+  // bit u of `used` clear: no thread has an entry in slot u.
   auto listed_batches = [&](auto fn) {
     if (head != 0u) {
 #pragma unroll
-      for (int b = 0; b < kAheadChunks * kAhead / kGather; ++b) {
-        if (b * kGather / kAhead < a.chunks) {
+      for (int b = 0; b < kHeadSlots / kGather; ++b) {
+        if ((b * kGather) >> head_shift < a.chunks) {
           u64 raw[kGather];
           bool valid[kGather];
+          uint32_t used = 0u;
 #pragma unroll
           for (int u = 0; u < kGather; ++u) {
-            const int q = b * kGather + u, c = q / kAhead;
+            const int q = b * kGather + u, c = q >> head_shift;
+            const uint32_t first = static_cast<uint32_t>(q & ((1 << head_shift) - 1)) * kFinishBlock;
+            const uint32_t cnt = c < a.chunks ? __builtin_amdgcn_readfirstlane(sh_cnt[c < a.chunks ? c : 0]) : 0u;
             raw[u] = pre[q];
-            valid[u] = c < a.chunks && static_cast<uint32_t>((q % kAhead) * kFinishBlock + tid) < sh_cnt[c < a.chunks ? c : 0];
+            valid[u] = first + tid < cnt;
+            used |= first < cnt ? 1u << u : 0u;
           }
-          fn(raw, valid);
+          fn(raw, valid, used);
         }
       }
     }
@@ -832,19 +844,18 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   bool presorted = false, ok = false;
   uint32_t n_c = 0u;
   if (!large_k && !gave_up && rmax != 0u) {
-    const ScoreBuckets bucket_of(rmax, thr);
-    for (int b = tid; b <= kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;
-    __syncthreads();
+    const ScoreBuckets bucket_of(rmax, thr);  // (the table is zero: cleared at the start, barriers since)
+    const float thr_score = key_to_float(thr);
     u64 below = best_below;
-    listed_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
+    listed_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t used) {
 #pragma unroll
       for (int u = 0; u < kGather; ++u) {
-        if (valid[u]) {
-          const uint32_t ok32 = order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)));
-          if (ok32 >= thr) {
-            atomicAdd(&bucket_start[bucket_of(ok32)], 1u);
+        if (((used >> u) & 1u) && valid[u]) {
+          const float score = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
+          if (score >= thr_score) {  // (the same test as on order keys: false for NaN, true for either zero against a zero)
+            atomicAdd(&bucket_start[bucket_of.of_score(score)], 1u);
           } else {
-            const u64 k64 = (static_cast<u64>(ok32) << 32) | (raw[u] & 0xffffffffull);
+            const u64 k64 = (static_cast<u64>(order_key(score)) << 32) | (raw[u] & 0xffffffffull);
             below = k64 > below ? k64 : below;
           }
         }
@@ -853,14 +864,15 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     __syncthreads();
     const TrimmedBuckets kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, kNucleusCap, red32, red64);
     if (kept.n != 0u) {
-      listed_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
+      listed_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t used) {
 #pragma unroll
         for (int u = 0; u < kGather; ++u) {
-          if (valid[u]) {
-            const uint32_t ok32 = order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)));
-            if (ok32 >= thr) {
-              const uint32_t b = bucket_of(ok32);
-              if (b <= kept.last_bucket) lds_keys[atomicAdd(&bucket_start[b], 1u)] = (static_cast<u64>(ok32) << 32) | (raw[u] & 0xffffffffull);
+          if (((used >> u) & 1u) && valid[u]) {
+            const float score = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
+            if (score >= thr_score) {
+              const uint32_t b = bucket_of.of_score(score);
+              if (b <= kept.last_bucket)
+                lds_keys[atomicAdd(&bucket_start[b], 1u)] = (static_cast<u64>(order_key(score)) << 32) | (raw[u] & 0xffffffffull);
             }
           }
         }
@@ -885,7 +897,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     for (int b = tid; b < kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;
     __syncthreads();
     const uint32_t thr0 = thr;
-    flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
+    flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
 #pragma unroll
       for (int u = 0; u < kGather; ++u) {
         const float x = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
@@ -933,7 +945,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // row's threshold) go to LDS at slots a wave reserves with one atomic per batch, the best of the
   // others is kept.
   uint32_t lowest = 0xffffffffu;  // lowest candidate key this thread has seen
-  auto consume = [&](const u64 (&raw)[kGather], const bool (&valid)[kGather]) {
+  auto consume = [&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
     u64 k64[kGather], hits[kGather];
     uint32_t wcnt = 0u;
 #pragma unroll

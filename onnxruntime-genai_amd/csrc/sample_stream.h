@@ -213,7 +213,8 @@ __device__ __forceinline__ float nucleus_depth(mi355x_sample_params prm, int voc
 // than those follows all of them in rank order, so its prefix is at least `mass` and the stop test holds once
 // exp((s-max)/T) <= mass * (1-p)/(p*V), with a margin of e^0.5 for the roundings on both sides (of the reference's
 // fp32 prefix, of this sum).  The depth never ends above the reach, or the sum would count elements that follow.
-constexpr float kDepthMassReach = 6.0f;
+constexpr float kDepthWaveReach = 6.0f, kDepthBlockSlack = 3.0f;  // below a wave's maximum; of that below the chunk's
+constexpr float kDepthMassReach = kDepthWaveReach + kDepthBlockSlack;
 __device__ __forceinline__ float nucleus_depth(mi355x_sample_params prm, int vocab, float mass) {
   float d = 105.0f;
   if (prm.p <= 0.0f) d = 0.0f;
@@ -697,8 +698,42 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     static_assert(kLargeKMax <= 4 * kSBlock && kSMaxWaves * kWaveListCap * sizeof(u64) >= 4 * kSBlock * sizeof(uint32_t),
                   "four offers per thread, sorted as 32-bit keys in the hit lists' LDS");
     constexpr bool large_k = LARGEK;
-    const uint32_t cmax = block_max<uint32_t>(lmax, sm.wave_val);
+    uint32_t cmax = 0u;
     float thr = -__builtin_inff();
+    if constexpr (!LARGEK) {
+      // The chunk's maximum and, with it, the mass of the chunk's elements near that maximum, which bounds the prefix
+      // of everything deeper (any element of the row that lies deeper than this chunk's threshold follows them in
+      // rank order) and so moves the threshold up.  One exchange between the waves serves both: a wave sums
+      // exp((s - its own maximum)/T) over its elements within kDepthWaveReach of that maximum (whole-wave tests
+      // skip the exponentials where no lane has such an element: hardly any has), and the waves whose maximum lies
+      // within kDepthBlockSlack of the chunk's contribute, rescaled.
+      const uint32_t wkey = wave_max<uint32_t>(lmax);
+      const float fw = key_to_float(wkey), inv_t = 1.0f / prm.temperature;  // (no number in the wave: NaN, every test fails)
+      const float lim = fw - kDepthWaveReach * prm.temperature;
+      float near = 0.0f;
+#pragma unroll
+      for (int e = 0; e < kSElems; ++e) {
+        const bool in = v[e] >= lim;
+        if (__ballot(in) != 0ull) near += in ? __expf((v[e] - fw) * inv_t) : 0.0f;
+      }
+      for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
+        const float ev = i0 + tid < n_extra ? sm.extra_val[i0 + tid] : kNaN;
+        near += ev >= lim ? __expf((ev - fw) * inv_t) : 0.0f;
+      }
+      near = wave_sum<float>(near);
+      if (lane == 0) sm.wave_val64[wave] = (static_cast<u64>(wkey) << 32) | __float_as_uint(near);
+      lds_barrier();
+      const u64 of_wave = lane < kSWaves ? sm.wave_val64[lane] : 0;
+      cmax = wave_max<uint32_t>(static_cast<uint32_t>(of_wave >> 32));
+      const float fcmax = key_to_float(cmax);
+      const float below = (key_to_float(static_cast<uint32_t>(of_wave >> 32)) - fcmax) * inv_t;
+      const float mass =
+          wave_sum<float>(below >= -kDepthBlockSlack ? __uint_as_float(static_cast<uint32_t>(of_wave)) * __expf(below) : 0.0f);
+      lds_barrier();
+      if (cmax != 0u) thr = fcmax - nucleus_depth(prm, V, mass);
+    } else {
+      cmax = block_max<uint32_t>(lmax, sm.wave_val);
+    }
     if (large_k) {
       const int kk = prm.k < V ? prm.k : V;
       if (kk <= kLargeKOneOffer) {
@@ -736,29 +771,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
         if (kth != 0u) thr = key_to_float(kth);
         __syncthreads();
       }
-    } else if (cmax != 0u) {
-      // the chunk's own elements near its maximum bound the prefix of everything deeper (any element of the row that
-      // lies deeper than this chunk's threshold follows them in rank order), which moves the threshold up
-      const float fcmax = key_to_float(cmax), inv_t = 1.0f / prm.temperature;
-      float near = 0.0f;
-#pragma unroll
-      for (int e = 0; e < kSElems; ++e) {
-        const float d = (v[e] - fcmax) * inv_t;
-        near += d >= -kDepthMassReach ? __expf(d) : 0.0f;  // (false for NaN)
-      }
-      for (uint32_t i = tid; i < n_extra; i += kSBlock) {
-        const float d = (sm.extra_val[i] - fcmax) * inv_t;
-        near += d >= -kDepthMassReach ? __expf(d) : 0.0f;
-      }
-      near = wave_sum<float>(near);
-      float* const wave_part = reinterpret_cast<float*>(sm.wave_val);
-      if (lane == 0) wave_part[wave] = near;
-      lds_barrier();
-      float mass = 0.0f;
-#pragma unroll
-      for (int w = 0; w < kSWaves; ++w) mass += wave_part[w];
-      lds_barrier();
-      thr = fcmax - nucleus_depth(prm, V, mass);
     }
     // First pass: the wave's number of candidates.
     uint32_t wcnt = 0u;
