@@ -118,9 +118,82 @@ struct SortInGlobalMemory {
   __device__ void operator()(u64* keys, int n2, int) const { block_sort_desc(keys, n2); }
 };
 
+// LDS for select_topk_desc: a list of kSelectCap keys, one word per thread, a few counters.
+constexpr int kSelectCap = 2048;
+struct TopkSelectLds {
+  u64* list;
+  uint32_t* maxima;  // blockDim.x words
+  uint32_t* words;   // 4 + blockDim.x / 64 words
+};
+
+// The kk (1 .. 64) largest of the n distinct keys of a row, key i belonging to id i (so that, among keys of one score,
+// a lower index is a larger key), sorted descending into s.list[0 .. kk): what a row that asks for its k best
+// needs of the full sort, at the cost of four passes over the keys.  The kk-th largest of the threads' best scores
+// is a score that at least kk keys reach; the keys above it are listed as they are found (fewer than kk of them,
+// unless threads hold several), and of the keys that tie with it -- all the masked ids of a row, for one -- the
+// first ones in index order fill up the kk, found by counting ties wave by wave over contiguous runs of indices.
+// Returns false, with nothing decided, when more than kSelectCap keys lie above that score.  Run by a whole block
+// (a power of two of threads, at least 64); contains barriers.
+__device__ __forceinline__ bool select_topk_desc(const u64* keys, int n, int kk, const TopkSelectLds& s) {
+  const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6, nw = static_cast<int>(blockDim.x) >> 6;
+  uint32_t best = 0u;
+  for (int i = tid; i < n; i += blockDim.x) {
+    const uint32_t score = key64_okey(keys[i]);
+    best = score > best ? score : best;
+  }
+  s.maxima[tid] = best;
+  if (tid == 0) s.words[0] = 0u;
+  __syncthreads();
+  block_sort_desc(s.maxima, static_cast<int>(blockDim.x));
+  const uint32_t tau = s.maxima[kk - 1];
+  const int seg = ((n + nw - 1) / nw + 63) & ~63;  // wave w owns the indices w * seg .. (w + 1) * seg - 1
+  const int lo = wave * seg, hi = lo + seg < n ? lo + seg : n;
+  uint32_t ties = 0u;
+  for (int i0 = lo; i0 < hi; i0 += 64) {
+    const int i = i0 + lane;
+    const u64 k = i < hi ? keys[i] : 0;
+    const bool above = i < hi && key64_okey(k) > tau;
+    const u64 ab = __ballot(above);
+    if (ab != 0ull) {
+      uint32_t base = 0u;
+      if (lane == 0) base = atomicAdd(&s.words[0], static_cast<uint32_t>(__popcll(ab)));
+      base = __builtin_amdgcn_readfirstlane(base);
+      const uint32_t pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(ab >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(ab), base));
+      if (above && pos < static_cast<uint32_t>(kSelectCap)) s.list[pos] = k;
+    }
+    ties += static_cast<uint32_t>(__popcll(__ballot(i < hi && key64_okey(k) == tau)));
+  }
+  if (lane == 0) s.words[4 + wave] = ties;
+  __syncthreads();
+  const uint32_t n_above = s.words[0];
+  if (n_above > static_cast<uint32_t>(kSelectCap)) return false;
+  uint32_t n_list = n_above;
+  if (n_above < static_cast<uint32_t>(kk)) {
+    const uint32_t want = static_cast<uint32_t>(kk) - n_above;  // at least that many keys tie
+    uint32_t run = 0u;
+    for (int w = 0; w < wave; ++w) run += s.words[4 + w];
+    for (int i0 = lo; i0 < hi && run < want; i0 += 64) {
+      const int i = i0 + lane;
+      const u64 k = i < hi ? keys[i] : 0;
+      const bool tie = i < hi && key64_okey(k) == tau;
+      const u64 tb = __ballot(tie);
+      const uint32_t rank = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(tb >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(tb), run));
+      if (tie && rank < want) s.list[n_above + rank] = k;
+      run += static_cast<uint32_t>(__popcll(tb));
+    }
+    n_list = static_cast<uint32_t>(kk);
+  }
+  const int n2 = next_pow2(static_cast<int>(n_list));  // (at least 64)
+  for (int i = static_cast<int>(n_list) + tid; i < n2; i += blockDim.x) s.list[i] = 0;
+  __syncthreads();
+  block_sort_desc(s.list, n2);
+  return true;
+}
+
 template <typename InT, typename SortFn = SortInGlobalMemory, int EPI_ITEMS = 4>
 __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const void* row0, const mi355x_sample_params prm,
-                                            u64* scratch, SeqShared& sh, SortFn sort_desc = SortFn{}) {
+                                            u64* scratch, SeqShared& sh, SortFn sort_desc = SortFn{},
+                                            const TopkSelectLds* select = nullptr) {
   const int V = a.vocab;
   const RowPtr<InT> lrow(row0, a.dtype);
   const int n2 = next_pow2(V);
@@ -166,24 +239,35 @@ __device__ __forceinline__ void general_row(const SampleArgs& a, int row, const 
     }
     __syncthreads();
   }
-  sort_desc(scratch, n2, V);  // descending; entries from V on are 0
+  // A row that asks for its k best (k <= 64) has them selected where the kernel provides the LDS for it; every other
+  // row is sorted whole.  `sc`: the row's keys in descending order, as many as the row's parameters ask for.
+  const u64* sc = scratch;
+  int n_sorted = V;
+  {
+    const int kk = prm.k < V ? prm.k : V;
+    if (select != nullptr && (a.emit_topk != 0 || prm.k > 1) && kk >= 1 && kk <= 64 && select_topk_desc(scratch, V, kk, *select)) {
+      sc = select->list;
+      n_sorted = kk;
+    } else {
+      sort_desc(scratch, n2, V);  // descending; entries from V on are 0
+    }
+  }
   if (a.emit_topk) {
     const int kk = prm.k < V ? prm.k : V;
     for (int j = threadIdx.x; j < kk; j += blockDim.x) {
-      const uint32_t id = key64_index(scratch[j]);
+      const uint32_t id = key64_index(sc[j]);
       a.out_tokens[static_cast<size_t>(row) * prm.k + j] = static_cast<int32_t>(id);
       if (a.out_scores) a.out_scores[static_cast<size_t>(row) * prm.k + j] = lrow[id];  // the value itself: keys do not tell -0 from +0
     }
     if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
     return;
   }
-  const float max_score = key_to_float(key64_okey(scratch[0]));
+  const float max_score = key_to_float(key64_okey(sc[0]));
   const float inv_temp = 1.0f / prm.temperature;
   const RowOutputs out = row_outputs(a, row);
-  const u64* sc = scratch;
   auto sorted = [=](int i) { return sc[i]; };
   auto exps = [=](int i) { return em::expf_exact((key_to_float(key64_okey(sc[i])) - max_score) * inv_temp); };
-  block_sample_epilogue<EPI_ITEMS>(sorted, exps, V, V, prm, a.uniforms[row], out, sh);
+  block_sample_epilogue<EPI_ITEMS>(sorted, exps, n_sorted, V, prm, a.uniforms[row], out, sh);
   if (threadIdx.x == 0) atomicAdd(a.fallback_rows, 1u);
 }
 
@@ -840,18 +924,25 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       if (any) fbk = order_key(-__builtin_inff());
     }
     const uint32_t ebk = key64_okey(extra_below);
-    const uint32_t bbk = block_max_lds<kSWaves, uint32_t>(fbk > ebk ? fbk : ebk, sm.wave_val);
-    u64 best_below = ebk == bbk ? extra_below : 0;
-    if (bbk != 0u && fbk == bbk) {
-      const float bbf = key_to_float(bbk);
-      int fe = 0;
+    const uint32_t own = fbk > ebk ? fbk : ebk;
+    const uint32_t wbk = wave_max<uint32_t>(own);  // (the wave first: one exchange between the waves, of whole keys)
+    u64 best_below = 0;
+    if (wbk != 0u && own == wbk) {
+      best_below = ebk == wbk ? extra_below : 0;
+      if (fbk == wbk) {
+        const float bbf = key_to_float(wbk);
+        int fe = 0;
 #pragma unroll
-      for (int e = kSElems - 1; e >= 0; --e)
-        if (v[e] == bbf) fe = e;
-      const u64 key = make_key64(bbk, static_cast<uint32_t>(elem_index<kSBlock, VEC>(chunk, fe >> 2, fe & 3)));
-      best_below = key > best_below ? key : best_below;
+        for (int e = kSElems - 1; e >= 0; --e)
+          if (v[e] == bbf) fe = e;
+        const u64 key = make_key64(wbk, static_cast<uint32_t>(elem_index<kSBlock, VEC>(chunk, fe >> 2, fe & 3)));
+        best_below = key > best_below ? key : best_below;
+      }
     }
-    best_below = block_max_lds<kSWaves, u64>(best_below, sm.wave_val64);  // its barriers also order the atomics on sm.count
+    best_below = wave_max<u64>(best_below);
+    if (lane == 0) sm.wave_val64[wave] = best_below;
+    lds_barrier();  // (also orders the atomics on sm.count)
+    best_below = wave_max<u64>(lane < kSWaves ? sm.wave_val64[lane] : 0);
     if (tid == 0) {
       const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
       a.chunk_cnt[ci] = extra_overflow ? kChunkCntOverflow : sm.count;
@@ -1393,7 +1484,10 @@ __device__ __forceinline__ void sample_fused_body(const SampleArgs& a) {
     // Rows the fast paths decline end here, in the exact general path (a single inlined call site keeps
     // the argument block in scalar registers instead of a scratch copy).
     __syncthreads();
-    general_row<InT>(a, row, row0, prm, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq);
+    static_assert(sizeof(sm.wave_list) >= kSelectCap * sizeof(u64) && sizeof(sm.lists) >= kTopkBlock * sizeof(uint32_t) &&
+                      sizeof(sm.pool) >= (4 + kTopkBlock / 64) * sizeof(uint32_t), "the selection's LDS");
+    const TopkSelectLds select{sm.wave_list, reinterpret_cast<uint32_t*>(sm.lists), sm.pool};
+    general_row<InT>(a, row, row0, prm, a.big + static_cast<size_t>(row) * a.big_stride, sm.seq, SortInGlobalMemory{}, &select);
   }
 }
 

@@ -356,6 +356,34 @@ def test_sample_ties_and_degenerate_rows(ctx, orc):
     sample_and_check(ctx, orc, x, u, 10, 0.0, 1.0)
 
 
+@pytest.mark.parametrize("vocab,k", [(128256, 50), (70000, 64), (40000, 2), (128256, 1)])
+def test_rows_that_tie_at_their_kth_score_are_selected_not_sorted(ctx, orc, vocab, k):
+    """Rows whose k best cannot be told from a chunk's bound -- all ids masked to lowest() but a few, NaNs needed to
+    fill the k, one score shared by thousands of ids, a few large values in one thread's run of ids -- leave the
+    single-pass path inside the streaming kernel; there the k best are selected exactly (the keys above the k-th
+    score, then the first ties in id order) and the tokens, kept ids and probabilities equal the oracle's."""
+    say("sample selection", vocab, k)
+    rng = np.random.default_rng(vocab + k)
+    rows = 6
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    x[0, :] = LOWEST
+    x[0, rng.integers(0, vocab, 5)] = [0.0, 1.0, -1.0, 0.5, 0.25]
+    x[1, :] = np.nan
+    x[1, rng.integers(0, vocab, 20)] = rng.standard_normal(20).astype(np.float32)
+    x[2, :] = 1.5
+    x[3, : vocab // 2] = 7.0   # above everything else: half the row ties for every place
+    x[4, 1000:1200] = 40.0 + rng.standard_normal(200).astype(np.float32)  # the best 200 in consecutive ids
+    u = rng.random(rows)
+    before = ctx.fallback_rows()
+    if k == 1:
+        got = ctx.argmax(torch.from_numpy(x).cuda()).cpu().numpy()
+        assert np.array_equal(got, orc.argmax_batch(x))
+    else:
+        sample_and_check(ctx, orc, x, u, k, 0.9, 0.7)
+        sample_and_check(ctx, orc, x, u, k, 0.0, 1.0)
+        assert ctx.fallback_rows() > before  # (rows 0 and 1 at least cannot stay on the single-pass path)
+
+
 @pytest.mark.parametrize("vocab", [2, 70, 5000, 40000])
 def test_sample_rows_without_finite_logits(ctx, orc, vocab):
     """A row of -inf logits (everything masked, then a penalty above 1 applied to lowest()) has NaN
