@@ -367,6 +367,15 @@ struct SortWithTile {
 // (i ^ (i >> 4)) & 7, which spreads those reads over all banks.
 __device__ __forceinline__ uint32_t exp_slot(uint32_t i) { return (i & ~7u) | ((i ^ (i >> 4)) & 7u); }
 
+// Where DeviceInterface::TopKScores wants a row's k best: ids and raw scores, best first (tokens null: not asked for).
+struct EmitTopk {
+  int32_t* tokens = nullptr;
+  float* scores = nullptr;
+  const void* row0 = nullptr;  // the row's logits, of type dtype
+  int dtype = 0;
+  __device__ __forceinline__ bool on() const { return tokens != nullptr; }
+};
+
 // The tail shared by the finish kernels: lds_keys[0 .. n_c) hold a row's candidates as key64s in any order,
 // best_below (0: none) is the best element of the row that is not among them.  Sorts them together in LDS,
 // caches the exponentials and runs the exact epilogue.  With cut_at_best_below the candidates that rank
@@ -377,13 +386,24 @@ __device__ __forceinline__ uint32_t exp_slot(uint32_t i) { return (i & ~7u) | ((
 __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucket_start, uint32_t n_c, u64 best_below,
                                                   uint32_t rmax, uint32_t thr, bool cut_at_best_below,
                                                   mi355x_sample_params prm, int V, double u, const RowOutputs& out,
-                                                  SeqShared& seqsh, uint32_t* red32, const SampleArgs* emit = nullptr,
-                                                  int emit_row = 0, const void* emit_row0 = nullptr, bool presorted = false) {
+                                                  SeqShared& seqsh, uint32_t* red32, EmitTopk emit = EmitTopk{},
+                                                  bool presorted = false) {
   const int tid = threadIdx.x;
   const u64* lk = lds_keys;
   auto sorted = [=](int i) { return lk[exp_slot(static_cast<uint32_t>(i))]; };
   auto exps = [=](int i) { return __uint_as_float(static_cast<uint32_t>(lk[exp_slot(static_cast<uint32_t>(i))] >> 32)); };
   // (presorted: the list is sorted and carries its exponentials already; one call of the epilogue serves both cases)
+  if (presorted && emit.on()) {
+    const int kk = prm.k < V ? prm.k : V;
+    if (n_c < static_cast<uint32_t>(kk)) return false;
+    const RowPtr<AnyDtype> lrow(emit.row0, emit.dtype);
+    for (int j = tid; j < kk; j += blockDim.x) {
+      const uint32_t id = key64_index(lk[exp_slot(static_cast<uint32_t>(j))]);
+      emit.tokens[j] = static_cast<int32_t>(id);
+      emit.scores[j] = lrow[id];
+    }
+    return true;
+  }
   if (!presorted) {
   if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
   if (best_below != 0) n_c += 1;
@@ -405,16 +425,16 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
       default: block_sort_desc_regs<16>(lds_keys); break;
     }
   }
-  if (emit) {
+  if (emit.on()) {
     // DeviceInterface::TopKScores: the k best ids and their raw scores, best first (the value itself is read again:
     // keys do not tell -0 from +0); fewer than k numbers among the candidates: the exact path decides
     const int kk = prm.k < V ? prm.k : V;
     if (n_c < static_cast<uint32_t>(kk) || lds_keys[kk - 1] == 0) return false;
-    const RowPtr<AnyDtype> lrow(emit_row0, emit->dtype);
+    const RowPtr<AnyDtype> lrow(emit.row0, emit.dtype);
     for (int j = tid; j < kk; j += blockDim.x) {
       const uint32_t id = key64_index(lds_keys[j]);
-      emit->out_tokens[static_cast<size_t>(emit_row) * prm.k + j] = static_cast<int32_t>(id);
-      emit->out_scores[static_cast<size_t>(emit_row) * prm.k + j] = lrow[id];
+      emit.tokens[j] = static_cast<int32_t>(id);
+      emit.scores[j] = lrow[id];
     }
     return true;
   }
@@ -590,17 +610,18 @@ struct TrimmedBuckets {
 // of buckets: it only has to be a bound, the epilogue decides on exact values and reports a nucleus that does not end
 // among the entries it is given), so the buckets past that point need neither places nor ranks; and no more buckets
 // are kept than fill room - 2 entries.  best_below: this thread's best element below the threshold (0: none); when
-// every bucket is kept, the block's best such element follows the candidates.  Contains barriers; every thread gets
-// the same result.
+// every bucket is kept, the block's best such element follows the candidates.  want > 0: the row asks for its `want`
+// best keys, whatever their mass: the kept buckets end with the thread's run that holds the want-th key.  Contains
+// barriers; every thread gets the same result.
 __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start, const ScoreBuckets& bucket_of, u64 best_below,
                                                                 mi355x_sample_params prm, int V, int room, uint32_t* red32,
-                                                                u64* red64) {
+                                                                u64* red64, int want = 0) {
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   // exclusive scan of the counts (consecutive buckets per thread) with a lower bound of the mass next to it: every
   // key of bucket b weighs at least exp(-(b + 1) * step) times the weight of `top`
   constexpr int kPer = kSortBuckets / kFinishBlock;
   const float step = bucket_of.scale > 0.0f ? (1.0f / prm.temperature) / bucket_of.scale : 0.0f;  // exponent per bucket
-  const bool trim = prm.p > 0.0f && prm.p < 1.0f && bucket_of.scale > 0.0f;
+  const bool trim = want == 0 && prm.p > 0.0f && prm.p < 1.0f && bucket_of.scale > 0.0f;
   const float ratio = __expf(-step);
   float edge = __expf(-static_cast<float>(t * kPer + 1) * step);
   uint32_t cnt[kPer], local = 0u, big = 0u;
@@ -635,6 +656,7 @@ __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start,
     if (m * (1.0f - pf) >= 1.02f * pf * static_cast<float>(static_cast<uint32_t>(V) - c) * __expf(-static_cast<float>(t * kPer - 1) * step))
       mine = static_cast<uint32_t>(t);
   }
+  if (want > 0 && c < static_cast<uint32_t>(want) && c + local >= static_cast<uint32_t>(want)) mine = static_cast<uint32_t>(t);
   if (c + local > static_cast<uint32_t>(room - 2)) {
     if (t == 0) big = 1u;
     else mine = static_cast<uint32_t>(t - 1) < mine ? static_cast<uint32_t>(t - 1) : mine;
@@ -741,8 +763,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     const int c = q >> head_shift, u = q & ((1 << head_shift) - 1);
     pre[q] = (a.chunks <= kAheadChunks && c < a.chunks) ? big_row[static_cast<size_t>(c) * kSChunk + u * kFinishBlock + tid] : 0;
   }
-  if (!large_k)  // the sort's table, while the loads are on their way
-    for (int b = tid; b <= kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;
+  for (int b = tid; b <= kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;  // the sort's table, while the loads are on their way
   // Thread c reads everything chunk c left behind; the barriers of the first reduction publish the counts.
   __shared__ uint32_t sh_cnt[kAllCap / kSmallCap];       // candidates per chunk
   __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // their prefix sums
@@ -753,7 +774,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   if (tid < a.chunks) {
     const uint32_t cnt = a.chunk_cnt[cbase + tid];
     m = cnt == kChunkCntOverflow ? 0xffffffffu : a.chunk_max[cbase + tid];  // above every key: the exact path
-    cthr = large_k ? 0u : a.chunk_thr[cbase + tid];
+    cthr = a.chunk_thr[cbase + tid];
     best_below = large_k ? 0 : a.chunk_next[cbase + tid];
     sh_cnt[tid] = cnt;
   }
@@ -761,9 +782,9 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   const uint32_t rmax = block_max<uint32_t>(m, red32);
   const bool gave_up = rmax == 0xffffffffu;
   // Every chunk's threshold holds for the whole row (no element of the row below it lies strictly inside the
-  // nucleus), so the highest one is the row's: every element at or above it is in its chunk's list.
-  uint32_t thr = 0u;
-  if (!large_k) thr = block_max<uint32_t>(cthr, red32);
+  // nucleus; a chunk alone has k elements at or above its own), so the highest one is the row's: every element at
+  // or above it is in its chunk's list.
+  uint32_t thr = block_max<uint32_t>(cthr, red32);
   if (rmax == 0u) thr = 0u;  // (no number in the row)
   if (tid == 0) {
     uint32_t all = 0u;
@@ -843,7 +864,8 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // the row to the steps below: the list in LDS, trimmed, and the sorting network.
   bool presorted = false, ok = false;
   uint32_t n_c = 0u;
-  if (!large_k && !gave_up && rmax != 0u) {
+  const int k_wanted = large_k ? (prm.k < V ? prm.k : V) : 0;
+  if (!gave_up && rmax != 0u) {
     const ScoreBuckets bucket_of(rmax, thr);  // (the table is zero: cleared at the start, barriers since)
     const float thr_score = key_to_float(thr);
     u64 below = best_below;
@@ -862,8 +884,8 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       }
     });
     __syncthreads();
-    const TrimmedBuckets kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, kNucleusCap, red32, red64);
-    if (kept.n != 0u) {
+    const TrimmedBuckets kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, kNucleusCap, red32, red64, k_wanted);
+    if (kept.n != 0u && kept.n_sorted >= static_cast<uint32_t>(k_wanted)) {  // (fewer than k numbers listed: the steps below decide)
       listed_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t used) {
 #pragma unroll
         for (int u = 0; u < kGather; ++u) {
@@ -979,9 +1001,11 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   }
   if (ok) {
     const bool emit = large_k && a.emit_topk == 1;
+    EmitTopk target;  // (by value: a pointer to the kernel's arguments would put all of them on the stack)
+    if (emit) target = EmitTopk{a.out_tokens + static_cast<size_t>(row) * prm.k, a.out_scores + static_cast<size_t>(row) * prm.k,
+                                row_start<INLINE>(a, row, dtype_bytes(a.dtype)), a.dtype};
     ok = finish_candidates(lds_keys, bucket_start, n_c, presorted ? 0 : best_below, rmax, thr, false, prm, V,
-                           emit ? 0.0 : a.uniforms[row], row_outputs(a, row), seqsh, red32, emit ? &a : nullptr, row,
-                           emit ? row_start<INLINE>(a, row, dtype_bytes(a.dtype)) : nullptr, presorted);
+                           emit ? 0.0 : a.uniforms[row], row_outputs(a, row), seqsh, red32, target, presorted);
   }
   if (!ok) {
     __syncthreads();
@@ -1363,7 +1387,7 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   n_c = sh_count;
   }
   return leave(finish_candidates(lds_keys, bucket_start, n_c, presorted ? 0 : best_below, rmax, thr, false, prm, V, a.uniforms[row],
-                                 row_outputs(a, row), seqsh, red32, nullptr, 0, nullptr, presorted));
+                                 row_outputs(a, row), seqsh, red32, EmitTopk{}, presorted));
 }
 
 template <bool INLINE>

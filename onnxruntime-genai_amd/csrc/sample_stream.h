@@ -520,6 +520,56 @@ __device__ __forceinline__ T block_max_lds(T v, T* scratch) {
   return r;
 }
 
+// The kk-th largest of the values the block's threads offer (N per thread; 1 <= kk <= N * blockDim.x), every thread
+// gets it: a radix selection from the top bits down, four bits a round.  A wave counts its offers that still match
+// the bits found so far, digit by digit, with whole-wave tests (no sorting, no contended atomics: sixteen lanes add
+// the wave's sixteen counts to the round's bins), and after one barrier every thread reads the round's bins and
+// picks the digit.  bins: 128 words of LDS that no thread uses for anything else until the function returns.
+template <int N>
+__device__ __forceinline__ uint32_t block_kth_largest(const uint32_t (&offer)[N], int kk, uint32_t* bins) {
+  const int tid = threadIdx.x, lane = lane_id();
+  if (tid < 128) bins[tid] = 0u;
+  lds_barrier();
+  uint32_t prefix = 0u, need = static_cast<uint32_t>(kk);
+#pragma unroll
+  for (int round = 0; round < 8; ++round) {
+    const int shift = 28 - 4 * round;
+    const uint32_t above_bits = round == 0 ? 0u : ~0u << (shift + 4);
+    bool match[N];
+    uint32_t digit[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      match[j] = ((offer[j] ^ prefix) & above_bits) == 0u;
+      digit[j] = (offer[j] >> shift) & 15u;
+    }
+    uint32_t mine = 0u;
+#pragma unroll
+    for (uint32_t d = 0; d < 16u; ++d) {
+      uint32_t c = 0u;
+#pragma unroll
+      for (int j = 0; j < N; ++j) c += static_cast<uint32_t>(__popcll(__ballot(match[j] && digit[j] == d)));
+      mine = static_cast<uint32_t>(lane) == d ? c : mine;
+    }
+    if (lane < 16 && mine != 0u) atomicAdd(&bins[round * 16 + lane], mine);
+    lds_barrier();
+    uint32_t above = 0u, pick = 0u;
+    bool found = false;
+#pragma unroll
+    for (int d = 15; d >= 0; --d) {
+      const uint32_t c = bins[round * 16 + d];
+      if (!found && above + c >= need) {
+        pick = static_cast<uint32_t>(d);
+        found = true;
+      }
+      if (!found) above += c;
+    }
+    need -= above;
+    prefix |= pick << shift;
+  }
+  lds_barrier();  // (the bins are free again)
+  return prefix;
+}
+
 // Applies the two LDS bitmaps of a chunk to the registers of a thread: an id whose bit in `allowed` is
 // clear becomes kLowest, an id whose bit in `history` is set becomes NaN (its processed value lives in
 // the extras list).  Branch-free: the bit, spread over a word, selects between the two bit patterns.
@@ -820,14 +870,11 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     }
     if (large_k) {
       const int kk = prm.k < V ? prm.k : V;
+      uint32_t* const bins = reinterpret_cast<uint32_t*>(sm.wave_list);
+      uint32_t kth;
       if (kk <= kLargeKOneOffer) {
-        u64* scratch = sm.wave_list;
-        scratch[tid] = static_cast<u64>(lmax);
-        __syncthreads();
-        block_sort_desc(scratch, kSBlock);
-        const uint32_t kth = static_cast<uint32_t>(scratch[kk - 1]);
-        if (kth != 0u) thr = key_to_float(kth);
-        __syncthreads();
+        const uint32_t offer[1] = {lmax};
+        kth = block_kth_largest<1>(offer, kk, bins);
       } else {
         // the four best elements of every thread (registers and its share of the history ids' list), as order
         // keys: at least k elements reach the k-th best of those offers, or fewer than k exist and all are kept
@@ -846,15 +893,9 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
 #pragma unroll
         for (int e = 0; e < kSElems; ++e) offer(v[e]);
         for (uint32_t i = tid; i < n_extra; i += kSBlock) offer(sm.extra_val[i]);
-        uint32_t* offers = reinterpret_cast<uint32_t*>(sm.wave_list);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) offers[tid * 4 + q] = best[q];
-        __syncthreads();
-        block_sort_desc(offers, 4 * kSBlock);
-        const uint32_t kth = offers[kk - 1];
-        if (kth != 0u) thr = key_to_float(kth);
-        __syncthreads();
+        kth = block_kth_largest<4>(best, kk, bins);
       }
+      if (kth != 0u) thr = key_to_float(kth);
     }
     // First pass: the wave's number of candidates.
     uint32_t wcnt = 0u;
