@@ -356,6 +356,95 @@ def test_sample_ties_and_degenerate_rows(ctx, orc):
     sample_and_check(ctx, orc, x, u, 10, 0.0, 1.0)
 
 
+def test_sparse_mask_rows_with_heavy_ties(ctx, orc):
+    """Nucleus rows under a sparse mask whose allowed logits are quantised (hundreds of ids per score, more than a
+    bucket of the counting sort holds), constant, or carry a block of equal values at the top: the row leaves the
+    bucket sort for the sorting network inside the same kernel; kept ids, probability bits and tokens equal the
+    oracle's, with and without the promise about the mask."""
+    say("sparse mask, heavy ties")
+    rng = np.random.default_rng(77)
+    rows, vocab = 5, 201088
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    x[0] = np.round(x[0] * 2) / 2
+    x[1] = np.round(x[1])
+    x[2, :] = np.float32(-1.25)
+    x[3, : vocab // 3] = np.float32(9.5)
+    mask = make_mask(rng, rows, vocab, 0.05)
+    allowed = np.unpackbits(mask.view(np.uint8), axis=1, bitorder="little")[:, :vocab].astype(bool)
+    hist = rng.integers(0, vocab, (rows, 300)).astype(np.int32)
+    u = rng.random(rows)
+    xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                           repetition_penalty=1.3)
+    proc = orc.apply_mask(x, mask)
+    cap = 16384
+    for promise in (0, int(allowed.sum(axis=1).max())):
+        xf.c.mask_allowed_max = promise
+        tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=0.9, temperature=1.0,
+                                     xf=xf, kept_capacity=cap)
+        tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+        for r in range(rows):
+            idx, probs = orc.sampled_categorical(orc.apply_repetition_penalty(proc[r], hist[r], 1.3), 0, 0.9, 1.0)
+            n = min(len(idx), cap)
+            assert kc[r] == len(idx), (promise, r, kc[r], len(idx))
+            assert np.array_equal(ki[r, :n], idx[:n]), (promise, r)
+            assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), (promise, r)
+            assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (promise, r)
+
+
+@pytest.mark.parametrize("sigma,p,t", [(4.0, 0.95, 1.0), (1.0, 0.9, 1.0), (5.0, 0.9, 1.0), (3.0, 0.5, 0.7)])
+def test_nucleus_rows_with_lists_near_and_beyond_the_sort(ctx, orc, sigma, p, t):
+    """Unmasked nucleus rows of 128256 ids whose chunks list a few thousand to tens of thousands of keys: nuclei that
+    fit the finish kernel's sort with room to spare, that fill it almost completely, and that exceed it (the exact
+    path takes those rows).  Kept counts, the first kept ids with their probability bits, and tokens equal the
+    oracle's."""
+    say("nucleus near the sort's capacity", sigma, p, t)
+    rng = np.random.default_rng(int(sigma * 10 + p * 100))
+    rows, vocab = 6, 128256
+    x = (rng.standard_normal((rows, vocab)) * sigma).astype(np.float32)
+    x[1] += np.float32(0.7)
+    x[2, : vocab // 2] -= np.float32(2.0)  # one half of the row lower: chunk thresholds differ
+    u = rng.random(rows)
+    cap = 4096
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=p, temperature=t,
+                                 kept_capacity=cap)
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    for r in range(rows):
+        idx, probs = orc.sampled_categorical(x[r], 0, p, t)
+        n = min(len(idx), cap)
+        assert kc[r] == len(idx), (r, kc[r], len(idx))
+        assert np.array_equal(ki[r, :n], idx[:n]), r
+        assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), r
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+
+
+@pytest.mark.parametrize("k", [100, 512, 2048])
+def test_large_k_rows_with_ties_nans_and_clustered_best_tokens(ctx, orc, k):
+    """Top-k rows with 64 < k <= 2048 at 128256 ids: fewer numbers than k (NaNs fill the rest), a score shared by
+    thousands of ids at the k-th place, the best tokens all in one chunk or in one thread's run of ids, one chunk
+    without a number.  Kept sets, probability bits and tokens equal the oracle's."""
+    say("large k, ties and NaNs", k)
+    rng = np.random.default_rng(k)
+    rows, vocab = 6, 128256
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    x[0, :] = np.nan
+    x[0, rng.integers(0, vocab, k // 2)] = rng.standard_normal(k // 2).astype(np.float32)
+    x[1] = np.round(x[1])
+    x[2, 40000:40000 + 3 * k] = 30.0 + rng.standard_normal(3 * k).astype(np.float32)
+    x[3, 70000:70032] = 50.0
+    x[4, 32768:65536] = np.nan
+    u = rng.random(rows)
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=k, p=0.9, temperature=0.8,
+                                 kept_capacity=2048)
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    for r in range(rows):
+        idx, probs = orc.sampled_categorical(x[r], k, 0.9, 0.8)
+        n = min(len(idx), 2048)
+        assert kc[r] == len(idx), (r, kc[r], len(idx))
+        assert np.array_equal(ki[r, :n], idx[:n]), r
+        assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), r
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+
+
 @pytest.mark.parametrize("vocab,k", [(128256, 50), (70000, 64), (40000, 2), (128256, 1)])
 def test_rows_that_tie_at_their_kth_score_are_selected_not_sorted(ctx, orc, vocab, k):
     """Rows whose k best cannot be told from a chunk's bound -- all ids masked to lowest() but a few, NaNs needed to
