@@ -521,52 +521,54 @@ __device__ __forceinline__ T block_max_lds(T v, T* scratch) {
 }
 
 // The kk-th largest of the values the block's threads offer (N per thread; 1 <= kk <= N * blockDim.x), every thread
-// gets it: a radix selection from the top bits down, four bits a round.  A wave counts its offers that still match
-// the bits found so far, digit by digit, with whole-wave tests (no sorting, no contended atomics: sixteen lanes add
-// the wave's sixteen counts to the round's bins), and after one barrier every thread reads the round's bins and
-// picks the digit.  bins: 128 words of LDS that no thread uses for anything else until the function returns.
+// gets it: a radix selection from the top byte down.  A round counts the offers that still match the bytes found so
+// far into 256 bins with LDS atomics (eight copies of every bin, chosen by the lane, so that offers sharing a byte --
+// all of them share the first -- do not queue on one word), 256 threads sum the copies of one bin each, scan the
+// sums from the top digit down and the thread whose bin holds the wanted rank publishes digit and rank.  No sort,
+// three barriers a round.  bins: kKthBinWords words of LDS that no thread uses for anything else until the function
+// returns; blockDim.x >= 256.
+constexpr int kKthBinCopies = 8, kKthBinWords = 256 * kKthBinCopies + 16;
 template <int N>
 __device__ __forceinline__ uint32_t block_kth_largest(const uint32_t (&offer)[N], int kk, uint32_t* bins) {
-  const int tid = threadIdx.x, lane = lane_id();
-  if (tid < 128) bins[tid] = 0u;
+  const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+  uint32_t* const wave_sum_of = bins + 256 * kKthBinCopies;  // [4], then the published digit and rank
+  uint32_t* const pick = wave_sum_of + 4;
+  for (int i = tid; i < 256 * kKthBinCopies; i += blockDim.x) bins[i] = 0u;
   lds_barrier();
   uint32_t prefix = 0u, need = static_cast<uint32_t>(kk);
 #pragma unroll
-  for (int round = 0; round < 8; ++round) {
-    const int shift = 28 - 4 * round;
-    const uint32_t above_bits = round == 0 ? 0u : ~0u << (shift + 4);
-    bool match[N];
-    uint32_t digit[N];
+  for (int round = 0; round < 4; ++round) {
+    const int shift = 24 - 8 * round;
 #pragma unroll
     for (int j = 0; j < N; ++j) {
-      match[j] = ((offer[j] ^ prefix) & above_bits) == 0u;
-      digit[j] = (offer[j] >> shift) & 15u;
+      const bool match = round == 0 || (offer[j] >> (shift + 8)) == (prefix >> (shift + 8));
+      if (match) atomicAdd(&bins[((offer[j] >> shift) & 255u) * kKthBinCopies + (lane & (kKthBinCopies - 1))], 1u);
     }
-    uint32_t mine = 0u;
-#pragma unroll
-    for (uint32_t d = 0; d < 16u; ++d) {
-      uint32_t c = 0u;
-#pragma unroll
-      for (int j = 0; j < N; ++j) c += static_cast<uint32_t>(__popcll(__ballot(match[j] && digit[j] == d)));
-      mine = static_cast<uint32_t>(lane) == d ? c : mine;
-    }
-    if (lane < 16 && mine != 0u) atomicAdd(&bins[round * 16 + lane], mine);
     lds_barrier();
-    uint32_t above = 0u, pick = 0u;
-    bool found = false;
+    uint32_t count = 0u, upto = 0u;
+    const uint32_t digit = 255u - static_cast<uint32_t>(tid);  // thread t owns digit 255 - t: a prefix sum counts the digits above
+    if (tid < 256) {
 #pragma unroll
-    for (int d = 15; d >= 0; --d) {
-      const uint32_t c = bins[round * 16 + d];
-      if (!found && above + c >= need) {
-        pick = static_cast<uint32_t>(d);
-        found = true;
-      }
-      if (!found) above += c;
+      for (int i = 0; i < kKthBinCopies; ++i) count += bins[digit * kKthBinCopies + i];
+      upto = wave_prefix_sum<uint32_t>(count);
+      if (lane == 63) wave_sum_of[wave] = upto;
     }
-    need -= above;
-    prefix |= pick << shift;
+    lds_barrier();
+    if (tid < 256) {
+      uint32_t above = upto - count;
+      for (int w = 0; w < wave; ++w) above += wave_sum_of[w];
+      if (above < need && need <= above + count) {
+        pick[0] = digit;
+        pick[1] = need - above;
+      }
+    }
+    if (round < 3)
+      for (int i = tid; i < 256 * kKthBinCopies; i += blockDim.x) bins[i] = 0u;  // (every read of this round's bins lies before the last barrier)
+    lds_barrier();
+    prefix |= pick[0] << shift;
+    need = pick[1];
   }
-  lds_barrier();  // (the bins are free again)
+  lds_barrier();  // (the words are free again)
   return prefix;
 }
 
@@ -826,11 +828,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     // the chunk's list with one LDS atomic and fills it; the slot of a candidate is the wave's running
     // count plus the number of candidate lanes below.
     // Rows with 64 < k <= kLargeKMax come here too: their candidates are the elements that reach the
-    // exact k-th best per-thread maximum of the chunk (at least k elements do; with fewer than k
-    // threads holding elements, all), which contain the chunk's k best.
-    static_assert(kLargeKOneOffer <= kSBlock && kSMaxWaves * kWaveListCap >= kSBlock, "one offer per thread, sorted in the hit lists' LDS");
-    static_assert(kLargeKMax <= 4 * kSBlock && kSMaxWaves * kWaveListCap * sizeof(u64) >= 4 * kSBlock * sizeof(uint32_t),
-                  "four offers per thread, sorted as 32-bit keys in the hit lists' LDS");
+    // k-th best of the chunk's per-thread maxima (or, for larger k, of the maxima of the quarters of every thread's
+    // elements: at least k elements do; with fewer than k numbers, all), which contain the chunk's k best.
+    static_assert(kLargeKOneOffer <= kSBlock && kLargeKMax <= 4 * kSBlock, "one offer per thread, or four");
+    static_assert(sizeof(sm.wave_list) >= kKthBinWords * sizeof(uint32_t) && kSBlock >= 256, "the selection's bins lie in the hit lists' LDS");
     constexpr bool large_k = LARGEK;
     uint32_t cmax = 0u;
     float thr = -__builtin_inff();
@@ -876,23 +877,19 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
         const uint32_t offer[1] = {lmax};
         kth = block_kth_largest<1>(offer, kk, bins);
       } else {
-        // the four best elements of every thread (registers and its share of the history ids' list), as order
-        // keys: at least k elements reach the k-th best of those offers, or fewer than k exist and all are kept
+        // the best element of each quarter of the thread's registers (its share of the history ids' list counts
+        // for the first), as order keys: at least k elements reach the k-th best of those offers, or fewer than k
+        // exist and all are kept
         uint32_t best[4] = {0u, 0u, 0u, 0u};
-        auto offer = [&](float x) {
-          uint32_t key = order_key(x);  // 0 for NaN: no element
-          if (key > best[3]) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const uint32_t hi = key > best[q] ? key : best[q];
-              key = key > best[q] ? best[q] : key;
-              best[q] = hi;
-            }
-          }
-        };
-#pragma unroll
-        for (int e = 0; e < kSElems; ++e) offer(v[e]);
-        for (uint32_t i = tid; i < n_extra; i += kSBlock) offer(sm.extra_val[i]);
+        for (int e = 0; e < kSElems; ++e) {
+          const uint32_t key = order_key(v[e]);  // 0 for NaN: no element
+          best[e / (kSElems / 4)] = key > best[e / (kSElems / 4)] ? key : best[e / (kSElems / 4)];
+        }
+        for (uint32_t i = tid; i < n_extra; i += kSBlock) {
+          const uint32_t key = order_key(sm.extra_val[i]);
+          best[0] = key > best[0] ? key : best[0];
+        }
         kth = block_kth_largest<4>(best, kk, bins);
       }
       if (kth != 0u) thr = key_to_float(kth);
