@@ -328,27 +328,35 @@ __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop
         }
       }
       if (walk) {
+        // From the exact prefix in front of the thread's elements the walk is the reference's own loop: real float
+        // additions, one per element (the step functions exist to compose runs in parallel; a thread that walks has
+        // its start).  A sum whose bit pattern reaches the next binade's first has left the binade.
+        const uint32_t lim = (static_cast<uint32_t>(st.se) << 23) + 0x800000u;
+        bool gone = nn >= kMantLimit;  // an earlier thread's element left the binade already
+        float s_run = seq_recompose(gone ? 0u : nn, st.se);
 #pragma unroll
         for (int j = 0; j < ITEMS; ++j) {
           const int idx = base + j;
           if (idx >= start && idx < wend) {
-            const uint32_t nn2 = step_apply(nn, seq_make_step(ev[j], st.se));
+            const float s_next = s_run + ev[j];
+            const bool leaves = gone || em::as_u32(s_next) >= lim;
             if (key == kNone) {
-              if (nn2 >= kMantLimit) {  // leaves the binade here (or an earlier thread's element did)
+              if (leaves) {  // leaves the binade here (or an earlier thread's element did)
                 key = (static_cast<uint32_t>(idx) << 1) | 1u;
-                pa = seq_recompose(nn < kMantLimit ? nn : 0u, st.se);
+                pa = s_run;
                 pb = ev[j];
               } else if (!kPlain) {
-                const float pf = seq_recompose(nn2, st.se);
-                if (stop(pf, ev[j], idx)) {
+                if (stop(s_next, ev[j], idx)) {
                   key = static_cast<uint32_t>(idx) << 1;
-                  pa = pf;
+                  pa = s_next;
                 }
               }
             }
-            nn = nn2;
+            gone = leaves;
+            s_run = s_next;
           }
         }
+        nn = gone ? kStepSat : seq_decompose(s_run).n;
       }
       if (wend - 1 >= base && wend - 1 < base + ITEMS) sh.n_last[par] = nn;
       const uint32_t wkey = wave_min_u32(key);
