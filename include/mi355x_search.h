@@ -156,7 +156,7 @@ int mi355x_argmax_static(void* stream, const void* logits, int dtype, int64_t ro
 /* Per-row k best (token id, raw fp32 score), best first: DeviceInterface::TopKScores
  * (src/smartptrs.h:254).  dtype MI355X_F32, MI355X_F16 or MI355X_BF16 (the scores of sixteen-bit rows are
  * the widened values).  out_tokens/out_scores: device [rows, k].  1 <= k <= vocab: up to 64 from the fused
- * kernel's candidate lists, up to 2048 from the candidate lists of the large-k sampling route, beyond that
+ * kernel's candidate lists, up to 8192 from the candidate lists of the large-k sampling route, beyond that
  * from the exact path's whole-row sort (the CUDA add-on serves any k as well, src/cuda/interface.cpp:503-553). */
 int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits, int dtype,
                        int64_t row_stride, int rows, int vocab, int k, int32_t* out_tokens,

@@ -31,7 +31,7 @@ constexpr int kModeTopkLarge = 3;  // 64 < k <= kLargeKMax: streamed and finishe
 // The per-chunk bound of such rows is the k-th best of what the 1024 threads of a nucleus workgroup offer: their
 // maxima up to k = 512 (tight up to half the threads: about 1.4 k elements reach it), their four best elements
 // each beyond that (about 1.1 k elements reach the k-th best of those 4096).
-constexpr int kLargeKMax = 2048;
+constexpr int kLargeKMax = 8192;
 constexpr int kLargeKOneOffer = 512;  // up to here one offer per thread is enough
 
 // Heterogeneous (k, p, T) of a batch of at most kInlineParamRows rows travel inside the kernel

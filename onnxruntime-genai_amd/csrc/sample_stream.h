@@ -830,7 +830,8 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     // Rows with 64 < k <= kLargeKMax come here too: their candidates are the elements that reach the
     // k-th best of the chunk's per-thread maxima (or, for larger k, of the maxima of the quarters of every thread's
     // elements: at least k elements do; with fewer than k numbers, all), which contain the chunk's k best.
-    static_assert(kLargeKOneOffer <= kSBlock && kLargeKMax <= 4 * kSBlock, "one offer per thread, or four");
+    static_assert(kLargeKOneOffer <= kSBlock && 4 * kLargeKOneOffer <= 4 * kSBlock && kLargeKMax <= kSChunk && kSElems % 4 == 0,
+                  "one offer per thread, four, or every element");
     static_assert(sizeof(sm.wave_list) >= kKthBinWords * sizeof(uint32_t) && kSBlock >= 256, "the selection's bins lie in the hit lists' LDS");
     constexpr bool large_k = LARGEK;
     uint32_t cmax = 0u;
@@ -877,20 +878,27 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
         const uint32_t offer[1] = {lmax};
         kth = block_kth_largest<1>(offer, kk, bins);
       } else {
-        // the best element of each quarter of the thread's registers (its share of the history ids' list counts
-        // for the first), as order keys: at least k elements reach the k-th best of those offers, or fewer than k
-        // exist and all are kept
-        uint32_t best[4] = {0u, 0u, 0u, 0u};
+        // the best element of each quarter of the thread's registers (up to k = 2048) or every element (a k that
+        // close to the number of offers would make a bound from maxima useless), as order keys; the thread's share
+        // of the history ids' list counts for the first.  At least k elements reach the k-th best of those offers,
+        // or fewer than k exist and all are kept
+        auto group_maxima = [&](auto groups) {
+          constexpr int G = decltype(groups)::value;
+          uint32_t best[G];
 #pragma unroll
-        for (int e = 0; e < kSElems; ++e) {
-          const uint32_t key = order_key(v[e]);  // 0 for NaN: no element
-          best[e / (kSElems / 4)] = key > best[e / (kSElems / 4)] ? key : best[e / (kSElems / 4)];
-        }
-        for (uint32_t i = tid; i < n_extra; i += kSBlock) {
-          const uint32_t key = order_key(sm.extra_val[i]);
-          best[0] = key > best[0] ? key : best[0];
-        }
-        kth = block_kth_largest<4>(best, kk, bins);
+          for (int q = 0; q < G; ++q) best[q] = 0u;
+#pragma unroll
+          for (int e = 0; e < kSElems; ++e) {
+            const uint32_t key = order_key(v[e]);  // 0 for NaN: no element
+            best[e / (kSElems / G)] = key > best[e / (kSElems / G)] ? key : best[e / (kSElems / G)];
+          }
+          for (uint32_t i = tid; i < n_extra; i += kSBlock) {
+            const uint32_t key = order_key(sm.extra_val[i]);
+            best[0] = key > best[0] ? key : best[0];
+          }
+          return block_kth_largest<G>(best, kk, bins);
+        };
+        kth = kk <= 4 * kLargeKOneOffer ? group_maxima(std::integral_constant<int, 4>{}) : group_maxima(std::integral_constant<int, kSElems>{});
       }
       if (kth != 0u) thr = key_to_float(kth);
     }

@@ -417,9 +417,9 @@ def test_nucleus_rows_with_lists_near_and_beyond_the_sort(ctx, orc, sigma, p, t)
         assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
 
 
-@pytest.mark.parametrize("k", [100, 512, 2048])
+@pytest.mark.parametrize("k", [100, 512, 2048, 6000])
 def test_large_k_rows_with_ties_nans_and_clustered_best_tokens(ctx, orc, k):
-    """Top-k rows with 64 < k <= 2048 at 128256 ids: fewer numbers than k (NaNs fill the rest), a score shared by
+    """Top-k rows with 64 < k <= 8192 at 128256 ids: fewer numbers than k (NaNs fill the rest), a score shared by
     thousands of ids at the k-th place, the best tokens all in one chunk or in one thread's run of ids, one chunk
     without a number.  Kept sets, probability bits and tokens equal the oracle's."""
     say("large k, ties and NaNs", k)
@@ -504,16 +504,17 @@ def test_sample_large_k_general_path(ctx, orc):
     (128256, 65, 0.9, 0.7, 0.0), (128256, 100, 1.0, 1.0, 0.0), (128256, 512, 0.95, 1.3, 0.0), (201088, 300, 0.0, 0.8, 0.0),
     (128256, 513, 0.95, 1.3, 0.0),  # from here four offers per thread bound the chunk
     (128256, 2048, 0.9, 1.0, 0.0), (201088, 2048, 0.0, 1.0, 0.0), (128256, 1500, 0.99, 0.8, 0.25), (5000, 2048, 0.9, 1.0, 0.0),
-    (128256, 2049, 0.95, 1.3, 0.0),  # beyond the limit of this route: the full-sort path
+    (128256, 2049, 0.95, 1.3, 0.0), (128256, 8192, 0.9, 1.0, 0.0), (201088, 5000, 0.0, 0.9, 0.0), (70000, 6000, 0.95, 1.1, 0.5),
+    (128256, 8193, 0.95, 1.3, 0.0),  # beyond the limit of this route: the full-sort path
     (33000, 100, 0.9, 1.0, 0.0),    # the short last chunk holds fewer than k threads' worth of elements
     (40000, 500, 0.99, 1.0, 0.25),  # ties across the cut
     (700, 500, 0.9, 1.0, 0.0),      # k close to the vocabulary
 ])
 def test_sample_large_k_through_the_candidate_lists(ctx, orc, vocab, k, p, t, quantum):
-    """Top-k rows with 64 < k <= 2048 are streamed like nucleus rows (candidates = elements at or above
-    the k-th best of the per-thread offers of their chunk: the maxima up to k = 512, the four best of every
-    thread beyond) and finished by the sorting kernel, not by the full-sort path; kept sets, probabilities
-    and tokens equal the oracle's."""
+    """Top-k rows with 64 < k <= 8192 are streamed like nucleus rows (candidates = elements at or above
+    the k-th best of the per-thread offers of their chunk: the maxima up to k = 512, beyond that the maxima of
+    the quarters or eighths of every thread's elements) and finished by the sorting kernel, not by the full-sort
+    path; kept sets, probabilities and tokens equal the oracle's."""
     say("sample large k", vocab, k, p, t, quantum)
     rng = np.random.default_rng(vocab + k)
     rows = 5
@@ -534,7 +535,7 @@ def test_sample_large_k_through_the_candidate_lists(ctx, orc, vocab, k, p, t, qu
         assert np.array_equal(ki[r, :n], idx[:n]), r
         assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), r
         assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
-    if k <= 2048 and not quantum:
+    if k <= 8192 and not quantum:
         assert ctx.fallback_rows() - before <= 1  # at most the constant row
 
 
