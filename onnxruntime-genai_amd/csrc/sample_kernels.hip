@@ -602,6 +602,9 @@ struct ScoreBuckets {
 struct TrimmedBuckets {
   uint32_t last_bucket, n_sorted, n;
   u64 best_below;
+  // not 0: the kept buckets end short of the bucket where the nucleus certainly ends, so the list does not hold the
+  // whole nucleus: 1: the room ends there, 2: the next thread's run has a bucket of more than bucket_cap keys
+  uint32_t more;
 };
 
 // After a counting pass has left the number of candidates per bucket in start[0 .. kSortBuckets): turns the counts
@@ -612,10 +615,10 @@ struct TrimmedBuckets {
 // are kept than fill room - 2 entries.  best_below: this thread's best element below the threshold (0: none); when
 // every bucket is kept, the block's best such element follows the candidates.  want > 0: the row asks for its `want`
 // best keys, whatever their mass: the kept buckets end with the thread's run that holds the want-th key.  Contains
-// barriers; every thread gets the same result.
+// barriers; every thread gets the same result.  bucket_cap: the most keys of one bucket the caller ranks.
 __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start, const ScoreBuckets& bucket_of, u64 best_below,
                                                                 mi355x_sample_params prm, int V, int room, uint32_t* red32,
-                                                                u64* red64, int want = 0) {
+                                                                u64* red64, int want = 0, int bucket_cap = kBucketCap) {
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   // exclusive scan of the counts (consecutive buckets per thread) with a lower bound of the mass next to it: every
   // key of bucket b weighs at least exp(-(b + 1) * step) times the weight of `top`
@@ -630,7 +633,7 @@ __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start,
   for (int i = 0; i < kPer; ++i) {
     cnt[i] = start[t * kPer + i];
     local += cnt[i];
-    big |= cnt[i] > static_cast<uint32_t>(kBucketCap) ? 1u : 0u;
+    big |= cnt[i] > static_cast<uint32_t>(bucket_cap) ? 1u : 0u;
     mass += static_cast<float>(cnt[i]) * edge;
     edge *= ratio;
   }
@@ -649,17 +652,20 @@ __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start,
   // (2 % to spare for the roundings); when b is empty, the element that satisfies the rule is the first one of the
   // next bucket that is not.  A thread tests the bucket before its own: the first thread that finds the property
   // there and has a key of its own owns the last buckets the sort keeps.  (Bucket 0 may hold keys above its upper
-  // edge: the test starts with thread 1.)  A thread whose buckets end beyond the room ends the kept ones before it.
-  uint32_t mine = static_cast<uint32_t>(kFinishBlock);
+  // edge: the test starts with thread 1.)  A thread whose buckets end beyond the room, or that has a bucket too full
+  // to rank, ends the kept ones before it.  (`mine` holds four times the thread that ends them, plus TrimmedBuckets::more:
+  // the lowest value wins, so the nucleus' own end goes first among equals.)
+  uint32_t mine = 4u * static_cast<uint32_t>(kFinishBlock);
   if (trim && t > 0 && local != 0u) {
     const float pf = prm.p;
     if (m * (1.0f - pf) >= 1.02f * pf * static_cast<float>(static_cast<uint32_t>(V) - c) * __expf(-static_cast<float>(t * kPer - 1) * step))
-      mine = static_cast<uint32_t>(t);
+      mine = 4u * static_cast<uint32_t>(t);
   }
-  if (want > 0 && c < static_cast<uint32_t>(want) && c + local >= static_cast<uint32_t>(want)) mine = static_cast<uint32_t>(t);
-  if (c + local > static_cast<uint32_t>(room - 2)) {
-    if (t == 0) big = 1u;
-    else mine = static_cast<uint32_t>(t - 1) < mine ? static_cast<uint32_t>(t - 1) : mine;
+  if (want > 0 && c < static_cast<uint32_t>(want) && c + local >= static_cast<uint32_t>(want)) mine = 4u * static_cast<uint32_t>(t);
+  if (c + local > static_cast<uint32_t>(room - 2) || big != 0u) {
+    const uint32_t before = 4u * static_cast<uint32_t>(t) - (big != 0u ? 2u : 3u);  // (thread t - 1, and why)
+    big = t == 0 ? 1u : 0u;
+    if (t != 0) mine = before < mine ? before : mine;
   }
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
@@ -668,9 +674,10 @@ __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start,
   }
   if (t == kFinishBlock - 1) start[kSortBuckets] = c;
   const uint32_t red = block_max<uint32_t>(big ? 0xffffffffu : ~mine, red32);  // its barriers also publish the starts
-  TrimmedBuckets r{static_cast<uint32_t>(kSortBuckets), n_cand, 0u, 0};
+  TrimmedBuckets r{static_cast<uint32_t>(kSortBuckets), n_cand, 0u, 0, 0u};
   if (red == 0xffffffffu) return r;
-  const uint32_t last_thread = ~red;
+  const uint32_t last_thread = (~red) >> 2;
+  r.more = (~red) & 3u;
   if (last_thread < static_cast<uint32_t>(kFinishBlock)) {
     r.last_bucket = last_thread * kPer + (kPer - 1);
     r.n_sorted = r.n = start[r.last_bucket + 1u];
@@ -863,6 +870,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // LDS.  However long the lists are, only what is kept has to fit.  A bucket with too many keys (heavy ties) leaves
   // the row to the steps below: the list in LDS, trimmed, and the sorting network.
   bool presorted = false, ok = false;
+  bool wide = false, wide_ok = false;  // the row went the way of nuclei wider than the sort / was finished there (else the steps below take it)
   uint32_t n_c = 0u;
   const int k_wanted = large_k ? (prm.k < V ? prm.k : V) : 0;
   if (!gave_up && rmax != 0u) {
@@ -885,7 +893,97 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     });
     __syncthreads();
     const TrimmedBuckets kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, kNucleusCap, red32, red64, k_wanted);
-    if (kept.n != 0u && kept.n_sorted >= static_cast<uint32_t>(k_wanted)) {  // (fewer than k numbers listed: the steps below decide)
+    if constexpr (!LARGEK) {
+      // The nucleus may need more keys than the sort has room for (a flat distribution, a high temperature), or a
+      // bucket too full for the usual ranking.  The same sort then runs in rounds, each over the next threads' runs
+      // of buckets that fit the room; a round's keys go from their ranks straight to the row's second key buffer in
+      // global memory, exponentials cached, and the epilogue reads the list from there.  Still a fraction of the
+      // exact path's work: the histogram's bound of the nucleus ends the rounds.  (Lists short enough for the head in
+      // registers fit the room: there only a bucket too full gets here, and the steps below take the row.)
+      if (kept.more != 0u && head == 0u && a.big2 != nullptr) {
+        wide = true;
+        constexpr int kPer = kSortBuckets / kFinishBlock;
+        constexpr int kWideBucketCap = 256;  // (a key's rank costs a compare per key of its bucket)
+        u64* const far = a.big2 + static_cast<size_t>(row) * a.big_stride;
+        // back from first places to counts, and scanned again with room for everything: where the nucleus ends
+        uint32_t s[kPer + 1];
+#pragma unroll
+        for (int i = 0; i <= kPer; ++i) s[i] = bucket_start[tid * kPer + i];
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) bucket_start[tid * kPer + i] = s[i + 1] - s[i];
+        __syncthreads();
+        const TrimmedBuckets all_kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, 0x7fffffff, red32, red64, 0, kWideBucketCap);
+        const uint32_t end_t = all_kept.last_bucket < static_cast<uint32_t>(kSortBuckets) ? all_kept.last_bucket / kPer + 1u
+                                                                                           : static_cast<uint32_t>(kFinishBlock);
+        bool in_rounds = all_kept.n != 0u && all_kept.more == 0u && static_cast<size_t>((all_kept.n + 7u) & ~7u) <= a.big_stride;
+        const float fmax = key_to_float(rmax), inv_temp = 1.0f / prm.temperature;
+        uint32_t first_t = 0u, done = 0u;
+        while (in_rounds && first_t < end_t) {
+          // the threads' runs of buckets first_t .. last_t - 1 fill the room at most (start[] of the buckets from
+          // first_t's on still holds their first places)
+          const uint32_t run_end = bucket_start[(tid + 1) * kPer];
+          const bool over = static_cast<uint32_t>(tid) >= first_t && static_cast<uint32_t>(tid) < end_t &&
+                            run_end - done > static_cast<uint32_t>(kNucleusCap);
+          const uint32_t first_over = block_max<uint32_t>(over ? static_cast<uint32_t>(kFinishBlock - tid) : 0u, red32);
+          const uint32_t last_t = first_over != 0u ? static_cast<uint32_t>(kFinishBlock) - first_over : end_t;
+          if (last_t == first_t) {  // one thread's buckets alone do not fit
+            in_rounds = false;
+            break;
+          }
+          const uint32_t n_round = bucket_start[last_t * kPer] - done;
+          const uint32_t first_b = first_t * kPer, end_b = last_t * kPer;
+          __syncthreads();  // (every thread has read the table as the last round left it)
+          flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
+#pragma unroll
+            for (int u = 0; u < kGather; ++u) {
+              if (valid[u]) {
+                const float score = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
+                if (score >= thr_score) {
+                  const uint32_t b = bucket_of.of_score(score);
+                  if (b >= first_b && b < end_b)
+                    lds_keys[atomicAdd(&bucket_start[b], 1u) - done] = (static_cast<u64>(order_key(score)) << 32) | (raw[u] & 0xffffffffull);
+                }
+              }
+            }
+          });
+          __syncthreads();
+          // (placing has counted every bucket's first place up to the next one's: bucket b lies between start[b - 1]
+          // and start[b], the row's places; the list in LDS starts at place `done`)
+          for (uint32_t pos = tid; pos < n_round; pos += kFinishBlock) {
+            const u64 k = lds_keys[pos];
+            const uint32_t b = bucket_of(key64_okey(k));
+            const uint32_t lo = (b > 0u ? bucket_start[b - 1u] : 0u) - done, hi = bucket_start[b] - done;
+            uint32_t rank = 0u;
+            for (uint32_t j = lo; j < hi; ++j) rank += lds_keys[j] > k ? 1u : 0u;
+            const float e = em::expf_exact((key_to_float(key64_okey(k)) - fmax) * inv_temp);
+            far[done + lo + rank] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k & 0xffffffffull);
+          }
+          __syncthreads();
+          done += n_round;
+          first_t = last_t;
+        }
+        if (in_rounds) {
+          // the best element below the candidates follows them when every bucket was needed; empty entries fill the
+          // last group of eight
+          const uint32_t n_list = all_kept.n;
+          if (static_cast<uint32_t>(tid) < ((n_list + 7u) & ~7u) - done) {
+            u64 entry = 0;
+            if (tid == 0 && done < n_list) {
+              const float e = em::expf_exact((key_to_float(key64_okey(all_kept.best_below)) - fmax) * inv_temp);
+              entry = (static_cast<u64>(__float_as_uint(e)) << 32) | (all_kept.best_below & 0xffffffffull);
+            }
+            far[done + tid] = entry;
+          }
+          __syncthreads();
+          const u64* list = far;
+          wide_ok = block_sample_epilogue<8>([=](int i) { return list[i]; },
+                                             [=](int i) { return __uint_as_float(static_cast<uint32_t>(list[i] >> 32)); },
+                                             static_cast<int>(n_list), V, prm, a.uniforms[row], row_outputs(a, row), seqsh);
+        }
+      }
+    }
+    if (!wide && kept.more != 2u && kept.n != 0u && kept.n_sorted >= static_cast<uint32_t>(k_wanted)) {  // (fewer than k numbers listed: the steps below decide)
       listed_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t used) {
 #pragma unroll
         for (int u = 0; u < kGather; ++u) {
@@ -905,7 +1003,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       n_c = kept.n;
     }
   }
-  if (!presorted) {
+  if (!presorted && !wide_ok) {
   bool trim_failed = false;
   if (!large_k && sh_all >= static_cast<uint32_t>(kNucleusCap)) {  // head == 0 here
     const float fmax = key_to_float(rmax), fthr = key_to_float(thr);
@@ -1007,7 +1105,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     ok = finish_candidates(lds_keys, bucket_start, n_c, presorted ? 0 : best_below, rmax, thr, false, prm, V,
                            emit ? 0.0 : a.uniforms[row], row_outputs(a, row), seqsh, red32, target, presorted);
   }
-  if (!ok) {
+  if (!ok && !wide_ok) {
     __syncthreads();
     general_row<AnyDtype, SortWithTile>(a, row, row_start<INLINE>(a, row, dtype_bytes(a.dtype)), prm, big_row, seqsh,
                           SortWithTile{a.big2 ? a.big2 + static_cast<size_t>(row) * a.big_stride : nullptr, lds_keys, red32, red64});
@@ -1103,7 +1201,7 @@ __device__ __forceinline__ uint32_t sort_counted(u64* keys, uint32_t* start, con
                                                  int V, uint32_t* red32, u64* red64) {
   __syncthreads();
   const TrimmedBuckets kept = scan_buckets_and_trim(start, bucket_of, best_below, prm, V, kNucleusCap, red32, red64);
-  if (kept.n == 0u) return 0u;
+  if (kept.n == 0u || kept.more == 2u) return 0u;  // (a bucket too full to rank among those the row needs)
   // every kept key to its bucket, in the order of arrival
 #pragma unroll
   for (int u = 0; u < kSparseRegs; ++u) {

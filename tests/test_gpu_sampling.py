@@ -394,8 +394,8 @@ def test_sparse_mask_rows_with_heavy_ties(ctx, orc):
 @pytest.mark.parametrize("sigma,p,t", [(4.0, 0.95, 1.0), (1.0, 0.9, 1.0), (5.0, 0.9, 1.0), (3.0, 0.5, 0.7)])
 def test_nucleus_rows_with_lists_near_and_beyond_the_sort(ctx, orc, sigma, p, t):
     """Unmasked nucleus rows of 128256 ids whose chunks list a few thousand to tens of thousands of keys: nuclei that
-    fit the finish kernel's sort with room to spare, that fill it almost completely, and that exceed it (the exact
-    path takes those rows).  Kept counts, the first kept ids with their probability bits, and tokens equal the
+    fit the finish kernel's sort with room to spare, that fill it almost completely, and that exceed it (sorted in
+    rounds).  Kept counts, the first kept ids with their probability bits, and tokens equal the
     oracle's."""
     say("nucleus near the sort's capacity", sigma, p, t)
     rng = np.random.default_rng(int(sigma * 10 + p * 100))
@@ -415,6 +415,40 @@ def test_nucleus_rows_with_lists_near_and_beyond_the_sort(ctx, orc, sigma, p, t)
         assert np.array_equal(ki[r, :n], idx[:n]), r
         assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), r
         assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+
+
+@pytest.mark.parametrize("sigma,p,t,wide_rows", [(3.0, 0.95, 1.0, 6), (2.0, 0.9, 1.0, 5), (4.0, 0.99, 1.5, 5), (1.0, 0.9, 1.0, 5)])
+def test_nucleus_rows_wider_than_the_sort(ctx, orc, sigma, p, t, wide_rows):
+    """Unmasked nucleus rows of 128256 ids whose nuclei hold 30000 to 90000 tokens, several times what the finish
+    kernel sorts at once: it sorts them in rounds into global memory.  One row is quantised to steps of 1/64 (dozens of
+    equal scores per step: buckets beyond the usual ranking), one to steps of 1/4 (thousands: those rows are the exact
+    path's).  Every kept id and probability bit, to the nucleus' last element, and the tokens equal the oracle's;
+    the rows without heavy ties stay off the exact path."""
+    say("nucleus wider than the sort", sigma, p, t)
+    rng = np.random.default_rng(int(sigma * 10 + p * 1000))
+    rows, vocab = 7, 128256
+    x = (rng.standard_normal((rows, vocab)) * sigma).astype(np.float32)
+    x[1] += np.float32(0.7)
+    x[2, : vocab // 2] -= np.float32(1.0)  # one half of the row lower: chunk thresholds differ
+    x[3, 1000:1040] = np.nan
+    x[4, 5] = 40.0  # one token far above the rest
+    x[5] = (np.round(x[5] * 64) / 64).astype(np.float32)
+    x[6] = (np.round(x[6] * 4) / 4).astype(np.float32)
+    u = rng.random(rows)
+    u[0] = 0.999999  # a draw from the nucleus' far end
+    before = ctx.fallback_rows()
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=p, temperature=t,
+                                 kept_capacity=vocab)
+    took_exact = ctx.fallback_rows() - before
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    for r in range(rows):
+        idx, probs = orc.sampled_categorical(x[r], 0, p, t)
+        n = len(idx)
+        assert kc[r] == n, (r, kc[r], n)
+        assert np.array_equal(ki[r, :n], idx), r
+        assert np.array_equal(bits(kp[r, :n]), bits(probs)), r
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+    assert took_exact <= rows - wide_rows, took_exact
 
 
 @pytest.mark.parametrize("k", [100, 512, 2048, 6000])
@@ -1112,7 +1146,7 @@ def exact_path_rows(name, rng, vocab):
 @pytest.mark.parametrize("vocab", [65, 511, 513, 4100, 10239, 10241, 16384, 70001, 128256, 201088])
 @pytest.mark.parametrize("name", ["gaussian", "constant", "rounded", "peaked", "mostly_lowest", "specials"])
 def test_exact_path_orders_whole_rows(ctx, orc, name, vocab):
-    """k above the candidate-list bound and sampling from the whole vocabulary (k = 0, p = 1) take the exact
+    """k above the candidate-list bound (8192) and sampling from the whole vocabulary (k = 0, p = 1) take the exact
     path, which sorts the entire row; the kept ids are that order, checked to the last element."""
     say("exact path", name, vocab)
     rng = np.random.default_rng(vocab + len(name))
@@ -1123,8 +1157,8 @@ def test_exact_path_orders_whole_rows(ctx, orc, name, vocab):
     sample_and_check(ctx, orc, x, u, 0, 1.0, 1.1, cap=vocab)
     if vocab > 2048:
         sample_and_check(ctx, orc, x, u, 2049, 0.97, 1.0, cap=2049)
-    # k <= 2048 goes through the candidate lists, which hand rows with ties or NaNs at their bound to the exact path too
-    assert ctx.fallback_rows() - before >= (6 if vocab > 2048 else 2)
+    # k <= 8192 goes through the candidate lists, which hand rows with ties or NaNs at their bound to the exact path too
+    assert ctx.fallback_rows() - before >= (4 if vocab > 8192 else 2)
 
 
 def test_exact_path_sixteen_bit_rows(ctx, orc):
