@@ -773,7 +773,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   for (int b = tid; b <= kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;  // the sort's table, while the loads are on their way
   // Thread c reads everything chunk c left behind; the barriers of the first reduction publish the counts.
   __shared__ uint32_t sh_cnt[kAllCap / kSmallCap];       // candidates per chunk
-  __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // their prefix sums
+  __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // rows of kFinishBlock entries the lists past their heads take, prefix sums
   __shared__ int sh_trim;
   __shared__ uint32_t sh_head, sh_all;
   uint32_t m = 0u, cthr = 0u;
@@ -798,10 +798,10 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     for (int c = 0; c < a.chunks; ++c) all += gave_up ? 0u : sh_cnt[c];
     const uint32_t head =
         (a.chunks <= kAheadChunks && all < static_cast<uint32_t>(kNucleusCap)) ? static_cast<uint32_t>(kFinishBlock) << head_shift : 0u;
-    uint32_t run = 0u;
+    uint32_t run = 0u;  // (in rows of kFinishBlock entries: a row lies in one chunk's list, so its chunk is found once for all threads)
     for (int c = 0; c < a.chunks; ++c) {
       sh_first[c] = run;
-      run += (gave_up || sh_cnt[c] <= head) ? 0u : sh_cnt[c] - head;
+      run += (gave_up || sh_cnt[c] <= head) ? 0u : (sh_cnt[c] - head + kFinishBlock - 1u) / kFinishBlock;
     }
     sh_first[a.chunks] = run;
     sh_head = head;
@@ -809,29 +809,51 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   }
   __syncthreads();
   const int lane = lane_id();
-  // Calls fn(entries, valid, used) for batches of kGather entries per thread (bit u of `used` clear: slot u is empty in every thread) of the flat sequence made of the
-  // chunks' lists past their heads (sh_first[c] = such entries of the chunks before c).
+  // The chunks' lists past their heads, as a sequence of rows of kFinishBlock entries (sh_first[c] = rows of the
+  // chunks before c; a list's last row may be short).  A cursor walks the rows in order; which chunk a row lies in
+  // is the same for every thread, so finding it costs the threads nothing.
   const uint32_t head = sh_head;
-  auto flat_batches = [&](auto fn) {
-    const uint32_t total = sh_first[a.chunks];
-    for (uint32_t f0 = 0; f0 < total; f0 += kGather * blockDim.x) {
-      u64 raw[kGather];
-      bool valid[kGather];
-      const uint32_t left = (total - f0 + blockDim.x - 1u) / blockDim.x;
-      const int n_slots = left < static_cast<uint32_t>(kGather) ? static_cast<int>(left) : kGather;  // no thread has an entry beyond
-      const uint32_t used = (1u << n_slots) - 1u;
+  struct ListCursor {
+    int chunk = -1;
+    uint32_t next_first = 0u, base = 0u, cnt = 0u;  // rows before the next chunk / before this one, entries of this one's list
+  };
+  // Loads the rows g0 .. g0 + n_slots - 1 (n_slots <= kGather, rows that exist) into raw[]; bit u of the result: the
+  // thread has an entry in row g0 + u.
+  auto load_rows = [&](ListCursor& cur, uint32_t g0, int n_slots, u64 (&raw)[kGather]) {
+    uint32_t have = 0u;
 #pragma unroll
-      for (int u = 0; u < kGather; ++u) {
-        const uint32_t f = f0 + u * blockDim.x + tid;
-        raw[u] = 0;
-        valid[u] = u < n_slots && f < total;
-        if (u < n_slots && valid[u]) {
-          int c = 0;
-          for (int cc = 1; cc < a.chunks; ++cc) c += f >= sh_first[cc] ? 1 : 0;
-          raw[u] = big_row[static_cast<size_t>(c) * kSChunk + head + (f - sh_first[c])];
+    for (int u = 0; u < kGather; ++u) {
+      raw[u] = 0;
+      if (u < n_slots) {
+        const uint32_t g = g0 + u;
+        while (g >= cur.next_first) {  // (ends: g is below the rows of all chunks)
+          ++cur.chunk;
+          cur.base = cur.next_first;
+          cur.next_first = __builtin_amdgcn_readfirstlane(sh_first[cur.chunk + 1]);
+          cur.cnt = __builtin_amdgcn_readfirstlane(sh_cnt[cur.chunk]);
+        }
+        const uint32_t i = head + (g - cur.base) * kFinishBlock + tid;
+        if (i < cur.cnt) {
+          raw[u] = big_row[static_cast<size_t>(cur.chunk) * kSChunk + i];
+          have |= 1u << u;
         }
       }
-      fn(raw, valid, used);
+    }
+    return have;
+  };
+  // Calls fn(entries, valid, used) for batches of kGather entries per thread (bit u of `used` clear: slot u is empty
+  // in every thread) of that sequence.
+  auto flat_batches = [&](auto fn) {
+    const uint32_t total = sh_first[a.chunks];
+    ListCursor cur;
+    for (uint32_t g0 = 0; g0 < total; g0 += kGather) {
+      u64 raw[kGather];
+      bool valid[kGather];
+      const int n_slots = total - g0 < static_cast<uint32_t>(kGather) ? static_cast<int>(total - g0) : kGather;
+      const uint32_t have = load_rows(cur, g0, n_slots, raw);
+#pragma unroll
+      for (int u = 0; u < kGather; ++u) valid[u] = (have >> u) & 1u;
+      fn(raw, valid, (1u << n_slots) - 1u);
     }
   };
   // More candidates listed than the sort holds (a flat distribution): the threshold is raised to the
@@ -895,10 +917,10 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     const TrimmedBuckets kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, kNucleusCap, red32, red64, k_wanted);
     if constexpr (!LARGEK) {
       // The nucleus may need more keys than the sort has room for (a flat distribution, a high temperature), or a
-      // bucket too full for the usual ranking.  The same sort then runs in rounds, each over the next threads' runs
-      // of buckets that fit the room; a round's keys go from their ranks straight to the row's second key buffer in
-      // global memory, exponentials cached, and the epilogue reads the list from there.  Still a fraction of the
-      // exact path's work: the histogram's bound of the nucleus ends the rounds.  (Lists short enough for the head in
+      // bucket too full for the usual ranking.  The same sort then runs over the row's second key buffer in global
+      // memory: every needed key goes to a place of its bucket's there, the buckets are ranked in rounds through LDS,
+      // and the epilogue reads the list from there.  Still a fraction of the exact path's work: the histogram's bound
+      // of the nucleus says which buckets are needed.  (Lists short enough for the head in
       // registers fit the room: there only a bucket too full gets here, and the steps below take the row.)
       if (kept.more != 0u && head == 0u && a.big2 != nullptr) {
         wide = true;
@@ -918,11 +940,36 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
                                                                                            : static_cast<uint32_t>(kFinishBlock);
         bool in_rounds = all_kept.n != 0u && all_kept.more == 0u && static_cast<size_t>((all_kept.n + 7u) & ~7u) <= a.big_stride;
         const float fmax = key_to_float(rmax), inv_temp = 1.0f / prm.temperature;
+        if (in_rounds) {
+          // One more pass over the lists gives every key of the needed buckets a place of its bucket's in the global
+          // buffer (the atomics of a batch are issued together).
+          const uint32_t end_b = end_t * kPer;
+          flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
+            uint32_t bucket[kGather], place[kGather];
+#pragma unroll
+            for (int u = 0; u < kGather; ++u) {
+              const float score = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
+              const uint32_t b = bucket_of.of_score(score);
+              bucket[u] = (valid[u] && score >= thr_score && b < end_b) ? b : 0xffffffffu;
+            }
+#pragma unroll
+            for (int u = 0; u < kGather; ++u)
+              if (bucket[u] != 0xffffffffu) place[u] = atomicAdd(&bucket_start[bucket[u]], 1u);
+#pragma unroll
+            for (int u = 0; u < kGather; ++u) {
+              if (bucket[u] != 0xffffffffu)
+                far[place[u]] = (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)))) << 32) | (raw[u] & 0xffffffffull);
+            }
+          });
+          __syncthreads();
+        }
+        // (Placing has counted every bucket's first place up to the next one's: bucket b now lies between start[b - 1]
+        // and start[b].)  The rounds: the next threads' runs of buckets that fit the room come to LDS as they lie, a
+        // key's rank inside its bucket comes from comparing whole keys, and the entry -- the exponential cached in
+        // it -- goes back to its final place.
         uint32_t first_t = 0u, done = 0u;
         while (in_rounds && first_t < end_t) {
-          // the threads' runs of buckets first_t .. last_t - 1 fill the room at most (start[] of the buckets from
-          // first_t's on still holds their first places)
-          const uint32_t run_end = bucket_start[(tid + 1) * kPer];
+          const uint32_t run_end = bucket_start[(tid + 1) * kPer - 1];
           const bool over = static_cast<uint32_t>(tid) >= first_t && static_cast<uint32_t>(tid) < end_t &&
                             run_end - done > static_cast<uint32_t>(kNucleusCap);
           const uint32_t first_over = block_max<uint32_t>(over ? static_cast<uint32_t>(kFinishBlock - tid) : 0u, red32);
@@ -931,33 +978,33 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
             in_rounds = false;
             break;
           }
-          const uint32_t n_round = bucket_start[last_t * kPer] - done;
-          const uint32_t first_b = first_t * kPer, end_b = last_t * kPer;
-          __syncthreads();  // (every thread has read the table as the last round left it)
-          flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
+          const uint32_t n_round = bucket_start[last_t * kPer - 1u] - done;
+          constexpr int kPerThread = kNucleusCap / kFinishBlock;
+          u64 mine[kPerThread];
 #pragma unroll
-            for (int u = 0; u < kGather; ++u) {
-              if (valid[u]) {
-                const float score = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
-                if (score >= thr_score) {
-                  const uint32_t b = bucket_of.of_score(score);
-                  if (b >= first_b && b < end_b)
-                    lds_keys[atomicAdd(&bucket_start[b], 1u) - done] = (static_cast<u64>(order_key(score)) << 32) | (raw[u] & 0xffffffffull);
-                }
-              }
-            }
-          });
+          for (int r = 0; r < kPerThread; ++r) {
+            const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + tid);
+            mine[r] = pos < n_round ? far[done + pos] : 0;
+          }
+#pragma unroll
+          for (int r = 0; r < kPerThread; ++r) lds_keys[r * kFinishBlock + tid] = mine[r];
           __syncthreads();
-          // (placing has counted every bucket's first place up to the next one's: bucket b lies between start[b - 1]
-          // and start[b], the row's places; the list in LDS starts at place `done`)
-          for (uint32_t pos = tid; pos < n_round; pos += kFinishBlock) {
-            const u64 k = lds_keys[pos];
-            const uint32_t b = bucket_of(key64_okey(k));
-            const uint32_t lo = (b > 0u ? bucket_start[b - 1u] : 0u) - done, hi = bucket_start[b] - done;
-            uint32_t rank = 0u;
-            for (uint32_t j = lo; j < hi; ++j) rank += lds_keys[j] > k ? 1u : 0u;
-            const float e = em::expf_exact((key_to_float(key64_okey(k)) - fmax) * inv_temp);
-            far[done + lo + rank] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k & 0xffffffffull);
+#pragma unroll 1
+          for (int r = 0; r < kPerThread; ++r) {
+            const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + tid);
+            if (pos < n_round) {
+              const u64 k = lds_keys[pos];
+              const uint32_t b = bucket_of(key64_okey(k));
+              const uint32_t lo = (b > 0u ? bucket_start[b - 1u] : 0u) - done, hi = bucket_start[b] - done;
+              uint32_t rank = 0u, j = lo;
+              for (; j + 4u <= hi; j += 4u) {  // (four reads under way at a time)
+                const u64 k0 = lds_keys[j], k1 = lds_keys[j + 1u], k2 = lds_keys[j + 2u], k3 = lds_keys[j + 3u];
+                rank += (k0 > k ? 1u : 0u) + (k1 > k ? 1u : 0u) + (k2 > k ? 1u : 0u) + (k3 > k ? 1u : 0u);
+              }
+              for (; j < hi; ++j) rank += lds_keys[j] > k ? 1u : 0u;
+              const float e = em::expf_exact((key_to_float(key64_okey(k)) - fmax) * inv_temp);
+              far[done + lo + rank] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k & 0xffffffffull);
+            }
           }
           __syncthreads();
           done += n_round;
