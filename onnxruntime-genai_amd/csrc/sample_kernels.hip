@@ -819,7 +819,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   };
   // Loads the rows g0 .. g0 + n_slots - 1 (n_slots <= kGather, rows that exist) into raw[]; bit u of the result: the
   // thread has an entry in row g0 + u.
-  auto load_rows = [&](ListCursor& cur, uint32_t g0, int n_slots, u64 (&raw)[kGather]) {
+  auto load_rows = [&](ListCursor& cur, uint32_t g0, int n_slots, u64 (&raw)[kGather]) __attribute__((always_inline)) {
     uint32_t have = 0u;
 #pragma unroll
     for (int u = 0; u < kGather; ++u) {
@@ -843,7 +843,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   };
   // Calls fn(entries, valid, used) for batches of kGather entries per thread (bit u of `used` clear: slot u is empty
   // in every thread) of that sequence.
-  auto flat_batches = [&](auto fn) {
+  auto flat_batches = [&](auto fn) __attribute__((always_inline)) {
     const uint32_t total = sh_first[a.chunks];
     ListCursor cur;
     for (uint32_t g0 = 0; g0 < total; g0 += kGather) {
@@ -863,7 +863,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // exact path.
   // The entries of the head (in registers) and then of the rest of the lists, in batches: fn(entries, valid, used),
   // bit u of `used` clear: no thread has an entry in slot u.
-  auto listed_batches = [&](auto fn) {
+  auto listed_batches = [&](auto fn) __attribute__((always_inline)) {
     if (head != 0u) {
 #pragma unroll
       for (int b = 0; b < kHeadSlots / kGather; ++b) {
@@ -892,7 +892,12 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // LDS.  However long the lists are, only what is kept has to fit.  A bucket with too many keys (heavy ties) leaves
   // the row to the steps below: the list in LDS, trimmed, and the sorting network.
   bool presorted = false, ok = false;
-  bool wide = false, wide_ok = false;  // the row went the way of nuclei wider than the sort / was finished there (else the steps below take it)
+  // A row that goes the way of nuclei wider than the sort (decided after the first scan, done at the kernel's end;
+  // kept in LDS, not in registers, in between): the threads whose runs of buckets the nucleus needs, the entries of
+  // its list, and the best element below the candidates when it follows them.
+  __shared__ uint32_t sh_wide_end_t, sh_wide_n;
+  __shared__ u64 sh_wide_below;
+  bool wide = false, wide_ok = false;  // such a row / finished that way
   uint32_t n_c = 0u;
   const int k_wanted = large_k ? (prm.k < V ? prm.k : V) : 0;
   if (!gave_up && rmax != 0u) {
@@ -920,13 +925,12 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       // bucket too full for the usual ranking.  The same sort then runs over the row's second key buffer in global
       // memory: every needed key goes to a place of its bucket's there, the buckets are ranked in rounds through LDS,
       // and the epilogue reads the list from there.  Still a fraction of the exact path's work: the histogram's bound
-      // of the nucleus says which buckets are needed.  (Lists short enough for the head in
-      // registers fit the room: there only a bucket too full gets here, and the steps below take the row.)
+      // of the nucleus says which buckets are needed.  Decided here, done at the kernel's end.  (Lists short enough
+      // for the head in registers fit the room: there only a bucket too full gets here, and the steps below take
+      // the row, as they do when a bucket is too full even for the rounds.)
       if (kept.more != 0u && head == 0u && a.big2 != nullptr) {
-        wide = true;
         constexpr int kPer = kSortBuckets / kFinishBlock;
         constexpr int kWideBucketCap = 256;  // (a key's rank costs a compare per key of its bucket)
-        u64* const far = a.big2 + static_cast<size_t>(row) * a.big_stride;
         // back from first places to counts, and scanned again with room for everything: where the nucleus ends
         uint32_t s[kPer + 1];
 #pragma unroll
@@ -936,97 +940,13 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
         for (int i = 0; i < kPer; ++i) bucket_start[tid * kPer + i] = s[i + 1] - s[i];
         __syncthreads();
         const TrimmedBuckets all_kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, 0x7fffffff, red32, red64, 0, kWideBucketCap);
-        const uint32_t end_t = all_kept.last_bucket < static_cast<uint32_t>(kSortBuckets) ? all_kept.last_bucket / kPer + 1u
-                                                                                           : static_cast<uint32_t>(kFinishBlock);
-        bool in_rounds = all_kept.n != 0u && all_kept.more == 0u && static_cast<size_t>((all_kept.n + 7u) & ~7u) <= a.big_stride;
-        const float fmax = key_to_float(rmax), inv_temp = 1.0f / prm.temperature;
-        if (in_rounds) {
-          // One more pass over the lists gives every key of the needed buckets a place of its bucket's in the global
-          // buffer (the atomics of a batch are issued together).
-          const uint32_t end_b = end_t * kPer;
-          flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
-            uint32_t bucket[kGather], place[kGather];
-#pragma unroll
-            for (int u = 0; u < kGather; ++u) {
-              const float score = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
-              const uint32_t b = bucket_of.of_score(score);
-              bucket[u] = (valid[u] && score >= thr_score && b < end_b) ? b : 0xffffffffu;
-            }
-#pragma unroll
-            for (int u = 0; u < kGather; ++u)
-              if (bucket[u] != 0xffffffffu) place[u] = atomicAdd(&bucket_start[bucket[u]], 1u);
-#pragma unroll
-            for (int u = 0; u < kGather; ++u) {
-              if (bucket[u] != 0xffffffffu)
-                far[place[u]] = (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)))) << 32) | (raw[u] & 0xffffffffull);
-            }
-          });
-          __syncthreads();
-        }
-        // (Placing has counted every bucket's first place up to the next one's: bucket b now lies between start[b - 1]
-        // and start[b].)  The rounds: the next threads' runs of buckets that fit the room come to LDS as they lie, a
-        // key's rank inside its bucket comes from comparing whole keys, and the entry -- the exponential cached in
-        // it -- goes back to its final place.
-        uint32_t first_t = 0u, done = 0u;
-        while (in_rounds && first_t < end_t) {
-          const uint32_t run_end = bucket_start[(tid + 1) * kPer - 1];
-          const bool over = static_cast<uint32_t>(tid) >= first_t && static_cast<uint32_t>(tid) < end_t &&
-                            run_end - done > static_cast<uint32_t>(kNucleusCap);
-          const uint32_t first_over = block_max<uint32_t>(over ? static_cast<uint32_t>(kFinishBlock - tid) : 0u, red32);
-          const uint32_t last_t = first_over != 0u ? static_cast<uint32_t>(kFinishBlock) - first_over : end_t;
-          if (last_t == first_t) {  // one thread's buckets alone do not fit
-            in_rounds = false;
-            break;
-          }
-          const uint32_t n_round = bucket_start[last_t * kPer - 1u] - done;
-          constexpr int kPerThread = kNucleusCap / kFinishBlock;
-          u64 mine[kPerThread];
-#pragma unroll
-          for (int r = 0; r < kPerThread; ++r) {
-            const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + tid);
-            mine[r] = pos < n_round ? far[done + pos] : 0;
-          }
-#pragma unroll
-          for (int r = 0; r < kPerThread; ++r) lds_keys[r * kFinishBlock + tid] = mine[r];
-          __syncthreads();
-#pragma unroll 1
-          for (int r = 0; r < kPerThread; ++r) {
-            const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + tid);
-            if (pos < n_round) {
-              const u64 k = lds_keys[pos];
-              const uint32_t b = bucket_of(key64_okey(k));
-              const uint32_t lo = (b > 0u ? bucket_start[b - 1u] : 0u) - done, hi = bucket_start[b] - done;
-              uint32_t rank = 0u, j = lo;
-              for (; j + 4u <= hi; j += 4u) {  // (four reads under way at a time)
-                const u64 k0 = lds_keys[j], k1 = lds_keys[j + 1u], k2 = lds_keys[j + 2u], k3 = lds_keys[j + 3u];
-                rank += (k0 > k ? 1u : 0u) + (k1 > k ? 1u : 0u) + (k2 > k ? 1u : 0u) + (k3 > k ? 1u : 0u);
-              }
-              for (; j < hi; ++j) rank += lds_keys[j] > k ? 1u : 0u;
-              const float e = em::expf_exact((key_to_float(key64_okey(k)) - fmax) * inv_temp);
-              far[done + lo + rank] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k & 0xffffffffull);
-            }
-          }
-          __syncthreads();
-          done += n_round;
-          first_t = last_t;
-        }
-        if (in_rounds) {
-          // the best element below the candidates follows them when every bucket was needed; empty entries fill the
-          // last group of eight
-          const uint32_t n_list = all_kept.n;
-          if (static_cast<uint32_t>(tid) < ((n_list + 7u) & ~7u) - done) {
-            u64 entry = 0;
-            if (tid == 0 && done < n_list) {
-              const float e = em::expf_exact((key_to_float(key64_okey(all_kept.best_below)) - fmax) * inv_temp);
-              entry = (static_cast<u64>(__float_as_uint(e)) << 32) | (all_kept.best_below & 0xffffffffull);
-            }
-            far[done + tid] = entry;
-          }
-          __syncthreads();
-          const u64* list = far;
-          wide_ok = block_sample_epilogue<8>([=](int i) { return list[i]; },
-                                             [=](int i) { return __uint_as_float(static_cast<uint32_t>(list[i] >> 32)); },
-                                             static_cast<int>(n_list), V, prm, a.uniforms[row], row_outputs(a, row), seqsh);
+        // (the table holds first places again; a row that does not go this way goes on as if nothing had happened)
+        wide = all_kept.n != 0u && all_kept.more == 0u && static_cast<size_t>((all_kept.n + 7u) & ~7u) <= a.big_stride;
+        if (wide && tid == 0) {
+          sh_wide_end_t = all_kept.last_bucket < static_cast<uint32_t>(kSortBuckets) ? all_kept.last_bucket / kPer + 1u
+                                                                                      : static_cast<uint32_t>(kFinishBlock);
+          sh_wide_n = all_kept.n;
+          sh_wide_below = all_kept.best_below;
         }
       }
     }
@@ -1050,7 +970,109 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       n_c = kept.n;
     }
   }
-  if (!presorted && !wide_ok) {
+  if constexpr (!LARGEK) {
+    if (wide) {  // (decided after the first scan; the table holds the buckets' first places)
+      __syncthreads();
+      const uint32_t wide_end_t = sh_wide_end_t;
+      const uint32_t wide_n = sh_wide_n;
+      const u64 wide_below = sh_wide_below;
+      constexpr int kPer = kSortBuckets / kFinishBlock;
+      u64* const far = a.big2 + static_cast<size_t>(row) * a.big_stride;
+      const ScoreBuckets bucket_of(rmax, thr);
+      const float thr_score = key_to_float(thr);
+      const float fmax = key_to_float(rmax), inv_temp = 1.0f / prm.temperature;
+      bool in_rounds = true;
+      {
+        // One more pass over the lists gives every key of the needed buckets a place of its bucket's in the global
+        // buffer (the atomics of a batch are issued together).
+        const uint32_t end_b = wide_end_t * kPer;
+        flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
+          uint32_t bucket[kGather], place[kGather];
+#pragma unroll
+          for (int u = 0; u < kGather; ++u) {
+            const float score = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
+            const uint32_t b = bucket_of.of_score(score);
+            bucket[u] = (valid[u] && score >= thr_score && b < end_b) ? b : 0xffffffffu;
+          }
+#pragma unroll
+          for (int u = 0; u < kGather; ++u)
+            if (bucket[u] != 0xffffffffu) place[u] = atomicAdd(&bucket_start[bucket[u]], 1u);
+#pragma unroll
+          for (int u = 0; u < kGather; ++u) {
+            if (bucket[u] != 0xffffffffu)
+              far[place[u]] = (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)))) << 32) | (raw[u] & 0xffffffffull);
+          }
+        });
+        __syncthreads();
+      }
+      // (Placing has counted every bucket's first place up to the next one's: bucket b now lies between start[b - 1]
+      // and start[b].)  The rounds: the next threads' runs of buckets that fit the room come to LDS as they lie, a
+      // key's rank inside its bucket comes from comparing whole keys, and the entry -- the exponential cached in
+      // it -- goes back to its final place.
+      uint32_t first_t = 0u, done = 0u;
+      while (in_rounds && first_t < wide_end_t) {
+        const uint32_t run_end = bucket_start[(tid + 1) * kPer - 1];
+        const bool over = static_cast<uint32_t>(tid) >= first_t && static_cast<uint32_t>(tid) < wide_end_t &&
+                          run_end - done > static_cast<uint32_t>(kNucleusCap);
+        const uint32_t first_over = block_max<uint32_t>(over ? static_cast<uint32_t>(kFinishBlock - tid) : 0u, red32);
+        const uint32_t last_t = first_over != 0u ? static_cast<uint32_t>(kFinishBlock) - first_over : wide_end_t;
+        if (last_t == first_t) {  // one thread's buckets alone do not fit
+          in_rounds = false;
+          break;
+        }
+        const uint32_t n_round = bucket_start[last_t * kPer - 1u] - done;
+        constexpr int kPerThread = kNucleusCap / kFinishBlock;
+        u64 mine[kPerThread];
+#pragma unroll
+        for (int r = 0; r < kPerThread; ++r) {
+          const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + tid);
+          mine[r] = pos < n_round ? far[done + pos] : 0;
+        }
+#pragma unroll
+        for (int r = 0; r < kPerThread; ++r) lds_keys[r * kFinishBlock + tid] = mine[r];
+        __syncthreads();
+#pragma unroll 1
+        for (int r = 0; r < kPerThread; ++r) {
+          const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + tid);
+          if (pos < n_round) {
+            const u64 k = lds_keys[pos];
+            const uint32_t b = bucket_of(key64_okey(k));
+            const uint32_t lo = (b > 0u ? bucket_start[b - 1u] : 0u) - done, hi = bucket_start[b] - done;
+            uint32_t rank = 0u, j = lo;
+            for (; j + 4u <= hi; j += 4u) {  // (four reads under way at a time)
+              const u64 k0 = lds_keys[j], k1 = lds_keys[j + 1u], k2 = lds_keys[j + 2u], k3 = lds_keys[j + 3u];
+              rank += (k0 > k ? 1u : 0u) + (k1 > k ? 1u : 0u) + (k2 > k ? 1u : 0u) + (k3 > k ? 1u : 0u);
+            }
+            for (; j < hi; ++j) rank += lds_keys[j] > k ? 1u : 0u;
+            const float e = em::expf_exact((key_to_float(key64_okey(k)) - fmax) * inv_temp);
+            far[done + lo + rank] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k & 0xffffffffull);
+          }
+        }
+        __syncthreads();
+        done += n_round;
+        first_t = last_t;
+      }
+      if (in_rounds) {
+        // the best element below the candidates follows them when every bucket was needed; empty entries fill the
+        // last group of eight
+        const uint32_t n_list = wide_n;
+        if (static_cast<uint32_t>(tid) < ((n_list + 7u) & ~7u) - done) {
+          u64 entry = 0;
+          if (tid == 0 && done < n_list) {
+            const float e = em::expf_exact((key_to_float(key64_okey(wide_below)) - fmax) * inv_temp);
+            entry = (static_cast<u64>(__float_as_uint(e)) << 32) | (wide_below & 0xffffffffull);
+          }
+          far[done + tid] = entry;
+        }
+        __syncthreads();
+        const u64* list = far;
+        wide_ok = block_sample_epilogue<8>([=](int i) { return list[i]; },
+                                           [=](int i) { return __uint_as_float(static_cast<uint32_t>(list[i] >> 32)); },
+                                           static_cast<int>(n_list), V, prm, a.uniforms[row], row_outputs(a, row), seqsh);
+      }
+    }
+  }
+  if (!presorted && !wide) {
   bool trim_failed = false;
   if (!large_k && sh_all >= static_cast<uint32_t>(kNucleusCap)) {  // head == 0 here
     const float fmax = key_to_float(rmax), fthr = key_to_float(thr);
