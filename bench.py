@@ -127,7 +127,7 @@ def hbm_copy_probe(torch, dev):
     return 2 * n * 4 * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
 
-def step_latencies(torch, np, step, tokens, side, W, K):
+def step_latencies(torch, np, step, tokens, side, W, K, prepare=None):
     """Distribution of the step latency, outside the timed region: every one of the K steps launched eagerly
     between its own pair of HIP events on the launch stream (GPU time of one step), and the host-clock time
     from the call of a single step to its token ids being on the host (launch + kernel + copy back)."""
@@ -163,6 +163,23 @@ def step_latencies(torch, np, step, tokens, side, W, K):
             side.synchronize()
             if not np.array_equal(view, tokens[W + j].cpu().numpy()):
                 sys.exit("PARITY FAILURE: tokens written to pinned host memory differ from the tokens in device memory")
+        # And with the call marshalled beforehand, as a serving loop with fixed buffers issues it (the Python
+        # binding's per-call tensor lookups are gone; the foreign call, the launch and the kernel remain).
+        prepared_t, prepared_ret = [], []
+        if prepare is not None:
+            calls = [prepare(W + j, pinned, side) for j in range(min(n, 64))]
+            for j, call in enumerate(calls):
+                view[:] = -1
+                t0 = time.perf_counter()
+                call()
+                prepared_ret.append((time.perf_counter() - t0) * 1e6)
+                while (view < 0).any():
+                    if time.perf_counter() - t0 > 5.0:
+                        sys.exit("tokens never arrived in pinned host memory")
+                prepared_t.append((time.perf_counter() - t0) * 1e6)
+                side.synchronize()
+                if not np.array_equal(view, tokens[W + j].cpu().numpy()):
+                    sys.exit("PARITY FAILURE: tokens of a prepared call differ from the tokens in device memory")
     torch.cuda.synchronize()
     return {"note": "informational: single eager launches, each between its own HIP events; host clock from the "
                     "call to the token ids on the host, first with a copy back from device memory, then with the "
@@ -174,7 +191,12 @@ def step_latencies(torch, np, step, tokens, side, W, K):
             "launch_to_result_us_p95": float(np.percentile(direct, 95)),
             "of_which_host_call_us_p50": float(np.percentile(returned, 50)),
             "launch_to_result_via_copy_us_p50": float(np.percentile(host, 50)),
-            "launch_to_result_via_copy_us_p95": float(np.percentile(host, 95))}
+            "launch_to_result_via_copy_us_p95": float(np.percentile(host, 95)),
+            "prepared_call": None if not prepared_t else {
+                "note": "the same step with its arguments marshalled once beforehand (SearchContext.prepared_sample)",
+                "launch_to_result_us_p50": float(np.percentile(prepared_t, 50)),
+                "launch_to_result_us_p95": float(np.percentile(prepared_t, 95)),
+                "of_which_host_call_us_p50": float(np.percentile(prepared_ret, 50))}}
 
 
 def main():
@@ -279,7 +301,10 @@ def main():
         bad = int((got != want).sum())
         sys.exit(f"PARITY FAILURE: {bad} of {got.size} sampled tokens differ from the CPU oracle")
     fallback = ctx.fallback_rows()
-    latency = step_latencies(torch, np, step, tokens, side, W, K)
+    def prepare(i, out, stream):
+        return ctx.prepared_sample(logits[i % pool], uniforms[i], out, k=TOP_K, p=TOP_P, temperature=TEMP, stream=stream)
+
+    latency = step_latencies(torch, np, step, tokens, side, W, K, prepare)
     # ---- CPU baseline: the reference's own functions where they were built, else the oracle ---------
     baseline = {"value": ROWS * n_cpu / cpu_s, "unit": "tokens/s", "cores": 1, "kind": "port",
                 "sample": "%d of the %d timed steps (same logits and uniforms), oracle/search_oracle.cpp "

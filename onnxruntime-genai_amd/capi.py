@@ -247,6 +247,28 @@ class SearchContext:
             return out, kc, ki, kp
         return out
 
+    def prepared_sample(self, logits, uniforms, out, k=0, p=0.0, temperature=1.0, xf=None, stream=None):
+        """Marshals one mi355x_sample call once and returns a function that issues it: what a serving loop with fixed
+        buffers does (the tensors, `xf` and the stream -- default: the stream current now -- must stay alive and
+        where they are; the function takes no arguments and raises on an error code).  `out` may be pinned host
+        memory.  The per-call cost is the foreign call alone, none of the tensor lookups of `sample`."""
+        rows, vocab, stride = self._rows(logits)
+        assert uniforms.dtype == torch.float64 and uniforms.numel() >= rows and out.dtype == torch.int32 and out.numel() >= rows
+        handle = C.c_void_p(stream.cuda_stream) if stream is not None else _stream()
+        typed = logits.dtype != torch.float32
+        fn = self.L.mi355x_sample_typed if typed else self.L.mi355x_sample
+        head = (self.h, handle, C.c_void_p(logits.data_ptr())) + ((C.c_int32(_DTYPE_CODES[logits.dtype]),) if typed else ())
+        args = head + (C.c_int64(stride), C.c_int32(rows), C.c_int32(vocab), C.byref(xf.c) if xf else None,
+                       SampleParams(int(k), float(p), float(temperature)), None, C.c_void_p(uniforms.data_ptr()),
+                       C.c_void_p(out.data_ptr()), None, None, None, C.c_int32(0))
+        keep = (logits, uniforms, out, xf, stream)
+        check = self._check
+
+        def issue(_args=args, _fn=fn, _keep=keep):
+            rc = _fn(*_args)
+            if rc != 0:
+                check(rc)
+        return issue
 
 
 

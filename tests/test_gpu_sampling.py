@@ -326,6 +326,38 @@ def test_results_written_straight_to_pinned_host_memory(ctx, orc):
     assert seqs[:, cur].cpu().tolist() == [5, 7, pad, pad]
 
 
+def test_prepared_sample_calls_give_the_same_tokens(ctx, orc):
+    """SearchContext.prepared_sample marshals a call once; issuing it -- repeatedly, on its stream, into pinned host
+    memory or device memory, fp32 or fp16 rows -- gives the tokens of the same call made through `sample`."""
+    say("prepared calls")
+    rng = np.random.default_rng(405)
+    rows, vocab = 64, 40000
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    u = rng.random(rows)
+    xd, ud = torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda()
+    want = orc.sample_batch(x, 50, 0.9, 0.7, u)
+    out_dev = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
+    out_pin = torch.full((rows,), -1, dtype=torch.int32).pin_memory()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    calls = [ctx.prepared_sample(xd, ud, out_dev, k=50, p=0.9, temperature=0.7),
+             ctx.prepared_sample(xd, ud, out_pin, k=50, p=0.9, temperature=0.7, stream=side)]
+    for _ in range(3):
+        out_dev.fill_(-1)
+        out_pin.fill_(-1)
+        torch.cuda.synchronize()
+        for call in calls:
+            call()
+        torch.cuda.synchronize()
+        assert np.array_equal(out_dev.cpu().numpy(), want)
+        assert np.array_equal(out_pin.numpy(), want)
+    xh = torch.from_numpy(x.astype(np.float16)).cuda()
+    call16 = ctx.prepared_sample(xh, ud, out_dev, k=0, p=0.9, temperature=1.0)
+    call16()
+    torch.cuda.synchronize()
+    assert np.array_equal(out_dev.cpu().numpy(), orc.sample_batch(xh.float().cpu().numpy(), 0, 0.9, 1.0, u))
+
+
 def test_config2_topk_topp_batch64(ctx, orc):
     """Benchmark configuration 2 at full size: batch 64, vocab 128256, N(0,3^2) logits + 8 peaks/row at +10,
     T=0.7, k=50, p=0.9, shared uniforms; 4 of the 128 steps."""
