@@ -893,10 +893,11 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // the row to the steps below: the list in LDS, trimmed, and the sorting network.
   bool presorted = false, ok = false;
   // A row that goes the way of nuclei wider than the sort (decided after the first scan, done at the kernel's end;
-  // kept in LDS, not in registers, in between): the threads whose runs of buckets the nucleus needs, the entries of
-  // its list, and the best element below the candidates when it follows them.
+  // kept in LDS, not in registers, in between): the threads whose runs of buckets the nucleus needs (0: not such a
+  // row), the entries of its list, and the best element below the candidates when it follows them.
   __shared__ uint32_t sh_wide_end_t, sh_wide_n;
   __shared__ u64 sh_wide_below;
+  if (tid == 0) sh_wide_end_t = 0u;  // (barriers follow before it is looked at)
   bool wide = false, wide_ok = false;  // such a row / finished that way
   uint32_t n_c = 0u;
   const int k_wanted = large_k ? (prm.k < V ? prm.k : V) : 0;
@@ -971,9 +972,9 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     }
   }
   if constexpr (!LARGEK) {
-    if (wide) {  // (decided after the first scan; the table holds the buckets' first places)
-      __syncthreads();
-      const uint32_t wide_end_t = sh_wide_end_t;
+    __syncthreads();
+    const uint32_t wide_end_t = sh_wide_end_t;
+    if (wide_end_t != 0u) {  // (decided after the first scan; the table holds the buckets' first places)
       const uint32_t wide_n = sh_wide_n;
       const u64 wide_below = sh_wide_below;
       constexpr int kPer = kSortBuckets / kFinishBlock;
