@@ -428,6 +428,7 @@ def run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, lengt
         assert dev.is_done() == (ref.is_done() or length == max_length)
         if dev.is_done():
             break
+    finished_early = sum(ref.hyp_count(b) for b in range(batch))  # hypotheses that ended with an EOS along the way
     ref.finalize(seq, length)
     for b in range(batch):
         for i in range(ref.hyp_count(b)):
@@ -435,6 +436,7 @@ def run_beam_search(ctx, orc, batch, beams, vocab, steps, eos, max_length, lengt
             got_t, got_s = dev.hypothesis(b, i)
             assert got_t == list(want_t) and np.float32(got_s) == np.float32(want_s), (b, i)
     dev.close()
+    return length - 3, finished_early
 
 
 @pytest.mark.parametrize("batch,beams,vocab", [(2, 8, 131072), (2, 8, 131073), (1, 16, 16384), (40, 4, 16385)])

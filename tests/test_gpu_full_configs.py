@@ -2,7 +2,8 @@
 (configuration 2 and the selection phase of 3 are covered at full size in test_gpu_sampling.py /
 test_gpu_beam_spec.py; here: all 256 rows of configuration 5, a heterogeneous batch of more than 64 rows
 at a 128K vocabulary, exact sums over more segments than the GPU runs at once, and the 56-tensor KV gather of
-configuration 3)."""
+configuration 3), and configurations 1 and 3 as whole runs of all their steps, where every step's state feeds
+the next."""
 import numpy as np
 import pytest
 import torch
@@ -117,3 +118,63 @@ def test_config3_kv_gather_all_56_tensors():
     for t, (p, q) in enumerate(zip(present, past)):
         assert torch.equal(q.view(torch.int16), p.view(torch.int16)[idx.long()]), t
     ctx.close()
+
+
+def test_config1_whole_run_of_256_steps_with_growing_history(orc):
+    """Benchmark configuration 1 as a whole generation, not step by step: batch 1, vocab 32064, greedy with
+    repetition penalty 1.1 over everything generated so far (a 256-token prompt, then 256 steps), EOS check, pad and
+    append on the device.  The state a step leaves (the sequence, which is the next step's history; the EOS flag)
+    feeds the next one on both sides; the sequences must agree token for token to the end, where a boosted EOS ends
+    the run."""
+    say("config1 whole run")
+    rng = np.random.default_rng(101)
+    vocab, prompt_len, steps, eos, pad = 32064, 256, 256, 17, 0
+    max_length = prompt_len + steps
+    ctx = pkg().SearchContext(1, vocab)
+    prompt = rng.integers(0, vocab, prompt_len).astype(np.int32)
+    prompt[prompt == eos] = eos + 1
+    seq = np.zeros(max_length, np.int32)
+    seq[:prompt_len] = prompt
+    d_seq = torch.zeros((1, max_length), dtype=torch.int32, device="cuda")
+    d_seq[0, :prompt_len] = torch.from_numpy(prompt).cuda()
+    d_seen = torch.zeros(1, dtype=torch.int32, device="cuda")
+    d_done = torch.zeros(1, dtype=torch.int32, device="cuda")
+    length, ended_at = prompt_len, None
+    for step in range(steps):
+        x = (rng.standard_normal((1, vocab)) * 2).astype(np.float32)
+        x[0, rng.integers(0, vocab)] += 8
+        if step % 3 == 0:  # a token already generated gets the spike: the penalty decides whether it still wins
+            x[0, seq[rng.integers(0, length)]] += 9
+        if step == steps - 6:
+            x[0, eos] += 40
+        xf = pkg().LogitsXform(history=d_seq[:, :length].contiguous(), repetition_penalty=1.1)
+        tok = ctx.argmax(torch.from_numpy(x).cuda(), xf=xf)
+        ctx.greedy_tail(tok, d_seen, [eos], pad, d_seq, length, d_done)
+        want = orc.argmax(orc.apply_repetition_penalty(x[0], seq[:length], 1.1))
+        assert tok.item() == want, step
+        if want == eos:
+            ended_at = step
+            assert d_done.item() == 1 and d_seen.item() == 1
+            break
+        assert d_done.item() == 0
+        seq[length] = want
+        length += 1
+        if step % 32 == 31:
+            assert np.array_equal(d_seq[0, :length].cpu().numpy(), seq[:length]), step
+    assert ended_at == steps - 6
+    assert np.array_equal(d_seq[0, :length].cpu().numpy(), seq[:length])
+    ctx.close()
+
+
+def test_config3_whole_beam_search_of_64_steps(orc):
+    """Benchmark configuration 3 as a whole search: batch 8, beams 4, vocab 151936 fp16, length penalty 1.0, all 64
+    steps through the fused per-step call, with an EOS boosted just enough that hypotheses finish along the way
+    while the search runs its full length.  After every step the scorer's state and the beam-reordered sequences
+    equal the oracle's; at the end the hypotheses do."""
+    from test_gpu_beam_spec import run_beam_search
+    say("config3 whole search")
+    ctx = pkg().SearchContext(32, 151936)
+    steps, finished_early = run_beam_search(ctx, orc, 8, 4, 151936, 64, [151935], 80, 1.0, False, 33, eos_boost=3.0,
+                                            fused=True)
+    ctx.close()
+    assert steps == 64 and finished_early >= 4, (steps, finished_early)
