@@ -17,6 +17,8 @@
 //   argmax, penalties, mask, sampled categorical (top-k and nucleus), discrete draw, softmax family,
 //   accept/correction math: pinned by the reference's own known-answer tests and, where it builds,
 //   by oracle/_ref (the unmodified reference headers compiled from /root/reference).
+//   the accept loops (sparse and dense): pinned as whole rounds on the reference's own functions driven by a
+//   real std::mt19937 (oracle/_ref); the dense one through selections that list the whole vocabulary.
 //   beam top-2B selection: pinned by brute force (full stable sort) on small inputs.
 //   argmax, BeamSearch_Cpu::SelectTop, BeamSearchScorer::Process (candidates that are not EOS), Finalize,
 //   GetBeamHypotheses and the beam sequence append: pinned by the reference's own golden generations

@@ -216,3 +216,38 @@ def test_sparse_accept_loop_matches_reference_with_real_engine(orc, ref):
         assert (acc1, tok1, used1) == (acc2, tok2, used2), case
         outcomes.add((acc1 == K, used1 - min(acc1 + 1, K)))
     assert outcomes == {(True, 0), (True, 2), (False, 0), (False, 2)}  # bonus / correction, with and without a draw
+
+
+def test_dense_accept_loop_matches_reference_with_real_engine(orc, ref):
+    """orc_spec_verify_dense as a loop against the reference: selections that list the whole vocabulary (ids
+    0 .. V-1) make the reference's accept loop -- its own ComputeAcceptProb, SampleCorrectionToken and
+    SampleSparseToken with a real std::mt19937 -- work on dense distributions; the dense oracle gets the same
+    uniforms in its explicit form (the categorical draw is the one the engine yields after the accept draws the
+    round has taken).  Accepted length and final token agree on rounds that accept everything, reject early and
+    reject late."""
+    rng = np.random.default_rng(22)
+    outcomes = set()
+    for case in range(200):
+        K = int(rng.integers(1, 9))
+        vocab = int(rng.choice([2, 17, 300]))
+        ids = np.arange(vocab, dtype=np.int32)
+        sharp = float(rng.choice([0.3, 1.0, 3.0]))
+        p = np.stack([orc.softmax((rng.standard_normal(vocab) * sharp).astype(np.float32), 1.0) for _ in range(K + 1)])
+        q = np.stack([orc.softmax((rng.standard_normal(vocab) * sharp).astype(np.float32), 1.0) for _ in range(K + 1)])
+        if case % 3 == 0:
+            q[:K] = p[:K]  # identical distributions: every proposal is accepted, and a correction would find no residual
+        if case % 7 == 0:
+            q[0] = 0.0
+            q[0, 0] = 1.0  # a draft certain of one token the target hardly wants
+        proposal = np.array([rng.choice(vocab, p=q[i].astype(np.float64) / q[i].astype(np.float64).sum())
+                             for i in range(K)], np.int32)
+        target = [(ids, p[i]) for i in range(K + 1)]
+        draft = [(ids, q[i]) for i in range(K)]
+        seed = int(rng.integers(0, 2 ** 31))
+        acc2, tok2, used2, au, su = ref.spec_round_sparse(proposal, target, draft, seed)
+        evaluated = min(acc2 + 1, K)
+        acc1, tok1 = orc.spec_verify_dense(p[None], q[None], proposal[None], np.asarray(au, np.float32)[None, :K],
+                                           np.array([su[evaluated]]))
+        assert (int(acc1[0]), int(tok1[0])) == (acc2, tok2), case
+        outcomes.add((acc2 == K, acc2 == 0))
+    assert outcomes >= {(True, False), (False, True), (False, False)}
