@@ -405,62 +405,62 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
     return true;
   }
   if (!presorted) {
-  if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
-  if (best_below != 0) n_c += 1;
-  __syncthreads();
-  bool sorted_done = false;
-  if (n_c > static_cast<uint32_t>(kFinishBlock) && rmax != 0u) {
-    sorted_done = bucket_sort_desc(lds_keys, bucket_start, static_cast<int>(n_c), key_to_float(rmax), key_to_float(thr), red32);
-  }
-  if (!sorted_done) {
-    const int n2 = next_pow2(static_cast<int>(n_c));
-    for (int p = static_cast<int>(n_c) + tid; p < n2; p += blockDim.x) lds_keys[p] = 0;
+    if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
+    if (best_below != 0) n_c += 1;
     __syncthreads();
-    switch (n2 / kFinishBlock) {
-      case 0:
-      case 1: block_sort_desc(lds_keys, n2); break;
-      case 2: block_sort_desc_regs<2>(lds_keys); break;
-      case 4: block_sort_desc_regs<4>(lds_keys); break;
-      case 8: block_sort_desc_regs<8>(lds_keys); break;
-      default: block_sort_desc_regs<16>(lds_keys); break;
+    bool sorted_done = false;
+    if (n_c > static_cast<uint32_t>(kFinishBlock) && rmax != 0u) {
+      sorted_done = bucket_sort_desc(lds_keys, bucket_start, static_cast<int>(n_c), key_to_float(rmax), key_to_float(thr), red32);
     }
-  }
-  if (emit.on()) {
-    // DeviceInterface::TopKScores: the k best ids and their raw scores, best first (the value itself is read again:
-    // keys do not tell -0 from +0); fewer than k numbers among the candidates: the exact path decides
-    const int kk = prm.k < V ? prm.k : V;
-    if (n_c < static_cast<uint32_t>(kk) || lds_keys[kk - 1] == 0) return false;
-    const RowPtr<AnyDtype> lrow(emit.row0, emit.dtype);
-    for (int j = tid; j < kk; j += blockDim.x) {
-      const uint32_t id = key64_index(lds_keys[j]);
-      emit.tokens[j] = static_cast<int32_t>(id);
-      emit.scores[j] = lrow[id];
+    if (!sorted_done) {
+      const int n2 = next_pow2(static_cast<int>(n_c));
+      for (int p = static_cast<int>(n_c) + tid; p < n2; p += blockDim.x) lds_keys[p] = 0;
+      __syncthreads();
+      switch (n2 / kFinishBlock) {
+        case 0:
+        case 1: block_sort_desc(lds_keys, n2); break;
+        case 2: block_sort_desc_regs<2>(lds_keys); break;
+        case 4: block_sort_desc_regs<4>(lds_keys); break;
+        case 8: block_sort_desc_regs<8>(lds_keys); break;
+        default: block_sort_desc_regs<16>(lds_keys); break;
+      }
     }
-    return true;
-  }
-  if (cut_at_best_below && best_below != 0) {
-    // keys are distinct: exactly one thread finds it
-    __shared__ uint32_t cut;
-    for (uint32_t i = tid; i < n_c; i += blockDim.x)
-      if (lds_keys[i] == best_below) cut = i + 1u;
+    if (emit.on()) {
+      // DeviceInterface::TopKScores: the k best ids and their raw scores, best first (the value itself is read again:
+      // keys do not tell -0 from +0); fewer than k numbers among the candidates: the exact path decides
+      const int kk = prm.k < V ? prm.k : V;
+      if (n_c < static_cast<uint32_t>(kk) || lds_keys[kk - 1] == 0) return false;
+      const RowPtr<AnyDtype> lrow(emit.row0, emit.dtype);
+      for (int j = tid; j < kk; j += blockDim.x) {
+        const uint32_t id = key64_index(lds_keys[j]);
+        emit.tokens[j] = static_cast<int32_t>(id);
+        emit.scores[j] = lrow[id];
+      }
+      return true;
+    }
+    if (cut_at_best_below && best_below != 0) {
+      // keys are distinct: exactly one thread finds it
+      __shared__ uint32_t cut;
+      for (uint32_t i = tid; i < n_c; i += blockDim.x)
+        if (lds_keys[i] == best_below) cut = i + 1u;
+      __syncthreads();
+      n_c = cut;
+    }
+    // cache exp((s - max)/T) in the score half of every entry.  The epilogue's threads each read eight consecutive
+    // entries, 64 bytes apart from lane to lane; entry i therefore moves inside its group of eight to slot
+    // (i ^ (i >> 4)) & 7, which spreads those reads over all banks.  A group is read and rewritten by eight
+    // neighbouring lanes in one pass of the loop, so the exchange happens in place.
+    const float max_score = key_to_float(key64_okey(lds_keys[0]));
     __syncthreads();
-    n_c = cut;
-  }
-  // cache exp((s - max)/T) in the score half of every entry.  The epilogue's threads each read eight consecutive
-  // entries, 64 bytes apart from lane to lane; entry i therefore moves inside its group of eight to slot
-  // (i ^ (i >> 4)) & 7, which spreads those reads over all banks.  A group is read and rewritten by eight
-  // neighbouring lanes in one pass of the loop, so the exchange happens in place.
-  const float max_score = key_to_float(key64_okey(lds_keys[0]));
-  __syncthreads();
-  const float inv_temp = 1.0f / prm.temperature;
-  auto slot_of = [](uint32_t i) { return exp_slot(i); };
-  static_assert(kFinishBlock % 8 == 0 && kNucleusCap % 8 == 0, "whole groups per pass");
-  for (uint32_t i = tid; i < ((n_c + 7u) & ~7u); i += blockDim.x) {
-    const u64 k64 = i < n_c ? lds_keys[i] : 0;
-    const float e = em::expf_exact((key_to_float(key64_okey(k64)) - max_score) * inv_temp);
-    lds_keys[slot_of(i)] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k64 & 0xffffffffull);
-  }
-  __syncthreads();
+    const float inv_temp = 1.0f / prm.temperature;
+    auto slot_of = [](uint32_t i) { return exp_slot(i); };
+    static_assert(kFinishBlock % 8 == 0 && kNucleusCap % 8 == 0, "whole groups per pass");
+    for (uint32_t i = tid; i < ((n_c + 7u) & ~7u); i += blockDim.x) {
+      const u64 k64 = i < n_c ? lds_keys[i] : 0;
+      const float e = em::expf_exact((key_to_float(key64_okey(k64)) - max_score) * inv_temp);
+      lds_keys[slot_of(i)] = (static_cast<u64>(__float_as_uint(e)) << 32) | (k64 & 0xffffffffull);
+    }
+    __syncthreads();
   }
   return block_sample_epilogue<8>(sorted, exps, static_cast<int>(n_c), V, prm, u, out, seqsh);
 }
@@ -1074,98 +1074,98 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     }
   }
   if (!presorted && !wide) {
-  bool trim_failed = false;
-  if (!large_k && sh_all >= static_cast<uint32_t>(kNucleusCap)) {  // head == 0 here
-    const float fmax = key_to_float(rmax), fthr = key_to_float(thr);
-    const float span = fmax - fthr;
-    const float scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
-    auto bucket_of = [=](float x) {
-      float bf = (fmax - x) * scale;
-      bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);
-      return bf > 0.0f ? static_cast<int>(bf) : 0;
-    };
-    for (int b = tid; b < kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;
-    __syncthreads();
-    const uint32_t thr0 = thr;
-    flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
+    bool trim_failed = false;
+    if (!large_k && sh_all >= static_cast<uint32_t>(kNucleusCap)) {  // head == 0 here
+      const float fmax = key_to_float(rmax), fthr = key_to_float(thr);
+      const float span = fmax - fthr;
+      const float scale = span > 0.0f ? static_cast<float>(kSortBuckets) / span : 0.0f;
+      auto bucket_of = [=](float x) {
+        float bf = (fmax - x) * scale;
+        bf = bf < static_cast<float>(kSortBuckets - 1) ? bf : static_cast<float>(kSortBuckets - 1);
+        return bf > 0.0f ? static_cast<int>(bf) : 0;
+      };
+      for (int b = tid; b < kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;
+      __syncthreads();
+      const uint32_t thr0 = thr;
+      flat_batches([&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
+#pragma unroll
+        for (int u = 0; u < kGather; ++u) {
+          const float x = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
+          if (valid[u] && order_key(x) >= thr0) atomicAdd(&bucket_start[bucket_of(x)], 1u);
+        }
+      });
+      __syncthreads();
+      // last bucket up to which the candidates fit (one slot stays free for the element after them)
+      if (tid < 64) {
+        constexpr int kPer = kSortBuckets / 64;
+        const uint32_t limit = static_cast<uint32_t>(kNucleusCap - 2);
+        uint32_t own = 0u;
+        for (int i = 0; i < kPer; ++i) own += bucket_start[tid * kPer + i];
+        uint32_t inc = wave_prefix_sum<uint32_t>(own);
+        const int crossing = first_lane(__ballot(inc > limit));  // -1: everything fits
+        if (crossing < 0) {
+          if (tid == 0) sh_trim = kSortBuckets - 1;
+        } else if (tid == crossing) {
+          uint32_t run = inc - own;
+          int last = tid * kPer - 1;
+          for (int i = 0; i < kPer; ++i) {
+            run += bucket_start[tid * kPer + i];
+            if (run > limit) break;
+            last = tid * kPer + i;
+          }
+          sh_trim = last;
+        }
+      }
+      __syncthreads();
+      const int last_bucket = sh_trim;
+      if (last_bucket < 0) {
+        trim_failed = true;  // the best bucket alone does not fit (heavy ties)
+      } else if (last_bucket < kSortBuckets - 1) {
+        // the lowest score whose bucket is still kept: the bucket is a non-increasing function of the score
+        uint32_t lo = thr, hi = rmax;
+        while (lo < hi) {
+          const uint32_t mid = lo + ((hi - lo) >> 1);
+          if (bucket_of(key_to_float(mid)) <= last_bucket) hi = mid;
+          else lo = mid + 1u;
+        }
+        thr = hi;
+      }
+    }
+    // A batch of kGather entries per thread: float bits become order keys, candidates (at or above the
+    // row's threshold) go to LDS at slots a wave reserves with one atomic per batch, the best of the
+    // others is kept.
+    uint32_t lowest = 0xffffffffu;  // lowest candidate key this thread has seen
+    auto consume = [&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
+      u64 k64[kGather], hits[kGather];
+      uint32_t wcnt = 0u;
 #pragma unroll
       for (int u = 0; u < kGather; ++u) {
-        const float x = __uint_as_float(static_cast<uint32_t>(raw[u] >> 32));
-        if (valid[u] && order_key(x) >= thr0) atomicAdd(&bucket_start[bucket_of(x)], 1u);
+        k64[u] = valid[u] ? (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)))) << 32) |
+                                (raw[u] & 0xffffffffull)
+                          : 0;
+        const bool cand = valid[u] && key64_okey(k64[u]) >= thr;
+        hits[u] = __ballot(cand);
+        wcnt += static_cast<uint32_t>(__popcll(hits[u]));
+        if (!cand) best_below = k64[u] > best_below ? k64[u] : best_below;
+        if (cand && key64_okey(k64[u]) < lowest) lowest = key64_okey(k64[u]);
       }
-    });
-    __syncthreads();
-    // last bucket up to which the candidates fit (one slot stays free for the element after them)
-    if (tid < 64) {
-      constexpr int kPer = kSortBuckets / 64;
-      const uint32_t limit = static_cast<uint32_t>(kNucleusCap - 2);
-      uint32_t own = 0u;
-      for (int i = 0; i < kPer; ++i) own += bucket_start[tid * kPer + i];
-      uint32_t inc = wave_prefix_sum<uint32_t>(own);
-      const int crossing = first_lane(__ballot(inc > limit));  // -1: everything fits
-      if (crossing < 0) {
-        if (tid == 0) sh_trim = kSortBuckets - 1;
-      } else if (tid == crossing) {
-        uint32_t run = inc - own;
-        int last = tid * kPer - 1;
-        for (int i = 0; i < kPer; ++i) {
-          run += bucket_start[tid * kPer + i];
-          if (run > limit) break;
-          last = tid * kPer + i;
-        }
-        sh_trim = last;
-      }
-    }
-    __syncthreads();
-    const int last_bucket = sh_trim;
-    if (last_bucket < 0) {
-      trim_failed = true;  // the best bucket alone does not fit (heavy ties)
-    } else if (last_bucket < kSortBuckets - 1) {
-      // the lowest score whose bucket is still kept: the bucket is a non-increasing function of the score
-      uint32_t lo = thr, hi = rmax;
-      while (lo < hi) {
-        const uint32_t mid = lo + ((hi - lo) >> 1);
-        if (bucket_of(key_to_float(mid)) <= last_bucket) hi = mid;
-        else lo = mid + 1u;
-      }
-      thr = hi;
-    }
-  }
-  // A batch of kGather entries per thread: float bits become order keys, candidates (at or above the
-  // row's threshold) go to LDS at slots a wave reserves with one atomic per batch, the best of the
-  // others is kept.
-  uint32_t lowest = 0xffffffffu;  // lowest candidate key this thread has seen
-  auto consume = [&](const u64 (&raw)[kGather], const bool (&valid)[kGather], uint32_t) {
-    u64 k64[kGather], hits[kGather];
-    uint32_t wcnt = 0u;
+      uint32_t base = 0u;
+      if (lane == 0 && wcnt != 0u) base = atomicAdd(&sh_count, wcnt);
+      base = __builtin_amdgcn_readfirstlane(base);
 #pragma unroll
-    for (int u = 0; u < kGather; ++u) {
-      k64[u] = valid[u] ? (static_cast<u64>(order_key(__uint_as_float(static_cast<uint32_t>(raw[u] >> 32)))) << 32) |
-                              (raw[u] & 0xffffffffull)
-                        : 0;
-      const bool cand = valid[u] && key64_okey(k64[u]) >= thr;
-      hits[u] = __ballot(cand);
-      wcnt += static_cast<uint32_t>(__popcll(hits[u]));
-      if (!cand) best_below = k64[u] > best_below ? k64[u] : best_below;
-      if (cand && key64_okey(k64[u]) < lowest) lowest = key64_okey(k64[u]);
-    }
-    uint32_t base = 0u;
-    if (lane == 0 && wcnt != 0u) base = atomicAdd(&sh_count, wcnt);
-    base = __builtin_amdgcn_readfirstlane(base);
-#pragma unroll
-    for (int u = 0; u < kGather; ++u) {
-      const uint32_t pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(hits[u] >> 32),
-                                                     __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(hits[u]), base));
-      if (((hits[u] >> lane) & 1ull) && pos < kNucleusCap) lds_keys[pos] = k64[u];
-      base += static_cast<uint32_t>(__popcll(hits[u]));
-    }
-  };
-  listed_batches(consume);
-  best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
-  n_c = sh_count;
-  ok = !gave_up && !trim_failed && n_c < kNucleusCap;  // room for the next-best element too
-  if (large_k) thr = ~block_max<uint32_t>(~lowest, red32);  // the lowest candidate score: the sort scales its buckets by it
-  if (ok && !large_k) trim_to_nucleus(lds_keys, bucket_start, n_c, best_below, rmax, thr, prm, V, red32, red64, &sh_count);
+      for (int u = 0; u < kGather; ++u) {
+        const uint32_t pos = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(hits[u] >> 32),
+                                                       __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(hits[u]), base));
+        if (((hits[u] >> lane) & 1ull) && pos < kNucleusCap) lds_keys[pos] = k64[u];
+        base += static_cast<uint32_t>(__popcll(hits[u]));
+      }
+    };
+    listed_batches(consume);
+    best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
+    n_c = sh_count;
+    ok = !gave_up && !trim_failed && n_c < kNucleusCap;  // room for the next-best element too
+    if (large_k) thr = ~block_max<uint32_t>(~lowest, red32);  // the lowest candidate score: the sort scales its buckets by it
+    if (ok && !large_k) trim_to_nucleus(lds_keys, bucket_start, n_c, best_below, rmax, thr, prm, V, red32, red64, &sh_count);
   }
   if (ok) {
     const bool emit = large_k && a.emit_topk == 1;
@@ -1522,37 +1522,37 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   }
   const bool presorted = n_c != 0u;
   if (!presorted) {
-  // candidates (at or above the threshold) go to the sort buffer at slots a wave reserves with one atomic per
-  // batch; the best of the others is kept
+    // candidates (at or above the threshold) go to the sort buffer at slots a wave reserves with one atomic per
+    // batch; the best of the others is kept
 #pragma unroll
-  for (int u0 = 0; u0 < kSparseIds + kSparseExtraRegs; u0 += 6) {
-    u64 hits[6];
-    uint32_t wcnt = 0u;
+    for (int u0 = 0; u0 < kSparseIds + kSparseExtraRegs; u0 += 6) {
+      u64 hits[6];
+      uint32_t wcnt = 0u;
 #pragma unroll
-    for (int u = u0; u < u0 + 6 && u < kSparseIds + kSparseExtraRegs; ++u) {
-      const bool have = ids[u] != 0xffffffffu;
-      const uint32_t ok32 = have ? ok[u] : 0u;
-      const bool cand = have && ok32 >= thr;
-      hits[u - u0] = __ballot(cand);
-      wcnt += static_cast<uint32_t>(__popcll(hits[u - u0]));
-      if (have && !cand) {
-        const u64 k64 = make_key64(ok32, ids[u]);
-        best_below = k64 > best_below ? k64 : best_below;
+      for (int u = u0; u < u0 + 6 && u < kSparseIds + kSparseExtraRegs; ++u) {
+        const bool have = ids[u] != 0xffffffffu;
+        const uint32_t ok32 = have ? ok[u] : 0u;
+        const bool cand = have && ok32 >= thr;
+        hits[u - u0] = __ballot(cand);
+        wcnt += static_cast<uint32_t>(__popcll(hits[u - u0]));
+        if (have && !cand) {
+          const u64 k64 = make_key64(ok32, ids[u]);
+          best_below = k64 > best_below ? k64 : best_below;
+        }
+      }
+      uint32_t base = 0u;
+      if (lane == 0 && wcnt != 0u) base = atomicAdd(&sh_count, wcnt);
+      base = __builtin_amdgcn_readfirstlane(base);
+#pragma unroll
+      for (int u = u0; u < u0 + 6 && u < kSparseIds + kSparseExtraRegs; ++u) {
+        const u64 b = hits[u - u0];
+        const uint32_t p = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), base));
+        if ((b >> lane) & 1ull) lds_keys[p] = make_key64(ok[u], ids[u]);
+        base += static_cast<uint32_t>(__popcll(b));
       }
     }
-    uint32_t base = 0u;
-    if (lane == 0 && wcnt != 0u) base = atomicAdd(&sh_count, wcnt);
-    base = __builtin_amdgcn_readfirstlane(base);
-#pragma unroll
-    for (int u = u0; u < u0 + 6 && u < kSparseIds + kSparseExtraRegs; ++u) {
-      const u64 b = hits[u - u0];
-      const uint32_t p = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(b >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(b), base));
-      if ((b >> lane) & 1ull) lds_keys[p] = make_key64(ok[u], ids[u]);
-      base += static_cast<uint32_t>(__popcll(b));
-    }
-  }
-  best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
-  n_c = sh_count;
+    best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
+    n_c = sh_count;
   }
   return leave(finish_candidates(lds_keys, bucket_start, n_c, presorted ? 0 : best_below, rmax, thr, false, prm, V, a.uniforms[row],
                                  row_outputs(a, row), seqsh, red32, EmitTopk{}, presorted));
