@@ -950,45 +950,49 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       const u64 key = make_key64(order_key(ev), ei);
       if (ev < thr2 && key > extra_below) extra_below = key;
     }
-    // The best element below the threshold, first of equals: the block agrees on the best score, then
-    // the few threads that hold it look up its lowest id.
-    float thr3 = thr;
-    asm volatile("" : "+v"(thr3));
-    float fb = -__builtin_inff();
-#pragma unroll
-    for (int e = 0; e < kSElems; ++e) {
-      if (v[e] < thr3 && v[e] > fb) fb = v[e];  // compares are false for NaN
-      __builtin_amdgcn_sched_barrier(0);        // each lane mask is used at once
-    }
-    uint32_t fbk = 0u;  // 0: the thread has no element below the threshold
-    if (fb > -__builtin_inff()) {
-      fbk = order_key(fb);
-    } else if (thr3 > -__builtin_inff()) {  // an element equal to -inf is one, too
-      bool any = false;
-#pragma unroll
-      for (int e = 0; e < kSElems; ++e) any = any || v[e] == -__builtin_inff();
-      if (any) fbk = order_key(-__builtin_inff());
-    }
-    const uint32_t ebk = key64_okey(extra_below);
-    const uint32_t own = fbk > ebk ? fbk : ebk;
-    const uint32_t wbk = wave_max<uint32_t>(own);  // (the wave first: one exchange between the waves, of whole keys)
     u64 best_below = 0;
-    if (wbk != 0u && own == wbk) {
-      best_below = ebk == wbk ? extra_below : 0;
-      if (fbk == wbk) {
-        const float bbf = key_to_float(wbk);
-        int fe = 0;
+    if constexpr (!LARGEK) {  // (a top-k row's kept set ends with its k-th element: nothing below the list is ever needed)
+      // The best element below the threshold, first of equals: the block agrees on the best score, then
+      // the few threads that hold it look up its lowest id.
+      float thr3 = thr;
+      asm volatile("" : "+v"(thr3));
+      float fb = -__builtin_inff();
 #pragma unroll
-        for (int e = kSElems - 1; e >= 0; --e)
-          if (v[e] == bbf) fe = e;
-        const u64 key = make_key64(wbk, static_cast<uint32_t>(elem_index<kSBlock, VEC>(chunk, fe >> 2, fe & 3)));
-        best_below = key > best_below ? key : best_below;
+      for (int e = 0; e < kSElems; ++e) {
+        if (v[e] < thr3 && v[e] > fb) fb = v[e];  // compares are false for NaN
+        __builtin_amdgcn_sched_barrier(0);        // each lane mask is used at once
+      }
+      uint32_t fbk = 0u;  // 0: the thread has no element below the threshold
+      if (fb > -__builtin_inff()) {
+        fbk = order_key(fb);
+      } else if (thr3 > -__builtin_inff()) {  // an element equal to -inf is one, too
+        bool any = false;
+#pragma unroll
+        for (int e = 0; e < kSElems; ++e) any = any || v[e] == -__builtin_inff();
+        if (any) fbk = order_key(-__builtin_inff());
+      }
+      const uint32_t ebk = key64_okey(extra_below);
+      const uint32_t own = fbk > ebk ? fbk : ebk;
+      const uint32_t wbk = wave_max<uint32_t>(own);  // (the wave first: one exchange between the waves, of whole keys)
+      if (wbk != 0u && own == wbk) {
+        best_below = ebk == wbk ? extra_below : 0;
+        if (fbk == wbk) {
+          const float bbf = key_to_float(wbk);
+          int fe = 0;
+#pragma unroll
+          for (int e = kSElems - 1; e >= 0; --e)
+            if (v[e] == bbf) fe = e;
+          const u64 key = make_key64(wbk, static_cast<uint32_t>(elem_index<kSBlock, VEC>(chunk, fe >> 2, fe & 3)));
+          best_below = key > best_below ? key : best_below;
+        }
       }
     }
-    best_below = wave_max<u64>(best_below);
-    if (lane == 0) sm.wave_val64[wave] = best_below;
+    if constexpr (!LARGEK) {
+      best_below = wave_max<u64>(best_below);
+      if (lane == 0) sm.wave_val64[wave] = best_below;
+    }
     lds_barrier();  // (also orders the atomics on sm.count)
-    best_below = wave_max<u64>(lane < kSWaves ? sm.wave_val64[lane] : 0);
+    if constexpr (!LARGEK) best_below = wave_max<u64>(lane < kSWaves ? sm.wave_val64[lane] : 0);
     if (tid == 0) {
       const size_t ci = static_cast<size_t>(row) * a.chunks + chunk;
       a.chunk_cnt[ci] = extra_overflow ? kChunkCntOverflow : sm.count;
