@@ -902,10 +902,16 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       }
       if (kth != 0u) thr = key_to_float(kth);
     }
-    // First pass: the wave's number of candidates.
+    // First pass: the wave's number of candidates, and (nucleus rows) the thread's best element below the threshold,
+    // from the same compare.
     uint32_t wcnt = 0u;
+    float fb = -__builtin_inff();
 #pragma unroll
-    for (int e = 0; e < kSElems; ++e) wcnt += static_cast<uint32_t>(__popcll(__ballot(v[e] >= thr)));  // false for NaN
+    for (int e = 0; e < kSElems; ++e) {
+      const bool cand = v[e] >= thr;  // false for NaN
+      wcnt += static_cast<uint32_t>(__popcll(__ballot(cand)));
+      if constexpr (!LARGEK) fb = fmaxf(fb, cand ? -__builtin_inff() : v[e]);  // (fmaxf passes a NaN by)
+    }
     for (uint32_t i0 = 0; i0 < n_extra; i0 += kSBlock) {
       const uint32_t i = i0 + tid;
       wcnt += static_cast<uint32_t>(__popcll(__ballot(i < n_extra && sm.extra_val[i] >= thr)));
@@ -956,12 +962,6 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       // the few threads that hold it look up its lowest id.
       float thr3 = thr;
       asm volatile("" : "+v"(thr3));
-      float fb = -__builtin_inff();
-#pragma unroll
-      for (int e = 0; e < kSElems; ++e) {
-        if (v[e] < thr3 && v[e] > fb) fb = v[e];  // compares are false for NaN
-        __builtin_amdgcn_sched_barrier(0);        // each lane mask is used at once
-      }
       uint32_t fbk = 0u;  // 0: the thread has no element below the threshold
       if (fb > -__builtin_inff()) {
         fbk = order_key(fb);
