@@ -771,44 +771,49 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
     pre[q] = (a.chunks <= kAheadChunks && c < a.chunks) ? big_row[static_cast<size_t>(c) * kSChunk + u * kFinishBlock + tid] : 0;
   }
   for (int b = tid; b <= kSortBuckets; b += kFinishBlock) bucket_start[b] = 0u;  // the sort's table, while the loads are on their way
-  // Thread c reads everything chunk c left behind; the barriers of the first reduction publish the counts.
+  // Lane c of every wave reads what chunk c left behind (at most 16 chunks), so the row's maximum and threshold
+  // are reductions inside the wave, with no exchange between the waves; wave 0 publishes the counts and where
+  // every list's rows begin, behind the one barrier that follows.
   __shared__ uint32_t sh_cnt[kAllCap / kSmallCap];       // candidates per chunk
   __shared__ uint32_t sh_first[kAllCap / kSmallCap + 1];  // rows of kFinishBlock entries the lists past their heads take, prefix sums
   __shared__ int sh_trim;
   __shared__ uint32_t sh_head, sh_all;
-  uint32_t m = 0u, cthr = 0u;
+  static_assert(kAllCap / kSmallCap < 64, "a lane per chunk, and one more");
+  const int lane = lane_id();
+  uint32_t cnt = 0u, m = 0u, cthr = 0u;
   u64 best_below = 0;
+  if (lane < a.chunks) {
+    cnt = a.chunk_cnt[cbase + lane];
+    m = cnt == kChunkCntOverflow ? 0xffffffffu : a.chunk_max[cbase + lane];  // above every key: the exact path
+    cthr = a.chunk_thr[cbase + lane];
+  }
   if (tid < a.chunks) {
-    const uint32_t cnt = a.chunk_cnt[cbase + tid];
-    m = cnt == kChunkCntOverflow ? 0xffffffffu : a.chunk_max[cbase + tid];  // above every key: the exact path
-    cthr = a.chunk_thr[cbase + tid];
     best_below = large_k ? 0 : a.chunk_next[cbase + tid];
     sh_cnt[tid] = cnt;
   }
   if (tid == 0) sh_count = 0u;
-  const uint32_t rmax = block_max<uint32_t>(m, red32);
+  const uint32_t rmax = wave_max<uint32_t>(m);
   const bool gave_up = rmax == 0xffffffffu;
   // Every chunk's threshold holds for the whole row (no element of the row below it lies strictly inside the
   // nucleus; a chunk alone has k elements at or above its own), so the highest one is the row's: every element at
   // or above it is in its chunk's list.
-  uint32_t thr = block_max<uint32_t>(cthr, red32);
+  uint32_t thr = wave_max<uint32_t>(cthr);
   if (rmax == 0u) thr = 0u;  // (no number in the row)
-  if (tid == 0) {
-    uint32_t all = 0u;
-    for (int c = 0; c < a.chunks; ++c) all += gave_up ? 0u : sh_cnt[c];
+  if (tid < 64) {
+    const uint32_t listed = gave_up ? 0u : cnt;
+    const uint32_t all = wave_sum<uint32_t>(listed);
     const uint32_t head =
         (a.chunks <= kAheadChunks && all < static_cast<uint32_t>(kNucleusCap)) ? static_cast<uint32_t>(kFinishBlock) << head_shift : 0u;
-    uint32_t run = 0u;  // (in rows of kFinishBlock entries: a row lies in one chunk's list, so its chunk is found once for all threads)
-    for (int c = 0; c < a.chunks; ++c) {
-      sh_first[c] = run;
-      run += (gave_up || sh_cnt[c] <= head) ? 0u : (sh_cnt[c] - head + kFinishBlock - 1u) / kFinishBlock;
+    // (in rows of kFinishBlock entries: a row lies in one chunk's list, so its chunk is found once for all threads)
+    const uint32_t rows = listed <= head ? 0u : (listed - head + kFinishBlock - 1u) / kFinishBlock;
+    const uint32_t before = wave_prefix_sum<uint32_t>(rows) - rows;
+    if (lane <= a.chunks) sh_first[lane] = before;  // (lane a.chunks: all of them)
+    if (lane == 0) {
+      sh_head = head;
+      sh_all = all;
     }
-    sh_first[a.chunks] = run;
-    sh_head = head;
-    sh_all = all;
   }
   __syncthreads();
-  const int lane = lane_id();
   // The chunks' lists past their heads, as a sequence of rows of kFinishBlock entries (sh_first[c] = rows of the
   // chunks before c; a list's last row may be short).  A cursor walks the rows in order; which chunk a row lies in
   // is the same for every thread, so finding it costs the threads nothing.
