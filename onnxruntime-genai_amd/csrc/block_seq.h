@@ -41,11 +41,9 @@ __device__ __forceinline__ void block_min2(int& a, int& b, SeqShared& sh) {
     sh.red_b[wave] = b;
   }
   __syncthreads();
-  int ra = sh.red_a[0], rb = sh.red_b[0];
-  for (int w = 1; w < nw; ++w) {
-    ra = sh.red_a[w] < ra ? sh.red_a[w] : ra;
-    rb = sh.red_b[w] < rb ? sh.red_b[w] : rb;
-  }
+  // lane w looks at wave w's pair (at most sixteen waves); ~v reverses the order of ints
+  const int ra = -1 - row16_max<int>(-1 - (lane < nw ? sh.red_a[lane] : kIntMax));
+  const int rb = -1 - row16_max<int>(-1 - (lane < nw ? sh.red_b[lane] : kIntMax));
   __syncthreads();
   a = ra;
   b = rb;
@@ -516,7 +514,7 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float
     }
     draw_scan_thread<ITEMS>(pv, wp + (inc - loc), loc, base, n, target, guard, first, risky);
     carry += block_total;
-    __syncthreads();
+    if (i0 + span < n) __syncthreads();  // (the next window writes the waves' sums again; after the last one nothing does)
   }
   int a = first, b = risky ? 0 : 1;
   block_min2(a, b, sh);

@@ -152,16 +152,30 @@ __device__ __forceinline__ T wave_sort_desc(T x) {
   return x;
 }
 
-// Block-wide maximum; every thread gets the result.  `scratch` holds >= blockDim/64 entries.
+// Maximum over the first sixteen lanes (four lane-shifting steps inside the row); every lane gets the result.
 template <typename T>
-__device__ __forceinline__ T block_max(T v, T* scratch) {
+__device__ __forceinline__ T row16_max(T v) {
+#define MS_STEP(CTRL)                                        \
+  {                                                          \
+    const T o = dpp_from_below_or<CTRL, 0xf, T>(v, v);       \
+    v = o > v ? o : v;                                       \
+  }
+  MS_STEP(0x111) MS_STEP(0x112) MS_STEP(0x114) MS_STEP(0x118)
+#undef MS_STEP
+  return wave_read_lane(v, 15);
+}
+
+// Block-wide maximum of unsigned values; every thread gets the result.  `scratch` holds >= blockDim/64 entries
+// (at most sixteen waves).  Two barriers: the second one lets the caller write `scratch` again at once; a caller
+// that leaves it alone until its next barrier passes reuse_at_once = false and saves it.
+template <typename T>
+__device__ __forceinline__ T block_max(T v, T* scratch, bool reuse_at_once = true) {
   v = wave_max(v);
   const int lane = lane_id(), wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   if (lane == 0) scratch[wave] = v;
   __syncthreads();
-  T r = scratch[0];
-  for (int w = 1; w < nw; ++w) r = scratch[w] > r ? scratch[w] : r;
-  __syncthreads();
+  const T r = row16_max<T>(lane < nw ? scratch[lane] : T(0));  // lane w looks at wave w's
+  if (reuse_at_once) __syncthreads();
   return r;
 }
 

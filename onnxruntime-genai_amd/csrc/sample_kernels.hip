@@ -673,7 +673,8 @@ __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start,
     c += cnt[i];
   }
   if (t == kFinishBlock - 1) start[kSortBuckets] = c;
-  const uint32_t red = block_max<uint32_t>(big ? 0xffffffffu : ~mine, red32);  // its barriers also publish the starts
+  // (its barrier also publishes the starts; red32 is not written again before the callers' next barrier)
+  const uint32_t red = block_max<uint32_t>(big ? 0xffffffffu : ~mine, red32, false);
   TrimmedBuckets r{static_cast<uint32_t>(kSortBuckets), n_cand, 0u, 0, 0u};
   if (red == 0xffffffffu) return r;
   const uint32_t last_thread = (~red) >> 2;
