@@ -31,8 +31,9 @@ struct SeqShared {
 
 __device__ __forceinline__ int wave_min_i(int v) { return -1 - wave_max<int>(-1 - v); }  // ~v reverses the order of ints
 
-// Minimum of two ints over the block (both reduced at once).  Contains two barriers.
-__device__ __forceinline__ void block_min2(int& a, int& b, SeqShared& sh) {
+// Minimum of two ints over the block (both reduced at once).  Contains two barriers; the second one lets the next
+// call follow at once, and a caller that has no next call before another barrier saves it (reuse_at_once = false).
+__device__ __forceinline__ void block_min2(int& a, int& b, SeqShared& sh, bool reuse_at_once = true) {
   a = wave_min_i(a);
   b = wave_min_i(b);
   const int lane = lane_id(), wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
@@ -44,7 +45,7 @@ __device__ __forceinline__ void block_min2(int& a, int& b, SeqShared& sh) {
   // lane w looks at wave w's pair (at most sixteen waves); ~v reverses the order of ints
   const int ra = -1 - row16_max<int>(-1 - (lane < nw ? sh.red_a[lane] : kIntMax));
   const int rb = -1 - row16_max<int>(-1 - (lane < nw ? sh.red_b[lane] : kIntMax));
-  __syncthreads();
+  if (reuse_at_once) __syncthreads();
   a = ra;
   b = rb;
 }
@@ -213,14 +214,14 @@ struct StopAtNucleus {
 // predicate holds.  Passes cost two barriers; there is one per window plus one per binade change.
 template <int ITEMS, typename GetE, typename StopFn>
 __device__ float block_seq_sum(float s0, int n, GetE get, StopFn stop, int* stop_index, SeqShared& sh,
-                               float* stage = nullptr, int head = 0) {
+                               float* stage = nullptr, int head = 0, bool synced = false) {
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6, nw = static_cast<int>(blockDim.x) >> 6;
   const int span = static_cast<int>(blockDim.x) * ITEMS;
   constexpr uint32_t kNone = 0xffffffffu;
   float s = s0;
   int found = -1;
   int par = 0;
-  __syncthreads();  // a previous call's readers are done with the parity-0 buffers
+  if (!synced) __syncthreads();  // a previous call's readers are done with the parity-0 buffers (synced: the caller vouches)
   // A sum that starts from nothing changes binade every few additions, and each change costs a pass
   // of the scan below.  The first `head` elements are therefore added for real, 64 at a time, by a
   // chain of lane-shifted float additions in wave 0 (about ten cycles per element).  The head ends early once 64
@@ -517,7 +518,7 @@ __device__ int block_discrete_draw(int n, GetW w, double u, SeqShared& sh, float
     if (i0 + span < n) __syncthreads();  // (the next window writes the waves' sums again; after the last one nothing does)
   }
   int a = first, b = risky ? 0 : 1;
-  block_min2(a, b, sh);
+  block_min2(a, b, sh, false);  // (the one reduction of a draw; the replay below has barriers of its own)
   if (b != 0) return a;
   // Sequential replay (reached with probability ~ n^2 * 1e-15 per draw).
   if (tid == 0) {
@@ -652,11 +653,12 @@ struct RowOutputs {
 // (src/sampling_distribution.h:218-297) on a row whose elements are available in rank order:
 // sorted(i) returns the key64 of the i-th best element for i < n_sorted.  exps(i) must return
 // exp((score_i - score_0) * inv_temp) as a float (callers may cache it).  Returns false -- without
-// writing outputs -- when the nucleus does not end inside the n_sorted available elements.
+// writing outputs -- when the nucleus does not end inside the n_sorted available elements.  synced: every thread
+// has passed a barrier since `sh` was last used, so the first sum need not begin with one.
 template <int ITEMS, typename Sorted, typename Exps>
 __device__ __forceinline__ bool block_sample_epilogue(Sorted sorted, Exps exps, int n_sorted, int vocab,
                                       mi355x_sample_params prm, double u, const RowOutputs& out,
-                                      SeqShared& sh) {
+                                      SeqShared& sh, bool synced = false) {
   int keep;
   float scale;     // kept probability j = base_j * scale, base_j = exps(j) or exps(j)/sum
   float sum = 1.0f;
@@ -665,7 +667,7 @@ __device__ __forceinline__ bool block_sample_epilogue(Sorted sorted, Exps exps, 
   if (prm.k > 1) {
     const int m = prm.k < vocab ? prm.k : vocab;
     if (m > n_sorted) return false;
-    sum = block_seq_sum<ITEMS>(0.0f, m, exps, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead);
+    sum = block_seq_sum<ITEMS>(0.0f, m, exps, NoStop{}, &idx_dummy, sh, nullptr, kEpiHead, synced);
     divide_by_sum = sum > 0.0f;
     const float ssum = sum;
     const bool dv = divide_by_sum;
@@ -700,7 +702,7 @@ __device__ __forceinline__ bool block_sample_epilogue(Sorted sorted, Exps exps, 
       const int b = base;
       int si;
       prefix = block_seq_sum<ITEMS>(prefix, limit - b, [=](int i) { return exps(i + b); }, StopAtNucleus{p, V, b}, &si, sh,
-                                    nullptr, b == 0 ? kEpiHead : 0);
+                                    nullptr, b == 0 ? kEpiHead : 0, synced && b == 0);
       if (si < 0) {
         if (limit != vocab) return false;
         cutoff = vocab;

@@ -462,7 +462,7 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
     }
     __syncthreads();
   }
-  return block_sample_epilogue<8>(sorted, exps, static_cast<int>(n_c), V, prm, u, out, seqsh);
+  return block_sample_epilogue<8>(sorted, exps, static_cast<int>(n_c), V, prm, u, out, seqsh, true);  // (a barrier has just passed)
 }
 
 // Drops the candidates that certainly lie past the end of the nucleus, so that only the rest is sorted.
@@ -1075,7 +1075,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
         const u64* list = far;
         wide_ok = block_sample_epilogue<8>([=](int i) { return list[i]; },
                                            [=](int i) { return __uint_as_float(static_cast<uint32_t>(list[i] >> 32)); },
-                                           static_cast<int>(n_list), V, prm, a.uniforms[row], row_outputs(a, row), seqsh);
+                                           static_cast<int>(n_list), V, prm, a.uniforms[row], row_outputs(a, row), seqsh, true);
       }
     }
   }
@@ -1303,7 +1303,7 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   float* const extra_val = reinterpret_cast<float*>(bucket_start);
   uint32_t* const extra_idx = bucket_start + kSparseExtras;
   __shared__ SeqShared seqsh;
-  __shared__ uint32_t red32[16];
+  __shared__ uint32_t red32[16], red32_rest[16];  // (two: the reductions below follow each other without a barrier between)
   __shared__ u64 red64[16];
   __shared__ uint32_t sh_extra, sh_count;
   const int row = blockIdx.x, tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
@@ -1496,7 +1496,7 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   uint32_t kmax = keys_of_slots(std::integral_constant<int, 0>{}, std::integral_constant<int, kFirstLoads>{});
 #pragma unroll
   for (int u = kSparseIds; u < kSparseRegs; ++u) kmax = ok[u] > kmax ? ok[u] : kmax;
-  const uint32_t rtop = block_max<uint32_t>(kmax, red32);  // its barriers end every read of the id list and the extras
+  const uint32_t rtop = block_max<uint32_t>(kmax, red32, false);  // (red32 is next written behind a later barrier)
   if (rtop == 0u) return leave(false);
   const uint32_t thr = order_key(key_to_float(rtop) - nucleus_depth(prm, V));
   if (thr <= order_key(kLowest)) return leave(false);  // masked ids would be candidates themselves
@@ -1508,7 +1508,7 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   }
   uint32_t rmax = rtop;
   if (static_cast<uint32_t>(kFirstLoads * kFinishBlock) < n_allowed) {
-    const uint32_t rest = block_max<uint32_t>(keys_of_slots(std::integral_constant<int, kFirstLoads>{}, std::integral_constant<int, kSparseIds>{}), red32);
+    const uint32_t rest = block_max<uint32_t>(keys_of_slots(std::integral_constant<int, kFirstLoads>{}, std::integral_constant<int, kSparseIds>{}), red32_rest, false);
     rmax = rest > rmax ? rest : rmax;
     if (direct) count_gathered<kFirstLoads, kSparseIds>(bucket_start, ids, ok, bucket_of, thr, best_below, n_allowed, n_extra);
   } else {

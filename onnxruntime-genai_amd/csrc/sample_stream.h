@@ -513,9 +513,8 @@ __device__ __forceinline__ T block_max_lds(T v, T* scratch) {
   const int lane = lane_id(), wave = threadIdx.x >> 6;
   if (lane == 0) scratch[wave] = v;
   lds_barrier();
-  T r = scratch[0];
-#pragma unroll
-  for (int w = 1; w < kSWaves; ++w) r = scratch[w] > r ? scratch[w] : r;
+  static_assert(kSWaves <= 16, "a lane per wave inside one row of lanes");
+  const T r = row16_max<T>(lane < kSWaves ? scratch[lane] : T(0));  // lane w looks at wave w's
   lds_barrier();
   return r;
 }
@@ -1059,9 +1058,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     lds_barrier();
     if (wave != 0 && !finisher) return false;
     if (wave == 0) {
-      uint32_t best = 0u;  // ~id of the lowest id
-#pragma unroll
-      for (int w = 0; w < kSWaves; ++w) best = sm.wave_val[w] > best ? sm.wave_val[w] : best;
+      const uint32_t best = row16_max<uint32_t>(lane < kSWaves ? sm.wave_val[lane] : 0u);  // ~id of the lowest id
       u64 key = best != 0u ? (static_cast<u64>(cmax) << 32) | best : 0;
       if (chunk == 0 && sm.nan0 != 0u) key = ~0ull;
       if (n_chunks == 1) {  // the row is this chunk: nothing to hand over
