@@ -14,7 +14,7 @@ HBM_PEAK_GBS = 8000.0
 # known-size copy; counters cannot be read from inside the process, so these are offline profile constants.
 # c3: KV gather 6.22 GB + selection kernels 0.04 GB; c5: the one sparse-mask kernel; topp: stream (fetch + write) and
 # finish kernel.  None where no counter run exists.
-MEASURED_TRAFFIC = {"c3": 6_222_000_000 + 42_000_000, "c5": 203_300_000, "topp": 33_000_000 + 5_300_000 + 9_200_000}
+MEASURED_TRAFFIC = {"c3": 6_222_000_000 + 42_000_000, "c5": 203_900_000, "topp": 33_000_000 + 5_300_000 + 9_200_000}
 TRAFFIC_SOURCE = {"c3": "offline profile constant: profiles/beam_step_kernels_config3.md",
                   "c5": "offline profile constant: profiles/nucleus_sparse_kernel_config5.md",
                   "topp": "offline profile constant: profiles/nucleus_stream_and_finish_kernels_top_p_and_large_k.md"}
