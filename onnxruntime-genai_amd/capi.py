@@ -251,7 +251,8 @@ class SearchContext:
         """Marshals one mi355x_sample call once and returns a function that issues it: what a serving loop with fixed
         buffers does (the tensors, `xf` and the stream -- default: the stream current now -- must stay alive and
         where they are; the function takes no arguments and raises on an error code).  `out` may be pinned host
-        memory.  The per-call cost is the foreign call alone, none of the tensor lookups of `sample`."""
+        memory.  The per-call cost is the foreign call alone, none of the tensor lookups of `sample`.  As with every
+        call, one context serves one stream at a time: calls prepared for different streams must not overlap."""
         rows, vocab, stride = self._rows(logits)
         assert uniforms.dtype == torch.float64 and uniforms.numel() >= rows and out.dtype == torch.int32 and out.numel() >= rows
         handle = C.c_void_p(stream.cuda_stream) if stream is not None else _stream()

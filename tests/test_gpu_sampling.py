@@ -346,9 +346,9 @@ def test_prepared_sample_calls_give_the_same_tokens(ctx, orc):
         out_dev.fill_(-1)
         out_pin.fill_(-1)
         torch.cuda.synchronize()
-        for call in calls:
+        for call in calls:  # (one after the other: calls on one context must not overlap, whatever their streams)
             call()
-        torch.cuda.synchronize()
+            torch.cuda.synchronize()
         assert np.array_equal(out_dev.cpu().numpy(), want)
         assert np.array_equal(out_pin.numpy(), want)
     xh = torch.from_numpy(x.astype(np.float16)).cuda()
