@@ -597,8 +597,8 @@ struct ScoreBuckets {
 };
 
 // What the scan keeps: the keys of buckets 0 .. last_bucket, n_sorted of them, in a list of n entries (one more
-// when best_below, the best element below every candidate, follows them).  n = 0: a bucket holds more than
-// kBucketCap keys (or the first thread's buckets alone overflow the room), the caller sorts another way.
+// when best_below, the best element below every candidate, follows them).  n = 0: the first thread's run of buckets
+// alone overflows the room or holds a bucket of more than bucket_cap keys; the caller sorts another way.
 struct TrimmedBuckets {
   uint32_t last_bucket, n_sorted, n;
   u64 best_below;
@@ -898,8 +898,8 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
   // LDS.  However long the lists are, only what is kept has to fit.  A bucket with too many keys (heavy ties) leaves
   // the row to the steps below: the list in LDS, trimmed, and the sorting network.
   bool presorted = false, ok = false;
-  // A row that goes the way of nuclei wider than the sort (decided after the first scan, done at the kernel's end;
-  // kept in LDS, not in registers, in between): the threads whose runs of buckets the nucleus needs (0: not such a
+  // A row that goes the way of nuclei wider than the sort (decided after the first scan, done behind the usual
+  // path's code; kept in LDS, not in registers, in between): the threads whose runs of buckets the nucleus needs (0: not such a
   // row), the entries of its list, and the best element below the candidates when it follows them.
   __shared__ uint32_t sh_wide_end_t, sh_wide_n;
   __shared__ u64 sh_wide_below;
@@ -932,7 +932,7 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       // bucket too full for the usual ranking.  The same sort then runs over the row's second key buffer in global
       // memory: every needed key goes to a place of its bucket's there, the buckets are ranked in rounds through LDS,
       // and the epilogue reads the list from there.  Still a fraction of the exact path's work: the histogram's bound
-      // of the nucleus says which buckets are needed.  Decided here, done at the kernel's end.  (Lists short enough
+      // of the nucleus says which buckets are needed.  Decided here, done behind the usual path's code.  (Lists short enough
       // for the head in registers fit the room: there only a bucket too full gets here, and the steps below take
       // the row, as they do when a bucket is too full even for the rounds.)
       if (kept.more != 0u && head == 0u && a.big2 != nullptr) {
