@@ -662,7 +662,8 @@ __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start,
       mine = 4u * static_cast<uint32_t>(t);
   }
   if (want > 0 && c < static_cast<uint32_t>(want) && c + local >= static_cast<uint32_t>(want)) mine = 4u * static_cast<uint32_t>(t);
-  if (c + local > static_cast<uint32_t>(room - 2) || big != 0u) {
+  const bool run_fits = !(c + local > static_cast<uint32_t>(room - 2) || big != 0u);  // (this thread's run, with all before it)
+  if (!run_fits) {
     const uint32_t before = 4u * static_cast<uint32_t>(t) - (big != 0u ? 2u : 3u);  // (thread t - 1, and why)
     big = t == 0 ? 1u : 0u;
     if (t != 0) mine = before < mine ? before : mine;
@@ -682,6 +683,26 @@ __device__ __forceinline__ TrimmedBuckets scan_buckets_and_trim(uint32_t* start,
   if (last_thread < static_cast<uint32_t>(kFinishBlock)) {
     r.last_bucket = last_thread * kPer + (kPer - 1);
     r.n_sorted = r.n = start[r.last_bucket + 1u];
+    // The reference's search notices a stop on the 16th, 64th, 256th ... element of a row only one element later
+    // (src/sampling_distribution.h:166-181), so a list that ends exactly there may be one element short: it also gets
+    // the next thread's run of buckets that holds a key, or, when nothing else is listed, the best element below.
+    const uint32_t n = r.n_sorted;
+    if (want == 0 && r.more == 0u && n >= 16u && (n & (n - 1u)) == 0u && ((__ffs(static_cast<int>(n)) - 1) & 1) == 0) {
+      if (n == n_cand) {
+        r.best_below = block_max<u64>(best_below, red64);
+        r.n = n + (r.best_below != 0 ? 1u : 0u);
+      } else {
+        __syncthreads();  // (the reduction above left red32 to its readers)
+        const bool later = static_cast<uint32_t>(t) > last_thread && local != 0u;
+        const uint32_t nearest =
+            block_max<uint32_t>(later ? (static_cast<uint32_t>(kFinishBlock - t) << 1) | (run_fits ? 1u : 0u) : 0u, red32);
+        if (nearest & 1u) {  // (a run that does not fit the room, or has a bucket too full: the list stays as it is)
+          const uint32_t next_thread = static_cast<uint32_t>(kFinishBlock) - (nearest >> 1);
+          r.last_bucket = next_thread * kPer + (kPer - 1);
+          r.n_sorted = r.n = start[r.last_bucket + 1u];
+        }
+      }
+    }
   } else {
     r.best_below = block_max<u64>(best_below, red64);  // ranks after every candidate
     r.n = n_cand + (r.best_below != 0 ? 1u : 0u);

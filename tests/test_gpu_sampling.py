@@ -449,6 +449,38 @@ def test_nucleus_rows_with_lists_near_and_beyond_the_sort(ctx, orc, sigma, p, t)
         assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
 
 
+def test_nucleus_whose_stop_falls_on_a_batch_end_stays_off_the_exact_path(ctx, orc):
+    """Peaked rows whose nucleus search stops on the 16th, 64th or 256th element: the reference notices such a stop
+    only one element later (src/sampling_distribution.h:166-181), so the kept set has 17, 65, 257 tokens, and a
+    candidate list trimmed right behind the stop would be one element short.  The finish kernel then takes the next
+    run of buckets along; the rows are finished on the fast path with the oracle's kept sets and tokens."""
+    say("nucleus stop on a batch end, peaked rows")
+    rng = np.random.default_rng(1664)
+    vocab, p, t = 128256, 0.9, 1.0
+    shapes = [(15, 11.5, 50, 11.6), (63, 10.0, 30, 10.2), (255, 8.8, 30, 9.3), (15, 11.5, 0, 0.0)]
+    x = (rng.standard_normal((len(shapes), vocab)) - 15.0).astype(np.float32)
+    for r, (n_top, stop_depth, n_after, after_depth) in enumerate(shapes):
+        ids = rng.choice(32768, n_top + 1 + n_after, replace=False)  # all in the first chunk
+        x[r, ids[:n_top]] = 20.0
+        x[r, ids[n_top]] = np.float32(20.0 - stop_depth)
+        x[r, ids[n_top + 1:]] = (20.0 - after_depth - 0.01 * rng.random(n_after)).astype(np.float32)
+    u = rng.random(len(shapes))
+    u[0] = 0.9999999  # the draw reaches the element behind the stop
+    before = ctx.fallback_rows()
+    tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=p, temperature=t,
+                                 kept_capacity=512)
+    took_exact = ctx.fallback_rows() - before
+    tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+    for r, (n_top, _, _, _) in enumerate(shapes):
+        idx, probs = orc.sampled_categorical(x[r], 0, p, t)
+        assert len(idx) == n_top + 2, (r, len(idx))  # the stop's element and the one behind it
+        assert kc[r] == len(idx), (r, kc[r], len(idx))
+        assert np.array_equal(ki[r, :len(idx)], idx), r
+        assert np.array_equal(bits(kp[r, :len(idx)]), bits(probs)), r
+        assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
+    assert took_exact == 0, took_exact
+
+
 @pytest.mark.parametrize("sigma,p,t,wide_rows", [(3.0, 0.95, 1.0, 6), (2.0, 0.9, 1.0, 5), (4.0, 0.99, 1.5, 5), (1.0, 0.9, 1.0, 5)])
 def test_nucleus_rows_wider_than_the_sort(ctx, orc, sigma, p, t, wide_rows):
     """Unmasked nucleus rows of 128256 ids whose nuclei hold 30000 to 90000 tokens, several times what the finish
