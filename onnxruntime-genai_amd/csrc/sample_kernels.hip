@@ -605,6 +605,8 @@ struct TrimmedBuckets {
   // not 0: the kept buckets end short of the bucket where the nucleus certainly ends, so the list does not hold the
   // whole nucleus: 1: the room ends there, 2: the next thread's run has a bucket of more than bucket_cap keys
   uint32_t more;
+  // the element after best_below in the row's order, when the caller found it (0: not in the list): entry n - 1 then
+  u64 second_below;
 };
 
 // After a counting pass has left the number of candidates per bucket in start[0 .. kSortBuckets): turns the counts
@@ -729,6 +731,7 @@ __device__ __forceinline__ void rank_and_cache_exps(u64* keys, const uint32_t* s
     if (static_cast<uint32_t>(r * kFinishBlock) < n_pad) {
       const uint32_t pos = static_cast<uint32_t>(r * kFinishBlock + t);
       k[r] = pos == kept.n_sorted && pos < kept.n ? kept.best_below : 0;
+      if (pos == kept.n_sorted + 1u && pos < kept.n) k[r] = kept.second_below;
       fin[r] = pos;
       if (pos < kept.n_sorted) {
         k[r] = keys[pos];
@@ -947,8 +950,28 @@ __device__ __forceinline__ void nucleus_finish_body(const SampleArgs& a) {
       }
     });
     __syncthreads();
-    const TrimmedBuckets kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, kNucleusCap, red32, red64, k_wanted);
+    TrimmedBuckets kept = scan_buckets_and_trim(bucket_start, bucket_of, below, prm, V, kNucleusCap, red32, red64, k_wanted);
     if constexpr (!LARGEK) {
+      // The list ends with the one element below the candidates and has 16, 64, 256 ... entries: should the search
+      // stop on that last element, the reference notices it one element later (src/sampling_distribution.h:166-181),
+      // and that element is in no list.  Rare enough to look for it in the row itself: the best key below
+      // best_below.  (Rows whose logits are processed on the way in would need that processing here: the exact path
+      // keeps those.)
+      const uint32_t n_list = kept.n;
+      if (kept.best_below != 0 && n_list == kept.n_sorted + 1u && kept.more == 0u && n_list >= 16u && (n_list & (n_list - 1u)) == 0u &&
+          ((__ffs(static_cast<int>(n_list)) - 1) & 1) == 0 && !a.xf.active()) {
+        const RowPtr<AnyDtype> lrow(row_start<INLINE>(a, row, dtype_bytes(a.dtype)), a.dtype);
+        u64 second = 0;
+        for (int i = tid; i < V; i += kFinishBlock) {
+          const u64 key = make_key64(order_key(lrow[i]), static_cast<uint32_t>(i));
+          if (key < kept.best_below && key > second && key64_okey(key) != 0u) second = key;  // (order key 0: not a number)
+        }
+        second = block_max<u64>(second, red64);
+        if (second != 0) {
+          kept.second_below = second;
+          kept.n = n_list + 1u;
+        }
+      }
       // The nucleus may need more keys than the sort has room for (a flat distribution, a high temperature), or a
       // bucket too full for the usual ranking.  The same sort then runs over the row's second key buffer in global
       // memory: every needed key goes to a place of its bucket's there, the buckets are ranked in rounds through LDS,

@@ -457,7 +457,11 @@ def test_nucleus_whose_stop_falls_on_a_batch_end_stays_off_the_exact_path(ctx, o
     say("nucleus stop on a batch end, peaked rows")
     rng = np.random.default_rng(1664)
     vocab, p, t = 128256, 0.9, 1.0
-    shapes = [(15, 11.5, 50, 11.6), (63, 10.0, 30, 10.2), (255, 8.8, 30, 9.3), (15, 11.5, 0, 0.0)]
+    # (tokens at the top, depth of the element the search stops on, elements behind it and their depth); in the last
+    # three rows the stop's element already lies below the candidates' threshold: the list ends with it, and the
+    # element behind it is in no list at all
+    shapes = [(15, 11.5, 50, 11.6), (63, 10.0, 30, 10.2), (255, 8.8, 30, 9.3), (15, 11.5, 0, 0.0),
+              (15, 12.5, 3, 13.0), (63, 11.0, 3, 11.5), (15, 12.5, 0, 0.0)]
     x = (rng.standard_normal((len(shapes), vocab)) - 15.0).astype(np.float32)
     for r, (n_top, stop_depth, n_after, after_depth) in enumerate(shapes):
         ids = rng.choice(32768, n_top + 1 + n_after, replace=False)  # all in the first chunk
@@ -479,6 +483,12 @@ def test_nucleus_whose_stop_falls_on_a_batch_end_stays_off_the_exact_path(ctx, o
         assert np.array_equal(bits(kp[r, :len(idx)]), bits(probs)), r
         assert tok[r] == idx[orc.discrete_draw(probs, u[r])], r
     assert took_exact == 0, took_exact
+    # the same rows as fp16
+    x16 = x.astype(np.float16)
+    before = ctx.fallback_rows()
+    tok16 = ctx.sample(torch.from_numpy(x16).cuda(), torch.from_numpy(u).cuda(), k=0, p=p, temperature=t).cpu().numpy()
+    assert np.array_equal(tok16, orc.sample_batch(x16.astype(np.float32), 0, p, t, u))
+    assert ctx.fallback_rows() == before
 
 
 @pytest.mark.parametrize("sigma,p,t,wide_rows", [(3.0, 0.95, 1.0, 6), (2.0, 0.9, 1.0, 5), (4.0, 0.99, 1.5, 5), (1.0, 0.9, 1.0, 5)])
