@@ -387,7 +387,7 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
                                                   uint32_t rmax, uint32_t thr, bool cut_at_best_below,
                                                   mi355x_sample_params prm, int V, double u, const RowOutputs& out,
                                                   SeqShared& seqsh, uint32_t* red32, EmitTopk emit = EmitTopk{},
-                                                  bool presorted = false) {
+                                                  bool presorted = false, u64 second_below = 0) {
   const int tid = threadIdx.x;
   const u64* lk = lds_keys;
   auto sorted = [=](int i) { return lk[exp_slot(static_cast<uint32_t>(i))]; };
@@ -405,8 +405,11 @@ __device__ __forceinline__ bool finish_candidates(u64* lds_keys, uint32_t* bucke
     return true;
   }
   if (!presorted) {
-    if (best_below != 0 && tid == 0) lds_keys[n_c] = best_below;
-    if (best_below != 0) n_c += 1;
+    if (best_below != 0 && tid == 0) {
+      lds_keys[n_c] = best_below;
+      if (second_below != 0) lds_keys[n_c + 1u] = second_below;  // (the element behind it, for lists that need it)
+    }
+    if (best_below != 0) n_c += second_below != 0 ? 2u : 1u;
     __syncthreads();
     bool sorted_done = false;
     if (n_c > static_cast<uint32_t>(kFinishBlock) && rmax != 0u) {
@@ -1563,6 +1566,7 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
     }
   }
   uint32_t n_c = 0u;
+  u64 second_below = 0;
   if (direct) {
     n_c = sort_counted(lds_keys, bucket_start, ids, ok, bucket_of, rmax, best_below, n_allowed, n_extra, prm, V, red32, red64);
     if (n_c == 0u) {  // heavy ties: the general tail, the candidates as they were
@@ -1603,9 +1607,44 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
     }
     best_below = block_max<u64>(best_below, red64);  // barriers inside also publish sh_count
     n_c = sh_count;
+    // A list that ends with best_below on its 16th, 64th, 256th ... entry: should the search stop on that entry, the
+    // reference notices it one element later (src/sampling_distribution.h:166-181).  That element is the best key
+    // below best_below among the elements that are no candidates and the masked ids; rows that came here straight
+    // (the short lists: a few allowed ids under a grammar) still have every element in its thread's registers.
+    const uint32_t n_list = n_c + 1u;
+    if (!direct && best_below != 0 && n_list >= 16u && (n_list & (n_list - 1u)) == 0u && ((__ffs(static_cast<int>(n_list)) - 1) & 1) == 0) {
+      u64 s = 0;
+#pragma unroll
+      for (int u = 0; u < kSparseIds + kSparseExtraRegs; ++u) {
+        const u64 k64 = make_key64(ok[u], ids[u]);
+        if (ids[u] != 0xffffffffu && ok[u] != 0u && ok[u] < thr && k64 < best_below && k64 > s) s = k64;
+      }
+      // The row's second masked id outside the history is wanted once in a long while: it is looked for here, behind
+      // the first, a block of ids at a time (the row's list is short: nearly every id is masked, the first batch has it).
+      uint32_t second_masked = 0xffffffffu;
+      if (first_masked != 0xffffffffu) {
+        for (uint32_t start = first_masked + 1u; start < static_cast<uint32_t>(V) && second_masked == 0xffffffffu;
+             start += static_cast<uint32_t>(kFinishBlock)) {
+          const uint32_t id = start + static_cast<uint32_t>(tid);
+          bool is_masked = false;
+          if (id < static_cast<uint32_t>(V)) {
+            uint32_t m = mrow[id >> 5];
+            for (int e = 0; e < n_eos; ++e)
+              if (a.xf.eos[e] == static_cast<int>(id)) m &= ~(1u << (id & 31u));
+            is_masked = ((m >> (id & 31u)) & 1u) == 0u;
+            for (int j = 0; is_masked && j < hlen; ++j) is_masked = h[j] != static_cast<int>(id);
+          }
+          second_masked = ~block_max<uint32_t>(is_masked ? ~id : 0u, red32);
+        }
+      }
+      const u64 km1 = make_key64(order_key(kLowest), first_masked), km2 = make_key64(order_key(kLowest), second_masked);
+      if (first_masked != 0xffffffffu && km1 < best_below && km1 > s) s = km1;
+      if (second_masked != 0xffffffffu && km2 < best_below && km2 > s) s = km2;
+      second_below = block_max<u64>(s, red64);
+    }
   }
   return leave(finish_candidates(lds_keys, bucket_start, n_c, presorted ? 0 : best_below, rmax, thr, false, prm, V, a.uniforms[row],
-                                 row_outputs(a, row), seqsh, red32, EmitTopk{}, presorted));
+                                 row_outputs(a, row), seqsh, red32, EmitTopk{}, presorted, presorted ? 0 : second_below));
 }
 
 template <bool INLINE>

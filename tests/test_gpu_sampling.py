@@ -423,6 +423,54 @@ def test_sparse_mask_rows_with_heavy_ties(ctx, orc):
             assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (promise, r)
 
 
+def test_grammar_rows_with_15_63_or_255_allowed_ids_stay_off_the_exact_path(ctx, orc):
+    """A grammar that lets 15, 63 or 255 ids through, all of them inside the nucleus: the search only stops on the
+    first masked id, which is the 16th, 64th, 256th element, and the reference notices such a stop one element later
+    (src/sampling_distribution.h:166-181): the kept set ends with two masked ids.  The sparse-mask kernel knows the
+    second one (and the elements behind the first in general); kept sets and tokens equal the oracle's, with and
+    without a repetition penalty over ids that include masked ones, and no row takes the exact path."""
+    say("grammar rows whose list ends on a batch end")
+    rng = np.random.default_rng(1563)
+    vocab = 201088
+    words = (vocab - 1) // 32 + 1
+    sizes = [15, 63, 255, 15, 63, 14, 16]
+    rows = len(sizes)
+    x = (rng.standard_normal((rows, vocab)) * 2).astype(np.float32)
+    bits_ = np.zeros((rows, words * 32), bool)
+    for r, n in enumerate(sizes):
+        ids = rng.choice(vocab, n, replace=False)
+        if r == 3:
+            ids[0] = 1  # id 0 is masked: the first masked id is 0, the second 2
+            ids[1] = 3
+        bits_[r, ids] = True
+        x[r, ids] = (5.0 + 0.1 * rng.standard_normal(n)).astype(np.float32)  # near-equal: the nucleus needs all of them
+    mask = np.ascontiguousarray(np.packbits(bits_.reshape(rows, words, 32), axis=-1, bitorder="little").view(np.uint32).reshape(rows, words))
+    proc = orc.apply_mask(x, mask)
+    u = rng.random(rows)
+    u[1] = 0.99999999
+    hist = rng.integers(0, 40, (rows, 24)).astype(np.int32)  # low ids: masked ones among them, 0 and 2 included
+    for penalty in (None, 1.3):
+        for promise in (0, 256):
+            xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(),
+                                   history=torch.from_numpy(hist).cuda() if penalty else None,
+                                   repetition_penalty=penalty or 1.0, mask_allowed_max=promise)
+            before = ctx.fallback_rows()
+            tok, kc, ki, kp = ctx.sample(torch.from_numpy(x).cuda(), torch.from_numpy(u).cuda(), k=0, p=0.9, temperature=1.0,
+                                         xf=xf, kept_capacity=512)
+            took_exact = ctx.fallback_rows() - before
+            tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+            for r in range(rows):
+                want = orc.apply_repetition_penalty(proc[r], hist[r], penalty) if penalty else proc[r]
+                idx, probs = orc.sampled_categorical(want, 0, 0.9, 1.0)
+                assert kc[r] == len(idx), (penalty, promise, r, kc[r], len(idx))
+                assert np.array_equal(ki[r, :len(idx)], idx), (penalty, promise, r)
+                assert np.array_equal(bits(kp[r, :len(idx)]), bits(probs)), (penalty, promise, r)
+                assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (penalty, promise, r)
+            if penalty is None:
+                assert [int(k) for k in kc] == [17, 65, 257, 17, 65, 15, 17], kc
+            assert took_exact == 0, (penalty, promise, took_exact)
+
+
 @pytest.mark.parametrize("sigma,p,t", [(4.0, 0.95, 1.0), (1.0, 0.9, 1.0), (5.0, 0.9, 1.0), (3.0, 0.5, 0.7)])
 def test_nucleus_rows_with_lists_near_and_beyond_the_sort(ctx, orc, sigma, p, t):
     """Unmasked nucleus rows of 128256 ids whose chunks list a few thousand to tens of thousands of keys: nuclei that
