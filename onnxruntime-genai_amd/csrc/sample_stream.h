@@ -616,7 +616,8 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const InT* lrow = static_cast<const InT*>(row0);
-  const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
+  constexpr bool kOneRun = XFORM && sizeof(InT) == 4;  // the loads of a chunk are one straight run, see there
+  const bool aligned = kOneRun || ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
   const float kNaN = __uint_as_float(0x7fc00000u);  // marks ids >= vocab: never a maximum, never >= a bound
   // The bitmap words and the first history ids of this thread are requested before the logits: loads come back in
   // the order they were asked for, and the history has a chain of its own to start (mark the ids, read their logits
@@ -632,6 +633,20 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   const bool hist_ahead = pen && a.xf.history_lens == nullptr;  // the length is known without a load
   int hist_pre[2] = {-1, -1};
   uint32_t mask_pre[kWordsPerThread];
+  // Kernels with logits processing also request the row's history length (where rows have lengths of their own) and
+  // the flag that sends every row to the exact path before the logits: whatever is requested before them arrives
+  // before them, so the processing's preparations run while the logits are in flight.  (Both used to be loaded where
+  // they were first needed, behind the logits, each a round trip of its own.)
+  int row_hlen = 0;
+  uint32_t flag_pre = 0u;
+  if constexpr (XFORM) {
+    const int uniform_hlen = arg_now(a.xf.history_len);
+    row_hlen = uniform_hlen;
+    // (indexed through a lane's register, so that the length stays in one: as a value common to the wave it would be
+    // moved to a scalar register at once, which waits for it)
+    if (active && a.xf.history_lens != nullptr) row_hlen = a.xf.history_lens[row + (lane >> 6)];
+    if (tid == 0) flag_pre = a.fallback_rows[1];
+  }
 #pragma unroll
   for (int q = 0; q < 2; ++q)
     if (hist_ahead && tid + q * kSBlock < a.xf.history_len) hist_pre[q] = hist[tid + q * kSBlock];
@@ -644,9 +659,106 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
     }
   }
   float v[kSElems];
+  // ---- logits processing ----------------------------------------------------------------------
+  // Grammar mask and min-length masking reach the registers as one LDS bitmap of allowed ids (a clear
+  // bit -> kLowest; ids past the vocabulary count as allowed and keep their NaN).  The ids of the row's
+  // history are few and their processing (a correctly rounded division, the n-gram ban) is long, so
+  // they leave the register arrays altogether: a second bitmap turns them into NaN there, and the
+  // threads that marked them compute their processed values into a short list in LDS, `extras`, which
+  // every later phase visits next to the registers.
+  // All of this but the application to the registers needs only what was requested before the logits, and it is
+  // called inside every path of the loads below, right behind that path's requests: there the number of requests
+  // behind the earlier ones is known exactly and a wait for those leaves the logits in flight.  (Where the paths
+  // join again the compiler has to assume the fewest requests any path may have made, none, and waits for the
+  // logits themselves at the first use of an earlier value: the preparations then start when the logits are there.)
+  uint32_t n_extra = 0u;
+  bool extra_overflow = false;
+  int n_eos_row = 0;
+  auto xform_prep = [&]() {
+    // One thread reads the flag that sends every row to the exact path, and the workgroup looks at that copy behind
+    // its first barrier: read by every wave for itself, at its own time, a flag raised in between would send some
+    // waves of a workgroup one way and the rest the other, with barriers waiting on both sides.
+    if (tid == 0) sm.poisoned = flag_pre;
+    if (!active) return;
+    // Xform::eos_count with the length that was requested before the logits
+    const int n_eos = (a.xf.history_lens && a.xf.min_length > 0 && row_hlen >= a.xf.min_length) ? 0 : a.xf.n_eos;
+    n_eos_row = n_eos;
+    if (tid == 0) {
+      sm.n_extra = 0u;
+      sm.nan0 = 0u;
+    }
+#pragma unroll
+    for (int q = 0; q < kWordsPerThread; ++q) {
+      const int i = tid + q * kSBlock;
+      const int w = chunk * (kSChunk / 32) + i;
+      uint32_t word = mask_pre[q];
+      for (int e = 0; e < n_eos; ++e)
+        if ((a.xf.eos[e] >> 5) == w) word &= ~(1u << (a.xf.eos[e] & 31));
+      const int n_real = V - w * 32;  // ids of this word inside the vocabulary
+      if (n_real < 32) word |= n_real <= 0 ? ~0u : (~0u << n_real);
+      sm.mask_bits[i] = word;
+      sm.hist_bits[i] = 0u;
+    }
+    lds_barrier();
+    if (pen) {
+      const int hlen = row_hlen;
+      const float penalty = a.xf.penalty;
+      const uint32_t* ban_row = a.xf.ban_row(row, V);
+      // the thread that is first to mark an id computes its processed value
+      auto visit = [&](int id) {
+        const int rel = id - chunk * kSChunk;
+        if (rel >= 0 && rel < kSChunk && id < V) {
+          const uint32_t bit = 1u << (rel & 31);
+          if (!(atomicOr(&sm.hist_bits[rel >> 5], bit) & bit)) {
+            const uint32_t slot = atomicAdd(&sm.n_extra, 1u);
+            if (slot < static_cast<uint32_t>(kExtraCap)) {
+              const uint32_t mw = has_mask ? mrow[id >> 5] : 0u;
+              const float val = xform_value(load_one<InT>(lrow, id), penalty, a.xf.eos, id, mw, has_mask, true, n_eos, ban_row);
+              sm.extra_val[slot] = val;
+              sm.extra_idx[slot] = static_cast<uint32_t>(id);
+              if (id == 0 && val != val) sm.nan0 = 1u;
+            }
+          }
+        }
+      };
+      int first = tid;
+      if (hist_ahead) {
+        if (tid < hlen) visit(hist_pre[0]);
+        if (tid + kSBlock < hlen) visit(hist_pre[1]);
+        first = tid + 2 * kSBlock;
+      }
+      for (int i = first; i < hlen; i += kSBlock) visit(hist[i]);
+      lds_barrier();
+      n_extra = sm.n_extra;
+      extra_overflow = n_extra > static_cast<uint32_t>(kExtraCap);  // the row takes the exact path
+      if (extra_overflow) n_extra = 0u;
+    }
+  };
   // a chunk that lies inside an aligned row requests its loads without a test between them
   const bool whole_chunk = aligned && (chunk + 1) * kSChunk <= V;
-  if constexpr (VEC == 4) {
+  if constexpr (kOneRun) {
+    // Kernels with logits processing request the loads of a chunk in one straight run, whatever the row's end and
+    // wherever the row starts: 128-bit loads that only need their elements' alignment (the hardware reads from any
+    // address; rows that do not start on a 16-byte boundary cost it more cache lines), a load that would cross the
+    // row's end reads the row's last four elements instead, one beyond it the row's first, and the registers are put
+    // right further down, after the processing's preparations.  The number of requests behind the earlier ones
+    // (history ids, mask words, the flag) is then known where those are first used, and the wait for them leaves the
+    // logits in flight.  With a branch per kind of chunk or row the compiler has to assume, where the branches join,
+    // the fewest requests any of them may have made -- and ahead of any joint continuation of two such paths it
+    // waits for everything -- so that the preparations would start when the logits are there.
+    typedef float v4f_any __attribute__((ext_vector_type(4), aligned(4)));
+#pragma unroll
+    for (int j = 0; j < kSLoads; ++j) {
+      const int i0 = elem_index<kSBlock, VEC>(chunk, j, 0);
+      const int from = i0 + 4 <= V ? i0 : (i0 < V ? V - 4 : 0);
+      const v4f_any q = __builtin_nontemporal_load(reinterpret_cast<const v4f_any*>(lrow + from));
+      v[j * 4 + 0] = q.x;
+      v[j * 4 + 1] = q.y;
+      v[j * 4 + 2] = q.z;
+      v[j * 4 + 3] = q.w;
+    }
+    xform_prep();
+  } else if constexpr (VEC == 4) {
     if (whole_chunk) {
       const v4f* src = reinterpret_cast<const v4f*>(lrow + static_cast<size_t>(chunk) * kSChunk) + tid;
 #pragma unroll
@@ -718,10 +830,10 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       }
     }
   }
-  // One thread reads the flag that sends every row to the exact path, and the workgroup looks at that copy behind
-  // its first barrier: read by every wave for itself, at its own time, a flag raised in between would send some
-  // waves of a workgroup one way and the rest the other, with barriers waiting on both sides.
-  if (tid == 0) sm.poisoned = a.fallback_rows[1];
+  if constexpr (XFORM && !kOneRun) xform_prep();  // (sixteen-bit rows)
+  if constexpr (!XFORM) {
+    if (tid == 0) sm.poisoned = a.fallback_rows[1];
+  }
   // The arguments the phases after the streaming pass need are fetched now, while the logits are in
   // flight, instead of one by one where they are first used.
   const int n_chunks = arg_now(a.chunks);
@@ -734,70 +846,29 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
                               arg_now(a.kept_ids),
                               arg_now(a.kept_probs),
                               arg_now(a.kept_capacity)};
-  // ---- logits processing ----------------------------------------------------------------------
-  // Grammar mask and min-length masking reach the registers as one LDS bitmap of allowed ids (a clear
-  // bit -> kLowest; ids past the vocabulary count as allowed and keep their NaN).  The ids of the row's
-  // history are few and their processing (a correctly rounded division, the n-gram ban) is long, so
-  // they leave the register arrays altogether: a second bitmap turns them into NaN there, and the
-  // threads that marked them compute their processed values into a short list in LDS, `extras`, which
-  // every later phase visits next to the registers.
-  uint32_t n_extra = 0u;
-  bool extra_overflow = false;
-  if (XFORM && active) {
-    const int n_eos = a.xf.eos_count(row);
-    if (tid == 0) {
-      sm.n_extra = 0u;
-      sm.nan0 = 0u;
-    }
+  if constexpr (XFORM) {
+    // fp32 rows: the registers past the row's end, see the loads above
+    if constexpr (kOneRun) {
+      if (!whole_chunk) {
 #pragma unroll
-    for (int q = 0; q < kWordsPerThread; ++q) {
-      const int i = tid + q * kSBlock;
-      const int w = chunk * (kSChunk / 32) + i;
-      uint32_t word = mask_pre[q];
-      for (int e = 0; e < n_eos; ++e)
-        if ((a.xf.eos[e] >> 5) == w) word &= ~(1u << (a.xf.eos[e] & 31));
-      const int n_real = V - w * 32;  // ids of this word inside the vocabulary
-      if (n_real < 32) word |= n_real <= 0 ? ~0u : (~0u << n_real);
-      sm.mask_bits[i] = word;
-      sm.hist_bits[i] = 0u;
-    }
-    lds_barrier();
-    if (pen) {
-      const int hlen = a.xf.hist_len(row);
-      const float penalty = a.xf.penalty;
-      const uint32_t* ban_row = a.xf.ban_row(row, V);
-      // the thread that is first to mark an id computes its processed value
-      auto visit = [&](int id) {
-        const int rel = id - chunk * kSChunk;
-        if (rel >= 0 && rel < kSChunk && id < V) {
-          const uint32_t bit = 1u << (rel & 31);
-          if (!(atomicOr(&sm.hist_bits[rel >> 5], bit) & bit)) {
-            const uint32_t slot = atomicAdd(&sm.n_extra, 1u);
-            if (slot < static_cast<uint32_t>(kExtraCap)) {
-              const uint32_t mw = has_mask ? mrow[id >> 5] : 0u;
-              const float val = xform_value(load_one<InT>(lrow, id), penalty, a.xf.eos, id, mw, has_mask, true, n_eos, ban_row);
-              sm.extra_val[slot] = val;
-              sm.extra_idx[slot] = static_cast<uint32_t>(id);
-              if (id == 0 && val != val) sm.nan0 = 1u;
-            }
+        for (int j = 0; j < kSLoads; ++j) {
+          const int i0 = elem_index<kSBlock, VEC>(chunk, j, 0);
+          if (i0 + 4 > V) {  // elements V-4 .. V-1 in the registers where i0 .. V-1 belong, or nothing of the row
+            const int r = i0 < V ? V - i0 : 0;  // elements of the quad that lie inside the row
+            const float q1 = v[j * 4 + 1], q2 = v[j * 4 + 2], q3 = v[j * 4 + 3];
+            v[j * 4 + 0] = r == 0 ? kNaN : (r == 1 ? q3 : (r == 2 ? q2 : q1));
+            v[j * 4 + 1] = r < 2 ? kNaN : (r == 2 ? q3 : q2);
+            v[j * 4 + 2] = r < 3 ? kNaN : q3;
+            v[j * 4 + 3] = kNaN;
           }
         }
-      };
-      int first = tid;
-      if (hist_ahead) {
-        if (tid < hlen) visit(hist_pre[0]);
-        if (tid + kSBlock < hlen) visit(hist_pre[1]);
-        first = tid + 2 * kSBlock;
       }
-      for (int i = first; i < hlen; i += kSBlock) visit(hist[i]);
-      lds_barrier();
-      n_extra = sm.n_extra;
-      extra_overflow = n_extra > static_cast<uint32_t>(kExtraCap);  // the row takes the exact path
-      if (extra_overflow) n_extra = 0u;
     }
-    // without a grammar mask and without EOS masking every id is allowed (ids past the vocabulary are NaN already)
-    if (has_mask || n_eos > 0) mask_registers<kSBlock, VEC, true, true>(v, sm.mask_bits, sm.hist_bits, tid);
-    else mask_registers<kSBlock, VEC, false, true>(v, sm.mask_bits, sm.hist_bits, tid);
+    if (active) {
+      // without a grammar mask and without EOS masking every id is allowed (ids past the vocabulary are NaN already)
+      if (has_mask || n_eos_row > 0) mask_registers<kSBlock, VEC, true, true>(v, sm.mask_bits, sm.hist_bits, tid);
+      else mask_registers<kSBlock, VEC, false, true>(v, sm.mask_bits, sm.hist_bits, tid);
+    }
   }
   // per-thread maximum in the float domain (fmaxf skips NaN), keeping the maximum of every float4
   float qm[kSVec];

@@ -847,6 +847,47 @@ def test_sample_long_and_dense_histories(ctx, orc, vocab, hist_len, span, k, p):
     assert (took_exact > 0) == (span == 2500), took_exact  # only the overflowing lists go to the exact path
 
 
+@pytest.mark.parametrize("vocab", [40001, 40002, 40003, 65539, 98305, 98308])
+def test_logits_processing_on_rows_of_any_alignment_and_end(ctx, orc, vocab):
+    """The kernels with logits processing request a chunk's fp32 logits as sixteen 128-bit loads per thread whatever
+    the row's alignment and end (a quad that straddles the end is read as the row's last four elements and put right
+    afterwards): rows that start on every 4-byte offset of a 16-byte line, vocabularies that end one, two and three
+    elements into a quad, a last chunk of a single element, history ids and masked ids on the row's last elements.
+    Argmax, top-k, k = 300 and nucleus rows against the oracle."""
+    say("rows of any alignment", vocab)
+    rng = np.random.default_rng(vocab)
+    rows = 6
+    x = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    x[0, vocab - 1] = 30.0   # the row's best on its last element ...
+    x[1, vocab - 2] = 30.0   # ... on the one before, penalised below
+    x[2, vocab - 3] = 30.0   # ... masked below
+    hist = rng.integers(0, vocab, (rows, 200)).astype(np.int32)
+    hist[:, 0] = vocab - 2
+    hist[:, 1] = vocab - 1
+    mask = make_mask(rng, rows, vocab, 0.8)
+    words = mask.reshape(rows, -1)
+    words[2, (vocab - 3) >> 5] &= ~np.uint32(1 << ((vocab - 3) & 31))
+    u = rng.random(rows)
+    xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                           repetition_penalty=1.6)
+    xd = torch.from_numpy(x).cuda()
+    proc = orc.apply_mask(x, mask)
+    want = [orc.apply_repetition_penalty(proc[r], hist[r], 1.6) for r in range(rows)]
+    got = ctx.argmax(xd, xf=xf).cpu().numpy()
+    for r in range(rows):
+        assert got[r] == orc.argmax(want[r]), r
+    for k, p, t in ((50, 0.9, 0.7), (300, 0.95, 1.0), (0, 0.9, 1.0)):
+        tok, kc, ki, kp = ctx.sample(xd, torch.from_numpy(u).cuda(), k=k, p=p, temperature=t, xf=xf, kept_capacity=2048)
+        tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+        for r in range(rows):
+            idx, probs = orc.sampled_categorical(want[r], k, p, t)
+            n = min(len(idx), 2048)
+            assert kc[r] == len(idx), (k, r)
+            assert np.array_equal(ki[r, :n], idx[:n]), (k, r)
+            assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), (k, r)
+            assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (k, r)
+
+
 @pytest.mark.parametrize("hist_len", [1500, 2500, 3400, 5000])
 def test_sparse_mask_rows_with_thousands_of_distinct_history_ids(orc, hist_len):
     """Nucleus rows under a sparse grammar mask whose history holds more distinct ids than the sparse-mask kernel's
