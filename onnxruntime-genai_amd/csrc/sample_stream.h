@@ -630,7 +630,12 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   const int words = (V - 1) / 32 + 1;
   const uint32_t* mrow = has_mask ? a.xf.mask + static_cast<size_t>(row) * words : nullptr;
   const int32_t* hist = pen ? a.xf.history + static_cast<size_t>(row) * a.xf.history_stride : nullptr;
-  const bool hist_ahead = pen && a.xf.history_lens == nullptr;  // the length is known without a load
+  // The first two history ids of every thread are requested before the logits: as many as the common length says,
+  // or, where rows have lengths of their own, as many as a row of the history holds (what lies beyond the row's
+  // length is fetched and not looked at).  A history shared by all rows (stride 0) has no such bound: its ids are
+  // fetched once the length is there.
+  const bool hist_ahead = pen && (a.xf.history_lens == nullptr || a.xf.history_stride > 0);
+  const int hist_ahead_ids = a.xf.history_lens == nullptr ? a.xf.history_len : a.xf.history_stride;
   int hist_pre[2] = {-1, -1};
   uint32_t mask_pre[kWordsPerThread];
   // Kernels with logits processing also request the row's history length (where rows have lengths of their own) and
@@ -649,7 +654,7 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   }
 #pragma unroll
   for (int q = 0; q < 2; ++q)
-    if (hist_ahead && tid + q * kSBlock < a.xf.history_len) hist_pre[q] = hist[tid + q * kSBlock];
+    if (hist_ahead && tid + q * kSBlock < hist_ahead_ids) hist_pre[q] = hist[tid + q * kSBlock];
 #pragma unroll
   for (int q = 0; q < kWordsPerThread; ++q) {
     mask_pre[q] = ~0u;
