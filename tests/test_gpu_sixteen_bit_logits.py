@@ -153,6 +153,35 @@ def test_argmax_sixteen_bit_rows(ctx, orc, dtype):
         assert np.array_equal(pkg().argmax_static(w, out).cpu().numpy(), orc.argmax_batch(widened(orc, w))), (rows, vocab)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("vocab", [50257, 51865, 98311])
+def test_rows_that_start_on_every_offset_of_a_16_byte_line(ctx, orc, dtype, vocab):
+    """Odd vocabularies put every row on a start of its own inside a 16-byte line, and a view can start anywhere: the
+    streaming kernels read such rows with the same 128-bit loads as aligned ones.  Nine rows cut out of one buffer
+    at element offsets 0 .. 8, argmax and every selection mode, against the oracle on the same elements."""
+    say("row starts", dtype, vocab)
+    g = torch.Generator(device="cuda").manual_seed(vocab)
+    rows = 9
+    big = (torch.randn(rows, vocab + 16, generator=g, device="cuda") * 3).to(dtype)
+    views = [big[r, r:r + vocab] for r in range(rows)]
+    dense = torch.stack(views).contiguous()  # rows vocab elements apart: starts differ row by row, too
+    wide = dense.cpu().numpy() if dtype == torch.float32 else widened(orc, dense)
+    assert np.array_equal(ctx.argmax(dense).cpu().numpy(), orc.argmax_batch(wide))
+    rng = np.random.default_rng(vocab)
+    u = rng.random(rows)
+    for k, p, t in ((50, 0.9, 0.7), (0, 0.9, 1.0), (300, 0.95, 1.0)):
+        for x in (dense, views):  # rows a stride apart, and rows scattered over memory with starts of their own
+            tok, kc, ki, kp = ctx.sample(x, torch.from_numpy(u).cuda(), k=k, p=p, temperature=t, kept_capacity=4096)
+            tok, kc, ki, kp = tok.cpu().numpy(), kc.cpu().numpy(), ki.cpu().numpy(), kp.cpu().numpy()
+            for r in range(rows):
+                idx, probs = orc.sampled_categorical(wide[r], k, p, t)
+                n = min(len(idx), 4096)
+                assert kc[r] == len(idx), (k, r)
+                assert np.array_equal(ki[r, :n], idx[:n]), (k, r)
+                assert np.array_equal(bits(kp[r, :n]), bits(probs[:n])), (k, r)
+                assert tok[r] == idx[orc.discrete_draw(probs, u[r])], (k, r)
+
+
 def test_config2_shape_in_fp16_equals_fp32_on_the_widened_rows(ctx, orc):
     """Benchmark configuration 2 with fp16 logits: identical tokens to the fp32 entry point fed the widened rows."""
     say("config2 fp16")
