@@ -14,9 +14,8 @@ __global__ __launch_bounds__(kBlock) void argmax_kernel(const ArgmaxArgs a) {
   __shared__ uint32_t hist_bits[kChunk / 32];
   __shared__ u64 red64[4];
   const InT* lrow = static_cast<const InT*>(a.logits) + static_cast<size_t>(row) * a.row_stride;
-  const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
   float v[kElems];
-  Loader<InT>::load(lrow, aligned, V, chunk, v);
+  Loader<InT>::load(lrow, V, chunk, v);
   if (a.xf.active()) {
     if (a.xf.use_penalty()) build_history_bitmap(a.xf, row, chunk * kChunk, hist_bits);
     xform_chunk<InT>(a.xf, row, V, chunk, hist_bits, v);
@@ -73,7 +72,6 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
   __shared__ uint32_t hist_bits[kRowKernelMaxVocab / 32];
   __shared__ u64 red64[16];
   const InT* lrow = logits + static_cast<size_t>(row) * row_stride;
-  const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
   const bool pen = history && (history_lens || history_len > 0) && (penalty != 1.0f || ban);  // Xform::use_penalty
   const bool has_mask = mask != nullptr;
   const bool active = has_mask || pen || n_eos_all > 0;
@@ -89,12 +87,12 @@ __global__ __launch_bounds__(1024) void argmax_row_kernel(const ArgmaxArgs a) {
     for (int j = 0; j < NB; ++j) {
       const int i0 = base + (j * 1024 + tid) * VEC;
       mw[j] = (has_mask && i0 < V) ? mrow[i0 >> 5] : 0u;  // VEC divides 32: one word covers the vector
-      if (aligned && i0 + VEC <= V) {
+      if (i0 + VEC <= V) {
         if constexpr (VEC == 4) {
-          const float4 q = *reinterpret_cast<const float4*>(lrow + i0);
+          const v4f_any q = *reinterpret_cast<const v4f_any*>(lrow + i0);
           v[j][0] = q.x, v[j][1] = q.y, v[j][2] = q.z, v[j][3] = q.w;
         } else {
-          const uint4 q = *reinterpret_cast<const uint4*>(lrow + i0);
+          const v4u_any q = *reinterpret_cast<const v4u_any*>(lrow + i0);
           const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
@@ -153,7 +151,7 @@ __global__ __launch_bounds__(kBlock) void process_logits_kernel(float* logits, i
   float* lrow = logits + static_cast<size_t>(row) * row_stride;
   const bool aligned = ((reinterpret_cast<uintptr_t>(lrow) & 15u) == 0);
   float v[kElems];
-  Loader<float>::load(lrow, aligned, vocab, chunk, v);
+  Loader<float>::load(lrow, vocab, chunk, v);
   if (xf.use_penalty()) build_history_bitmap(xf, row, chunk * kChunk, hist_bits);
   xform_chunk<float>(xf, row, vocab, chunk, hist_bits, v);
 #pragma unroll

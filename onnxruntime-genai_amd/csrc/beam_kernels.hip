@@ -16,15 +16,14 @@ constexpr int kBeamListCap = 1024;  // candidates a row may hold in LDS before t
 template <typename InT, typename Fn>
 __device__ __forceinline__ void row_for_each(const InT* x, int V, Fn fn) {
   constexpr int VEC = 16 / sizeof(InT);
-  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
   const int step = static_cast<int>(blockDim.x) * VEC;
   for (int base = 0; base < V; base += 4 * step) {
     float v[4][VEC];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int i0 = base + r * step + static_cast<int>(threadIdx.x) * VEC;
-      if (aligned && i0 + VEC <= V) {
-        const uint4 q = *reinterpret_cast<const uint4*>(x + i0);
+      if (i0 + VEC <= V) {
+        const v4u_any q = *reinterpret_cast<const v4u_any*>(x + i0);
         const uint32_t w[4] = {q.x, q.y, q.z, q.w};
         if constexpr (VEC == 4) {
 #pragma unroll

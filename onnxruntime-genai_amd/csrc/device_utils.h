@@ -345,6 +345,12 @@ __device__ __forceinline__ float xform_value(float x, float penalty, const int* 
   return x;
 }
 
+// 128-bit vectors that assume no more than their elements' alignment.  The hardware reads them from any address, so
+// rows that do not start on a 16-byte boundary (odd vocabularies such as 50257, views into larger buffers) are read
+// with the same loads as aligned rows; they only touch more cache lines.
+typedef float v4f_any __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t v4u_any __attribute__((ext_vector_type(4), aligned(2)));
+
 // Loads the kElems logits a thread owns in chunk `chunk` of a row, widened to fp32 and processed.
 // Thread t owns, for j = 0..NV-1, the VEC consecutive ids starting at
 // chunk*kChunk + (j*kBlock + t)*VEC; ids >= vocab yield 0 and must be ignored by the caller.
@@ -358,13 +364,12 @@ struct Loader<float> {
   __device__ static __forceinline__ int index_of(int chunk, int j, int c) {
     return chunk * kChunk + (j * kBlock + static_cast<int>(threadIdx.x)) * VEC + c;
   }
-  __device__ static __forceinline__ void load(const float* row, bool aligned, int vocab, int chunk,
-                                              float (&v)[kElems]) {
+  __device__ static __forceinline__ void load(const float* row, int vocab, int chunk, float (&v)[kElems]) {
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int i0 = index_of(chunk, j, 0);
-      if (aligned && i0 + VEC <= vocab) {
-        const float4 q = *reinterpret_cast<const float4*>(row + i0);
+      if (i0 + VEC <= vocab) {
+        const v4f_any q = *reinterpret_cast<const v4f_any*>(row + i0);
         v[j * 4 + 0] = q.x;
         v[j * 4 + 1] = q.y;
         v[j * 4 + 2] = q.z;
@@ -384,14 +389,13 @@ struct Loader16 {  // sixteen-bit elements: IEEE binary16 bit patterns (uint16_t
   __device__ static __forceinline__ int index_of(int chunk, int j, int c) {
     return chunk * kChunk + (j * kBlock + static_cast<int>(threadIdx.x)) * VEC + c;
   }
-  __device__ static __forceinline__ void load(const T16* row, bool aligned, int vocab, int chunk,
-                                              float (&v)[kElems]) {
+  __device__ static __forceinline__ void load(const T16* row, int vocab, int chunk, float (&v)[kElems]) {
     const uint16_t* const bits = reinterpret_cast<const uint16_t*>(row);
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int i0 = index_of(chunk, j, 0);
-      if (aligned && i0 + VEC <= vocab) {
-        const uint4 q = *reinterpret_cast<const uint4*>(bits + i0);
+      if (i0 + VEC <= vocab) {
+        const v4u_any q = *reinterpret_cast<const v4u_any*>(bits + i0);
         const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int c = 0; c < 4; ++c) {

@@ -617,11 +617,9 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
   u64* big_row = a.big + static_cast<size_t>(row) * a.big_stride;
   const InT* lrow = static_cast<const InT*>(row0);
   constexpr bool kOneRun = XFORM && sizeof(InT) == 4;  // the loads of a chunk are one straight run, see there
-  // 128-bit loads that assume no more than their elements' alignment: the hardware reads from any address, and rows
-  // that do not start on a 16-byte boundary (an odd vocabulary: 50257, 51865) only cost it more cache lines.  (Such
-  // rows used to be read element by element: 64 loads per thread where 16 do, 3.5 us more per step at 64 x 50257.)
-  typedef float v4f_any __attribute__((ext_vector_type(4), aligned(4)));
-  typedef uint32_t v4u_any __attribute__((ext_vector_type(4), aligned(2)));
+  // (The loads below are 128-bit loads that assume no more than their elements' alignment, v4f_any / v4u_any: rows
+  // that do not start on a 16-byte boundary used to be read element by element, 64 loads per thread where 16 do,
+  // 3.5 us more per step at 64 x 50257.)
   const float kNaN = __uint_as_float(0x7fc00000u);  // marks ids >= vocab: never a maximum, never >= a bound
   // The bitmap words and the first history ids of this thread are requested before the logits: loads come back in
   // the order they were asked for, and the history has a chain of its own to start (mark the ids, read their logits

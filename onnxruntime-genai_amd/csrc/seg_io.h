@@ -15,19 +15,18 @@ constexpr int kSegPer = kSegElems / kSegBlock;  // 16 elements per thread
 // Loads the 16 elements of thread t in segment `seg`: for j, the VEC consecutive ids starting at
 // seg*kSegElems + (j*256 + t)*VEC (VEC = 4 for fp32, 8 for fp16 and bf16).  Ids >= vocab yield `fill`.
 template <typename InT>
-__device__ __forceinline__ void seg_load(const InT* row, bool aligned, int vocab, int seg, float fill,
-                                         float (&v)[kSegPer]) {
+__device__ __forceinline__ void seg_load(const InT* row, int vocab, int seg, float fill, float (&v)[kSegPer]) {
   constexpr int VEC = sizeof(InT) == 4 ? 4 : 8;
   constexpr int NV = kSegPer / VEC;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int i0 = seg * kSegElems + (j * kSegBlock + static_cast<int>(threadIdx.x)) * VEC;
-    if (aligned && i0 + VEC <= vocab) {
+    if (i0 + VEC <= vocab) {
       if constexpr (VEC == 4) {
-        const v4f q = *reinterpret_cast<const v4f*>(row + i0);
+        const v4f_any q = *reinterpret_cast<const v4f_any*>(row + i0);
         v[j * 4] = q.x, v[j * 4 + 1] = q.y, v[j * 4 + 2] = q.z, v[j * 4 + 3] = q.w;
       } else {
-        const v4u q = *reinterpret_cast<const v4u*>(row + i0);
+        const v4u q = *reinterpret_cast<const v4u_any*>(row + i0);
         if constexpr (__is_same(InT, uint16_t)) {
           widen_half8(q, &v[j * 8]);  // the hardware conversion, redone by the bit formula where it differs
         } else {

@@ -74,9 +74,8 @@ __device__ __forceinline__ void seqsum_exp_step_body(const SeqSumArgs& a, const 
   double* const wave_parts = sh.wave_parts;
   const int seg = blockIdx.x, row = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const InT* x = static_cast<const InT*>(a.x) + static_cast<size_t>(row) * a.row_stride;
-  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
   float v[kSegPer];
-  seg_load<InT>(x, aligned, FULL ? (seg + 1) * kSegElems : a.vocab, seg, 0.0f, v);
+  seg_load<InT>(x, FULL ? (seg + 1) * kSegElems : a.vocab, seg, 0.0f, v);
   if (tid < 32) exp_tab[tid] = em::exp2_tab(static_cast<uint32_t>(tid));
   const float max_score = row_max_of_segments(a, row, red);  // its barriers also publish the table
   const uint64_t* const tab = exp_tab;

@@ -29,9 +29,8 @@ __global__ __launch_bounds__(kSegBlock) void seqsum_max_kernel(const SeqSumArgs 
   __shared__ uint32_t red[4];
   const int seg = blockIdx.x, row = blockIdx.y;
   const InT* x = static_cast<const InT*>(a.x) + static_cast<size_t>(row) * a.row_stride;
-  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
   float v[kSegPer];
-  seg_load<InT>(x, aligned, a.vocab, seg, -__builtin_inff(), v);
+  seg_load<InT>(x, a.vocab, seg, -__builtin_inff(), v);
   float fm = -__builtin_inff();
 #pragma unroll
   for (int e = 0; e < kSegPer; ++e) fm = fmaxf(fm, v[e]);

@@ -78,7 +78,7 @@ def test_topk_scores_large_k_of_sixteen_bit_rows(ctx, orc, dtype):
             assert np.array_equal(bits(sc[r]), bits(wide[r][order])), (k, r)
 
 
-@pytest.mark.parametrize("rows,vocab,t", [(4, 1000, 1.0), (3, 151936, 1.0), (2, 32064, 0.7), (2, 7, 2.0)])
+@pytest.mark.parametrize("rows,vocab,t", [(4, 1000, 1.0), (3, 151936, 1.0), (2, 32064, 0.7), (2, 7, 2.0), (5, 50257, 1.0)])
 def test_softmax_bit_exact(ctx, orc, rows, vocab, t):
     say("softmax", rows, vocab, t)
     rng = np.random.default_rng(vocab)
