@@ -338,8 +338,7 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
   // to four windows are read once per draw.
   constexpr int kItems = 8, kWindows = 4;
   const bool once = vocab <= kWindows * kItems * 1024;
-  // both rows start on a 16-byte boundary: their weights can be read eight at a time
-  const bool rows_aligned = ((reinterpret_cast<uintptr_t>(pt) | reinterpret_cast<uintptr_t>(pd)) & 15u) == 0;
+  // (the weights are read eight at a time, with 128-bit loads that take rows of any alignment)
   int pos = 0;
   bool from_target = n >= K;
   if (!from_target) {
@@ -348,8 +347,8 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
       return d > 0.0f ? d : 0.0f;
     };
     auto w8 = [=](int i, float (&out)[kItems]) {
-      const float4 t0 = *reinterpret_cast<const float4*>(pt + i), t1 = *reinterpret_cast<const float4*>(pt + i + 4);
-      const float4 d0 = *reinterpret_cast<const float4*>(pd + i), d1 = *reinterpret_cast<const float4*>(pd + i + 4);
+      const v4f_any t0 = *reinterpret_cast<const v4f_any*>(pt + i), t1 = *reinterpret_cast<const v4f_any*>(pt + i + 4);
+      const v4f_any d0 = *reinterpret_cast<const v4f_any*>(pd + i), d1 = *reinterpret_cast<const v4f_any*>(pd + i + 4);
       const float t[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
       const float d[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
 #pragma unroll
@@ -358,10 +357,8 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
         out[j] = r > 0.0f ? r : 0.0f;
       }
     };
-    if (once && rows_aligned) {
+    if (once) {
       pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &from_target, w8);
-    } else if (once) {
-      pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &from_target);
     } else {
       int any = 0;
 #pragma unroll 8
@@ -374,12 +371,11 @@ __global__ __launch_bounds__(1024) void spec_verify_kernel(const float* p_target
   if (from_target) {
     auto w = [=](int i) { return pt[i]; };
     auto w8 = [=](int i, float (&out)[kItems]) {
-      const float4 t0 = *reinterpret_cast<const float4*>(pt + i), t1 = *reinterpret_cast<const float4*>(pt + i + 4);
+      const v4f_any t0 = *reinterpret_cast<const v4f_any*>(pt + i), t1 = *reinterpret_cast<const v4f_any*>(pt + i + 4);
       out[0] = t0.x, out[1] = t0.y, out[2] = t0.z, out[3] = t0.w, out[4] = t1.x, out[5] = t1.y, out[6] = t1.z, out[7] = t1.w;
     };
     bool unused;
-    if (once && rows_aligned) pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &unused, w8);
-    else if (once) pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &unused);
+    if (once) pos = block_discrete_draw_once<kItems, kWindows>(vocab, w, sample_u[b], sh, stage, &unused, w8);
     else pos = block_discrete_draw<kItems>(vocab, w, sample_u[b], sh, stage);
   }
   if (threadIdx.x == 0) {

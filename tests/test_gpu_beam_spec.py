@@ -538,7 +538,8 @@ def softmax64(x):
     return (e / e.sum(-1, keepdims=True)).astype(np.float32)
 
 
-@pytest.mark.parametrize("batch,K,vocab", [(16, 8, 32064), (4, 3, 500), (5, 1, 2)])
+@pytest.mark.parametrize("batch,K,vocab", [(16, 8, 32064), (4, 3, 500), (5, 1, 2), (6, 8, 32001), (6, 6, 32003),
+                                             (6, 8, 4099)])  # (the last three: rows on every offset of a 16-byte line)
 def test_spec_verify(ctx, orc, batch, K, vocab):
     """Benchmark configuration 4 (first case): target/draft probabilities from N(0,2^2) logits, draft = target
     logits + N(0,0.5^2); accept tests and residual / bonus resampling with shared uniforms."""
