@@ -7,8 +7,10 @@
  * unless stated otherwise.  Return value: 0 on success, a negative MI355X_E_* code on failure, with a
  * thread-local message available from mi355x_search_last_error().
  *
- * Graph capture: every entry point only launches kernels on `stream`, with workspace from the context, and
- * can be captured into a HIP graph -- except the synchronous ones (create / destroy, *_is_done,
+ * Graph capture: every entry point only launches kernels on `stream` (mi355x_sample* with per-row parameters that
+ * put rows in several selection modes also on two streams of the context's own, which fork from `stream` behind
+ * an event and join it again before the call returns: part of the capture like any fork and join), with workspace
+ * from the context, and can be captured into a HIP graph -- except the synchronous ones (create / destroy, *_is_done,
  * *_hypothesis, *_fallback_rows, *_wait_gave_up, beam_scorer_set_prompt) and the two that advance a scorer's
  * host-side state (mi355x_beam_scorer_step, mi355x_beam_search_step: the sequence length and the buffer the
  * sequences live in are part of the launch, so a replay would repeat one step; they return

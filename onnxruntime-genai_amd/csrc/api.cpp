@@ -88,6 +88,7 @@ struct mi355x_search_ctx {
   // records a copy from the slot to the device table.  Slots of the ring are reused once the copy that read them
   // is done (an event per slot); a call on a capturing stream gets a slot of its own that is never reused, so the
   // copy node of its graph reads the same bytes at every replay.
+  ms::SideStreams sides{};  // where the kernels of a call with rows in several modes run side by side
   static constexpr int kStageRing = 8, kStageCaptured = 56;
   char* stage{};
   size_t stage_slot_bytes{};
@@ -237,6 +238,10 @@ int mi355x_search_create(int device, int max_rows, int max_vocab, mi355x_search_
   }
   for (int i = 0; i < mi355x_search_ctx::kStageRing && e == hipSuccess; ++i)
     e = hipEventCreateWithFlags(&c->stage_event[i], hipEventDisableTiming);
+  for (hipStream_t& st : c->sides.side)
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&st, hipStreamNonBlocking);
+  for (hipEvent_t* ev : {&c->sides.fork, &c->sides.join[0], &c->sides.join[1]})
+    if (e == hipSuccess) e = hipEventCreateWithFlags(ev, hipEventDisableTiming);
   if (e == hipSuccess) e = ms_sample_init();
   if (e == hipSuccess) e = ms_static_scratch_setup();  // set-up of mi355x_argmax_static on this device
   // the fills above ran on the null stream: done before a caller's stream, which need not wait for it, uses them
@@ -254,6 +259,10 @@ void mi355x_search_destroy(mi355x_search_ctx* ctx) {
   (void)hipSetDevice(ctx->device);
   for (void* p : ctx->allocs) (void)hipFree(p);
   for (hipEvent_t ev : ctx->stage_event)
+    if (ev) (void)hipEventDestroy(ev);
+  for (hipStream_t st : ctx->sides.side)
+    if (st) (void)hipStreamDestroy(st);
+  for (hipEvent_t ev : {ctx->sides.fork, ctx->sides.join[0], ctx->sides.join[1]})
     if (ev) (void)hipEventDestroy(ev);
   if (ctx->stage) (void)hipHostFree(ctx->stage);
   delete ctx;
@@ -307,7 +316,7 @@ int mi355x_argmax(mi355x_search_ctx* ctx, void* stream, const void* logits, int 
     f.big_stride = ctx->big_stride;
     f.fallback_rows = ctx->fallback_rows;
     f.poll_limit = ctx->poll_limit;
-    HIP_TRY(ms_launch_sample(&f, nullptr, true, false, false, s));
+    HIP_TRY(ms_launch_sample(&f, nullptr, true, false, false, s, nullptr));
     return MI355X_OK;
   }
   ms::ArgmaxArgs a{};
@@ -439,7 +448,7 @@ int SampleImpl(mi355x_search_ctx* ctx, hipStream_t s, const void* logits, const 
     const int64_t listed = static_cast<int64_t>(xf->mask_allowed_max) + (a.xf.use_penalty() ? hist : 0) + 2;
     a.sparse_only = listed <= ms::kNucleusCap && hist <= 2048;  // (what the kernel can list; beyond, all three kernels)
   }
-  HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_other, any_nucleus, any_large_k, s));
+  HIP_TRY(ms_launch_sample(&a, use_table ? &table : nullptr, any_other, any_nucleus, any_large_k, s, &ctx->sides));
   return MI355X_OK;
 }
 
@@ -537,7 +546,7 @@ int mi355x_topk_scores(mi355x_search_ctx* ctx, void* stream, const void* logits,
   const bool large_k = fits && k > 64 && k <= ms::kLargeKMax;
   const bool exact = vocab > 64 && (!fits || k > ms::kLargeKMax);
   a.exact_kernel = exact ? 1 : 0;
-  HIP_TRY(ms_launch_sample(&a, nullptr, !large_k && !exact, false, large_k, s));
+  HIP_TRY(ms_launch_sample(&a, nullptr, !large_k && !exact, false, large_k, s, nullptr));
   return MI355X_OK;
 }
 

@@ -43,6 +43,11 @@ struct InlineParams {
   const void* row_ptr[kInlineParamRows];  // where each row starts, for rows scattered over memory; null: row_stride apart
 };
 
+struct SideStreams {
+  hipStream_t side[2];
+  hipEvent_t fork, join[2];
+};
+
 struct SampleArgs {
   const void* logits;   // rows of fp32, fp16 or bf16 values (dtype), row_stride elements apart
   int64_t row_stride;
@@ -189,8 +194,11 @@ hipError_t ms_sample_init();
 // any_nucleus / any_large_k / any_other: some row may be in nucleus mode / a top-k row with
 // 64 < k <= kLargeKMax / in another mode (each mode has kernels of its own); a->exact_kernel: some row's
 // parameters send it to the exact path.
+// sides, when not null: streams and events of the context on which the kernels of a call whose rows are in several
+// modes run side by side (each mode's kernels skip the other modes' rows and share no state with them): they fork
+// from `stream` behind an event, and `stream` waits for them before the exact rows' kernel and before the call returns.
 hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_other, bool any_nucleus,
-                            bool any_large_k, hipStream_t stream);
+                            bool any_large_k, hipStream_t stream, const ms::SideStreams* sides);
 hipError_t ms_launch_argmax(const ms::ArgmaxArgs* a, int dtype, hipStream_t stream);
 hipError_t ms_launch_process_logits(float* logits, int64_t row_stride, int rows, int vocab,
                                     const ms::Xform* xf, hipStream_t stream);

@@ -1696,38 +1696,63 @@ __global__ __launch_bounds__(kFinishBlock) void exact_rows_rows_kernel(const Sam
 MS_STREAM_KERNELS(, float)  // the fp32 streaming kernels live here, next to the finish kernels
 
 extern "C" hipError_t ms_launch_sample(const ms::SampleArgs* a, const ms::InlineParams* table, bool any_other,
-                                       bool any_nucleus, bool any_large_k, hipStream_t stream) {
+                                       bool any_nucleus, bool any_large_k, hipStream_t stream,
+                                       const ms::SideStreams* sides) {
   const dim3 fgrid(a->rows), fblock(ms::kFinishBlock);
   auto launch_stream = a->dtype == MI355X_F16 ? ms_launch_stream_f16 : a->dtype == MI355X_BF16 ? ms_launch_stream_bf16 : ms_launch_stream;
+  // A call whose rows are in several modes launches the kernels of every mode present; one after the other their
+  // chains of dependent phases add up (12 + 42 + 39 us for top-k, nucleus and large-k rows in one batch of 64 x
+  // 128256), side by side the longest decides.  The nucleus rows' kernels, the longest chain, stay on the caller's
+  // stream.
+  const int modes = (any_other ? 1 : 0) + (any_nucleus ? 1 : 0) + (any_large_k ? 1 : 0);
+  const bool fork = sides != nullptr && modes > 1;
+  int forked = 0;
   hipError_t e = hipSuccess;
-  if (any_other) {
-    e = launch_stream(a, table, 0, stream);
+  auto stream_of_mode = [&](bool stays) -> hipStream_t {
+    if (!fork || stays) return stream;
+    hipStream_t s = sides->side[forked++];
+    if (e == hipSuccess) e = hipStreamWaitEvent(s, sides->fork, 0);
+    return s;
+  };
+  if (fork) {
+    e = hipEventRecord(sides->fork, stream);
     if (e != hipSuccess) return e;
   }
-  if (any_nucleus) {
+  if (any_other) {
+    const hipStream_t s = stream_of_mode(!any_nucleus && !any_large_k);
+    if (e == hipSuccess) e = launch_stream(a, table, 0, s);
+  }
+  if (any_large_k && e == hipSuccess) {
+    const hipStream_t s = stream_of_mode(!any_nucleus);
+    if (e == hipSuccess) e = launch_stream(a, table, 2, s);
+    if (e == hipSuccess) {
+      if (table) hipLaunchKernelGGL(ms::largek_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, s, *a, *table);
+      else hipLaunchKernelGGL(ms::largek_finish_kernel, fgrid, fblock, ms::kFinishLds, s, *a);
+      e = hipGetLastError();
+    }
+  }
+  if (any_nucleus && e == hipSuccess) {
     if (a->xf.mask && a->row_done) {  // rows under a sparse grammar mask are finished here; the next two kernels skip them
       if (table) hipLaunchKernelGGL(ms::nucleus_sparse_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
       else hipLaunchKernelGGL(ms::nucleus_sparse_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
       e = hipGetLastError();
-      if (e != hipSuccess) return e;
     }
-    if (!(a->xf.mask && a->row_done && a->sparse_only)) {
+    if (e == hipSuccess && !(a->xf.mask && a->row_done && a->sparse_only)) {
       e = launch_stream(a, table, 1, stream);
-      if (e != hipSuccess) return e;
-      if (table) hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
-      else hipLaunchKernelGGL(ms::nucleus_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
-      e = hipGetLastError();
-      if (e != hipSuccess) return e;
+      if (e == hipSuccess) {
+        if (table) hipLaunchKernelGGL(ms::nucleus_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
+        else hipLaunchKernelGGL(ms::nucleus_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
+        e = hipGetLastError();
+      }
     }
   }
-  if (any_large_k) {
-    e = launch_stream(a, table, 2, stream);
-    if (e != hipSuccess) return e;
-    if (table) hipLaunchKernelGGL(ms::largek_finish_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
-    else hipLaunchKernelGGL(ms::largek_finish_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);
-    e = hipGetLastError();
-    if (e != hipSuccess) return e;
+  // (the forked streams join even after an error: a stream left forked would poison a capture)
+  for (int i = 0; i < forked; ++i) {
+    hipError_t j = hipEventRecord(sides->join[i], sides->side[i]);
+    if (j == hipSuccess) j = hipStreamWaitEvent(stream, sides->join[i], 0);
+    if (e == hipSuccess) e = j;
   }
+  if (e != hipSuccess) return e;
   if (a->exact_kernel) {
     if (table) hipLaunchKernelGGL(ms::exact_rows_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a, *table);
     else hipLaunchKernelGGL(ms::exact_rows_kernel, fgrid, fblock, ms::kFinishLds, stream, *a);

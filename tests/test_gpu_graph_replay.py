@@ -120,6 +120,58 @@ def test_host_tables_are_staged_for_graph_capture(orc):
     ctx.close()
 
 
+def test_rows_in_several_modes_run_side_by_side(orc):
+    """A call whose rows are in several modes (top-k up to 64, nucleus, 64 < k) runs each mode's kernels on a stream
+    of the context's own, forked from the caller's stream and joined to it before the call returns.  Two such calls
+    in a row on a stream that is not the default one, with different inputs, then both captured into one graph and
+    replayed with eager calls of the same kind between the replays: tokens and kept sets equal the oracle's."""
+    say("modes side by side")
+    rows, vocab = 40, 70001
+    ctx = pkg().SearchContext(rows, vocab)
+    g = torch.Generator(device="cuda").manual_seed(29)
+    xs = [torch.randn(rows, vocab, generator=g, device="cuda") * 4 for _ in range(2)]
+    us = [torch.rand(rows, generator=g, device="cuda", dtype=torch.float64) for _ in range(2)]
+    menu = [(50, 0.9, 0.7), (0, 0.9, 1.0), (1, 0.0, 1.0), (200, 0.95, 1.0), (0, 0.5, 0.8), (64, 0.0, 1.2), (1000, 0.9, 1.0)]
+    params = [menu[(r * 5 + r // 7) % len(menu)] for r in range(rows)]
+    want = []
+    for x, u in zip(xs, us):
+        xh, uh = x.cpu().numpy(), u.cpu().numpy()
+        want.append(np.array([orc.sample_row(xh[r], *params[r], uh[r]) for r in range(rows)], np.int32))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    outs = [torch.zeros(rows, dtype=torch.int32, device="cuda") for _ in range(2)]
+    with torch.cuda.stream(side):
+        for i in range(2):
+            ctx.sample(xs[i], us[i], per_row=params, out=outs[i])
+    side.synchronize()
+    for i in range(2):
+        assert np.array_equal(outs[i].cpu().numpy(), want[i]), i
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(2):
+                ctx.sample(xs[i], us[i], per_row=params, out=outs[i])
+    torch.cuda.synchronize()
+    for replay in range(3):
+        for o in outs:
+            o.zero_()
+        with torch.cuda.stream(side):
+            graph.replay()
+        side.synchronize()
+        for i in range(2):
+            assert np.array_equal(outs[i].cpu().numpy(), want[i]), (replay, i)
+        tok, kc, ki, kp = ctx.sample(xs[replay % 2], us[replay % 2], per_row=params, kept_capacity=1024)
+        torch.cuda.synchronize()
+        assert np.array_equal(tok.cpu().numpy(), want[replay % 2]), replay
+        xh = xs[replay % 2].cpu().numpy()
+        for r in range(0, rows, 9):
+            idx, probs = orc.sampled_categorical(xh[r], *params[r])
+            n = min(len(idx), 1024)
+            assert kc[r].item() == len(idx) and np.array_equal(ki[r, :n].cpu().numpy(), idx[:n]), (replay, r)
+    assert ctx.fallback_rows() == 0
+    ctx.close()
+
+
 def test_scorer_steps_refuse_a_capturing_stream():
     """The scorer's steps carry host-side state (sequence length, which of two buffers holds the sequences):
     recording one into a graph would replay the same step, so they decline on a capturing stream."""
