@@ -207,7 +207,7 @@ def main():
     ap.add_argument("--pool", type=int, default=32, help="distinct logits buffers cycled through")
     ap.add_argument("--cpu-steps", type=int, default=24, help="steps replayed on the CPU oracle")
     ap.add_argument("--traffic", type=str, default=None, help="JSON {fetch_bytes, write_bytes} from rocprofv3 --pmc")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "topp", "largek", "topp_wide"],
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "topp", "largek", "topp_wide", "odd_vocab", "mixed_modes"],
                     help="c2 (default) is the headline configuration; the others time the remaining "
                          "configurations with the same JSON shape")
     ap.add_argument("--other-configs", type=int, default=1,
@@ -349,7 +349,7 @@ def main():
     other = {}
     if args.other_configs:
         import bench_workloads
-        for name in ("c1", "c3", "c4", "c5", "topp", "largek", "topp_wide"):
+        for name in ("c1", "c3", "c4", "c5", "topp", "largek", "topp_wide", "odd_vocab", "mixed_modes"):
             sub = argparse.Namespace(**vars(args))
             sub.workload = name
             line = bench_workloads.run(sub, pkg, orc, orc_lib, dev)

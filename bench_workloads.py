@@ -322,7 +322,50 @@ def topp(args, pkg, orc, dev, k=0, sigma=5.0):
                  _cpu(rows_cpu / cpu_s, "tokens/s", "%d rows of one step, one thread" % rows_cpu, cpu_s / rows_cpu * B * 1e3))
 
 
+def variant(args, pkg, orc, dev, name):
+    """Two workloads beside the configurations: `odd_vocab`, config 2's parameters on 64 x 50257 rows (GPT-2's
+    vocabulary: rows 50257 fp32 elements apart start on every 4-byte offset of a 16-byte line), and `mixed_modes`,
+    64 x 128256 rows whose per-row parameters put them in four selection modes (k = 50 with p = 0.9, top-p only,
+    greedy, k = 200), whose kernels run side by side."""
+    B = 64
+    V = 50257 if name == "odd_vocab" else 128256
+    K = args.steps if args.steps != 128 else 32
+    W = min(args.warmup, 4)
+    g = torch.Generator(device=dev).manual_seed(13)
+    pool = 8
+    logits = [torch.randn(B, V, generator=g, device=dev) * 5.0 for _ in range(pool)]
+    u_host = np.random.default_rng(77).random((K + W, B))
+    uniforms = torch.from_numpy(u_host).to(dev)
+    tokens = torch.empty((K + W, B), dtype=torch.int32, device=dev)
+    ctx = pkg.SearchContext(B, V)
+    menu = [(50, 0.9, 0.7), (0, 0.9, 1.0), (1, 0.0, 1.0), (200, 0.95, 1.0)]
+    params = [menu[0]] * B if name == "odd_vocab" else [menu[r % 4] for r in range(B)]
+    if name == "odd_vocab":
+        step = lambda i: ctx.sample(logits[i % pool], uniforms[i], k=50, p=0.9, temperature=0.7, out=tokens[i])
+    else:
+        step = lambda i: ctx.sample(logits[i % pool], uniforms[i], per_row=params, out=tokens[i])
+    ms = _timed(step, K, W)
+    rows_cpu = 16
+    x = logits[W % pool][:rows_cpu].cpu().numpy()
+    t0 = time.perf_counter()
+    want = [orc.sample_row(x[r], *params[r], u_host[W, r]) for r in range(rows_cpu)]
+    cpu_s = time.perf_counter() - t0
+    got = tokens[W, :rows_cpu].cpu().numpy()
+    assert np.array_equal(got, np.array(want, np.int32)), "PARITY FAILURE (%s)" % name
+    what = ("top-k/top-p sampling (T=0.7 k=50 p=0.9), batch 64 x vocab 50257 fp32: rows off 16-byte boundaries"
+            if name == "odd_vocab" else
+            "rows in four selection modes (k=50 p=0.9 T=0.7 / top-p 0.9 / greedy / k=200 p=0.95), batch 64 x vocab 128256 fp32")
+    return _line(args, "sampled tokens/sec + step latency, " + ("B=64 V=50257 top-k/p" if name == "odd_vocab" else "B=64 V=128256 mixed modes"),
+                 "tokens/s", B * K / (ms * 1e-3), ms, K, W, "f32",
+                 "%s, %d steps replayed from a HIP graph over %d logits buffers" % (what, K, pool),
+                 {"general_path_rows": ctx.fallback_rows(),
+                  "parity": "%d rows of one step bit-identical to the CPU oracle" % rows_cpu}, B * V * 4,
+                 _cpu(rows_cpu / cpu_s, "tokens/s", "%d rows of one step, one thread" % rows_cpu, cpu_s / rows_cpu * B * 1e3))
+
+
 def run(args, pkg, orc, orc_lib, dev):
+    if args.workload in ("odd_vocab", "mixed_modes"):
+        return variant(args, pkg, orc, dev, args.workload)
     if args.workload == "topp":
         return topp(args, pkg, orc, dev)
     if args.workload == "largek":
