@@ -68,7 +68,8 @@ typedef struct mi355x_search_ctx mi355x_search_ctx;
  *   history  device [rows, history_stride] int32 token ids, the first history_len of each row valid
  *            (Sequences::GetSequence, src/sequences.h:18); every DISTINCT in-range id has its logit
  *            s replaced by s<0 ? s*penalty : s/penalty (src/sampling_distribution.h:41-62).
- *            NULL or penalty == 1.0f = none.  history_stride 0 lets all rows share one buffer.
+ *            NULL or penalty == 1.0f = none.  history_stride 0 lets all rows share one buffer.  (All
+ *            history_stride ids of a row may be read, whatever its length: the buffer holds them all.)
  *   eos_ids  with apply_min_length != 0 each in-range id gets lowest()
  *            (src/sampling_distribution.h:26-35; the caller evaluates current_length < min_length).
  *   history_lens  optional device [rows] int32: row r uses the first history_lens[r] ids of its
