@@ -806,30 +806,68 @@ __device__ __forceinline__ bool stream_row(const SampleArgs& a, int row, const v
       }
     }
   } else {
-    // sixteen-bit rows: all loads are requested before the first is widened
     v4u raw[kSLoads];
-    uint32_t whole = 0u;  // bit j: load j lies inside the row
+    if constexpr (XFORM) {
+      // Sixteen-bit rows of the kernels with logits processing: eight 128-bit loads per thread in one straight run,
+      // like the fp32 rows' sixteen, and the processing's preparations right behind them.  A load that would cross
+      // the row's end reads from the row's start instead; the (at most seven) elements of the one group of eight
+      // that straddles the end are fetched once more, one by one and by every thread alike, and the registers past
+      // the end are put right after the widening.
+      float row_end[VEC - 1];
+      if (!whole_chunk) {  // (ahead of the run, which so is the same number of requests for every chunk)
 #pragma unroll
-    for (int j = 0; j < kSLoads; ++j) {
-      const int i0 = elem_index<kSBlock, VEC>(chunk, 2 * j, 0);
-      if (i0 + VEC <= V) {
-        raw[j] = __builtin_nontemporal_load(reinterpret_cast<const v4u_any*>(lrow + i0));
-        whole |= 1u << j;
+        for (int c = 0; c < VEC - 1; ++c) {
+          const int i = (V & ~(VEC - 1)) + c;
+          row_end[c] = load_one<InT>(lrow, i < V ? i : 0);
+        }
       }
-    }
 #pragma unroll
-    for (int j = 0; j < kSLoads; ++j) {
-      const int i0 = elem_index<kSBlock, VEC>(chunk, 2 * j, 0);
-      if ((whole >> j) & 1u) {
+      for (int j = 0; j < kSLoads; ++j) {
+        const int i0 = elem_index<kSBlock, VEC>(chunk, 2 * j, 0);
+        raw[j] = __builtin_nontemporal_load(reinterpret_cast<const v4u_any*>(lrow + (i0 + VEC <= V ? i0 : 0)));
+      }
+      xform_prep();
+#pragma unroll
+      for (int j = 0; j < kSLoads; ++j) {
         if constexpr (sizeof(InT) == 2 && !__is_same(InT, bf16_t)) widen_half8(raw[j], &v[j * VEC]);
         else widen_bf16x8(raw[j], &v[j * VEC]);
-      } else {
+      }
+      if (!whole_chunk) {
+        const int r = V & (VEC - 1);  // elements of the straddling group that lie inside the row
 #pragma unroll
-        for (int c = 0; c < VEC; ++c) v[j * VEC + c] = (i0 + c < V) ? load_one<InT>(lrow, i0 + c) : kNaN;
+        for (int j = 0; j < kSLoads; ++j) {
+          const int i0 = elem_index<kSBlock, VEC>(chunk, 2 * j, 0);
+          if (i0 + VEC > V) {
+            const bool straddles = i0 < V;
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) v[j * VEC + c] = (straddles && c < r) ? row_end[c < VEC - 1 ? c : 0] : kNaN;
+          }
+        }
+      }
+    } else {
+      // sixteen-bit rows: all loads are requested before the first is widened
+      uint32_t whole = 0u;  // bit j: load j lies inside the row
+#pragma unroll
+      for (int j = 0; j < kSLoads; ++j) {
+        const int i0 = elem_index<kSBlock, VEC>(chunk, 2 * j, 0);
+        if (i0 + VEC <= V) {
+          raw[j] = __builtin_nontemporal_load(reinterpret_cast<const v4u_any*>(lrow + i0));
+          whole |= 1u << j;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kSLoads; ++j) {
+        const int i0 = elem_index<kSBlock, VEC>(chunk, 2 * j, 0);
+        if ((whole >> j) & 1u) {
+          if constexpr (sizeof(InT) == 2 && !__is_same(InT, bf16_t)) widen_half8(raw[j], &v[j * VEC]);
+          else widen_bf16x8(raw[j], &v[j * VEC]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) v[j * VEC + c] = (i0 + c < V) ? load_one<InT>(lrow, i0 + c) : kNaN;
+        }
       }
     }
   }
-  if constexpr (XFORM && !kOneRun) xform_prep();  // (sixteen-bit rows)
   if constexpr (!XFORM) {
     if (tid == 0) sm.poisoned = a.fallback_rows[1];
   }
