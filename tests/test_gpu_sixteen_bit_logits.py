@@ -136,6 +136,39 @@ def test_sixteen_bit_rows_with_logits_processing(ctx, orc, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("vocab", [40001, 40002, 40003, 40004, 40005, 40006, 40007, 98305])
+def test_sixteen_bit_rows_with_logits_processing_that_end_inside_a_group_of_eight(ctx, orc, dtype, vocab):
+    """The kernels with logits processing read a sixteen-bit chunk as eight 128-bit loads per thread whatever the
+    row's end; the group of eight that straddles it is fetched once more element by element.  Vocabularies that end
+    one to seven elements into a group (and a last chunk of one element), the row's best tokens on its last
+    elements, some of them penalised or masked."""
+    say("16-bit xform row ends", dtype, vocab)
+    rows = 5
+    g = torch.Generator(device="cuda").manual_seed(vocab)
+    x = (torch.randn(rows, vocab, generator=g, device="cuda") * 3).to(dtype)
+    x[0, vocab - 1] = 30.0
+    x[1, vocab - 2] = 30.0
+    x[2, vocab - 3] = 30.0
+    x[3, vocab - 1] = 29.0
+    x[3, vocab - 5] = 30.0
+    rng = np.random.default_rng(vocab)
+    mask = make_mask(rng, rows, vocab, 0.8)
+    mask[2, (vocab - 3) >> 5] &= ~np.uint32(1 << ((vocab - 3) & 31))
+    hist = rng.integers(0, vocab, (rows, 120)).astype(np.int32)
+    hist[:, 0] = vocab - 2
+    hist[:, 1] = vocab - 1
+    u = rng.random(rows)
+    xf = pkg().LogitsXform(mask=torch.from_numpy(mask.view(np.int32)).cuda(), history=torch.from_numpy(hist).cuda(),
+                           repetition_penalty=1.5)
+    proc = orc.apply_mask(widened(orc, x), mask)
+    for r in range(rows):
+        proc[r] = orc.apply_repetition_penalty(proc[r], hist[r], 1.5)
+    check_sample(ctx, orc, x, u, [(50, 0.9, 0.7), (0, 0.9, 1.0), (1, 0.0, 1.0), (300, 0.95, 1.0), (8, 0.0, 1.0)], xf=xf, proc=proc,
+                 cap=4096)
+    assert np.array_equal(ctx.argmax(x, xf).cpu().numpy(), orc.argmax_batch(proc))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_argmax_sixteen_bit_rows(ctx, orc, dtype):
     say("argmax 16-bit", dtype)
     g = torch.Generator(device="cuda").manual_seed(21)
