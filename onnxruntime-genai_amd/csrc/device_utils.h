@@ -297,7 +297,15 @@ struct Xform {
   __host__ __device__ __forceinline__ bool use_penalty() const {
     return history && (history_lens || history_len > 0) && (penalty != 1.0f || ban);
   }
-  __device__ __forceinline__ int hist_len(int row) const { return history_lens ? history_lens[row] : history_len; }
+  // (The common length passes through a register before the branch: as a plain `lens ? lens[row] : len` the compiler
+  // loads through a selected pointer, which for the common length is a round trip to the kernel arguments in memory
+  // and, being a load that may go anywhere, makes every wait behind it a wait for all loads.)
+  __device__ __forceinline__ int hist_len(int row) const {
+    int n = history_len;
+    asm volatile("" : "+s"(n));
+    if (history_lens) n = history_lens[row];
+    return n;
+  }
   __device__ __forceinline__ int eos_count(int row) const {
     return (history_lens && min_length > 0 && history_lens[row] >= min_length) ? 0 : n_eos;
   }

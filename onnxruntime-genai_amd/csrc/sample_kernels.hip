@@ -1454,6 +1454,10 @@ __device__ __forceinline__ int nucleus_sparse_body(const SampleArgs& a) {
   // at once would have every wave wait at its load instructions, the queues being full, and reach the history
   // only when the gather is nearly over.)
   constexpr int kFirstLoads = 6;
+  // (What the history needs of the loads requested further up has long arrived; the wait for it stands here, ahead
+  // of the gather: behind it the compiler, which cannot count requests made under conditions, would wait for the
+  // gather's loads as well.)
+  asm volatile("" ::"v"(mw0), "v"(raw0));
   gather_slots(std::integral_constant<int, 0>{}, std::integral_constant<int, kFirstLoads>{});
   asm volatile("" ::: "memory");
   // history ids: marked in a bitmap of the whole row; whoever marks an id first computes its processed value
