@@ -139,16 +139,20 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(const void* const* prese
   char* dst = static_cast<char*>(past[t]) + static_cast<size_t>(row) * block_bytes + tile0;
   const size_t remain = block_bytes - tile0;
   const int n16 = static_cast<int>((remain < static_cast<size_t>(kGatherTile) ? remain : kGatherTile) / 16);
+  // (The tensors' addresses come out of a table in memory, which tells the compiler nothing about where they point:
+  // they are device memory, and the accesses say so -- plain global loads and stores instead of flat ones.)
+  typedef __attribute__((address_space(1))) const v4u* DeviceVec;
+  typedef __attribute__((address_space(1))) v4u* DeviceVecOut;
   v4u regs[kGatherTile / 16 / 256];
 #pragma unroll
   for (int j = 0; j < kGatherTile / 16 / 256; ++j) {
     const int i = j * 256 + threadIdx.x;
-    if (i < n16) regs[j] = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(src) + i);
+    if (i < n16) regs[j] = __builtin_nontemporal_load((DeviceVec)src + i);
   }
 #pragma unroll
   for (int j = 0; j < kGatherTile / 16 / 256; ++j) {
     const int i = j * 256 + threadIdx.x;
-    if (i < n16) __builtin_nontemporal_store(regs[j], reinterpret_cast<v4u*>(dst) + i);
+    if (i < n16) __builtin_nontemporal_store(regs[j], (DeviceVecOut)dst + i);
   }
 }
 
